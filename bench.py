@@ -1,0 +1,320 @@
+#!/usr/bin/env python3
+"""bench.py — throughput of the deepxIR op hot path on one MI355X.
+
+A "step" is one pass of BASELINE config 2 (the reductions workload) through libdxhip's C ABI
+on synthetic tensors already resident in HBM:
+    X fp32 [8192,8192] N(0,1):  sum axis 1, sum axis 0, reducemax axis 1, reducemin axis 1
+    P fp32 [8192,64]  U(.9,1.1): prod axis 1
+each with keepdims true and false (keepdims only changes the caller's view of the output, so
+both launches run the same kernel) = 10 ops, 2,152,005,632 algorithmic bytes per step
+(inputs read once + outputs written once per op).  X exists in three copies that the ops
+rotate through, so no launch finds its input in the 256 MiB Infinity Cache.
+
+Prints ONE JSON line: value = algorithmic GB/s over the timed region (all ops), `roofline`
+for the dominant kernel (reduce_row_kernel, the contiguous-axis reduction: 6 of the 10 ops)
+from HIP events recorded on the launch stream inside the timed region, `cpu_baseline` from
+the oracle's restatement of op-ompsimd's per-element reduce on the host cores, and `per_op`
+with every other BASELINE op measured the same way (events around each launch).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+MFMA_BF16_PEAK_TF = 2500.0  # dense bf16
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-per-op", action="store_true", help="skip the per-op table of the other configs")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this executor path runs on ONE GPU (no sharding, no collectives); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from deepx_amd import lib as dx
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    L = dx.load()
+    torch.cuda.init()
+    dev = torch.device("cuda:0")
+    name = C.create_string_buffer(256)
+    L.dxh_device_name(name, 256)
+
+    class Events:
+        """pairs of hipEvents recorded on the NULL stream, the stream every op is launched on"""
+
+        def __init__(self):
+            self.pairs = []
+
+        def pair(self):
+            a, b = C.c_void_p(), C.c_void_p()
+            dx.check(L.dxh_event_create(C.byref(a)))
+            dx.check(L.dxh_event_create(C.byref(b)))
+            self.pairs.append((a, b))
+            return a, b
+
+        @staticmethod
+        def ms(a, b):
+            out = C.c_float()
+            dx.check(L.dxh_event_elapsed_ms(a, b, C.byref(out)))
+            return out.value
+
+    def ptr(t):
+        return C.c_void_p(t.data_ptr())
+
+    # ---------------- config 2: the step --------------------------------------------------
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    NX = 3
+    Xs = [torch.randn(8192, 8192, generator=g, device=dev, dtype=torch.float32) for _ in range(NX)]
+    g.manual_seed(4)
+    Ps = [torch.rand(8192, 64, generator=g, device=dev, dtype=torch.float32) * 0.2 + 0.9 for _ in range(NX)]
+    out = torch.empty(8192, device=dev, dtype=torch.float32)
+    shX, shP = dx.i32arr([8192, 8192]), dx.i32arr([8192, 64])
+    ax0, ax1 = dx.i32arr([0]), dx.i32arr([1])
+    wsb = C.c_size_t(0)
+    dx.check(L.dxh_reduce_workspace_bytes(dx.F32, shX, 2, ax0, 1, C.byref(wsb)))
+    ws = torch.empty(max(1, wsb.value), device=dev, dtype=torch.uint8)
+    XB = 8192 * 8192 * 4 + 8192 * 4
+    PB = 8192 * 64 * 4 + 8192 * 4
+    # (label, fn, shape, axis, which buffers, algorithmic bytes, kernel)
+    ops = []
+    for kd in ("kd1", "kd0"):
+        ops += [
+            ("sum_axis1_" + kd, L.dxh_sum, shX, ax1, Xs, XB, "reduce_row_kernel"),
+            ("sum_axis0_" + kd, L.dxh_sum, shX, ax0, Xs, XB, "reduce_col_kernel"),
+            ("reducemax_axis1_" + kd, L.dxh_reducemax, shX, ax1, Xs, XB, "reduce_row_kernel"),
+            ("reducemin_axis1_" + kd, L.dxh_reducemin, shX, ax1, Xs, XB, "reduce_row_kernel"),
+            ("prod_8192x64_axis1_" + kd, L.dxh_prod, shP, ax1, Ps, PB, "reduce_row_kernel(small)"),
+        ]
+    step_bytes = sum(o[5] for o in ops)
+    rot = [0]
+
+    def run_step(events=None):
+        for i, (label, fn, sh, ax, bufs, nbytes, kern) in enumerate(ops):
+            buf = bufs[rot[0] % NX]
+            rot[0] += 1
+            if events is not None:
+                a, b = events[i]
+                L.dxh_event_record(a, None)
+            rc = fn(dx.F32, ptr(buf), sh, 2, ax, 1, ptr(out), ptr(ws), wsb.value, None)
+            if events is not None:
+                L.dxh_event_record(b, None)
+            if rc != 0:
+                dx.check(rc, label)
+
+    ev = Events()
+    step_events = [[ev.pair() for _ in ops] for _ in range(args.steps)]
+    for _ in range(args.warmup):
+        run_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        run_step(step_events[s])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    per_label = {}
+    for s in range(args.steps):
+        for i, o in enumerate(ops):
+            per_label.setdefault(o[0], []).append(Events.ms(*step_events[s][i]))
+    c2 = {}
+    for o in ops:
+        ms = float(np.mean(per_label[o[0]]))
+        c2[o[0]] = {"ms": round(ms, 5), "GB/s": round(o[5] / ms / 1e6, 1), "frac_hbm": round(o[5] / ms / 1e6 / HBM_PEAK_GBS, 4),
+                    "bytes": o[5], "kernel": o[6]}
+    dom = [per_label[o[0]] for o in ops if o[6] == "reduce_row_kernel"]
+    dom_ms = float(np.mean(np.concatenate(dom)))
+    achieved = XB / dom_ms / 1e6
+    roofline = {"bound": "hbm", "kernel": "reduce_row_kernel<sum|max|min,f32> [8192,8192] axis 1",
+                "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "avg_launch_ms": round(dom_ms, 5),
+                "bytes_per_launch": XB, "traffic": None}
+
+    # ---------------- the other BASELINE configs, one op at a time ----------------------------
+    per_op = {"config2": c2}
+    if not args.no_per_op:
+        del Xs, Ps
+        torch.cuda.empty_cache()
+        per_op.update(bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr))
+
+    # ---------------- CPU baseline: the oracle's restatement of op-ompsimd's reduce ---------
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(np, dx)
+
+    line = {
+        "metric": "achieved HBM GB/s & % of peak per deepxIR op; matmul TFLOP/s; vs op-ompsimd",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config2: reductions on fp32 [8192,8192] (sum axis1/axis0, reducemax, reducemin) + prod [8192,64], keepdims true+false, 10 ops/step",
+                   "bytes_per_step": step_bytes, "input_copies_rotated": NX, "device": name.value.decode()},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "per_op": per_op,
+    }
+    print(json.dumps(line))
+
+
+def time_op(L, dx, torch, Events, ev, launch, reps=20, warm=3):
+    """average hipEvent time (ms) of `launch(i)` over `reps` launches on the NULL stream"""
+    for i in range(warm):
+        launch(i)
+    torch.cuda.synchronize()
+    pairs = [ev.pair() for _ in range(reps)]
+    for i, (a, b) in enumerate(pairs):
+        L.dxh_event_record(a, None)
+        rc = launch(warm + i)
+        L.dxh_event_record(b, None)
+        if rc:
+            dx.check(rc, "bench op")
+    torch.cuda.synchronize()
+    import numpy as np
+    return float(np.mean([Events.ms(a, b) for a, b in pairs]))
+
+
+def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
+    res = {}
+
+    def entry(ms, nbytes=None, flops=None):
+        e = {"ms": round(ms, 5)}
+        if nbytes is not None:
+            e.update({"GB/s": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes})
+        if flops is not None:
+            e.update({"TFLOP/s": round(flops / ms / 1e9, 2), "frac_mfma_bf16": round(flops / ms / 1e9 / MFMA_BF16_PEAK_TF, 4), "flops": flops})
+        return e
+
+    # ---- config 1: fp32 [4096,4096] elementwise chain; 4 rotating buffer sets (64 MiB tensors)
+    n = 4096 * 4096
+    R = 4
+    A = [torch.rand(n, device=dev) * 2 - 1 for _ in range(R)]
+    B = [torch.rand(n, device=dev) * 2 - 1 for _ in range(R)]
+    O = [torch.empty(n, device=dev) for _ in range(R)]
+    half = dx.scalar(0.5)
+    c1 = {}
+    c1["add"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_add(dx.F32, ptr(A[i % R]), ptr(B[i % R]), ptr(O[i % R]), n, None)), 3 * n * 4)
+    c1["mul"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_mul(dx.F32, ptr(A[i % R]), ptr(B[i % R]), ptr(O[i % R]), n, None)), 3 * n * 4)
+    c1["max"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_max(dx.F32, ptr(A[i % R]), ptr(B[i % R]), ptr(O[i % R]), n, None)), 3 * n * 4)
+    c1["div"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_div(dx.F32, ptr(A[i % R]), ptr(B[i % R]), ptr(O[i % R]), n, None)), 3 * n * 4)
+    c1["addscalar"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_addscalar(dx.F32, ptr(A[i % R]), half, ptr(O[i % R]), n, None)), 2 * n * 4)
+    c1["mulscalar"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_mulscalar(dx.F32, ptr(A[i % R]), half, ptr(O[i % R]), n, None)), 2 * n * 4)
+    c1["exp"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_exp(dx.F32, ptr(A[i % R]), ptr(O[i % R]), n, None)), 2 * n * 4)
+    res["config1"] = c1
+    del A, B, O
+    torch.cuda.empty_cache()
+
+    # ---- config 3: changeshape on 16-bit tensors
+    c3 = {}
+    shape = [32, 2048, 14, 64]
+    nt = 32 * 2048 * 14 * 64
+    T = [torch.randn(nt, device=dev).to(torch.bfloat16) for _ in range(3)]
+    TO = [torch.empty(nt, device=dev, dtype=torch.bfloat16) for _ in range(3)]
+    sh, od = dx.i32arr(shape), dx.i32arr([0, 2, 1, 3])
+    c3["transpose_bf16_32x2048x14x64_0213"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_transpose(dx.BF16, ptr(T[i % 3]), sh, 4, od, ptr(TO[i % 3]), None)), 2 * nt * 2)
+    del T, TO
+    torch.cuda.empty_cache()
+    nc = 16 * 1024 * 4096
+    cs = [torch.randn(nc, device=dev).to(torch.float16) for _ in range(3)]
+    co = [torch.empty(3 * nc, device=dev, dtype=torch.float16) for _ in range(2)]
+    ins = dx.ptrarr([t.data_ptr() for t in cs])
+    axs, osh = dx.i32arr([1024] * 3), dx.i32arr([16, 3072, 4096])
+    c3["concat_fp16_3x16x1024x4096_axis1"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_concat(dx.F16, ins, 3, axs, osh, 3, 1, ptr(co[i % 2]), None)), 2 * 3 * nc * 2)
+    del cs, co
+    torch.cuda.empty_cache()
+    r = torch.randn(4096, device=dev).to(torch.bfloat16)
+    bo = [torch.empty(8192 * 4096, device=dev, dtype=torch.bfloat16) for _ in range(5)]
+    ish, bsh = dx.i32arr([1, 4096]), dx.i32arr([8192, 4096])
+    c3["broadcastTo_bf16_1x4096_to_8192x4096"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_broadcastTo(dx.BF16, ptr(r), ish, 2, bsh, 2, ptr(bo[i % 5]), None)), 8192 + 8192 * 4096 * 2)
+    del bo
+    torch.cuda.empty_cache()
+    res["config3"] = c3
+
+    # ---- config 4: int32 2^26 and the embedding gather
+    c4 = {}
+    n = 1 << 26
+    a = [torch.randint(-2 ** 20, 2 ** 20 + 1, (n,), device=dev, dtype=torch.int32) for _ in range(2)]
+    b = [torch.randint(-2 ** 20, 2 ** 20 + 1, (n,), device=dev, dtype=torch.int32) for _ in range(2)]
+    o = [torch.empty(n, device=dev, dtype=torch.int32) for _ in range(2)]
+    m = [torch.empty(n, device=dev, dtype=torch.uint8) for _ in range(2)]
+    c4["max_i32_2^26"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_max(dx.I32, ptr(a[i % 2]), ptr(b[i % 2]), ptr(o[i % 2]), n, None)), 3 * n * 4)
+    c4["min_i32_2^26"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_min(dx.I32, ptr(a[i % 2]), ptr(b[i % 2]), ptr(o[i % 2]), n, None)), 3 * n * 4)
+    c4["greater_i32_2^26"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_greater(dx.I32, ptr(a[i % 2]), ptr(b[i % 2]), ptr(m[i % 2]), n, None)), 2 * n * 4 + n)
+    sw = [dx.ptrarr([b[j].data_ptr(), a[j].data_ptr()]) for j in range(2)]
+    c4["where_i32_2^26(switch)"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_switch(dx.I32, sw[i % 2], 2, dx.BOOL, ptr(m[i % 2]), ptr(o[i % 2]), n, None)), n + 3 * n * 4)
+    del a, b, o, m
+    torch.cuda.empty_cache()
+    E = (torch.randn(151936, 896, device=dev) * 0.02).to(torch.bfloat16)
+    idx = [torch.randint(0, 151936, (4096,), device=dev, dtype=torch.int64) for _ in range(4)]
+    eo = torch.empty(4096 * 896, device=dev, dtype=torch.bfloat16)
+    esh, xsh = dx.i32arr([151936, 896]), dx.i32arr([4096])
+    c4["indexselect_bf16_4096_of_151936x896(latency-bound)"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_indexselect(dx.BF16, ptr(E), esh, 2, dx.I64, ptr(idx[i % 4]), xsh, 1, 0, ptr(eo), None)), 2 * 4096 * 896 * 2 + 4096 * 8)
+    del E, eo
+    torch.cuda.empty_cache()
+    res["config4"] = c4
+
+    # ---- config 5: the three bf16 GEMMs of the Qwen2-0.5B MLP (fp32 accumulate)
+    c5 = {}
+    for label, (mm, kk, nn) in [("matmul_bf16_2048x896x4864", (2048, 896, 4864)), ("matmul_bf16_2048x4864x896", (2048, 4864, 896))]:
+        Am = torch.randn(mm * kk, device=dev).to(torch.bfloat16)
+        Bm = (torch.randn(kk * nn, device=dev) * 0.02).to(torch.bfloat16)
+        Cm = torch.empty(mm * nn, device=dev, dtype=torch.bfloat16)
+        c5[label] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_matmul(dx.BF16, ptr(Am), ptr(Bm), ptr(Cm), 1, mm, kk, nn, None)), flops=2 * mm * kk * nn)
+    res["config5"] = c5
+    return res
+
+
+def cpu_baseline(np, dx):
+    """The oracle's restatement of op-ompsimd's reduce (one callback per input element, index
+    vector, atomic accumulate) on this host's cores, on the same step."""
+    from tests import helpers as H
+    orc = H.oracle()
+    cores = orc.orc_num_threads()
+    rows = 8192
+    rng = np.random.default_rng(3)
+    X = rng.standard_normal((rows, 8192), dtype=np.float32)
+    P = np.random.default_rng(4).uniform(0.9, 1.1, (8192, 64)).astype(np.float32)
+    out = np.empty(8192, dtype=np.float32)
+    shX, shP = dx.i32arr([rows, 8192]), dx.i32arr([8192, 64])
+    plan = [(0, X, shX, [1]), (0, X, shX, [0]), (2, X, shX, [1]), (3, X, shX, [1]), (1, P, shP, [1])]
+    nbytes = 0
+    # one untimed pass to fault the pages in, then one timed pass of the 5 distinct ops x 2 keepdims
+    for op, arr, sh, ax in plan:
+        orc.orc_faithful_reduce_f32(op, H.hp(arr), sh, 2, dx.i32arr(ax), 1, 0, H.hp(out))
+    t0 = time.perf_counter()
+    for kd in (1, 0):
+        for op, arr, sh, ax in plan:
+            assert orc.orc_faithful_reduce_f32(op, H.hp(arr), sh, 2, dx.i32arr(ax), 1, kd, H.hp(out)) == 0
+            nbytes += arr.nbytes + 8192 * 4
+    dt = time.perf_counter() - t0
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.startswith("model name"):
+                    model = ln.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"one full config-2 step (10 ops, {nbytes} bytes) in {dt:.2f} s; OMP threads={cores}; cpu='{model}'; -O2, AVX2 auto-vectorisation"}
+
+
+if __name__ == "__main__":
+    main()

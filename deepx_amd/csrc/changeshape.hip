@@ -1,0 +1,510 @@
+// changeshape.hip — transpose, concat, broadcastTo, indexselect, repeat (gfx950).
+//
+// Semantics: executor/op-ompsimd/src/deepx/tensorfunc/changeshape_miaobyte.hpp:45-200 with the
+// shape rules of executor/deepxcore/src/deepx/shape_changeshape.cpp.  The reference moves one
+// element per callback through index vectors; every op here is pure byte movement, so the
+// kernels are chosen by layout, not dtype:
+//
+//   gather_rows   the innermost run of the output is also contiguous in the input (transpose
+//                 that keeps the last axis, broadcastTo, indexselect): one lane moves one
+//                 16-byte unit (or the widest power of two that divides the run), the output
+//                 is written fully contiguously, the input row start comes from a mixed-radix
+//                 decomposition of the row number (strides may be 0 = broadcast).
+//   tile_transpose the last axis moves: 64x64 tiles staged through padded LDS so that both the
+//                 global read (along the input's last axis) and the global write (along the
+//                 output's last axis) are coalesced.
+//   concat        one launch for up to 8 sources; each source is a 2-D strided copy into the
+//                 output rows.
+// All are HBM-bound: algorithmic bytes = bytes read once + bytes written once.
+#include "common.hpp"
+#include <vector>
+
+namespace dxh {
+
+constexpr int kGatherUnroll = 4;
+constexpr int kMaxOuter = DXH_MAX_DIMS;
+
+struct OuterDims {
+    int n;                        // number of outer (row-indexing) dims
+    uint32_t size[kMaxOuter];     // output extent of each
+    int64_t stride[kMaxOuter];    // input stride of each, in units
+};
+
+// widest power-of-two unit (<= 16 bytes) dividing `bytes` and every pointer in `ptrs`
+inline int unit_bytes(int64_t run_bytes, std::initializer_list<const void *> ptrs) {
+    int u = kVecBytes;
+    while (u > 1 && run_bytes % u != 0) u >>= 1;
+    for (const void *p : ptrs) while (u > 1 && !aligned(p, u)) u >>= 1;
+    return u;
+}
+
+// ---- gather_rows -------------------------------------------------------------------------
+// out is [rows, Lu] units, contiguous.  in row start = sum_i idx_i * stride_i (units) where idx
+// is the mixed-radix decomposition of the row number over `od`.  SPLAT: the input contributes a
+// single element of type E per row position (innermost axis broadcast) that fills the unit.
+template <typename U, typename I, bool SPLAT, typename E>
+__global__ __launch_bounds__(kBlock) void gather_rows_kernel(const void *__restrict__ in_, U *__restrict__ out, I total,
+                                                              I Lu, OuterDims od) {
+    const I tile = (I)kBlock * kGatherUnroll;
+    const I stride = (I)gridDim.x * tile;
+    for (I base = (I)blockIdx.x * tile; base < total; base += stride) {
+        U x[kGatherUnroll];
+        I g[kGatherUnroll];
+#pragma unroll
+        for (int u = 0; u < kGatherUnroll; ++u) {
+            g[u] = base + (I)u * kBlock + threadIdx.x;
+            if (g[u] < total) {
+                I row = g[u] / Lu;
+                I v = g[u] - row * Lu;
+                int64_t off = 0;
+                for (int d = od.n - 1; d >= 0; --d) {
+                    I q = row / od.size[d];
+                    off += (int64_t)(row - q * od.size[d]) * od.stride[d];
+                    row = q;
+                }
+                if constexpr (SPLAT) {
+                    E e = reinterpret_cast<const E *>(in_)[off];
+                    constexpr int N = sizeof(U) / sizeof(E);
+                    vec_t<E, N> r;
+#pragma unroll
+                    for (int k = 0; k < N; ++k) r.v[k] = e;
+                    x[u] = __builtin_bit_cast(U, r);
+                } else {
+                    x[u] = reinterpret_cast<const U *>(in_)[off + (int64_t)v];
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kGatherUnroll; ++u)
+            if (g[u] < total) out[g[u]] = x[u];
+    }
+}
+
+template <int UB, bool SPLAT, typename E>
+int launch_gather_unit(const void *in, void *out, int64_t rows, int64_t Lu, const OuterDims &od, hipStream_t st) {
+    using U = typename raw_of<UB>::type;
+    const int64_t total = rows * Lu;
+    unsigned grid = stream_grid(total, (int64_t)kBlock * kGatherUnroll, 8);
+    if (total < (int64_t)1 << 31)
+        gather_rows_kernel<U, uint32_t, SPLAT, E><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint32_t)total, (uint32_t)Lu, od);
+    else
+        gather_rows_kernel<U, uint64_t, SPLAT, E><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint64_t)total, (uint64_t)Lu, od);
+    return launch_status();
+}
+
+// rows x run_bytes bytes per row; od.stride in ELEMENT-of-esize units on entry, converted here
+inline int launch_gather(const void *in, void *out, int64_t rows, int64_t run_elems, int esize, OuterDims od, hipStream_t st) {
+    if (rows * run_elems == 0) return DXH_OK;
+    const int ub = unit_bytes(run_elems * esize, {in, out});
+    const int64_t Lu = run_elems * esize / ub;
+    for (int d = 0; d < od.n; ++d) od.stride[d] = od.stride[d] * esize / ub;  // strides are multiples of the run
+    switch (ub) {
+    case 16: return launch_gather_unit<16, false, uint8_t>(in, out, rows, Lu, od, st);
+    case 8: return launch_gather_unit<8, false, uint8_t>(in, out, rows, Lu, od, st);
+    case 4: return launch_gather_unit<4, false, uint8_t>(in, out, rows, Lu, od, st);
+    case 2: return launch_gather_unit<2, false, uint8_t>(in, out, rows, Lu, od, st);
+    default: return launch_gather_unit<1, false, uint8_t>(in, out, rows, Lu, od, st);
+    }
+}
+
+// innermost axis broadcast: every output row of `run_elems` elements repeats one input element
+template <typename E>
+int launch_splat(const void *in, void *out, int64_t rows, int64_t run_elems, const OuterDims &od, hipStream_t st) {
+    if (rows * run_elems == 0) return DXH_OK;
+    int ub = unit_bytes(run_elems * (int64_t)sizeof(E), {out});
+    if (ub < (int)sizeof(E)) ub = sizeof(E);
+    const int64_t Lu = run_elems * sizeof(E) / ub;
+    switch (ub) {
+    case 16: return launch_gather_unit<16, true, E>(in, out, rows, Lu, od, st);
+    case 8: if constexpr (sizeof(E) <= 8) return launch_gather_unit<8, true, E>(in, out, rows, Lu, od, st);
+    case 4: if constexpr (sizeof(E) <= 4) return launch_gather_unit<4, true, E>(in, out, rows, Lu, od, st);
+    case 2: if constexpr (sizeof(E) <= 2) return launch_gather_unit<2, true, E>(in, out, rows, Lu, od, st);
+    default: if constexpr (sizeof(E) == 1) return launch_gather_unit<1, true, E>(in, out, rows, Lu, od, st);
+    }
+    return DXH_ERR_ARG;
+}
+
+// ---- tile_transpose ----------------------------------------------------------------------
+// Input viewed through `bd` batch dims plus two tiled axes: axis A (size nA, input stride sA,
+// contiguous in the OUTPUT) and axis C (size nC, contiguous in the INPUT, output stride oC).
+struct BatchDims {
+    int n;
+    uint32_t size[kMaxOuter];
+    int64_t istride[kMaxOuter];
+    int64_t ostride[kMaxOuter];
+};
+constexpr int kTile = 64;
+
+template <typename E>
+__global__ __launch_bounds__(kBlock) void tile_transpose_kernel(const E *__restrict__ in, E *__restrict__ out, int64_t nA,
+                                                                 int64_t sA, int64_t nC, int64_t oC, int tilesA, int tilesC,
+                                                                 BatchDims bd) {
+    __shared__ E tile[kTile][kTile + 1];
+    int64_t b = blockIdx.x;
+    const int tc = (int)(b % tilesC); b /= tilesC;
+    const int ta = (int)(b % tilesA); b /= tilesA;
+    int64_t ioff = 0, ooff = 0;
+    for (int d = bd.n - 1; d >= 0; --d) {
+        int64_t q = b / bd.size[d];
+        int64_t r = b - q * bd.size[d];
+        ioff += r * bd.istride[d];
+        ooff += r * bd.ostride[d];
+        b = q;
+    }
+    const int tx = threadIdx.x % kTile, ty = threadIdx.x / kTile;  // 64 x 4
+    const int64_t a0 = (int64_t)ta * kTile, c0 = (int64_t)tc * kTile;
+    // read: rows along A, lanes along C (contiguous in the input)
+#pragma unroll 4
+    for (int r = ty; r < kTile; r += kBlock / kTile) {
+        int64_t a = a0 + r, c = c0 + tx;
+        if (a < nA && c < nC) tile[r][tx] = in[ioff + a * sA + c];
+    }
+    __syncthreads();
+    // write: rows along C, lanes along A (contiguous in the output)
+#pragma unroll 4
+    for (int r = ty; r < kTile; r += kBlock / kTile) {
+        int64_t c = c0 + r, a = a0 + tx;
+        if (a < nA && c < nC) out[ooff + c * oC + a] = tile[tx][r];
+    }
+}
+
+// ---- concat --------------------------------------------------------------------------------
+constexpr int kConcatMax = 8;
+struct ConcatSrcs {
+    int n;
+    const void *ptr[kConcatMax];
+    int64_t run[kConcatMax];     // units per outer row of this source
+    int64_t pref[kConcatMax];    // unit offset of this source inside an output row
+    int64_t cum[kConcatMax + 1]; // units before this source in the flattened work list
+};
+
+template <typename U>
+__global__ __launch_bounds__(kBlock) void concat_kernel(ConcatSrcs s, U *__restrict__ out, int64_t out_row, int64_t total) {
+    const int64_t tile = (int64_t)kBlock * kGatherUnroll;
+    const int64_t stride = (int64_t)gridDim.x * tile;
+    for (int64_t base = (int64_t)blockIdx.x * tile; base < total; base += stride) {
+        U x[kGatherUnroll];
+        int64_t dst[kGatherUnroll];
+#pragma unroll
+        for (int u = 0; u < kGatherUnroll; ++u) {
+            int64_t g = base + (int64_t)u * kBlock + threadIdx.x;
+            dst[u] = -1;
+            if (g < total) {
+                int i = 0;
+#pragma unroll
+                for (int k = 1; k < kConcatMax; ++k) if (k < s.n && g >= s.cum[k]) i = k;
+                int64_t local = g - s.cum[i];
+                int64_t o = local / s.run[i];
+                int64_t v = local - o * s.run[i];
+                x[u] = reinterpret_cast<const U *>(s.ptr[i])[local];
+                dst[u] = o * out_row + s.pref[i] + v;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kGatherUnroll; ++u)
+            if (dst[u] >= 0) out[dst[u]] = x[u];
+    }
+}
+
+// ---- indexselect ---------------------------------------------------------------------------
+template <typename U, typename IT>
+__global__ __launch_bounds__(kBlock) void indexselect_kernel(const U *__restrict__ in, const IT *__restrict__ index,
+                                                              U *__restrict__ out, int64_t total, int64_t Lu, int64_t M,
+                                                              int64_t adim) {
+    const int64_t tile = (int64_t)kBlock * kGatherUnroll;
+    const int64_t stride = (int64_t)gridDim.x * tile;
+    for (int64_t base = (int64_t)blockIdx.x * tile; base < total; base += stride) {
+        U x[kGatherUnroll];
+        int64_t g[kGatherUnroll];
+#pragma unroll
+        for (int u = 0; u < kGatherUnroll; ++u) {
+            g[u] = base + (int64_t)u * kBlock + threadIdx.x;
+            if (g[u] < total) {
+                int64_t row = g[u] / Lu, v = g[u] - row * Lu;
+                int64_t p = row / M, j = row - p * M;
+                int64_t k = (int64_t)index[j];
+                k = k < 0 ? 0 : (k >= adim ? adim - 1 : k);
+                x[u] = in[(p * adim + k) * Lu + v];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kGatherUnroll; ++u)
+            if (g[u] < total) out[g[u]] = x[u];
+    }
+}
+
+// ---- repeat --------------------------------------------------------------------------------
+struct RepeatDims {
+    int n;
+    uint32_t osize[kMaxOuter];
+    uint32_t reps[kMaxOuter];
+    int64_t istride[kMaxOuter];
+};
+template <typename E>
+__global__ __launch_bounds__(kBlock) void repeat_kernel(const E *__restrict__ in, E *__restrict__ out, int64_t total, RepeatDims rd) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t g = (int64_t)blockIdx.x * kBlock + threadIdx.x; g < total; g += stride) {
+        int64_t rem = g, off = 0;
+        for (int d = rd.n - 1; d >= 0; --d) {
+            int64_t q = rem / rd.osize[d];
+            int64_t r = rem - q * rd.osize[d];
+            off += (r / rd.reps[d]) * rd.istride[d];
+            rem = q;
+        }
+        out[g] = in[off];
+    }
+}
+
+inline bool valid_shape(const int32_t *shape, int ndim, int64_t *size) {
+    if (!shape || ndim < 1 || ndim > DXH_MAX_DIMS) return false;
+    int64_t n = 1;
+    for (int i = 0; i < ndim; ++i) { if (shape[i] < 0) return false; n *= shape[i]; }
+    *size = n;
+    return true;
+}
+
+}  // namespace dxh
+
+using namespace dxh;
+
+extern "C" {
+
+int dxh_transpose(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *order, void *out, void *stream) {
+    const int es = dtype_size(dtype);
+    if (!es) return DXH_ERR_DTYPE;
+    int64_t n;
+    if (!valid_shape(shape, ndim, &n) || !order) return DXH_ERR_ARG;
+    bool seen[DXH_MAX_DIMS] = {false};
+    for (int i = 0; i < ndim; ++i) {
+        if (order[i] < 0 || order[i] >= ndim || seen[order[i]]) return DXH_ERR_ARG;
+        seen[order[i]] = true;
+    }
+    if (n == 0) return DXH_OK;
+    if (!in || !out) return DXH_ERR_ARG;
+    if (!aligned(in, es) || !aligned(out, es)) return DXH_ERR_ALIGN;
+    hipStream_t st = as_stream(stream);
+    // input strides (elements)
+    int64_t istr[DXH_MAX_DIMS];
+    { int64_t s = 1; for (int i = ndim - 1; i >= 0; --i) { istr[i] = s; s *= shape[i]; } }
+    // output dims in output order: (size, input stride); drop size-1, merge input-adjacent runs
+    int64_t osz[DXH_MAX_DIMS], ost[DXH_MAX_DIMS];
+    int nd = 0;
+    for (int i = 0; i < ndim; ++i) {
+        int64_t sz = shape[order[i]], sd = istr[order[i]];
+        if (sz == 1) continue;
+        if (nd > 0 && ost[nd - 1] == sd * sz) { osz[nd - 1] *= sz; ost[nd - 1] = sd; }
+        else { osz[nd] = sz; ost[nd] = sd; ++nd; }
+    }
+    if (nd <= 1) {  // identity permutation
+        if (in == out) return DXH_OK;
+        return (int)hipMemcpyAsync(out, in, (size_t)n * es, hipMemcpyDeviceToDevice, st);
+    }
+    for (int i = 0; i < nd; ++i) if (osz[i] > 0xffffffffLL) return DXH_ERR_SHAPE;
+    if (ost[nd - 1] == 1) {
+        // the innermost output run is contiguous in the input too
+        OuterDims od{};
+        od.n = nd - 1;
+        int64_t rows = 1;
+        for (int i = 0; i < nd - 1; ++i) { od.size[i] = (uint32_t)osz[i]; od.stride[i] = ost[i]; rows *= osz[i]; }
+        return launch_gather(in, out, rows, osz[nd - 1], es, od, st);
+    }
+    // the last axis moves: tile over (A = output-last axis, C = input-last axis)
+    int64_t ostr[DXH_MAX_DIMS];
+    { int64_t s = 1; for (int i = nd - 1; i >= 0; --i) { ostr[i] = s; s *= osz[i]; } }
+    int qc = -1;
+    for (int i = 0; i < nd; ++i) if (ost[i] == 1) qc = i;
+    if (qc < 0) return DXH_ERR_ARG;  // cannot happen: some merged dim holds the input's last axis
+    const int64_t nA = osz[nd - 1], sA = ost[nd - 1], nC = osz[qc], oC = ostr[qc];
+    BatchDims bd{};
+    int64_t batch = 1;
+    for (int i = 0; i < nd - 1; ++i) {
+        if (i == qc) continue;
+        bd.size[bd.n] = (uint32_t)osz[i]; bd.istride[bd.n] = ost[i]; bd.ostride[bd.n] = ostr[i]; ++bd.n;
+        batch *= osz[i];
+    }
+    const int64_t tilesA = (nA + kTile - 1) / kTile, tilesC = (nC + kTile - 1) / kTile;
+    const int64_t blocks = batch * tilesA * tilesC;
+    if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
+    switch (es) {
+    case 8: tile_transpose_kernel<uint64_t><<<(unsigned)blocks, kBlock, 0, st>>>((const uint64_t *)in, (uint64_t *)out, nA, sA, nC, oC, (int)tilesA, (int)tilesC, bd); break;
+    case 4: tile_transpose_kernel<uint32_t><<<(unsigned)blocks, kBlock, 0, st>>>((const uint32_t *)in, (uint32_t *)out, nA, sA, nC, oC, (int)tilesA, (int)tilesC, bd); break;
+    case 2: tile_transpose_kernel<uint16_t><<<(unsigned)blocks, kBlock, 0, st>>>((const uint16_t *)in, (uint16_t *)out, nA, sA, nC, oC, (int)tilesA, (int)tilesC, bd); break;
+    default: tile_transpose_kernel<uint8_t><<<(unsigned)blocks, kBlock, 0, st>>>((const uint8_t *)in, (uint8_t *)out, nA, sA, nC, oC, (int)tilesA, (int)tilesC, bd); break;
+    }
+    return launch_status();
+}
+
+int dxh_concat(int dtype, const void *const *ins, int nins, const int32_t *axis_sizes, const int32_t *out_shape, int ndim,
+               int axis, void *out, void *stream) {
+    const int es = dtype_size(dtype);
+    if (!es) return DXH_ERR_DTYPE;
+    int64_t n;
+    if (!valid_shape(out_shape, ndim, &n) || !ins || !axis_sizes || nins < 1 || axis < 0 || axis >= ndim) return DXH_ERR_ARG;
+    int64_t total_axis = 0;
+    for (int i = 0; i < nins; ++i) { if (axis_sizes[i] < 0) return DXH_ERR_ARG; total_axis += axis_sizes[i]; }
+    if (total_axis != out_shape[axis]) return DXH_ERR_SHAPE;
+    if (n == 0) return DXH_OK;
+    if (!out) return DXH_ERR_ARG;
+    int64_t outer = 1, inner = 1;
+    for (int i = 0; i < axis; ++i) outer *= out_shape[i];
+    for (int i = axis + 1; i < ndim; ++i) inner *= out_shape[i];
+    // unit: widest power of two dividing every run and every pointer
+    int ub = unit_bytes(inner * es * total_axis, {out});
+    for (int i = 0; i < nins; ++i) {
+        if (axis_sizes[i] == 0) continue;
+        if (!ins[i]) return DXH_ERR_ARG;
+        ub = std::min(ub, unit_bytes((int64_t)axis_sizes[i] * inner * es, {ins[i]}));
+    }
+    if (ub < es && (!aligned(out, es))) return DXH_ERR_ALIGN;
+    const int64_t out_row = total_axis * inner * es / ub;
+    hipStream_t st = as_stream(stream);
+    int64_t pref = 0;
+    int i = 0;
+    while (i < nins) {
+        ConcatSrcs s{};
+        int64_t cum = 0;
+        while (i < nins && s.n < kConcatMax) {
+            int64_t run = (int64_t)axis_sizes[i] * inner * es / ub;
+            if (run > 0) {
+                s.ptr[s.n] = ins[i]; s.run[s.n] = run; s.pref[s.n] = pref; s.cum[s.n] = cum;
+                cum += run * outer;
+                ++s.n;
+            }
+            pref += run;
+            ++i;
+        }
+        s.cum[s.n] = cum;
+        if (s.n == 0 || cum == 0) continue;
+        unsigned grid = stream_grid(cum, (int64_t)kBlock * kGatherUnroll, 8);
+        switch (ub) {
+        case 16: concat_kernel<uint4><<<grid, kBlock, 0, st>>>(s, (uint4 *)out, out_row, cum); break;
+        case 8: concat_kernel<uint64_t><<<grid, kBlock, 0, st>>>(s, (uint64_t *)out, out_row, cum); break;
+        case 4: concat_kernel<uint32_t><<<grid, kBlock, 0, st>>>(s, (uint32_t *)out, out_row, cum); break;
+        case 2: concat_kernel<uint16_t><<<grid, kBlock, 0, st>>>(s, (uint16_t *)out, out_row, cum); break;
+        default: concat_kernel<uint8_t><<<grid, kBlock, 0, st>>>(s, (uint8_t *)out, out_row, cum); break;
+        }
+        int rc = launch_status();
+        if (rc != DXH_OK) return rc;
+    }
+    return DXH_OK;
+}
+
+int dxh_broadcastTo(int dtype, const void *in, const int32_t *in_shape, int in_ndim, const int32_t *out_shape, int out_ndim,
+                    void *out, void *stream) {
+    const int es = dtype_size(dtype);
+    if (!es) return DXH_ERR_DTYPE;
+    int64_t nin, nout;
+    if (!valid_shape(in_shape, in_ndim, &nin) || !valid_shape(out_shape, out_ndim, &nout)) return DXH_ERR_ARG;
+    if (in_ndim > out_ndim) return DXH_ERR_SHAPE;
+    const int shift = out_ndim - in_ndim;
+    int64_t istr[DXH_MAX_DIMS];
+    { int64_t s = 1; for (int i = in_ndim - 1; i >= 0; --i) { istr[i] = s; s *= in_shape[i]; } }
+    // per output axis: input stride, 0 where the axis is broadcast (broadcastMap, shape_changeshape.cpp:79-104)
+    int64_t sz[DXH_MAX_DIMS], sd[DXH_MAX_DIMS];
+    int nd = 0;
+    for (int i = 0; i < out_ndim; ++i) {
+        int64_t stride = 0;
+        if (i >= shift) {
+            if (in_shape[i - shift] == out_shape[i]) stride = istr[i - shift];
+            else if (in_shape[i - shift] == 1) stride = 0;
+            else return DXH_ERR_SHAPE;
+        }
+        if (out_shape[i] == 1) continue;
+        // merge: both broadcast, or both dense and adjacent in the input
+        if (nd > 0 && ((sd[nd - 1] == 0 && stride == 0) || (stride != 0 && sd[nd - 1] == stride * out_shape[i]))) {
+            sz[nd - 1] *= out_shape[i];
+            sd[nd - 1] = stride;
+        } else { sz[nd] = out_shape[i]; sd[nd] = stride; ++nd; }
+    }
+    if (nout == 0) return DXH_OK;
+    if (!in || !out) return DXH_ERR_ARG;
+    if (!aligned(in, es) || !aligned(out, es)) return DXH_ERR_ALIGN;
+    hipStream_t st = as_stream(stream);
+    if (nd == 0 || (nd == 1 && sd[0] == 1)) {
+        if (in == out) return DXH_OK;
+        return (int)hipMemcpyAsync(out, in, (size_t)nout * es, hipMemcpyDeviceToDevice, st);
+    }
+    for (int i = 0; i < nd; ++i) if (sz[i] > 0xffffffffLL) return DXH_ERR_SHAPE;
+    OuterDims od{};
+    od.n = nd - 1;
+    int64_t rows = 1;
+    for (int i = 0; i < nd - 1; ++i) { od.size[i] = (uint32_t)sz[i]; od.stride[i] = sd[i]; rows *= sz[i]; }
+    if (sd[nd - 1] == 1) return launch_gather(in, out, rows, sz[nd - 1], es, od, st);
+    // innermost axis is broadcast: splat one element per row position
+    switch (es) {
+    case 8: return launch_splat<uint64_t>(in, out, rows, sz[nd - 1], od, st);
+    case 4: return launch_splat<uint32_t>(in, out, rows, sz[nd - 1], od, st);
+    case 2: return launch_splat<uint16_t>(in, out, rows, sz[nd - 1], od, st);
+    default: return launch_splat<uint8_t>(in, out, rows, sz[nd - 1], od, st);
+    }
+}
+
+int dxh_indexselect(int dtype, const void *in, const int32_t *in_shape, int in_ndim, int index_dtype, const void *index,
+                    const int32_t *index_shape, int index_ndim, int axis, void *out, void *stream) {
+    const int es = dtype_size(dtype);
+    if (!es) return DXH_ERR_DTYPE;
+    if (index_dtype != DXH_I32 && index_dtype != DXH_I64) return DXH_ERR_DTYPE;
+    int64_t nin, m;
+    if (!valid_shape(in_shape, in_ndim, &nin) || !valid_shape(index_shape, index_ndim, &m)) return DXH_ERR_ARG;
+    if (axis < 0) axis += in_ndim;
+    if (axis < 0 || axis >= in_ndim) return DXH_ERR_ARG;
+    int64_t pre = 1, post = 1;
+    for (int i = 0; i < axis; ++i) pre *= in_shape[i];
+    for (int i = axis + 1; i < in_ndim; ++i) post *= in_shape[i];
+    const int64_t adim = in_shape[axis];
+    if (pre * m * post == 0) return DXH_OK;
+    if (adim == 0) return DXH_ERR_SHAPE;
+    if (!in || !index || !out) return DXH_ERR_ARG;
+    if (!aligned(in, es) || !aligned(out, es) || !aligned(index, index_dtype == DXH_I64 ? 8 : 4)) return DXH_ERR_ALIGN;
+    const int ub = unit_bytes(post * es, {in, out});
+    const int64_t Lu = post * es / ub;
+    const int64_t total = pre * m * Lu;
+    hipStream_t st = as_stream(stream);
+    unsigned grid = stream_grid(total, (int64_t)kBlock * kGatherUnroll, 8);
+#define DXH_IS(U)                                                                                                      \
+    if (index_dtype == DXH_I64)                                                                                        \
+        indexselect_kernel<U, int64_t><<<grid, kBlock, 0, st>>>((const U *)in, (const int64_t *)index, (U *)out, total, Lu, m, adim); \
+    else                                                                                                               \
+        indexselect_kernel<U, int32_t><<<grid, kBlock, 0, st>>>((const U *)in, (const int32_t *)index, (U *)out, total, Lu, m, adim);
+    switch (ub) {
+    case 16: DXH_IS(uint4) break;
+    case 8: DXH_IS(uint64_t) break;
+    case 4: DXH_IS(uint32_t) break;
+    case 2: DXH_IS(uint16_t) break;
+    default: DXH_IS(uint8_t) break;
+    }
+#undef DXH_IS
+    return launch_status();
+}
+
+int dxh_repeat(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *repeats, void *out, void *stream) {
+    const int es = dtype_size(dtype);
+    if (!es) return DXH_ERR_DTYPE;
+    int64_t nin;
+    if (!valid_shape(shape, ndim, &nin) || !repeats) return DXH_ERR_ARG;
+    RepeatDims rd{};
+    rd.n = ndim;
+    int64_t total = 1, s = 1;
+    for (int i = ndim - 1; i >= 0; --i) {
+        if (repeats[i] < 1) return DXH_ERR_ARG;
+        int64_t o = (int64_t)shape[i] * repeats[i];
+        if (o > 0xffffffffLL) return DXH_ERR_SHAPE;
+        rd.osize[i] = (uint32_t)o; rd.reps[i] = (uint32_t)repeats[i]; rd.istride[i] = s;
+        s *= shape[i];
+        total *= o;
+    }
+    if (total == 0) return DXH_OK;
+    if (!in || !out) return DXH_ERR_ARG;
+    if (!aligned(in, es) || !aligned(out, es)) return DXH_ERR_ALIGN;
+    hipStream_t st = as_stream(stream);
+    unsigned grid = stream_grid(total, kBlock, 16);
+    switch (es) {
+    case 8: repeat_kernel<uint64_t><<<grid, kBlock, 0, st>>>((const uint64_t *)in, (uint64_t *)out, total, rd); break;
+    case 4: repeat_kernel<uint32_t><<<grid, kBlock, 0, st>>>((const uint32_t *)in, (uint32_t *)out, total, rd); break;
+    case 2: repeat_kernel<uint16_t><<<grid, kBlock, 0, st>>>((const uint16_t *)in, (uint16_t *)out, total, rd); break;
+    default: repeat_kernel<uint8_t><<<grid, kBlock, 0, st>>>((const uint8_t *)in, (uint8_t *)out, total, rd); break;
+    }
+    return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,101 @@
+// common.hpp — shared device/host helpers of libdxhip (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <type_traits>
+#include "../../include/dxhip.h"
+
+namespace dxh {
+
+constexpr int kWave = 64;          // CDNA wavefront width
+constexpr int kBlock = 256;        // 4 waves per workgroup: one per SIMD of a CU
+constexpr int kCUs = 256;          // MI355X: 8 XCDs x 32 CUs
+constexpr int kVecBytes = 16;      // one global_load_dwordx4 per lane
+
+// ---- storage types ---------------------------------------------------------------------
+// 16-bit floats are carried as raw bits; arithmetic happens in fp32 and is rounded once
+// (RNE) on store.
+struct bf16_t { uint16_t bits; };
+struct f16_t { uint16_t bits; };
+struct bool_t { uint8_t v; };
+
+template <typename T> struct acc_of { using type = T; };
+template <> struct acc_of<bf16_t> { using type = float; };
+template <> struct acc_of<f16_t> { using type = float; };
+template <typename T> using acc_t = typename acc_of<T>::type;
+
+__host__ __device__ inline float bits_to_float(uint32_t u) { return __builtin_bit_cast(float, u); }
+__host__ __device__ inline uint32_t float_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+__host__ __device__ inline float load_acc(bf16_t x) { return bits_to_float(uint32_t(x.bits) << 16); }
+__host__ __device__ inline float load_acc(f16_t x) { return float(__builtin_bit_cast(_Float16, x.bits)); }
+template <typename T> __host__ __device__ inline T load_acc(T x) { return x; }
+
+__host__ __device__ inline bf16_t to_bf16(float f) {
+    uint32_t u = float_to_bits(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return bf16_t{uint16_t((u >> 16) | 0x0040u)};
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return bf16_t{uint16_t(u >> 16)};
+}
+__host__ __device__ inline f16_t to_f16(float f) {
+    return f16_t{__builtin_bit_cast(uint16_t, (_Float16)f)};  // v_cvt_f16_f32, RNE
+}
+template <typename T> __host__ __device__ inline T store_acc(acc_t<T> v) {
+    if constexpr (std::is_same_v<T, bf16_t>) return to_bf16(v);
+    else if constexpr (std::is_same_v<T, f16_t>) return to_f16(v);
+    else return v;
+}
+
+// scalar operand -> storage type, mirroring T(std::stof(text)) upstream of the ABI
+template <typename T> inline T scalar_to(const dxh_scalar &s) {
+    if constexpr (std::is_same_v<T, bf16_t>) return to_bf16(float(s.f));
+    else if constexpr (std::is_same_v<T, f16_t>) return to_f16(float(s.f));
+    else if constexpr (std::is_floating_point_v<T>) return T(s.f);
+    else return T(s.i);
+}
+
+// ---- 16-byte vectors -------------------------------------------------------------------
+template <typename T, int N> struct alignas(sizeof(T) * N) vec_t { T v[N]; };
+template <typename T> constexpr int vec_len = kVecBytes / (int)sizeof(T);
+
+template <int BYTES> struct raw_of;
+template <> struct raw_of<1> { using type = uint8_t; };
+template <> struct raw_of<2> { using type = uint16_t; };
+template <> struct raw_of<4> { using type = uint32_t; };
+template <> struct raw_of<8> { using type = uint64_t; };
+template <> struct raw_of<16> { using type = uint4; };
+
+inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+inline int dtype_size(int dtype) {
+    switch (dtype) {
+    case DXH_F64: case DXH_I64: return 8;
+    case DXH_F32: case DXH_I32: return 4;
+    case DXH_F16: case DXH_BF16: case DXH_I16: return 2;
+    case DXH_I8: case DXH_BOOL: return 1;
+    default: return 0;
+    }
+}
+
+// ---- launch helpers --------------------------------------------------------------------
+inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Number of workgroups for a streaming kernel whose workgroup consumes `per_block` work
+// items per loop trip: enough to cover the work, capped at `waves_per_cu` resident
+// workgroups per CU so the grid-stride loop keeps every CU's queues full.
+inline unsigned stream_grid(int64_t items, int64_t per_block, int blocks_per_cu) {
+    int64_t need = (items + per_block - 1) / per_block;
+    int64_t cap = (int64_t)kCUs * blocks_per_cu;
+    if (need < 1) need = 1;
+    return (unsigned)(need < cap ? need : cap);
+}
+
+inline int launch_status() {
+    hipError_t e = hipGetLastError();
+    return (int)e;
+}
+
+#define DXH_CHECK_N(n) do { if ((n) < 0) return DXH_ERR_ARG; if ((n) == 0) return DXH_OK; } while (0)
+#define DXH_CHECK_PTR(p) do { if (!(p)) return DXH_ERR_ARG; } while (0)
+
+}  // namespace dxh

@@ -1,0 +1,319 @@
+// elementwise.hip — streaming elementwise kernels of libdxhip (gfx950).
+//
+// Every op here is HBM-bound: one 16-byte global load per lane per operand
+// (global_load_dwordx4), UNROLL independent vectors in flight per lane, a grid-stride
+// loop over workgroup tiles of 256*UNROLL vectors, and a grid capped at a few resident
+// workgroups per CU.  Arithmetic follows executor/op-ompsimd's
+// tensorfunc/elementwise_miaobyte.hpp (cited per op in include/dxhip.h); 16-bit floats
+// compute in fp32 and round once.
+#include "common.hpp"
+
+namespace dxh {
+
+constexpr int kUnroll = 4;
+constexpr int kBlocksPerCU = 8;
+
+// ---- op functors on the accumulate type -----------------------------------------------
+template <typename A> __device__ inline A wrap_add(A a, A b) { using U = std::make_unsigned_t<A>; return A(U(U(a) + U(b))); }
+template <typename A> __device__ inline A wrap_sub(A a, A b) { using U = std::make_unsigned_t<A>; return A(U(U(a) - U(b))); }
+template <typename A> __device__ inline A wrap_mul(A a, A b) {
+    using U = std::conditional_t<(sizeof(A) < 4), uint32_t, std::make_unsigned_t<A>>;
+    return A(U(U(a) * U(b)));
+}
+template <typename A> __device__ inline A wrap_div(A a, A b) {
+    if (b == 0) return A(0);
+    if (b == A(-1)) return wrap_sub<A>(A(0), a);
+    return A(a / b);
+}
+
+struct OpAdd { template <typename A> __device__ static A f(A a, A b) { if constexpr (std::is_integral_v<A>) return wrap_add(a, b); else return a + b; } };
+struct OpSub { template <typename A> __device__ static A f(A a, A b) { if constexpr (std::is_integral_v<A>) return wrap_sub(a, b); else return a - b; } };
+struct OpRSub { template <typename A> __device__ static A f(A a, A b) { return OpSub::f(b, a); } };
+struct OpMul { template <typename A> __device__ static A f(A a, A b) { if constexpr (std::is_integral_v<A>) return wrap_mul(a, b); else return a * b; } };
+struct OpDiv { template <typename A> __device__ static A f(A a, A b) { if constexpr (std::is_integral_v<A>) return wrap_div(a, b); else return a / b; } };
+struct OpRDiv { template <typename A> __device__ static A f(A a, A b) { return OpDiv::f(b, a); } };
+// std::max / std::min of the reference: (a<b)?b:a and (b<a)?b:a
+struct OpMax { template <typename A> __device__ static A f(A a, A b) { return (a < b) ? b : a; } };
+struct OpMin { template <typename A> __device__ static A f(A a, A b) { return (b < a) ? b : a; } };
+struct OpPow {
+    __device__ static float f(float a, float b) { return powf(a, b); }
+    __device__ static double f(double a, double b) { return pow(a, b); }
+};
+struct OpRPow { template <typename A> __device__ static A f(A a, A b) { return OpPow::f(b, a); } };
+
+struct OpSqrt { __device__ static float f(float a) { return sqrtf(a); } __device__ static double f(double a) { return sqrt(a); } };
+struct OpExp { __device__ static float f(float a) { return expf(a); } __device__ static double f(double a) { return exp(a); } };
+struct OpLog { __device__ static float f(float a) { return logf(a); } __device__ static double f(double a) { return log(a); } };
+struct OpSin { __device__ static float f(float a) { return sinf(a); } __device__ static double f(double a) { return sin(a); } };
+struct OpCos { __device__ static float f(float a) { return cosf(a); } __device__ static double f(double a) { return cos(a); } };
+struct OpTan { __device__ static float f(float a) { return tanf(a); } __device__ static double f(double a) { return tan(a); } };
+struct OpInvert {
+    template <typename A> __device__ static A f(A a) {
+        if constexpr (std::is_same_v<A, bool_t>) return bool_t{uint8_t(a.v ? 0 : 1)};
+        else return A(~a);
+    }
+};
+
+// ---- tile loop --------------------------------------------------------------------------
+// Calls body(vector_index) for every vector index in [0, nv), UNROLL*256 per workgroup trip.
+// `full` tiles run without bounds checks so the UNROLL loads issue back to back.
+template <int U, typename Body> __device__ inline void tile_loop(int64_t nv, Body body) {
+    const int64_t tile = (int64_t)kBlock * U;
+    const int64_t stride = (int64_t)gridDim.x * tile;
+    for (int64_t base = (int64_t)blockIdx.x * tile; base < nv; base += stride) {
+        if (base + tile <= nv) {
+            body(base + threadIdx.x, std::true_type{});
+        } else {
+            body(base + threadIdx.x, std::false_type{});
+        }
+    }
+}
+
+template <typename T, int V, typename Op>
+__global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a, const T *__restrict__ b,
+                                                         T *__restrict__ c, int64_t n) {
+    using VT = vec_t<T, V>;
+    using A = acc_t<T>;
+    const int64_t nv = n / V;
+    const VT *va = reinterpret_cast<const VT *>(a);
+    const VT *vb = reinterpret_cast<const VT *>(b);
+    VT *vc = reinterpret_cast<VT *>(c);
+    tile_loop<kUnroll>(nv, [&](int64_t i, auto full) {
+        VT x[kUnroll], y[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            int64_t j = i + u * kBlock;
+            if (decltype(full)::value || j < nv) { x[u] = va[j]; y[u] = vb[j]; }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            int64_t j = i + u * kBlock;
+            if (decltype(full)::value || j < nv) {
+                VT r;
+#pragma unroll
+                for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(A(load_acc(x[u].v[k])), A(load_acc(y[u].v[k]))));
+                vc[j] = r;
+            }
+        }
+    });
+    // scalar tail (n not a multiple of V)
+    if (blockIdx.x == 0) {
+        int64_t j = nv * V + threadIdx.x;
+        if (j < n) c[j] = store_acc<T>(Op::f(A(load_acc(a[j])), A(load_acc(b[j]))));
+    }
+}
+
+template <typename T, int V, typename Op>
+__global__ __launch_bounds__(kBlock) void scalar_kernel(const T *__restrict__ a, const T s, T *__restrict__ c, int64_t n) {
+    using VT = vec_t<T, V>;
+    using A = acc_t<T>;
+    const int64_t nv = n / V;
+    const A sv = load_acc(s);
+    const VT *va = reinterpret_cast<const VT *>(a);
+    VT *vc = reinterpret_cast<VT *>(c);
+    tile_loop<kUnroll>(nv, [&](int64_t i, auto full) {
+        VT x[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            int64_t j = i + u * kBlock;
+            if (decltype(full)::value || j < nv) x[u] = va[j];
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            int64_t j = i + u * kBlock;
+            if (decltype(full)::value || j < nv) {
+                VT r;
+#pragma unroll
+                for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(A(load_acc(x[u].v[k])), sv));
+                vc[j] = r;
+            }
+        }
+    });
+    if (blockIdx.x == 0) {
+        int64_t j = nv * V + threadIdx.x;
+        if (j < n) c[j] = store_acc<T>(Op::f(A(load_acc(a[j])), sv));
+    }
+}
+
+template <typename T, int V, typename Op>
+__global__ __launch_bounds__(kBlock) void unary_kernel(const T *__restrict__ a, T *__restrict__ c, int64_t n) {
+    using VT = vec_t<T, V>;
+    const int64_t nv = n / V;
+    const VT *va = reinterpret_cast<const VT *>(a);
+    VT *vc = reinterpret_cast<VT *>(c);
+    tile_loop<kUnroll>(nv, [&](int64_t i, auto full) {
+        VT x[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            int64_t j = i + u * kBlock;
+            if (decltype(full)::value || j < nv) x[u] = va[j];
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            int64_t j = i + u * kBlock;
+            if (decltype(full)::value || j < nv) {
+                VT r;
+#pragma unroll
+                for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(load_acc(x[u].v[k])));
+                vc[j] = r;
+            }
+        }
+    });
+    if (blockIdx.x == 0) {
+        int64_t j = nv * V + threadIdx.x;
+        if (j < n) c[j] = store_acc<T>(Op::f(load_acc(a[j])));
+    }
+}
+
+// ---- host launchers ---------------------------------------------------------------------
+template <typename T, typename Op>
+int launch_binary(const void *a, const void *b, void *c, int64_t n, hipStream_t st) {
+    if (!aligned(a, sizeof(T)) || !aligned(b, sizeof(T)) || !aligned(c, sizeof(T))) return DXH_ERR_ALIGN;
+    constexpr int V = vec_len<T>;
+    if (aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes)) {
+        unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnroll, kBlocksPerCU);
+        binary_kernel<T, V, Op><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n);
+    } else {
+        unsigned g = stream_grid(n, (int64_t)kBlock * kUnroll, kBlocksPerCU);
+        binary_kernel<T, 1, Op><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n);
+    }
+    return launch_status();
+}
+template <typename T, typename Op>
+int launch_scalar(const void *a, dxh_scalar s, void *c, int64_t n, hipStream_t st) {
+    if (!aligned(a, sizeof(T)) || !aligned(c, sizeof(T))) return DXH_ERR_ALIGN;
+    constexpr int V = vec_len<T>;
+    const T sv = scalar_to<T>(s);
+    if (aligned(a, kVecBytes) && aligned(c, kVecBytes)) {
+        unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnroll, kBlocksPerCU);
+        scalar_kernel<T, V, Op><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n);
+    } else {
+        unsigned g = stream_grid(n, (int64_t)kBlock * kUnroll, kBlocksPerCU);
+        scalar_kernel<T, 1, Op><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n);
+    }
+    return launch_status();
+}
+template <typename T, typename Op>
+int launch_unary(const void *a, void *c, int64_t n, hipStream_t st) {
+    if (!aligned(a, sizeof(T)) || !aligned(c, sizeof(T))) return DXH_ERR_ALIGN;
+    constexpr int V = vec_len<T>;
+    if (aligned(a, kVecBytes) && aligned(c, kVecBytes)) {
+        unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnroll, kBlocksPerCU);
+        unary_kernel<T, V, Op><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n);
+    } else {
+        unsigned g = stream_grid(n, (int64_t)kBlock * kUnroll, kBlocksPerCU);
+        unary_kernel<T, 1, Op><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n);
+    }
+    return launch_status();
+}
+
+template <typename Op> int binary_all(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream) {
+    DXH_CHECK_N(n);
+    DXH_CHECK_PTR(a); DXH_CHECK_PTR(b); DXH_CHECK_PTR(c);
+    hipStream_t st = as_stream(stream);
+    switch (dtype) {
+    case DXH_F64: return launch_binary<double, Op>(a, b, c, n, st);
+    case DXH_F32: return launch_binary<float, Op>(a, b, c, n, st);
+    case DXH_F16: return launch_binary<f16_t, Op>(a, b, c, n, st);
+    case DXH_BF16: return launch_binary<bf16_t, Op>(a, b, c, n, st);
+    case DXH_I64: return launch_binary<int64_t, Op>(a, b, c, n, st);
+    case DXH_I32: return launch_binary<int32_t, Op>(a, b, c, n, st);
+    case DXH_I16: return launch_binary<int16_t, Op>(a, b, c, n, st);
+    case DXH_I8: return launch_binary<int8_t, Op>(a, b, c, n, st);
+    default: return DXH_ERR_DTYPE;
+    }
+}
+template <typename Op> int scalar_all(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) {
+    DXH_CHECK_N(n);
+    DXH_CHECK_PTR(a); DXH_CHECK_PTR(c);
+    hipStream_t st = as_stream(stream);
+    switch (dtype) {
+    case DXH_F64: return launch_scalar<double, Op>(a, s, c, n, st);
+    case DXH_F32: return launch_scalar<float, Op>(a, s, c, n, st);
+    case DXH_F16: return launch_scalar<f16_t, Op>(a, s, c, n, st);
+    case DXH_BF16: return launch_scalar<bf16_t, Op>(a, s, c, n, st);
+    case DXH_I64: return launch_scalar<int64_t, Op>(a, s, c, n, st);
+    case DXH_I32: return launch_scalar<int32_t, Op>(a, s, c, n, st);
+    case DXH_I16: return launch_scalar<int16_t, Op>(a, s, c, n, st);
+    case DXH_I8: return launch_scalar<int8_t, Op>(a, s, c, n, st);
+    default: return DXH_ERR_DTYPE;
+    }
+}
+template <typename Op> int binary_f32f64(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream) {
+    DXH_CHECK_N(n);
+    DXH_CHECK_PTR(a); DXH_CHECK_PTR(b); DXH_CHECK_PTR(c);
+    switch (dtype) {
+    case DXH_F64: return launch_binary<double, Op>(a, b, c, n, as_stream(stream));
+    case DXH_F32: return launch_binary<float, Op>(a, b, c, n, as_stream(stream));
+    default: return DXH_ERR_DTYPE;
+    }
+}
+template <typename Op> int scalar_f32f64(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) {
+    DXH_CHECK_N(n);
+    DXH_CHECK_PTR(a); DXH_CHECK_PTR(c);
+    switch (dtype) {
+    case DXH_F64: return launch_scalar<double, Op>(a, s, c, n, as_stream(stream));
+    case DXH_F32: return launch_scalar<float, Op>(a, s, c, n, as_stream(stream));
+    default: return DXH_ERR_DTYPE;
+    }
+}
+template <typename Op, bool HALF> int unary_float(int dtype, const void *a, void *c, int64_t n, void *stream) {
+    DXH_CHECK_N(n);
+    DXH_CHECK_PTR(a); DXH_CHECK_PTR(c);
+    hipStream_t st = as_stream(stream);
+    switch (dtype) {
+    case DXH_F64: return launch_unary<double, Op>(a, c, n, st);
+    case DXH_F32: return launch_unary<float, Op>(a, c, n, st);
+    case DXH_F16: if constexpr (HALF) return launch_unary<f16_t, Op>(a, c, n, st); else return DXH_ERR_DTYPE;
+    case DXH_BF16: if constexpr (HALF) return launch_unary<bf16_t, Op>(a, c, n, st); else return DXH_ERR_DTYPE;
+    default: return DXH_ERR_DTYPE;
+    }
+}
+
+}  // namespace dxh
+
+using namespace dxh;
+
+extern "C" {
+
+int dxh_add(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream) { return binary_all<OpAdd>(dtype, a, b, c, n, stream); }
+int dxh_sub(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream) { return binary_all<OpSub>(dtype, a, b, c, n, stream); }
+int dxh_mul(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream) { return binary_all<OpMul>(dtype, a, b, c, n, stream); }
+int dxh_div(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream) { return binary_all<OpDiv>(dtype, a, b, c, n, stream); }
+int dxh_max(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream) { return binary_all<OpMax>(dtype, a, b, c, n, stream); }
+int dxh_min(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream) { return binary_all<OpMin>(dtype, a, b, c, n, stream); }
+int dxh_pow(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream) { return binary_f32f64<OpPow>(dtype, a, b, c, n, stream); }
+
+int dxh_addscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) { return scalar_all<OpAdd>(dtype, a, s, c, n, stream); }
+int dxh_subscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) { return scalar_all<OpSub>(dtype, a, s, c, n, stream); }
+int dxh_rsubscalar(int dtype, dxh_scalar s, const void *a, void *c, int64_t n, void *stream) { return scalar_all<OpRSub>(dtype, a, s, c, n, stream); }
+int dxh_mulscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) { return scalar_all<OpMul>(dtype, a, s, c, n, stream); }
+int dxh_divscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) { return scalar_all<OpDiv>(dtype, a, s, c, n, stream); }
+int dxh_rdivscalar(int dtype, dxh_scalar s, const void *a, void *c, int64_t n, void *stream) { return scalar_all<OpRDiv>(dtype, a, s, c, n, stream); }
+int dxh_maxscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) { return scalar_all<OpMax>(dtype, a, s, c, n, stream); }
+int dxh_minscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) { return scalar_all<OpMin>(dtype, a, s, c, n, stream); }
+int dxh_powscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) { return scalar_f32f64<OpPow>(dtype, a, s, c, n, stream); }
+int dxh_rpowscalar(int dtype, dxh_scalar s, const void *a, void *c, int64_t n, void *stream) { return scalar_f32f64<OpRPow>(dtype, a, s, c, n, stream); }
+
+int dxh_sqrt(int dtype, const void *a, void *c, int64_t n, void *stream) { return unary_float<OpSqrt, true>(dtype, a, c, n, stream); }
+int dxh_exp(int dtype, const void *a, void *c, int64_t n, void *stream) { return unary_float<OpExp, true>(dtype, a, c, n, stream); }
+int dxh_log(int dtype, const void *a, void *c, int64_t n, void *stream) { return unary_float<OpLog, true>(dtype, a, c, n, stream); }
+int dxh_sin(int dtype, const void *a, void *c, int64_t n, void *stream) { return unary_float<OpSin, true>(dtype, a, c, n, stream); }
+int dxh_cos(int dtype, const void *a, void *c, int64_t n, void *stream) { return unary_float<OpCos, true>(dtype, a, c, n, stream); }
+int dxh_tan(int dtype, const void *a, void *c, int64_t n, void *stream) { return unary_float<OpTan, false>(dtype, a, c, n, stream); }
+
+int dxh_invert(int dtype, const void *a, void *c, int64_t n, void *stream) {
+    DXH_CHECK_N(n);
+    DXH_CHECK_PTR(a); DXH_CHECK_PTR(c);
+    hipStream_t st = as_stream(stream);
+    switch (dtype) {
+    case DXH_I64: return launch_unary<int64_t, OpInvert>(a, c, n, st);
+    case DXH_I32: return launch_unary<int32_t, OpInvert>(a, c, n, st);
+    case DXH_I16: return launch_unary<int16_t, OpInvert>(a, c, n, st);
+    case DXH_I8: return launch_unary<int8_t, OpInvert>(a, c, n, st);
+    case DXH_BOOL: return launch_unary<bool_t, OpInvert>(a, c, n, st);
+    default: return DXH_ERR_DTYPE;
+    }
+}
+
+}  // extern "C"

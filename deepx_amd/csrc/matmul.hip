@@ -1,0 +1,238 @@
+// matmul.hip — batched row-major GEMM  C[b,m,n] = sum_k A[b,m,k] * B[b,k,n]  (gfx950).
+//
+// Replaces cublasSgemm(StridedBatched) of executor/op-cuda/src/deepx/tensorfunc/matmul_cublas.hpp:16-145
+// and cblas_sgemm of executor/op-ompsimd/src/deepx/tensorfunc/matmul_cblas.hpp:11-60 (alpha=1, beta=0).
+//
+//   bf16 / f16   MFMA v_mfma_f32_32x32x16_{bf16,f16}, fp32 accumulate, one RNE rounding of C.
+//                Workgroup tile 128x128x32, four waves in a 2x2 grid, each wave a 64x64 patch
+//                = 2x2 MFMA tiles.  A is staged in LDS k-contiguous; B arrives n-contiguous
+//                (row-major [K,N]) and is transposed on the way into LDS so that both MFMA
+//                operands are read as one 16-byte ds_read per lane.
+//   f32 / f64 / integers   LDS-tiled 64x64x16 FMA kernel, 4x4 outputs per lane; accumulate in
+//                the storage type (integers wrap).
+#include "common.hpp"
+
+namespace dxh {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128, BK = 32;
+constexpr int LDK = BK + 8;  // padded k-stride (elements) of both LDS tiles: 80 bytes, keeps 16-byte alignment
+
+template <typename T> __device__ inline f32x16 mfma32(uint4 a, uint4 b, f32x16 c) {
+    if constexpr (std::is_same_v<T, bf16_t>)
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+// VEC_A: rows of A are 16-byte aligned (K % 8 == 0, base aligned); VEC_B likewise for B (N % 8 == 0).
+template <typename T, bool VEC_A, bool VEC_B>
+__global__ __launch_bounds__(kBlock) void matmul_mfma_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
+                                                              int M, int K, int N, int tiles_m, int tiles_n) {
+    __shared__ __attribute__((aligned(16))) uint16_t As[BM * LDK];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[BN * LDK];  // transposed: [n][k]
+    int64_t bid = blockIdx.x;
+    const int tn = (int)(bid % tiles_n); bid /= tiles_n;
+    const int tm = (int)(bid % tiles_m); bid /= tiles_m;
+    const int64_t batch = bid;
+    A += batch * (int64_t)M * K;
+    B += batch * (int64_t)K * N;
+    C += batch * (int64_t)M * N;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+    const int wm = w >> 1, wn = w & 1;
+    const uint16_t *Ar = reinterpret_cast<const uint16_t *>(A);
+    const uint16_t *Br = reinterpret_cast<const uint16_t *>(B);
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        // ---- A tile: 128 rows x 32 k, 16 bytes (8 k) per lane, two rows per lane
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int r = (t >> 2) + h * 64, kc = (t & 3) * 8;
+            const int gm = m0 + r, gk = k0 + kc;
+            vec_t<uint16_t, 8> x;
+            if (VEC_A && gm < M && gk + 8 <= K) {
+                x = *reinterpret_cast<const vec_t<uint16_t, 8> *>(Ar + (int64_t)gm * K + gk);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) x.v[j] = (gm < M && gk + j < K) ? Ar[(int64_t)gm * K + gk + j] : (uint16_t)0;
+            }
+            *reinterpret_cast<vec_t<uint16_t, 8> *>(&As[r * LDK + kc]) = x;
+        }
+        // ---- B tile: 32 k x 128 n, 16 bytes (8 n) per lane, transposed into Bs[n][k]
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int kr = (t >> 4) + h * 16, nc = (t & 15) * 8;
+            const int gk = k0 + kr, gn = n0 + nc;
+            vec_t<uint16_t, 8> x;
+            if (VEC_B && gk < K && gn + 8 <= N) {
+                x = *reinterpret_cast<const vec_t<uint16_t, 8> *>(Br + (int64_t)gk * N + gn);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) x.v[j] = (gk < K && gn + j < N) ? Br[(int64_t)gk * N + gn + j] : (uint16_t)0;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) Bs[(nc + j) * LDK + kr] = x.v[j];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 16) {
+            uint4 af[2], bf[2];
+            const int ko = kk + (lane >> 5) * 8;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) af[i] = *reinterpret_cast<const uint4 *>(&As[(wm * 64 + i * 32 + (lane & 31)) * LDK + ko]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) bf[j] = *reinterpret_cast<const uint4 *>(&Bs[(wn * 64 + j * 32 + (lane & 31)) * LDK + ko]);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = mfma32<T>(af[i], bf[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+    // ---- epilogue: D[row][col], col = lane%32, row = 8*(v/4) + 4*(lane/32) + v%4
+    uint16_t *Cr = reinterpret_cast<uint16_t *>(C);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = m0 + wm * 64 + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+                if (row < M && col < N) Cr[(int64_t)row * N + col] = store_acc<T>(acc[i][j][v]).bits;
+            }
+}
+
+// ---- generic tiled kernel (f32, f64, integers) ------------------------------------------
+constexpr int GT = 64, GK = 16;
+template <typename T>
+__global__ __launch_bounds__(kBlock) void matmul_tiled_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
+                                                               int M, int K, int N, int tiles_m, int tiles_n) {
+    __shared__ T As[GK][GT + 1];  // [k][m]
+    __shared__ T Bs[GK][GT + 1];  // [k][n]
+    int64_t bid = blockIdx.x;
+    const int tn = (int)(bid % tiles_n); bid /= tiles_n;
+    const int tm = (int)(bid % tiles_m); bid /= tiles_m;
+    A += bid * (int64_t)M * K;
+    B += bid * (int64_t)K * N;
+    C += bid * (int64_t)M * N;
+    const int m0 = tm * GT, n0 = tn * GT;
+    const int t = threadIdx.x, tx = t & 15, ty = t >> 4;
+    T acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = T(0);
+    for (int k0 = 0; k0 < K; k0 += GK) {
+        // A tile 64x16: lanes along k (contiguous), 4 rows per lane
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+            const int r = (t >> 4) + h * 16, kc = t & 15;
+            const int gm = m0 + r, gk = k0 + kc;
+            As[kc][r] = (gm < M && gk < K) ? A[(int64_t)gm * K + gk] : T(0);
+        }
+        // B tile 16x64: lanes along n (contiguous), 4 k-rows per lane
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+            const int kr = (t >> 6) + h * 4, nc = t & 63;
+            const int gk = k0 + kr, gn = n0 + nc;
+            Bs[kr][nc] = (gk < K && gn < N) ? B[(int64_t)gk * N + gn] : T(0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < GK; ++kk) {
+            T a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = Bs[kk][tx + j * 16];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if constexpr (std::is_integral_v<T>) {
+                        using U = std::conditional_t<(sizeof(T) < 4), uint32_t, std::make_unsigned_t<T>>;
+                        acc[i][j] = T(U(U(acc[i][j]) + U(U(a[i]) * U(b[j]))));
+                    } else {
+                        acc[i][j] = __builtin_fma(a[i], b[j], acc[i][j]);
+                    }
+                }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = m0 + ty * 4 + i, col = n0 + tx + j * 16;
+            if (row < M && col < N) C[(int64_t)row * N + col] = acc[i][j];
+        }
+}
+
+template <typename T>
+int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
+    const int64_t blocks = batch * tiles_m * tiles_n;
+    if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
+    const bool va = (k % 8 == 0) && aligned(a, kVecBytes);
+    const bool vb = (n % 8 == 0) && aligned(b, kVecBytes);
+#define DXH_MM(VA, VB) matmul_mfma_kernel<T, VA, VB><<<(unsigned)blocks, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n)
+    if (va && vb) DXH_MM(true, true);
+    else if (va) DXH_MM(true, false);
+    else if (vb) DXH_MM(false, true);
+    else DXH_MM(false, false);
+#undef DXH_MM
+    return launch_status();
+}
+template <typename T>
+int launch_tiled(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    const int64_t tiles_m = (m + GT - 1) / GT, tiles_n = (n + GT - 1) / GT;
+    const int64_t blocks = batch * tiles_m * tiles_n;
+    if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
+    matmul_tiled_kernel<T><<<(unsigned)blocks, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
+    return launch_status();
+}
+
+}  // namespace dxh
+
+using namespace dxh;
+
+extern "C" int dxh_matmul(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n,
+                          void *stream) {
+    if (batch < 0 || m < 0 || k < 0 || n < 0) return DXH_ERR_ARG;
+    if (m > 0x7fffffff || k > 0x7fffffff || n > 0x7fffffff) return DXH_ERR_SHAPE;
+    const int es = dtype_size(dtype);
+    if (!es || dtype == DXH_BOOL) return DXH_ERR_DTYPE;
+    if (batch * m * n == 0) return DXH_OK;
+    if (!c) return DXH_ERR_ARG;
+    hipStream_t st = as_stream(stream);
+    if (k == 0) {  // empty sum: a fill kernel rather than a memset node, so the call stays graph-capturable
+        dxh_scalar zero = {0.0, 0};
+        return dxh_constant(dtype, c, batch * m * n, zero, stream);
+    }
+    if (!a || !b) return DXH_ERR_ARG;
+    if (!aligned(a, es) || !aligned(b, es) || !aligned(c, es)) return DXH_ERR_ALIGN;
+    switch (dtype) {
+    case DXH_BF16: return launch_mfma<bf16_t>(a, b, c, batch, m, k, n, st);
+    case DXH_F16: return launch_mfma<f16_t>(a, b, c, batch, m, k, n, st);
+    case DXH_F32: return launch_tiled<float>(a, b, c, batch, m, k, n, st);
+    case DXH_F64: return launch_tiled<double>(a, b, c, batch, m, k, n, st);
+    case DXH_I64: return launch_tiled<int64_t>(a, b, c, batch, m, k, n, st);
+    case DXH_I32: return launch_tiled<int32_t>(a, b, c, batch, m, k, n, st);
+    case DXH_I16: return launch_tiled<int16_t>(a, b, c, batch, m, k, n, st);
+    case DXH_I8: return launch_tiled<int8_t>(a, b, c, batch, m, k, n, st);
+    default: return DXH_ERR_DTYPE;
+    }
+}

@@ -1,0 +1,462 @@
+// reduce.hip — sum / prod / reducemax / reducemin over arbitrary axes (gfx950).
+//
+// Semantics: executor/op-ompsimd/src/deepx/tensorfunc/reduce_miaobyte.hpp:19-345 with the
+// axis handling of executor/deepxcore/src/deepx/shape_reduce.cpp:11-85.  The reference
+// visits every input element and accumulates into the output under an atomic; here the
+// shape is first canonicalised (size-1 axes dropped, neighbouring axes of equal
+// kept/reduced status merged), then reduced axis-group by axis-group, last group first:
+//
+//   row stage   [pre, R]        R contiguous: a group of G lanes (G = 1..64, or the whole
+//                               256-thread workgroup) owns one row chunk; 16-byte loads,
+//                               V independent accumulators per lane, wave shuffle
+//                               reduction, LDS across the four waves.
+//   col stage   [pre, R, post]  R strided: lanes run along `post` (coalesced 16-byte
+//                               loads), TY row-lanes per workgroup walk R, LDS tree
+//                               across the row-lanes.
+//
+// When a stage has too few workgroups to fill 256 CUs, R is split into S chunks whose
+// partials ([pre, S, post], accumulate type) go to the caller's workspace and are reduced
+// by one more stage; results are deterministic (no atomics).  Both stage kinds are
+// HBM-bound: algorithmic bytes = input once + output once.
+#include "common.hpp"
+#include <limits>
+#include <vector>
+
+namespace dxh {
+
+enum RedKind { R_SUM = 0, R_PROD = 1, R_MAX = 2, R_MIN = 3 };
+
+template <typename T> struct racc_of { using type = T; };
+template <> struct racc_of<bf16_t> { using type = float; };
+template <> struct racc_of<f16_t> { using type = float; };
+template <> struct racc_of<int16_t> { using type = int32_t; };
+template <> struct racc_of<int8_t> { using type = int32_t; };
+template <typename T> using racc_t = typename racc_of<T>::type;
+
+template <typename A, typename T> __device__ inline A rload(T x) {
+    if constexpr (std::is_same_v<T, bf16_t> || std::is_same_v<T, f16_t>) return load_acc(x);
+    else return A(x);
+}
+template <typename T, typename A> __device__ inline T rstore(A v) {
+    if constexpr (std::is_same_v<T, bf16_t>) return to_bf16(v);
+    else if constexpr (std::is_same_v<T, f16_t>) return to_f16(v);
+    else return T(v);  // integers truncate: wrap-around arithmetic is width independent
+}
+
+// identity element: 0 / 1 / lowest() / max() of the STORAGE type, as the reference
+// pre-fills the result (reduce_miaobyte.hpp:24,101,191,274)
+template <int K, typename A, typename TS> __host__ __device__ inline A rinit() {
+    if constexpr (K == R_SUM) return A(0);
+    else if constexpr (K == R_PROD) return A(1);
+    else if constexpr (std::is_same_v<TS, bf16_t>) return K == R_MAX ? -3.3895313892515355e38f : 3.3895313892515355e38f;
+    else if constexpr (std::is_same_v<TS, f16_t>) return K == R_MAX ? -65504.0f : 65504.0f;
+    else return K == R_MAX ? A(std::numeric_limits<TS>::lowest()) : A(std::numeric_limits<TS>::max());
+}
+template <int K, typename A> __device__ inline A rop(A a, A b) {
+    if constexpr (K == R_SUM) {
+        if constexpr (std::is_integral_v<A>) { using U = std::make_unsigned_t<A>; return A(U(a) + U(b)); }
+        else return a + b;
+    } else if constexpr (K == R_PROD) {
+        if constexpr (std::is_integral_v<A>) { using U = std::make_unsigned_t<A>; return A(U(a) * U(b)); }
+        else return a * b;
+    } else if constexpr (K == R_MAX) return (a < b) ? b : a;
+    else return (b < a) ? b : a;
+}
+
+template <typename A> __device__ inline A shfl_xor_any(A v, int off) {
+    if constexpr (sizeof(A) == 8) {
+        uint64_t u = __builtin_bit_cast(uint64_t, v);
+        uint32_t lo = __shfl_xor((int)(uint32_t)u, off, kWave);
+        uint32_t hi = __shfl_xor((int)(uint32_t)(u >> 32), off, kWave);
+        return __builtin_bit_cast(A, (uint64_t(hi) << 32) | lo);
+    } else {
+        return __builtin_bit_cast(A, __shfl_xor(__builtin_bit_cast(int, v), off, kWave));
+    }
+}
+
+// ---- row stage ---------------------------------------------------------------------------
+// in [pre, R] (R contiguous) -> out [pre, S]; chunk s covers r in [s*chunk, min(R,(s+1)*chunk)).
+// G lanes cooperate on one (row, chunk); G in {1,2,..,64} packs 256/G rows per workgroup,
+// G == 256 gives the whole workgroup to one row.
+template <int K, typename Tin, typename Tout, typename TS, int V>
+__global__ __launch_bounds__(kBlock) void reduce_row_kernel(const Tin *__restrict__ in, Tout *__restrict__ out,
+                                                             int64_t pre, int64_t R, int S, int64_t chunk, int G) {
+    using A = racc_t<TS>;
+    using VT = vec_t<Tin, V>;
+    __shared__ A lds[kBlock / kWave];
+    const int rows_per_block = kBlock / G;
+    const int lane = threadIdx.x % G;
+    const int64_t row = (int64_t)blockIdx.x * rows_per_block + threadIdx.x / G;
+    const int s = blockIdx.y;
+    const bool active = row < pre;
+    A acc[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) acc[k] = rinit<K, A, TS>();
+    if (active) {
+        const int64_t r0 = (int64_t)s * chunk;
+        const int64_t r1 = (r0 + chunk < R) ? r0 + chunk : R;
+        const int64_t len = r1 - r0;
+        const Tin *p = in + row * R + r0;
+        const VT *pv = reinterpret_cast<const VT *>(p);
+        const int64_t lv = len / V;
+        int64_t i = lane;
+        for (; i + 3 * (int64_t)G < lv; i += 4 * (int64_t)G) {
+            VT x0 = pv[i], x1 = pv[i + G], x2 = pv[i + 2 * (int64_t)G], x3 = pv[i + 3 * (int64_t)G];
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                A t0 = rop<K, A>(rload<A>(x0.v[k]), rload<A>(x1.v[k]));
+                A t1 = rop<K, A>(rload<A>(x2.v[k]), rload<A>(x3.v[k]));
+                acc[k] = rop<K, A>(acc[k], rop<K, A>(t0, t1));
+            }
+        }
+        for (; i < lv; i += G) {
+            VT x = pv[i];
+#pragma unroll
+            for (int k = 0; k < V; ++k) acc[k] = rop<K, A>(acc[k], rload<A>(x.v[k]));
+        }
+        for (int64_t j = lv * V + lane; j < len; j += G) acc[0] = rop<K, A>(acc[0], rload<A>(p[j]));
+    }
+    A v = acc[0];
+#pragma unroll
+    for (int k = 1; k < V; ++k) v = rop<K, A>(v, acc[k]);
+    // lanes of one group are adjacent, so xor-shuffles below G stay inside the group
+    const int gw = G < kWave ? G : kWave;
+    for (int off = gw >> 1; off > 0; off >>= 1) v = rop<K, A>(v, shfl_xor_any<A>(v, off));
+    if (G == kBlock) {
+        if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = v;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            A r = lds[0];
+#pragma unroll
+            for (int w = 1; w < kBlock / kWave; ++w) r = rop<K, A>(r, lds[w]);
+            if (active) out[row * S + s] = rstore<Tout, A>(r);
+        }
+    } else if (lane == 0 && active) {
+        out[row * S + s] = rstore<Tout, A>(v);
+    }
+}
+
+// ---- col stage ---------------------------------------------------------------------------
+// in [pre, R, post] -> out [pre, S, post].  Workgroup = TX column-lanes x TY row-lanes
+// (TX*TY == 256); a column-lane owns V adjacent columns.  Linear block id -> (p, s, ctile).
+template <int K, typename Tin, typename Tout, typename TS, int V>
+__global__ __launch_bounds__(kBlock) void reduce_col_kernel(const Tin *__restrict__ in, Tout *__restrict__ out,
+                                                             int64_t pre, int64_t R, int64_t post, int S, int64_t chunk,
+                                                             int TX, int ctiles) {
+    using A = racc_t<TS>;
+    using VT = vec_t<Tin, V>;
+    __shared__ A lds[kBlock * V];
+    const int TY = kBlock / TX;
+    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+    int64_t b = blockIdx.x;
+    const int ct = (int)(b % ctiles); b /= ctiles;
+    const int s = (int)(b % S);
+    const int64_t p = b / S;
+    const int64_t postv = post / V;  // launcher guarantees post % V == 0
+    const int64_t cv = (int64_t)ct * TX + tx;
+    const bool active = cv < postv;
+    A acc[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) acc[k] = rinit<K, A, TS>();
+    if (active) {
+        const int64_t r0 = (int64_t)s * chunk;
+        const int64_t r1 = (r0 + chunk < R) ? r0 + chunk : R;
+        const VT *base = reinterpret_cast<const VT *>(in + p * R * post) + cv;
+        int64_t r = r0 + ty;
+        for (; r + 3 * (int64_t)TY < r1; r += 4 * (int64_t)TY) {
+            VT x0 = base[r * postv], x1 = base[(r + TY) * postv], x2 = base[(r + 2 * TY) * postv], x3 = base[(r + 3 * TY) * postv];
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                A t0 = rop<K, A>(rload<A>(x0.v[k]), rload<A>(x1.v[k]));
+                A t1 = rop<K, A>(rload<A>(x2.v[k]), rload<A>(x3.v[k]));
+                acc[k] = rop<K, A>(acc[k], rop<K, A>(t0, t1));
+            }
+        }
+        for (; r < r1; r += TY) {
+            VT x = base[r * postv];
+#pragma unroll
+            for (int k = 0; k < V; ++k) acc[k] = rop<K, A>(acc[k], rload<A>(x.v[k]));
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < V; ++k) lds[(k * TY + ty) * TX + tx] = acc[k];
+    __syncthreads();
+    for (int h = TY >> 1; h > 0; h >>= 1) {
+        if (ty < h) {
+#pragma unroll
+            for (int k = 0; k < V; ++k)
+                lds[(k * TY + ty) * TX + tx] = rop<K, A>(lds[(k * TY + ty) * TX + tx], lds[(k * TY + ty + h) * TX + tx]);
+        }
+        __syncthreads();
+    }
+    if (ty == 0 && active) {
+        Tout *o = out + (p * S + s) * post + cv * V;
+#pragma unroll
+        for (int k = 0; k < V; ++k) o[k] = rstore<Tout, A>(lds[(k * TY) * TX + tx]);
+    }
+}
+
+// fill `n` outputs with the identity (a reduced axis of size 0), or copy (nothing to reduce)
+template <int K, typename TS>
+__global__ __launch_bounds__(kBlock) void reduce_fill_kernel(TS *__restrict__ out, int64_t n) {
+    using A = racc_t<TS>;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) out[i] = rstore<TS, A>(rinit<K, A, TS>());
+}
+
+// ---- host-side plan ----------------------------------------------------------------------
+struct Stage {
+    bool row;            // row stage (post == 1) or col stage
+    int64_t pre, R, post;
+    int S;               // chunks of R
+    int64_t chunk;
+    int G;               // row: lanes per row
+    int TX, ctiles;      // col: column lanes, column tiles
+    int V;               // vector length in elements of the stage's input type (1 or 16/size)
+    bool in_is_acc, out_is_acc;
+    size_t out_off;      // offset of the output inside the workspace when out_is_acc
+};
+struct Plan {
+    int64_t nout = 0, nred = 1;
+    bool copy_only = false;
+    std::vector<Stage> stages;
+    size_t ws_bytes = 0;
+};
+
+inline int pow2_ceil(int64_t x) { int p = 1; while (p < x && p < (1 << 30)) p <<= 1; return p; }
+constexpr int kTargetBlocks = 4 * kCUs;
+
+// normalise dims like checkedDims (shape_reduce.cpp:11-45); returns false if out of range
+inline bool reduced_mask(int ndim, const int32_t *dims, int ndims, bool *mask) {
+    for (int i = 0; i < ndim; ++i) mask[i] = (ndims == 0);
+    for (int i = 0; i < ndims; ++i) {
+        int d = dims[i];
+        if (d < 0) d += ndim;
+        if (d < 0 || d >= ndim) return false;
+        mask[d] = true;
+    }
+    return true;
+}
+
+inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, const int32_t *dims, int ndims, Plan &pl) {
+    if (!shape || ndim < 1 || ndim > DXH_MAX_DIMS || ndims < 0 || (ndims > 0 && !dims)) return DXH_ERR_ARG;
+    bool mask[DXH_MAX_DIMS];
+    if (!reduced_mask(ndim, dims, ndims, mask)) return DXH_ERR_ARG;
+    struct D { int64_t n; bool red; };
+    std::vector<D> d;
+    pl.nout = 1; pl.nred = 1;
+    for (int i = 0; i < ndim; ++i) {
+        if (shape[i] < 0) return DXH_ERR_ARG;
+        if (mask[i]) pl.nred *= shape[i]; else pl.nout *= shape[i];
+        if (shape[i] == 1) continue;
+        if (!d.empty() && d.back().red == mask[i]) d.back().n *= shape[i];
+        else d.push_back({shape[i], mask[i]});
+    }
+    if (pl.nout == 0 || pl.nred == 0) return DXH_OK;  // nothing to read
+    bool any = false;
+    for (auto &x : d) any |= x.red;
+    if (!any) { pl.copy_only = true; return DXH_OK; }
+
+    bool first = true;
+    size_t off = 0;
+    auto push = [&](Stage st, bool last) {
+        st.in_is_acc = !first;
+        st.out_is_acc = !last;
+        const int in_size = st.in_is_acc ? asize : esize;
+        const int vfull = kVecBytes / in_size;
+        if (st.row) {
+            // vector loads need every row chunk to start on a 16-byte boundary
+            st.V = (st.R % vfull == 0 && st.chunk % vfull == 0) ? vfull : 1;
+        } else {
+            st.V = (st.post % vfull == 0) ? vfull : 1;
+            int64_t postv = st.post / st.V;
+            st.TX = (int)std::min<int64_t>(64, pow2_ceil(postv));
+            st.ctiles = (int)((postv + st.TX - 1) / st.TX);
+        }
+        if (st.out_is_acc) {
+            st.out_off = off;
+            size_t bytes = (size_t)(st.pre * st.S * st.post) * asize;
+            off += (bytes + 255) & ~(size_t)255;
+        }
+        pl.stages.push_back(st);
+        first = false;
+    };
+
+    while (true) {
+        int p = -1, groups = 0;
+        for (int i = 0; i < (int)d.size(); ++i) if (d[i].red) { p = i; ++groups; }
+        if (p < 0) break;
+        int64_t pre = 1, post = 1;
+        for (int i = 0; i < p; ++i) pre *= d[i].n;
+        for (int i = p + 1; i < (int)d.size(); ++i) post *= d[i].n;
+        const int64_t R = d[p].n;
+        const bool last_group = groups == 1;
+        Stage st{};
+        st.pre = pre; st.R = R; st.post = post; st.row = (post == 1);
+        const int in_size = pl.stages.empty() ? esize : asize;
+        const int vfull = kVecBytes / in_size;
+        int S = 1;
+        if (st.row) {
+            // lanes per row: one 16-byte vector per lane per trip, up to the whole workgroup
+            int64_t vecs = (R + vfull - 1) / vfull;
+            int G = vecs >= 2 * kWave ? kBlock : (int)std::min<int64_t>(kWave, pow2_ceil(vecs));
+            int64_t blocks0 = (pre + (kBlock / G) - 1) / (kBlock / G);
+            if (G == kBlock && blocks0 < kTargetBlocks) {
+                int64_t min_chunk = 8192;  // elements: 8+ vector trips per lane
+                int64_t smax = std::max<int64_t>(1, R / min_chunk);
+                S = (int)std::min<int64_t>((kTargetBlocks + blocks0 - 1) / blocks0, smax);
+            }
+            st.G = G;
+        } else {
+            int V = (post % vfull == 0) ? vfull : 1;
+            int64_t postv = post / V;
+            int TX = (int)std::min<int64_t>(64, pow2_ceil(postv));
+            int TY = kBlock / TX;
+            int64_t blocks0 = pre * ((postv + TX - 1) / TX);
+            if (blocks0 < kTargetBlocks) {
+                int64_t min_rows = (int64_t)TY * 16;
+                int64_t smax = std::max<int64_t>(1, R / min_rows);
+                S = (int)std::min<int64_t>((kTargetBlocks + blocks0 - 1) / blocks0, smax);
+            }
+        }
+        st.S = S;
+        int64_t chunk = (R + S - 1) / S;
+        chunk = (chunk + vfull - 1) / vfull * vfull;  // keep chunk starts vector aligned
+        st.chunk = chunk;
+        st.S = (int)((R + chunk - 1) / chunk);
+        push(st, last_group && st.S == 1);
+        if (st.S > 1) {
+            // second pass over the S partials: [pre, S, post]
+            Stage s2{};
+            s2.pre = pre; s2.R = st.S; s2.post = post; s2.row = (post == 1); s2.S = 1; s2.chunk = st.S;
+            if (s2.row) {
+                int64_t vecs = (s2.R + (kVecBytes / asize) - 1) / (kVecBytes / asize);
+                s2.G = vecs >= 2 * kWave ? kBlock : (int)std::min<int64_t>(kWave, pow2_ceil(vecs));
+            }
+            push(s2, last_group);
+        }
+        // drop the reduced group and re-merge the kept neighbours
+        d.erase(d.begin() + p);
+        if (p > 0 && p < (int)d.size() && !d[p - 1].red && !d[p].red) { d[p - 1].n *= d[p].n; d.erase(d.begin() + p); }
+    }
+    pl.ws_bytes = off;
+    return DXH_OK;
+}
+
+template <int K, typename Tin, typename Tout, typename TS>
+int launch_stage(const Stage &st, const void *in, void *out, hipStream_t stream) {
+    constexpr int VF = kVecBytes / (int)sizeof(Tin);
+    if (st.row) {
+        const int rows_per_block = kBlock / st.G;
+        int64_t gx = (st.pre + rows_per_block - 1) / rows_per_block;
+        if (gx > 0x7fffffff || st.S > 65535) return DXH_ERR_SHAPE;
+        dim3 grid((unsigned)gx, (unsigned)st.S);
+        if (st.V == VF && aligned(in, kVecBytes))
+            reduce_row_kernel<K, Tin, Tout, TS, VF><<<grid, kBlock, 0, stream>>>((const Tin *)in, (Tout *)out, st.pre, st.R, st.S, st.chunk, st.G);
+        else
+            reduce_row_kernel<K, Tin, Tout, TS, 1><<<grid, kBlock, 0, stream>>>((const Tin *)in, (Tout *)out, st.pre, st.R, st.S, st.chunk, st.G);
+    } else {
+        bool vec = st.V == VF && aligned(in, kVecBytes);
+        int TX = st.TX, ctiles = st.ctiles;
+        if (!vec && st.V != 1) {  // planned for vectors but the pointer is misaligned
+            TX = (int)std::min<int64_t>(64, pow2_ceil(st.post));
+            ctiles = (int)((st.post + TX - 1) / TX);
+        }
+        int64_t gx = st.pre * st.S * ctiles;
+        if (gx > 0x7fffffff) return DXH_ERR_SHAPE;
+        if (vec)
+            reduce_col_kernel<K, Tin, Tout, TS, VF><<<(unsigned)gx, kBlock, 0, stream>>>((const Tin *)in, (Tout *)out, st.pre, st.R, st.post, st.S, st.chunk, TX, ctiles);
+        else
+            reduce_col_kernel<K, Tin, Tout, TS, 1><<<(unsigned)gx, kBlock, 0, stream>>>((const Tin *)in, (Tout *)out, st.pre, st.R, st.post, st.S, st.chunk, TX, ctiles);
+    }
+    return launch_status();
+}
+
+template <int K, typename TS>
+int reduce_typed(const void *in, const int32_t *shape, int ndim, const int32_t *dims, int ndims, void *out,
+                 void *workspace, size_t workspace_bytes, hipStream_t stream) {
+    using A = racc_t<TS>;
+    Plan pl;
+    int rc = build_plan(sizeof(TS), sizeof(A), shape, ndim, dims, ndims, pl);
+    if (rc != DXH_OK) return rc;
+    if (pl.nout == 0) return DXH_OK;
+    if (!out) return DXH_ERR_ARG;
+    if (!aligned(out, sizeof(TS))) return DXH_ERR_ALIGN;
+    if (pl.nred == 0) {
+        reduce_fill_kernel<K, TS><<<stream_grid(pl.nout, kBlock, 8), kBlock, 0, stream>>>((TS *)out, pl.nout);
+        return launch_status();
+    }
+    if (!in) return DXH_ERR_ARG;
+    if (!aligned(in, sizeof(TS))) return DXH_ERR_ALIGN;
+    if (pl.copy_only) {
+        if (in == out) return DXH_OK;
+        return (int)hipMemcpyAsync(out, in, (size_t)pl.nout * sizeof(TS), hipMemcpyDeviceToDevice, stream);
+    }
+    if (pl.ws_bytes > 0 && (!workspace || workspace_bytes < pl.ws_bytes || !aligned(workspace, 256))) return DXH_ERR_WORKSPACE;
+    const void *cur = in;
+    for (const Stage &st : pl.stages) {
+        void *dst = st.out_is_acc ? (void *)((char *)workspace + st.out_off) : out;
+        if (!st.in_is_acc && !st.out_is_acc) rc = launch_stage<K, TS, TS, TS>(st, cur, dst, stream);
+        else if (!st.in_is_acc && st.out_is_acc) rc = launch_stage<K, TS, A, TS>(st, cur, dst, stream);
+        else if (st.in_is_acc && st.out_is_acc) rc = launch_stage<K, A, A, TS>(st, cur, dst, stream);
+        else rc = launch_stage<K, A, TS, TS>(st, cur, dst, stream);
+        if (rc != DXH_OK) return rc;
+        cur = dst;
+    }
+    return DXH_OK;
+}
+
+template <int K>
+int reduce_all(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims, int ndims, void *out,
+               void *ws, size_t wsb, void *stream) {
+    hipStream_t st = as_stream(stream);
+    switch (dtype) {
+    case DXH_F64: return reduce_typed<K, double>(in, shape, ndim, dims, ndims, out, ws, wsb, st);
+    case DXH_F32: return reduce_typed<K, float>(in, shape, ndim, dims, ndims, out, ws, wsb, st);
+    case DXH_F16: return reduce_typed<K, f16_t>(in, shape, ndim, dims, ndims, out, ws, wsb, st);
+    case DXH_BF16: return reduce_typed<K, bf16_t>(in, shape, ndim, dims, ndims, out, ws, wsb, st);
+    case DXH_I64: return reduce_typed<K, int64_t>(in, shape, ndim, dims, ndims, out, ws, wsb, st);
+    case DXH_I32: return reduce_typed<K, int32_t>(in, shape, ndim, dims, ndims, out, ws, wsb, st);
+    case DXH_I16: return reduce_typed<K, int16_t>(in, shape, ndim, dims, ndims, out, ws, wsb, st);
+    case DXH_I8: return reduce_typed<K, int8_t>(in, shape, ndim, dims, ndims, out, ws, wsb, st);
+    default: return DXH_ERR_DTYPE;
+    }
+}
+
+}  // namespace dxh
+
+using namespace dxh;
+
+extern "C" {
+
+int dxh_reduce_workspace_bytes(int dtype, const int32_t *shape, int ndim, const int32_t *dims, int ndims, size_t *bytes) {
+    if (!bytes) return DXH_ERR_ARG;
+    *bytes = 0;
+    int es = dtype_size(dtype);
+    if (!es || dtype == DXH_BOOL) return DXH_ERR_DTYPE;
+    int as = (dtype == DXH_F64 || dtype == DXH_I64) ? 8 : 4;
+    Plan pl;
+    int rc = build_plan(es, as, shape, ndim, dims, ndims, pl);
+    if (rc != DXH_OK) return rc;
+    *bytes = pl.ws_bytes;
+    return DXH_OK;
+}
+
+int dxh_sum(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims, int ndims, void *out,
+            void *workspace, size_t workspace_bytes, void *stream) {
+    return reduce_all<R_SUM>(dtype, in, shape, ndim, dims, ndims, out, workspace, workspace_bytes, stream);
+}
+int dxh_prod(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims, int ndims, void *out,
+             void *workspace, size_t workspace_bytes, void *stream) {
+    return reduce_all<R_PROD>(dtype, in, shape, ndim, dims, ndims, out, workspace, workspace_bytes, stream);
+}
+int dxh_reducemax(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims, int ndims, void *out,
+                  void *workspace, size_t workspace_bytes, void *stream) {
+    return reduce_all<R_MAX>(dtype, in, shape, ndim, dims, ndims, out, workspace, workspace_bytes, stream);
+}
+int dxh_reducemin(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims, int ndims, void *out,
+                  void *workspace, size_t workspace_bytes, void *stream) {
+    return reduce_all<R_MIN>(dtype, in, shape, ndim, dims, ndims, out, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,107 @@
+// runtime.hip — device memory, copies, streams and events behind the C ABI.
+// Replaces the cudaMalloc/cudaFree/cudaMemcpy calls of
+// executor/op-cuda/src/deepx/tensorfunc/tensorlife_miaobyte.hpp:16-68.
+#include "common.hpp"
+#include <cstdio>
+#include <cstring>
+
+using namespace dxh;
+
+extern "C" {
+
+int dxh_version(void) { return 100; }
+
+const char *dxh_error_string(int code) {
+    switch (code) {
+    case DXH_OK: return "ok";
+    case DXH_ERR_DTYPE: return "dtype not supported by this op";
+    case DXH_ERR_ARG: return "invalid argument";
+    case DXH_ERR_SHAPE: return "shape mismatch";
+    case DXH_ERR_WORKSPACE: return "workspace missing or too small";
+    case DXH_ERR_ALIGN: return "pointer not aligned to its element size";
+    default: break;
+    }
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "unknown error";
+}
+
+int dxh_device_count(int *count) {
+    if (!count) return DXH_ERR_ARG;
+    hipError_t e = hipGetDeviceCount(count);
+    if (e != hipSuccess) { *count = 0; (void)hipGetLastError(); }
+    return (int)e;
+}
+int dxh_set_device(int device) { return (int)hipSetDevice(device); }
+int dxh_device_name(char *buf, size_t buflen) {
+    if (!buf || buflen == 0) return DXH_ERR_ARG;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return (int)e;
+    snprintf(buf, buflen, "%s %s cus=%d clock_khz=%d", prop.name, prop.gcnArchName, prop.multiProcessorCount, prop.clockRate);
+    return DXH_OK;
+}
+
+int dxh_malloc(void **ptr, size_t bytes) {
+    if (!ptr) return DXH_ERR_ARG;
+    *ptr = nullptr;
+    if (bytes == 0) bytes = 1;  // a zero-element tensor still owns a distinct pointer
+    return (int)hipMalloc(ptr, bytes);
+}
+int dxh_free(void *ptr) { return ptr ? (int)hipFree(ptr) : DXH_OK; }
+
+int dxh_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes == 0) return DXH_OK;
+    if (!dst || !src) return DXH_ERR_ARG;
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream));
+    if (e != hipSuccess) return (int)e;
+    return (int)hipStreamSynchronize(as_stream(stream));  // pageable source must stay valid
+}
+int dxh_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes == 0) return DXH_OK;
+    if (!dst || !src) return DXH_ERR_ARG;
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_stream(stream));
+    if (e != hipSuccess) return (int)e;
+    return (int)hipStreamSynchronize(as_stream(stream));
+}
+int dxh_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes == 0) return DXH_OK;
+    if (!dst || !src) return DXH_ERR_ARG;
+    return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream));
+}
+
+int dxh_stream_create(void **stream) {
+    if (!stream) return DXH_ERR_ARG;
+    hipStream_t s = nullptr;
+    hipError_t e = hipStreamCreate(&s);  // default priority only
+    *stream = (void *)s;
+    return (int)e;
+}
+int dxh_stream_destroy(void *stream) { return stream ? (int)hipStreamDestroy(as_stream(stream)) : DXH_OK; }
+int dxh_stream_sync(void *stream) { return (int)hipStreamSynchronize(as_stream(stream)); }
+int dxh_device_sync(void) { return (int)hipDeviceSynchronize(); }
+
+int dxh_event_create(void **event) {
+    if (!event) return DXH_ERR_ARG;
+    hipEvent_t ev = nullptr;
+    hipError_t e = hipEventCreate(&ev);
+    *event = (void *)ev;
+    return (int)e;
+}
+int dxh_event_destroy(void *event) { return event ? (int)hipEventDestroy((hipEvent_t)event) : DXH_OK; }
+int dxh_event_record(void *event, void *stream) {
+    if (!event) return DXH_ERR_ARG;
+    return (int)hipEventRecord((hipEvent_t)event, as_stream(stream));
+}
+int dxh_event_sync(void *event) {
+    if (!event) return DXH_ERR_ARG;
+    return (int)hipEventSynchronize((hipEvent_t)event);
+}
+int dxh_event_elapsed_ms(void *start, void *stop, float *ms) {
+    if (!start || !stop || !ms) return DXH_ERR_ARG;
+    return (int)hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop);
+}
+
+}  // extern "C"

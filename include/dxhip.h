@@ -1,0 +1,234 @@
+/*
+ * dxhip.h — C ABI of libdxhip, the MI355X (gfx950) kernel layer of the deepx
+ * `op-mem-hip` executor.
+ *
+ * This is the host<->kernel seam of the executor.  In the reference it is the set
+ * of `launch_*` C++ templates that executor/op-cuda declares in
+ *   executor/op-cuda/src/deepx/tensorfunc/elementwise_miaobyte_basic.cuh:11-98
+ *   executor/op-cuda/src/deepx/tensorfunc/elementwise_miaobyte_sqrt.cuh:14-51
+ *   executor/op-cuda/src/deepx/tensorfunc/elementwise_miaobyte_sin.cuh:19-33
+ *   executor/op-cuda/src/deepx/tensorfunc/elementwise_miaobyte_compare.cuh:15-116
+ *   executor/op-cuda/src/deepx/tensorfunc/reduce_miaobyte.cuh:16-52
+ *   executor/op-cuda/src/deepx/tensorfunc/changeshape_miaobyte.cuh:16-79
+ *   executor/op-cuda/src/deepx/tensorfunc/init_miaobyte.cuh:18-47
+ *   executor/op-cuda/src/deepx/tensorfunc/matmul_cublas.hpp:16-145
+ *   executor/op-cuda/src/deepx/tensorfunc/tensorlife_miaobyte.hpp:16-68
+ * and whose arithmetic is defined by executor/op-ompsimd (the parity oracle).
+ *
+ * Conventions
+ *  - plain pointers and sizes, no C++ types; every entry point returns an int:
+ *    0 = ok, >0 = a hipError_t value, <0 = one of the DXH_ERR_* codes below.
+ *    Nothing throws across the boundary.
+ *  - all tensor pointers are DEVICE pointers to contiguous row-major storage
+ *    (executor/deepxcore/src/deepx/shape.cpp:21-32); shape/axis arrays are HOST
+ *    pointers and are consumed before the call returns.
+ *  - `dtype` is the reference's Precision bit value
+ *    (executor/deepxcore/src/deepx/dtype.hpp:120-146), so the executor passes
+ *    `shape.dtype` through unchanged.
+ *  - bool tensors are one byte per element holding 0 or 1.
+ *  - fp16 / bf16 ops compute in fp32 and round once (RNE) to the storage type,
+ *    the convention of executor/op-cuda/src/deepx/tensorfunc/cuda_math.cuh:243-251.
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls
+ *    are asynchronous: they return after enqueueing, like the reference's launches.
+ *  - element counts are 64-bit; kernels never allocate.  Entry points that need
+ *    device scratch take a caller-provided workspace (size from the matching
+ *    *_workspace_bytes query).
+ */
+#ifndef DXHIP_H
+#define DXHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DXH_API __attribute__((visibility("default")))
+
+/* Precision bit values, executor/deepxcore/src/deepx/dtype.hpp:120-146 */
+enum dxh_dtype {
+    DXH_F64  = 1 << 0,
+    DXH_F32  = 1 << 1,
+    DXH_F16  = 1 << 2,
+    DXH_BF16 = 1 << 3,
+    DXH_I64  = 1 << 8,
+    DXH_I32  = 1 << 9,
+    DXH_I16  = 1 << 10,
+    DXH_I8   = 1 << 11,
+    DXH_BOOL = 1 << 13
+};
+
+enum dxh_error {
+    DXH_OK = 0,
+    DXH_ERR_DTYPE = -1,      /* dtype not supported by this op */
+    DXH_ERR_ARG = -2,        /* null pointer, negative size, bad axis ... */
+    DXH_ERR_SHAPE = -3,      /* shapes inconsistent for this op */
+    DXH_ERR_WORKSPACE = -4,  /* workspace missing or too small */
+    DXH_ERR_ALIGN = -5       /* pointer not aligned to its element size */
+};
+
+/* A scalar operand.  Floating dtypes read `f`, integer and bool dtypes read `i`.
+ * The executor fills both from T(std::stof(text)), the reference's scalar rule
+ * (executor/deepxcore/src/deepx/tf/tf.hpp:119-123). */
+typedef struct dxh_scalar {
+    double f;
+    int64_t i;
+} dxh_scalar;
+
+#define DXH_MAX_DIMS 12 /* the reference instantiates DIM 1..12, reduce_miaobyte.cu:61-107 */
+
+/* ---- runtime: replaces cudaMalloc/cudaFree/cudaMemcpy of
+ * executor/op-cuda/src/deepx/tensorfunc/tensorlife_miaobyte.hpp:16-68 ---------- */
+DXH_API int dxh_version(void);
+DXH_API const char *dxh_error_string(int code);
+DXH_API int dxh_device_count(int *count);
+DXH_API int dxh_set_device(int device);
+DXH_API int dxh_device_name(char *buf, size_t buflen);
+DXH_API int dxh_malloc(void **ptr, size_t bytes);
+DXH_API int dxh_free(void *ptr);
+DXH_API int dxh_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream);
+DXH_API int dxh_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream);
+DXH_API int dxh_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
+DXH_API int dxh_stream_create(void **stream);
+DXH_API int dxh_stream_destroy(void *stream);
+DXH_API int dxh_stream_sync(void *stream);
+DXH_API int dxh_device_sync(void);
+/* hipEvent helpers so a harness can time on the stream the kernels run on. */
+DXH_API int dxh_event_create(void **event);
+DXH_API int dxh_event_destroy(void *event);
+DXH_API int dxh_event_record(void *event, void *stream);
+DXH_API int dxh_event_sync(void *event);
+DXH_API int dxh_event_elapsed_ms(void *start, void *stop, float *ms);
+
+/* ---- elementwise, C[i] = A[i] op B[i]
+ * launch_add/sub/mul/div  elementwise_miaobyte_basic.cuh:16-98
+ * launch_max/min          elementwise_miaobyte_compare.cuh:15-44
+ * launch_pow              elementwise_miaobyte_sqrt.cuh:22-28   (f32/f64 only)
+ * arithmetic per executor/op-ompsimd/src/deepx/tensorfunc/elementwise_miaobyte.hpp:115-318,430-448,599-764
+ * dtypes: f64 f32 f16 bf16 i64 i32 i16 i8.  Integer division by zero yields 0. */
+DXH_API int dxh_add(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream);
+DXH_API int dxh_sub(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream);
+DXH_API int dxh_mul(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream);
+DXH_API int dxh_div(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream);
+DXH_API int dxh_max(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream);
+DXH_API int dxh_min(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream);
+DXH_API int dxh_pow(int dtype, const void *a, const void *b, void *c, int64_t n, void *stream);
+
+/* ---- elementwise with a scalar operand
+ * launch_addscalar ... launch_rdivscalar  elementwise_miaobyte_basic.cuh:24-98
+ * launch_maxscalar/minscalar             elementwise_miaobyte_compare.cuh:22-44
+ * launch_powscalar/rpowscalar            elementwise_miaobyte_sqrt.cuh:30-44 (f32/f64 only)
+ * r*scalar forms compute scalar op A[i]. */
+DXH_API int dxh_addscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream);
+DXH_API int dxh_subscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream);
+DXH_API int dxh_rsubscalar(int dtype, dxh_scalar s, const void *a, void *c, int64_t n, void *stream);
+DXH_API int dxh_mulscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream);
+DXH_API int dxh_divscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream);
+DXH_API int dxh_rdivscalar(int dtype, dxh_scalar s, const void *a, void *c, int64_t n, void *stream);
+DXH_API int dxh_maxscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream);
+DXH_API int dxh_minscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream);
+DXH_API int dxh_powscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream);
+DXH_API int dxh_rpowscalar(int dtype, dxh_scalar s, const void *a, void *c, int64_t n, void *stream);
+
+/* ---- unary
+ * launch_sqrt/log/exp  elementwise_miaobyte_sqrt.cuh:14-20,46-51 (f64 f32 f16 bf16)
+ * launch_sin/cos/tan   elementwise_miaobyte_sin.cuh:19-33        (tan: f64 f32)
+ * launch_invert        elementwise_miaobyte_basic.cuh:94-98      (i64 i32 i16 i8: ~x, bool: !x) */
+DXH_API int dxh_sqrt(int dtype, const void *a, void *c, int64_t n, void *stream);
+DXH_API int dxh_exp(int dtype, const void *a, void *c, int64_t n, void *stream);
+DXH_API int dxh_log(int dtype, const void *a, void *c, int64_t n, void *stream);
+DXH_API int dxh_sin(int dtype, const void *a, void *c, int64_t n, void *stream);
+DXH_API int dxh_cos(int dtype, const void *a, void *c, int64_t n, void *stream);
+DXH_API int dxh_tan(int dtype, const void *a, void *c, int64_t n, void *stream);
+DXH_API int dxh_invert(int dtype, const void *a, void *c, int64_t n, void *stream);
+
+/* ---- cast: launch_todtype elementwise_miaobyte_basic.cuh:11-16.
+ * C[i] = static_cast<dst>(A[i]) (float->int truncates toward zero, saturating at
+ * the integer range; float->f16/bf16 rounds RNE).  Same dtype = device copy. */
+DXH_API int dxh_todtype(int src_dtype, const void *a, int dst_dtype, void *c, int64_t n, void *stream);
+
+/* ---- compare -> bool mask (one byte, 0/1)
+ * launch_equal/notequal(+scalar) with epsilon  elementwise_miaobyte_compare.cuh:46-84
+ * launch_less/greater(+scalar)                 elementwise_miaobyte_compare.cuh:86-108
+ * epsilon semantics follow op-ompsimd (elementwise_miaobyte.hpp:767-886):
+ *   equal:    eps==0 ? a==b : |a-b| <= eps        notequal: eps==0 ? a!=b : |a-b| > eps */
+DXH_API int dxh_equal(int dtype, const void *a, const void *b, float epsilon, void *mask, int64_t n, void *stream);
+DXH_API int dxh_notequal(int dtype, const void *a, const void *b, float epsilon, void *mask, int64_t n, void *stream);
+DXH_API int dxh_equalscalar(int dtype, const void *a, dxh_scalar s, float epsilon, void *mask, int64_t n, void *stream);
+DXH_API int dxh_notequalscalar(int dtype, const void *a, dxh_scalar s, float epsilon, void *mask, int64_t n, void *stream);
+DXH_API int dxh_less(int dtype, const void *a, const void *b, void *mask, int64_t n, void *stream);
+DXH_API int dxh_greater(int dtype, const void *a, const void *b, void *mask, int64_t n, void *stream);
+DXH_API int dxh_lessscalar(int dtype, const void *a, dxh_scalar s, void *mask, int64_t n, void *stream);
+DXH_API int dxh_greaterscalar(int dtype, const void *a, dxh_scalar s, void *mask, int64_t n, void *stream);
+
+/* ---- switch: launch_switch elementwise_miaobyte_compare.cuh:110-116.
+ * C[i] = tensors[cases[i]][i]; cases_dtype is DXH_I32 or DXH_BOOL (bool needs exactly
+ * two tensors, elementwise_miaobyte.hpp:1001-1024).  `tensors` is a HOST array of
+ * `ntensors` device pointers, 1 <= ntensors <= DXH_SWITCH_MAX; it is passed to the
+ * kernel by value (no device-side pointer table, no allocation).  A case value
+ * outside [0, ntensors) selects nothing and writes zero bits. */
+#define DXH_SWITCH_MAX 8
+DXH_API int dxh_switch(int dtype, const void *const *tensors, int ntensors, int cases_dtype,
+                       const void *cases, void *c, int64_t n, void *stream);
+
+/* ---- reduce: launch_sum/prod/reducemax/reducemin reduce_miaobyte.cuh:16-52.
+ * `shape[ndim]` is the input shape; `dims[ndims]` the reduced axes (negative allowed;
+ * normalised, sorted, de-duplicated as executor/deepxcore/src/deepx/shape_reduce.cpp:11-45;
+ * ndims==0 reduces every axis).  The output holds prod(kept dims) elements; keepdims
+ * only changes the caller's view of it (shape_reduce.cpp:47-74).  f16/bf16 accumulate
+ * in fp32, f32 in fp32, f64 in f64, integers wrap in their own width.
+ * `workspace` may be NULL when dxh_reduce_workspace_bytes reports 0. */
+DXH_API int dxh_reduce_workspace_bytes(int dtype, const int32_t *shape, int ndim,
+                                       const int32_t *dims, int ndims, size_t *bytes);
+DXH_API int dxh_sum(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims,
+                    int ndims, void *out, void *workspace, size_t workspace_bytes, void *stream);
+DXH_API int dxh_prod(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims,
+                     int ndims, void *out, void *workspace, size_t workspace_bytes, void *stream);
+DXH_API int dxh_reducemax(int dtype, const void *in, const int32_t *shape, int ndim,
+                          const int32_t *dims, int ndims, void *out, void *workspace,
+                          size_t workspace_bytes, void *stream);
+DXH_API int dxh_reducemin(int dtype, const void *in, const int32_t *shape, int ndim,
+                          const int32_t *dims, int ndims, void *out, void *workspace,
+                          size_t workspace_bytes, void *stream);
+
+/* ---- changeshape: changeshape_miaobyte.cuh:16-79.  Pure data movement, bit-exact,
+ * chosen by element size, so every dtype above (and bool) is accepted.
+ * transpose:   out[o] = in[p], p[dim_order[i]] = o[i]  (changeshape_miaobyte.hpp:45-67)
+ * concat:      `ins` HOST array of device pointers, `axis_sizes[i]` = shape of source i on
+ *              `axis`; `out_shape` is the result shape             (:69-100)
+ * broadcastTo: numpy trailing-aligned rules, shape_changeshape.cpp:59-104
+ * indexselect: out[pre,idx...,post] = in[pre, index[idx...], post]; index_dtype I32|I64;
+ *              out-of-range indices are clamped into [0, shape[axis]) rather than read
+ *              out of bounds (the reference does not check, :155-178)
+ * repeat:      out[i] = in[i / repeats]                             (:181-200) */
+DXH_API int dxh_transpose(int dtype, const void *in, const int32_t *shape, int ndim,
+                          const int32_t *dim_order, void *out, void *stream);
+DXH_API int dxh_concat(int dtype, const void *const *ins, int nins, const int32_t *axis_sizes,
+                       const int32_t *out_shape, int ndim, int axis, void *out, void *stream);
+DXH_API int dxh_broadcastTo(int dtype, const void *in, const int32_t *in_shape, int in_ndim,
+                            const int32_t *out_shape, int out_ndim, void *out, void *stream);
+DXH_API int dxh_indexselect(int dtype, const void *in, const int32_t *in_shape, int in_ndim,
+                            int index_dtype, const void *index, const int32_t *index_shape,
+                            int index_ndim, int axis, void *out, void *stream);
+DXH_API int dxh_repeat(int dtype, const void *in, const int32_t *shape, int ndim,
+                       const int32_t *repeats, void *out, void *stream);
+
+/* ---- init: launch_constant / launch_arange init_miaobyte.cuh:18-30.
+ * arange: out[i] = start + i*step computed in the dtype's arithmetic
+ * (executor/op-ompsimd/src/deepx/tensorfunc/init_miaobyte.hpp:59-70). */
+DXH_API int dxh_constant(int dtype, void *out, int64_t n, dxh_scalar value, void *stream);
+DXH_API int dxh_arange(int dtype, void *out, int64_t n, dxh_scalar start, dxh_scalar step, void *stream);
+
+/* ---- matmul: replaces cublasSgemm(StridedBatched) matmul_cublas.hpp:16-145 and
+ * cblas_sgemm executor/op-ompsimd/src/deepx/tensorfunc/matmul_cblas.hpp:11-60.
+ * C[b,m,n] = sum_k A[b,m,k] * B[b,k,n], row-major, alpha=1 beta=0, `batch` = product of
+ * the leading dims.  f16/bf16: MFMA with fp32 accumulate, one RNE rounding of the
+ * result; f32/f64 accumulate in their own type; integers wrap. */
+DXH_API int dxh_matmul(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m,
+                       int64_t k, int64_t n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DXHIP_H */

@@ -1,0 +1,895 @@
+// oracle.cpp — CPU restatement of the deepx op-ompsimd executor's arithmetic.
+//
+// TEST INFRASTRUCTURE ONLY.  This file is the parity checker for libdxhip: it is
+// linked and called by tests/, by __graft_entry__.smoke() and by bench.py's
+// cpu_baseline leg, never by the product (deepx_amd/).  It has no third-party
+// dependencies (the reference needs Highway, OpenBLAS, jemalloc and yaml-cpp).
+//
+// Every function names the reference code it restates.  Paths are relative to the
+// reference checkout.  `E` = executor/op-ompsimd/src/deepx/tensorfunc.
+//
+// What pins each group (tests/test_oracle_*.py):
+//   add/sub/mul/div/sqrt      IEEE-754 correctly rounded => numpy float32/float64 bit-equal
+//   integer ops, compare, switch, invert   exact integer semantics => numpy + brute force
+//   max/min                   (a<b)?b:a, numpy maximum/minimum on non-NaN inputs
+//   exp/log/pow/sin/cos/tan   glibc libm on this host; numpy within 1 ulp; special values
+//   todtype                   numpy astype (in-range), torch bfloat16 / numpy float16 RNE
+//   sum/prod                  float64 accumulation + closed forms (arange, ones)
+//   reducemax/reducemin       numpy amax/amin (order independent)
+//   reduced shape             table in executor/op-ompsimd/test/tensorfunc/5_tensor_sum.cpp:40-49
+//   transpose/concat/broadcastTo/indexselect/repeat   numpy permute/concatenate/
+//                             broadcast_to/take/tile; concat also against the expectation
+//                             in executor/op-ompsimd/test/tensorfunc/8_tensor_concat.cpp:47-129
+//   matmul                    known answer in executor/op-ompsimd/test/tensorfunc/
+//                             4_tensor_matmul.cpp:18-36 + float64 numpy matmul.
+// Parity unpinned (only a running reference could pin them): the exact bits of fp32
+// sum/prod (the reference accumulates under `omp atomic` in thread-schedule order,
+// E/reduce_miaobyte.hpp:30-44) and of OpenBLAS sgemm (E/matmul_cblas.hpp:51-57);
+// both are checked to the stated relative tolerance instead.
+//
+// Deliberate differences from the reference source, each a reference defect:
+//   * Shape::rangeElementwiseParallel passes an absolute end where every lambda expects
+//     a length (executor/deepxcore/src/deepx/shape_range.cpp:116-135); chunks here use
+//     correct bounds.
+//   * reducemax/reducemin update the result without synchronisation
+//     (E/reduce_miaobyte.hpp:206,290); here each output is owned by one thread.
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <limits>
+#include <type_traits>
+#include <vector>
+#include <omp.h>
+
+namespace {
+
+enum : int {
+    F64 = 1 << 0, F32 = 1 << 1, F16 = 1 << 2, BF16 = 1 << 3,
+    I64 = 1 << 8, I32 = 1 << 9, I16 = 1 << 10, I8 = 1 << 11, BOOL = 1 << 13
+};
+enum : int { OK = 0, ERR_DTYPE = -1, ERR_ARG = -2, ERR_SHAPE = -3 };
+
+struct scalar_t { double f; int64_t i; };
+
+// ---- 16-bit float storage types: bit patterns + conversions (RNE) -------------
+// Convention of executor/op-cuda/src/deepx/tensorfunc/cuda_math.cuh:243-251
+// (__float2bfloat16 / __float2half round to nearest even).
+struct bf16 { uint16_t bits; };
+struct f16 { uint16_t bits; };
+
+inline float bits2f(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
+inline uint32_t f2bits(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
+
+inline float bf16_to_f32(bf16 h) { return bits2f(uint32_t(h.bits) << 16); }
+inline bf16 f32_to_bf16(float f) {
+    uint32_t u = f2bits(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return bf16{uint16_t((u >> 16) | 0x0040u)};  // quiet NaN
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;
+    return bf16{uint16_t(u >> 16)};
+}
+inline float f16_to_f32(f16 h) {
+    uint32_t s = uint32_t(h.bits & 0x8000u) << 16;
+    uint32_t e = (h.bits >> 10) & 0x1fu;
+    uint32_t m = h.bits & 0x3ffu;
+    if (e == 0) {
+        if (m == 0) return bits2f(s);
+        // subnormal: value = m * 2^-24
+        float v = float(m) * 5.9604644775390625e-08f;
+        return s ? -v : v;
+    }
+    if (e == 31) return bits2f(s | 0x7f800000u | (m << 13));
+    return bits2f(s | ((e + 112u) << 23) | (m << 13));
+}
+inline f16 f32_to_f16(float f) {
+    uint32_t u = f2bits(f);
+    uint16_t s = uint16_t((u >> 16) & 0x8000u);
+    uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return f16{uint16_t(s | 0x7e00u | ((a >> 13) & 0x3ffu))};  // NaN
+    if (a >= 0x47800000u) return f16{uint16_t(s | 0x7c00u)};  // >= 65536 -> inf (65520 handled below)
+    if (a >= 0x38800000u) {  // normal half range
+        uint32_t r = a - 0x38000000u;  // rebias exponent 127 -> 15
+        uint32_t lsb = (r >> 13) & 1u;
+        r += 0xfffu + lsb;
+        return f16{uint16_t(s | (r >> 13))};  // may carry into inf, which is correct RNE
+    }
+    if (a < 0x33000000u) return f16{s};  // < 2^-25 rounds to zero (2^-25 itself ties to even = 0)
+    // subnormal half: shift mantissa with implicit bit
+    uint32_t e = a >> 23;
+    uint32_t m = (a & 0x7fffffu) | 0x800000u;
+    uint32_t shift = 126u - e;  // 14..24
+    uint32_t q = m >> shift;
+    uint32_t rem = m & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) q++;
+    return f16{uint16_t(s | q)};
+}
+// double -> 16-bit: round double to float with round-to-odd, then RNE, which equals a
+// single RNE from double (the float keeps >= 2 extra bits plus a sticky bit).
+inline float f64_to_f32_round_odd(double d) {
+    float f = float(d);
+    if (std::isnan(d) || std::isinf(f) || double(f) == d) return f;
+    uint32_t u = f2bits(f);
+    // choose the truncated neighbour (toward zero), then force the last bit odd
+    if (std::fabs(double(f)) > std::fabs(d)) u -= 1;
+    u |= 1u;
+    return bits2f(u);
+}
+
+// compute type and load/store per storage type
+template <typename T> struct acc { using type = T; };
+template <> struct acc<bf16> { using type = float; };
+template <> struct acc<f16> { using type = float; };
+template <typename T> using acc_t = typename acc<T>::type;
+
+template <typename T> inline acc_t<T> ld(const T &x) { return x; }
+inline float ld(const bf16 &x) { return bf16_to_f32(x); }
+inline float ld(const f16 &x) { return f16_to_f32(x); }
+template <typename T> inline void st(T &dst, acc_t<T> v) { dst = v; }
+inline void st(bf16 &dst, float v) { dst = f32_to_bf16(v); }
+inline void st(f16 &dst, float v) { dst = f32_to_f16(v); }
+
+template <typename T> constexpr bool is_fp = std::is_floating_point_v<acc_t<T>>;
+
+template <typename T> inline T scalar_as(const scalar_t &s) {
+    if constexpr (std::is_same_v<T, bf16>) return f32_to_bf16(float(s.f));
+    else if constexpr (std::is_same_v<T, f16>) return f32_to_f16(float(s.f));
+    else if constexpr (std::is_floating_point_v<T>) return T(s.f);
+    else return T(s.i);
+}
+
+// ---- chunked parallel loop: Shape::rangeElementwiseParallel,
+// executor/deepxcore/src/deepx/shape_range.cpp:116-135 (hardware_concurrency() chunks,
+// at least 256 elements each), with correct chunk bounds.
+template <typename F> void range_elementwise(int64_t n, F body) {
+    int nt = omp_get_max_threads();
+    int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(nt, n / 256));
+    int64_t per = (n + chunks - 1) / chunks;
+#pragma omp parallel for schedule(static) num_threads((int)chunks)
+    for (int64_t c = 0; c < chunks; ++c) {
+        int64_t lo = c * per, hi = std::min(n, lo + per);
+        if (lo < hi) body(lo, hi);
+    }
+}
+
+// wrapping integer arithmetic without UB
+template <typename T> inline T wadd(T a, T b) { using U = std::make_unsigned_t<T>; return T(U(U(a) + U(b))); }
+template <typename T> inline T wsub(T a, T b) { using U = std::make_unsigned_t<T>; return T(U(U(a) - U(b))); }
+template <typename T> inline T wmul(T a, T b) {
+    using U = std::conditional_t<(sizeof(T) < 4), uint32_t, std::make_unsigned_t<T>>;
+    return T(U(U(a) * U(b)));
+}
+template <typename T> inline T wdiv(T a, T b) {
+    if (b == 0) return T(0);
+    if (b == T(-1)) return wsub<T>(T(0), a);
+    return T(a / b);
+}
+
+enum BinOp { ADD, SUB, RSUB, MUL, DIV, RDIV, MAX, MIN, POW, RPOW };
+
+// E/elementwise_miaobyte.hpp:115-318 (add..rdivscalar), :430-489 (pow family),
+// :599-764 (max/min: std::max / std::min, i.e. (a<b)?b:a and (b<a)?b:a).
+template <BinOp OP, typename A> inline A apply(A a, A b) {
+    if constexpr (OP == ADD) { if constexpr (std::is_integral_v<A>) return wadd(a, b); else return a + b; }
+    else if constexpr (OP == SUB) { if constexpr (std::is_integral_v<A>) return wsub(a, b); else return a - b; }
+    else if constexpr (OP == RSUB) { if constexpr (std::is_integral_v<A>) return wsub(b, a); else return b - a; }
+    else if constexpr (OP == MUL) { if constexpr (std::is_integral_v<A>) return wmul(a, b); else return a * b; }
+    else if constexpr (OP == DIV) { if constexpr (std::is_integral_v<A>) return wdiv(a, b); else return a / b; }
+    else if constexpr (OP == RDIV) { if constexpr (std::is_integral_v<A>) return wdiv(b, a); else return b / a; }
+    else if constexpr (OP == MAX) return (a < b) ? b : a;
+    else if constexpr (OP == MIN) return (b < a) ? b : a;
+    else if constexpr (OP == POW) return std::pow(a, b);
+    else return std::pow(b, a);
+}
+
+template <BinOp OP, typename T> int binary_t(const void *a_, const void *b_, void *c_, int64_t n) {
+    const T *a = (const T *)a_; const T *b = (const T *)b_; T *c = (T *)c_;
+    range_elementwise(n, [&](int64_t lo, int64_t hi) {
+        for (int64_t i = lo; i < hi; ++i) st(c[i], apply<OP, acc_t<T>>(ld(a[i]), ld(b[i])));
+    });
+    return OK;
+}
+template <BinOp OP, typename T> int scalar_op_t(const void *a_, scalar_t s, void *c_, int64_t n) {
+    const T *a = (const T *)a_; T *c = (T *)c_;
+    const acc_t<T> sv = ld(scalar_as<T>(s));
+    range_elementwise(n, [&](int64_t lo, int64_t hi) {
+        for (int64_t i = lo; i < hi; ++i) st(c[i], apply<OP, acc_t<T>>(ld(a[i]), sv));
+    });
+    return OK;
+}
+
+#define DISPATCH_ALL(dtype, CALL)                                   \
+    switch (dtype) {                                                \
+    case F64: return CALL(double);                                  \
+    case F32: return CALL(float);                                   \
+    case F16: return CALL(f16);                                     \
+    case BF16: return CALL(bf16);                                   \
+    case I64: return CALL(int64_t);                                 \
+    case I32: return CALL(int32_t);                                 \
+    case I16: return CALL(int16_t);                                 \
+    case I8: return CALL(int8_t);                                   \
+    default: return ERR_DTYPE;                                      \
+    }
+enum UnOp { SQRT, EXP, LOG, SIN, COS, TAN };
+// E/elementwise_miaobyte.hpp:364-428 (sqrt), :491-596 (log/exp/sin/cos/tan): libm per element.
+template <UnOp OP, typename T> int unary_t(const void *a_, void *c_, int64_t n) {
+    const T *a = (const T *)a_; T *c = (T *)c_;
+    range_elementwise(n, [&](int64_t lo, int64_t hi) {
+        for (int64_t i = lo; i < hi; ++i) {
+            acc_t<T> x = ld(a[i]), y;
+            if constexpr (OP == SQRT) y = std::sqrt(x);
+            else if constexpr (OP == EXP) y = std::exp(x);
+            else if constexpr (OP == LOG) y = std::log(x);
+            else if constexpr (OP == SIN) y = std::sin(x);
+            else if constexpr (OP == COS) y = std::cos(x);
+            else y = std::tan(x);
+            st(c[i], y);
+        }
+    });
+    return OK;
+}
+
+// ---- todtype: E/elementwise_miaobyte.hpp:103-112, C[i] = static_cast<Dtype>(A[i]).
+// Out-of-range float->int is undefined in C++; defined here as saturation, NaN -> 0.
+template <typename D, typename S> inline D cast_one(S v) {
+    if constexpr (std::is_same_v<S, bf16> || std::is_same_v<S, f16>) {
+        return cast_one<D, float>(ld(v));
+    } else if constexpr (std::is_same_v<D, bf16>) {
+        if constexpr (std::is_same_v<S, float>) return f32_to_bf16(v);
+        else return f32_to_bf16(f64_to_f32_round_odd(double(v)));
+    } else if constexpr (std::is_same_v<D, f16>) {
+        if constexpr (std::is_same_v<S, float>) return f32_to_f16(v);
+        else return f32_to_f16(f64_to_f32_round_odd(double(v)));
+    } else if constexpr (std::is_floating_point_v<S> && std::is_integral_v<D>) {
+        if (std::isnan(v)) return D(0);
+        const double lo = double(std::numeric_limits<D>::min());
+        const double hi = double(std::numeric_limits<D>::max());  // 2^63 for int64 after rounding
+        double d = std::trunc(double(v));
+        if (d <= lo) return std::numeric_limits<D>::min();
+        if (d >= hi) return std::numeric_limits<D>::max();
+        return D(d);
+    } else {
+        return D(v);
+    }
+}
+template <typename S, typename D> int cast_t(const void *a_, void *c_, int64_t n) {
+    const S *a = (const S *)a_; D *c = (D *)c_;
+    range_elementwise(n, [&](int64_t lo, int64_t hi) {
+        for (int64_t i = lo; i < hi; ++i) c[i] = cast_one<D, S>(a[i]);
+    });
+    return OK;
+}
+template <typename S> int cast_from(const void *a, int dst, void *c, int64_t n) {
+    switch (dst) {
+    case F64: return cast_t<S, double>(a, c, n);
+    case F32: return cast_t<S, float>(a, c, n);
+    case F16: return cast_t<S, f16>(a, c, n);
+    case BF16: return cast_t<S, bf16>(a, c, n);
+    case I64: return cast_t<S, int64_t>(a, c, n);
+    case I32: return cast_t<S, int32_t>(a, c, n);
+    case I16: return cast_t<S, int16_t>(a, c, n);
+    case I8: return cast_t<S, int8_t>(a, c, n);
+    default: return ERR_DTYPE;
+    }
+}
+
+// ---- compare: E/elementwise_miaobyte.hpp:767-974 -> Tensor<bool> (one byte).
+enum CmpOp { EQ, NE, LT, GT };
+template <typename A> inline bool within_eps(A a, A b, float eps) {
+    if constexpr (std::is_integral_v<A>) {
+        // std::abs(a-b) <= epsilon: integer difference, compared after conversion to float
+        int64_t d = (int64_t)wsub<int64_t>((int64_t)a, (int64_t)b);
+        uint64_t ad = d < 0 ? (uint64_t)0 - (uint64_t)d : (uint64_t)d;
+        return float(ad) <= eps;
+    } else {
+        return std::abs(a - b) <= eps;
+    }
+}
+// notequal with eps>0 is |a-b| > eps (false when NaN is involved, like the reference's `>`).
+template <typename A> inline bool ne_eps(A a, A b, float eps) {
+    if constexpr (std::is_integral_v<A>) return !within_eps(a, b, eps);
+    else return std::abs(a - b) > eps;
+}
+template <CmpOp OP, typename T>
+int compare_t(const void *a_, const void *b_, bool bscalar, scalar_t s, float eps, void *m_, int64_t n) {
+    const T *a = (const T *)a_; const T *b = (const T *)b_; uint8_t *m = (uint8_t *)m_;
+    using A = acc_t<T>;
+    const A sv = bscalar ? ld(scalar_as<T>(s)) : A(0);
+    range_elementwise(n, [&](int64_t lo, int64_t hi) {
+        for (int64_t i = lo; i < hi; ++i) {
+            A x = ld(a[i]);
+            A y = bscalar ? sv : ld(b[i]);
+            bool r;
+            if constexpr (OP == EQ) r = (eps == 0) ? (x == y) : within_eps<A>(x, y, eps);
+            else if constexpr (OP == NE) r = (eps == 0) ? (x != y) : ne_eps<A>(x, y, eps);
+            else if constexpr (OP == LT) r = x < y;
+            else r = x > y;
+            m[i] = r ? 1 : 0;
+        }
+    });
+    return OK;
+}
+
+// ---- switch: E/elementwise_miaobyte.hpp:977-1027.
+template <int ESIZE> struct raw;
+template <> struct raw<1> { using type = uint8_t; };
+template <> struct raw<2> { using type = uint16_t; };
+template <> struct raw<4> { using type = uint32_t; };
+template <> struct raw<8> { using type = uint64_t; };
+
+template <typename R>
+int switch_t(const void *const *tensors, int nt, int cases_dtype, const void *cases, void *c_, int64_t n) {
+    R *c = (R *)c_;
+    if (cases_dtype == BOOL) {
+        if (nt != 2) return ERR_ARG;
+        const uint8_t *cs = (const uint8_t *)cases;
+        range_elementwise(n, [&](int64_t lo, int64_t hi) {
+            for (int64_t i = lo; i < hi; ++i) c[i] = ((const R *)tensors[cs[i] ? 1 : 0])[i];
+        });
+    } else if (cases_dtype == I32) {
+        const int32_t *cs = (const int32_t *)cases;
+        range_elementwise(n, [&](int64_t lo, int64_t hi) {
+            for (int64_t i = lo; i < hi; ++i) {
+                int32_t w = cs[i];
+                c[i] = (w >= 0 && w < nt) ? ((const R *)tensors[w])[i] : R(0);
+            }
+        });
+    } else return ERR_DTYPE;
+    return OK;
+}
+
+int esize(int dtype) {
+    switch (dtype) {
+    case F64: case I64: return 8;
+    case F32: case I32: return 4;
+    case F16: case BF16: case I16: return 2;
+    case I8: case BOOL: return 1;
+    default: return 0;
+    }
+}
+
+// ---- reduce: E/reduce_miaobyte.hpp:19-345 + executor/deepxcore/src/deepx/shape_reduce.cpp.
+// checkedDims (shape_reduce.cpp:11-45): negative dims normalised, sorted, de-duplicated;
+// empty = all.  Returns false on out-of-range.
+bool checked_dims(int ndim, const int32_t *dims, int ndims, std::vector<int> &reduced /*0/1 per axis*/) {
+    reduced.assign(ndim, 0);
+    if (ndims == 0) { std::fill(reduced.begin(), reduced.end(), 1); return true; }
+    for (int i = 0; i < ndims; ++i) {
+        int d = dims[i];
+        if (d < 0) d += ndim;
+        if (d < 0 || d >= ndim) return false;
+        reduced[d] = 1;
+    }
+    return true;
+}
+
+enum RedOp { RSUM, RPROD, RMAX, RMIN };
+template <RedOp OP, typename T> int reduce_t(const void *in_, const int32_t *shape, int ndim,
+                                              const int32_t *dims, int ndims, void *out_) {
+    using A = acc_t<T>;
+    const T *in = (const T *)in_; T *out = (T *)out_;
+    std::vector<int> red;
+    if (ndim < 1 || !checked_dims(ndim, dims, ndims, red)) return ERR_ARG;
+    // split axes into kept and reduced, each with its input stride
+    std::vector<int64_t> stride(ndim);
+    int64_t s = 1;
+    for (int i = ndim - 1; i >= 0; --i) { stride[i] = s; s *= shape[i]; }
+    std::vector<int64_t> kshape, kstride, rshape, rstride;
+    for (int i = 0; i < ndim; ++i) {
+        if (red[i]) { rshape.push_back(shape[i]); rstride.push_back(stride[i]); }
+        else { kshape.push_back(shape[i]); kstride.push_back(stride[i]); }
+    }
+    int64_t nout = 1, nred = 1;
+    for (auto v : kshape) nout *= v;
+    for (auto v : rshape) nred *= v;
+    // Each output accumulates its elements in increasing linear input order — the order a
+    // single-threaded run of the reference's per-element loop produces
+    // (E/reduce_miaobyte.hpp:30-44; result pre-filled with 0 / 1 / lowest() / max(),
+    // :24, :101, :191, :274).
+#pragma omp parallel for schedule(static)
+    for (int64_t o = 0; o < nout; ++o) {
+        int64_t base = 0, rem = o;
+        for (int i = (int)kshape.size() - 1; i >= 0; --i) { base += (rem % kshape[i]) * kstride[i]; rem /= kshape[i]; }
+        A accv;
+        if constexpr (OP == RSUM) accv = A(0);
+        else if constexpr (OP == RPROD) accv = A(1);
+        else if constexpr (OP == RMAX) accv = std::numeric_limits<A>::lowest();
+        else accv = std::numeric_limits<A>::max();
+        std::vector<int64_t> idx(rshape.size(), 0);
+        for (int64_t r = 0; r < nred; ++r) {
+            int64_t off = base;
+            for (size_t i = 0; i < rshape.size(); ++i) off += idx[i] * rstride[i];
+            A x = ld(in[off]);
+            if constexpr (OP == RSUM) { if constexpr (std::is_integral_v<A>) accv = wadd(accv, x); else accv += x; }
+            else if constexpr (OP == RPROD) { if constexpr (std::is_integral_v<A>) accv = wmul(accv, x); else accv *= x; }
+            else if constexpr (OP == RMAX) accv = (accv < x) ? x : accv;
+            else accv = (x < accv) ? x : accv;
+            for (int i = (int)rshape.size() - 1; i >= 0; --i) { if (++idx[i] < rshape[i]) break; idx[i] = 0; }
+        }
+        st(out[o], accv);
+    }
+    return OK;
+}
+
+// The same reduction with the reference's own decomposition, for CPU-baseline timing only:
+// one callback per INPUT element, output index rebuilt through an index vector, atomic
+// accumulate (E/reduce_miaobyte.hpp:30-44 sum, :193-207 reducemax without atomic).
+template <RedOp OP> int reduce_faithful_f32(const float *in, const int32_t *shape, int ndim,
+                                            const int32_t *dims, int ndims, bool keepdims, float *out) {
+    std::vector<int> red;
+    if (!checked_dims(ndim, dims, ndims, red)) return ERR_ARG;
+    std::vector<int> oshape;
+    for (int i = 0; i < ndim; ++i) { if (!red[i]) oshape.push_back(shape[i]); else if (keepdims) oshape.push_back(1); }
+    if (oshape.empty()) oshape.push_back(1);
+    std::vector<int64_t> ostride(oshape.size());
+    int64_t nout = 1;
+    for (int i = (int)oshape.size() - 1; i >= 0; --i) { ostride[i] = nout; nout *= oshape[i]; }
+    std::vector<int64_t> stride(ndim);
+    int64_t n = 1;
+    for (int i = ndim - 1; i >= 0; --i) { stride[i] = n; n *= shape[i]; }
+    const float init = OP == RSUM ? 0.f : OP == RPROD ? 1.f : OP == RMAX ? std::numeric_limits<float>::lowest()
+                                                                         : std::numeric_limits<float>::max();
+    for (int64_t i = 0; i < nout; ++i) out[i] = init;
+#pragma omp parallel
+    {
+        std::vector<int> indices(ndim), oidx(oshape.size());
+#pragma omp for schedule(static)
+        for (int64_t lin = 0; lin < n; ++lin) {
+            int64_t rem = lin;
+            for (int i = 0; i < ndim; ++i) { indices[i] = int(rem / stride[i]); rem %= stride[i]; }
+            size_t j = 0;
+            for (int i = 0; i < ndim; ++i) {
+                if (!red[i]) oidx[j++] = indices[i];
+                else if (keepdims) oidx[j++] = 0;
+            }
+            int64_t o = 0;
+            for (size_t k = 0; k < j; ++k) o += oidx[k] * ostride[k];
+            if constexpr (OP == RSUM) {
+#pragma omp atomic
+                out[o] += in[lin];
+            } else if constexpr (OP == RPROD) {
+#pragma omp atomic
+                out[o] *= in[lin];
+            } else if constexpr (OP == RMAX) {
+                // the reference's plain read-modify-write races; a CAS loop keeps the
+                // per-element cost comparable without losing updates
+                float cur = out[o];
+                while (cur < in[lin] && !__atomic_compare_exchange(&out[o], &cur, &in[lin], true, __ATOMIC_RELAXED, __ATOMIC_RELAXED)) {}
+            } else {
+                float cur = out[o];
+                while (in[lin] < cur && !__atomic_compare_exchange(&out[o], &cur, &in[lin], true, __ATOMIC_RELAXED, __ATOMIC_RELAXED)) {}
+            }
+        }
+    }
+    return OK;
+}
+
+// ---- changeshape: E/changeshape_miaobyte.hpp, on raw element bits.
+struct Strides {
+    std::vector<int64_t> v; int64_t size;
+    Strides(const int32_t *shape, int ndim) : v(ndim) { size = 1; for (int i = ndim - 1; i >= 0; --i) { v[i] = size; size *= shape[i]; } }
+};
+
+// transpose, :45-67: for every output index o, p[dim_order[i]] = o[i], out[o] = in[p].
+template <typename R> int transpose_t(const void *in_, const int32_t *shape, int ndim, const int32_t *order, void *out_) {
+    const R *in = (const R *)in_; R *out = (R *)out_;
+    std::vector<int32_t> oshape(ndim);
+    std::vector<int> seen(ndim, 0);
+    for (int i = 0; i < ndim; ++i) {
+        if (order[i] < 0 || order[i] >= ndim || seen[order[i]]++) return ERR_ARG;
+        oshape[i] = shape[order[i]];
+    }
+    Strides is(shape, ndim), os(oshape.data(), ndim);
+#pragma omp parallel for schedule(static)
+    for (int64_t lin = 0; lin < os.size; ++lin) {
+        int64_t rem = lin, src = 0;
+        for (int i = 0; i < ndim; ++i) { int64_t oi = rem / os.v[i]; rem %= os.v[i]; src += oi * is.v[order[i]]; }
+        out[lin] = in[src];
+    }
+    return OK;
+}
+
+// concat, :69-100: iterate the first axis+1 output dims; locate the source tensor by
+// walking the axis sizes; copy a run of strides[axis] elements.
+template <typename R> int concat_t(const void *const *ins, int nins, const int32_t *axis_sizes,
+                                   const int32_t *out_shape, int ndim, int axis, void *out_) {
+    R *out = (R *)out_;
+    if (axis < 0 || axis >= ndim || nins < 1) return ERR_ARG;
+    int64_t total = 0;
+    for (int i = 0; i < nins; ++i) total += axis_sizes[i];
+    if (total != out_shape[axis]) return ERR_SHAPE;
+    int64_t outer = 1, inner = 1;
+    for (int i = 0; i < axis; ++i) outer *= out_shape[i];
+    for (int i = axis + 1; i < ndim; ++i) inner *= out_shape[i];
+    int64_t rows = outer * out_shape[axis];
+#pragma omp parallel for schedule(static)
+    for (int64_t row = 0; row < rows; ++row) {
+        int64_t o = row / out_shape[axis], a = row % out_shape[axis];
+        int t = 0;
+        while (t < nins && a >= axis_sizes[t]) { a -= axis_sizes[t]; ++t; }
+        const R *src = (const R *)ins[t] + (o * axis_sizes[t] + a) * inner;
+        std::copy(src, src + inner, out + row * inner);
+    }
+    return OK;
+}
+
+// broadcastTo, :122-139 with broadcastShape/broadcastMap of
+// executor/deepxcore/src/deepx/shape_changeshape.cpp:59-104.
+template <typename R> int broadcast_t(const void *in_, const int32_t *ishape, int indim,
+                                      const int32_t *oshape, int ondim, void *out_) {
+    const R *in = (const R *)in_; R *out = (R *)out_;
+    if (indim > ondim) return ERR_SHAPE;
+    int shift = ondim - indim;
+    Strides is(ishape, indim), os(oshape, ondim);
+    std::vector<int64_t> map(ondim, 0);  // input stride per output axis; 0 = broadcast
+    for (int i = shift; i < ondim; ++i) {
+        if (ishape[i - shift] == oshape[i]) map[i] = is.v[i - shift];
+        else if (ishape[i - shift] == 1) map[i] = 0;
+        else return ERR_SHAPE;
+    }
+#pragma omp parallel for schedule(static)
+    for (int64_t lin = 0; lin < os.size; ++lin) {
+        int64_t rem = lin, src = 0;
+        for (int i = 0; i < ondim; ++i) { int64_t oi = rem / os.v[i]; rem %= os.v[i]; src += oi * map[i]; }
+        out[lin] = in[src];
+    }
+    return OK;
+}
+
+// indexselect, :141-178 with indexselectShape shape_changeshape.cpp:124-144:
+// out[pre..., idx..., post...] = in[pre..., index[idx...], post...].
+template <typename R, typename IT>
+int indexselect_t(const void *in_, const int32_t *ishape, int indim, const void *index_,
+                  const int32_t *xshape, int xndim, int axis, void *out_) {
+    const R *in = (const R *)in_; const IT *index = (const IT *)index_; R *out = (R *)out_;
+    if (axis < 0) axis += indim;
+    if (axis < 0 || axis >= indim) return ERR_ARG;
+    int64_t pre = 1, post = 1, m = 1;
+    for (int i = 0; i < axis; ++i) pre *= ishape[i];
+    for (int i = axis + 1; i < indim; ++i) post *= ishape[i];
+    for (int i = 0; i < xndim; ++i) m *= xshape[i];
+    const int64_t adim = ishape[axis];
+#pragma omp parallel for schedule(static)
+    for (int64_t row = 0; row < pre * m; ++row) {
+        int64_t p = row / m, j = row % m;
+        int64_t k = (int64_t)index[j];
+        if (k < 0) k = 0;
+        if (k >= adim) k = adim - 1;
+        const R *src = in + (p * adim + k) * post;
+        std::copy(src, src + post, out + row * post);
+    }
+    return OK;
+}
+
+// repeat, :181-200: B[i] = A[i / repeats] per axis.
+template <typename R> int repeat_t(const void *in_, const int32_t *shape, int ndim, const int32_t *reps, void *out_) {
+    const R *in = (const R *)in_; R *out = (R *)out_;
+    std::vector<int32_t> oshape(ndim);
+    for (int i = 0; i < ndim; ++i) { if (reps[i] < 1) return ERR_ARG; oshape[i] = shape[i] * reps[i]; }
+    Strides is(shape, ndim), os(oshape.data(), ndim);
+#pragma omp parallel for schedule(static)
+    for (int64_t lin = 0; lin < os.size; ++lin) {
+        int64_t rem = lin, src = 0;
+        for (int i = 0; i < ndim; ++i) { int64_t oi = rem / os.v[i]; rem %= os.v[i]; src += (oi / reps[i]) * is.v[i]; }
+        out[lin] = in[src];
+    }
+    return OK;
+}
+
+#define DISPATCH_RAW(dtype, CALL)                 \
+    switch (esize(dtype)) {                       \
+    case 8: return CALL(uint64_t);                \
+    case 4: return CALL(uint32_t);                \
+    case 2: return CALL(uint16_t);                \
+    case 1: return CALL(uint8_t);                 \
+    default: return ERR_DTYPE;                    \
+    }
+
+// ---- init: E/init_miaobyte.hpp:16-70.
+template <typename T> int constant_t(void *out_, int64_t n, scalar_t v) {
+    T *out = (T *)out_; T x = scalar_as<T>(v);
+    range_elementwise(n, [&](int64_t lo, int64_t hi) { for (int64_t i = lo; i < hi; ++i) out[i] = x; });
+    return OK;
+}
+// arange, :59-70: data[i] = start + i*step in T's arithmetic (16-bit floats in fp32).
+template <typename T> int arange_t(void *out_, int64_t n, scalar_t s0, scalar_t s1) {
+    T *out = (T *)out_;
+    using A = acc_t<T>;
+    A start = ld(scalar_as<T>(s0)), step = ld(scalar_as<T>(s1));
+    range_elementwise(n, [&](int64_t lo, int64_t hi) {
+        for (int64_t i = lo; i < hi; ++i) {
+            if constexpr (std::is_integral_v<A>) st(out[i], wadd<A>(start, wmul<A>(A(i), step)));
+            else st(out[i], start + A(i) * step);
+        }
+    });
+    return OK;
+}
+
+// ---- matmul: E/matmul_cblas.hpp:11-60 — per batch cblas_sgemm(RowMajor, NoTrans, NoTrans,
+// m,n,k, 1, A,k, B,n, 0, C,n).  OpenBLAS is third party (unpinned version; apt
+// libopenblas-dev, executor/op-ompsimd/Dockerfile:7), so its summation order is not
+// restated: floating types accumulate in float64 and round once, the anchor the
+// tolerance rel 1e-5*sqrt(K) (fp32) / 1e-2 (bf16) is measured from.
+template <typename T> int matmul_t(const void *a_, const void *b_, void *c_, int64_t batch, int64_t m, int64_t k, int64_t n) {
+    const T *A = (const T *)a_; const T *B = (const T *)b_; T *C = (T *)c_;
+    using A_t = acc_t<T>;
+    using Acc = std::conditional_t<std::is_integral_v<A_t>, A_t, double>;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int64_t bi = 0; bi < batch; ++bi) {
+        for (int64_t i = 0; i < m; ++i) {
+            std::vector<Acc> row(n, Acc(0));
+            const T *a = A + (bi * m + i) * k;
+            for (int64_t p = 0; p < k; ++p) {
+                Acc av = Acc(ld(a[p]));
+                const T *b = B + (bi * k + p) * n;
+                for (int64_t j = 0; j < n; ++j) {
+                    if constexpr (std::is_integral_v<A_t>) row[j] = wadd<A_t>(row[j], wmul<A_t>(av, ld(b[j])));
+                    else row[j] += av * Acc(ld(b[j]));
+                }
+            }
+            T *c = C + (bi * m + i) * n;
+            for (int64_t j = 0; j < n; ++j) {
+                if constexpr (std::is_same_v<T, bf16> || std::is_same_v<T, f16>) st(c[j], f64_to_f32_round_odd(row[j]));
+                else st(c[j], A_t(row[j]));
+            }
+        }
+    }
+    return OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int orc_num_threads(void) { return omp_get_max_threads(); }
+
+#define CALL_BIN(OP) [&]() -> int {                                  \
+        switch (dtype) {                                             \
+        case F64: return binary_t<OP, double>(a, b, c, n);           \
+        case F32: return binary_t<OP, float>(a, b, c, n);            \
+        case F16: return binary_t<OP, f16>(a, b, c, n);              \
+        case BF16: return binary_t<OP, bf16>(a, b, c, n);            \
+        case I64: return binary_t<OP, int64_t>(a, b, c, n);          \
+        case I32: return binary_t<OP, int32_t>(a, b, c, n);          \
+        case I16: return binary_t<OP, int16_t>(a, b, c, n);          \
+        case I8: return binary_t<OP, int8_t>(a, b, c, n);            \
+        default: return ERR_DTYPE; } }()
+#define CALL_SCL(OP) [&]() -> int {                                  \
+        switch (dtype) {                                             \
+        case F64: return scalar_op_t<OP, double>(a, s, c, n);        \
+        case F32: return scalar_op_t<OP, float>(a, s, c, n);         \
+        case F16: return scalar_op_t<OP, f16>(a, s, c, n);           \
+        case BF16: return scalar_op_t<OP, bf16>(a, s, c, n);         \
+        case I64: return scalar_op_t<OP, int64_t>(a, s, c, n);       \
+        case I32: return scalar_op_t<OP, int32_t>(a, s, c, n);       \
+        case I16: return scalar_op_t<OP, int16_t>(a, s, c, n);       \
+        case I8: return scalar_op_t<OP, int8_t>(a, s, c, n);         \
+        default: return ERR_DTYPE; } }()
+
+int orc_add(int dtype, const void *a, const void *b, void *c, int64_t n) { return CALL_BIN(ADD); }
+int orc_sub(int dtype, const void *a, const void *b, void *c, int64_t n) { return CALL_BIN(SUB); }
+int orc_mul(int dtype, const void *a, const void *b, void *c, int64_t n) { return CALL_BIN(MUL); }
+int orc_div(int dtype, const void *a, const void *b, void *c, int64_t n) { return CALL_BIN(DIV); }
+int orc_max(int dtype, const void *a, const void *b, void *c, int64_t n) { return CALL_BIN(MAX); }
+int orc_min(int dtype, const void *a, const void *b, void *c, int64_t n) { return CALL_BIN(MIN); }
+int orc_pow(int dtype, const void *a, const void *b, void *c, int64_t n) {
+    switch (dtype) {
+    case F64: return binary_t<POW, double>(a, b, c, n);
+    case F32: return binary_t<POW, float>(a, b, c, n);
+    default: return ERR_DTYPE;
+    }
+}
+int orc_addscalar(int dtype, const void *a, scalar_t s, void *c, int64_t n) { return CALL_SCL(ADD); }
+int orc_subscalar(int dtype, const void *a, scalar_t s, void *c, int64_t n) { return CALL_SCL(SUB); }
+int orc_rsubscalar(int dtype, scalar_t s, const void *a, void *c, int64_t n) { return CALL_SCL(RSUB); }
+int orc_mulscalar(int dtype, const void *a, scalar_t s, void *c, int64_t n) { return CALL_SCL(MUL); }
+int orc_divscalar(int dtype, const void *a, scalar_t s, void *c, int64_t n) { return CALL_SCL(DIV); }
+int orc_rdivscalar(int dtype, scalar_t s, const void *a, void *c, int64_t n) { return CALL_SCL(RDIV); }
+int orc_maxscalar(int dtype, const void *a, scalar_t s, void *c, int64_t n) { return CALL_SCL(MAX); }
+int orc_minscalar(int dtype, const void *a, scalar_t s, void *c, int64_t n) { return CALL_SCL(MIN); }
+int orc_powscalar(int dtype, const void *a, scalar_t s, void *c, int64_t n) {
+    switch (dtype) {
+    case F64: return scalar_op_t<POW, double>(a, s, c, n);
+    case F32: return scalar_op_t<POW, float>(a, s, c, n);
+    default: return ERR_DTYPE;
+    }
+}
+int orc_rpowscalar(int dtype, scalar_t s, const void *a, void *c, int64_t n) {
+    switch (dtype) {
+    case F64: return scalar_op_t<RPOW, double>(a, s, c, n);
+    case F32: return scalar_op_t<RPOW, float>(a, s, c, n);
+    default: return ERR_DTYPE;
+    }
+}
+
+#define UN_FLOAT(OP) switch (dtype) {                          \
+    case F64: return unary_t<OP, double>(a, c, n);             \
+    case F32: return unary_t<OP, float>(a, c, n);              \
+    case F16: return unary_t<OP, f16>(a, c, n);                \
+    case BF16: return unary_t<OP, bf16>(a, c, n);              \
+    default: return ERR_DTYPE; }
+int orc_sqrt(int dtype, const void *a, void *c, int64_t n) { UN_FLOAT(SQRT) }
+int orc_exp(int dtype, const void *a, void *c, int64_t n) { UN_FLOAT(EXP) }
+int orc_log(int dtype, const void *a, void *c, int64_t n) { UN_FLOAT(LOG) }
+int orc_sin(int dtype, const void *a, void *c, int64_t n) { UN_FLOAT(SIN) }
+int orc_cos(int dtype, const void *a, void *c, int64_t n) { UN_FLOAT(COS) }
+int orc_tan(int dtype, const void *a, void *c, int64_t n) {
+    switch (dtype) {
+    case F64: return unary_t<TAN, double>(a, c, n);
+    case F32: return unary_t<TAN, float>(a, c, n);
+    default: return ERR_DTYPE;
+    }
+}
+// invert, E/elementwise_miaobyte.hpp:321-361: ~x for integers, !x for bool.
+int orc_invert(int dtype, const void *a_, void *c_, int64_t n) {
+    int es = esize(dtype);
+    if (dtype == BOOL) {
+        const uint8_t *a = (const uint8_t *)a_; uint8_t *c = (uint8_t *)c_;
+        for (int64_t i = 0; i < n; ++i) c[i] = a[i] ? 0 : 1;
+        return OK;
+    }
+    if (!(dtype == I64 || dtype == I32 || dtype == I16 || dtype == I8)) return ERR_DTYPE;
+    const uint8_t *a = (const uint8_t *)a_; uint8_t *c = (uint8_t *)c_;
+    for (int64_t i = 0; i < n * es; ++i) c[i] = uint8_t(~a[i]);
+    return OK;
+}
+
+int orc_todtype(int src, const void *a, int dst, void *c, int64_t n) {
+    if (src == dst) { std::memcpy(c, a, size_t(n) * esize(src)); return esize(src) ? OK : ERR_DTYPE; }
+    switch (src) {
+    case F64: return cast_from<double>(a, dst, c, n);
+    case F32: return cast_from<float>(a, dst, c, n);
+    case F16: return cast_from<f16>(a, dst, c, n);
+    case BF16: return cast_from<bf16>(a, dst, c, n);
+    case I64: return cast_from<int64_t>(a, dst, c, n);
+    case I32: return cast_from<int32_t>(a, dst, c, n);
+    case I16: return cast_from<int16_t>(a, dst, c, n);
+    case I8: return cast_from<int8_t>(a, dst, c, n);
+    default: return ERR_DTYPE;
+    }
+}
+
+#define CMP_ALL(OP, B, BS, S, EPS) switch (dtype) {                                     \
+    case F64: return compare_t<OP, double>(a, B, BS, S, EPS, m, n);                     \
+    case F32: return compare_t<OP, float>(a, B, BS, S, EPS, m, n);                      \
+    case F16: return compare_t<OP, f16>(a, B, BS, S, EPS, m, n);                        \
+    case BF16: return compare_t<OP, bf16>(a, B, BS, S, EPS, m, n);                      \
+    case I64: return compare_t<OP, int64_t>(a, B, BS, S, EPS, m, n);                    \
+    case I32: return compare_t<OP, int32_t>(a, B, BS, S, EPS, m, n);                    \
+    case I16: return compare_t<OP, int16_t>(a, B, BS, S, EPS, m, n);                    \
+    case I8: return compare_t<OP, int8_t>(a, B, BS, S, EPS, m, n);                      \
+    default: return ERR_DTYPE; }
+static const scalar_t kNoScalar = {0.0, 0};
+int orc_equal(int dtype, const void *a, const void *b, float eps, void *m, int64_t n) { CMP_ALL(EQ, b, false, kNoScalar, eps) }
+int orc_notequal(int dtype, const void *a, const void *b, float eps, void *m, int64_t n) { CMP_ALL(NE, b, false, kNoScalar, eps) }
+int orc_equalscalar(int dtype, const void *a, scalar_t s, float eps, void *m, int64_t n) { CMP_ALL(EQ, a, true, s, eps) }
+int orc_notequalscalar(int dtype, const void *a, scalar_t s, float eps, void *m, int64_t n) { CMP_ALL(NE, a, true, s, eps) }
+int orc_less(int dtype, const void *a, const void *b, void *m, int64_t n) { CMP_ALL(LT, b, false, kNoScalar, 0.f) }
+int orc_greater(int dtype, const void *a, const void *b, void *m, int64_t n) { CMP_ALL(GT, b, false, kNoScalar, 0.f) }
+int orc_lessscalar(int dtype, const void *a, scalar_t s, void *m, int64_t n) { CMP_ALL(LT, a, true, s, 0.f) }
+int orc_greaterscalar(int dtype, const void *a, scalar_t s, void *m, int64_t n) { CMP_ALL(GT, a, true, s, 0.f) }
+
+int orc_switch(int dtype, const void *const *tensors, int nt, int cases_dtype, const void *cases, void *c, int64_t n) {
+    if (nt < 1) return ERR_ARG;
+#define SW(R) switch_t<R>(tensors, nt, cases_dtype, cases, c, n)
+    DISPATCH_RAW(dtype, SW)
+#undef SW
+}
+
+#define RED_ALL(OP) switch (dtype) {                                                 \
+    case F64: return reduce_t<OP, double>(in, shape, ndim, dims, ndims, out);        \
+    case F32: return reduce_t<OP, float>(in, shape, ndim, dims, ndims, out);         \
+    case F16: return reduce_t<OP, f16>(in, shape, ndim, dims, ndims, out);           \
+    case BF16: return reduce_t<OP, bf16>(in, shape, ndim, dims, ndims, out);         \
+    case I64: return reduce_t<OP, int64_t>(in, shape, ndim, dims, ndims, out);       \
+    case I32: return reduce_t<OP, int32_t>(in, shape, ndim, dims, ndims, out);       \
+    case I16: return reduce_t<OP, int16_t>(in, shape, ndim, dims, ndims, out);       \
+    case I8: return reduce_t<OP, int8_t>(in, shape, ndim, dims, ndims, out);         \
+    default: return ERR_DTYPE; }
+int orc_sum(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims, int ndims, void *out) { RED_ALL(RSUM) }
+int orc_prod(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims, int ndims, void *out) { RED_ALL(RPROD) }
+int orc_reducemax(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims, int ndims, void *out) { RED_ALL(RMAX) }
+int orc_reducemin(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims, int ndims, void *out) { RED_ALL(RMIN) }
+
+// reducedShape + reducedDim, executor/deepxcore/src/deepx/shape_reduce.cpp:47-85, literally:
+// `dims` are already-checked (non-negative) axes and an EMPTY list marks nothing as reduced
+// (the "all axes" rule lives in checkedDims, which callers apply first).  Returns the
+// output rank (>=1) or a negative error; out_shape must hold max(ndim,1) entries.
+int orc_reduced_shape(const int32_t *shape, int ndim, const int32_t *dims, int ndims, int keepdims, int32_t *out_shape) {
+    std::vector<int> red(ndim, 0);
+    for (int i = 0; i < ndims; ++i) {
+        if (dims[i] < 0 || dims[i] >= ndim) return ERR_ARG;
+        red[dims[i]] = 1;
+    }
+    int j = 0;
+    for (int i = 0; i < ndim; ++i) {
+        if (!red[i]) out_shape[j++] = shape[i];
+        else if (keepdims) out_shape[j++] = 1;
+    }
+    if (j == 0) out_shape[j++] = 1;
+    return j;
+}
+
+// checkedDims, shape_reduce.cpp:11-45: negative axes normalised, sorted, de-duplicated; an empty
+// list becomes every axis.  Returns the count written to out_dims, or a negative error.
+int orc_checked_dims(int ndim, const int32_t *dims, int ndims, int32_t *out_dims) {
+    std::vector<int> red;
+    if (!checked_dims(ndim, dims, ndims, red)) return ERR_ARG;
+    int j = 0;
+    for (int i = 0; i < ndim; ++i) if (red[i]) out_dims[j++] = i;
+    return j;
+}
+
+// op: 0 sum, 1 prod, 2 reducemax, 3 reducemin — the reference's per-element decomposition.
+int orc_faithful_reduce_f32(int op, const float *in, const int32_t *shape, int ndim, const int32_t *dims,
+                            int ndims, int keepdims, float *out) {
+    switch (op) {
+    case 0: return reduce_faithful_f32<RSUM>(in, shape, ndim, dims, ndims, keepdims != 0, out);
+    case 1: return reduce_faithful_f32<RPROD>(in, shape, ndim, dims, ndims, keepdims != 0, out);
+    case 2: return reduce_faithful_f32<RMAX>(in, shape, ndim, dims, ndims, keepdims != 0, out);
+    case 3: return reduce_faithful_f32<RMIN>(in, shape, ndim, dims, ndims, keepdims != 0, out);
+    default: return ERR_ARG;
+    }
+}
+
+int orc_transpose(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *order, void *out) {
+#define TR(R) transpose_t<R>(in, shape, ndim, order, out)
+    DISPATCH_RAW(dtype, TR)
+#undef TR
+}
+int orc_concat(int dtype, const void *const *ins, int nins, const int32_t *axis_sizes, const int32_t *out_shape,
+               int ndim, int axis, void *out) {
+#define CC(R) concat_t<R>(ins, nins, axis_sizes, out_shape, ndim, axis, out)
+    DISPATCH_RAW(dtype, CC)
+#undef CC
+}
+int orc_broadcastTo(int dtype, const void *in, const int32_t *ishape, int indim, const int32_t *oshape, int ondim, void *out) {
+#define BC(R) broadcast_t<R>(in, ishape, indim, oshape, ondim, out)
+    DISPATCH_RAW(dtype, BC)
+#undef BC
+}
+int orc_indexselect(int dtype, const void *in, const int32_t *ishape, int indim, int index_dtype, const void *index,
+                    const int32_t *xshape, int xndim, int axis, void *out) {
+    if (index_dtype == I64) {
+#define IS(R) indexselect_t<R, int64_t>(in, ishape, indim, index, xshape, xndim, axis, out)
+        DISPATCH_RAW(dtype, IS)
+#undef IS
+    } else if (index_dtype == I32) {
+#define IS(R) indexselect_t<R, int32_t>(in, ishape, indim, index, xshape, xndim, axis, out)
+        DISPATCH_RAW(dtype, IS)
+#undef IS
+    }
+    return ERR_DTYPE;
+}
+int orc_repeat(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *reps, void *out) {
+#define RP(R) repeat_t<R>(in, shape, ndim, reps, out)
+    DISPATCH_RAW(dtype, RP)
+#undef RP
+}
+
+int orc_constant(int dtype, void *out, int64_t n, scalar_t v) {
+    if (dtype == BOOL) { std::memset(out, v.i ? 1 : 0, size_t(n)); return OK; }
+#define CT(T) constant_t<T>(out, n, v)
+    DISPATCH_ALL(dtype, CT)
+#undef CT
+}
+int orc_arange(int dtype, void *out, int64_t n, scalar_t start, scalar_t step) {
+#define AR(T) arange_t<T>(out, n, start, step)
+    DISPATCH_ALL(dtype, AR)
+#undef AR
+}
+int orc_matmul(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n) {
+#define MM(T) matmul_t<T>(a, b, c, batch, m, k, n)
+    DISPATCH_ALL(dtype, MM)
+#undef MM
+}
+
+// conversions exposed so the tests can pin them against numpy float16 / torch bfloat16
+uint16_t orc_f32_to_bf16(float f) { return f32_to_bf16(f).bits; }
+uint16_t orc_f32_to_f16(float f) { return f32_to_f16(f).bits; }
+float orc_bf16_to_f32(uint16_t h) { return bf16_to_f32(bf16{h}); }
+float orc_f16_to_f32(uint16_t h) { return f16_to_f32(f16{h}); }
+
+}  // extern "C"

@@ -1,0 +1,81 @@
+"""GPU parity: matmul vs the oracle (float64 accumulation) and the reference's known answer.
+
+Bars: fp32/f64 within rel 1e-5*sqrt(K) (f64: 1e-13*sqrt(K)) of |A||B| row-column magnitude;
+bf16/f16 (MFMA, fp32 accumulate, one rounding) within rel 1e-2; integers bit-exact.
+"""
+import numpy as np
+import pytest
+
+from deepx_amd import lib as dx
+from tests import helpers as H
+from tests.helpers import Dev, hp
+
+pytestmark = pytest.mark.gpu
+
+
+def run(dxh, orc, dtype, A, B, batch, m, k, n):
+    dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, A.dtype)
+    dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+    want = np.empty(batch * m * n, dtype=A.dtype)
+    assert orc.orc_matmul(dtype, hp(A), hp(B), hp(want), batch, m, k, n) == 0
+    return dC.get(), want
+
+
+SHAPES = [(1, 1, 1, 1), (1, 3, 4, 5), (2, 3, 4, 5), (1, 64, 64, 64), (1, 128, 32, 128), (3, 130, 70, 150),
+          (1, 257, 129, 65), (2, 31, 200, 17), (1, 256, 896, 384)]
+
+
+@pytest.mark.parametrize("dtype", [dx.F32, dx.F64, dx.BF16, dx.F16])
+def test_matmul_float(dxh, orc, dtype):
+    rng = np.random.default_rng(90 + dtype)
+    for batch, m, k, n in SHAPES:
+        A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
+        B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
+        got, want = run(dxh, orc, dtype, A, B, batch, m, k, n)
+        g, w = H.to_float(got, dtype), H.to_float(want, dtype)
+        Af = np.abs(H.to_float(A, dtype)).reshape(batch, m, k)
+        Bf = np.abs(H.to_float(B, dtype)).reshape(batch, k, n)
+        mag = np.matmul(Af, Bf).reshape(-1)  # sum_k |a||b|: the scale rounding errors grow with
+        rel = {dx.F32: 1e-5 * np.sqrt(k), dx.F64: 1e-13 * np.sqrt(k), dx.BF16: 1e-2, dx.F16: 1e-2}[dtype]
+        assert np.all(np.abs(g - w) <= rel * np.maximum(mag, 1e-30)), (dtype, batch, m, k, n, np.max(np.abs(g - w) / np.maximum(mag, 1e-30)))
+
+
+@pytest.mark.parametrize("dtype", H.INTS)
+def test_matmul_int_exact(dxh, orc, dtype):
+    rng = np.random.default_rng(95 + dtype)
+    for batch, m, k, n in SHAPES[:7]:
+        A = rng.integers(-5, 6, batch * m * k).astype(H.NP[dtype])
+        B = rng.integers(-5, 6, batch * k * n).astype(H.NP[dtype])
+        got, want = run(dxh, orc, dtype, A, B, batch, m, k, n)
+        assert np.array_equal(got, want)
+
+
+def test_matmul_reference_known_answer(dxh):
+    """arange(24).reshape(2,3,4) @ arange(40).reshape(2,4,5), the expectation held in
+    executor/op-ompsimd/test/tensorfunc/4_tensor_matmul.cpp:18-36."""
+    A = np.arange(24, dtype=np.float32)
+    B = np.arange(40, dtype=np.float32)
+    dA, dB, dC = Dev(A), Dev(B), Dev.empty(30, np.float32)
+    dx.check(dxh.dxh_matmul(dx.F32, dA.ptr, dB.ptr, dC.ptr, 2, 3, 4, 5, None))
+    want = np.array([[[70, 76, 82, 88, 94], [190, 212, 234, 256, 278], [310, 348, 386, 424, 462]],
+                     [[1510, 1564, 1618, 1672, 1726], [1950, 2020, 2090, 2160, 2230], [2390, 2476, 2562, 2648, 2734]]],
+                    dtype=np.float32)
+    assert np.array_equal(dC.get().reshape(2, 3, 5), want)
+
+
+def test_config5_gemm_shapes_bf16(dxh, orc):
+    """BASELINE config 5 GEMM shapes, bf16 in / fp32 accumulate / bf16 out, checked against
+    float64 numpy on a row sample (the oracle's triple loop is too slow at full size)."""
+    rng = np.random.default_rng(14)
+    for (m, k, n), seed in [((2048, 896, 4864), 15), ((2048, 4864, 896), 17)]:
+        A = H.f32_to_bf16_bits(rng.standard_normal(m * k).astype(np.float32))
+        B = H.f32_to_bf16_bits(np.random.default_rng(seed).standard_normal(k * n).astype(np.float32) * 0.02)
+        dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, np.uint16)
+        dx.check(dxh.dxh_matmul(dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+        got = H.bf16_bits_to_f32(dC.get()).reshape(m, n).astype(np.float64)
+        rows = rng.choice(m, 64, replace=False)
+        Af = H.bf16_bits_to_f32(A).reshape(m, k).astype(np.float64)[rows]
+        Bf = H.bf16_bits_to_f32(B).reshape(k, n).astype(np.float64)
+        ref = Af @ Bf
+        mag = np.abs(Af) @ np.abs(Bf)
+        assert np.all(np.abs(got[rows] - ref) <= 1e-2 * mag)

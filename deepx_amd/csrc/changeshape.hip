@@ -21,7 +21,7 @@
 
 namespace dxh {
 
-constexpr int kGatherUnroll = 4;
+constexpr int kGatherUnroll = 1;  // one unit per lane, one tile per workgroup: fastest measured copy shape
 constexpr int kMaxOuter = DXH_MAX_DIMS;
 
 struct OuterDims {
@@ -42,7 +42,7 @@ inline int unit_bytes(int64_t run_bytes, std::initializer_list<const void *> ptr
 // out is [rows, Lu] units, contiguous.  in row start = sum_i idx_i * stride_i (units) where idx
 // is the mixed-radix decomposition of the row number over `od`.  SPLAT: the input contributes a
 // single element of type E per row position (innermost axis broadcast) that fills the unit.
-template <typename U, typename I, bool SPLAT, typename E>
+template <typename U, typename I, bool SPLAT, typename E, bool REUSE>
 __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const void *__restrict__ in_, U *__restrict__ out, I total,
                                                               I Lu, OuterDims od) {
     const I tile = (I)kBlock * kGatherUnroll;
@@ -70,34 +70,46 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const void *__restr
                     for (int k = 0; k < N; ++k) r.v[k] = e;
                     x[u] = __builtin_bit_cast(U, r);
                 } else {
-                    x[u] = reinterpret_cast<const U *>(in_)[off + (int64_t)v];
+                    // REUSE: input rows are read many times (broadcast) and should stay cached
+                    if constexpr (REUSE) x[u] = reinterpret_cast<const U *>(in_)[off + (int64_t)v];
+                    else x[u] = ld_nt(reinterpret_cast<const U *>(in_) + off + (int64_t)v);
                 }
             }
         }
 #pragma unroll
         for (int u = 0; u < kGatherUnroll; ++u)
-            if (g[u] < total) out[g[u]] = x[u];
+            if (g[u] < total) st_nt(&out[g[u]], x[u]);
     }
 }
 
-template <int UB, bool SPLAT, typename E>
+template <int UB, bool SPLAT, typename E, bool REUSE = false>
 int launch_gather_unit(const void *in, void *out, int64_t rows, int64_t Lu, const OuterDims &od, hipStream_t st) {
     using U = typename raw_of<UB>::type;
     const int64_t total = rows * Lu;
-    unsigned grid = stream_grid(total, (int64_t)kBlock * kGatherUnroll, 8);
+    unsigned grid = stream_grid(total, (int64_t)kBlock * kGatherUnroll, 0);
     if (total < (int64_t)1 << 31)
-        gather_rows_kernel<U, uint32_t, SPLAT, E><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint32_t)total, (uint32_t)Lu, od);
+        gather_rows_kernel<U, uint32_t, SPLAT, E, REUSE><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint32_t)total, (uint32_t)Lu, od);
     else
-        gather_rows_kernel<U, uint64_t, SPLAT, E><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint64_t)total, (uint64_t)Lu, od);
+        gather_rows_kernel<U, uint64_t, SPLAT, E, REUSE><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint64_t)total, (uint64_t)Lu, od);
     return launch_status();
 }
 
 // rows x run_bytes bytes per row; od.stride in ELEMENT-of-esize units on entry, converted here
-inline int launch_gather(const void *in, void *out, int64_t rows, int64_t run_elems, int esize, OuterDims od, hipStream_t st) {
+inline int launch_gather(const void *in, void *out, int64_t rows, int64_t run_elems, int esize, OuterDims od, hipStream_t st,
+                         bool reuse = false) {
     if (rows * run_elems == 0) return DXH_OK;
     const int ub = unit_bytes(run_elems * esize, {in, out});
     const int64_t Lu = run_elems * esize / ub;
     for (int d = 0; d < od.n; ++d) od.stride[d] = od.stride[d] * esize / ub;  // strides are multiples of the run
+    if (reuse) {
+        switch (ub) {
+        case 16: return launch_gather_unit<16, false, uint8_t, true>(in, out, rows, Lu, od, st);
+        case 8: return launch_gather_unit<8, false, uint8_t, true>(in, out, rows, Lu, od, st);
+        case 4: return launch_gather_unit<4, false, uint8_t, true>(in, out, rows, Lu, od, st);
+        case 2: return launch_gather_unit<2, false, uint8_t, true>(in, out, rows, Lu, od, st);
+        default: return launch_gather_unit<1, false, uint8_t, true>(in, out, rows, Lu, od, st);
+        }
+    }
     switch (ub) {
     case 16: return launch_gather_unit<16, false, uint8_t>(in, out, rows, Lu, od, st);
     case 8: return launch_gather_unit<8, false, uint8_t>(in, out, rows, Lu, od, st);
@@ -196,13 +208,13 @@ __global__ __launch_bounds__(kBlock) void concat_kernel(ConcatSrcs s, U *__restr
                 int64_t local = g - s.cum[i];
                 int64_t o = local / s.run[i];
                 int64_t v = local - o * s.run[i];
-                x[u] = reinterpret_cast<const U *>(s.ptr[i])[local];
+                x[u] = ld_nt(reinterpret_cast<const U *>(s.ptr[i]) + local);
                 dst[u] = o * out_row + s.pref[i] + v;
             }
         }
 #pragma unroll
         for (int u = 0; u < kGatherUnroll; ++u)
-            if (dst[u] >= 0) out[dst[u]] = x[u];
+            if (dst[u] >= 0) st_nt(&out[dst[u]], x[u]);
     }
 }
 
@@ -229,7 +241,7 @@ __global__ __launch_bounds__(kBlock) void indexselect_kernel(const U *__restrict
         }
 #pragma unroll
         for (int u = 0; u < kGatherUnroll; ++u)
-            if (g[u] < total) out[g[u]] = x[u];
+            if (g[u] < total) st_nt(&out[g[u]], x[u]);
     }
 }
 
@@ -375,7 +387,7 @@ int dxh_concat(int dtype, const void *const *ins, int nins, const int32_t *axis_
         }
         s.cum[s.n] = cum;
         if (s.n == 0 || cum == 0) continue;
-        unsigned grid = stream_grid(cum, (int64_t)kBlock * kGatherUnroll, 8);
+        unsigned grid = stream_grid(cum, (int64_t)kBlock * kGatherUnroll, 0);
         switch (ub) {
         case 16: concat_kernel<uint4><<<grid, kBlock, 0, st>>>(s, (uint4 *)out, out_row, cum); break;
         case 8: concat_kernel<uint64_t><<<grid, kBlock, 0, st>>>(s, (uint64_t *)out, out_row, cum); break;
@@ -429,7 +441,7 @@ int dxh_broadcastTo(int dtype, const void *in, const int32_t *in_shape, int in_n
     od.n = nd - 1;
     int64_t rows = 1;
     for (int i = 0; i < nd - 1; ++i) { od.size[i] = (uint32_t)sz[i]; od.stride[i] = sd[i]; rows *= sz[i]; }
-    if (sd[nd - 1] == 1) return launch_gather(in, out, rows, sz[nd - 1], es, od, st);
+    if (sd[nd - 1] == 1) return launch_gather(in, out, rows, sz[nd - 1], es, od, st, /*reuse=*/true);
     // innermost axis is broadcast: splat one element per row position
     switch (es) {
     case 8: return launch_splat<uint64_t>(in, out, rows, sz[nd - 1], od, st);
@@ -460,7 +472,7 @@ int dxh_indexselect(int dtype, const void *in, const int32_t *in_shape, int in_n
     const int64_t Lu = post * es / ub;
     const int64_t total = pre * m * Lu;
     hipStream_t st = as_stream(stream);
-    unsigned grid = stream_grid(total, (int64_t)kBlock * kGatherUnroll, 8);
+    unsigned grid = stream_grid(total, (int64_t)kBlock * kGatherUnroll, 0);
 #define DXH_IS(U)                                                                                                      \
     if (index_dtype == DXH_I64)                                                                                        \
         indexselect_kernel<U, int64_t><<<grid, kBlock, 0, st>>>((const U *)in, (const int64_t *)index, (U *)out, total, Lu, m, adim); \

@@ -65,6 +65,25 @@ template <> struct raw_of<4> { using type = uint32_t; };
 template <> struct raw_of<8> { using type = uint64_t; };
 template <> struct raw_of<16> { using type = uint4; };
 
+// ---- streaming (non-temporal) global access ------------------------------------------------
+// Every tensor of an elementwise / changeshape / reduce op is touched exactly once, so loads and
+// stores carry the `nt` hint: on MI355X this lifted a streaming add from ~5.0 to ~6.5 TB/s.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+template <int BYTES> struct nt_raw;
+template <> struct nt_raw<1> { using type = uint8_t; };
+template <> struct nt_raw<2> { using type = uint16_t; };
+template <> struct nt_raw<4> { using type = uint32_t; };
+template <> struct nt_raw<8> { using type = uint64_t; };
+template <> struct nt_raw<16> { using type = u32x4_t; };
+template <typename VT> __device__ inline VT ld_nt(const VT *p) {
+    using R = typename nt_raw<sizeof(VT)>::type;
+    return __builtin_bit_cast(VT, __builtin_nontemporal_load(reinterpret_cast<const R *>(p)));
+}
+template <typename VT> __device__ inline void st_nt(VT *p, const VT &v) {
+    using R = typename nt_raw<sizeof(VT)>::type;
+    __builtin_nontemporal_store(__builtin_bit_cast(R, v), reinterpret_cast<R *>(p));
+}
+
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 inline int dtype_size(int dtype) {
@@ -85,7 +104,9 @@ inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s);
 // workgroups per CU so the grid-stride loop keeps every CU's queues full.
 inline unsigned stream_grid(int64_t items, int64_t per_block, int blocks_per_cu) {
     int64_t need = (items + per_block - 1) / per_block;
-    int64_t cap = (int64_t)kCUs * blocks_per_cu;
+    // blocks_per_cu == 0: one tile per workgroup, no grid-stride trips (the fastest shape measured
+    // for pure streaming: the hardware dispatcher balances CUs better than a fixed-stride loop)
+    int64_t cap = blocks_per_cu > 0 ? (int64_t)kCUs * blocks_per_cu : ((int64_t)1 << 30);
     if (need < 1) need = 1;
     return (unsigned)(need < cap ? need : cap);
 }

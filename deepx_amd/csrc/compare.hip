@@ -10,8 +10,8 @@
 
 namespace dxh {
 
-constexpr int kUnrollC = 4;
-constexpr int kBlocksPerCUC = 8;
+constexpr int kUnrollC = 1;
+constexpr int kBlocksPerCUC = 0;
 
 template <int U, typename Body> __device__ inline void tile_loop_c(int64_t nv, Body body) {
     const int64_t tile = (int64_t)kBlock * U;
@@ -68,8 +68,8 @@ __global__ __launch_bounds__(kBlock) void compare_kernel(const T *__restrict__ a
         for (int u = 0; u < kUnrollC; ++u) {
             int64_t j = i + u * kBlock;
             if (decltype(full)::value || j < nv) {
-                x[u] = va[j];
-                if constexpr (!SCALAR) y[u] = vb[j];
+                x[u] = ld_nt(&va[j]);
+                if constexpr (!SCALAR) y[u] = ld_nt(&vb[j]);
             }
         }
 #pragma unroll
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kBlock) void compare_kernel(const T *__restrict__ a
                     if constexpr (SCALAR) bb = sv; else bb = A(load_acc(y[u].v[k]));
                     r.v[k] = cmp_one<K, A>(A(load_acc(x[u].v[k])), bb, eps);
                 }
-                vm[j] = r;
+                st_nt(&vm[j], r);
             }
         }
     });
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(kBlock) void switch_bool_kernel(const R *__restrict
 #pragma unroll
         for (int u = 0; u < kUnrollC; ++u) {
             int64_t j = i + u * kBlock;
-            if (decltype(full)::value || j < nv) { x[u] = v0[j]; y[u] = v1[j]; w[u] = vm[j]; }
+            if (decltype(full)::value || j < nv) { x[u] = ld_nt(&v0[j]); y[u] = ld_nt(&v1[j]); w[u] = ld_nt(&vm[j]); }
         }
 #pragma unroll
         for (int u = 0; u < kUnrollC; ++u) {
@@ -160,7 +160,7 @@ __global__ __launch_bounds__(kBlock) void switch_bool_kernel(const R *__restrict
                 VT r;
 #pragma unroll
                 for (int k = 0; k < V; ++k) r.v[k] = w[u].v[k] ? y[u].v[k] : x[u].v[k];
-                vc[j] = r;
+                st_nt(&vc[j], r);
             }
         }
     });
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(kBlock) void cast_kernel(const S *__restrict__ a, D
 #pragma unroll
         for (int u = 0; u < kUnrollC; ++u) {
             int64_t j = i + u * kBlock;
-            if (decltype(full)::value || j < nv) x[u] = va[j];
+            if (decltype(full)::value || j < nv) x[u] = ld_nt(&va[j]);
         }
 #pragma unroll
         for (int u = 0; u < kUnrollC; ++u) {
@@ -261,7 +261,7 @@ __global__ __launch_bounds__(kBlock) void cast_kernel(const S *__restrict__ a, D
                 VD r;
 #pragma unroll
                 for (int k = 0; k < V; ++k) r.v[k] = cast_elem<D, S>(x[u].v[k]);
-                vc[j] = r;
+                st_nt(&vc[j], r);
             }
         }
     });

@@ -1,17 +1,17 @@
 // elementwise.hip — streaming elementwise kernels of libdxhip (gfx950).
 //
-// Every op here is HBM-bound: one 16-byte global load per lane per operand
-// (global_load_dwordx4), UNROLL independent vectors in flight per lane, a grid-stride
-// loop over workgroup tiles of 256*UNROLL vectors, and a grid capped at a few resident
-// workgroups per CU.  Arithmetic follows executor/op-ompsimd's
+// Every op here is HBM-bound: one 16-byte non-temporal global load per lane per operand
+// (global_load_dwordx4 ... nt), one 16-byte non-temporal store, one tile of 256 vectors per
+// workgroup and as many workgroups as tiles (measured fastest on MI355X against unrolled
+// grid-stride variants: 6.5 TB/s vs 5.0 TB/s for a 3-stream add).  Arithmetic follows executor/op-ompsimd's
 // tensorfunc/elementwise_miaobyte.hpp (cited per op in include/dxhip.h); 16-bit floats
 // compute in fp32 and round once.
 #include "common.hpp"
 
 namespace dxh {
 
-constexpr int kUnroll = 4;
-constexpr int kBlocksPerCU = 8;
+constexpr int kUnroll = 1;       // vectors in flight per lane and operand
+constexpr int kBlocksPerCU = 0;  // 0 = one tile per workgroup (see stream_grid)
 
 // ---- op functors on the accumulate type -----------------------------------------------
 template <typename A> __device__ inline A wrap_add(A a, A b) { using U = std::make_unsigned_t<A>; return A(U(U(a) + U(b))); }
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a,
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             int64_t j = i + u * kBlock;
-            if (decltype(full)::value || j < nv) { x[u] = va[j]; y[u] = vb[j]; }
+            if (decltype(full)::value || j < nv) { x[u] = ld_nt(&va[j]); y[u] = ld_nt(&vb[j]); }
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a,
                 VT r;
 #pragma unroll
                 for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(A(load_acc(x[u].v[k])), A(load_acc(y[u].v[k]))));
-                vc[j] = r;
+                st_nt(&vc[j], r);
             }
         }
     });
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(kBlock) void scalar_kernel(const T *__restrict__ a,
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             int64_t j = i + u * kBlock;
-            if (decltype(full)::value || j < nv) x[u] = va[j];
+            if (decltype(full)::value || j < nv) x[u] = ld_nt(&va[j]);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kBlock) void scalar_kernel(const T *__restrict__ a,
                 VT r;
 #pragma unroll
                 for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(A(load_acc(x[u].v[k])), sv));
-                vc[j] = r;
+                st_nt(&vc[j], r);
             }
         }
     });
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kBlock) void unary_kernel(const T *__restrict__ a, 
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             int64_t j = i + u * kBlock;
-            if (decltype(full)::value || j < nv) x[u] = va[j];
+            if (decltype(full)::value || j < nv) x[u] = ld_nt(&va[j]);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(kBlock) void unary_kernel(const T *__restrict__ a, 
                 VT r;
 #pragma unroll
                 for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(load_acc(x[u].v[k])));
-                vc[j] = r;
+                st_nt(&vc[j], r);
             }
         }
     });

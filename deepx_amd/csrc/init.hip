@@ -13,7 +13,7 @@ __global__ __launch_bounds__(kBlock) void constant_kernel(T *__restrict__ out, i
     for (int k = 0; k < V; ++k) r.v[k] = value;
     VT *vo = reinterpret_cast<VT *>(out);
     const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nv; i += stride) vo[i] = r;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nv; i += stride) st_nt(&vo[i], r);
     if (blockIdx.x == 0) {
         int64_t j = nv * V + threadIdx.x;
         if (j < n) out[j] = value;
@@ -41,7 +41,7 @@ template <typename T> int launch_constant(void *out, int64_t n, dxh_scalar v, hi
     T x;
     if constexpr (std::is_same_v<T, bool_t>) x = bool_t{uint8_t(v.i ? 1 : 0)}; else x = scalar_to<T>(v);
     if (aligned(out, kVecBytes)) {
-        unsigned g = stream_grid(n / V + 1, kBlock, 16);
+        unsigned g = stream_grid(n / V + 1, kBlock, 0);
         constant_kernel<T, V><<<g, kBlock, 0, st>>>((T *)out, n, x);
     } else {
         unsigned g = stream_grid(n, kBlock, 16);

@@ -100,8 +100,20 @@ __global__ __launch_bounds__(kBlock) void reduce_row_kernel(const Tin *__restric
         const VT *pv = reinterpret_cast<const VT *>(p);
         const int64_t lv = len / V;
         int64_t i = lane;
+        // 8 independent 16-byte non-temporal loads in flight per lane, then 4, then singles
+        for (; i + 7 * (int64_t)G < lv; i += 8 * (int64_t)G) {
+            VT x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) x[u] = ld_nt(&pv[i + u * (int64_t)G]);
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                A t0 = rop<K, A>(rop<K, A>(rload<A>(x[0].v[k]), rload<A>(x[1].v[k])), rop<K, A>(rload<A>(x[2].v[k]), rload<A>(x[3].v[k])));
+                A t1 = rop<K, A>(rop<K, A>(rload<A>(x[4].v[k]), rload<A>(x[5].v[k])), rop<K, A>(rload<A>(x[6].v[k]), rload<A>(x[7].v[k])));
+                acc[k] = rop<K, A>(acc[k], rop<K, A>(t0, t1));
+            }
+        }
         for (; i + 3 * (int64_t)G < lv; i += 4 * (int64_t)G) {
-            VT x0 = pv[i], x1 = pv[i + G], x2 = pv[i + 2 * (int64_t)G], x3 = pv[i + 3 * (int64_t)G];
+            VT x0 = ld_nt(&pv[i]), x1 = ld_nt(&pv[i + G]), x2 = ld_nt(&pv[i + 2 * (int64_t)G]), x3 = ld_nt(&pv[i + 3 * (int64_t)G]);
 #pragma unroll
             for (int k = 0; k < V; ++k) {
                 A t0 = rop<K, A>(rload<A>(x0.v[k]), rload<A>(x1.v[k]));
@@ -110,7 +122,7 @@ __global__ __launch_bounds__(kBlock) void reduce_row_kernel(const Tin *__restric
             }
         }
         for (; i < lv; i += G) {
-            VT x = pv[i];
+            VT x = ld_nt(&pv[i]);
 #pragma unroll
             for (int k = 0; k < V; ++k) acc[k] = rop<K, A>(acc[k], rload<A>(x.v[k]));
         }
@@ -163,17 +175,19 @@ __global__ __launch_bounds__(kBlock) void reduce_col_kernel(const Tin *__restric
         const int64_t r1 = (r0 + chunk < R) ? r0 + chunk : R;
         const VT *base = reinterpret_cast<const VT *>(in + p * R * post) + cv;
         int64_t r = r0 + ty;
-        for (; r + 3 * (int64_t)TY < r1; r += 4 * (int64_t)TY) {
-            VT x0 = base[r * postv], x1 = base[(r + TY) * postv], x2 = base[(r + 2 * TY) * postv], x3 = base[(r + 3 * TY) * postv];
+        for (; r + 7 * (int64_t)TY < r1; r += 8 * (int64_t)TY) {
+            VT x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) x[u] = ld_nt(&base[(r + u * (int64_t)TY) * postv]);
 #pragma unroll
             for (int k = 0; k < V; ++k) {
-                A t0 = rop<K, A>(rload<A>(x0.v[k]), rload<A>(x1.v[k]));
-                A t1 = rop<K, A>(rload<A>(x2.v[k]), rload<A>(x3.v[k]));
+                A t0 = rop<K, A>(rop<K, A>(rload<A>(x[0].v[k]), rload<A>(x[1].v[k])), rop<K, A>(rload<A>(x[2].v[k]), rload<A>(x[3].v[k])));
+                A t1 = rop<K, A>(rop<K, A>(rload<A>(x[4].v[k]), rload<A>(x[5].v[k])), rop<K, A>(rload<A>(x[6].v[k]), rload<A>(x[7].v[k])));
                 acc[k] = rop<K, A>(acc[k], rop<K, A>(t0, t1));
             }
         }
         for (; r < r1; r += TY) {
-            VT x = base[r * postv];
+            VT x = ld_nt(&base[r * postv]);
 #pragma unroll
             for (int k = 0; k < V; ++k) acc[k] = rop<K, A>(acc[k], rload<A>(x.v[k]));
         }

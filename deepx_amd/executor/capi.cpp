@@ -1,0 +1,74 @@
+// capi.cpp — libdxexec.so: the executor's dispatch core behind a C ABI, so a harness (or an
+// embedding scheduler) can feed deepxIR lines without a socket.  Same code path as the UDP binary.
+#include <cstring>
+#include <string>
+#include "executor.hpp"
+
+using namespace deepx;
+
+#define DXE_API extern "C" __attribute__((visibility("default")))
+
+static size_t copy_out(const std::string &s, char *buf, size_t buflen) {
+    if (buf && buflen) {
+        size_t n = s.size() < buflen - 1 ? s.size() : buflen - 1;
+        std::memcpy(buf, s.data(), n);
+        buf[n] = '\0';
+    }
+    return s.size();
+}
+
+DXE_API void *dxe_create(void) { try { return new Executor(); } catch (...) { return nullptr; } }
+DXE_API void dxe_destroy(void *ex) { delete static_cast<Executor *>(ex); }
+// executes one IR line; writes the reply line; returns the reply length (may exceed buflen)
+DXE_API size_t dxe_execute(void *ex, const char *line, char *reply, size_t buflen) {
+    return copy_out(static_cast<Executor *>(ex)->execute(line ? line : ""), reply, buflen);
+}
+// parse + print round trip (no execution): "name(args)->(returns) //metadata", or "error: ..."
+DXE_API size_t dxe_parse(const char *line, char *out, size_t buflen) {
+    try {
+        TF tf(line ? line : "");
+        return copy_out(tf.to_string(true), out, buflen);
+    } catch (const std::exception &e) {
+        return copy_out(std::string("error: ") + e.what(), out, buflen);
+    }
+}
+// which registered signature a call resolves to: "author|signature", or "none: <reason>"
+DXE_API size_t dxe_match(void *ex, const char *line, char *out, size_t buflen) {
+    try {
+        TF call(line ? line : "");
+        std::string why;
+        auto tf = static_cast<Executor *>(ex)->factory.get_tf(call, &why);
+        if (!tf) return copy_out("none: " + why, out, buflen);
+        // report the REGISTERED signature: look it up again without cloning the call's metadata
+        const auto &fam = static_cast<Executor *>(ex)->factory.families.at(call.name);
+        auto ait = fam.by_author.find(call.metadata.author);
+        const std::string author = ait == fam.by_author.end() ? fam.author_order.front() : call.metadata.author;
+        for (const auto &r : fam.by_author.at(author))
+            if (TfFactory::signature_matches(call, *r)) return copy_out(author + "|" + r->to_string(), out, buflen);
+        return copy_out("none", out, buflen);
+    } catch (const std::exception &e) {
+        return copy_out(std::string("error: ") + e.what(), out, buflen);
+    }
+}
+DXE_API size_t dxe_op_table(void *ex, const char *executor_name, char *out, size_t buflen) {
+    return copy_out(static_cast<Executor *>(ex)->factory.print_markdown(executor_name ? executor_name : "op-mem-hip"), out, buflen);
+}
+DXE_API size_t dxe_typedef_roundtrip(const char *text, char *out, size_t buflen) {
+    TypeDef t = typedef_from(text ? text : "");
+    return copy_out(typedef_str(t) + " " + std::to_string((int)t.category) + " " + std::to_string((int)t.precision), out, buflen);
+}
+// tensor metadata as the reference's .shape YAML; "error: ..." if the tensor does not exist
+DXE_API size_t dxe_tensor_yaml(void *ex, const char *name, char *out, size_t buflen) {
+    try {
+        return copy_out(static_cast<Executor *>(ex)->mem.gettensor(name)->shape.to_yaml(), out, buflen);
+    } catch (const std::exception &e) {
+        return copy_out(std::string("error: ") + e.what(), out, buflen);
+    }
+}
+DXE_API size_t dxe_shape_yaml_roundtrip(const char *yaml, char *out, size_t buflen) {
+    try {
+        return copy_out(Shape::from_yaml(yaml).to_yaml(), out, buflen);
+    } catch (const std::exception &e) {
+        return copy_out(std::string("error: ") + e.what(), out, buflen);
+    }
+}

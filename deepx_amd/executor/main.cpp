@@ -1,0 +1,45 @@
+// deepx-executor-hip — the MI355X executor process: a drop-in for executor/op-cuda's and
+// executor/op-ompsimd's `main` (executor/op-cuda/src/client/main.cpp:23-105).
+//   DEEPX_PORT     UDP port (default 9090, op-cuda's port and the front's default endpoint)
+//   DEEPX_DEVICE   HIP device ordinal (default 0)
+//   DEEPX_IR_LOG   1|true: echo every instruction
+//   DEEPX_SYNC     0: reply at launch instead of at completion
+//   DEEPX_OPLIST   path: write the generated op table (markdown) there, as the reference writes
+//                  docs/executor/op-mem-*/list.md at start-up
+#include <csignal>
+#include <cstdlib>
+#include <fstream>
+#include <iostream>
+#include "udpserver.hpp"
+
+static deepx::UdpServer *g_server = nullptr;
+static void on_signal(int) { if (g_server) g_server->stop(); }
+
+int main() {
+    const char *port_env = std::getenv("DEEPX_PORT");
+    const int port = port_env ? std::atoi(port_env) : 9090;
+    const char *dev_env = std::getenv("DEEPX_DEVICE");
+    int count = 0;
+    int rc = dxh_device_count(&count);
+    if (rc != DXH_OK || count == 0) {
+        std::cerr << "deepx-executor-hip: no HIP device (" << dxh_error_string(rc) << "); tensor ops will answer with errors" << std::endl;
+    } else {
+        rc = dxh_set_device(dev_env ? std::atoi(dev_env) : 0);
+        if (rc != DXH_OK) { std::cerr << "dxh_set_device: " << dxh_error_string(rc) << std::endl; return 1; }
+        char name[256];
+        if (dxh_device_name(name, sizeof name) == DXH_OK) std::cerr << "deepx-executor-hip: " << name << std::endl;
+    }
+    deepx::Executor ex;
+    if (const char *oplist = std::getenv("DEEPX_OPLIST")) {
+        std::ofstream md(oplist);
+        if (md.is_open()) md << ex.factory.print_markdown("op-mem-hip");
+    }
+    deepx::UdpServer server(port);
+    if (!server.open()) return 1;
+    g_server = &server;
+    std::signal(SIGINT, on_signal);
+    std::signal(SIGTERM, on_signal);
+    std::cerr << "deepx-executor-hip: listening on udp " << port << std::endl;
+    server.serve(ex);
+    return 0;
+}

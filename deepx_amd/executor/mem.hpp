@@ -1,0 +1,95 @@
+// mem.hpp — the executor's name -> tensor / argument store, HIP flavour.
+//
+// One Mem per process owns every tensor by name (executor/deepxcore/src/deepx/mem/mem.hpp:15-175;
+// the CUDA twin executor/op-cuda/src/deepx/mem/mem_cuda.hpp).  Tensor storage is device memory
+// obtained through the C ABI (dxh_malloc / dxh_free), the counterpart of the alloc/free/copy
+// function pointers the reference installs in Tensor<T> (executor/deepxcore/src/deepx/tensor.hpp:17-37,
+// executor/op-cuda/src/deepx/tensorfunc/tensorlife_miaobyte.hpp:70-85).
+#pragma once
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <variant>
+#include <vector>
+#include "../../include/dxhip.h"
+#include "shape.hpp"
+
+namespace deepx {
+
+struct DxhError : std::runtime_error {
+    int code;
+    DxhError(int c, const std::string &what) : std::runtime_error(what + ": " + dxh_error_string(c)), code(c) {}
+};
+inline void dxh_check(int code, const char *what) { if (code != DXH_OK) throw DxhError(code, what); }
+
+// A device tensor: metadata + an owned HBM allocation.
+struct Tensor {
+    Shape shape;
+    void *data = nullptr;
+
+    Tensor() = default;
+    Tensor(const std::vector<int> &dims, Precision p) : shape(dims, p) {
+        if (precision_bytes(p) == 0) throw std::invalid_argument("unsupported precision: " + precision_str(p));
+        dxh_check(dxh_malloc(&data, (size_t)shape.bytes()), "dxh_malloc");
+    }
+    Tensor(const Tensor &) = delete;
+    Tensor &operator=(const Tensor &) = delete;
+    ~Tensor() { if (data) dxh_free(data); }
+    int dtype() const { return (int)shape.dtype; }  // Precision value == dxh_dtype value
+};
+
+using ArgValue = std::variant<int32_t, int64_t, float, double, bool, std::string, std::vector<int32_t>,
+                              std::vector<int64_t>, std::vector<float>, std::vector<double>, std::vector<std::string>>;
+
+class Mem {
+public:
+    bool existstensor(const std::string &name) const { return tensors_.count(name) != 0; }
+    std::shared_ptr<Tensor> gettensor(const std::string &name) const {
+        auto it = tensors_.find(name);
+        if (it == tensors_.end()) throw std::runtime_error("tensor not found: " + name);
+        return it->second;
+    }
+    // like MemBase::addtensor, an existing name is kept (mem.hpp:66-99) and reported
+    bool addtensor(const std::string &name, std::shared_ptr<Tensor> t) { return tensors_.emplace(name, std::move(t)).second; }
+    void delete_tensor(const std::string &name) { tensors_.erase(name); }
+    void rename_tensor(const std::string &old_name, const std::string &new_name) {
+        auto it = tensors_.find(old_name);
+        if (it == tensors_.end()) throw std::runtime_error("tensor not found: " + old_name);
+        auto t = it->second;
+        tensors_.erase(it);
+        tensors_[new_name] = t;
+    }
+    size_t tensor_count() const { return tensors_.size(); }
+
+    bool existarg(const std::string &name) const { return args_.count(name) != 0; }
+    void setarg(const std::string &name, ArgValue v) { args_[name] = std::move(v); }
+    const ArgValue &getarg(const std::string &name) const {
+        auto it = args_.find(name);
+        if (it == args_.end()) throw std::runtime_error("arg not found: " + name);
+        return it->second;
+    }
+    void clear() { tensors_.clear(); args_.clear(); }
+
+    // reusable device scratch for reductions (grown on demand, never shrunk)
+    void *workspace(size_t bytes) {
+        if (bytes > ws_bytes_) {
+            if (ws_) { dxh_device_sync(); dxh_free(ws_); ws_ = nullptr; ws_bytes_ = 0; }
+            size_t want = std::max<size_t>(bytes, (size_t)4 << 20);
+            dxh_check(dxh_malloc(&ws_, want), "workspace dxh_malloc");
+            ws_bytes_ = want;
+        }
+        return ws_;
+    }
+    size_t workspace_bytes() const { return ws_bytes_; }
+    ~Mem() { tensors_.clear(); if (ws_) dxh_free(ws_); }
+
+private:
+    std::unordered_map<std::string, std::shared_ptr<Tensor>> tensors_;
+    std::unordered_map<std::string, ArgValue> args_;
+    void *ws_ = nullptr;
+    size_t ws_bytes_ = 0;
+};
+
+}  // namespace deepx

@@ -1,0 +1,532 @@
+// ops.cpp — the executor's op table: every deepxIR op, its registered signature and the host
+// wrapper that turns a parsed instruction into one C-ABI kernel call.
+//
+// The table is the union of the reference executors' registrations
+// (executor/op-ompsimd/src/client/tfs.cpp:19-689, executor/op-cuda/src/client/tfs.cpp:20-646; the
+// generated lists docs/executor/op-mem-{ompsimd,cuda}/list.md): same op names, authors, tftypes,
+// argument order, categories and precision masks, so front/py dispatches unchanged.  Where the
+// reference has one TF class per op (executor/op-ompsimd/src/deepx/tf/*.hpp), this file has one
+// table row per op and a handful of wrapper templates keyed by the C-ABI function they call.
+//
+// Behaviour kept from the reference wrappers: dtype is read from the STORED tensors, mismatches
+// give "Type mismatch: a != b"; a missing tensor gives "tensor not found: <name>"; scalars are
+// T(std::stof(text)) or a named arg (tf.hpp:84-125); vectors are "[3 4 5]" (tf.hpp:127-158).
+// The wrapper defects listed against op-ompsimd (PowScalar/MinScalar reading the dtype from the
+// scalar, RSubScalar reading the scalar from the tensor slot) are NOT reproduced: the registered
+// signature and the front's emission order (front/py/deepx/nn/functional/rtf_*.py) are the contract.
+#include <algorithm>
+#include <cctype>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <functional>
+#include <iostream>
+#include "factory.hpp"
+#include "mem.hpp"
+#include "tensorio.hpp"
+
+namespace deepx {
+
+namespace {
+
+using RunFn = std::function<int(const TF &, Mem &, std::string &)>;
+
+class OpTF : public TF {
+public:
+    std::string formula;
+    RunFn fn;
+    int run(Mem &mem, std::string &error) override {
+        try {
+            return fn(*this, mem, error);
+        } catch (const std::exception &e) {  // the reference lets these kill the process; here they become error replies
+            error = e.what();
+            return 1;
+        }
+    }
+    std::string math_formula() const override { return formula; }
+    std::shared_ptr<TF> clone() const override { return std::make_shared<OpTF>(*this); }
+};
+
+void reg(TfFactory &f, const char *name, const char *author, const char *tftype, const char *formula,
+         std::initializer_list<const char *> args, std::initializer_list<const char *> returns, RunFn fn) {
+    auto tf = std::make_shared<OpTF>();
+    tf->name = name;
+    tf->metadata.author = author;
+    tf->tftype = tftype;
+    tf->formula = formula;
+    for (const char *a : args) tf->args.push_back(Param::parse(a));
+    for (const char *r : returns) tf->returns.push_back(Param::parse(r));
+    tf->fn = std::move(fn);
+    f.add_tf(tf);
+}
+
+// ---- argument access -------------------------------------------------------------------------
+std::shared_ptr<Tensor> tensor_of(const Param &p, Mem &mem) { return mem.gettensor(p.textvalue); }
+
+int fail(std::string &error, const std::string &msg) { error = msg; return 1; }
+int hip_result(int rc, const char *op, std::string &error) {
+    if (rc == DXH_OK) return 0;
+    if (rc == DXH_ERR_DTYPE) return fail(error, std::string("Unsupported dtype for ") + op);
+    return fail(error, std::string(op) + ": " + dxh_error_string(rc));
+}
+
+// T(std::stof(text)) for every T when the text parses as a float, else a named arg (tf.hpp:119-124)
+dxh_scalar scalar_of(const Param &p, Mem &mem) {
+    dxh_scalar s{0.0, 0};
+    if (text_is_float(p.textvalue)) {
+        float v = std::stof(p.textvalue);
+        s.f = (double)v;
+        if (std::isnan(v)) s.i = 0;
+        else if (v >= 9.2233720368547758e18f) s.i = INT64_MAX;
+        else if (v <= -9.2233720368547758e18f) s.i = INT64_MIN;
+        else s.i = (int64_t)v;
+        return s;
+    }
+    if (!mem.existarg(p.textvalue)) throw std::runtime_error("arg not found: " + p.textvalue);
+    const ArgValue &a = mem.getarg(p.textvalue);
+    if (auto v = std::get_if<int32_t>(&a)) { s.f = *v; s.i = *v; }
+    else if (auto v = std::get_if<int64_t>(&a)) { s.f = (double)*v; s.i = *v; }
+    else if (auto v = std::get_if<float>(&a)) { s.f = *v; s.i = (int64_t)*v; }
+    else if (auto v = std::get_if<double>(&a)) { s.f = *v; s.i = (int64_t)*v; }
+    else if (auto v = std::get_if<bool>(&a)) { s.f = *v; s.i = *v; }
+    else throw std::runtime_error("arg is not a number: " + p.textvalue);
+    return s;
+}
+int int_of(const Param &p, Mem &mem) { return (int)scalar_of(p, mem).i; }
+float float_of(const Param &p, Mem &mem) { return (float)scalar_of(p, mem).f; }
+
+bool bool_of(const Param &p) {
+    std::string v = p.textvalue;
+    std::transform(v.begin(), v.end(), v.begin(), [](unsigned char c) { return std::tolower(c); });
+    if (v == "true") return true;
+    if (v == "false") return false;
+    throw std::invalid_argument("Invalid bool value:" + p.textvalue);
+}
+std::vector<std::string> words_of(const Param &p) {
+    std::string t = p.textvalue;
+    size_t a = t.find_first_not_of("[]"), b = t.find_last_not_of("[]");
+    t = a == std::string::npos ? "" : t.substr(a, b - a + 1);
+    std::vector<std::string> out;
+    std::istringstream in(t);
+    std::string w;
+    while (in >> w) out.push_back(w);
+    return out;
+}
+// "[3 4 5]" -> ints; an empty list is an error like tf.hpp:146-150; a bare name looks up a vecset vector
+std::vector<int> ints_of(const Param &p, Mem &mem) {
+    auto words = words_of(p);
+    if (words.empty()) throw std::invalid_argument("Invalid argument index");
+    if (words.size() == 1 && !text_is_float(words[0]) && mem.existarg(words[0])) {
+        const ArgValue &a = mem.getarg(words[0]);
+        std::vector<int> out;
+        if (auto v = std::get_if<std::vector<int32_t>>(&a)) out.assign(v->begin(), v->end());
+        else if (auto v = std::get_if<std::vector<int64_t>>(&a)) out.assign(v->begin(), v->end());
+        else throw std::runtime_error("arg is not an int vector: " + words[0]);
+        return out;
+    }
+    std::vector<int> out;
+    for (auto &w : words) out.push_back((int)std::stof(w));
+    return out;
+}
+
+bool same_dtype(std::initializer_list<const Tensor *> ts, std::string &error) {
+    const Tensor *first = *ts.begin();
+    bool ok = true;
+    for (const Tensor *t : ts) ok &= t->shape.dtype == first->shape.dtype;
+    if (!ok) {
+        error = "Type mismatch: ";
+        bool lead = true;
+        for (const Tensor *t : ts) { if (!lead) error += " != "; error += precision_str(t->shape.dtype); lead = false; }
+    }
+    return ok;
+}
+bool same_size(std::initializer_list<const Tensor *> ts, std::string &error) {
+    const Tensor *first = *ts.begin();
+    for (const Tensor *t : ts)
+        if (t->shape.size != first->shape.size) { error = "shape mismatch: " + dims_str(first->shape.shape) + " vs " + dims_str(t->shape.shape); return false; }
+    return true;
+}
+
+// ---- wrapper templates -----------------------------------------------------------------------
+using BinaryFn = int (*)(int, const void *, const void *, void *, int64_t, void *);
+using ScalarFn = int (*)(int, const void *, dxh_scalar, void *, int64_t, void *);
+using RScalarFn = int (*)(int, dxh_scalar, const void *, void *, int64_t, void *);
+using UnaryFn = int (*)(int, const void *, void *, int64_t, void *);
+
+RunFn binary(BinaryFn f, const char *op) {  // (A, B) -> (C)
+    return [f, op](const TF &c, Mem &mem, std::string &error) {
+        auto A = tensor_of(c.args[0], mem), B = tensor_of(c.args[1], mem), C = tensor_of(c.returns[0], mem);
+        if (!same_dtype({A.get(), B.get(), C.get()}, error) || !same_size({A.get(), B.get(), C.get()}, error)) return 1;
+        return hip_result(f(A->dtype(), A->data, B->data, C->data, C->shape.size, nullptr), op, error);
+    };
+}
+RunFn with_scalar(ScalarFn f, const char *op) {  // (A, scalar) -> (C)
+    return [f, op](const TF &c, Mem &mem, std::string &error) {
+        auto A = tensor_of(c.args[0], mem), C = tensor_of(c.returns[0], mem);
+        if (!same_dtype({A.get(), C.get()}, error) || !same_size({A.get(), C.get()}, error)) return 1;
+        return hip_result(f(A->dtype(), A->data, scalar_of(c.args[1], mem), C->data, C->shape.size, nullptr), op, error);
+    };
+}
+RunFn with_rscalar(RScalarFn f, const char *op) {  // (scalar, A) -> (C)
+    return [f, op](const TF &c, Mem &mem, std::string &error) {
+        auto A = tensor_of(c.args[1], mem), C = tensor_of(c.returns[0], mem);
+        if (!same_dtype({A.get(), C.get()}, error) || !same_size({A.get(), C.get()}, error)) return 1;
+        return hip_result(f(A->dtype(), scalar_of(c.args[0], mem), A->data, C->data, C->shape.size, nullptr), op, error);
+    };
+}
+RunFn unary(UnaryFn f, const char *op) {  // (A) -> (C)
+    return [f, op](const TF &c, Mem &mem, std::string &error) {
+        auto A = tensor_of(c.args[0], mem), C = tensor_of(c.returns[0], mem);
+        if (!same_dtype({A.get(), C.get()}, error) || !same_size({A.get(), C.get()}, error)) return 1;
+        return hip_result(f(A->dtype(), A->data, C->data, C->shape.size, nullptr), op, error);
+    };
+}
+bool mask_ok(const Tensor &m, std::string &error) {
+    if (m.shape.dtype != Precision::Bool) { error = "mask must be a bool tensor, got " + precision_str(m.shape.dtype); return false; }
+    return true;
+}
+using CmpEpsFn = int (*)(int, const void *, const void *, float, void *, int64_t, void *);
+using CmpEpsScalarFn = int (*)(int, const void *, dxh_scalar, float, void *, int64_t, void *);
+RunFn compare_eps(CmpEpsFn f, const char *op) {  // (A, B, epsilon) -> (mask)
+    return [f, op](const TF &c, Mem &mem, std::string &error) {
+        auto A = tensor_of(c.args[0], mem), B = tensor_of(c.args[1], mem), M = tensor_of(c.returns[0], mem);
+        if (!same_dtype({A.get(), B.get()}, error) || !mask_ok(*M, error) || !same_size({A.get(), B.get(), M.get()}, error)) return 1;
+        return hip_result(f(A->dtype(), A->data, B->data, float_of(c.args[2], mem), M->data, M->shape.size, nullptr), op, error);
+    };
+}
+RunFn compare_eps_scalar(CmpEpsScalarFn f, const char *op) {  // (A, scalar, epsilon) -> (mask)
+    return [f, op](const TF &c, Mem &mem, std::string &error) {
+        auto A = tensor_of(c.args[0], mem), M = tensor_of(c.returns[0], mem);
+        if (!mask_ok(*M, error) || !same_size({A.get(), M.get()}, error)) return 1;
+        return hip_result(f(A->dtype(), A->data, scalar_of(c.args[1], mem), float_of(c.args[2], mem), M->data, M->shape.size, nullptr), op, error);
+    };
+}
+RunFn compare(BinaryFn f, const char *op) {  // (A, B) -> (mask)
+    return [f, op](const TF &c, Mem &mem, std::string &error) {
+        auto A = tensor_of(c.args[0], mem), B = tensor_of(c.args[1], mem), M = tensor_of(c.returns[0], mem);
+        if (!same_dtype({A.get(), B.get()}, error) || !mask_ok(*M, error) || !same_size({A.get(), B.get(), M.get()}, error)) return 1;
+        return hip_result(f(A->dtype(), A->data, B->data, M->data, M->shape.size, nullptr), op, error);
+    };
+}
+RunFn compare_scalar(ScalarFn f, const char *op) {  // (A, scalar) -> (mask)
+    return [f, op](const TF &c, Mem &mem, std::string &error) {
+        auto A = tensor_of(c.args[0], mem), M = tensor_of(c.returns[0], mem);
+        if (!mask_ok(*M, error) || !same_size({A.get(), M.get()}, error)) return 1;
+        return hip_result(f(A->dtype(), A->data, scalar_of(c.args[1], mem), M->data, M->shape.size, nullptr), op, error);
+    };
+}
+
+using ReduceFn = int (*)(int, const void *, const int32_t *, int, const int32_t *, int, void *, void *, size_t, void *);
+RunFn reduce(ReduceFn f, const char *op) {  // (A, vector dims, bool keepdims) -> (B)
+    return [f, op](const TF &c, Mem &mem, std::string &error) {
+        auto A = tensor_of(c.args[0], mem), B = tensor_of(c.returns[0], mem);
+        std::vector<int> dims = checked_dims(A->shape.shape, ints_of(c.args[1], mem));
+        const bool keepdims = bool_of(c.args[2]);
+        if (!same_dtype({A.get(), B.get()}, error)) return 1;
+        std::vector<int> want = reduced_shape(A->shape.shape, dims, keepdims);
+        if (Shape(want).size != B->shape.size)
+            return fail(error, "Shape mismatch: reduced shape " + dims_str(want) + " vs output " + dims_str(B->shape.shape));
+        size_t need = 0;
+        int rc = dxh_reduce_workspace_bytes(A->dtype(), A->shape.shape.data(), A->shape.dim(), dims.data(), (int)dims.size(), &need);
+        if (rc != DXH_OK) return hip_result(rc, op, error);
+        void *ws = need ? mem.workspace(need) : nullptr;
+        return hip_result(f(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), dims.data(), (int)dims.size(), B->data, ws,
+                            need ? mem.workspace_bytes() : 0, nullptr), op, error);
+    };
+}
+
+std::shared_ptr<Tensor> new_tensor(const std::vector<int> &shape, Precision p) {
+    for (int d : shape) if (d < 0) throw std::invalid_argument("negative dimension in shape " + dims_str(shape));
+    if (shape.empty()) throw std::invalid_argument("newtensor: empty shape");
+    auto t = std::make_shared<Tensor>(shape, p);
+    dxh_scalar zero{0.0, 0};
+    // zero-filled like op-cuda's "T1 = zeros(shape)"; bool/f8 tensors fill as bytes
+    int dt = (p == Precision::Float8E5M2 || p == Precision::Float8E4M3) ? (int)DXH_I8 : (int)p;
+    dxh_check(dxh_constant(dt, t->data, t->shape.size, zero, nullptr), "newtensor zero fill");
+    return t;
+}
+
+}  // namespace
+
+int register_all(TfFactory &f) {
+    // ---- tensorlife (tf/tensorlife.hpp) ---------------------------------------------------------
+    auto newtensor = [](const TF &c, Mem &mem, std::string &error) {
+        const TypeDef &t = c.returns[0].dtype;
+        if ((uint8_t(t.category) & uint8_t(DataCategory::Tensor)) == 0) return fail(error, "newtensor: return type must include tensor category");
+        if (precision_bytes(t.precision) == 0) return fail(error, "newtensor: unsupported precision " + precision_str(t.precision));
+        if (t.precision == Precision::Float8E5M2 || t.precision == Precision::Float8E4M3)
+            return fail(error, "newtensor: " + precision_str(t.precision) + " has not been implemented");
+        auto tensor = new_tensor(ints_of(c.args[0], mem), t.precision);
+        if (!mem.addtensor(c.returns[0].textvalue, tensor)) std::cerr << "tensor already exists: " << c.returns[0].textvalue << std::endl;
+        return 0;
+    };
+    reg(f, "newtensor", "", "tensorlife", "T1 = zeros(shape)", {"vector<int32>:shape"}, {"tensor<any>:t"}, newtensor);
+    reg(f, "newtensor", "", "tensorlife", "T1 = zeros(shape)", {"var<string>:shape"}, {"tensor<any>:t"}, newtensor);
+    reg(f, "copytensor", "", "tensorlife", "T2.data = T1.data", {"tensor<any>:src"}, {"tensor<any>:dst"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto S = tensor_of(c.args[0], mem), D = tensor_of(c.returns[0], mem);
+            if (S->shape.dtype != D->shape.dtype) return fail(error, "copytensor: input type and return type must be the same");
+            if (!same_size({S.get(), D.get()}, error)) return 1;
+            return hip_result(dxh_memcpy_d2d(D->data, S->data, (size_t)S->shape.bytes(), nullptr), "copytensor", error);
+        });
+    reg(f, "deltensor", "", "tensorlife", "del->T1", {}, {"tensor<any>:t"},
+        [](const TF &c, Mem &mem, std::string &) { mem.delete_tensor(c.returns[0].textvalue); return 0; });
+    reg(f, "renametensor", "", "tensorlife", "rename(newname)->T1", {"var<string>:new_name"}, {"tensor<any>:t"},
+        [](const TF &c, Mem &mem, std::string &) { mem.rename_tensor(c.returns[0].textvalue, c.args[0].textvalue); return 0; });
+
+    // ---- arg (tf/arg.hpp) -----------------------------------------------------------------------
+    reg(f, "argset", "", "arg", "argvalue->argname", {"var<any>:value"}, {"var<any>:name"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            const TypeDef &t = c.returns[0].dtype;
+            if ((uint8_t(t.category) & uint8_t(DataCategory::Var)) == 0) return fail(error, "datatype must be var");
+            const std::string &v = c.args[0].textvalue, &name = c.returns[0].textvalue;
+            switch (t.precision) {
+            case Precision::Int32: mem.setarg(name, (int32_t)std::atoi(v.c_str())); break;
+            case Precision::Int64: mem.setarg(name, (int64_t)std::stoll(v)); break;
+            case Precision::Float32: mem.setarg(name, std::stof(v)); break;
+            case Precision::Float64: mem.setarg(name, std::stod(v)); break;
+            case Precision::Bool: mem.setarg(name, bool_of(c.args[0])); break;
+            case Precision::String: mem.setarg(name, v); break;
+            default: return fail(error, "Unsupported dtype: " + typedef_str(c.args[0].dtype));
+            }
+            return 0;
+        });
+    reg(f, "vecset", "", "arg", "[3  4  5]->shape", {"vector<any>:value"}, {"vector<any>:name"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            const TypeDef &t = c.returns[0].dtype;
+            if ((uint8_t(t.category) & uint8_t(DataCategory::Vector)) == 0) return fail(error, "datatype must be vector");
+            auto words = words_of(c.args[0]);
+            const std::string &name = c.returns[0].textvalue;
+            switch (t.precision) {
+            case Precision::Int64: { std::vector<int64_t> v; for (auto &w : words) v.push_back(std::stoll(w)); mem.setarg(name, v); break; }
+            case Precision::Int32: case Precision::Int16: case Precision::Int8: {
+                std::vector<int32_t> v; for (auto &w : words) v.push_back(std::stoi(w)); mem.setarg(name, v); break; }
+            case Precision::Float64: { std::vector<double> v; for (auto &w : words) v.push_back(std::stod(w)); mem.setarg(name, v); break; }
+            case Precision::Float32: { std::vector<float> v; for (auto &w : words) v.push_back(std::stof(w)); mem.setarg(name, v); break; }
+            case Precision::String: mem.setarg(name, words); break;
+            default: return fail(error, "Unsupported dtype: " + typedef_str(t));
+            }
+            return 0;
+        });
+
+    // ---- init (tf/init.hpp) ----------------------------------------------------------------------
+    reg(f, "constant", "miaobyte", "init", "constant(value)->T1", {"var<any>:value"}, {"tensor<any>:t"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto T = tensor_of(c.returns[0], mem);
+            dxh_scalar v = T->shape.dtype == Precision::Bool && !text_is_float(c.args[0].textvalue)
+                               ? dxh_scalar{bool_of(c.args[0]) ? 1.0 : 0.0, bool_of(c.args[0]) ? 1 : 0} : scalar_of(c.args[0], mem);
+            return hip_result(dxh_constant(T->dtype(), T->data, T->shape.size, v, nullptr), "constant", error);
+        });
+    reg(f, "arange", "miaobyte", "init", "arange(start,step)->T1", {"var<any>:start", "var<any>:step"}, {"tensor<any>:t"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto T = tensor_of(c.returns[0], mem);
+            return hip_result(dxh_arange(T->dtype(), T->data, T->shape.size, scalar_of(c.args[0], mem), scalar_of(c.args[1], mem), nullptr), "arange", error);
+        });
+    reg(f, "uniform", "miaobyte", "init", "uniform(low,high,seed)->T1", {"var<any>:low", "var<any>:high", "var<int32>:seed"}, {"tensor<any>:t"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto T = tensor_of(c.returns[0], mem);
+            return hip_result(dxh_uniform(T->dtype(), T->data, T->shape.size, scalar_of(c.args[0], mem), scalar_of(c.args[1], mem),
+                                          (uint32_t)int_of(c.args[2], mem), nullptr), "uniform", error);
+        });
+    reg(f, "normal", "miaobyte", "init", "normal(mean,stddev,seed)->T1", {"var<any>:mean", "var<any>:stddev", "var<int32>:seed"}, {"tensor<any>:t"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto T = tensor_of(c.returns[0], mem);
+            return hip_result(dxh_normal(T->dtype(), T->data, T->shape.size, scalar_of(c.args[0], mem), scalar_of(c.args[1], mem),
+                                         (uint32_t)int_of(c.args[2], mem), nullptr), "normal", error);
+        });
+    reg(f, "dropout", "miaobyte", "init", "dropout(p,seed)->A", {"var<float32>:p", "var<int32>:seed"}, {"tensor<any>:A"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto T = tensor_of(c.returns[0], mem);
+            return hip_result(dxh_dropout(T->dtype(), T->data, T->shape.size, float_of(c.args[0], mem), (uint32_t)int_of(c.args[1], mem), nullptr), "dropout", error);
+        });
+
+    // ---- io (tf/io.hpp) --------------------------------------------------------------------------
+    auto print = [](const TF &c, Mem &mem, std::string &error) {
+        if (!mem.existstensor(c.args[0].textvalue)) return fail(error, "print " + c.args[0].textvalue + " not found");
+        auto T = tensor_of(c.args[0], mem);
+        print_tensor(*T, c.args.size() > 1 ? c.args[1].textvalue : std::string(), std::cout);
+        return 0;
+    };
+    reg(f, "print", "miaobyte", "io", "print(T1)", {"tensor<any>:t"}, {}, print);
+    reg(f, "print", "miaobyte", "io", "print(T1)", {"tensor<any>:t", "var<string>:format"}, {}, print);
+    reg(f, "save", "", "io", "save(T1,path)", {"tensor<any>:t", "var<string>:path"}, {},
+        [](const TF &c, Mem &mem, std::string &error) {
+            if (!mem.existstensor(c.args[0].textvalue)) return fail(error, "save " + c.args[0].textvalue + " not found");
+            save_tensor(*tensor_of(c.args[0], mem), c.args[1].textvalue);
+            return 0;
+        });
+    reg(f, "load", "", "io", "load(path)", {"var<string>:path"}, {},
+        [](const TF &c, Mem &mem, std::string &) {
+            auto [name, tensor] = load_tensor(c.args[0].textvalue);
+            if (mem.existstensor(name)) mem.delete_tensor(name);  // the reference replaces with a warning
+            mem.addtensor(name, tensor);
+            return 0;
+        });
+    reg(f, "loadtensordata", "", "io", "loadtensordata(path)->tensor", {"var<string>:path"}, {"tensor<any>:t"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            if (!mem.existstensor(c.returns[0].textvalue)) return fail(error, "loadtensordata " + c.returns[0].textvalue + " not found");
+            load_tensor_data(c.args[0].textvalue, *tensor_of(c.returns[0], mem));
+            return 0;
+        });
+
+    // ---- elementwise (tf/elementwise.hpp; op-cuda tf/elementwise_*.hpp) ---------------------------
+    reg(f, "todtype", "", "elementwise", "T3(dtypeA)->T1(dtypeB)", {"tensor<any>:A"}, {"tensor<any>:C"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto A = tensor_of(c.args[0], mem), C = tensor_of(c.returns[0], mem);
+            if (A->shape.size != C->shape.size) return fail(error, "Shape mismatch: " + std::to_string(A->shape.size) + " != " + std::to_string(C->shape.size));
+            return hip_result(dxh_todtype(A->dtype(), A->data, C->dtype(), C->data, C->shape.size, nullptr), "todtype", error);
+        });
+#define T_ANY "tensor<any>"
+    reg(f, "add", "miaobyte", "elementwise", "T3=T1+T2", {T_ANY ":a", T_ANY ":b"}, {T_ANY ":c"}, binary(dxh_add, "add"));
+    // the reference registers a second author for add (cblas / cublas); both names reach the same kernel
+    reg(f, "add", "cublas", "elementwise", "T3=T1+T2", {T_ANY ":a", T_ANY ":b"}, {T_ANY ":c"}, binary(dxh_add, "add"));
+    reg(f, "add", "cblas", "elementwise", "T3=T1+T2", {T_ANY ":a", T_ANY ":b"}, {T_ANY ":c"}, binary(dxh_add, "add"));
+    reg(f, "addscalar", "miaobyte", "elementwise", "T3=T1+scalar", {T_ANY ":a", "var<any>:scalar"}, {T_ANY ":c"}, with_scalar(dxh_addscalar, "addscalar"));
+    reg(f, "sub", "miaobyte", "elementwise", "T3=T1-T2", {T_ANY ":a", T_ANY ":b"}, {T_ANY ":c"}, binary(dxh_sub, "sub"));
+    reg(f, "subscalar", "miaobyte", "elementwise", "T3=T1-scalar", {T_ANY ":a", "var<any>:scalar"}, {T_ANY ":c"}, with_scalar(dxh_subscalar, "subscalar"));
+    reg(f, "rsubscalar", "miaobyte", "elementwise", "T3=scalar-T1", {"var<any>:scalar", T_ANY ":a"}, {T_ANY ":c"}, with_rscalar(dxh_rsubscalar, "rsubscalar"));
+    reg(f, "mul", "miaobyte", "elementwise", "T3=T1*T2", {T_ANY ":A", T_ANY ":B"}, {T_ANY ":C"}, binary(dxh_mul, "mul"));
+    reg(f, "mulscalar", "miaobyte", "elementwise", "T3=T1*scalar", {T_ANY ":A", "var<any>:b"}, {T_ANY ":C"}, with_scalar(dxh_mulscalar, "mulscalar"));
+    reg(f, "div", "miaobyte", "elementwise", "T3=T1/T2", {T_ANY ":A", T_ANY ":B"}, {T_ANY ":C"}, binary(dxh_div, "div"));
+    reg(f, "divscalar", "miaobyte", "elementwise", "T3=T1/scalar", {T_ANY ":A", "var<any>:scalar"}, {T_ANY ":C"}, with_scalar(dxh_divscalar, "divscalar"));
+    reg(f, "rdivscalar", "miaobyte", "elementwise", "T3=scalar/T1", {"var<any>:scalar", T_ANY ":A"}, {T_ANY ":C"}, with_rscalar(dxh_rdivscalar, "rdivscalar"));
+    reg(f, "invert", "miaobyte", "elementwise", "T3=~T1", {"tensor<int64|int32|int16|int8|bool>:A"}, {"tensor<int64|int32|int16|int8|bool>:C"}, unary(dxh_invert, "invert"));
+    reg(f, "sqrt", "miaobyte", "elementwise", "T3=sqrt(T1)", {T_ANY ":A"}, {T_ANY ":C"}, unary(dxh_sqrt, "sqrt"));
+    reg(f, "pow", "miaobyte", "elementwise", "T3=T1^T2", {T_ANY ":A", T_ANY ":B"}, {T_ANY ":C"}, binary(dxh_pow, "pow"));
+    reg(f, "powscalar", "miaobyte", "elementwise", "T3=T1^scalar", {T_ANY ":A", "var<any>:scalar"}, {T_ANY ":C"}, with_scalar(dxh_powscalar, "powscalar"));
+    reg(f, "rpowscalar", "miaobyte", "elementwise", "T3=scalar^T1", {"var<any>:scalar", T_ANY ":A"}, {T_ANY ":C"}, with_rscalar(dxh_rpowscalar, "rpowscalar"));
+    reg(f, "log", "miaobyte", "elementwise", "T3=log(T1)", {T_ANY ":A"}, {T_ANY ":C"}, unary(dxh_log, "log"));
+    reg(f, "exp", "miaobyte", "elementwise", "T3=exp(T1)", {T_ANY ":A"}, {T_ANY ":C"}, unary(dxh_exp, "exp"));
+    reg(f, "sin", "miaobyte", "elementwise", "T3=sin(T1)", {T_ANY ":A"}, {T_ANY ":C"}, unary(dxh_sin, "sin"));
+    reg(f, "cos", "miaobyte", "elementwise", "T3=cos(T1)", {T_ANY ":A"}, {T_ANY ":C"}, unary(dxh_cos, "cos"));
+    reg(f, "tan", "miaobyte", "elementwise", "T3=tan(T1)", {T_ANY ":A"}, {T_ANY ":C"}, unary(dxh_tan, "tan"));
+    reg(f, "max", "miaobyte", "elementwise", "T3=max(T1,T2)", {T_ANY ":A", T_ANY ":B"}, {T_ANY ":C"}, binary(dxh_max, "max"));
+    reg(f, "maxscalar", "miaobyte", "elementwise", "T3=max(T1,scalar)", {T_ANY ":A", "var<any>:scalar"}, {T_ANY ":C"}, with_scalar(dxh_maxscalar, "maxscalar"));
+    reg(f, "min", "miaobyte", "elementwise", "T3=min(T1,T2)", {T_ANY ":A", T_ANY ":B"}, {T_ANY ":C"}, binary(dxh_min, "min"));
+    reg(f, "minscalar", "miaobyte", "elementwise", "T3=min(T1,scalar)", {T_ANY ":A", "var<any>:scalar"}, {T_ANY ":C"}, with_scalar(dxh_minscalar, "minscalar"));
+    reg(f, "equal", "miaobyte", "elementwise", "equal(T1,T2)->mask", {T_ANY ":A", T_ANY ":B", "var<float32>:epsilon"}, {"tensor<bool>:mask"}, compare_eps(dxh_equal, "equal"));
+    reg(f, "equalscalar", "miaobyte", "elementwise", "mask=equal(T1,scalar)", {T_ANY ":A", "var<any>:scalar", "var<float32>:epsilon"}, {"tensor<bool>:mask"}, compare_eps_scalar(dxh_equalscalar, "equalscalar"));
+    reg(f, "notequal", "miaobyte", "elementwise", "notequal(T1,T2)->mask", {T_ANY ":A", T_ANY ":B", "var<float32>:epsilon"}, {"tensor<bool>:mask"}, compare_eps(dxh_notequal, "notequal"));
+    reg(f, "notequalscalar", "miaobyte", "elementwise", "mask=notequal(T1,scalar)", {T_ANY ":A", "var<any>:scalar", "var<float32>:epsilon"}, {"tensor<bool>:mask"}, compare_eps_scalar(dxh_notequalscalar, "notequalscalar"));
+    reg(f, "less", "miaobyte", "elementwise", "mask=less(T1,T2)", {T_ANY ":A", T_ANY ":B"}, {"tensor<bool>:mask"}, compare(dxh_less, "less"));
+    reg(f, "lessscalar", "miaobyte", "elementwise", "mask=less(T1,scalar)", {T_ANY ":A", "var<any>:scalar"}, {"tensor<bool>:mask"}, compare_scalar(dxh_lessscalar, "lessscalar"));
+    reg(f, "greater", "miaobyte", "elementwise", "mask=greater(T1,T2)", {T_ANY ":A", T_ANY ":B"}, {"tensor<bool>:mask"}, compare(dxh_greater, "greater"));
+    reg(f, "greaterscalar", "miaobyte", "elementwise", "mask=greater(T1,scalar)", {T_ANY ":A", "var<any>:scalar"}, {"tensor<bool>:mask"}, compare_scalar(dxh_greaterscalar, "greaterscalar"));
+    reg(f, "switch", "miaobyte", "elementwise", "C=switch([tensors],case)", {"listtensor<any>:tensors", "tensor<int32|bool>:cases"}, {T_ANY ":C"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto names = words_of(c.args[0]);
+            if (names.empty() || names.size() > DXH_SWITCH_MAX) return fail(error, "switch takes 1.." + std::to_string(DXH_SWITCH_MAX) + " tensors");
+            auto cases = tensor_of(c.args[1], mem), C = tensor_of(c.returns[0], mem);
+            std::vector<std::shared_ptr<Tensor>> ts;
+            std::vector<const void *> ptrs;
+            for (auto &n : names) {
+                ts.push_back(mem.gettensor(n));
+                if (ts.back()->shape.dtype != C->shape.dtype) return fail(error, "Type mismatch: " + precision_str(ts.back()->shape.dtype) + " != " + precision_str(C->shape.dtype));
+                if (!same_size({ts.back().get(), C.get()}, error)) return 1;
+                ptrs.push_back(ts.back()->data);
+            }
+            if (!same_size({cases.get(), C.get()}, error)) return 1;
+            if (cases->shape.dtype == Precision::Bool && names.size() != 2) return fail(error, "For bool cases, tensors size must be 2");
+            return hip_result(dxh_switch(C->dtype(), ptrs.data(), (int)ptrs.size(), cases->dtype(), cases->data, C->data, C->shape.size, nullptr), "switch", error);
+        });
+
+    // ---- reduce (tf/reduce.hpp) ------------------------------------------------------------------
+    reg(f, "sum", "miaobyte", "reduce", "B = sum(A, axis=[1 2], keepdims=false)", {T_ANY ":A", "vector<int32>:axis", "var<bool>:keepdims"}, {T_ANY ":B"}, reduce(dxh_sum, "sum"));
+    reg(f, "prod", "miaobyte", "reduce", "B = prod(A, axis=[1 2], keepdims=false)", {T_ANY ":A", "vector<int32>:axis", "var<bool>:keepdims"}, {T_ANY ":B"}, reduce(dxh_prod, "prod"));
+    reg(f, "reducemax", "miaobyte", "reduce", "B = reducemax(A, axis=[1 2], keepdims=false)", {T_ANY ":A", "vector<int32>:axis", "var<bool>:keepdims"}, {T_ANY ":B"}, reduce(dxh_reducemax, "reducemax"));
+    reg(f, "reducemin", "miaobyte", "reduce", "B = reducemin(A, axis=[1 2], keepdims=false)", {T_ANY ":A", "vector<int32>:axis", "var<bool>:keepdims"}, {T_ANY ":B"}, reduce(dxh_reducemin, "reducemin"));
+
+    // ---- changeshape (tf/changeshape.hpp) ---------------------------------------------------------
+    reg(f, "reshape", "miaobyte", "changeshape", "T1.reshape(shape)->T2", {T_ANY ":A", "vector<int32>:shape"}, {T_ANY ":B"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto A = tensor_of(c.args[0], mem), B = tensor_of(c.returns[0], mem);
+            if (!same_dtype({A.get(), B.get()}, error)) return 1;
+            std::vector<int> shape = ints_of(c.args[1], mem);
+            Shape ns(shape, B->shape.dtype);
+            if (ns.size != A->shape.size || ns.size != B->shape.size) return fail(error, "Shape size mismatch");
+            B->shape = ns;  // metadata only when A and B are the same tensor, else a copy too
+            if (A->data != B->data) return hip_result(dxh_memcpy_d2d(B->data, A->data, (size_t)A->shape.bytes(), nullptr), "reshape", error);
+            return 0;
+        });
+    reg(f, "transpose", "miaobyte", "changeshape", "T1.transpose(dimorder=[1,0])->T2", {T_ANY ":A", "vector<int32>:dim_order"}, {T_ANY ":C"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto A = tensor_of(c.args[0], mem), C = tensor_of(c.returns[0], mem);
+            if (!same_dtype({A.get(), C.get()}, error)) return 1;
+            std::vector<int> order = ints_of(c.args[1], mem);
+            std::vector<int> want = transpose_shape(A->shape.shape, order);
+            if (C->shape.size != A->shape.size) return fail(error, "transpose error!shape");
+            if (A->data == C->data) return fail(error, "transpose cannot run in place");
+            (void)want;
+            return hip_result(dxh_transpose(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), order.data(), C->data, nullptr), "transpose", error);
+        });
+    reg(f, "concat", "miaobyte", "changeshape", "Tresult = concat([T1, T2...], axis=3)", {"listtensor<any>:tensors", "var<int32>:dim"}, {T_ANY ":result"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto names = words_of(c.args[0]);
+            if (names.empty()) return fail(error, "concat needs at least one tensor");
+            auto R = tensor_of(c.returns[0], mem);
+            int axis = int_of(c.args[1], mem);
+            if (axis < 0) axis += R->shape.dim();
+            std::vector<std::shared_ptr<Tensor>> ts;
+            std::vector<const void *> ptrs;
+            std::vector<std::vector<int>> shapes;
+            std::vector<int32_t> axis_sizes;
+            for (auto &n : names) {
+                ts.push_back(mem.gettensor(n));
+                if (ts.back()->shape.dtype != R->shape.dtype) return fail(error, "Type mismatch: " + precision_str(ts.back()->shape.dtype) + " != " + precision_str(R->shape.dtype));
+                shapes.push_back(ts.back()->shape.shape);
+                ptrs.push_back(ts.back()->data);
+            }
+            std::vector<int> want = concat_shape(shapes, axis);
+            if (want != R->shape.shape) return fail(error, "Output tensor shape size must match the sum of input tensor shape sizes for concat");
+            for (auto &s : shapes) axis_sizes.push_back(s[axis]);
+            return hip_result(dxh_concat(R->dtype(), ptrs.data(), (int)ptrs.size(), axis_sizes.data(), want.data(), (int)want.size(), axis, R->data, nullptr), "concat", error);
+        });
+    reg(f, "broadcastTo", "miaobyte", "changeshape", "T2 = T1.broadcastTo(new_shape=[4,3,2])", {T_ANY ":A", "vector<int32>:new_shape"}, {T_ANY ":B"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto A = tensor_of(c.args[0], mem), B = tensor_of(c.returns[0], mem);
+            if (!same_dtype({A.get(), B.get()}, error)) return 1;
+            std::vector<int> ns = ints_of(c.args[1], mem);
+            if (broadcast_shape(A->shape.shape, ns) != ns) return fail(error, "Broadcast shape mismatch");
+            if (Shape(ns).size != B->shape.size) return fail(error, "Broadcast shape mismatch: output is " + dims_str(B->shape.shape));
+            return hip_result(dxh_broadcastTo(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), ns.data(), (int)ns.size(), B->data, nullptr), "broadcastTo", error);
+        });
+    reg(f, "indexselect", "miaobyte", "changeshape", "T2 = T1.indexselect(index=T3, axis=3)", {T_ANY ":A", "tensor<int64|int32>:index", "var<int32>:axis"}, {T_ANY ":B"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto A = tensor_of(c.args[0], mem), I = tensor_of(c.args[1], mem), B = tensor_of(c.returns[0], mem);
+            if (!same_dtype({A.get(), B.get()}, error)) return 1;
+            if (I->shape.dtype != Precision::Int64 && I->shape.dtype != Precision::Int32) return fail(error, "index only support int32 or int64");
+            int axis = int_of(c.args[2], mem);
+            int ga = axis < 0 ? axis + A->shape.dim() : axis;
+            if (ga < 0 || ga >= A->shape.dim()) return fail(error, "Axis is out of bounds");
+            if (indexselect_shape(A->shape.shape, I->shape.shape, ga) != B->shape.shape) return fail(error, "Indexselect shape mismatch");
+            return hip_result(dxh_indexselect(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), I->dtype(), I->data, I->shape.shape.data(),
+                                              I->shape.dim(), ga, B->data, nullptr), "indexselect", error);
+        });
+    reg(f, "repeat", "miaobyte", "changeshape", "T1.repeat(repeats=[4,3,2])->T2", {T_ANY ":A", "vector<int32>:repeats"}, {T_ANY ":B"},
+        [](const TF &c, Mem &mem, std::string &error) {
+            auto A = tensor_of(c.args[0], mem), B = tensor_of(c.returns[0], mem);
+            if (!same_dtype({A.get(), B.get()}, error)) return 1;
+            std::vector<int> reps = ints_of(c.args[1], mem);
+            if (repeat_shape(A->shape.shape, reps) != B->shape.shape) return fail(error, "Repeat shape mismatch");
+            return hip_result(dxh_repeat(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), reps.data(), B->data, nullptr), "repeat", error);
+        });
+
+    // ---- matmul (tf/matmul.hpp).  The front asks for author "cublas" (authormap.py:60), op-ompsimd
+    // registers "cblas" and "miaobyte": all three names reach the same MFMA / tiled kernel.
+    auto matmul = [](const TF &c, Mem &mem, std::string &error) {
+        auto A = tensor_of(c.args[0], mem), B = tensor_of(c.args[1], mem), C = tensor_of(c.returns[0], mem);
+        if (!same_dtype({A.get(), B.get(), C.get()}, error)) return 1;
+        std::vector<int> want = matmul_shape(A->shape.shape, B->shape.shape);
+        if (want != C->shape.shape) return fail(error, "matmul: output shape " + dims_str(C->shape.shape) + " != " + dims_str(want));
+        int64_t batch = 1;
+        for (int i = 0; i + 2 < A->shape.dim(); ++i) batch *= A->shape.shape[i];
+        return hip_result(dxh_matmul(A->dtype(), A->data, B->data, C->data, batch, A->shape.at(-2), A->shape.at(-1), B->shape.at(-1), nullptr), "matmul", error);
+    };
+    for (const char *author : {"cublas", "cblas", "miaobyte"})
+        reg(f, "matmul", author, "matmul", "T3=T1 @ T2", {T_ANY ":A", T_ANY ":B"}, {T_ANY ":C"}, matmul);
+#undef T_ANY
+    return 0;
+}
+
+}  // namespace deepx

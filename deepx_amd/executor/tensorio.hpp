@@ -1,0 +1,150 @@
+// tensorio.hpp — tensor files and printing.
+//
+// A saved tensor is two files (executor/deepxcore/src/deepx/shape.cpp:93-143,
+// executor/deepxcore/src/stdutil/fs.cpp:18-50, executor/op-cuda/src/deepx/tensorfunc/io_miaobyte.hpp):
+//   <path>.shape  YAML {dtype, dim, shape, stride, size}
+//   <path>.data   raw little-endian contiguous elements (bf16/f16 as their 16-bit patterns,
+//                 front/py/deepxutil/torch/io.py:11-12)
+// The tensor's name on load is the file stem (shape.cpp:140-142).  Device data moves through
+// one staged host copy.  print follows executor/deepxcore/src/stdutil/print.hpp:80-129.
+#pragma once
+#include <cstdio>
+#include <fstream>
+#include <memory>
+#include <ostream>
+#include <string>
+#include <vector>
+#include "mem.hpp"
+
+namespace deepx {
+
+inline std::string file_stem(const std::string &path) {
+    std::string name = path.substr(path.find_last_of('/') + 1);
+    size_t dot = name.find_last_of('.');
+    return dot == std::string::npos ? name : name.substr(0, dot);
+}
+
+inline std::vector<char> to_host(const Tensor &t) {
+    std::vector<char> host((size_t)t.shape.bytes());
+    dxh_check(dxh_memcpy_d2h(host.data(), t.data, host.size(), nullptr), "copy to host");
+    return host;
+}
+
+inline void save_tensor(const Tensor &t, const std::string &path) {
+    {
+        std::ofstream fs(path + ".shape", std::ios::binary | std::ios::trunc);
+        if (!fs.is_open()) throw std::runtime_error("Failed to open file for writing: " + path + ".shape");
+        fs << t.shape.to_yaml();
+    }
+    std::vector<char> host = to_host(t);
+    std::ofstream fs(path + ".data", std::ios::binary | std::ios::trunc);
+    if (!fs.is_open()) throw std::runtime_error("Failed to open file for writing: " + path + ".data");
+    fs.write(host.data(), (std::streamsize)host.size());
+    if (!fs) throw std::runtime_error("Failed to write data to file: " + path + ".data");
+}
+
+inline std::vector<char> read_exact(const std::string &path, size_t want) {
+    std::ifstream fs(path, std::ios::binary);
+    if (!fs.is_open()) throw std::runtime_error("Failed to open file: " + path);
+    fs.seekg(0, std::ios::end);
+    size_t size = (size_t)fs.tellg();
+    fs.seekg(0, std::ios::beg);
+    if (size != want) throw std::runtime_error("file size mismatch: " + path);
+    std::vector<char> buf(size);
+    fs.read(buf.data(), (std::streamsize)size);
+    if (fs.fail()) throw std::runtime_error("Failed to read file: " + path);
+    return buf;
+}
+
+inline void load_tensor_data(const std::string &path, Tensor &t) {
+    // accept both "<path>" and "<path>.data" like the two reference loaders do between them
+    std::string file = path;
+    if (file.size() < 5 || file.substr(file.size() - 5) != ".data") file += ".data";
+    std::vector<char> buf = read_exact(file, (size_t)t.shape.bytes());
+    dxh_check(dxh_memcpy_h2d(t.data, buf.data(), buf.size(), nullptr), "copy to device");
+}
+
+inline std::pair<std::string, std::shared_ptr<Tensor>> load_tensor(const std::string &path) {
+    std::ifstream fs(path + ".shape", std::ios::binary);
+    if (!fs.is_open()) throw std::runtime_error("Failed to open shape file: " + path + ".shape");
+    std::string text((std::istreambuf_iterator<char>(fs)), std::istreambuf_iterator<char>());
+    Shape s = Shape::from_yaml(text);
+    if (precision_bytes(s.dtype) == 0) throw std::runtime_error("unsupported dtype in " + path + ".shape");
+    auto t = std::make_shared<Tensor>(s.shape, s.dtype);
+    load_tensor_data(path, *t);
+    // the reference takes the stem of the last path component ("a/b/w.x" -> "w"); a path without a
+    // dot keeps its whole last component
+    return {file_stem(path), t};
+}
+
+inline float half_bits_to_float(uint16_t h) {
+    uint32_t s = uint32_t(h & 0x8000u) << 16, e = (h >> 10) & 0x1f, m = h & 0x3ff, u;
+    if (e == 0) {
+        if (m == 0) u = s;
+        else { int sh = 0; while (!(m & 0x400)) { m <<= 1; ++sh; } u = s | ((113 - sh) << 23) | ((m & 0x3ff) << 13); }
+    } else if (e == 31) u = s | 0x7f800000u | (m << 13);
+    else u = s | ((e + 112) << 23) | (m << 13);
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+
+inline void print_element(std::ostream &os, const char *data, int64_t i, Precision p, const std::string &fmt) {
+    char buf[128];
+    switch (p) {
+    case Precision::Float64: std::snprintf(buf, sizeof buf, fmt.c_str(), ((const double *)data)[i]); break;
+    case Precision::Float32: std::snprintf(buf, sizeof buf, fmt.c_str(), (double)((const float *)data)[i]); break;
+    case Precision::Float16: std::snprintf(buf, sizeof buf, fmt.c_str(), (double)half_bits_to_float(((const uint16_t *)data)[i])); break;
+    case Precision::BFloat16: {
+        uint32_t u = uint32_t(((const uint16_t *)data)[i]) << 16;
+        float f;
+        std::memcpy(&f, &u, 4);
+        std::snprintf(buf, sizeof buf, fmt.c_str(), (double)f);
+        break;
+    }
+    case Precision::Int64: std::snprintf(buf, sizeof buf, fmt.find('l') == std::string::npos ? "%lld" : fmt.c_str(), (long long)((const int64_t *)data)[i]); break;
+    case Precision::Int32: std::snprintf(buf, sizeof buf, fmt.c_str(), ((const int32_t *)data)[i]); break;
+    case Precision::Int16: std::snprintf(buf, sizeof buf, fmt.c_str(), (int)((const int16_t *)data)[i]); break;
+    case Precision::Int8: std::snprintf(buf, sizeof buf, fmt.c_str(), (int)((const int8_t *)data)[i]); break;
+    case Precision::Bool: std::snprintf(buf, sizeof buf, fmt.c_str(), (int)((const uint8_t *)data)[i]); break;
+    default: buf[0] = '?'; buf[1] = 0;
+    }
+    os << buf;
+}
+
+inline void print_tensor(const Tensor &t, std::string fmt, std::ostream &os) {
+    const Precision p = t.shape.dtype;
+    const bool is_float = (uint16_t(p) & uint16_t(Precision::Float)) != 0;
+    if (fmt.empty()) fmt = is_float ? "%.4f" : "%d";
+    std::vector<char> host = to_host(t);
+    const Shape &s = t.shape;
+    os << "shape:[";
+    for (int i = 0; i < s.dim(); ++i) os << s.shape[i] << (i + 1 < s.dim() ? ", " : "");
+    os << "]" << std::endl;
+    if (s.dim() == 1) {
+        os << "[";
+        for (int i = 0; i < s.shape[0]; ++i) { if (i) os << " "; print_element(os, host.data(), i, p, fmt); }
+        os << "]" << std::endl;
+        return;
+    }
+    const int rows = s.at(-2), cols = s.at(-1);
+    const int64_t per = (int64_t)rows * cols;
+    const int64_t mats = per > 0 ? s.size / per : 0;
+    for (int64_t m = 0; m < mats; ++m) {
+        // index of this matrix over the leading dims
+        os << "[";
+        int64_t rem = m;
+        std::vector<int> idx(s.dim() - 2);
+        for (int d = s.dim() - 3; d >= 0; --d) { idx[d] = (int)(rem % s.shape[d]); rem /= s.shape[d]; }
+        for (size_t d = 0; d < idx.size(); ++d) os << idx[d] << (d + 1 < idx.size() ? ", " : "");
+        os << "]=[" << std::endl;
+        for (int i = 0; i < rows; ++i) {
+            os << " [";
+            for (int j = 0; j < cols; ++j) { if (j) os << " "; print_element(os, host.data(), (m * rows + i) * cols + j, p, fmt); }
+            os << "]" << (i + 1 < rows ? "," : "") << std::endl;
+        }
+        os << "]" << std::endl;
+    }
+}
+
+}  // namespace deepx

@@ -1,0 +1,72 @@
+// udpserver.hpp — the wire: UDP/IPv4, newline-separated IR lines in, one reply datagram per line.
+//
+// Protocol of executor/deepxcore/src/client/udpserver.cpp:20-65 (bind INADDR_ANY:<port>, split the
+// datagram on '\n', reply to the sender with sendto).  Differences, all to remove crashes: the
+// receive buffer is 64 KiB with the terminator inside it (the reference writes buffer[1024]), a
+// parse failure answers with an error line instead of unwinding the receiver thread, and replies go
+// to the address each datagram came from rather than to "the last client".
+#pragma once
+#include <arpa/inet.h>
+#include <sys/socket.h>
+#include <unistd.h>
+#include <atomic>
+#include <cstdio>
+#include <cstring>
+#include <sstream>
+#include <string>
+#include "executor.hpp"
+
+namespace deepx {
+
+class UdpServer {
+public:
+    explicit UdpServer(int port) : port_(port) {}
+    ~UdpServer() { if (fd_ >= 0) ::close(fd_); }
+
+    bool open() {
+        fd_ = ::socket(AF_INET, SOCK_DGRAM, 0);
+        if (fd_ < 0) { perror("socket creation failed"); return false; }
+        int rcv = 4 << 20;
+        ::setsockopt(fd_, SOL_SOCKET, SO_RCVBUF, &rcv, sizeof rcv);
+        sockaddr_in addr{};
+        addr.sin_family = AF_INET;
+        addr.sin_addr.s_addr = INADDR_ANY;
+        addr.sin_port = htons((uint16_t)port_);
+        if (::bind(fd_, (const sockaddr *)&addr, sizeof addr) < 0) { perror("bind failed"); return false; }
+        timeval tv{0, 200000};  // wake up to notice stop()
+        ::setsockopt(fd_, SOL_SOCKET, SO_RCVTIMEO, &tv, sizeof tv);
+        return true;
+    }
+
+    // Receive, execute, reply, until stop().  The front keeps exactly one instruction in flight
+    // (front/py/deepx/scheduler/client/udpconn.py:17-48), so executing on the receiving thread
+    // serialises ops exactly as the reference's queue + single consumer does.
+    void serve(Executor &ex) {
+        std::vector<char> buf(65536);
+        while (!stop_) {
+            sockaddr_in cli{};
+            socklen_t len = sizeof cli;
+            ssize_t n = ::recvfrom(fd_, buf.data(), buf.size() - 1, 0, (sockaddr *)&cli, &len);
+            if (n <= 0) continue;
+            buf[(size_t)n] = '\0';
+            TimePoint recv_at = std::chrono::system_clock::now();
+            std::istringstream lines(std::string(buf.data(), (size_t)n));
+            std::string line;
+            while (std::getline(lines, line)) {
+                if (!line.empty() && line.back() == '\r') line.pop_back();
+                if (line.empty()) continue;
+                if (line == "__quit__") { stop_ = true; break; }
+                std::string reply = ex.execute(line, recv_at);
+                ::sendto(fd_, reply.data(), reply.size(), 0, (const sockaddr *)&cli, len);
+            }
+        }
+    }
+    void stop() { stop_ = true; }
+
+private:
+    int port_;
+    int fd_ = -1;
+    std::atomic<bool> stop_{false};
+};
+
+}  // namespace deepx

@@ -92,6 +92,9 @@ SIGNATURES = {
     "dxh_repeat": ([_i, _p, _pi32, _i, _pi32, _p, _p], _i),
     "dxh_constant": ([_i, _p, _i64, Scalar, _p], _i),
     "dxh_arange": ([_i, _p, _i64, Scalar, Scalar, _p], _i),
+    "dxh_uniform": ([_i, _p, _i64, Scalar, Scalar, C.c_uint32, _p], _i),
+    "dxh_normal": ([_i, _p, _i64, Scalar, Scalar, C.c_uint32, _p], _i),
+    "dxh_dropout": ([_i, _p, _i64, _f, C.c_uint32, _p], _i),
     "dxh_matmul": ([_i, _p, _p, _p, _i64, _i64, _i64, _i64, _p], _i),
 }
 

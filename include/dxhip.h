@@ -219,6 +219,16 @@ DXH_API int dxh_repeat(int dtype, const void *in, const int32_t *shape, int ndim
  * (executor/op-ompsimd/src/deepx/tensorfunc/init_miaobyte.hpp:59-70). */
 DXH_API int dxh_constant(int dtype, void *out, int64_t n, dxh_scalar value, void *stream);
 DXH_API int dxh_arange(int dtype, void *out, int64_t n, dxh_scalar start, dxh_scalar step, void *stream);
+/* launch_uniform / launch_normal / launch_dropout init_miaobyte.cuh:32-47.
+ * uniform: out[i] = T(U[low,high));  normal: out[i] = T(N(mean,stddev));  dropout: inout[i] = 0
+ * where U[0,1) < p, other elements unchanged (no rescale, init_miaobyte.hpp:26-54).
+ * The random streams are counter based (a hash of seed and element index), reproducible for a
+ * given seed != 0; seed == 0 draws a fresh seed, as the reference does.  The reference's own
+ * two executors use different generators (libstdc++ minstd vs curand), so the bit stream is
+ * not part of the contract — only the distribution is. */
+DXH_API int dxh_uniform(int dtype, void *out, int64_t n, dxh_scalar low, dxh_scalar high, uint32_t seed, void *stream);
+DXH_API int dxh_normal(int dtype, void *out, int64_t n, dxh_scalar mean, dxh_scalar stddev, uint32_t seed, void *stream);
+DXH_API int dxh_dropout(int dtype, void *inout, int64_t n, float p, uint32_t seed, void *stream);
 
 /* ---- matmul: replaces cublasSgemm(StridedBatched) matmul_cublas.hpp:16-145 and
  * cblas_sgemm executor/op-ompsimd/src/deepx/tensorfunc/matmul_cblas.hpp:11-60.

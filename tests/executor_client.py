@@ -1,0 +1,155 @@
+"""Test-side clients of the executor: the in-process C API (libdxexec.so) and the UDP binary.
+
+The UDP client formats requests exactly like front/py/deepx/nn/deepxir.py:133-159 prints a DeepxIR
+and reads replies like DeepxIRResp (:161-204)."""
+import ctypes as C
+import os
+import socket
+import subprocess
+import time
+
+import numpy as np
+import yaml
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EXEC_DIR = os.path.join(ROOT, "deepx_amd", "executor")
+BIN = os.path.join(EXEC_DIR, "deepx-executor-hip")
+LIB = os.path.join(EXEC_DIR, "libdxexec.so")
+
+
+class InProc:
+    def __init__(self):
+        L = C.CDLL(LIB)
+        L.dxe_create.restype = C.c_void_p
+        L.dxe_destroy.argtypes = [C.c_void_p]
+        for name, args in [("dxe_execute", [C.c_void_p, C.c_char_p]), ("dxe_parse", [C.c_char_p]), ("dxe_match", [C.c_void_p, C.c_char_p]),
+                           ("dxe_op_table", [C.c_void_p, C.c_char_p]), ("dxe_typedef_roundtrip", [C.c_char_p]),
+                           ("dxe_tensor_yaml", [C.c_void_p, C.c_char_p]), ("dxe_shape_yaml_roundtrip", [C.c_char_p])]:
+            fn = getattr(L, name)
+            fn.argtypes = args + [C.c_char_p, C.c_size_t]
+            fn.restype = C.c_size_t
+        self.L = L
+        self.ex = L.dxe_create()
+        assert self.ex
+
+    def _call(self, fn, *args):
+        buf = C.create_string_buffer(1 << 18)
+        fn(*args, buf, len(buf))
+        return buf.value.decode("utf-8")
+
+    def execute(self, line): return self._call(self.L.dxe_execute, self.ex, line.encode())
+    def parse(self, line): return self._call(self.L.dxe_parse, line.encode())
+    def match(self, line): return self._call(self.L.dxe_match, self.ex, line.encode())
+    def op_table(self, name="op-mem-hip"): return self._call(self.L.dxe_op_table, self.ex, name.encode())
+    def typedef(self, text): return self._call(self.L.dxe_typedef_roundtrip, text.encode())
+    def tensor_yaml(self, name): return self._call(self.L.dxe_tensor_yaml, self.ex, name.encode())
+    def shape_yaml(self, text): return self._call(self.L.dxe_shape_yaml_roundtrip, text.encode())
+
+
+def free_port():
+    s = socket.socket(socket.AF_INET, socket.SOCK_DGRAM)
+    s.bind(("127.0.0.1", 0))
+    p = s.getsockname()[1]
+    s.close()
+    return p
+
+
+class Resp:
+    """'<id> ok// recv_at=.. start_at=.. finish_at=.. [message]' as DeepxIRResp splits it"""
+
+    def __init__(self, text):
+        self.text = text
+        front, _, extra = text.partition("//")
+        parts = front.strip().split(" ", 2)
+        self.id = parts[0] if parts else None
+        self.result = parts[1] if len(parts) > 1 else ""
+        self.times, msg = {}, []
+        for tok in extra.strip().split(" "):
+            k, eq, v = tok.partition("=")
+            if eq and k in ("recv_at", "start_at", "finish_at") and not msg:
+                self.times[k] = int(v)
+            elif tok:
+                msg.append(tok)
+        self.message = " ".join(msg)
+
+    @property
+    def ok(self): return self.result == "ok"
+
+
+class UdpExecutor:
+    """Runs deepx-executor-hip as a child process and talks deepxIR to it over UDP."""
+
+    def __init__(self, env=None):
+        self.port = free_port()
+        e = dict(os.environ, DEEPX_PORT=str(self.port))
+        e.update(env or {})
+        self.proc = subprocess.Popen([BIN], env=e, stdout=subprocess.PIPE, stderr=subprocess.PIPE)
+        self.sock = socket.socket(socket.AF_INET, socket.SOCK_DGRAM)
+        self.sock.settimeout(60)
+        self._id = 0
+        deadline = time.time() + 120
+        while True:  # wait until it answers
+            try:
+                self.sock.settimeout(1)
+                self.sock.sendto(b"argset(var<int32>:1)->(var<int32>:__ready) // id=0", ("127.0.0.1", self.port))
+                self.sock.recvfrom(65536)
+                break
+            except socket.timeout:
+                if self.proc.poll() is not None or time.time() > deadline:
+                    raise RuntimeError("executor did not start: " + self.proc.stderr.read().decode())
+        self.sock.settimeout(60)
+
+    def raw(self, text, nreplies=1):
+        self.sock.sendto(text.encode("utf-8"), ("127.0.0.1", self.port))
+        return [Resp(self.sock.recvfrom(65536)[0].decode("utf-8")) for _ in range(nreplies)]
+
+    def send(self, op, args, returns, author="miaobyte", extra=""):
+        """format like str(DeepxIR): 'name (a, b) -> (c) // author=x  id=n  created_at=t  sent_at=t'"""
+        self._id += 1
+        now = time.time()
+        meta = []
+        if author:
+            meta.append(f"author={author}")
+        meta += [f" id={self._id}", f" created_at={now}", f" sent_at={now}"]
+        if extra:
+            meta.append(" " + extra)
+        line = " ".join([op, "(" + ", ".join(args) + ")", "->", "(" + ", ".join(returns) + ")", "//", " ".join(meta)])
+        r = self.raw(line)[0]
+        assert r.id == str(self._id), (r.text, self._id)
+        return r
+
+    def must(self, op, args, returns, author="miaobyte", extra=""):
+        r = self.send(op, args, returns, author, extra)
+        assert r.ok, f"{op}: {r.text}"
+        return r
+
+    def close(self):
+        try:
+            self.sock.sendto(b"__quit__", ("127.0.0.1", self.port))
+            self.proc.wait(timeout=10)
+        except Exception:
+            self.proc.kill()
+        self.sock.close()
+
+
+# ---- deepx tensor files (the format of front/py/deepxutil/numpy/io.py and shape.cpp:93-101) ------
+NP_OF = {"float64": np.float64, "float32": np.float32, "float16": np.uint16, "bfloat16": np.uint16, "int64": np.int64,
+         "int32": np.int32, "int16": np.int16, "int8": np.int8, "bool": np.uint8}
+
+
+def write_tensor(path, arr, dtype_name):
+    arr = np.ascontiguousarray(arr)
+    strides, s = [], 1
+    for d in reversed(arr.shape):
+        strides.insert(0, s)
+        s *= d
+    with open(path + ".shape", "w") as f:  # what PyYAML writes for the front (shape.py:185-191)
+        yaml.safe_dump({"dtype": dtype_name, "dim": arr.ndim, "shape": list(arr.shape), "stride": strides, "size": int(arr.size)}, f)
+    arr.tofile(path + ".data")
+
+
+def read_tensor(path):
+    meta = yaml.safe_load(open(path + ".shape"))
+    data = np.fromfile(path + ".data", dtype=NP_OF[meta["dtype"]])
+    assert data.size == meta["size"]
+    return data.reshape(meta["shape"]), meta

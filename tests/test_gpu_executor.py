@@ -244,35 +244,35 @@ def test_config5_mlp_block_over_ir(srv, tmp_path):
     Wg = f2b((rng.standard_normal((Hd, I)) * 0.02).astype(np.float32))
     Wu = f2b((rng.standard_normal((Hd, I)) * 0.02).astype(np.float32))
     Wd = f2b((rng.standard_normal((I, Hd)) * 0.02).astype(np.float32))
-    for name, arr in [("x", x), ("w", w.reshape(1, Hd)), ("Wg", Wg), ("Wu", Wu), ("Wd", Wd)]:
+    for name, arr in [("q5_x", x), ("q5_w", w.reshape(1, Hd)), ("q5_Wg", Wg), ("q5_Wu", Wu), ("q5_Wd", Wd)]:
         load(srv, tmp_path, name, arr, "bfloat16")
     B16, F32 = "bfloat16", "float32"
     new = lambda name, shape, dt: srv.must("newtensor", [V(shape)], [T(name, dt)], author="")
     # RMSNorm in fp32 (front/py/deepx/nn/modules/norm/t5layernorm.py:17-22)
-    new("xf", [S, Hd], F32); srv.must("todtype", [T("x", B16)], [T("xf", F32)], author="")
-    new("sq", [S, Hd], F32); srv.must("powscalar", [T("xf"), "var<float32>:2"], [T("sq")])
-    new("var", [S, 1], F32); srv.must("sum", [T("sq"), V([-1]), "var<bool>:True"], [T("var")])
-    srv.must("divscalar", [T("var"), f"var<float32>:{Hd}"], [T("var")])
-    srv.must("addscalar", [T("var"), "var<float32>:1e-06"], [T("var")])
-    srv.must("sqrt", [T("var")], [T("var")])
-    srv.must("rdivscalar", ["var<float32>:1", T("var")], [T("var")])
-    new("rs", [S, Hd], F32); srv.must("broadcastTo", [T("var"), V([S, Hd])], [T("rs")])
-    new("xn", [S, Hd], F32); srv.must("mul", [T("xf"), T("rs")], [T("xn")])
-    new("wf1", [1, Hd], F32); srv.must("todtype", [T("w", B16)], [T("wf1")], author="")
-    new("wf", [S, Hd], F32); srv.must("broadcastTo", [T("wf1"), V([S, Hd])], [T("wf")])
-    srv.must("mul", [T("wf"), T("xn")], [T("xn")])
-    new("h", [S, Hd], B16); srv.must("todtype", [T("xn")], [T("h", B16)], author="")
+    new("q5_xf", [S, Hd], F32); srv.must("todtype", [T("q5_x", B16)], [T("q5_xf", F32)], author="")
+    new("q5_sq", [S, Hd], F32); srv.must("powscalar", [T("q5_xf"), "var<float32>:2"], [T("q5_sq")])
+    new("q5_var", [S, 1], F32); srv.must("sum", [T("q5_sq"), V([-1]), "var<bool>:True"], [T("q5_var")])
+    srv.must("divscalar", [T("q5_var"), f"var<float32>:{Hd}"], [T("q5_var")])
+    srv.must("addscalar", [T("q5_var"), "var<float32>:1e-06"], [T("q5_var")])
+    srv.must("sqrt", [T("q5_var")], [T("q5_var")])
+    srv.must("rdivscalar", ["var<float32>:1", T("q5_var")], [T("q5_var")])
+    new("q5_rs", [S, Hd], F32); srv.must("broadcastTo", [T("q5_var"), V([S, Hd])], [T("q5_rs")])
+    new("q5_xn", [S, Hd], F32); srv.must("mul", [T("q5_xf"), T("q5_rs")], [T("q5_xn")])
+    new("q5_wf1", [1, Hd], F32); srv.must("todtype", [T("q5_w", B16)], [T("q5_wf1")], author="")
+    new("q5_wf", [S, Hd], F32); srv.must("broadcastTo", [T("q5_wf1"), V([S, Hd])], [T("q5_wf")])
+    srv.must("mul", [T("q5_wf"), T("q5_xn")], [T("q5_xn")])
+    new("q5_h", [S, Hd], B16); srv.must("todtype", [T("q5_xn")], [T("q5_h", B16)], author="")
     # gated MLP (front/py/deepx/nn/modules/mlp/gatedmlp.py:20-26), SiLU = x * 1/(1+exp(-x)) (activite.py:11-18)
-    new("g", [S, I], B16); srv.must("matmul", [T("h", B16), T("Wg", B16)], [T("g", B16)], author="cublas")
-    new("u", [S, I], B16); srv.must("matmul", [T("h", B16), T("Wu", B16)], [T("u", B16)], author="cublas")
-    new("sg", [S, I], B16); srv.must("mulscalar", [T("g", B16), "var<float32>:-1"], [T("sg", B16)])
-    srv.must("exp", [T("sg", B16)], [T("sg", B16)])
-    srv.must("addscalar", [T("sg", B16), "var<float32>:1"], [T("sg", B16)])
-    srv.must("rdivscalar", ["var<float32>:1", T("sg", B16)], [T("sg", B16)])
-    srv.must("mul", [T("g", B16), T("sg", B16)], [T("sg", B16)])
-    srv.must("mul", [T("sg", B16), T("u", B16)], [T("sg", B16)])
-    new("y", [S, Hd], B16); srv.must("matmul", [T("sg", B16), T("Wd", B16)], [T("y", B16)], author="cublas")
-    y = b2f(fetch(srv, tmp_path, "y")[0]).astype(np.float64)
+    new("q5_g", [S, I], B16); srv.must("matmul", [T("q5_h", B16), T("q5_Wg", B16)], [T("q5_g", B16)], author="cublas")
+    new("q5_u", [S, I], B16); srv.must("matmul", [T("q5_h", B16), T("q5_Wu", B16)], [T("q5_u", B16)], author="cublas")
+    new("q5_sg", [S, I], B16); srv.must("mulscalar", [T("q5_g", B16), "var<float32>:-1"], [T("q5_sg", B16)])
+    srv.must("exp", [T("q5_sg", B16)], [T("q5_sg", B16)])
+    srv.must("addscalar", [T("q5_sg", B16), "var<float32>:1"], [T("q5_sg", B16)])
+    srv.must("rdivscalar", ["var<float32>:1", T("q5_sg", B16)], [T("q5_sg", B16)])
+    srv.must("mul", [T("q5_g", B16), T("q5_sg", B16)], [T("q5_sg", B16)])
+    srv.must("mul", [T("q5_sg", B16), T("q5_u", B16)], [T("q5_sg", B16)])
+    new("q5_y", [S, Hd], B16); srv.must("matmul", [T("q5_sg", B16), T("q5_Wd", B16)], [T("q5_y", B16)], author="cublas")
+    y = b2f(fetch(srv, tmp_path, "q5_y")[0]).astype(np.float64)
     # float64 model of the same graph, with bf16 rounding where the graph stores bf16
     rb = lambda a: b2f(f2b(a.astype(np.float32))).astype(np.float64)
     xf = b2f(x).astype(np.float64)
@@ -282,7 +282,7 @@ def test_config5_mlp_block_over_ir(srv, tmp_path):
     act = rb(rb(g * rb(1.0 / rb(1.0 + rb(np.exp(rb(-g)))))) * u)
     yref = act @ b2f(Wd).astype(np.float64)
     assert np.abs(y - yref).max() <= 3e-2 * np.abs(yref).max()
-    hg = b2f(fetch(srv, tmp_path, "h")[0]).astype(np.float64)
+    hg = b2f(fetch(srv, tmp_path, "q5_h")[0]).astype(np.float64)
     assert np.abs(hg - h).max() <= 1e-2 * np.abs(h).max()
 
 

@@ -42,7 +42,7 @@ inline int unit_bytes(int64_t run_bytes, std::initializer_list<const void *> ptr
 // out is [rows, Lu] units, contiguous.  in row start = sum_i idx_i * stride_i (units) where idx
 // is the mixed-radix decomposition of the row number over `od`.  SPLAT: the input contributes a
 // single element of type E per row position (innermost axis broadcast) that fills the unit.
-template <typename U, typename I, bool SPLAT, typename E, bool REUSE>
+template <typename U, typename I, bool SPLAT, typename E, bool REUSE, bool NTS>
 __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const void *__restrict__ in_, U *__restrict__ out, I total,
                                                               I Lu, OuterDims od) {
     const I tile = (I)kBlock * kGatherUnroll;
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const void *__restr
         }
 #pragma unroll
         for (int u = 0; u < kGatherUnroll; ++u)
-            if (g[u] < total) st_nt(&out[g[u]], x[u]);
+            if (g[u] < total) st_sel<NTS>(&out[g[u]], x[u]);
     }
 }
 
@@ -87,10 +87,13 @@ int launch_gather_unit(const void *in, void *out, int64_t rows, int64_t Lu, cons
     using U = typename raw_of<UB>::type;
     const int64_t total = rows * Lu;
     unsigned grid = stream_grid(total, (int64_t)kBlock * kGatherUnroll, 0);
-    if (total < (int64_t)1 << 31)
-        gather_rows_kernel<U, uint32_t, SPLAT, E, REUSE><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint32_t)total, (uint32_t)Lu, od);
-    else
-        gather_rows_kernel<U, uint64_t, SPLAT, E, REUSE><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint64_t)total, (uint64_t)Lu, od);
+    const bool nts = use_nt_store((size_t)total * UB);
+    if (total < (int64_t)1 << 31) {
+        if (nts) gather_rows_kernel<U, uint32_t, SPLAT, E, REUSE, true><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint32_t)total, (uint32_t)Lu, od);
+        else gather_rows_kernel<U, uint32_t, SPLAT, E, REUSE, false><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint32_t)total, (uint32_t)Lu, od);
+    } else {
+        gather_rows_kernel<U, uint64_t, SPLAT, E, REUSE, true><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint64_t)total, (uint64_t)Lu, od);
+    }
     return launch_status();
 }
 

@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kBlock) void compare_kernel(const T *__restrict__ a
                     if constexpr (SCALAR) bb = sv; else bb = A(load_acc(y[u].v[k]));
                     r.v[k] = cmp_one<K, A>(A(load_acc(x[u].v[k])), bb, eps);
                 }
-                st_nt(&vm[j], r);
+                vm[j] = r;  // masks are a quarter or less of the traffic: plain stores
             }
         }
     });
@@ -135,7 +135,7 @@ int compare_all(int dtype, const void *a, const void *b, dxh_scalar s, float eps
 struct SwitchPtrs { const void *p[DXH_SWITCH_MAX]; };
 
 // bool cases, two tensors: C[i] = cases[i] ? t1[i] : t0[i]; both sources stream.
-template <typename R, int V>
+template <typename R, int V, bool NTS>
 __global__ __launch_bounds__(kBlock) void switch_bool_kernel(const R *__restrict__ t0, const R *__restrict__ t1,
                                                               const uint8_t *__restrict__ cases, R *__restrict__ c, int64_t n) {
     using VT = vec_t<R, V>;
@@ -160,7 +160,7 @@ __global__ __launch_bounds__(kBlock) void switch_bool_kernel(const R *__restrict
                 VT r;
 #pragma unroll
                 for (int k = 0; k < V; ++k) r.v[k] = w[u].v[k] ? y[u].v[k] : x[u].v[k];
-                st_nt(&vc[j], r);
+                st_sel<NTS>(&vc[j], r);
             }
         }
     });
@@ -194,10 +194,11 @@ int launch_switch(const void *const *tensors, int nt, int cases_dtype, const voi
         constexpr int V = kVecBytes / (int)sizeof(R);
         if (aligned(tensors[0], kVecBytes) && aligned(tensors[1], kVecBytes) && aligned(c, kVecBytes) && aligned(cases, V)) {
             unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
-            switch_bool_kernel<R, V><<<g, kBlock, 0, st>>>((const R *)tensors[0], (const R *)tensors[1], (const uint8_t *)cases, (R *)c, n);
+            if (use_nt_store((size_t)n * sizeof(R))) switch_bool_kernel<R, V, true><<<g, kBlock, 0, st>>>((const R *)tensors[0], (const R *)tensors[1], (const uint8_t *)cases, (R *)c, n);
+            else switch_bool_kernel<R, V, false><<<g, kBlock, 0, st>>>((const R *)tensors[0], (const R *)tensors[1], (const uint8_t *)cases, (R *)c, n);
         } else {
             unsigned g = stream_grid(n, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
-            switch_bool_kernel<R, 1><<<g, kBlock, 0, st>>>((const R *)tensors[0], (const R *)tensors[1], (const uint8_t *)cases, (R *)c, n);
+            switch_bool_kernel<R, 1, false><<<g, kBlock, 0, st>>>((const R *)tensors[0], (const R *)tensors[1], (const uint8_t *)cases, (R *)c, n);
         }
     } else if (cases_dtype == DXH_I32) {
         if (!aligned(cases, 4)) return DXH_ERR_ALIGN;
@@ -240,7 +241,7 @@ template <typename D, typename S> __device__ inline D cast_elem(S v) {
     }
 }
 
-template <typename S, typename D, int V>
+template <typename S, typename D, int V, bool NTS>
 __global__ __launch_bounds__(kBlock) void cast_kernel(const S *__restrict__ a, D *__restrict__ c, int64_t n) {
     using VS = vec_t<S, V>;
     using VD = vec_t<D, V>;
@@ -261,7 +262,7 @@ __global__ __launch_bounds__(kBlock) void cast_kernel(const S *__restrict__ a, D
                 VD r;
 #pragma unroll
                 for (int k = 0; k < V; ++k) r.v[k] = cast_elem<D, S>(x[u].v[k]);
-                st_nt(&vc[j], r);
+                st_sel<NTS>(&vc[j], r);
             }
         }
     });
@@ -277,10 +278,11 @@ template <typename S, typename D> int launch_cast(const void *a, void *c, int64_
     constexpr int V = kVecBytes / W;  // the wider side moves 16 bytes per lane
     if (aligned(a, V * sizeof(S)) && aligned(c, V * sizeof(D))) {
         unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
-        cast_kernel<S, D, V><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n);
+        if (use_nt_store((size_t)n * sizeof(D))) cast_kernel<S, D, V, true><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n);
+        else cast_kernel<S, D, V, false><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n);
     } else {
         unsigned g = stream_grid(n, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
-        cast_kernel<S, D, 1><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n);
+        cast_kernel<S, D, 1, false><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n);
     }
     return launch_status();
 }

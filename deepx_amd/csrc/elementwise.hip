@@ -69,7 +69,7 @@ template <int U, typename Body> __device__ inline void tile_loop(int64_t nv, Bod
     }
 }
 
-template <typename T, int V, typename Op>
+template <typename T, int V, typename Op, bool NTS>
 __global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a, const T *__restrict__ b,
                                                          T *__restrict__ c, int64_t n) {
     using VT = vec_t<T, V>;
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a,
                 VT r;
 #pragma unroll
                 for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(A(load_acc(x[u].v[k])), A(load_acc(y[u].v[k]))));
-                st_nt(&vc[j], r);
+                st_sel<NTS>(&vc[j], r);
             }
         }
     });
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a,
     }
 }
 
-template <typename T, int V, typename Op>
+template <typename T, int V, typename Op, bool NTS>
 __global__ __launch_bounds__(kBlock) void scalar_kernel(const T *__restrict__ a, const T s, T *__restrict__ c, int64_t n) {
     using VT = vec_t<T, V>;
     using A = acc_t<T>;
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kBlock) void scalar_kernel(const T *__restrict__ a,
                 VT r;
 #pragma unroll
                 for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(A(load_acc(x[u].v[k])), sv));
-                st_nt(&vc[j], r);
+                st_sel<NTS>(&vc[j], r);
             }
         }
     });
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kBlock) void scalar_kernel(const T *__restrict__ a,
     }
 }
 
-template <typename T, int V, typename Op>
+template <typename T, int V, typename Op, bool NTS>
 __global__ __launch_bounds__(kBlock) void unary_kernel(const T *__restrict__ a, T *__restrict__ c, int64_t n) {
     using VT = vec_t<T, V>;
     const int64_t nv = n / V;
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(kBlock) void unary_kernel(const T *__restrict__ a, 
                 VT r;
 #pragma unroll
                 for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(load_acc(x[u].v[k])));
-                st_nt(&vc[j], r);
+                st_sel<NTS>(&vc[j], r);
             }
         }
     });
@@ -172,10 +172,11 @@ int launch_binary(const void *a, const void *b, void *c, int64_t n, hipStream_t 
     constexpr int V = vec_len<T>;
     if (aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes)) {
         unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnroll, kBlocksPerCU);
-        binary_kernel<T, V, Op><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n);
+        if (use_nt_store((size_t)n * sizeof(T))) binary_kernel<T, V, Op, true><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n);
+        else binary_kernel<T, V, Op, false><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n);
     } else {
         unsigned g = stream_grid(n, (int64_t)kBlock * kUnroll, kBlocksPerCU);
-        binary_kernel<T, 1, Op><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n);
+        binary_kernel<T, 1, Op, false><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n);
     }
     return launch_status();
 }
@@ -186,10 +187,11 @@ int launch_scalar(const void *a, dxh_scalar s, void *c, int64_t n, hipStream_t s
     const T sv = scalar_to<T>(s);
     if (aligned(a, kVecBytes) && aligned(c, kVecBytes)) {
         unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnroll, kBlocksPerCU);
-        scalar_kernel<T, V, Op><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n);
+        if (use_nt_store((size_t)n * sizeof(T))) scalar_kernel<T, V, Op, true><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n);
+        else scalar_kernel<T, V, Op, false><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n);
     } else {
         unsigned g = stream_grid(n, (int64_t)kBlock * kUnroll, kBlocksPerCU);
-        scalar_kernel<T, 1, Op><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n);
+        scalar_kernel<T, 1, Op, false><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n);
     }
     return launch_status();
 }
@@ -199,10 +201,11 @@ int launch_unary(const void *a, void *c, int64_t n, hipStream_t st) {
     constexpr int V = vec_len<T>;
     if (aligned(a, kVecBytes) && aligned(c, kVecBytes)) {
         unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnroll, kBlocksPerCU);
-        unary_kernel<T, V, Op><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n);
+        if (use_nt_store((size_t)n * sizeof(T))) unary_kernel<T, V, Op, true><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n);
+        else unary_kernel<T, V, Op, false><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n);
     } else {
         unsigned g = stream_grid(n, (int64_t)kBlock * kUnroll, kBlocksPerCU);
-        unary_kernel<T, 1, Op><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n);
+        unary_kernel<T, 1, Op, false><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n);
     }
     return launch_status();
 }

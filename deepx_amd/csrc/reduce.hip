@@ -227,6 +227,7 @@ struct Stage {
     int G;               // row: lanes per row
     int TX, ctiles;      // col: column lanes, column tiles
     int V;               // vector length in elements of the stage's input type (1 or 16/size)
+    bool may_split;      // col stage: parallelism may come from splitting R
     bool in_is_acc, out_is_acc;
     size_t out_off;      // offset of the output inside the workspace when out_is_acc
 };
@@ -238,7 +239,17 @@ struct Plan {
 };
 
 inline int pow2_ceil(int64_t x) { int p = 1; while (p < x && p < (1 << 30)) p <<= 1; return p; }
-constexpr int kTargetBlocks = 4 * kCUs;
+
+// Column-lane count of a col stage.  Splittable stages (large R) give every workgroup the widest
+// contiguous row segment (TX = 256 lanes x 16 bytes = 4 KiB, TY = 1: no cross-lane reduction, the
+// DRAM-friendliest pattern) and get their parallelism from splitting R.  Stages that may not split
+// (the second pass over partials) narrow TX instead until enough workgroups exist.
+inline int col_lanes(int64_t pre, int64_t postv, bool may_split) {
+    int tx = (int)std::min<int64_t>(tuning().reduce_col_max_lanes, pow2_ceil(postv));
+    if (may_split) return tx;
+    while (tx > 16 && pre * ((postv + tx - 1) / tx) < kCUs) tx >>= 1;
+    return tx;
+}
 
 // normalise dims like checkedDims (shape_reduce.cpp:11-45); returns false if out of range
 inline bool reduced_mask(int ndim, const int32_t *dims, int ndims, bool *mask) {
@@ -271,6 +282,7 @@ inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, cons
     for (auto &x : d) any |= x.red;
     if (!any) { pl.copy_only = true; return DXH_OK; }
 
+    const int64_t kTarget = tuning().reduce_target_blocks;
     bool first = true;
     size_t off = 0;
     auto push = [&](Stage st, bool last) {
@@ -284,7 +296,7 @@ inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, cons
         } else {
             st.V = (st.post % vfull == 0) ? vfull : 1;
             int64_t postv = st.post / st.V;
-            st.TX = (int)std::min<int64_t>(64, pow2_ceil(postv));
+            st.TX = col_lanes(st.pre, postv, st.may_split);
             st.ctiles = (int)((postv + st.TX - 1) / st.TX);
         }
         if (st.out_is_acc) {
@@ -315,23 +327,26 @@ inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, cons
             int64_t vecs = (R + vfull - 1) / vfull;
             int G = vecs >= 2 * kWave ? kBlock : (int)std::min<int64_t>(kWave, pow2_ceil(vecs));
             int64_t blocks0 = (pre + (kBlock / G) - 1) / (kBlock / G);
-            if (G == kBlock && blocks0 < kTargetBlocks) {
+            if (G == kBlock && blocks0 < kTarget) {
                 int64_t min_chunk = 8192;  // elements: 8+ vector trips per lane
                 int64_t smax = std::max<int64_t>(1, R / min_chunk);
-                S = (int)std::min<int64_t>((kTargetBlocks + blocks0 - 1) / blocks0, smax);
+                S = (int)std::min<int64_t>((kTarget + blocks0 - 1) / blocks0, smax);
             }
             st.G = G;
         } else {
             int V = (post % vfull == 0) ? vfull : 1;
             int64_t postv = post / V;
-            int TX = (int)std::min<int64_t>(64, pow2_ceil(postv));
+            st.may_split = true;
+            int TX = col_lanes(pre, postv, true);
             int TY = kBlock / TX;
             int64_t blocks0 = pre * ((postv + TX - 1) / TX);
-            if (blocks0 < kTargetBlocks) {
-                int64_t min_rows = (int64_t)TY * 16;
+            const int64_t col_target = tuning().reduce_col_target_blocks;
+            if (blocks0 < col_target) {
+                int64_t min_rows = (int64_t)TY * tuning().reduce_col_min_rows;
                 int64_t smax = std::max<int64_t>(1, R / min_rows);
-                S = (int)std::min<int64_t>((kTargetBlocks + blocks0 - 1) / blocks0, smax);
+                S = (int)std::min<int64_t>((col_target + blocks0 - 1) / blocks0, smax);
             }
+            if (S == 1) st.may_split = false;  // nothing to split: narrow TX for parallelism instead
         }
         st.S = S;
         int64_t chunk = (R + S - 1) / S;
@@ -373,7 +388,7 @@ int launch_stage(const Stage &st, const void *in, void *out, hipStream_t stream)
         bool vec = st.V == VF && aligned(in, kVecBytes);
         int TX = st.TX, ctiles = st.ctiles;
         if (!vec && st.V != 1) {  // planned for vectors but the pointer is misaligned
-            TX = (int)std::min<int64_t>(64, pow2_ceil(st.post));
+            TX = col_lanes(st.pre, st.post, st.may_split);
             ctiles = (int)((st.post + TX - 1) / TX);
         }
         int64_t gx = st.pre * st.S * ctiles;

@@ -7,9 +7,30 @@
 
 using namespace dxh;
 
+namespace dxh {
+Tuning &tuning() {
+    static Tuning t;
+    return t;
+}
+}  // namespace dxh
+
 extern "C" {
 
 int dxh_version(void) { return 100; }
+
+int dxh_tune(int knob, int64_t value) {
+    Tuning &t = tuning();
+    switch (knob) {
+    case DXH_TUNE_NT_STORE_BYTES: t.nt_store_bytes = value; return DXH_OK;
+    case DXH_TUNE_REDUCE_TARGET_BLOCKS: if (value < 1) return DXH_ERR_ARG; t.reduce_target_blocks = value; t.reduce_col_target_blocks = value; return DXH_OK;
+    case DXH_TUNE_REDUCE_COL_MIN_ROWS: if (value < 1) return DXH_ERR_ARG; t.reduce_col_min_rows = value; return DXH_OK;
+    case DXH_TUNE_REDUCE_COL_MAX_LANES:
+        if (value != 16 && value != 32 && value != 64 && value != 128 && value != 256) return DXH_ERR_ARG;
+        t.reduce_col_max_lanes = value;
+        return DXH_OK;
+    default: return DXH_ERR_ARG;
+    }
+}
 
 const char *dxh_error_string(int code) {
     switch (code) {

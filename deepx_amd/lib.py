@@ -49,6 +49,7 @@ _RED = [_i, _p, _pi32, _i, _pi32, _i, _p, _p, _sz, _p]
 SIGNATURES = {
     "dxh_version": ([], _i),
     "dxh_error_string": ([_i], C.c_char_p),
+    "dxh_tune": ([_i, _i64], _i),
     "dxh_device_count": ([C.POINTER(_i)], _i),
     "dxh_set_device": ([_i], _i),
     "dxh_device_name": ([C.c_char_p, _sz], _i),

@@ -72,3 +72,27 @@ DXE_API size_t dxe_shape_yaml_roundtrip(const char *yaml, char *out, size_t bufl
         return copy_out(std::string("error: ") + e.what(), out, buflen);
     }
 }
+// shape inference helpers by name, result as space-separated ints or "error: ...":
+//   transpose(a=shape, b=order) broadcast(a, b) indexselect(a=input, b=index shape, extra=axis)
+//   repeat(a=shape, b=repeats) checked_dims(a=shape, b=dims) reduced(a=shape, b=checked dims, extra=keepdims)
+//   concat2(a, b, extra=axis) matmul(a, b)
+DXE_API size_t dxe_infer_shape(const char *op, const int *a, int na, const int *b, int nb, int extra, char *out, size_t buflen) {
+    try {
+        std::vector<int> A(a, a + na), B(b, b + nb), r;
+        std::string o = op ? op : "";
+        if (o == "transpose") r = transpose_shape(A, B);
+        else if (o == "broadcast") r = broadcast_shape(A, B);
+        else if (o == "indexselect") r = indexselect_shape(A, B, extra);
+        else if (o == "repeat") r = repeat_shape(A, B);
+        else if (o == "checked_dims") r = checked_dims(A, B);
+        else if (o == "reduced") r = reduced_shape(A, B, extra != 0);
+        else if (o == "concat2") r = concat_shape({A, B}, extra);
+        else if (o == "matmul") r = matmul_shape(A, B);
+        else return copy_out("error: unknown op", out, buflen);
+        std::string s;
+        for (size_t i = 0; i < r.size(); ++i) s += (i ? " " : "") + std::to_string(r[i]);
+        return copy_out(s, out, buflen);
+    } catch (const std::exception &e) {
+        return copy_out(std::string("error: ") + e.what(), out, buflen);
+    }
+}

@@ -81,9 +81,12 @@ inline Precision precision_word(const std::string &w) {
     if (w == "float8") return Precision::Float8;
     return Precision::Any;
 }
-// The reference's precision() takes a single word; its own op tables print unions
-// ("float64|float32"), so unions are accepted here too and OR-ed together.
-inline Precision precision_from(const std::string &s) {
+// On the wire the reference's precision() takes a single word, so a union such as
+// "float64|float32" is an unknown word and means "any" (dtype.hpp:321-364) — kept as is.
+inline Precision precision_from(const std::string &s) { return precision_word(s); }
+// Registration side only: the op table is written with unions ("int64|int32|bool"), which the
+// reference builds from Precision bit-ors in C++ (tfs.cpp) and prints in this form.
+inline Precision precision_union_from(const std::string &s) {
     if (s.find('|') == std::string::npos) return precision_word(s);
     uint16_t bits = 0;
     for (const auto &w : split_bar(s)) bits |= uint16_t(precision_word(w));
@@ -116,6 +119,11 @@ inline TypeDef typedef_from(const std::string &s) {
     size_t lt = s.find('<'), gt = s.find('>');
     if (lt == std::string::npos || gt == std::string::npos) return TypeDef(category_from(s), Precision::Any);
     return TypeDef(category_from(s.substr(0, lt)), precision_from(s.substr(lt + 1, gt - lt - 1)));
+}
+inline TypeDef typedef_union_from(const std::string &s) {
+    size_t lt = s.find('<'), gt = s.find('>');
+    if (lt == std::string::npos || gt == std::string::npos) return TypeDef(category_from(s), Precision::Any);
+    return TypeDef(category_from(s.substr(0, lt)), precision_union_from(s.substr(lt + 1, gt - lt - 1)));
 }
 inline std::string typedef_str(const TypeDef &t) { return category_str(t.category) + "<" + precision_str(t.precision) + ">"; }
 

@@ -55,8 +55,16 @@ void reg(TfFactory &f, const char *name, const char *author, const char *tftype,
     tf->metadata.author = author;
     tf->tftype = tftype;
     tf->formula = formula;
-    for (const char *a : args) tf->args.push_back(Param::parse(a));
-    for (const char *r : returns) tf->returns.push_back(Param::parse(r));
+    auto registered = [](const char *text) {  // "type:name" with precision unions allowed
+        std::string t = text;
+        size_t colon = t.find(':');
+        Param p;
+        p.dtype = typedef_union_from(t.substr(0, colon));
+        p.textvalue = t.substr(colon + 1);
+        return p;
+    };
+    for (const char *a : args) tf->args.push_back(registered(a));
+    for (const char *r : returns) tf->returns.push_back(registered(r));
     tf->fn = std::move(fn);
     f.add_tf(tf);
 }

@@ -28,6 +28,8 @@ class InProc:
             fn = getattr(L, name)
             fn.argtypes = args + [C.c_char_p, C.c_size_t]
             fn.restype = C.c_size_t
+        L.dxe_infer_shape.argtypes = [C.c_char_p, C.POINTER(C.c_int), C.c_int, C.POINTER(C.c_int), C.c_int, C.c_int, C.c_char_p, C.c_size_t]
+        L.dxe_infer_shape.restype = C.c_size_t
         self.L = L
         self.ex = L.dxe_create()
         assert self.ex
@@ -44,6 +46,51 @@ class InProc:
     def typedef(self, text): return self._call(self.L.dxe_typedef_roundtrip, text.encode())
     def tensor_yaml(self, name): return self._call(self.L.dxe_tensor_yaml, self.ex, name.encode())
     def shape_yaml(self, text): return self._call(self.L.dxe_shape_yaml_roundtrip, text.encode())
+
+    def infer(self, op, a, b=(), extra=0):
+        A = (C.c_int * max(1, len(a)))(*a)
+        B = (C.c_int * max(1, len(b)))(*b)
+        return self._call(self.L.dxe_infer_shape, op.encode(), A, len(a), B, len(b), extra)
+
+
+REF_SO = os.path.join(ROOT, "oracle", "_ref", "libdeepxref.so")
+
+
+class Reference:
+    """The reference's own deepxcore code (IR parser, dtype strings, factory, shape inference),
+    compiled by oracle/ref.mk from the reference checkout.  Test-side only."""
+
+    def __init__(self):
+        L = C.CDLL(REF_SO)
+        ip = C.POINTER(C.c_int)
+        sigs = {"ref_parse": [C.c_char_p], "ref_typedef": [C.c_char_p], "ref_match": [C.c_char_p, C.c_char_p],
+                "ref_transpose_shape": [ip, C.c_int, ip], "ref_broadcast_shape": [ip, C.c_int, ip, C.c_int],
+                "ref_indexselect_shape": [ip, C.c_int, ip, C.c_int, C.c_int], "ref_repeat_shape": [ip, C.c_int, ip, C.c_int],
+                "ref_checked_dims": [ip, C.c_int, ip, C.c_int], "ref_reduced_shape": [ip, C.c_int, ip, C.c_int, C.c_int]}
+        for name, args in sigs.items():
+            fn = getattr(L, name)
+            fn.argtypes = args + [C.c_char_p, C.c_size_t]
+            fn.restype = C.c_size_t
+        self.L = L
+
+    def _call(self, fn, *args):
+        buf = C.create_string_buffer(1 << 16)
+        fn(*args, buf, len(buf))
+        return buf.value.decode("utf-8")
+
+    @staticmethod
+    def _arr(v):
+        return (C.c_int * max(1, len(v)))(*v)
+
+    def parse(self, line): return self._call(self.L.ref_parse, line.encode())
+    def typedef(self, text): return self._call(self.L.ref_typedef, text.encode())
+    def match(self, registered_rows, call): return self._call(self.L.ref_match, "\n".join(registered_rows).encode(), call.encode())
+    def transpose_shape(self, s, o): return self._call(self.L.ref_transpose_shape, self._arr(s), len(s), self._arr(o))
+    def broadcast_shape(self, a, b): return self._call(self.L.ref_broadcast_shape, self._arr(a), len(a), self._arr(b), len(b))
+    def indexselect_shape(self, a, b, axis): return self._call(self.L.ref_indexselect_shape, self._arr(a), len(a), self._arr(b), len(b), axis)
+    def repeat_shape(self, a, b): return self._call(self.L.ref_repeat_shape, self._arr(a), len(a), self._arr(b), len(b))
+    def checked_dims(self, s, d): return self._call(self.L.ref_checked_dims, self._arr(s), len(s), self._arr(d), len(d))
+    def reduced_shape(self, s, d, keep): return self._call(self.L.ref_reduced_shape, self._arr(s), len(s), self._arr(d), len(d), int(keep))
 
 
 def free_port():

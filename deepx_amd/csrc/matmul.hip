@@ -115,6 +115,149 @@ __global__ __launch_bounds__(kBlock) void matmul_mfma_kernel(const T *__restrict
             }
 }
 
+// ---- pipelined MFMA kernel ----------------------------------------------------------------
+// Workgroup tile 128x128, K step 64, 4 waves (2x2), each wave 64x64 = 2x2 MFMA 32x32x16 tiles and
+// 4 k-substeps per K step.  Requirements (checked by the launcher): K % 8 == 0, N % 8 == 0 and
+// 16-byte aligned A, B, C.
+//   LDS   two stages of {A tile [128 m][64 k], B tile transposed [128 n][64 k]}, rows of exactly
+//         128 bytes; the 16-byte chunk c of row r lives at chunk c ^ ((r ^ (r >> 3)) & 7), which
+//         makes the MFMA operand reads (32 consecutive rows, one chunk), the A stores (one row,
+//         8 chunks) and the B stores (rows 4 apart) all bank-conflict free.
+//   A     16-byte global loads straight into ds_write_b128.
+//   B     arrives n-contiguous: a lane loads 8 k-rows x 4 n (8 bytes each, 256 B contiguous per
+//         wave row), transposes 8x4 -> 4x8 in registers with v_perm_b32 and stores four 16-byte
+//         k-runs.
+//   pipe  the global loads of K step t+1 are issued before the MFMAs of step t and land in the
+//         other LDS stage afterwards: one barrier per K step.
+//   C     fp32 accumulators -> RNE to bf16/f16 -> staged through LDS -> 16-byte row stores.
+constexpr int PM = 128, PN = 128, PK = 64;
+constexpr int kStageElems = PM * PK;  // elements per operand tile per stage
+
+__device__ inline int swz(int row, int chunk) { return chunk ^ ((row ^ (row >> 3)) & 7); }
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void matmul_mfma_pipe_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
+                                                                   int M, int K, int N, int tiles_m, int tiles_n) {
+    // 2 stages x (A + B) x 16 KiB = 64 KiB; the epilogue reuses it as a [128][136] staging tile
+    __shared__ __attribute__((aligned(16))) uint16_t lds[4 * kStageElems];
+    int64_t bid = blockIdx.x;
+    const int tn = (int)(bid % tiles_n); bid /= tiles_n;
+    const int tm = (int)(bid % tiles_m); bid /= tiles_m;
+    A += bid * (int64_t)M * K;
+    B += bid * (int64_t)K * N;
+    C += bid * (int64_t)M * N;
+    const int m0 = tm * PM, n0 = tn * PN;
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+    const int wm = w >> 1, wn = w & 1;
+    const uint16_t *Ar = reinterpret_cast<const uint16_t *>(A);
+    const uint16_t *Br = reinterpret_cast<const uint16_t *>(B);
+
+    // per-lane global coordinates of its loads
+    // A: 4 x 16 bytes: chunk index t + i*256 -> row (0..127), chunk (0..7)
+    // B: 8 x 8 bytes:  n4 = t % 32 (4 columns), kg = t / 32 (8 k-rows)
+    const int bn4 = t & 31, bkg = t >> 5;
+    uint4 ra[4];
+    uint2 rb[8];
+
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = t + i * kBlock, row = c >> 3, ch = c & 7;
+            const int gm = m0 + row, gk = k0 + ch * 8;
+            ra[i] = (gm < M && gk < K) ? *reinterpret_cast<const uint4 *>(Ar + (int64_t)gm * K + gk) : uint4{0, 0, 0, 0};
+        }
+        const int gn = n0 + bn4 * 4;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const int gk = k0 + bkg * 8 + r;
+            rb[r] = (gk < K && gn < N) ? *reinterpret_cast<const uint2 *>(Br + (int64_t)gk * N + gn) : uint2{0, 0};
+        }
+    };
+    auto store_lds = [&](int stage) {
+        uint16_t *As = lds + stage * 2 * kStageElems, *Bs = As + kStageElems;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = t + i * kBlock, row = c >> 3, ch = c & 7;
+            *reinterpret_cast<uint4 *>(As + row * PK + swz(row, ch) * 8) = ra[i];
+        }
+        // 8x4 -> 4x8 transpose: column j of the 8 loaded rows becomes one 16-byte k-run
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint4 v;
+            uint32_t *vp = reinterpret_cast<uint32_t *>(&v);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t lo = (j < 2) ? rb[2 * q].x : rb[2 * q].y, hi = (j < 2) ? rb[2 * q + 1].x : rb[2 * q + 1].y;
+                vp[q] = (j & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u) : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+            }
+            const int row = bn4 * 4 + j;
+            *reinterpret_cast<uint4 *>(Bs + row * PK + swz(row, bkg) * 8) = v;
+        }
+    };
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    const int KT = (K + PK - 1) / PK;
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const int stage = kt & 1;
+        if (kt + 1 < KT) load_global((kt + 1) * PK);
+        const uint16_t *As = lds + stage * 2 * kStageElems, *Bs = As + kStageElems;
+#pragma unroll
+        for (int ks = 0; ks < PK / 16; ++ks) {
+            uint4 af[2], bf[2];
+            const int ch = ks * 2 + (lane >> 5);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int row = wm * 64 + i * 32 + (lane & 31);
+                af[i] = *reinterpret_cast<const uint4 *>(As + row * PK + swz(row, ch) * 8);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int row = wn * 64 + j * 32 + (lane & 31);
+                bf[j] = *reinterpret_cast<const uint4 *>(Bs + row * PK + swz(row, ch) * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = mfma32<T>(af[i], bf[j], acc[i][j]);
+        }
+        if (kt + 1 < KT) store_lds(stage ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: stage the 128x128 result tile in LDS, then 16-byte row stores
+    constexpr int LDC = PN + 8;  // 272-byte rows
+    uint16_t *Cs = lds;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = wm * 64 + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                const int col = wn * 64 + j * 32 + (lane & 31);
+                Cs[row * LDC + col] = store_acc<T>(acc[i][j][v]).bits;
+            }
+    __syncthreads();
+    uint16_t *Cr = reinterpret_cast<uint16_t *>(C);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int c = t + i * kBlock, row = c >> 4, ch = c & 15;
+        const int gm = m0 + row, gn = n0 + ch * 8;
+        if (gm < M && gn < N)  // N % 8 == 0: a chunk is either fully inside or fully outside
+            st_nt(reinterpret_cast<uint4 *>(Cr + (int64_t)gm * N + gn), *reinterpret_cast<const uint4 *>(Cs + row * LDC + ch * 8));
+    }
+}
+
 // ---- generic tiled kernel (f32, f64, integers) ------------------------------------------
 constexpr int GT = 64, GK = 16;
 template <typename T>
@@ -183,6 +326,13 @@ __global__ __launch_bounds__(kBlock) void matmul_tiled_kernel(const T *__restric
 
 template <typename T>
 int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    if (k % 8 == 0 && n % 8 == 0 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes) && m >= 64 && n >= 64) {
+        const int64_t ptm = (m + PM - 1) / PM, ptn = (n + PN - 1) / PN;
+        const int64_t pblocks = batch * ptm * ptn;
+        if (pblocks > 0x7fffffff) return DXH_ERR_SHAPE;
+        matmul_mfma_pipe_kernel<T><<<(unsigned)pblocks, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, (int)ptm, (int)ptn);
+        return launch_status();
+    }
     const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     const int64_t blocks = batch * tiles_m * tiles_n;
     if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;

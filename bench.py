@@ -28,6 +28,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 MFMA_BF16_PEAK_TF = 2500.0  # dense bf16
+REDUCE_ROW_TRAFFIC_BYTES = 268646213  # measured, see profiles/bench_pmc_hbm_traffic.md
 
 
 def main():
@@ -144,7 +145,10 @@ def main():
     roofline = {"bound": "hbm", "kernel": "reduce_row_kernel<sum|max|min,f32> [8192,8192] axis 1 (6 of 10 launches per step)",
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "avg_launch_ms": round(dom_ms, 5),
-                "bytes_per_launch": XB, "traffic": None}
+                "bytes_per_launch": XB,
+                # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the
+                # reading of a plain copy kernel of known size (profiles/bench_pmc_hbm_traffic.md)
+                "traffic": REDUCE_ROW_TRAFFIC_BYTES}
 
     # ---------------- the other BASELINE configs, one op at a time ----------------------------
     per_op = {"config2": c2}

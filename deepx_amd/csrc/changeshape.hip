@@ -28,6 +28,8 @@ struct OuterDims {
     int n;                        // number of outer (row-indexing) dims
     uint32_t size[kMaxOuter];     // output extent of each
     int64_t stride[kMaxOuter];    // input stride of each, in units
+    FastDiv fsize[kMaxOuter];     // divide-free division by size[d] (32-bit index path)
+    FastDiv fLu;                  // ... and by the units per row
 };
 
 // widest power-of-two unit (<= 16 bytes) dividing `bytes` and every pointer in `ptrs`
@@ -42,7 +44,7 @@ inline int unit_bytes(int64_t run_bytes, std::initializer_list<const void *> ptr
 // out is [rows, Lu] units, contiguous.  in row start = sum_i idx_i * stride_i (units) where idx
 // is the mixed-radix decomposition of the row number over `od`.  SPLAT: the input contributes a
 // single element of type E per row position (innermost axis broadcast) that fills the unit.
-template <typename U, typename I, bool SPLAT, typename E, bool REUSE, bool NTS>
+template <typename U, typename I, bool SPLAT, typename E, bool REUSE, bool NTS, int ND>
 __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const void *__restrict__ in_, U *__restrict__ out, I total,
                                                               I Lu, OuterDims od) {
     const I tile = (I)kBlock * kGatherUnroll;
@@ -54,13 +56,35 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const void *__restr
         for (int u = 0; u < kGatherUnroll; ++u) {
             g[u] = base + (I)u * kBlock + threadIdx.x;
             if (g[u] < total) {
-                I row = g[u] / Lu;
-                I v = g[u] - row * Lu;
+                I row, v;
                 int64_t off = 0;
-                for (int d = od.n - 1; d >= 0; --d) {
-                    I q = row / od.size[d];
-                    off += (int64_t)(row - q * od.size[d]) * od.stride[d];
-                    row = q;
+                if constexpr (sizeof(I) == 4 && ND >= 0) {
+                    // ND outer dims, fully unrolled: every extent, stride and magic number sits in
+                    // scalar registers loaded once, and the address chain has no memory access in it
+                    row = fast_div(g[u], od.fLu);
+                    v = g[u] - row * Lu;
+#pragma unroll
+                    for (int d = ND - 1; d >= 0; --d) {
+                        uint32_t q = fast_div(row, od.fsize[d]);
+                        off += (int64_t)(row - q * od.size[d]) * od.stride[d];
+                        row = q;
+                    }
+                } else if constexpr (sizeof(I) == 4) {
+                    row = fast_div(g[u], od.fLu);
+                    v = g[u] - row * Lu;
+                    for (int d = od.n - 1; d >= 0; --d) {
+                        uint32_t q = fast_div(row, od.fsize[d]);
+                        off += (int64_t)(row - q * od.size[d]) * od.stride[d];
+                        row = q;
+                    }
+                } else {
+                    row = g[u] / Lu;
+                    v = g[u] - row * Lu;
+                    for (int d = od.n - 1; d >= 0; --d) {
+                        I q = row / od.size[d];
+                        off += (int64_t)(row - q * od.size[d]) * od.stride[d];
+                        row = q;
+                    }
                 }
                 if constexpr (SPLAT) {
                     E e = reinterpret_cast<const E *>(in_)[off];
@@ -83,16 +107,26 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const void *__restr
 }
 
 template <int UB, bool SPLAT, typename E, bool REUSE = false>
-int launch_gather_unit(const void *in, void *out, int64_t rows, int64_t Lu, const OuterDims &od, hipStream_t st) {
+int launch_gather_unit(const void *in, void *out, int64_t rows, int64_t Lu, const OuterDims &od_in, hipStream_t st) {
     using U = typename raw_of<UB>::type;
     const int64_t total = rows * Lu;
+    OuterDims od = od_in;
+    for (int d = 0; d < od.n; ++d) od.fsize[d] = make_fastdiv(od.size[d]);
+    od.fLu = make_fastdiv((uint32_t)std::min<int64_t>(Lu, 0xffffffffLL));
     unsigned grid = stream_grid(total, (int64_t)kBlock * kGatherUnroll, 0);
-    const bool nts = use_nt_store((size_t)total * UB);
     if (total < (int64_t)1 << 31) {
-        if (nts) gather_rows_kernel<U, uint32_t, SPLAT, E, REUSE, true><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint32_t)total, (uint32_t)Lu, od);
-        else gather_rows_kernel<U, uint32_t, SPLAT, E, REUSE, false><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint32_t)total, (uint32_t)Lu, od);
+#define DXH_G(ND) gather_rows_kernel<U, uint32_t, SPLAT, E, REUSE, true, ND><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint32_t)total, (uint32_t)Lu, od)
+        switch (od.n) {
+        case 0: DXH_G(0); break;
+        case 1: DXH_G(1); break;
+        case 2: DXH_G(2); break;
+        case 3: DXH_G(3); break;
+        case 4: DXH_G(4); break;
+        default: DXH_G(-1); break;
+        }
+#undef DXH_G
     } else {
-        gather_rows_kernel<U, uint64_t, SPLAT, E, REUSE, true><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint64_t)total, (uint64_t)Lu, od);
+        gather_rows_kernel<U, uint64_t, SPLAT, E, REUSE, true, -1><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint64_t)total, (uint64_t)Lu, od);
     }
     return launch_status();
 }
@@ -191,33 +225,33 @@ struct ConcatSrcs {
     int64_t run[kConcatMax];     // units per outer row of this source
     int64_t pref[kConcatMax];    // unit offset of this source inside an output row
     int64_t cum[kConcatMax + 1]; // units before this source in the flattened work list
+    FastDiv frun[kConcatMax];    // divide-free division by run[i] when everything fits 32 bits
 };
 
-template <typename U>
-__global__ __launch_bounds__(kBlock) void concat_kernel(ConcatSrcs s, U *__restrict__ out, int64_t out_row, int64_t total) {
-    const int64_t tile = (int64_t)kBlock * kGatherUnroll;
-    const int64_t stride = (int64_t)gridDim.x * tile;
-    for (int64_t base = (int64_t)blockIdx.x * tile; base < total; base += stride) {
-        U x[kGatherUnroll];
-        int64_t dst[kGatherUnroll];
+// blockIdx.y = source, so run / prefix / pointer are wave-uniform scalars and the only per-lane
+// work before the data load is one divide-free division.
+template <typename U, bool FAST>
+__global__ __launch_bounds__(kBlock) void concat_kernel(ConcatSrcs s, U *__restrict__ out, int64_t out_row, int64_t outer) {
+    const int i = blockIdx.y;
+    const U *__restrict__ src = nullptr;
+    int64_t run = 1, pref = 0;
+    FastDiv frun{1, 0, 0};
 #pragma unroll
-        for (int u = 0; u < kGatherUnroll; ++u) {
-            int64_t g = base + (int64_t)u * kBlock + threadIdx.x;
-            dst[u] = -1;
-            if (g < total) {
-                int i = 0;
-#pragma unroll
-                for (int k = 1; k < kConcatMax; ++k) if (k < s.n && g >= s.cum[k]) i = k;
-                int64_t local = g - s.cum[i];
-                int64_t o = local / s.run[i];
-                int64_t v = local - o * s.run[i];
-                x[u] = ld_nt(reinterpret_cast<const U *>(s.ptr[i]) + local);
-                dst[u] = o * out_row + s.pref[i] + v;
-            }
+    for (int k = 0; k < kConcatMax; ++k)
+        if (k == i) { src = reinterpret_cast<const U *>(s.ptr[k]); run = s.run[k]; pref = s.pref[k]; frun = s.frun[k]; }
+    const int64_t total = run * outer;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t g = (int64_t)blockIdx.x * kBlock + threadIdx.x; g < total; g += stride) {
+        int64_t o, v;
+        if constexpr (FAST) {
+            const uint32_t oo = fast_div((uint32_t)g, frun);
+            o = oo;
+            v = (uint32_t)g - oo * (uint32_t)run;
+        } else {
+            o = g / run;
+            v = g - o * run;
         }
-#pragma unroll
-        for (int u = 0; u < kGatherUnroll; ++u)
-            if (dst[u] >= 0) st_nt(&out[dst[u]], x[u]);
+        st_nt(&out[o * out_row + pref + v], ld_nt(&src[g]));
     }
 }
 
@@ -225,7 +259,7 @@ __global__ __launch_bounds__(kBlock) void concat_kernel(ConcatSrcs s, U *__restr
 template <typename U, typename IT>
 __global__ __launch_bounds__(kBlock) void indexselect_kernel(const U *__restrict__ in, const IT *__restrict__ index,
                                                               U *__restrict__ out, int64_t total, int64_t Lu, int64_t M,
-                                                              int64_t adim) {
+                                                              int64_t adim, FastDiv fLu, FastDiv fM, bool fast) {
     const int64_t tile = (int64_t)kBlock * kGatherUnroll;
     const int64_t stride = (int64_t)gridDim.x * tile;
     for (int64_t base = (int64_t)blockIdx.x * tile; base < total; base += stride) {
@@ -235,8 +269,15 @@ __global__ __launch_bounds__(kBlock) void indexselect_kernel(const U *__restrict
         for (int u = 0; u < kGatherUnroll; ++u) {
             g[u] = base + (int64_t)u * kBlock + threadIdx.x;
             if (g[u] < total) {
-                int64_t row = g[u] / Lu, v = g[u] - row * Lu;
-                int64_t p = row / M, j = row - p * M;
+                int64_t row, v, p, j;
+                if (fast) {  // everything fits 32 bits: divide-free
+                    const uint32_t r32 = fast_div((uint32_t)g[u], fLu), p32 = fast_div(r32, fM);
+                    row = r32; v = (uint32_t)g[u] - r32 * (uint32_t)Lu;
+                    p = p32; j = r32 - p32 * (uint32_t)M;
+                } else {
+                    row = g[u] / Lu; v = g[u] - row * Lu;
+                    p = row / M; j = row - p * M;
+                }
                 int64_t k = (int64_t)index[j];
                 k = k < 0 ? 0 : (k >= adim ? adim - 1 : k);
                 x[u] = in[(p * adim + k) * Lu + v];
@@ -382,6 +423,7 @@ int dxh_concat(int dtype, const void *const *ins, int nins, const int32_t *axis_
             int64_t run = (int64_t)axis_sizes[i] * inner * es / ub;
             if (run > 0) {
                 s.ptr[s.n] = ins[i]; s.run[s.n] = run; s.pref[s.n] = pref; s.cum[s.n] = cum;
+                s.frun[s.n] = make_fastdiv((uint32_t)std::min<int64_t>(run, 0xffffffffLL));
                 cum += run * outer;
                 ++s.n;
             }
@@ -390,14 +432,21 @@ int dxh_concat(int dtype, const void *const *ins, int nins, const int32_t *axis_
         }
         s.cum[s.n] = cum;
         if (s.n == 0 || cum == 0) continue;
-        unsigned grid = stream_grid(cum, (int64_t)kBlock * kGatherUnroll, 0);
+        int64_t max_units = 0;
+        for (int k = 0; k < s.n; ++k) max_units = std::max(max_units, s.run[k] * outer);
+        const bool fast = max_units < ((int64_t)1 << 32);
+        dim3 grid(stream_grid(max_units, kBlock, 0) > 0x7fffffffu ? 0x7fffffffu : stream_grid(max_units, kBlock, 0), (unsigned)s.n);
+#define DXH_CC(U)                                                                           \
+        if (fast) concat_kernel<U, true><<<grid, kBlock, 0, st>>>(s, (U *)out, out_row, outer); \
+        else concat_kernel<U, false><<<grid, kBlock, 0, st>>>(s, (U *)out, out_row, outer);
         switch (ub) {
-        case 16: concat_kernel<uint4><<<grid, kBlock, 0, st>>>(s, (uint4 *)out, out_row, cum); break;
-        case 8: concat_kernel<uint64_t><<<grid, kBlock, 0, st>>>(s, (uint64_t *)out, out_row, cum); break;
-        case 4: concat_kernel<uint32_t><<<grid, kBlock, 0, st>>>(s, (uint32_t *)out, out_row, cum); break;
-        case 2: concat_kernel<uint16_t><<<grid, kBlock, 0, st>>>(s, (uint16_t *)out, out_row, cum); break;
-        default: concat_kernel<uint8_t><<<grid, kBlock, 0, st>>>(s, (uint8_t *)out, out_row, cum); break;
+        case 16: DXH_CC(uint4) break;
+        case 8: DXH_CC(uint64_t) break;
+        case 4: DXH_CC(uint32_t) break;
+        case 2: DXH_CC(uint16_t) break;
+        default: DXH_CC(uint8_t) break;
         }
+#undef DXH_CC
         int rc = launch_status();
         if (rc != DXH_OK) return rc;
     }
@@ -476,11 +525,13 @@ int dxh_indexselect(int dtype, const void *in, const int32_t *in_shape, int in_n
     const int64_t total = pre * m * Lu;
     hipStream_t st = as_stream(stream);
     unsigned grid = stream_grid(total, (int64_t)kBlock * kGatherUnroll, 0);
+    const bool fast = total < ((int64_t)1 << 32) && Lu < ((int64_t)1 << 32) && m < ((int64_t)1 << 32);
+    const FastDiv fLu = make_fastdiv((uint32_t)std::min<int64_t>(Lu, 0xffffffffLL)), fM = make_fastdiv((uint32_t)std::min<int64_t>(m, 0xffffffffLL));
 #define DXH_IS(U)                                                                                                      \
     if (index_dtype == DXH_I64)                                                                                        \
-        indexselect_kernel<U, int64_t><<<grid, kBlock, 0, st>>>((const U *)in, (const int64_t *)index, (U *)out, total, Lu, m, adim); \
+        indexselect_kernel<U, int64_t><<<grid, kBlock, 0, st>>>((const U *)in, (const int64_t *)index, (U *)out, total, Lu, m, adim, fLu, fM, fast); \
     else                                                                                                               \
-        indexselect_kernel<U, int32_t><<<grid, kBlock, 0, st>>>((const U *)in, (const int32_t *)index, (U *)out, total, Lu, m, adim);
+        indexselect_kernel<U, int32_t><<<grid, kBlock, 0, st>>>((const U *)in, (const int32_t *)index, (U *)out, total, Lu, m, adim, fLu, fM, fast);
     switch (ub) {
     case 16: DXH_IS(uint4) break;
     case 8: DXH_IS(uint64_t) break;

@@ -111,6 +111,30 @@ inline int dtype_size(int dtype) {
     }
 }
 
+// ---- division by a run-time constant without a divide ----------------------------------------
+// q = n / d for any 32-bit n, d >= 1: one v_mul_hi_u32, a subtract, two shifts, an add (round-up
+// method with a 33-bit magic number).  Index decompositions in the changeshape kernels divide by
+// shape extents several times per 16-byte unit; a hardware-free divide costs ~25 instructions each.
+struct FastDiv { uint32_t d, magic, shift; };
+inline FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f{d, 0, 0};
+    if (d <= 1) return f;
+    uint32_t L = 0;
+    while ((1ull << L) < d) ++L;  // ceil(log2 d)
+    f.magic = (uint32_t)(((1ull << 32) * ((1ull << L) - d)) / d + 1);
+    f.shift = L - 1;
+    return f;
+}
+__host__ __device__ inline uint32_t fast_div(uint32_t n, const FastDiv &f) {
+    if (f.d <= 1) return n;
+#if defined(__HIP_DEVICE_COMPILE__)
+    uint32_t t = __umulhi(n, f.magic);
+#else
+    uint32_t t = (uint32_t)(((uint64_t)n * f.magic) >> 32);
+#endif
+    return (t + ((n - t) >> 1)) >> f.shift;
+}
+
 // ---- launch helpers --------------------------------------------------------------------
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 

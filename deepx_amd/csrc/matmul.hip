@@ -117,7 +117,7 @@ __global__ __launch_bounds__(kBlock) void matmul_mfma_kernel(const T *__restrict
 
 // ---- pipelined MFMA kernel ----------------------------------------------------------------
 // Workgroup tile 128x128, K step 64, 4 waves (2x2), each wave 64x64 = 2x2 MFMA 32x32x16 tiles and
-// 4 k-substeps per K step.  Requirements (checked by the launcher): K % 8 == 0, N % 8 == 0 and
+// 4 k-substeps per K step.  Requirements (checked by the launcher): K % 64 == 0, N % 8 == 0 and
 // 16-byte aligned A, B, C.
 //   LDS   two stages of {A tile [128 m][64 k], B tile transposed [128 n][64 k]}, rows of exactly
 //         128 bytes; the 16-byte chunk c of row r lives at chunk c ^ ((r ^ (r >> 3)) & 7), which
@@ -136,7 +136,7 @@ constexpr int kStageElems = PM * PK;  // elements per operand tile per stage
 __device__ inline int swz(int row, int chunk) { return chunk ^ ((row ^ (row >> 3)) & 7); }
 
 template <typename T>
-__global__ __launch_bounds__(kBlock) void matmul_mfma_pipe_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
+__global__ __launch_bounds__(kBlock, 2) void matmul_mfma_pipe_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
                                                                    int M, int K, int N, int tiles_m, int tiles_n) {
     // 2 stages x (A + B) x 16 KiB = 64 KiB; the epilogue reuses it as a [128][136] staging tile
     __shared__ __attribute__((aligned(16))) uint16_t lds[4 * kStageElems];
@@ -156,44 +156,57 @@ __global__ __launch_bounds__(kBlock) void matmul_mfma_pipe_kernel(const T *__res
     // A: 4 x 16 bytes: chunk index t + i*256 -> row (0..127), chunk (0..7)
     // B: 8 x 8 bytes:  n4 = t % 32 (4 columns), kg = t / 32 (8 k-rows)
     const int bn4 = t & 31, bkg = t >> 5;
-    uint4 ra[4];
-    uint2 rb[8];
+    // two K steps in flight in registers (prefetch distance 2): set 0 and set 1
+    // (scalars, not arrays: arrays of these ended up in scratch memory)
+    uint4 a0_0, a0_1, a0_2, a0_3, a1_0, a1_1, a1_2, a1_3;
+    uint2 b0_0, b0_1, b0_2, b0_3, b0_4, b0_5, b0_6, b0_7, b1_0, b1_1, b1_2, b1_3, b1_4, b1_5, b1_6, b1_7;
 
-    auto load_global = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int c = t + i * kBlock, row = c >> 3, ch = c & 7;
-            const int gm = m0 + row, gk = k0 + ch * 8;
-            ra[i] = (gm < M && gk < K) ? *reinterpret_cast<const uint4 *>(Ar + (int64_t)gm * K + gk) : uint4{0, 0, 0, 0};
-        }
-        const int gn = n0 + bn4 * 4;
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            const int gk = k0 + bkg * 8 + r;
-            rb[r] = (gk < K && gn < N) ? *reinterpret_cast<const uint2 *>(Br + (int64_t)gk * N + gn) : uint2{0, 0};
-        }
-    };
-    auto store_lds = [&](int stage) {
-        uint16_t *As = lds + stage * 2 * kStageElems, *Bs = As + kStageElems;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int c = t + i * kBlock, row = c >> 3, ch = c & 7;
-            *reinterpret_cast<uint4 *>(As + row * PK + swz(row, ch) * 8) = ra[i];
-        }
-        // 8x4 -> 4x8 transpose: column j of the 8 loaded rows becomes one 16-byte k-run
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            uint4 v;
-            uint32_t *vp = reinterpret_cast<uint32_t *>(&v);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const uint32_t lo = (j < 2) ? rb[2 * q].x : rb[2 * q].y, hi = (j < 2) ? rb[2 * q + 1].x : rb[2 * q + 1].y;
-                vp[q] = (j & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u) : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-            }
-            const int row = bn4 * 4 + j;
-            *reinterpret_cast<uint4 *>(Bs + row * PK + swz(row, bkg) * 8) = v;
-        }
-    };
+    // Branch-free loads: rows past M and columns past N are clamped onto valid memory (their
+    // products land in accumulator rows/columns the epilogue never stores) and K is a multiple of
+    // the K step, so the compiler sees straight-line code and can wait on exactly the older
+    // register set while the newer one is still in flight.
+    const int arow = t >> 3, ach = t & 7;
+    const uint16_t *ap0 = Ar + (int64_t)(m0 + arow < M ? m0 + arow : M - 1) * K + ach * 8;
+    const uint16_t *ap1 = Ar + (int64_t)(m0 + arow + 32 < M ? m0 + arow + 32 : M - 1) * K + ach * 8;
+    const uint16_t *ap2 = Ar + (int64_t)(m0 + arow + 64 < M ? m0 + arow + 64 : M - 1) * K + ach * 8;
+    const uint16_t *ap3 = Ar + (int64_t)(m0 + arow + 96 < M ? m0 + arow + 96 : M - 1) * K + ach * 8;
+    const int gn_b = (n0 + bn4 * 4 < N) ? n0 + bn4 * 4 : N - 4;
+    const uint16_t *b_ptr = Br + (int64_t)(bkg * 8) * N + gn_b;
+#define DXH_LOAD_GLOBAL(S, K0)                                                              \
+    do {                                                                                    \
+        const int k0_ = (K0);                                                               \
+        a##S##_0 = *reinterpret_cast<const uint4 *>(ap0 + k0_);                              \
+        a##S##_1 = *reinterpret_cast<const uint4 *>(ap1 + k0_);                              \
+        a##S##_2 = *reinterpret_cast<const uint4 *>(ap2 + k0_);                              \
+        a##S##_3 = *reinterpret_cast<const uint4 *>(ap3 + k0_);                              \
+        const uint16_t *bp_ = b_ptr + (int64_t)k0_ * N;                                     \
+        b##S##_0 = *reinterpret_cast<const uint2 *>(bp_);                                    \
+        b##S##_1 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)N);                       \
+        b##S##_2 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)2 * N);                   \
+        b##S##_3 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)3 * N);                   \
+        b##S##_4 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)4 * N);                   \
+        b##S##_5 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)5 * N);                   \
+        b##S##_6 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)6 * N);                   \
+        b##S##_7 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)7 * N);                   \
+    } while (0)
+    // A: 16-byte chunk (row, ach) -> swizzled chunk; B: 8x4 -> 4x8 register transpose, column j of
+    // the 8 loaded k-rows becomes one 16-byte k-run of LDS row bn4*4+j
+#define DXH_PLO(hi, lo) __builtin_amdgcn_perm((hi), (lo), 0x05040100u)
+#define DXH_PHI(hi, lo) __builtin_amdgcn_perm((hi), (lo), 0x07060302u)
+#define DXH_STORE_B(BS, ROW, V) *reinterpret_cast<uint4 *>((BS) + (ROW) * PK + swz((ROW), bkg) * 8) = (V)
+#define DXH_STORE_LDS(S, STAGE)                                                             \
+    do {                                                                                    \
+        uint16_t *As_ = lds + (STAGE) * 2 * kStageElems, *Bs_ = As_ + kStageElems;          \
+        *reinterpret_cast<uint4 *>(As_ + (arow) * PK + swz(arow, ach) * 8) = a##S##_0;       \
+        *reinterpret_cast<uint4 *>(As_ + (arow + 32) * PK + swz(arow + 32, ach) * 8) = a##S##_1; \
+        *reinterpret_cast<uint4 *>(As_ + (arow + 64) * PK + swz(arow + 64, ach) * 8) = a##S##_2; \
+        *reinterpret_cast<uint4 *>(As_ + (arow + 96) * PK + swz(arow + 96, ach) * 8) = a##S##_3; \
+        const int br_ = bn4 * 4;                                                            \
+        DXH_STORE_B(Bs_, br_ + 0, (uint4{DXH_PLO(b##S##_1.x, b##S##_0.x), DXH_PLO(b##S##_3.x, b##S##_2.x), DXH_PLO(b##S##_5.x, b##S##_4.x), DXH_PLO(b##S##_7.x, b##S##_6.x)})); \
+        DXH_STORE_B(Bs_, br_ + 1, (uint4{DXH_PHI(b##S##_1.x, b##S##_0.x), DXH_PHI(b##S##_3.x, b##S##_2.x), DXH_PHI(b##S##_5.x, b##S##_4.x), DXH_PHI(b##S##_7.x, b##S##_6.x)})); \
+        DXH_STORE_B(Bs_, br_ + 2, (uint4{DXH_PLO(b##S##_1.y, b##S##_0.y), DXH_PLO(b##S##_3.y, b##S##_2.y), DXH_PLO(b##S##_5.y, b##S##_4.y), DXH_PLO(b##S##_7.y, b##S##_6.y)})); \
+        DXH_STORE_B(Bs_, br_ + 3, (uint4{DXH_PHI(b##S##_1.y, b##S##_0.y), DXH_PHI(b##S##_3.y, b##S##_2.y), DXH_PHI(b##S##_5.y, b##S##_4.y), DXH_PHI(b##S##_7.y, b##S##_6.y)})); \
+    } while (0)
 
     f32x16 acc[2][2];
 #pragma unroll
@@ -203,13 +216,7 @@ __global__ __launch_bounds__(kBlock) void matmul_mfma_pipe_kernel(const T *__res
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    const int KT = (K + PK - 1) / PK;
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-        const int stage = kt & 1;
-        if (kt + 1 < KT) load_global((kt + 1) * PK);
+    auto compute = [&](int stage) {
         const uint16_t *As = lds + stage * 2 * kStageElems, *Bs = As + kStageElems;
 #pragma unroll
         for (int ks = 0; ks < PK / 16; ++ks) {
@@ -230,9 +237,38 @@ __global__ __launch_bounds__(kBlock) void matmul_mfma_pipe_kernel(const T *__res
 #pragma unroll
                 for (int j = 0; j < 2; ++j) acc[i][j] = mfma32<T>(af[i], bf[j], acc[i][j]);
         }
-        if (kt + 1 < KT) store_lds(stage ^ 1);
+    };
+
+    // Pipeline: LDS stage (kt & 1) holds K step kt; registers hold steps kt+1 and kt+2.  The loads
+    // for step kt+3 are issued right after step kt+1 moved from registers to LDS, so every global
+    // load has two full K steps of MFMA work (of two co-resident workgroups) to complete.
+    // Loads past the last K step are clamped onto the last step (valid memory, never stored to
+    // LDS), which keeps the loop body free of branches around memory instructions.
+    const int KT = K / PK;
+    auto k_of = [&](int step) { return (step < KT ? step : KT - 1) * PK; };
+    DXH_LOAD_GLOBAL(0, k_of(0));
+    DXH_LOAD_GLOBAL(1, k_of(1));
+    DXH_STORE_LDS(0, 0);
+    DXH_LOAD_GLOBAL(0, k_of(2));
+    __syncthreads();
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+        compute(0);                               // step kt
+        DXH_STORE_LDS(1, 1);                      // step kt+1
+        DXH_LOAD_GLOBAL(1, k_of(kt + 3));
+        __syncthreads();
+        compute(1);                               // step kt+1
+        DXH_STORE_LDS(0, 0);                      // step kt+2 (a clamped duplicate when kt+2 == KT: unused)
+        DXH_LOAD_GLOBAL(0, k_of(kt + 4));
         __syncthreads();
     }
+    if (kt < KT) compute(0);              // odd number of K steps
+    __syncthreads();
+#undef DXH_LOAD_GLOBAL
+#undef DXH_STORE_LDS
+#undef DXH_STORE_B
+#undef DXH_PLO
+#undef DXH_PHI
 
     // ---- epilogue: stage the 128x128 result tile in LDS, then 16-byte row stores
     constexpr int LDC = PN + 8;  // 272-byte rows
@@ -326,7 +362,7 @@ __global__ __launch_bounds__(kBlock) void matmul_tiled_kernel(const T *__restric
 
 template <typename T>
 int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    if (k % 8 == 0 && n % 8 == 0 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes) && m >= 64 && n >= 64) {
+    if (k % PK == 0 && n % 8 == 0 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes) && m >= 64 && n >= 64) {
         const int64_t ptm = (m + PM - 1) / PM, ptn = (n + PN - 1) / PN;
         const int64_t pblocks = batch * ptm * ptn;
         if (pblocks > 0x7fffffff) return DXH_ERR_SHAPE;

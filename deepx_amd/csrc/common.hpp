@@ -92,6 +92,7 @@ struct Tuning {
     int64_t reduce_col_target_blocks = 16 * 256;  // strided-axis stages like more, smaller workgroups
     int64_t reduce_col_min_rows = 16;             // DXH_TUNE_REDUCE_COL_MIN_ROWS
     int64_t reduce_col_max_lanes = 128;           // DXH_TUNE_REDUCE_COL_MAX_LANES
+    int64_t matmul_tile = 0;                      // DXH_TUNE_MATMUL_TILE: 0 = chosen per shape
 };
 Tuning &tuning();  // runtime.hip
 inline bool use_nt_store(size_t out_bytes) { return (int64_t)out_bytes > tuning().nt_store_bytes; }

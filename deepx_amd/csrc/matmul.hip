@@ -4,10 +4,9 @@
 // and cblas_sgemm of executor/op-ompsimd/src/deepx/tensorfunc/matmul_cblas.hpp:11-60 (alpha=1, beta=0).
 //
 //   bf16 / f16   MFMA v_mfma_f32_32x32x16_{bf16,f16}, fp32 accumulate, one RNE rounding of C.
-//                Workgroup tile 128x128x32, four waves in a 2x2 grid, each wave a 64x64 patch
-//                = 2x2 MFMA tiles.  A is staged in LDS k-contiguous; B arrives n-contiguous
-//                (row-major [K,N]) and is transposed on the way into LDS so that both MFMA
-//                operands are read as one 16-byte ds_read per lane.
+//                Aligned shapes (K % 64 == 0, N % 8 == 0): matmul_mfma_tile_kernel, 128x128 or
+//                256x256 workgroup tiles, software-pipelined over K.  Anything else:
+//                matmul_mfma_kernel, a plain 128x128x32 tile with element-wise edge handling.
 //   f32 / f64 / integers   LDS-tiled 64x64x16 FMA kernel, 4x4 outputs per lane; accumulate in
 //                the storage type (integers wrap).
 #include "common.hpp"
@@ -21,7 +20,10 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 constexpr int BM = 128, BN = 128, BK = 32;
 constexpr int LDK = BK + 8;  // padded k-stride (elements) of both LDS tiles: 80 bytes, keeps 16-byte alignment
 
-template <typename T> __device__ inline f32x16 mfma32(uint4 a, uint4 b, f32x16 c) {
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // native vector: arrays of it stay in registers
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename T, typename V> __device__ inline f32x16 mfma32(V a, V b, f32x16 c) {
     if constexpr (std::is_same_v<T, bf16_t>)
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     else
@@ -115,179 +117,224 @@ __global__ __launch_bounds__(kBlock) void matmul_mfma_kernel(const T *__restrict
             }
 }
 
-// ---- pipelined MFMA kernel ----------------------------------------------------------------
-// Workgroup tile 128x128, K step 64, 4 waves (2x2), each wave 64x64 = 2x2 MFMA 32x32x16 tiles and
-// 4 k-substeps per K step.  Requirements (checked by the launcher): K % 64 == 0, N % 8 == 0 and
-// 16-byte aligned A, B, C.
-//   LDS   two stages of {A tile [128 m][64 k], B tile transposed [128 n][64 k]}, rows of exactly
-//         128 bytes; the 16-byte chunk c of row r lives at chunk c ^ ((r ^ (r >> 3)) & 7), which
-//         makes the MFMA operand reads (32 consecutive rows, one chunk), the A stores (one row,
-//         8 chunks) and the B stores (rows 4 apart) all bank-conflict free.
-//   A     16-byte global loads straight into ds_write_b128.
-//   B     arrives n-contiguous: a lane loads 8 k-rows x 4 n (8 bytes each, 256 B contiguous per
-//         wave row), transposes 8x4 -> 4x8 in registers with v_perm_b32 and stores four 16-byte
-//         k-runs.
-//   pipe  the global loads of K step t+1 are issued before the MFMAs of step t and land in the
-//         other LDS stage afterwards: one barrier per K step.
-//   C     fp32 accumulators -> RNE to bf16/f16 -> staged through LDS -> 16-byte row stores.
-constexpr int PM = 128, PN = 128, PK = 64;
-constexpr int kStageElems = PM * PK;  // elements per operand tile per stage
-
+constexpr int PK = 64;  // K step of the MFMA tile kernel
 __device__ inline int swz(int row, int chunk) { return chunk ^ ((row ^ (row >> 3)) & 7); }
 
-template <typename T>
-__global__ __launch_bounds__(kBlock, 2) void matmul_mfma_pipe_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
-                                                                   int M, int K, int N, int tiles_m, int tiles_n) {
-    // 2 stages x (A + B) x 16 KiB = 64 KiB; the epilogue reuses it as a [128][136] staging tile
-    __shared__ __attribute__((aligned(16))) uint16_t lds[4 * kStageElems];
-    int64_t bid = blockIdx.x;
-    const int tn = (int)(bid % tiles_n); bid /= tiles_n;
-    const int tm = (int)(bid % tiles_m); bid /= tiles_m;
-    A += bid * (int64_t)M * K;
-    B += bid * (int64_t)K * N;
-    C += bid * (int64_t)M * N;
-    const int m0 = tm * PM, n0 = tn * PN;
-    const int t = threadIdx.x, lane = t & 63, w = t >> 6;
-    const int wm = w >> 1, wn = w & 1;
-    const uint16_t *Ar = reinterpret_cast<const uint16_t *>(A);
-    const uint16_t *Br = reinterpret_cast<const uint16_t *>(B);
+// ---- MFMA kernel with the B transposition done by the LDS read ------------------------------
+// Workgroup tile TM x TN (128 or 256 each), K step 64, 4 waves in a 2x2 grid, each wave a
+// (TM/2) x (TN/2) patch of 32x32x16 MFMAs.  Requirements (checked by the launcher): K % 64 == 0,
+// N % 8 == 0, 16-byte aligned A, B, C.
+//   loads  every global load is 16 bytes per lane (a wave instruction occupies the vector cache for
+//          the same 16 cycles whatever its width, so 8-byte loads halve its throughput).
+//   A      [TM m][64 k] in LDS, 128-byte rows, 16-byte chunk c of row r at chunk c ^ swizzle(r).
+//   B      stays n-contiguous in LDS, [64 k][TN n] with rows padded by 64 bytes; the MFMA operand
+//          (8 consecutive k of one column per lane) is assembled by two ds_read_b64_tr_b16.
+//   pipe   PD K steps in flight in registers, two LDS stages, one barrier per K step; the stores
+//          into the next stage and the global loads are spread over the four k-substeps.
+//   roles  the MFMA runs on (B^T, A^T): a lane of the result then holds 4 consecutive n of one row
+//          m, which packs into 8-byte LDS stores for the epilogue.
+//   map    blockIdx -> tile is XCD-aware: workgroups are dealt round-robin to the 8 XCDs, so XCD x
+//          takes the contiguous tile range [x*chunk, (x+1)*chunk) of a grouped (group_m tile rows
+//          at a time) ordering and its private L2 sees a compact set of A and B panels.
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &f, std::integer_sequence<int, I...>) { (f(std::integral_constant<int, I>{}), ...); }
+template <int N, typename F> __device__ __forceinline__ void static_for(F f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
+template <int V> using ic = std::integral_constant<int, V>;
 
-    // per-lane global coordinates of its loads
-    // A: 4 x 16 bytes: chunk index t + i*256 -> row (0..127), chunk (0..7)
-    // B: 8 x 8 bytes:  n4 = t % 32 (4 columns), kg = t / 32 (8 k-rows)
-    const int bn4 = t & 31, bkg = t >> 5;
-    // two K steps in flight in registers (prefetch distance 2): set 0 and set 1
-    // (scalars, not arrays: arrays of these ended up in scratch memory)
-    uint4 a0_0, a0_1, a0_2, a0_3, a1_0, a1_1, a1_2, a1_3;
-    uint2 b0_0, b0_1, b0_2, b0_3, b0_4, b0_5, b0_6, b0_7, b1_0, b1_1, b1_2, b1_3, b1_4, b1_5, b1_6, b1_7;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+// two fp32 accumulators -> one dword of two bf16/f16, round to nearest even (v_cvt_pk_bf16_f32 /
+// v_cvt_pk_f16_f32); element a in the low half
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    if constexpr (std::is_same_v<T, bf16_t>) return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+    else return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, f16x2));
+}
+// Within each group of 16 lanes, lane i passes the address of 4 consecutive 16-bit elements
+// ("row i") and receives element i%4 of rows i/4, 4 + i/4, 8 + i/4, 12 + i/4.
+__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t *p) {
+    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p);
+    return __builtin_bit_cast(u32x2, v);
+}
 
-    // Branch-free loads: rows past M and columns past N are clamped onto valid memory (their
-    // products land in accumulator rows/columns the epilogue never stores) and K is a multiple of
-    // the K step, so the compiler sees straight-line code and can wait on exactly the older
-    // register set while the newer one is still in flight.
+template <typename T, int TM, int TN, int PD>
+__global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul_mfma_tile_kernel(
+    const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int K, int N, int tiles_m, int tiles_n,
+    int total_tiles, int chunk, int group_m) {
+    constexpr int FM = TM / 64, FN = TN / 64;      // 32x32 MFMA tiles per wave along m and n
+    constexpr int A_LD = TM / 32, B_LD = TN / 32;  // 16-byte global loads per lane per K step
+    constexpr int CB = TN / 8;                     // 16-byte chunks per B row
+    constexpr int KR = kBlock / CB;                // B rows covered by one load of the workgroup
+    constexpr int B_ROW = TN + 32;                 // elements per k-row of the B stage (64-byte pad)
+    constexpr int A_STAGE = TM * PK, STAGE = A_STAGE + PK * B_ROW;
+    constexpr int LDC = TN + 8;
+    constexpr int LDS_ELEMS = (2 * STAGE > TM * LDC) ? 2 * STAGE : TM * LDC;
+    __shared__ __attribute__((aligned(16))) uint16_t lds[LDS_ELEMS];
+
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    int logical = xcd * chunk + slot;
+    if (logical >= total_tiles) return;
+    const int per_batch = tiles_m * tiles_n;
+    const int batch = logical / per_batch;
+    logical -= batch * per_batch;
+    const int in_group = group_m * tiles_n;
+    const int first_m = (logical / in_group) * group_m;
+    const int size_m = (tiles_m - first_m < group_m) ? tiles_m - first_m : group_m;
+    const int within = logical % in_group;
+    const int tm = first_m + within % size_m, tn = within / size_m;
+    const int m0 = tm * TM, n0 = tn * TN;
+
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
+    const uint16_t *Ab = reinterpret_cast<const uint16_t *>(A) + ((int64_t)batch * M + m0) * K;
+    const uint16_t *Bb = reinterpret_cast<const uint16_t *>(B) + (int64_t)batch * K * N + n0;
+
+    // Branch-free loads: rows past M and columns past N are clamped onto valid memory; their
+    // products land in accumulator rows/columns that the epilogue never stores.
     const int arow = t >> 3, ach = t & 7;
-    const uint16_t *ap0 = Ar + (int64_t)(m0 + arow < M ? m0 + arow : M - 1) * K + ach * 8;
-    const uint16_t *ap1 = Ar + (int64_t)(m0 + arow + 32 < M ? m0 + arow + 32 : M - 1) * K + ach * 8;
-    const uint16_t *ap2 = Ar + (int64_t)(m0 + arow + 64 < M ? m0 + arow + 64 : M - 1) * K + ach * 8;
-    const uint16_t *ap3 = Ar + (int64_t)(m0 + arow + 96 < M ? m0 + arow + 96 : M - 1) * K + ach * 8;
-    const int gn_b = (n0 + bn4 * 4 < N) ? n0 + bn4 * 4 : N - 4;
-    const uint16_t *b_ptr = Br + (int64_t)(bkg * 8) * N + gn_b;
-#define DXH_LOAD_GLOBAL(S, K0)                                                              \
-    do {                                                                                    \
-        const int k0_ = (K0);                                                               \
-        a##S##_0 = *reinterpret_cast<const uint4 *>(ap0 + k0_);                              \
-        a##S##_1 = *reinterpret_cast<const uint4 *>(ap1 + k0_);                              \
-        a##S##_2 = *reinterpret_cast<const uint4 *>(ap2 + k0_);                              \
-        a##S##_3 = *reinterpret_cast<const uint4 *>(ap3 + k0_);                              \
-        const uint16_t *bp_ = b_ptr + (int64_t)k0_ * N;                                     \
-        b##S##_0 = *reinterpret_cast<const uint2 *>(bp_);                                    \
-        b##S##_1 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)N);                       \
-        b##S##_2 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)2 * N);                   \
-        b##S##_3 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)3 * N);                   \
-        b##S##_4 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)4 * N);                   \
-        b##S##_5 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)5 * N);                   \
-        b##S##_6 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)6 * N);                   \
-        b##S##_7 = *reinterpret_cast<const uint2 *>(bp_ + (int64_t)7 * N);                   \
-    } while (0)
-    // A: 16-byte chunk (row, ach) -> swizzled chunk; B: 8x4 -> 4x8 register transpose, column j of
-    // the 8 loaded k-rows becomes one 16-byte k-run of LDS row bn4*4+j
-#define DXH_PLO(hi, lo) __builtin_amdgcn_perm((hi), (lo), 0x05040100u)
-#define DXH_PHI(hi, lo) __builtin_amdgcn_perm((hi), (lo), 0x07060302u)
-#define DXH_STORE_B(BS, ROW, V) *reinterpret_cast<uint4 *>((BS) + (ROW) * PK + swz((ROW), bkg) * 8) = (V)
-#define DXH_STORE_LDS(S, STAGE)                                                             \
-    do {                                                                                    \
-        uint16_t *As_ = lds + (STAGE) * 2 * kStageElems, *Bs_ = As_ + kStageElems;          \
-        *reinterpret_cast<uint4 *>(As_ + (arow) * PK + swz(arow, ach) * 8) = a##S##_0;       \
-        *reinterpret_cast<uint4 *>(As_ + (arow + 32) * PK + swz(arow + 32, ach) * 8) = a##S##_1; \
-        *reinterpret_cast<uint4 *>(As_ + (arow + 64) * PK + swz(arow + 64, ach) * 8) = a##S##_2; \
-        *reinterpret_cast<uint4 *>(As_ + (arow + 96) * PK + swz(arow + 96, ach) * 8) = a##S##_3; \
-        const int br_ = bn4 * 4;                                                            \
-        DXH_STORE_B(Bs_, br_ + 0, (uint4{DXH_PLO(b##S##_1.x, b##S##_0.x), DXH_PLO(b##S##_3.x, b##S##_2.x), DXH_PLO(b##S##_5.x, b##S##_4.x), DXH_PLO(b##S##_7.x, b##S##_6.x)})); \
-        DXH_STORE_B(Bs_, br_ + 1, (uint4{DXH_PHI(b##S##_1.x, b##S##_0.x), DXH_PHI(b##S##_3.x, b##S##_2.x), DXH_PHI(b##S##_5.x, b##S##_4.x), DXH_PHI(b##S##_7.x, b##S##_6.x)})); \
-        DXH_STORE_B(Bs_, br_ + 2, (uint4{DXH_PLO(b##S##_1.y, b##S##_0.y), DXH_PLO(b##S##_3.y, b##S##_2.y), DXH_PLO(b##S##_5.y, b##S##_4.y), DXH_PLO(b##S##_7.y, b##S##_6.y)})); \
-        DXH_STORE_B(Bs_, br_ + 3, (uint4{DXH_PHI(b##S##_1.y, b##S##_0.y), DXH_PHI(b##S##_3.y, b##S##_2.y), DXH_PHI(b##S##_5.y, b##S##_4.y), DXH_PHI(b##S##_7.y, b##S##_6.y)})); \
-    } while (0)
+    int a_off[A_LD], a_lds[A_LD];
+    static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
+        const int r = arow + 32 * i;
+        a_off[i] = (m0 + r < M ? r : M - 1 - m0) * K + ach * 8;
+        a_lds[i] = r * PK + swz(r, ach) * 8;
+    });
+    const int brow = t / CB, bch = t % CB;
+    const int b_off = brow * N + (n0 + bch * 8 < N ? bch * 8 : N - 8 - n0);
+    const int b_lds = brow * B_ROW + bch * 8;
 
-    f32x16 acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-    auto compute = [&](int stage) {
-        const uint16_t *As = lds + stage * 2 * kStageElems, *Bs = As + kStageElems;
-#pragma unroll
-        for (int ks = 0; ks < PK / 16; ++ks) {
-            uint4 af[2], bf[2];
-            const int ch = ks * 2 + (lane >> 5);
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int row = wm * 64 + i * 32 + (lane & 31);
-                af[i] = *reinterpret_cast<const uint4 *>(As + row * PK + swz(row, ch) * 8);
-            }
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int row = wn * 64 + j * 32 + (lane & 31);
-                bf[j] = *reinterpret_cast<const uint4 *>(Bs + row * PK + swz(row, ch) * 8);
-            }
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = mfma32<T>(af[i], bf[j], acc[i][j]);
-        }
+    u32x4 ra[PD][A_LD], rb[PD][B_LD];
+    auto load_part = [&](auto set, auto part, int k0) __attribute__((always_inline)) {
+        static_for<A_LD / 4>([&](auto q) __attribute__((always_inline)) {
+            constexpr int i = decltype(part)::value * (A_LD / 4) + decltype(q)::value;
+            ra[set][i] = *reinterpret_cast<const u32x4 *>(Ab + a_off[i] + k0);
+        });
+        static_for<B_LD / 4>([&](auto q) __attribute__((always_inline)) {
+            constexpr int i = decltype(part)::value * (B_LD / 4) + decltype(q)::value;
+            rb[set][i] = *reinterpret_cast<const u32x4 *>(Bb + (int64_t)(k0 + i * KR) * N + b_off);
+        });
+    };
+    auto store_part = [&](auto set, auto part, auto stage) __attribute__((always_inline)) {
+        uint16_t *As = lds + decltype(stage)::value * STAGE, *Bs = As + A_STAGE;
+        static_for<A_LD / 4>([&](auto q) __attribute__((always_inline)) {
+            constexpr int i = decltype(part)::value * (A_LD / 4) + decltype(q)::value;
+            *reinterpret_cast<u32x4 *>(As + a_lds[i]) = ra[set][i];
+        });
+        static_for<B_LD / 4>([&](auto q) __attribute__((always_inline)) {
+            constexpr int i = decltype(part)::value * (B_LD / 4) + decltype(q)::value;
+            *reinterpret_cast<u32x4 *>(Bs + b_lds + i * KR * B_ROW) = rb[set][i];
+        });
     };
 
-    // Pipeline: LDS stage (kt & 1) holds K step kt; registers hold steps kt+1 and kt+2.  The loads
-    // for step kt+3 are issued right after step kt+1 moved from registers to LDS, so every global
-    // load has two full K steps of MFMA work (of two co-resident workgroups) to complete.
-    // Loads past the last K step are clamped onto the last step (valid memory, never stored to
-    // LDS), which keeps the loop body free of branches around memory instructions.
+    // fragment registers, double-buffered over the k-substeps
+    u32x4 fa[2][FM], fb[2][FN];
+    const int fa_row = wm * (TM / 2) + (lane & 31), fch = lane >> 5;
+    const int fb_off = (8 * fch + ((lane & 15) >> 2)) * B_ROW + wn * (TN / 2) + (lane & 16) + 4 * (lane & 3);
+    auto read_frags = [&](auto buf, auto stage, auto ks) __attribute__((always_inline)) {
+        const uint16_t *As = lds + decltype(stage)::value * STAGE, *Bs = As + A_STAGE;
+        static_for<FM>([&](auto i) __attribute__((always_inline)) {
+            const int row = fa_row + 32 * i, ch = decltype(ks)::value * 2 + fch;
+            fa[buf][i] = *reinterpret_cast<const u32x4 *>(As + row * PK + swz(row, ch) * 8);
+        });
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
+            const uint16_t *p = Bs + fb_off + decltype(ks)::value * 16 * B_ROW + 32 * j;
+            const u32x2 lo = lds_read_tr16(p), hi = lds_read_tr16(p + 4 * B_ROW);
+            fb[buf][j] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        });
+    };
+
+    f32x16 acc[FM][FN];
+    static_for<FM>([&](auto i) __attribute__((always_inline)) {
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        });
+    });
+    constexpr int NM = FM * FN;                                 // MFMAs per k-substep
+    constexpr int ND = FM + 2 * FN, NW = (A_LD + B_LD) / 4;     // LDS reads, LDS writes (= global loads) per substep
+    auto mma = [&](auto buf, auto lo, auto hi) __attribute__((always_inline)) {
+        static_for<decltype(hi)::value - decltype(lo)::value>([&](auto x) __attribute__((always_inline)) {
+            constexpr int idx = decltype(lo)::value + decltype(x)::value, i = idx / FN, j = idx % FN;
+            acc[i][j] = mfma32<T>(fb[buf][j], fa[buf][i], acc[i][j]);
+        });
+    };
+    // Issue order inside a scheduling region: after each of `mfmas` MFMAs an even share of the
+    // region's LDS reads, LDS writes and global loads, so that the matrix pipe always has the next
+    // MFMA queued while the memory instructions are issued underneath it.
+    auto interleave = [&](auto mfmas, auto reads, auto writes, auto loads) __attribute__((always_inline)) {
+        constexpr int nm = decltype(mfmas)::value, nr = decltype(reads)::value, nw = decltype(writes)::value, nl = decltype(loads)::value;
+        static_for<nm>([&](auto x) __attribute__((always_inline)) {
+            constexpr int m = decltype(x)::value;
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            constexpr int r = nr * (m + 1) / nm - nr * m / nm, wr = nw * (m + 1) / nm - nw * m / nm, l = nl * (m + 1) / nm - nl * m / nm;
+            if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+            if constexpr (wr > 0) __builtin_amdgcn_sched_group_barrier(0x200, wr, 0);
+            if constexpr (l > 0) __builtin_amdgcn_sched_group_barrier(0x020, l, 0);
+        });
+    };
+
+    // One K step: LDS stage S is multiplied; register set R (the next K step) moves into stage
+    // S^1 and is refilled with the K step PD further on.  Fragment buffer 0 holds substep 0 on
+    // entry.  The last substep straddles the barrier: half of its MFMAs are queued before it and
+    // the other half runs under the first fragment reads of stage S^1.
+    auto step = [&](auto S, auto R, int k_load) __attribute__((always_inline)) {
+        constexpr int s = decltype(S)::value;
+        static_for<4>([&](auto ks) __attribute__((always_inline)) {
+            constexpr int cur = decltype(ks)::value & 1;
+            if constexpr (decltype(ks)::value < 3) {
+                read_frags(ic<cur ^ 1>{}, S, ic<decltype(ks)::value + 1>{});
+                store_part(R, ks, ic<s ^ 1>{});
+                load_part(R, ks, k_load);
+                mma(ic<cur>{}, ic<0>{}, ic<NM>{});
+                interleave(ic<NM>{}, ic<ND>{}, ic<NW>{}, ic<NW>{});
+            } else {
+                store_part(R, ks, ic<s ^ 1>{});
+                load_part(R, ks, k_load);
+                mma(ic<cur>{}, ic<0>{}, ic<NM / 2>{});
+                interleave(ic<NM / 2>{}, ic<0>{}, ic<NW>{}, ic<NW>{});
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();
+                read_frags(ic<cur ^ 1>{}, ic<s ^ 1>{}, ic<0>{});
+                mma(ic<cur>{}, ic<NM / 2>{}, ic<NM>{});
+                interleave(ic<NM - NM / 2>{}, ic<ND>{}, ic<0>{}, ic<0>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+
     const int KT = K / PK;
-    auto k_of = [&](int step) { return (step < KT ? step : KT - 1) * PK; };
-    DXH_LOAD_GLOBAL(0, k_of(0));
-    DXH_LOAD_GLOBAL(1, k_of(1));
-    DXH_STORE_LDS(0, 0);
-    DXH_LOAD_GLOBAL(0, k_of(2));
+    auto k_of = [&](int stepno) __attribute__((always_inline)) { return (stepno < KT ? stepno : KT - 1) * PK; };
+    static_for<4>([&](auto part) __attribute__((always_inline)) { load_part(ic<0>{}, part, k_of(0)); });
+    static_for<4>([&](auto part) __attribute__((always_inline)) { store_part(ic<0>{}, part, ic<0>{}); });
+    static_for<PD>([&](auto d) __attribute__((always_inline)) { static_for<4>([&](auto part) __attribute__((always_inline)) { load_part(ic<(decltype(d)::value + 1) % PD>{}, part, k_of(decltype(d)::value + 1)); }); });
     __syncthreads();
+    read_frags(ic<0>{}, ic<0>{}, ic<0>{});
     int kt = 0;
     for (; kt + 1 < KT; kt += 2) {
-        compute(0);                               // step kt
-        DXH_STORE_LDS(1, 1);                      // step kt+1
-        DXH_LOAD_GLOBAL(1, k_of(kt + 3));
-        __syncthreads();
-        compute(1);                               // step kt+1
-        DXH_STORE_LDS(0, 0);                      // step kt+2 (a clamped duplicate when kt+2 == KT: unused)
-        DXH_LOAD_GLOBAL(0, k_of(kt + 4));
-        __syncthreads();
+        step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1 + PD));
+        step(ic<1>{}, ic<2 % PD>{}, k_of(kt + 2 + PD));
     }
-    if (kt < KT) compute(0);              // odd number of K steps
+    if (kt < KT) step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1 + PD));
     __syncthreads();
-#undef DXH_LOAD_GLOBAL
-#undef DXH_STORE_LDS
-#undef DXH_STORE_B
-#undef DXH_PLO
-#undef DXH_PHI
 
-    // ---- epilogue: stage the 128x128 result tile in LDS, then 16-byte row stores
-    constexpr int LDC = PN + 8;  // 272-byte rows
+    // ---- epilogue: result lane holds row m = lane%32 of its MFMA tile and, per group g of 4
+    // registers, columns 8g + 4*(lane/32) .. +3: one 8-byte LDS store each, then 16-byte row stores
     uint16_t *Cs = lds;
+    static_for<FM>([&](auto i) __attribute__((always_inline)) {
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = wm * 64 + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-                const int col = wn * 64 + j * 32 + (lane & 31);
-                Cs[row * LDC + col] = store_acc<T>(acc[i][j][v]).bits;
+            for (int g = 0; g < 4; ++g) {
+                const int row = wm * (TM / 2) + 32 * i + (lane & 31);
+                const int col = wn * (TN / 2) + 32 * j + 8 * g + 4 * (lane >> 5);
+                *reinterpret_cast<u32x2 *>(Cs + row * LDC + col) =
+                    u32x2{pack2<T>(acc[i][j][4 * g], acc[i][j][4 * g + 1]), pack2<T>(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3])};
             }
+        });
+    });
     __syncthreads();
-    uint16_t *Cr = reinterpret_cast<uint16_t *>(C);
+    uint16_t *Cr = reinterpret_cast<uint16_t *>(C) + (int64_t)batch * M * N;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int c = t + i * kBlock, row = c >> 4, ch = c & 15;
+    for (int i = 0; i < TM * CB / kBlock; ++i) {
+        const int c = t + i * kBlock, row = c / CB, ch = c % CB;
         const int gm = m0 + row, gn = n0 + ch * 8;
         if (gm < M && gn < N)  // N % 8 == 0: a chunk is either fully inside or fully outside
             st_nt(reinterpret_cast<uint4 *>(Cr + (int64_t)gm * N + gn), *reinterpret_cast<const uint4 *>(Cs + row * LDC + ch * 8));
@@ -360,14 +407,50 @@ __global__ __launch_bounds__(kBlock) void matmul_tiled_kernel(const T *__restric
         }
 }
 
+template <typename T, int TM, int TN, int PD>
+int launch_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    const int64_t tiles_m = (m + TM - 1) / TM, tiles_n = (n + TN - 1) / TN, total = batch * tiles_m * tiles_n;
+    if (total > 0x0fffffff) return DXH_ERR_SHAPE;
+    const int chunk = (int)((total + 7) / 8);  // tiles per XCD
+    // tile rows per group: the chunk of one XCD should cover a roughly square patch of C
+    int group_m = 1;
+    while ((int64_t)(group_m + 1) * (group_m + 1) * TM <= (int64_t)chunk * TN && group_m + 1 <= tiles_m) ++group_m;
+    matmul_mfma_tile_kernel<T, TM, TN, PD><<<(unsigned)(8 * chunk), kBlock, 0, st>>>(
+        (const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n, (int)total, chunk, group_m);
+    return launch_status();
+}
+
+inline int compute_units() {
+    static const int cus = [] {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) {
+            (void)hipGetLastError();
+            v = 256;
+        }
+        return v;
+    }();
+    return cus;
+}
+
 template <typename T>
 int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    if (k % PK == 0 && n % 8 == 0 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes) && m >= 64 && n >= 64) {
-        const int64_t ptm = (m + PM - 1) / PM, ptn = (n + PN - 1) / PN;
-        const int64_t pblocks = batch * ptm * ptn;
-        if (pblocks > 0x7fffffff) return DXH_ERR_SHAPE;
-        matmul_mfma_pipe_kernel<T><<<(unsigned)pblocks, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, (int)ptm, (int)ptn);
-        return launch_status();
+    const bool fast = k % PK == 0 && n % 8 == 0 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes) &&
+                      k <= (1 << 22) && n <= (1 << 24);
+    int64_t choice = tuning().matmul_tile;
+    if (fast && choice == 0) {
+        // 256x256 tiles halve the bytes every CU pulls through its vector cache per flop, but need
+        // about one tile per CU to pay off; below that the 128x128 tiles (two workgroups per CU)
+        // spread the work better.
+        const int64_t tiles256 = batch * ((m + 255) / 256) * ((n + 255) / 256);
+        choice = (tiles256 * 10 >= (int64_t)compute_units() * 9) ? 4 : 1;
+    }
+    if (fast) {
+        switch (choice) {
+        case 2: return launch_tile<T, 256, 128, 2>(a, b, c, batch, m, k, n, st);
+        case 3: return launch_tile<T, 128, 256, 2>(a, b, c, batch, m, k, n, st);
+        case 4: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, st);
+        default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, st);
+        }
     }
     const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     const int64_t blocks = batch * tiles_m * tiles_n;

@@ -88,7 +88,8 @@ enum dxh_tune_knob {
     DXH_TUNE_NT_STORE_BYTES = 0,       /* outputs above this many bytes use non-temporal stores */
     DXH_TUNE_REDUCE_TARGET_BLOCKS = 1, /* workgroups a reduction stage aims for before it stops splitting R */
     DXH_TUNE_REDUCE_COL_MIN_ROWS = 2,  /* strided-axis stage: fewest rows per lane when R is split */
-    DXH_TUNE_REDUCE_COL_MAX_LANES = 3  /* strided-axis stage: widest column-lane count (16..256) */
+    DXH_TUNE_REDUCE_COL_MAX_LANES = 3, /* strided-axis stage: widest column-lane count (16..256) */
+    DXH_TUNE_MATMUL_TILE = 4           /* bf16/f16 matmul workgroup tile: 0 per shape, 1 128x128, 2 256x128, 3 128x256, 4 256x256 */
 };
 DXH_API int dxh_tune(int knob, int64_t value);
 DXH_API int dxh_device_count(int *count);

@@ -79,3 +79,52 @@ def test_config5_gemm_shapes_bf16(dxh, orc):
         ref = Af @ Bf
         mag = np.abs(Af) @ np.abs(Bf)
         assert np.all(np.abs(got[rows] - ref) <= 1e-2 * mag)
+
+
+TILE_KNOB = 4  # DXH_TUNE_MATMUL_TILE
+
+
+@pytest.mark.parametrize("tile", [1, 2, 3, 4])
+@pytest.mark.parametrize("dtype", [dx.BF16, dx.F16])
+def test_matmul_tile_configs(dxh, dtype, tile):
+    """Every workgroup tile of the MFMA kernel (forced through the tuning knob) on aligned shapes
+    with ragged tile edges, more than one batch and M, N below one tile; float64 numpy is the
+    reference, bar rel 1e-2 of sum_k |a||b| as above."""
+    rng = np.random.default_rng(300 + tile + dtype)
+    dx.check(dxh.dxh_tune(TILE_KNOB, tile))
+    try:
+        for batch, m, k, n in [(2, 300, 128, 264), (1, 520, 192, 520), (3, 70, 64, 8), (1, 257, 64, 1032), (1, 1, 64, 16),
+                               (1, 1024, 448, 768)]:
+            A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
+            B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
+            dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, A.dtype)
+            dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+            got = H.to_float(dC.get(), dtype).astype(np.float64).reshape(batch, m, n)
+            Af = H.to_float(A, dtype).astype(np.float64).reshape(batch, m, k)
+            Bf = H.to_float(B, dtype).astype(np.float64).reshape(batch, k, n)
+            ref, mag = np.matmul(Af, Bf), np.matmul(np.abs(Af), np.abs(Bf))
+            assert np.all(np.abs(got - ref) <= 1e-2 * np.maximum(mag, 1e-30)), (tile, dtype, batch, m, k, n)
+    finally:
+        dx.check(dxh.dxh_tune(TILE_KNOB, 0))
+
+
+def test_matmul_tiles_exact_on_small_integers(dxh):
+    """Small integer operands are exact in bf16 and their dot products exact in fp32, whatever the
+    summation order: every tile must return the exact product rounded once (RNE) to bf16.  A wrong
+    fragment, k-permutation or edge clamp changes an integer and fails bit-exactly."""
+    rng = np.random.default_rng(77)
+    m, k, n = 384, 256, 520
+    Ai, Bi = rng.integers(-4, 5, (m, k)), rng.integers(-4, 5, (k, n))
+    A = H.to_storage(Ai.astype(np.float64).reshape(-1), dx.BF16)
+    B = H.to_storage(Bi.astype(np.float64).reshape(-1), dx.BF16)
+    want = (Ai @ Bi).astype(np.float64)  # |sum| <= 16*256 = 4096: exact in fp32
+    dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, np.uint16)
+    for tile in (0, 1, 2, 3, 4):
+        dx.check(dxh.dxh_tune(TILE_KNOB, tile))
+        try:
+            dx.check(dxh.dxh_matmul(dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+            got = H.to_float(dC.get(), dx.BF16).astype(np.float64).reshape(m, n)
+        finally:
+            dx.check(dxh.dxh_tune(TILE_KNOB, 0))
+        # one RNE rounding of the exact integer to bf16
+        assert np.array_equal(got, H.to_float(H.to_storage(want.reshape(-1), dx.BF16), dx.BF16).astype(np.float64).reshape(m, n)), tile

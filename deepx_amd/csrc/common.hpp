@@ -89,7 +89,8 @@ template <typename VT> __device__ inline void st_nt(VT *p, const VT &v) {
 struct Tuning {
     int64_t nt_store_bytes = 0;                    // DXH_TUNE_NT_STORE_BYTES: 0 = always non-temporal
     int64_t reduce_target_blocks = 4 * 256;       // DXH_TUNE_REDUCE_TARGET_BLOCKS
-    int64_t reduce_col_target_blocks = 16 * 256;  // strided-axis stages like more, smaller workgroups
+    int64_t reduce_col_target_blocks = 256;       // strided-axis stages: about one workgroup per CU, each
+                                                  // walking its rows with software-pipelined loads
     int64_t reduce_col_min_rows = 16;             // DXH_TUNE_REDUCE_COL_MIN_ROWS
     int64_t reduce_col_max_lanes = 128;           // DXH_TUNE_REDUCE_COL_MAX_LANES
     int64_t matmul_tile = 0;                      // DXH_TUNE_MATMUL_TILE: 0 = chosen per shape

@@ -175,16 +175,30 @@ __global__ __launch_bounds__(kBlock) void reduce_col_kernel(const Tin *__restric
         const int64_t r1 = (r0 + chunk < R) ? r0 + chunk : R;
         const VT *base = reinterpret_cast<const VT *>(in + p * R * post) + cv;
         int64_t r = r0 + ty;
-        for (; r + 7 * (int64_t)TY < r1; r += 8 * (int64_t)TY) {
+        // batches of 8 rows per lane, software-pipelined: the loads of the next batch are issued
+        // before the current one is folded, so 8..16 loads per lane stay in flight
+        if (r + 7 * (int64_t)TY < r1) {
             VT x[8];
 #pragma unroll
             for (int u = 0; u < 8; ++u) x[u] = ld_nt(&base[(r + u * (int64_t)TY) * postv]);
+            r += 8 * (int64_t)TY;
+            auto fold = [&](const VT(&b)[8]) __attribute__((always_inline)) {
 #pragma unroll
-            for (int k = 0; k < V; ++k) {
-                A t0 = rop<K, A>(rop<K, A>(rload<A>(x[0].v[k]), rload<A>(x[1].v[k])), rop<K, A>(rload<A>(x[2].v[k]), rload<A>(x[3].v[k])));
-                A t1 = rop<K, A>(rop<K, A>(rload<A>(x[4].v[k]), rload<A>(x[5].v[k])), rop<K, A>(rload<A>(x[6].v[k]), rload<A>(x[7].v[k])));
-                acc[k] = rop<K, A>(acc[k], rop<K, A>(t0, t1));
+                for (int k = 0; k < V; ++k) {
+                    A t0 = rop<K, A>(rop<K, A>(rload<A>(b[0].v[k]), rload<A>(b[1].v[k])), rop<K, A>(rload<A>(b[2].v[k]), rload<A>(b[3].v[k])));
+                    A t1 = rop<K, A>(rop<K, A>(rload<A>(b[4].v[k]), rload<A>(b[5].v[k])), rop<K, A>(rload<A>(b[6].v[k]), rload<A>(b[7].v[k])));
+                    acc[k] = rop<K, A>(acc[k], rop<K, A>(t0, t1));
+                }
+            };
+            for (; r + 7 * (int64_t)TY < r1; r += 8 * (int64_t)TY) {
+                VT y[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) y[u] = ld_nt(&base[(r + u * (int64_t)TY) * postv]);
+                fold(x);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) x[u] = y[u];
             }
+            fold(x);
         }
         for (; r < r1; r += TY) {
             VT x = ld_nt(&base[r * postv]);
@@ -240,14 +254,14 @@ struct Plan {
 
 inline int pow2_ceil(int64_t x) { int p = 1; while (p < x && p < (1 << 30)) p <<= 1; return p; }
 
-// Column-lane count of a col stage.  Splittable stages (large R) give every workgroup the widest
-// contiguous row segment (TX = 256 lanes x 16 bytes = 4 KiB, TY = 1: no cross-lane reduction, the
-// DRAM-friendliest pattern) and get their parallelism from splitting R.  Stages that may not split
-// (the second pass over partials) narrow TX instead until enough workgroups exist.
+// Column-lane count of a col stage: as wide as the tuning allows (long contiguous row segments),
+// narrowed while that leaves fewer workgroups than CUs.  A stage that may still split R stops at
+// 32 lanes (512-byte segments) and gets the rest of its parallelism from the split; the second
+// pass over partials cannot split and narrows down to 16.
 inline int col_lanes(int64_t pre, int64_t postv, bool may_split) {
     int tx = (int)std::min<int64_t>(tuning().reduce_col_max_lanes, pow2_ceil(postv));
-    if (may_split) return tx;
-    while (tx > 16 && pre * ((postv + tx - 1) / tx) < kCUs) tx >>= 1;
+    const int floor_tx = may_split ? 32 : 16;
+    while (tx > floor_tx && pre * ((postv + tx - 1) / tx) < kCUs) tx >>= 1;
     return tx;
 }
 

@@ -25,7 +25,7 @@ int dxh_tune(int knob, int64_t value) {
     case DXH_TUNE_REDUCE_TARGET_BLOCKS: if (value < 1) return DXH_ERR_ARG; t.reduce_target_blocks = value; t.reduce_col_target_blocks = value; return DXH_OK;
     case DXH_TUNE_REDUCE_COL_MIN_ROWS: if (value < 1) return DXH_ERR_ARG; t.reduce_col_min_rows = value; return DXH_OK;
     case DXH_TUNE_REDUCE_COL_MAX_LANES:
-        if (value != 16 && value != 32 && value != 64 && value != 128 && value != 256) return DXH_ERR_ARG;
+        if (value != 4 && value != 8 && value != 16 && value != 32 && value != 64 && value != 128 && value != 256) return DXH_ERR_ARG;
         t.reduce_col_max_lanes = value;
         return DXH_OK;
     case DXH_TUNE_MATMUL_TILE: if (value < 0 || value > 4) return DXH_ERR_ARG; t.matmul_tile = value; return DXH_OK;

@@ -341,6 +341,141 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
     }
 }
 
+// ---- fp32 MFMA kernel ------------------------------------------------------------------------
+// v_mfma_f32_32x32x2_f32 (fp32 operands, fp32 accumulate: 157 TFLOP/s peak, 64 cycles each).  A
+// fp32 GEMM on the matrix pipe is compute bound by a wide margin (8x fewer flops per operand
+// byte than bf16 at 1/16 of the rate), so this kernel is a plain double-buffered one: workgroup
+// tile (64 FM) x (64 FN), K step 16, 4 waves 2x2, each wave FM x FN MFMA tiles.
+//   A      LDS [m][16 k] with rows padded to 20 floats; a lane reads the 8 consecutive k of its
+//          row half with two ds_read_b128 (the k order inside a K step is a free permutation as
+//          long as both operands use it: MFMA j of lane half h multiplies k = 8h + j).
+//   B      LDS [16 k][n] as loaded, rows padded by 4 floats; one ds_read_b32 per lane and k.
+//   roles  MFMA on (B^T, A^T): a result lane holds 4 consecutive n of one row m -> 16-byte stores.
+//   VEC    K % 4 == 0, N % 4 == 0 and 16-byte aligned pointers: 16-byte loads and stores with
+//          clamped rows/columns; otherwise element-wise accesses with bounds checks.
+constexpr int FK = 16, FA_ROW = FK + 4;
+template <int FM, int FN, bool VEC>
+__global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float *__restrict__ A, const float *__restrict__ B,
+                                                                    float *__restrict__ C, int M, int K, int N, int tiles_m,
+                                                                    int tiles_n) {
+    constexpr int TM = 64 * FM, TN = 64 * FN, FB_ROW = TN + 4;
+    constexpr int STAGE = TM * FA_ROW + FK * FB_ROW;  // floats
+    constexpr int CB = TN / 4;                        // 16-byte chunks per B row
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    __shared__ __attribute__((aligned(16))) float lds[2 * STAGE];
+    int64_t bid = blockIdx.x;
+    const int tn = (int)(bid % tiles_n); bid /= tiles_n;
+    const int tm = (int)(bid % tiles_m); bid /= tiles_m;
+    A += bid * (int64_t)M * K;
+    B += bid * (int64_t)K * N;
+    C += bid * (int64_t)M * N;
+    const int m0 = tm * TM, n0 = tn * TN;
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
+
+    // per-lane load coordinates: A chunk (row = t/4 + 64 i, c = t%4), B chunk (krow = id / CB, c = id % CB)
+    f32x4 ra[FM], rb[FN];
+    auto load_global = [&](int k0) __attribute__((always_inline)) {
+        static_for<FM>([&](auto i) __attribute__((always_inline)) {
+            const int row = (t >> 2) + 64 * i, kk = k0 + (t & 3) * 4, gm = m0 + row;
+            if constexpr (VEC) {
+                const float *p = A + (int64_t)(gm < M ? gm : M - 1) * K + (kk < K ? kk : 0);
+                f32x4 v = *reinterpret_cast<const f32x4 *>(p);
+                ra[i] = (kk < K) ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+            } else {
+                f32x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = (gm < M && kk + e < K) ? A[(int64_t)gm * K + kk + e] : 0.f;
+                ra[i] = v;
+            }
+        });
+        static_for<FN>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i, krow = id / CB, gk = k0 + krow, gn = n0 + (id % CB) * 4;
+            if constexpr (VEC) {
+                const float *p = B + (int64_t)(gk < K ? gk : 0) * N + (gn < N ? gn : N - 4);
+                f32x4 v = *reinterpret_cast<const f32x4 *>(p);
+                rb[i] = (gk < K) ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+            } else {
+                f32x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = (gk < K && gn + e < N) ? B[(int64_t)gk * N + gn + e] : 0.f;
+                rb[i] = v;
+            }
+        });
+    };
+    auto store_lds = [&](int stage) __attribute__((always_inline)) {
+        float *As = lds + stage * STAGE, *Bs = As + TM * FA_ROW;
+        static_for<FM>([&](auto i) __attribute__((always_inline)) {
+            *reinterpret_cast<f32x4 *>(As + ((t >> 2) + 64 * i) * FA_ROW + (t & 3) * 4) = ra[i];
+        });
+        static_for<FN>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i;
+            *reinterpret_cast<f32x4 *>(Bs + (id / CB) * FB_ROW + (id % CB) * 4) = rb[i];
+        });
+    };
+
+    f32x16 acc[FM][FN];
+    static_for<FM>([&](auto i) __attribute__((always_inline)) {
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        });
+    });
+    const int h = lane >> 5, l32 = lane & 31;
+    auto compute = [&](int stage) __attribute__((always_inline)) {
+        const float *As = lds + stage * STAGE, *Bs = As + TM * FA_ROW;
+        f32x4 fa[FM][2];
+        float fb[FN][8];
+        static_for<FM>([&](auto i) __attribute__((always_inline)) {
+            const float *p = As + (wm * 32 * FM + 32 * i + l32) * FA_ROW + 8 * h;
+            fa[i][0] = *reinterpret_cast<const f32x4 *>(p);
+            fa[i][1] = *reinterpret_cast<const f32x4 *>(p + 4);
+        });
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) fb[j][e] = Bs[(8 * h + e) * FB_ROW + wn * 32 * FN + 32 * j + l32];
+        });
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            static_for<FM>([&](auto i) __attribute__((always_inline)) {
+                static_for<FN>([&](auto j) __attribute__((always_inline)) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][e], fa[i][e >> 2][e & 3], acc[i][j], 0, 0, 0);
+                });
+            });
+    };
+
+    const int KT = (K + FK - 1) / FK;
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const bool more = kt + 1 < KT;
+        if (more) load_global((kt + 1) * FK);
+        compute(kt & 1);
+        if (more) store_lds((kt + 1) & 1);
+        __syncthreads();
+    }
+
+    // result lane: row m = lane%32 of its MFMA tile; register group g holds columns 8g + 4h .. +3
+    static_for<FM>([&](auto i) __attribute__((always_inline)) {
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
+            const int gm = m0 + wm * 32 * FM + 32 * i + l32;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int gn = n0 + wn * 32 * FN + 32 * j + 8 * g + 4 * h;
+                if constexpr (VEC) {
+                    if (gm < M && gn < N)
+                        __builtin_nontemporal_store(f32x4{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]},
+                                                    reinterpret_cast<f32x4 *>(C + (int64_t)gm * N + gn));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (gm < M && gn + e < N) C[(int64_t)gm * N + gn + e] = acc[i][j][4 * g + e];
+                }
+            }
+        });
+    });
+}
+
 // ---- generic tiled kernel (f32, f64, integers) ------------------------------------------
 constexpr int GT = 64, GK = 16;
 template <typename T>
@@ -474,6 +609,32 @@ int launch_tiled(const void *a, const void *b, void *c, int64_t batch, int64_t m
     return launch_status();
 }
 
+template <int FM, int FN>
+int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, hipStream_t st) {
+    const int64_t tiles_m = (m + 64 * FM - 1) / (64 * FM), tiles_n = (n + 64 * FN - 1) / (64 * FN), blocks = batch * tiles_m * tiles_n;
+    if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
+    if (vec) matmul_mfma_f32_kernel<FM, FN, true><<<(unsigned)blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
+    else matmul_mfma_f32_kernel<FM, FN, false><<<(unsigned)blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
+    return launch_status();
+}
+
+// fp32: the matrix pipe is the bound, so the tile only has to balance the CUs: the largest of
+// 128x128 / 128x64 / 64x64 whose workgroup count wastes under ~10 % in the last round (two
+// workgroups per CU), else the smallest.
+inline int launch_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    const bool vec = k % 4 == 0 && n % 4 == 0 && n >= 4 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes);
+    const int64_t slots = 2 * (int64_t)compute_units();
+    auto waste = [&](int tm, int tn) {
+        const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn), rounds = (tiles + slots - 1) / slots;
+        return 1.0 - (double)tiles / (double)(rounds * slots);
+    };
+    const float *af = (const float *)a, *bf = (const float *)b;
+    float *cf = (float *)c;
+    if (m > 64 && n > 64 && waste(128, 128) < 0.10) return launch_f32_tile<2, 2>(af, bf, cf, batch, m, k, n, vec, st);
+    if (m > 64 && waste(128, 64) < 0.10) return launch_f32_tile<2, 1>(af, bf, cf, batch, m, k, n, vec, st);
+    return launch_f32_tile<1, 1>(af, bf, cf, batch, m, k, n, vec, st);
+}
+
 }  // namespace dxh
 
 using namespace dxh;
@@ -496,7 +657,7 @@ extern "C" int dxh_matmul(int dtype, const void *a, const void *b, void *c, int6
     switch (dtype) {
     case DXH_BF16: return launch_mfma<bf16_t>(a, b, c, batch, m, k, n, st);
     case DXH_F16: return launch_mfma<f16_t>(a, b, c, batch, m, k, n, st);
-    case DXH_F32: return launch_tiled<float>(a, b, c, batch, m, k, n, st);
+    case DXH_F32: return launch_f32(a, b, c, batch, m, k, n, st);
     case DXH_F64: return launch_tiled<double>(a, b, c, batch, m, k, n, st);
     case DXH_I64: return launch_tiled<int64_t>(a, b, c, batch, m, k, n, st);
     case DXH_I32: return launch_tiled<int32_t>(a, b, c, batch, m, k, n, st);

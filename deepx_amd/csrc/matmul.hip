@@ -7,8 +7,9 @@
 //                Aligned shapes (K % 64 == 0, N % 8 == 0): matmul_mfma_tile_kernel, 128x128 or
 //                256x256 workgroup tiles, software-pipelined over K.  Anything else:
 //                matmul_mfma_kernel, a plain 128x128x32 tile with element-wise edge handling.
-//   f32 / f64 / integers   LDS-tiled 64x64x16 FMA kernel, 4x4 outputs per lane; accumulate in
-//                the storage type (integers wrap).
+//   f32          MFMA v_mfma_f32_32x32x2_f32 (fp32 operands and accumulate): matmul_mfma_f32_kernel.
+//   f64 / integers   LDS-tiled 64x64x16 FMA kernel, 4x4 outputs per lane; accumulate in the
+//                storage type (integers wrap).
 #include "common.hpp"
 
 namespace dxh {
@@ -345,22 +346,24 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
 // v_mfma_f32_32x32x2_f32 (fp32 operands, fp32 accumulate: 157 TFLOP/s peak, 64 cycles each).  A
 // fp32 GEMM on the matrix pipe is compute bound by a wide margin (8x fewer flops per operand
 // byte than bf16 at 1/16 of the rate), so this kernel is a plain double-buffered one: workgroup
-// tile (64 FM) x (64 FN), K step 16, 4 waves 2x2, each wave FM x FN MFMA tiles.
-//   A      LDS [m][16 k] with rows padded to 20 floats; a lane reads the 8 consecutive k of its
-//          row half with two ds_read_b128 (the k order inside a K step is a free permutation as
-//          long as both operands use it: MFMA j of lane half h multiplies k = 8h + j).
-//   B      LDS [16 k][n] as loaded, rows padded by 4 floats; one ds_read_b32 per lane and k.
+// tile (64 FM) x (64 FN), K step FK, 4 waves 2x2, each wave FM x FN MFMA tiles, PD K steps held
+// in registers ahead of the LDS stage being multiplied.
+//   A      LDS [m][FK k] with rows padded by 4 floats; a lane reads the FK/2 consecutive k of its
+//          row half with ds_read_b128 (the k order inside a K step is a free permutation as
+//          long as both operands use it: MFMA e of lane half h multiplies k = (FK/2) h + e).
+//   B      LDS [FK k][n] as loaded, rows padded by 4 floats; one ds_read_b32 per lane and k.
 //   roles  MFMA on (B^T, A^T): a result lane holds 4 consecutive n of one row m -> 16-byte stores.
 //   VEC    K % 4 == 0, N % 4 == 0 and 16-byte aligned pointers: 16-byte loads and stores with
 //          clamped rows/columns; otherwise element-wise accesses with bounds checks.
-constexpr int FK = 16, FA_ROW = FK + 4;
-template <int FM, int FN, bool VEC>
+template <int FM, int FN, int FK, int PD, bool VEC>
 __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float *__restrict__ A, const float *__restrict__ B,
                                                                     float *__restrict__ C, int M, int K, int N, int tiles_m,
                                                                     int tiles_n) {
-    constexpr int TM = 64 * FM, TN = 64 * FN, FB_ROW = TN + 4;
+    constexpr int TM = 64 * FM, TN = 64 * FN, FA_ROW = FK + 4, FB_ROW = TN + 4;
     constexpr int STAGE = TM * FA_ROW + FK * FB_ROW;  // floats
-    constexpr int CB = TN / 4;                        // 16-byte chunks per B row
+    constexpr int CA = FK / 4, CB = TN / 4;           // 16-byte chunks per A row / B row
+    constexpr int A_LD = TM * CA / kBlock, B_LD = FK * CB / kBlock;
+    constexpr int HK = FK / 2;                        // k values per lane half
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     __shared__ __attribute__((aligned(16))) float lds[2 * STAGE];
     int64_t bid = blockIdx.x;
@@ -372,44 +375,45 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
     const int m0 = tm * TM, n0 = tn * TN;
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
 
-    // per-lane load coordinates: A chunk (row = t/4 + 64 i, c = t%4), B chunk (krow = id / CB, c = id % CB)
-    f32x4 ra[FM], rb[FN];
-    auto load_global = [&](int k0) __attribute__((always_inline)) {
-        static_for<FM>([&](auto i) __attribute__((always_inline)) {
-            const int row = (t >> 2) + 64 * i, kk = k0 + (t & 3) * 4, gm = m0 + row;
+    // per-lane chunks: A (row = id / CA, c = id % CA), B (krow = id / CB, c = id % CB), id = t + 256 i
+    f32x4 ra[PD][A_LD], rb[PD][B_LD];
+    auto load_global = [&](auto set, int k0) __attribute__((always_inline)) {
+        static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i, row = id / CA, kk = k0 + (id % CA) * 4, gm = m0 + row;
             if constexpr (VEC) {
                 const float *p = A + (int64_t)(gm < M ? gm : M - 1) * K + (kk < K ? kk : 0);
                 f32x4 v = *reinterpret_cast<const f32x4 *>(p);
-                ra[i] = (kk < K) ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+                ra[set][i] = (kk < K) ? v : f32x4{0.f, 0.f, 0.f, 0.f};
             } else {
                 f32x4 v;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = (gm < M && kk + e < K) ? A[(int64_t)gm * K + kk + e] : 0.f;
-                ra[i] = v;
+                ra[set][i] = v;
             }
         });
-        static_for<FN>([&](auto i) __attribute__((always_inline)) {
+        static_for<B_LD>([&](auto i) __attribute__((always_inline)) {
             const int id = t + kBlock * i, krow = id / CB, gk = k0 + krow, gn = n0 + (id % CB) * 4;
             if constexpr (VEC) {
                 const float *p = B + (int64_t)(gk < K ? gk : 0) * N + (gn < N ? gn : N - 4);
                 f32x4 v = *reinterpret_cast<const f32x4 *>(p);
-                rb[i] = (gk < K) ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+                rb[set][i] = (gk < K) ? v : f32x4{0.f, 0.f, 0.f, 0.f};
             } else {
                 f32x4 v;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = (gk < K && gn + e < N) ? B[(int64_t)gk * N + gn + e] : 0.f;
-                rb[i] = v;
+                rb[set][i] = v;
             }
         });
     };
-    auto store_lds = [&](int stage) __attribute__((always_inline)) {
-        float *As = lds + stage * STAGE, *Bs = As + TM * FA_ROW;
-        static_for<FM>([&](auto i) __attribute__((always_inline)) {
-            *reinterpret_cast<f32x4 *>(As + ((t >> 2) + 64 * i) * FA_ROW + (t & 3) * 4) = ra[i];
-        });
-        static_for<FN>([&](auto i) __attribute__((always_inline)) {
+    auto store_lds = [&](auto set, auto stage) __attribute__((always_inline)) {
+        float *As = lds + decltype(stage)::value * STAGE, *Bs = As + TM * FA_ROW;
+        static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
             const int id = t + kBlock * i;
-            *reinterpret_cast<f32x4 *>(Bs + (id / CB) * FB_ROW + (id % CB) * 4) = rb[i];
+            *reinterpret_cast<f32x4 *>(As + (id / CA) * FA_ROW + (id % CA) * 4) = ra[set][i];
+        });
+        static_for<B_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i;
+            *reinterpret_cast<f32x4 *>(Bs + (id / CB) * FB_ROW + (id % CB) * 4) = rb[set][i];
         });
     };
 
@@ -421,39 +425,52 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
         });
     });
     const int h = lane >> 5, l32 = lane & 31;
-    auto compute = [&](int stage) __attribute__((always_inline)) {
-        const float *As = lds + stage * STAGE, *Bs = As + TM * FA_ROW;
-        f32x4 fa[FM][2];
-        float fb[FN][8];
-        static_for<FM>([&](auto i) __attribute__((always_inline)) {
-            const float *p = As + (wm * 32 * FM + 32 * i + l32) * FA_ROW + 8 * h;
-            fa[i][0] = *reinterpret_cast<const f32x4 *>(p);
-            fa[i][1] = *reinterpret_cast<const f32x4 *>(p + 4);
-        });
-        static_for<FN>([&](auto j) __attribute__((always_inline)) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) fb[j][e] = Bs[(8 * h + e) * FB_ROW + wn * 32 * FN + 32 * j + l32];
-        });
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
+    // MFMA e of lane half h multiplies k = HK*h + e of the K step (both operands use this order)
+    auto compute = [&](auto stage) __attribute__((always_inline)) {
+        const float *As = lds + decltype(stage)::value * STAGE, *Bs = As + TM * FA_ROW;
+        static_for<HK / 8>([&](auto q) __attribute__((always_inline)) {  // 8 k per lane half at a time
+            f32x4 fa[FM][2];
+            float fb[FN][8];
             static_for<FM>([&](auto i) __attribute__((always_inline)) {
-                static_for<FN>([&](auto j) __attribute__((always_inline)) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][e], fa[i][e >> 2][e & 3], acc[i][j], 0, 0, 0);
-                });
+                const float *p = As + (wm * 32 * FM + 32 * i + l32) * FA_ROW + HK * h + 8 * decltype(q)::value;
+                fa[i][0] = *reinterpret_cast<const f32x4 *>(p);
+                fa[i][1] = *reinterpret_cast<const f32x4 *>(p + 4);
             });
+            static_for<FN>([&](auto j) __attribute__((always_inline)) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) fb[j][e] = Bs[(HK * h + 8 * decltype(q)::value + e) * FB_ROW + wn * 32 * FN + 32 * j + l32];
+            });
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                static_for<FM>([&](auto i) __attribute__((always_inline)) {
+                    static_for<FN>([&](auto j) __attribute__((always_inline)) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][e], fa[i][e >> 2][e & 3], acc[i][j], 0, 0, 0);
+                    });
+                });
+        });
     };
 
+    // LDS stage (kt & 1) holds K step kt, register set (kt + 1) % PD holds step kt + 1 and is
+    // refilled with step kt + 1 + PD once it has moved to LDS.  Steps past the end are clamped
+    // onto the last one (loaded, never multiplied).
     const int KT = (K + FK - 1) / FK;
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-        const bool more = kt + 1 < KT;
-        if (more) load_global((kt + 1) * FK);
-        compute(kt & 1);
-        if (more) store_lds((kt + 1) & 1);
+    auto k_of = [&](int stepno) { return (stepno < KT ? stepno : KT - 1) * FK; };
+    auto step = [&](auto S, auto R, int k_load) __attribute__((always_inline)) {
+        compute(S);
+        store_lds(R, ic<decltype(S)::value ^ 1>{});
+        load_global(R, k_load);
         __syncthreads();
+    };
+    load_global(ic<0>{}, 0);
+    store_lds(ic<0>{}, ic<0>{});
+    static_for<PD>([&](auto d) __attribute__((always_inline)) { load_global(ic<(decltype(d)::value + 1) % PD>{}, k_of(decltype(d)::value + 1)); });
+    __syncthreads();
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+        step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1 + PD));
+        step(ic<1>{}, ic<2 % PD>{}, k_of(kt + 2 + PD));
     }
+    if (kt < KT) compute(ic<0>{});
 
     // result lane: row m = lane%32 of its MFMA tile; register group g holds columns 8g + 4h .. +3
     static_for<FM>([&](auto i) __attribute__((always_inline)) {
@@ -609,30 +626,43 @@ int launch_tiled(const void *a, const void *b, void *c, int64_t batch, int64_t m
     return launch_status();
 }
 
-template <int FM, int FN>
+template <int FM, int FN, int FK, int PD>
 int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, hipStream_t st) {
     const int64_t tiles_m = (m + 64 * FM - 1) / (64 * FM), tiles_n = (n + 64 * FN - 1) / (64 * FN), blocks = batch * tiles_m * tiles_n;
     if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
-    if (vec) matmul_mfma_f32_kernel<FM, FN, true><<<(unsigned)blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
-    else matmul_mfma_f32_kernel<FM, FN, false><<<(unsigned)blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
+    if (vec) matmul_mfma_f32_kernel<FM, FN, FK, PD, true><<<(unsigned)blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
+    else matmul_mfma_f32_kernel<FM, FN, FK, PD, false><<<(unsigned)blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
     return launch_status();
 }
 
-// fp32: the matrix pipe is the bound, so the tile only has to balance the CUs: the largest of
-// 128x128 / 128x64 / 64x64 whose workgroup count wastes under ~10 % in the last round (two
-// workgroups per CU), else the smallest.
+// fp32: the matrix pipe is the bound, so the tile is chosen for CU balance.  Cost model per tile
+// shape: two workgroups share a CU; a CU's time is (rounds of two tiles) x tile flops / efficiency,
+// where a last round that leaves at most one workgroup per CU counts 0.6 (a lone workgroup runs
+// faster than two that share the pipe) and the efficiencies are the measured large-square rates
+// relative to the 128x128 tile.  Small tiles take longer K steps and a deeper prefetch: with few
+// MFMAs per step only that hides the global-load latency.
 inline int launch_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     const bool vec = k % 4 == 0 && n % 4 == 0 && n >= 4 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes);
-    const int64_t slots = 2 * (int64_t)compute_units();
-    auto waste = [&](int tm, int tn) {
-        const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn), rounds = (tiles + slots - 1) / slots;
-        return 1.0 - (double)tiles / (double)(rounds * slots);
+    const int64_t cus = compute_units();
+    auto cost = [&](int tm, int tn, double eff) {
+        const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn);
+        const int64_t full = tiles / (2 * cus), rem = tiles % (2 * cus);
+        const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.6 : 0.0);
+        return rounds * (double)tm * (double)tn / eff;
     };
     const float *af = (const float *)a, *bf = (const float *)b;
     float *cf = (float *)c;
-    if (m > 64 && n > 64 && waste(128, 128) < 0.10) return launch_f32_tile<2, 2>(af, bf, cf, batch, m, k, n, vec, st);
-    if (m > 64 && waste(128, 64) < 0.10) return launch_f32_tile<2, 1>(af, bf, cf, batch, m, k, n, vec, st);
-    return launch_f32_tile<1, 1>(af, bf, cf, batch, m, k, n, vec, st);
+    int64_t choice = tuning().matmul_tile;
+    if (choice == 0) {
+        const double c1 = cost(128, 128, 1.0), c2 = cost(128, 64, 0.95), c3 = cost(64, 64, 0.86);
+        choice = (c1 <= c2 && c1 <= c3) ? 1 : (c2 <= c3) ? 2 : 3;
+    }
+    switch (choice) {
+    case 1: return launch_f32_tile<2, 2, 32, 1>(af, bf, cf, batch, m, k, n, vec, st);
+    case 2: return launch_f32_tile<2, 1, 32, 2>(af, bf, cf, batch, m, k, n, vec, st);
+    case 4: return launch_f32_tile<2, 2, 16, 1>(af, bf, cf, batch, m, k, n, vec, st);
+    default: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, st);
+    }
 }
 
 }  // namespace dxh

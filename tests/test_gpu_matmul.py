@@ -128,3 +128,31 @@ def test_matmul_tiles_exact_on_small_integers(dxh):
             dx.check(dxh.dxh_tune(TILE_KNOB, 0))
         # one RNE rounding of the exact integer to bf16
         assert np.array_equal(got, H.to_float(H.to_storage(want.reshape(-1), dx.BF16), dx.BF16).astype(np.float64).reshape(m, n)), tile
+
+
+@pytest.mark.parametrize("tile", [1, 2, 3, 4])
+def test_matmul_f32_tile_configs(dxh, tile):
+    """Every tile of the fp32 matrix-pipe kernel, on 16-byte-friendly shapes (vector path) and on
+    odd K / N / unaligned bases (element-wise path), ragged edges, batches and a K that is not a
+    multiple of the K step.  Bar: rel 1e-5*sqrt(K) of sum_k |a||b| against float64 numpy."""
+    rng = np.random.default_rng(500 + tile)
+    dx.check(dxh.dxh_tune(TILE_KNOB, tile))
+    try:
+        for batch, m, k, n in [(2, 300, 128, 264), (1, 130, 100, 68), (3, 70, 33, 9), (1, 257, 64, 1030), (1, 1, 4, 4),
+                               (1, 520, 1000, 260), (2, 65, 7, 129)]:
+            A = rng.standard_normal(batch * m * k).astype(np.float32)
+            B = rng.standard_normal(batch * k * n).astype(np.float32)
+            dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, np.float32)
+            dx.check(dxh.dxh_matmul(dx.F32, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+            got = dC.get().astype(np.float64).reshape(batch, m, n)
+            Af, Bf = A.astype(np.float64).reshape(batch, m, k), B.astype(np.float64).reshape(batch, k, n)
+            ref, mag = np.matmul(Af, Bf), np.matmul(np.abs(Af), np.abs(Bf))
+            assert np.all(np.abs(got - ref) <= 1e-5 * np.sqrt(k) * np.maximum(mag, 1e-30)), (tile, batch, m, k, n)
+        # exact on small integers whatever the summation order
+        m, k, n = 200, 96, 132
+        Ai, Bi = rng.integers(-8, 9, (m, k)), rng.integers(-8, 9, (k, n))
+        dA, dB, dC = Dev(Ai.astype(np.float32).reshape(-1)), Dev(Bi.astype(np.float32).reshape(-1)), Dev.empty(m * n, np.float32)
+        dx.check(dxh.dxh_matmul(dx.F32, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+        assert np.array_equal(dC.get().reshape(m, n), (Ai @ Bi).astype(np.float32))
+    finally:
+        dx.check(dxh.dxh_tune(TILE_KNOB, 0))

@@ -27,6 +27,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+MFMA_F32_PEAK_TF = 157.3
 MFMA_BF16_PEAK_TF = 2500.0  # dense bf16
 REDUCE_ROW_TRAFFIC_BYTES = 268646159  # measured, see profiles/bench_pmc_hbm_traffic.md
 
@@ -196,12 +197,12 @@ def time_op(L, dx, torch, Events, ev, launch, reps=20, warm=3):
 def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
     res = {}
 
-    def entry(ms, nbytes=None, flops=None):
+    def entry(ms, nbytes=None, flops=None, peak_tf=MFMA_BF16_PEAK_TF, peak_name="frac_mfma_bf16"):
         e = {"ms": round(ms, 5)}
         if nbytes is not None:
             e.update({"GB/s": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes})
         if flops is not None:
-            e.update({"TFLOP/s": round(flops / ms / 1e9, 2), "frac_mfma_bf16": round(flops / ms / 1e9 / MFMA_BF16_PEAK_TF, 4), "flops": flops})
+            e.update({"TFLOP/s": round(flops / ms / 1e9, 2), peak_name: round(flops / ms / 1e9 / peak_tf, 4), "flops": flops})
         return e
 
     # ---- config 1: fp32 [4096,4096] elementwise chain; 4 rotating buffer sets (64 MiB tensors)
@@ -279,6 +280,13 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
         Bm = (torch.randn(kk * nn, device=dev) * 0.02).to(torch.bfloat16)
         Cm = torch.empty(mm * nn, device=dev, dtype=torch.bfloat16)
         c5[label] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_matmul(dx.BF16, ptr(Am), ptr(Bm), ptr(Cm), 1, mm, kk, nn, None)), flops=2 * mm * kk * nn)
+    # the same shapes in fp32, the dtype the reference's own matmul (cublasSgemm / cblas_sgemm) runs in
+    for label, (mm, kk, nn) in [("matmul_f32_2048x896x4864", (2048, 896, 4864)), ("matmul_f32_2048x4864x896", (2048, 4864, 896))]:
+        Am = torch.randn(mm * kk, device=dev)
+        Bm = torch.randn(kk * nn, device=dev) * 0.02
+        Cm = torch.empty(mm * nn, device=dev)
+        c5[label] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_matmul(dx.F32, ptr(Am), ptr(Bm), ptr(Cm), 1, mm, kk, nn, None)),
+                          flops=2 * mm * kk * nn, peak_tf=MFMA_F32_PEAK_TF, peak_name="frac_mfma_f32")
     res["config5"] = c5
     return res
 

@@ -4,7 +4,7 @@
 // and cblas_sgemm of executor/op-ompsimd/src/deepx/tensorfunc/matmul_cblas.hpp:11-60 (alpha=1, beta=0).
 //
 //   bf16 / f16   MFMA v_mfma_f32_32x32x16_{bf16,f16}, fp32 accumulate, one RNE rounding of C.
-//                Aligned shapes (K % 64 == 0, N % 8 == 0): matmul_mfma_tile_kernel, 128x128 or
+//                Aligned shapes (K % 64 == 0, N % 8 == 0): matmul_mfma_tile_kernel, 64x64 to
 //                256x256 workgroup tiles, software-pipelined over K.  Anything else:
 //                matmul_mfma_kernel, a plain 128x128x32 tile with element-wise edge handling.
 //   f32          MFMA v_mfma_f32_32x32x2_f32 (fp32 operands and accumulate): matmul_mfma_f32_kernel.
@@ -122,7 +122,7 @@ constexpr int PK = 64;  // K step of the MFMA tile kernel
 __device__ inline int swz(int row, int chunk) { return chunk ^ ((row ^ (row >> 3)) & 7); }
 
 // ---- MFMA kernel with the B transposition done by the LDS read ------------------------------
-// Workgroup tile TM x TN (128 or 256 each), K step 64, 4 waves in a 2x2 grid, each wave a
+// Workgroup tile TM x TN (64, 128 or 256 each), K step 64, 4 waves in a 2x2 grid, each wave a
 // (TM/2) x (TN/2) patch of 32x32x16 MFMAs.  Requirements (checked by the launcher): K % 64 == 0,
 // N % 8 == 0, 16-byte aligned A, B, C.
 //   loads  every global load is 16 bytes per lane (a wave instruction occupies the vector cache for
@@ -158,6 +158,10 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t *p) {
     s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p);
     return __builtin_bit_cast(u32x2, v);
 }
+
+// the `count` loads of a K step are dealt out over its four k-substeps
+constexpr int part_first(int count, int part) { return count * part / 4; }
+constexpr int part_count(int count, int part) { return count * (part + 1) / 4 - count * part / 4; }
 
 template <typename T, int TM, int TN, int PD>
 __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul_mfma_tile_kernel(
@@ -205,23 +209,23 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
 
     u32x4 ra[PD][A_LD], rb[PD][B_LD];
     auto load_part = [&](auto set, auto part, int k0) __attribute__((always_inline)) {
-        static_for<A_LD / 4>([&](auto q) __attribute__((always_inline)) {
-            constexpr int i = decltype(part)::value * (A_LD / 4) + decltype(q)::value;
+        static_for<part_count(A_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
+            constexpr int i = part_first(A_LD, decltype(part)::value) + decltype(q)::value;
             ra[set][i] = *reinterpret_cast<const u32x4 *>(Ab + a_off[i] + k0);
         });
-        static_for<B_LD / 4>([&](auto q) __attribute__((always_inline)) {
-            constexpr int i = decltype(part)::value * (B_LD / 4) + decltype(q)::value;
+        static_for<part_count(B_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
+            constexpr int i = part_first(B_LD, decltype(part)::value) + decltype(q)::value;
             rb[set][i] = *reinterpret_cast<const u32x4 *>(Bb + (int64_t)(k0 + i * KR) * N + b_off);
         });
     };
     auto store_part = [&](auto set, auto part, auto stage) __attribute__((always_inline)) {
         uint16_t *As = lds + decltype(stage)::value * STAGE, *Bs = As + A_STAGE;
-        static_for<A_LD / 4>([&](auto q) __attribute__((always_inline)) {
-            constexpr int i = decltype(part)::value * (A_LD / 4) + decltype(q)::value;
+        static_for<part_count(A_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
+            constexpr int i = part_first(A_LD, decltype(part)::value) + decltype(q)::value;
             *reinterpret_cast<u32x4 *>(As + a_lds[i]) = ra[set][i];
         });
-        static_for<B_LD / 4>([&](auto q) __attribute__((always_inline)) {
-            constexpr int i = decltype(part)::value * (B_LD / 4) + decltype(q)::value;
+        static_for<part_count(B_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
+            constexpr int i = part_first(B_LD, decltype(part)::value) + decltype(q)::value;
             *reinterpret_cast<u32x4 *>(Bs + b_lds + i * KR * B_ROW) = rb[set][i];
         });
     };
@@ -251,7 +255,7 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
         });
     });
     constexpr int NM = FM * FN;                                 // MFMAs per k-substep
-    constexpr int ND = FM + 2 * FN, NW = (A_LD + B_LD) / 4;     // LDS reads, LDS writes (= global loads) per substep
+    constexpr int ND = FM + 2 * FN;                             // LDS fragment reads per substep
     auto mma = [&](auto buf, auto lo, auto hi) __attribute__((always_inline)) {
         static_for<decltype(hi)::value - decltype(lo)::value>([&](auto x) __attribute__((always_inline)) {
             constexpr int idx = decltype(lo)::value + decltype(x)::value, i = idx / FN, j = idx % FN;
@@ -281,6 +285,7 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
         constexpr int s = decltype(S)::value;
         static_for<4>([&](auto ks) __attribute__((always_inline)) {
             constexpr int cur = decltype(ks)::value & 1;
+            constexpr int NW = part_count(A_LD, decltype(ks)::value) + part_count(B_LD, decltype(ks)::value);  // LDS writes = global loads
             if constexpr (decltype(ks)::value < 3) {
                 read_frags(ic<cur ^ 1>{}, S, ic<decltype(ks)::value + 1>{});
                 store_part(R, ks, ic<s ^ 1>{});
@@ -591,16 +596,22 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
     int64_t choice = tuning().matmul_tile;
     if (fast && choice == 0) {
         // 256x256 tiles halve the bytes every CU pulls through its vector cache per flop, but need
-        // about one tile per CU to pay off; below that the 128x128 tiles (two workgroups per CU)
-        // spread the work better.
-        const int64_t tiles256 = batch * ((m + 255) / 256) * ((n + 255) / 256);
-        choice = (tiles256 * 10 >= (int64_t)compute_units() * 9) ? 4 : 1;
+        // about one tile per CU to pay off.  Below that, 128x128 tiles (two workgroups per CU) as
+        // long as they still give every CU a workgroup and a half; skinny outputs go to 128x64 or
+        // 64x64 tiles so that all CUs (and their vector caches) take part.
+        const int64_t cus = compute_units();
+        auto tiles = [&](int tm, int tn) { return batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn); };
+        if (tiles(256, 256) * 10 >= cus * 9) choice = 4;
+        else if (tiles(128, 128) * 2 >= cus * 3) choice = 1;
+        else if (tiles(128, 64) * 2 >= cus) choice = 2;
+        else choice = 5;
     }
     if (fast) {
         switch (choice) {
-        case 2: return launch_tile<T, 256, 128, 2>(a, b, c, batch, m, k, n, st);
-        case 3: return launch_tile<T, 128, 256, 2>(a, b, c, batch, m, k, n, st);
+        case 2: return launch_tile<T, 128, 64, 1>(a, b, c, batch, m, k, n, st);
+        case 3: return launch_tile<T, 64, 128, 1>(a, b, c, batch, m, k, n, st);
         case 4: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, st);
+        case 5: return launch_tile<T, 64, 64, 1>(a, b, c, batch, m, k, n, st);
         default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, st);
         }
     }
@@ -660,6 +671,7 @@ inline int launch_f32(const void *a, const void *b, void *c, int64_t batch, int6
     switch (choice) {
     case 1: return launch_f32_tile<2, 2, 32, 1>(af, bf, cf, batch, m, k, n, vec, st);
     case 2: return launch_f32_tile<2, 1, 32, 2>(af, bf, cf, batch, m, k, n, vec, st);
+    case 3: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, st);
     case 4: return launch_f32_tile<2, 2, 16, 1>(af, bf, cf, batch, m, k, n, vec, st);
     default: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, st);
     }

@@ -126,4 +126,30 @@ int dxh_event_elapsed_ms(void *start, void *stop, float *ms) {
     return (int)hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop);
 }
 
+int dxh_graph_begin_capture(void *stream) {
+    if (!stream) return DXH_ERR_ARG;  // the NULL stream cannot be captured
+    return (int)hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal);
+}
+int dxh_graph_end_capture(void *stream, void **graph_exec) {
+    if (!stream || !graph_exec) return DXH_ERR_ARG;
+    *graph_exec = nullptr;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(as_stream(stream), &graph);
+    if (e != hipSuccess || !graph) {
+        (void)hipGetLastError();
+        return e != hipSuccess ? (int)e : DXH_ERR_ARG;
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return (int)e;
+    *graph_exec = (void *)exec;
+    return DXH_OK;
+}
+int dxh_graph_launch(void *graph_exec, void *stream) {
+    if (!graph_exec || !stream) return DXH_ERR_ARG;
+    return (int)hipGraphLaunch((hipGraphExec_t)graph_exec, as_stream(stream));
+}
+int dxh_graph_destroy(void *graph_exec) { return graph_exec ? (int)hipGraphExecDestroy((hipGraphExec_t)graph_exec) : DXH_OK; }
+
 }  // extern "C"

@@ -1,7 +1,9 @@
 // capi.cpp — libdxexec.so: the executor's dispatch core behind a C ABI, so a harness (or an
 // embedding scheduler) can feed deepxIR lines without a socket.  Same code path as the UDP binary.
 #include <cstring>
+#include <sstream>
 #include <string>
+#include <vector>
 #include "executor.hpp"
 
 using namespace deepx;
@@ -22,6 +24,25 @@ DXE_API void dxe_destroy(void *ex) { delete static_cast<Executor *>(ex); }
 // executes one IR line; writes the reply line; returns the reply length (may exceed buflen)
 DXE_API size_t dxe_execute(void *ex, const char *line, char *reply, size_t buflen) {
     return copy_out(static_cast<Executor *>(ex)->execute(line ? line : ""), reply, buflen);
+}
+// executes the newline-separated IR lines of `text` as one batch (what the UDP server does with a
+// datagram); writes the replies joined by '\n'; returns their total length
+DXE_API size_t dxe_execute_batch(void *ex, const char *text, char *reply, size_t buflen) {
+    std::vector<std::string> lines;
+    std::istringstream in(text ? text : "");
+    std::string line;
+    while (std::getline(in, line)) if (!line.empty()) lines.push_back(line);
+    if (lines.empty()) return copy_out("", reply, buflen);
+    std::string out;
+    for (const std::string &r : static_cast<Executor *>(ex)->execute_batch(lines)) { if (!out.empty()) out += '\n'; out += r; }
+    return copy_out(out, reply, buflen);
+}
+// graph recording on/off (the DEEPX_GRAPH switch) and the batch counters: "batches captures replays rejects"
+DXE_API void dxe_set_graphs(void *ex, int on) { static_cast<Executor *>(ex)->use_graphs = on != 0; }
+DXE_API size_t dxe_stats(void *ex, char *out, size_t buflen) {
+    const auto &s = static_cast<Executor *>(ex)->stats;
+    return copy_out(std::to_string(s.batches) + " " + std::to_string(s.graph_captures) + " " + std::to_string(s.graph_replays) + " " +
+                    std::to_string(s.graph_rejects), out, buflen);
 }
 // parse + print round trip (no execution): "name(args)->(returns) //metadata", or "error: ..."
 DXE_API size_t dxe_parse(const char *line, char *out, size_t buflen) {

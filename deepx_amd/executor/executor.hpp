@@ -8,9 +8,14 @@
 #pragma once
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <iostream>
 #include <mutex>
+#include <sstream>
 #include <string>
+#include <unordered_map>
+#include <unordered_set>
+#include <vector>
 #include "factory.hpp"
 #include "mem.hpp"
 
@@ -23,6 +28,10 @@ public:
     bool ir_log = false;    // DEEPX_IR_LOG=1|true echoes every instruction (main.cpp:17-21)
     bool sync_each = true;  // wait for the kernels before stamping finish_at; DEEPX_SYNC=0 replies at launch like op-cuda
     bool has_device = false;
+    // DEEPX_GRAPH=1: a datagram of several graph-safe lines that arrives a second time is recorded
+    // into a HIP graph and replayed from then on (one launch instead of one per kernel)
+    bool use_graphs = false;
+    struct Stats { uint64_t batches = 0, graph_captures = 0, graph_replays = 0, graph_rejects = 0; } stats;
 
     Executor() {
         register_all(factory);
@@ -32,6 +41,12 @@ public:
         if (s && !std::strcmp(s, "0")) sync_each = false;
         int count = 0;
         has_device = dxh_device_count(&count) == DXH_OK && count > 0;
+        const char *g = std::getenv("DEEPX_GRAPH");
+        use_graphs = g && !std::strcmp(g, "1");
+    }
+    ~Executor() {
+        for (auto &kv : graphs_) dxh_graph_destroy(kv.second.exec);
+        if (graph_stream_) dxh_stream_destroy(graph_stream_);
     }
 
     std::string execute(const std::string &line, TimePoint recv_at = std::chrono::system_clock::now()) {
@@ -77,8 +92,199 @@ public:
         return resp.to_string();
     }
 
+    // All lines of one datagram (udpserver.cpp:49-58 splits them the same way), one reply per line,
+    // in order.  The kernels of the whole datagram are launched back to back and waited for once,
+    // instead of once per line; finish_at of every line is then the end of the batch.  Each line
+    // still succeeds or fails on its own, as when sent one by one.
+    std::vector<std::string> execute_batch(const std::vector<std::string> &lines, TimePoint recv_at = std::chrono::system_clock::now()) {
+        if (lines.size() == 1) return {execute(lines[0], recv_at)};
+        std::lock_guard<std::mutex> lock(mu_);
+        ++stats.batches;
+        struct Item { TF call; std::shared_ptr<TF> tf; OpResp resp; bool failed = false; };
+        std::vector<Item> items(lines.size());
+        bool graphable = use_graphs && has_device;
+        std::string key;
+        for (size_t i = 0; i < lines.size(); ++i) {
+            Item &it = items[i];
+            it.resp.recv_at = it.resp.start_at = recv_at;
+            try {
+                it.call.parse(lines[i]);
+            } catch (const std::exception &e) {
+                it.resp.error(e.what());
+                it.failed = true;
+                graphable = false;
+                continue;
+            }
+            it.call.metadata.recv_at = recv_at;
+            it.resp.id = it.call.metadata.id;
+            if (ir_log) std::cout << "~" << it.call.to_string(true) << std::endl;
+            std::string why;
+            it.tf = factory.get_tf(it.call, &why);
+            if (!it.tf) {
+                std::cerr << why << std::endl;
+                it.resp.error("op" + it.call.name + " not found");
+                it.failed = true;
+                graphable = false;
+                continue;
+            }
+            it.tf->name = it.call.name;
+            it.tf->args = it.call.args;
+            it.tf->returns = it.call.returns;
+            graphable = graphable && it.tf->graph_safe && it.tf->metadata.benchmark_repeat <= 1 && !uses_named_arg(it.call);
+            key += it.call.to_string(false);
+            key += '\n';
+        }
+        bool done = false;
+        if (graphable) {
+            if (run_as_graph(key, items.size(), [&](size_t i, std::string &msg) { return items[i].tf->run(mem, msg); }, [&](size_t i) -> const TF & { return items[i].call; })) {
+                for (Item &it : items) { it.resp.start_at = recv_at; it.resp.finish(""); }
+                done = true;
+            }
+        }
+        if (!done) {
+            for (Item &it : items) {
+                if (it.failed) continue;
+                it.resp.start_at = std::chrono::system_clock::now();
+                int rc = 0;
+                std::string message;
+                const int repeat = it.tf->metadata.benchmark_repeat > 1 ? it.tf->metadata.benchmark_repeat : 1;
+                for (int r = 0; r < repeat && rc == 0; ++r) rc = it.tf->run(mem, message);
+                if (rc != 0) {
+                    std::cerr << message << std::endl;
+                    it.resp.error(message);
+                    it.failed = true;
+                }
+            }
+            std::string sync_error;
+            if (sync_each && has_device) {
+                int s = dxh_stream_sync(nullptr);
+                if (s != DXH_OK) sync_error = std::string("hip: ") + dxh_error_string(s);
+            }
+            for (Item &it : items) {
+                if (it.failed) continue;
+                if (!sync_error.empty()) it.resp.error(sync_error);
+                else it.resp.finish("");
+            }
+        }
+        std::vector<std::string> replies;
+        replies.reserve(items.size());
+        for (Item &it : items) replies.push_back(it.resp.to_string());
+        return replies;
+    }
+
 private:
+    struct Pinned { std::string name; const void *data; int64_t bytes; int dtype; };
+    struct Graph { void *exec = nullptr; std::vector<Pinned> tensors; const void *workspace = nullptr; };
+
+    // every tensor a call names (bare names, typed params and [a b c] lists alike)
+    void tensors_of(const TF &call, std::vector<std::string> &names) const {
+        auto scan = [&](const std::vector<Param> &ps) {
+            for (const Param &p : ps) {
+                std::string t = p.textvalue;
+                for (char &c : t) if (c == '[' || c == ']') c = ' ';
+                std::istringstream in(t);
+                std::string w;
+                while (in >> w) if (mem.existstensor(w)) names.push_back(w);
+            }
+        };
+        scan(call.args);
+        scan(call.returns);
+    }
+    // a scalar or vector taken from the arg store would be frozen into a recorded graph
+    bool uses_named_arg(const TF &call) const {
+        for (const Param &p : call.args) {
+            std::string t = p.textvalue;
+            for (char &c : t) if (c == '[' || c == ']') c = ' ';
+            std::istringstream in(t);
+            std::string w;
+            while (in >> w) if (!mem.existstensor(w) && mem.existarg(w)) return true;
+        }
+        return false;
+    }
+    bool snapshot(size_t n, const std::function<const TF &(size_t)> &call_at, Graph &g) const {
+        std::vector<std::string> names;
+        for (size_t i = 0; i < n; ++i) tensors_of(call_at(i), names);
+        g.tensors.clear();
+        for (const std::string &name : names) {
+            auto t = mem.gettensor(name);
+            g.tensors.push_back({name, t->data, t->shape.bytes(), t->dtype()});
+        }
+        g.workspace = mem.workspace_ptr();
+        return true;
+    }
+    static bool same_pins(const Graph &a, const Graph &b) {
+        if (a.workspace != b.workspace || a.tensors.size() != b.tensors.size()) return false;
+        for (size_t i = 0; i < a.tensors.size(); ++i)
+            if (a.tensors[i].name != b.tensors[i].name || a.tensors[i].data != b.tensors[i].data ||
+                a.tensors[i].bytes != b.tensors[i].bytes || a.tensors[i].dtype != b.tensors[i].dtype) return false;
+        return true;
+    }
+
+    // Returns true when the whole batch ran (was replayed or recorded and launched) as one graph.
+    // false = nothing ran on the device: the caller executes the lines eagerly.  A batch is only
+    // recorded on its second arrival (the first, eager, pass also sizes the reduction workspace),
+    // and replayed only while every tensor it names still has the address, size and dtype it was
+    // recorded with.
+    bool run_as_graph(const std::string &key, size_t n, const std::function<int(size_t, std::string &)> &run_at,
+                      const std::function<const TF &(size_t)> &call_at) {
+        if (rejected_.count(key)) return false;
+        Graph now;
+        try {
+            snapshot(n, call_at, now);
+        } catch (const std::exception &) {
+            return false;  // a missing tensor: the eager path reports it per line
+        }
+        auto it = graphs_.find(key);
+        if (it != graphs_.end() && !same_pins(it->second, now)) {
+            dxh_graph_destroy(it->second.exec);
+            graphs_.erase(it);
+            it = graphs_.end();
+        }
+        if (it == graphs_.end()) {
+            if (seen_.insert(key).second) return false;  // first arrival: run eagerly
+            if (!graph_stream_ && dxh_stream_create(&graph_stream_) != DXH_OK) { graph_stream_ = nullptr; return false; }
+            if (dxh_stream_sync(nullptr) != DXH_OK) return false;
+            if (dxh_graph_begin_capture(graph_stream_) != DXH_OK) return false;
+            mem.stream = graph_stream_;
+            mem.recording = true;
+            bool ok = true;
+            for (size_t i = 0; i < n && ok; ++i) {
+                std::string message;
+                ok = run_at(i, message) == 0;
+            }
+            mem.stream = nullptr;
+            mem.recording = false;
+            void *exec = nullptr;
+            int rc = dxh_graph_end_capture(graph_stream_, &exec);
+            if (!ok || rc != DXH_OK || !exec) {
+                if (exec) dxh_graph_destroy(exec);
+                rejected_.insert(key);
+                ++stats.graph_rejects;
+                return false;
+            }
+            if (graphs_.size() >= 64) {  // bounded cache: start over rather than track recency
+                for (auto &kv : graphs_) dxh_graph_destroy(kv.second.exec);
+                graphs_.clear();
+            }
+            now.exec = exec;
+            it = graphs_.emplace(key, now).first;
+            ++stats.graph_captures;
+        } else {
+            ++stats.graph_replays;
+        }
+        if (dxh_graph_launch(it->second.exec, graph_stream_) != DXH_OK || dxh_stream_sync(graph_stream_) != DXH_OK) {
+            dxh_graph_destroy(it->second.exec);
+            graphs_.erase(it);
+            rejected_.insert(key);
+            return false;
+        }
+        return true;
+    }
+
     std::mutex mu_;
+    void *graph_stream_ = nullptr;
+    std::unordered_map<std::string, Graph> graphs_;
+    std::unordered_set<std::string> seen_, rejected_;
 };
 
 }  // namespace deepx

@@ -122,6 +122,9 @@ public:
     std::string name, tftype;
     std::vector<Param> args, returns;
     TFMetadata metadata;
+    // true for ops that only launch kernels on Mem's stream (no allocation, host copy, file I/O or
+    // fresh random seed): those may be recorded into a HIP graph by the batch path
+    bool graph_safe = false;
 
     TF() = default;
     explicit TF(const std::string &text) { parse(text); }

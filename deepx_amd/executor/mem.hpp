@@ -72,9 +72,16 @@ public:
     }
     void clear() { tensors_.clear(); args_.clear(); }
 
+    // Stream every op launches on: NULL (the default stream) except while the executor records or
+    // replays a graph.  While recording nothing may allocate, so a workspace that would have to
+    // grow aborts the recording instead.
+    void *stream = nullptr;
+    bool recording = false;
+
     // reusable device scratch for reductions (grown on demand, never shrunk)
     void *workspace(size_t bytes) {
         if (bytes > ws_bytes_) {
+            if (recording) throw std::runtime_error("workspace would grow while recording a graph");
             if (ws_) { dxh_device_sync(); dxh_free(ws_); ws_ = nullptr; ws_bytes_ = 0; }
             size_t want = std::max<size_t>(bytes, (size_t)4 << 20);
             dxh_check(dxh_malloc(&ws_, want), "workspace dxh_malloc");
@@ -83,6 +90,7 @@ public:
         return ws_;
     }
     size_t workspace_bytes() const { return ws_bytes_; }
+    const void *workspace_ptr() const { return ws_; }
     ~Mem() { tensors_.clear(); if (ws_) dxh_free(ws_); }
 
 private:

@@ -66,6 +66,10 @@ void reg(TfFactory &f, const char *name, const char *author, const char *tftype,
     for (const char *a : args) tf->args.push_back(registered(a));
     for (const char *r : returns) tf->returns.push_back(registered(r));
     tf->fn = std::move(fn);
+    const std::string kind = tftype, op = name;
+    tf->graph_safe = kind == "elementwise" || kind == "reduce" || kind == "changeshape" || op == "matmul" ||
+                     op == "constant" || op == "arange";
+    if (op == "reshape") tf->graph_safe = false;  // rewrites the tensor's shape on the host
     f.add_tf(tf);
 }
 
@@ -166,28 +170,28 @@ RunFn binary(BinaryFn f, const char *op) {  // (A, B) -> (C)
     return [f, op](const TF &c, Mem &mem, std::string &error) {
         auto A = tensor_of(c.args[0], mem), B = tensor_of(c.args[1], mem), C = tensor_of(c.returns[0], mem);
         if (!same_dtype({A.get(), B.get(), C.get()}, error) || !same_size({A.get(), B.get(), C.get()}, error)) return 1;
-        return hip_result(f(A->dtype(), A->data, B->data, C->data, C->shape.size, nullptr), op, error);
+        return hip_result(f(A->dtype(), A->data, B->data, C->data, C->shape.size, mem.stream), op, error);
     };
 }
 RunFn with_scalar(ScalarFn f, const char *op) {  // (A, scalar) -> (C)
     return [f, op](const TF &c, Mem &mem, std::string &error) {
         auto A = tensor_of(c.args[0], mem), C = tensor_of(c.returns[0], mem);
         if (!same_dtype({A.get(), C.get()}, error) || !same_size({A.get(), C.get()}, error)) return 1;
-        return hip_result(f(A->dtype(), A->data, scalar_of(c.args[1], mem), C->data, C->shape.size, nullptr), op, error);
+        return hip_result(f(A->dtype(), A->data, scalar_of(c.args[1], mem), C->data, C->shape.size, mem.stream), op, error);
     };
 }
 RunFn with_rscalar(RScalarFn f, const char *op) {  // (scalar, A) -> (C)
     return [f, op](const TF &c, Mem &mem, std::string &error) {
         auto A = tensor_of(c.args[1], mem), C = tensor_of(c.returns[0], mem);
         if (!same_dtype({A.get(), C.get()}, error) || !same_size({A.get(), C.get()}, error)) return 1;
-        return hip_result(f(A->dtype(), scalar_of(c.args[0], mem), A->data, C->data, C->shape.size, nullptr), op, error);
+        return hip_result(f(A->dtype(), scalar_of(c.args[0], mem), A->data, C->data, C->shape.size, mem.stream), op, error);
     };
 }
 RunFn unary(UnaryFn f, const char *op) {  // (A) -> (C)
     return [f, op](const TF &c, Mem &mem, std::string &error) {
         auto A = tensor_of(c.args[0], mem), C = tensor_of(c.returns[0], mem);
         if (!same_dtype({A.get(), C.get()}, error) || !same_size({A.get(), C.get()}, error)) return 1;
-        return hip_result(f(A->dtype(), A->data, C->data, C->shape.size, nullptr), op, error);
+        return hip_result(f(A->dtype(), A->data, C->data, C->shape.size, mem.stream), op, error);
     };
 }
 bool mask_ok(const Tensor &m, std::string &error) {
@@ -200,28 +204,28 @@ RunFn compare_eps(CmpEpsFn f, const char *op) {  // (A, B, epsilon) -> (mask)
     return [f, op](const TF &c, Mem &mem, std::string &error) {
         auto A = tensor_of(c.args[0], mem), B = tensor_of(c.args[1], mem), M = tensor_of(c.returns[0], mem);
         if (!same_dtype({A.get(), B.get()}, error) || !mask_ok(*M, error) || !same_size({A.get(), B.get(), M.get()}, error)) return 1;
-        return hip_result(f(A->dtype(), A->data, B->data, float_of(c.args[2], mem), M->data, M->shape.size, nullptr), op, error);
+        return hip_result(f(A->dtype(), A->data, B->data, float_of(c.args[2], mem), M->data, M->shape.size, mem.stream), op, error);
     };
 }
 RunFn compare_eps_scalar(CmpEpsScalarFn f, const char *op) {  // (A, scalar, epsilon) -> (mask)
     return [f, op](const TF &c, Mem &mem, std::string &error) {
         auto A = tensor_of(c.args[0], mem), M = tensor_of(c.returns[0], mem);
         if (!mask_ok(*M, error) || !same_size({A.get(), M.get()}, error)) return 1;
-        return hip_result(f(A->dtype(), A->data, scalar_of(c.args[1], mem), float_of(c.args[2], mem), M->data, M->shape.size, nullptr), op, error);
+        return hip_result(f(A->dtype(), A->data, scalar_of(c.args[1], mem), float_of(c.args[2], mem), M->data, M->shape.size, mem.stream), op, error);
     };
 }
 RunFn compare(BinaryFn f, const char *op) {  // (A, B) -> (mask)
     return [f, op](const TF &c, Mem &mem, std::string &error) {
         auto A = tensor_of(c.args[0], mem), B = tensor_of(c.args[1], mem), M = tensor_of(c.returns[0], mem);
         if (!same_dtype({A.get(), B.get()}, error) || !mask_ok(*M, error) || !same_size({A.get(), B.get(), M.get()}, error)) return 1;
-        return hip_result(f(A->dtype(), A->data, B->data, M->data, M->shape.size, nullptr), op, error);
+        return hip_result(f(A->dtype(), A->data, B->data, M->data, M->shape.size, mem.stream), op, error);
     };
 }
 RunFn compare_scalar(ScalarFn f, const char *op) {  // (A, scalar) -> (mask)
     return [f, op](const TF &c, Mem &mem, std::string &error) {
         auto A = tensor_of(c.args[0], mem), M = tensor_of(c.returns[0], mem);
         if (!mask_ok(*M, error) || !same_size({A.get(), M.get()}, error)) return 1;
-        return hip_result(f(A->dtype(), A->data, scalar_of(c.args[1], mem), M->data, M->shape.size, nullptr), op, error);
+        return hip_result(f(A->dtype(), A->data, scalar_of(c.args[1], mem), M->data, M->shape.size, mem.stream), op, error);
     };
 }
 
@@ -240,7 +244,7 @@ RunFn reduce(ReduceFn f, const char *op) {  // (A, vector dims, bool keepdims) -
         if (rc != DXH_OK) return hip_result(rc, op, error);
         void *ws = need ? mem.workspace(need) : nullptr;
         return hip_result(f(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), dims.data(), (int)dims.size(), B->data, ws,
-                            need ? mem.workspace_bytes() : 0, nullptr), op, error);
+                            need ? mem.workspace_bytes() : 0, mem.stream), op, error);
     };
 }
 
@@ -276,7 +280,7 @@ int register_all(TfFactory &f) {
             auto S = tensor_of(c.args[0], mem), D = tensor_of(c.returns[0], mem);
             if (S->shape.dtype != D->shape.dtype) return fail(error, "copytensor: input type and return type must be the same");
             if (!same_size({S.get(), D.get()}, error)) return 1;
-            return hip_result(dxh_memcpy_d2d(D->data, S->data, (size_t)S->shape.bytes(), nullptr), "copytensor", error);
+            return hip_result(dxh_memcpy_d2d(D->data, S->data, (size_t)S->shape.bytes(), mem.stream), "copytensor", error);
         });
     reg(f, "deltensor", "", "tensorlife", "del->T1", {}, {"tensor<any>:t"},
         [](const TF &c, Mem &mem, std::string &) { mem.delete_tensor(c.returns[0].textvalue); return 0; });
@@ -324,29 +328,29 @@ int register_all(TfFactory &f) {
             auto T = tensor_of(c.returns[0], mem);
             dxh_scalar v = T->shape.dtype == Precision::Bool && !text_is_float(c.args[0].textvalue)
                                ? dxh_scalar{bool_of(c.args[0]) ? 1.0 : 0.0, bool_of(c.args[0]) ? 1 : 0} : scalar_of(c.args[0], mem);
-            return hip_result(dxh_constant(T->dtype(), T->data, T->shape.size, v, nullptr), "constant", error);
+            return hip_result(dxh_constant(T->dtype(), T->data, T->shape.size, v, mem.stream), "constant", error);
         });
     reg(f, "arange", "miaobyte", "init", "arange(start,step)->T1", {"var<any>:start", "var<any>:step"}, {"tensor<any>:t"},
         [](const TF &c, Mem &mem, std::string &error) {
             auto T = tensor_of(c.returns[0], mem);
-            return hip_result(dxh_arange(T->dtype(), T->data, T->shape.size, scalar_of(c.args[0], mem), scalar_of(c.args[1], mem), nullptr), "arange", error);
+            return hip_result(dxh_arange(T->dtype(), T->data, T->shape.size, scalar_of(c.args[0], mem), scalar_of(c.args[1], mem), mem.stream), "arange", error);
         });
     reg(f, "uniform", "miaobyte", "init", "uniform(low,high,seed)->T1", {"var<any>:low", "var<any>:high", "var<int32>:seed"}, {"tensor<any>:t"},
         [](const TF &c, Mem &mem, std::string &error) {
             auto T = tensor_of(c.returns[0], mem);
             return hip_result(dxh_uniform(T->dtype(), T->data, T->shape.size, scalar_of(c.args[0], mem), scalar_of(c.args[1], mem),
-                                          (uint32_t)int_of(c.args[2], mem), nullptr), "uniform", error);
+                                          (uint32_t)int_of(c.args[2], mem), mem.stream), "uniform", error);
         });
     reg(f, "normal", "miaobyte", "init", "normal(mean,stddev,seed)->T1", {"var<any>:mean", "var<any>:stddev", "var<int32>:seed"}, {"tensor<any>:t"},
         [](const TF &c, Mem &mem, std::string &error) {
             auto T = tensor_of(c.returns[0], mem);
             return hip_result(dxh_normal(T->dtype(), T->data, T->shape.size, scalar_of(c.args[0], mem), scalar_of(c.args[1], mem),
-                                         (uint32_t)int_of(c.args[2], mem), nullptr), "normal", error);
+                                         (uint32_t)int_of(c.args[2], mem), mem.stream), "normal", error);
         });
     reg(f, "dropout", "miaobyte", "init", "dropout(p,seed)->A", {"var<float32>:p", "var<int32>:seed"}, {"tensor<any>:A"},
         [](const TF &c, Mem &mem, std::string &error) {
             auto T = tensor_of(c.returns[0], mem);
-            return hip_result(dxh_dropout(T->dtype(), T->data, T->shape.size, float_of(c.args[0], mem), (uint32_t)int_of(c.args[1], mem), nullptr), "dropout", error);
+            return hip_result(dxh_dropout(T->dtype(), T->data, T->shape.size, float_of(c.args[0], mem), (uint32_t)int_of(c.args[1], mem), mem.stream), "dropout", error);
         });
 
     // ---- io (tf/io.hpp) --------------------------------------------------------------------------
@@ -383,7 +387,7 @@ int register_all(TfFactory &f) {
         [](const TF &c, Mem &mem, std::string &error) {
             auto A = tensor_of(c.args[0], mem), C = tensor_of(c.returns[0], mem);
             if (A->shape.size != C->shape.size) return fail(error, "Shape mismatch: " + std::to_string(A->shape.size) + " != " + std::to_string(C->shape.size));
-            return hip_result(dxh_todtype(A->dtype(), A->data, C->dtype(), C->data, C->shape.size, nullptr), "todtype", error);
+            return hip_result(dxh_todtype(A->dtype(), A->data, C->dtype(), C->data, C->shape.size, mem.stream), "todtype", error);
         });
 #define T_ANY "tensor<any>"
     reg(f, "add", "miaobyte", "elementwise", "T3=T1+T2", {T_ANY ":a", T_ANY ":b"}, {T_ANY ":c"}, binary(dxh_add, "add"));
@@ -436,7 +440,7 @@ int register_all(TfFactory &f) {
             }
             if (!same_size({cases.get(), C.get()}, error)) return 1;
             if (cases->shape.dtype == Precision::Bool && names.size() != 2) return fail(error, "For bool cases, tensors size must be 2");
-            return hip_result(dxh_switch(C->dtype(), ptrs.data(), (int)ptrs.size(), cases->dtype(), cases->data, C->data, C->shape.size, nullptr), "switch", error);
+            return hip_result(dxh_switch(C->dtype(), ptrs.data(), (int)ptrs.size(), cases->dtype(), cases->data, C->data, C->shape.size, mem.stream), "switch", error);
         });
 
     // ---- reduce (tf/reduce.hpp) ------------------------------------------------------------------
@@ -454,7 +458,7 @@ int register_all(TfFactory &f) {
             Shape ns(shape, B->shape.dtype);
             if (ns.size != A->shape.size || ns.size != B->shape.size) return fail(error, "Shape size mismatch");
             B->shape = ns;  // metadata only when A and B are the same tensor, else a copy too
-            if (A->data != B->data) return hip_result(dxh_memcpy_d2d(B->data, A->data, (size_t)A->shape.bytes(), nullptr), "reshape", error);
+            if (A->data != B->data) return hip_result(dxh_memcpy_d2d(B->data, A->data, (size_t)A->shape.bytes(), mem.stream), "reshape", error);
             return 0;
         });
     reg(f, "transpose", "miaobyte", "changeshape", "T1.transpose(dimorder=[1,0])->T2", {T_ANY ":A", "vector<int32>:dim_order"}, {T_ANY ":C"},
@@ -466,7 +470,7 @@ int register_all(TfFactory &f) {
             if (C->shape.size != A->shape.size) return fail(error, "transpose error!shape");
             if (A->data == C->data) return fail(error, "transpose cannot run in place");
             (void)want;
-            return hip_result(dxh_transpose(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), order.data(), C->data, nullptr), "transpose", error);
+            return hip_result(dxh_transpose(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), order.data(), C->data, mem.stream), "transpose", error);
         });
     reg(f, "concat", "miaobyte", "changeshape", "Tresult = concat([T1, T2...], axis=3)", {"listtensor<any>:tensors", "var<int32>:dim"}, {T_ANY ":result"},
         [](const TF &c, Mem &mem, std::string &error) {
@@ -488,7 +492,7 @@ int register_all(TfFactory &f) {
             std::vector<int> want = concat_shape(shapes, axis);
             if (want != R->shape.shape) return fail(error, "Output tensor shape size must match the sum of input tensor shape sizes for concat");
             for (auto &s : shapes) axis_sizes.push_back(s[axis]);
-            return hip_result(dxh_concat(R->dtype(), ptrs.data(), (int)ptrs.size(), axis_sizes.data(), want.data(), (int)want.size(), axis, R->data, nullptr), "concat", error);
+            return hip_result(dxh_concat(R->dtype(), ptrs.data(), (int)ptrs.size(), axis_sizes.data(), want.data(), (int)want.size(), axis, R->data, mem.stream), "concat", error);
         });
     reg(f, "broadcastTo", "miaobyte", "changeshape", "T2 = T1.broadcastTo(new_shape=[4,3,2])", {T_ANY ":A", "vector<int32>:new_shape"}, {T_ANY ":B"},
         [](const TF &c, Mem &mem, std::string &error) {
@@ -497,7 +501,7 @@ int register_all(TfFactory &f) {
             std::vector<int> ns = ints_of(c.args[1], mem);
             if (broadcast_shape(A->shape.shape, ns) != ns) return fail(error, "Broadcast shape mismatch");
             if (Shape(ns).size != B->shape.size) return fail(error, "Broadcast shape mismatch: output is " + dims_str(B->shape.shape));
-            return hip_result(dxh_broadcastTo(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), ns.data(), (int)ns.size(), B->data, nullptr), "broadcastTo", error);
+            return hip_result(dxh_broadcastTo(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), ns.data(), (int)ns.size(), B->data, mem.stream), "broadcastTo", error);
         });
     reg(f, "indexselect", "miaobyte", "changeshape", "T2 = T1.indexselect(index=T3, axis=3)", {T_ANY ":A", "tensor<int64|int32>:index", "var<int32>:axis"}, {T_ANY ":B"},
         [](const TF &c, Mem &mem, std::string &error) {
@@ -509,7 +513,7 @@ int register_all(TfFactory &f) {
             if (ga < 0 || ga >= A->shape.dim()) return fail(error, "Axis is out of bounds");
             if (indexselect_shape(A->shape.shape, I->shape.shape, ga) != B->shape.shape) return fail(error, "Indexselect shape mismatch");
             return hip_result(dxh_indexselect(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), I->dtype(), I->data, I->shape.shape.data(),
-                                              I->shape.dim(), ga, B->data, nullptr), "indexselect", error);
+                                              I->shape.dim(), ga, B->data, mem.stream), "indexselect", error);
         });
     reg(f, "repeat", "miaobyte", "changeshape", "T1.repeat(repeats=[4,3,2])->T2", {T_ANY ":A", "vector<int32>:repeats"}, {T_ANY ":B"},
         [](const TF &c, Mem &mem, std::string &error) {
@@ -517,7 +521,7 @@ int register_all(TfFactory &f) {
             if (!same_dtype({A.get(), B.get()}, error)) return 1;
             std::vector<int> reps = ints_of(c.args[1], mem);
             if (repeat_shape(A->shape.shape, reps) != B->shape.shape) return fail(error, "Repeat shape mismatch");
-            return hip_result(dxh_repeat(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), reps.data(), B->data, nullptr), "repeat", error);
+            return hip_result(dxh_repeat(A->dtype(), A->data, A->shape.shape.data(), A->shape.dim(), reps.data(), B->data, mem.stream), "repeat", error);
         });
 
     // ---- matmul (tf/matmul.hpp).  The front asks for author "cublas" (authormap.py:60), op-ompsimd
@@ -529,7 +533,7 @@ int register_all(TfFactory &f) {
         if (want != C->shape.shape) return fail(error, "matmul: output shape " + dims_str(C->shape.shape) + " != " + dims_str(want));
         int64_t batch = 1;
         for (int i = 0; i + 2 < A->shape.dim(); ++i) batch *= A->shape.shape[i];
-        return hip_result(dxh_matmul(A->dtype(), A->data, B->data, C->data, batch, A->shape.at(-2), A->shape.at(-1), B->shape.at(-1), nullptr), "matmul", error);
+        return hip_result(dxh_matmul(A->dtype(), A->data, B->data, C->data, batch, A->shape.at(-2), A->shape.at(-1), B->shape.at(-1), mem.stream), "matmul", error);
     };
     for (const char *author : {"cublas", "cblas", "miaobyte"})
         reg(f, "matmul", author, "matmul", "T3=T1 @ T2", {T_ANY ":A", T_ANY ":B"}, {T_ANY ":C"}, matmul);

@@ -52,13 +52,17 @@ public:
             TimePoint recv_at = std::chrono::system_clock::now();
             std::istringstream lines(std::string(buf.data(), (size_t)n));
             std::string line;
+            std::vector<std::string> batch;
             while (std::getline(lines, line)) {
                 if (!line.empty() && line.back() == '\r') line.pop_back();
                 if (line.empty()) continue;
                 if (line == "__quit__") { stop_ = true; break; }
-                std::string reply = ex.execute(line, recv_at);
-                ::sendto(fd_, reply.data(), reply.size(), 0, (const sockaddr *)&cli, len);
+                batch.push_back(line);
             }
+            if (batch.empty()) continue;
+            // the lines of one datagram run as one batch: one wait for the device, one reply per line
+            for (const std::string &reply : ex.execute_batch(batch, recv_at))
+                ::sendto(fd_, reply.data(), reply.size(), 0, (const sockaddr *)&cli, len);
         }
     }
     void stop() { stop_ = true; }

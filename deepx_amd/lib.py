@@ -67,6 +67,10 @@ SIGNATURES = {
     "dxh_event_record": ([_p, _p], _i),
     "dxh_event_sync": ([_p], _i),
     "dxh_event_elapsed_ms": ([_p, _p, C.POINTER(_f)], _i),
+    "dxh_graph_begin_capture": ([_p], _i),
+    "dxh_graph_end_capture": ([_p, C.POINTER(_p)], _i),
+    "dxh_graph_launch": ([_p, _p], _i),
+    "dxh_graph_destroy": ([_p], _i),
     "dxh_add": (_BIN, _i), "dxh_sub": (_BIN, _i), "dxh_mul": (_BIN, _i), "dxh_div": (_BIN, _i),
     "dxh_max": (_BIN, _i), "dxh_min": (_BIN, _i), "dxh_pow": (_BIN, _i),
     "dxh_addscalar": (_SCL, _i), "dxh_subscalar": (_SCL, _i), "dxh_rsubscalar": (_RSCL, _i),

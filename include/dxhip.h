@@ -112,6 +112,18 @@ DXH_API int dxh_event_record(void *event, void *stream);
 DXH_API int dxh_event_sync(void *event);
 DXH_API int dxh_event_elapsed_ms(void *start, void *stop, float *ms);
 
+/* ---- HIP graphs: record the kernels a sequence of dxh_* calls launches on `stream` once, replay
+ * them with one launch.  No counterpart in the reference (it launches op by op on the default
+ * stream); used by the executor for datagrams that carry several deepxIR lines
+ * (executor/deepxcore/src/client/udpserver.cpp:49-58 already splits them).  `stream` must be a
+ * stream from dxh_stream_create, not NULL.  Between begin and end only kernel-launching dxh_* calls
+ * and dxh_memcpy_d2d may run on it; no allocation, synchronisation or host copy.  end_capture
+ * returns an executable graph (NULL with an error code if the capture was invalidated). */
+DXH_API int dxh_graph_begin_capture(void *stream);
+DXH_API int dxh_graph_end_capture(void *stream, void **graph_exec);
+DXH_API int dxh_graph_launch(void *graph_exec, void *stream);
+DXH_API int dxh_graph_destroy(void *graph_exec);
+
 /* ---- elementwise, C[i] = A[i] op B[i]
  * launch_add/sub/mul/div  elementwise_miaobyte_basic.cuh:16-98
  * launch_max/min          elementwise_miaobyte_compare.cuh:15-44

@@ -172,3 +172,22 @@ def test_udp_server_error_paths_and_framing():
     finally:
         srv.close()
     assert srv.proc.returncode == 0
+
+
+def test_inproc_batch_replies_in_order(ex):
+    """A datagram's lines as one batch: one reply per line, in order, each line failing or
+    succeeding on its own (same replies as when the lines are sent one by one)."""
+    lines = ["argset(var<int32>:1)->(var<int32>:ba) // id=201", "frobnicate(tensor<float32>:a)->(tensor<float32>:c) // id=202",
+             "garbage", "add(tensor<float32>:nope, tensor<float32>:b)->(tensor<float32>:c) // id=204",
+             "vecset(vector<int32>:[4 5])->(vector<int32>:bv) // id=205"]
+    before = ex.stats()["batches"]
+    rs = ex.execute_batch(lines)
+    assert len(rs) == 5
+    assert rs[0].startswith("201 ok//") and rs[4].startswith("205 ok//")
+    assert rs[1].startswith("202 error//") and rs[1].endswith("opfrobnicate not found")
+    assert rs[2].endswith("Invalid IR format: missing arrow")
+    assert rs[3].startswith("204 error//") and rs[3].endswith("tensor not found: nope")
+    assert ex.stats()["batches"] == before + 1
+    # a batch of one line is the plain path
+    assert ex.execute_batch(["argset(var<int32>:9)->(var<int32>:bz) // id=206"])[0].startswith("206 ok//")
+    assert ex.stats()["batches"] == before + 1

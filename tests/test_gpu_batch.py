@@ -1,0 +1,187 @@
+"""GPU: several deepxIR lines per datagram — run as one batch (one wait for the device) and, with
+DEEPX_GRAPH=1, recorded into a HIP graph on the second arrival and replayed afterwards.  Every
+replay is checked bit for bit against the same lines executed one by one, with eager work and
+synchronisations between the replays."""
+import numpy as np
+import pytest
+
+from tests.executor_client import InProc, UdpExecutor, read_tensor, write_tensor
+
+pytestmark = pytest.mark.gpu
+
+
+def T(name, dt="float32"):
+    return f"tensor<{dt}>:{name}"
+
+
+def V(values):
+    return "vector<int32>:[" + " ".join(str(v) for v in values) + "]"
+
+
+class Host:
+    """tensor upload/download through the executor's own load/save ops"""
+
+    def __init__(self, ex, tmp_path):
+        self.ex, self.tmp, self.n = ex, tmp_path, 0
+
+    def run(self, line):
+        self.n += 1
+        r = self.ex.execute(f"{line} // id={self.n}")
+        assert r.startswith(f"{self.n} ok//"), r
+
+    def put(self, name, arr, dtype_name="float32"):
+        p = str(self.tmp / name)
+        write_tensor(p, arr, dtype_name)
+        self.run(f"load(var<string>:{p})->()")
+
+    def get(self, name):
+        p = str(self.tmp / (name + "_out"))
+        self.run(f"save({T(name, 'any')}, var<string>:{p})->()")
+        return read_tensor(p)[0]
+
+
+CHAIN = ["add({A}, {B})->({C})", "mul({C}, {B})->({D})", "addscalar({D}, var<float32>:0.5)->({E})", "exp({E})->({F})",
+         "mulscalar({B}, var<float32>:-1)->({nB})", "max({B}, {nB})->({absB})", "addscalar({absB}, var<float32>:1)->({den})",
+         "div({F}, {den})->({G})"]
+NAMES = ["A", "B", "C", "D", "E", "F", "nB", "absB", "den", "G"]
+
+
+def chain_lines(prefix, first_id):
+    names = {n: T(prefix + n) for n in NAMES}
+    return [line.format(**names) + f" // author=miaobyte id={first_id + i}" for i, line in enumerate(CHAIN)]
+
+
+def make_chain(h, prefix, shape, rng):
+    for n in NAMES[2:]:
+        h.run(f"newtensor({V(shape)})->({T(prefix + n)})")
+    h.put(prefix + "A", rng.uniform(-1, 1, shape).astype(np.float32))
+    h.put(prefix + "B", rng.uniform(-1, 1, shape).astype(np.float32))
+
+
+def test_batch_equals_line_by_line(tmp_path):
+    ex = InProc()
+    h = Host(ex, tmp_path)
+    rng = np.random.default_rng(41)
+    make_chain(h, "s_", [257, 129], rng)
+    for line in chain_lines("s_", 1000):
+        assert ex.execute(line).split(" ")[1].startswith("ok")
+    want = {n: h.get("s_" + n) for n in NAMES[2:]}
+    for n in NAMES[2:]:
+        h.run(f"constant(var<float32>:0)->({T('s_' + n)})")
+    rs = ex.execute_batch(chain_lines("s_", 2000))
+    assert [r.split(" ")[0] for r in rs] == [str(2000 + i) for i in range(8)] and all(r.split(" ")[1].startswith("ok") for r in rs)
+    for n in NAMES[2:]:
+        assert np.array_equal(h.get("s_" + n).view(np.uint32), want[n].view(np.uint32)), n
+    assert ex.stats()["captures"] == 0  # graphs are off unless asked for
+
+
+def test_graph_replays_track_new_inputs(tmp_path):
+    ex = InProc()
+    ex.set_graphs(True)
+    h = Host(ex, tmp_path)
+    rng = np.random.default_rng(42)
+    shape = [300, 200]
+    make_chain(h, "g_", shape, rng)
+    # a reduction (workspace), a transpose and a matmul ride along in the same datagram
+    h.run(f"newtensor({V([200])})->({T('g_colsum')})")
+    h.run(f"newtensor({V([200, 300])})->({T('g_Gt')})")
+    h.run(f"newtensor({V([300, 300])})->({T('g_GGt')})")
+    extra = [f"sum({T('g_G')}, {V([0])}, var<bool>:false)->({T('g_colsum')}) // author=miaobyte id=3008",
+             f"transpose({T('g_G')}, {V([1, 0])})->({T('g_Gt')}) // author=miaobyte id=3009",
+             f"matmul({T('g_G')}, {T('g_Gt')})->({T('g_GGt')}) // author=cublas id=3010"]
+    lines = chain_lines("g_", 3000) + extra
+    outs = NAMES[2:] + ["colsum", "Gt", "GGt"]
+    for round_no in range(5):
+        a = rng.uniform(-1, 1, shape).astype(np.float32)
+        b = rng.uniform(-1, 1, shape).astype(np.float32)
+        h.put("g_A", a)   # load replaces an existing tensor by a fresh allocation: a recorded graph must notice
+        h.put("g_B", b)   # new addresses and record again, or replay if the allocator handed the old ones back
+        for line in lines:  # line by line: the expectation
+            assert ex.execute(line).split(" ")[1].startswith("ok")
+        want = {n: h.get("g_" + n) for n in outs}
+        for n in outs:
+            h.run(f"constant(var<float32>:0)->({T('g_' + n)})")
+        rs = ex.execute_batch(lines)
+        assert all(r.split(" ")[1].startswith("ok") for r in rs), rs
+        for n in outs:
+            got = h.get("g_" + n)
+            assert np.array_equal(got.view(np.uint32), want[n].view(np.uint32)), (round_no, n)
+    st = ex.stats()
+    assert st["rejects"] == 0 and st["captures"] >= 1 and st["captures"] + st["replays"] == 4, st
+
+
+def test_graph_replay_with_stable_addresses(tmp_path):
+    """Inputs refreshed in place (copytensor into the same allocation): the recorded graph is
+    replayed, not re-recorded, and every replay sees the new data."""
+    ex = InProc()
+    ex.set_graphs(True)
+    h = Host(ex, tmp_path)
+    rng = np.random.default_rng(43)
+    shape = [64, 96]
+    make_chain(h, "r_", shape, rng)
+    lines = chain_lines("r_", 4000)
+    for round_no in range(6):
+        h.put("r_stageA", rng.uniform(-1, 1, shape).astype(np.float32))
+        h.put("r_stageB", rng.uniform(-1, 1, shape).astype(np.float32))
+        h.run(f"copytensor({T('r_stageA')})->({T('r_A')})")
+        h.run(f"copytensor({T('r_stageB')})->({T('r_B')})")
+        for line in lines:
+            assert ex.execute(line).split(" ")[1].startswith("ok")
+        want = h.get("r_G")
+        h.run(f"constant(var<float32>:0)->({T('r_G')})")
+        assert all(r.split(" ")[1].startswith("ok") for r in ex.execute_batch(lines))
+        assert np.array_equal(h.get("r_G").view(np.uint32), want.view(np.uint32)), round_no
+    st = ex.stats()
+    assert st == {"batches": 6, "captures": 1, "replays": 4, "rejects": 0}, st
+
+
+def test_batches_that_must_not_be_recorded(tmp_path):
+    ex = InProc()
+    ex.set_graphs(True)
+    h = Host(ex, tmp_path)
+    h.put("n_A", np.arange(12, dtype=np.float32).reshape(3, 4))
+    h.run(f"newtensor({V([3, 4])})->({T('n_C')})")
+    h.run("argset(var<float32>:2)->(var<float32>:two)")
+    named = [f"mulscalar({T('n_A')}, var<float32>:two)->({T('n_C')}) // id=5001", f"addscalar({T('n_C')}, var<float32>:1)->({T('n_C')}) // id=5002"]
+    for _ in range(3):
+        assert all(r.split(" ")[1].startswith("ok") for r in ex.execute_batch(named))
+    assert np.array_equal(h.get("n_C"), np.arange(12, dtype=np.float32).reshape(3, 4) * 2 + 1)
+    h.run("argset(var<float32>:3)->(var<float32>:two)")  # the named scalar changes: a recorded graph would have frozen it
+    assert all(r.split(" ")[1].startswith("ok") for r in ex.execute_batch(named))
+    assert np.array_equal(h.get("n_C"), np.arange(12, dtype=np.float32).reshape(3, 4) * 3 + 1)
+    lifecycle = [f"newtensor({V([2, 2])})->({T('n_tmp')}) // id=5003", f"constant(var<float32>:7)->({T('n_tmp')}) // id=5004",
+                 f"deltensor()->({T('n_tmp')}) // id=5005"]
+    for _ in range(3):
+        assert all(r.split(" ")[1].startswith("ok") for r in ex.execute_batch(lifecycle))
+    failing = [f"add({T('n_A')}, {T('n_missing')})->({T('n_C')}) // id=5006", f"addscalar({T('n_A')}, var<float32>:1)->({T('n_C')}) // id=5007"]
+    for _ in range(3):
+        rs = ex.execute_batch(failing)
+        assert rs[0].endswith("tensor not found: n_missing") and rs[1].split(" ")[1].startswith("ok")
+    assert ex.stats()["captures"] == 0 and ex.stats()["replays"] == 0
+
+
+def test_graphs_over_udp(tmp_path):
+    srv = UdpExecutor(env={"DEEPX_GRAPH": "1"})
+    try:
+        rng = np.random.default_rng(44)
+        a, b = rng.uniform(-1, 1, (50, 70)).astype(np.float32), rng.uniform(-1, 1, (50, 70)).astype(np.float32)
+        for name, arr in (("u_A", a), ("u_B", b)):
+            p = str(tmp_path / name)
+            write_tensor(p, arr, "float32")
+            srv.must("load", [f"var<string>:{p}"], [], author="")
+        for n in NAMES[2:]:
+            srv.must("newtensor", [V([50, 70])], [T("u_" + n)], author="")
+        datagram = "\n".join(chain_lines("u_", 6000))
+        for _ in range(4):
+            srv.must("constant", ["var<float32>:0"], [T("u_G")])
+            rs = srv.raw(datagram, 8)
+            assert [r.id for r in rs] == [str(6000 + i) for i in range(8)] and all(r.ok for r in rs)
+            p = str(tmp_path / "u_G_out")
+            srv.must("save", [T("u_G", "any"), f"var<string>:{p}"], [], author="")
+            f = np.exp((a + b) * b + np.float32(0.5))
+            want = f / (np.maximum(b, -b) + np.float32(1))
+            got = read_tensor(p)[0]
+            assert np.allclose(got, want, rtol=1e-6, atol=0)
+    finally:
+        srv.close()
+    assert srv.proc.returncode == 0

@@ -100,10 +100,49 @@ public:
         if (lines.size() == 1) return {execute(lines[0], recv_at)};
         std::lock_guard<std::mutex> lock(mu_);
         ++stats.batches;
+        // graphs are keyed by the instruction text without the per-call metadata (ids, timestamps)
+        std::string key;
+        for (const std::string &line : lines) {
+            size_t end = line.find("//");
+            if (end == std::string::npos) end = line.size();
+            while (end > 0 && line[end - 1] == ' ') --end;
+            key.append(line, 0, end);
+            key += '\n';
+        }
+        if (use_graphs && has_device) {  // a batch recorded earlier whose tensors are all where they were: no parsing at all
+            auto hit = graphs_.find(key);
+            if (hit != graphs_.end() && pins_hold(hit->second)) {
+                std::vector<int> ids;
+                bool plain = true;  // ids readable, no benchmark.repeat: otherwise take the parsing path
+                try {
+                    for (const std::string &line : lines) {
+                        TFMetadata m;
+                        size_t meta = line.find("//");
+                        if (meta != std::string::npos) m.parse(line.substr(meta + 2));
+                        plain = plain && m.benchmark_repeat <= 1;
+                        ids.push_back(m.id);
+                    }
+                } catch (const std::exception &) {
+                    plain = false;
+                }
+                if (plain && launch_graph(hit->second)) {
+                    ++stats.graph_replays;
+                    std::vector<std::string> replies;
+                    replies.reserve(lines.size());
+                    for (int id : ids) {
+                        OpResp resp;
+                        resp.recv_at = resp.start_at = recv_at;
+                        resp.id = id;
+                        resp.finish("");
+                        replies.push_back(resp.to_string());
+                    }
+                    return replies;
+                }
+            }
+        }
         struct Item { TF call; std::shared_ptr<TF> tf; OpResp resp; bool failed = false; };
         std::vector<Item> items(lines.size());
         bool graphable = use_graphs && has_device;
-        std::string key;
         for (size_t i = 0; i < lines.size(); ++i) {
             Item &it = items[i];
             it.resp.recv_at = it.resp.start_at = recv_at;
@@ -131,8 +170,6 @@ public:
             it.tf->args = it.call.args;
             it.tf->returns = it.call.returns;
             graphable = graphable && it.tf->graph_safe && it.tf->metadata.benchmark_repeat <= 1 && !uses_named_arg(it.call);
-            key += it.call.to_string(false);
-            key += '\n';
         }
         bool done = false;
         if (graphable) {
@@ -211,6 +248,17 @@ private:
         }
         g.workspace = mem.workspace_ptr();
         return true;
+    }
+    bool pins_hold(const Graph &g) const {
+        if (g.workspace != mem.workspace_ptr()) return false;
+        for (const Pinned &p : g.tensors) {
+            auto t = mem.findtensor(p.name);
+            if (!t || t->data != p.data || t->shape.bytes() != p.bytes || t->dtype() != p.dtype) return false;
+        }
+        return true;
+    }
+    bool launch_graph(const Graph &g) {
+        return dxh_graph_launch(g.exec, graph_stream_) == DXH_OK && dxh_stream_sync(graph_stream_) == DXH_OK;
     }
     static bool same_pins(const Graph &a, const Graph &b) {
         if (a.workspace != b.workspace || a.tensors.size() != b.tensors.size()) return false;

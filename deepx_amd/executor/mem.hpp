@@ -51,6 +51,10 @@ public:
         if (it == tensors_.end()) throw std::runtime_error("tensor not found: " + name);
         return it->second;
     }
+    std::shared_ptr<Tensor> findtensor(const std::string &name) const {  // nullptr instead of throwing
+        auto it = tensors_.find(name);
+        return it == tensors_.end() ? nullptr : it->second;
+    }
     // like MemBase::addtensor, an existing name is kept (mem.hpp:66-99) and reported
     bool addtensor(const std::string &name, std::shared_ptr<Tensor> t) { return tensors_.emplace(name, std::move(t)).second; }
     void delete_tensor(const std::string &name) { tensors_.erase(name); }

@@ -29,7 +29,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 MFMA_F32_PEAK_TF = 157.3
 MFMA_BF16_PEAK_TF = 2500.0  # dense bf16
-REDUCE_ROW_TRAFFIC_BYTES = 268646159  # measured, see profiles/bench_pmc_hbm_traffic.md
+REDUCE_ROW_TRAFFIC_BYTES = 268646271  # measured, see profiles/bench_pmc_hbm_traffic.md
 
 
 def main():
@@ -280,6 +280,7 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
         Bm = (torch.randn(kk * nn, device=dev) * 0.02).to(torch.bfloat16)
         Cm = torch.empty(mm * nn, device=dev, dtype=torch.bfloat16)
         c5[label] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_matmul(dx.BF16, ptr(Am), ptr(Bm), ptr(Cm), 1, mm, kk, nn, None)), flops=2 * mm * kk * nn)
+        c5[label]["hipblaslt_TFLOP/s"] = vendor_gemm_tflops(torch, Am.view(mm, kk), Bm.view(kk, nn), Cm.view(mm, nn))
     # the same shapes in fp32, the dtype the reference's own matmul (cublasSgemm / cblas_sgemm) runs in
     for label, (mm, kk, nn) in [("matmul_f32_2048x896x4864", (2048, 896, 4864)), ("matmul_f32_2048x4864x896", (2048, 4864, 896))]:
         Am = torch.randn(mm * kk, device=dev)
@@ -287,8 +288,25 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
         Cm = torch.empty(mm * nn, device=dev)
         c5[label] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_matmul(dx.F32, ptr(Am), ptr(Bm), ptr(Cm), 1, mm, kk, nn, None)),
                           flops=2 * mm * kk * nn, peak_tf=MFMA_F32_PEAK_TF, peak_name="frac_mfma_f32")
+        c5[label]["hipblaslt_TFLOP/s"] = vendor_gemm_tflops(torch, Am.view(mm, kk), Bm.view(kk, nn), Cm.view(mm, nn))
     res["config5"] = c5
     return res
+
+
+def vendor_gemm_tflops(torch, A, B, C, reps=20, warm=5):
+    """torch.matmul (hipBLASLt / rocBLAS) on the same operands, for context next to our kernel's rate.
+    Timed with torch's own events on torch's current stream, which is where torch launches it."""
+    for _ in range(warm):
+        torch.matmul(A, B, out=C)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        torch.matmul(A, B, out=C)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    return round(2.0 * A.shape[0] * A.shape[1] * B.shape[1] / ms / 1e9, 2)
 
 
 def cpu_baseline(np, dx):

@@ -10,6 +10,13 @@ from tests.executor_client import InProc, UdpExecutor, read_tensor, write_tensor
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _torch_owns_the_hip_runtime(dxh):
+    """The in-process executor pulls in the HIP runtime; torch must have loaded its own copy first
+    (the session fixture imports torch), or a later torch import in this process finds no GPU."""
+    yield
+
+
 def T(name, dt="float32"):
     return f"tensor<{dt}>:{name}"
 

@@ -167,6 +167,7 @@ template <typename T, int TM, int TN, int PD>
 __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul_mfma_tile_kernel(
     const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int K, int N, int tiles_m, int tiles_n,
     int total_tiles, int chunk, int group_m) {
+    static_assert(TM % 64 == 0 && (TN == 64 || TN == 128 || TN == 256), "B rows must split evenly over the 256 lanes");
     constexpr int FM = TM / 64, FN = TN / 64;      // 32x32 MFMA tiles per wave along m and n
     constexpr int A_LD = TM / 32, B_LD = TN / 32;  // 16-byte global loads per lane per K step
     constexpr int CB = TN / 8;                     // 16-byte chunks per B row

@@ -8,7 +8,8 @@
 //                256x256 workgroup tiles, software-pipelined over K.  Anything else:
 //                matmul_mfma_kernel, a plain 128x128x32 tile with element-wise edge handling.
 //   f32          MFMA v_mfma_f32_32x32x2_f32 (fp32 operands and accumulate): matmul_mfma_f32_kernel.
-//   f64 / integers   LDS-tiled 64x64x16 FMA kernel, 4x4 outputs per lane; accumulate in the
+//   f64          MFMA v_mfma_f64_16x16x4_f64: matmul_mfma_f64_kernel.
+//   integers     LDS-tiled 64x64x16 multiply-add kernel, 4x4 outputs per lane; accumulate in the
 //                storage type (integers wrap).
 #include "common.hpp"
 
@@ -499,6 +500,126 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
     });
 }
 
+// ---- fp64 MFMA kernel ------------------------------------------------------------------------
+// v_mfma_f64_16x16x4_f64 (78.6 TFLOP/s peak, 64 cycles each): lane L supplies A[row L%16][k L/16]
+// and B[k L/16][col L%16]; the result lane holds D[4v + L/16][L%16] in register v.  Same plan as
+// the fp32 kernel: workgroup tile (64 FM) x (64 FN), K step 16, 4 waves 2x2, each wave
+// (2 FM) x (2 FN) MFMA tiles, double-buffered LDS with one K step prefetched in registers.  MFMA e
+// of lane class q = L/16 multiplies k = 4q + e, so a lane reads its four A values of a K step as
+// two 16-byte LDS loads.  Result rows are contiguous over 16 lanes: plain 8-byte stores coalesce.
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+template <int FM, int FN, bool VEC>
+__global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double *__restrict__ A, const double *__restrict__ B,
+                                                                    double *__restrict__ C, int M, int K, int N, int tiles_m,
+                                                                    int tiles_n) {
+    constexpr int DK = 16, TM = 64 * FM, TN = 64 * FN, DA_ROW = DK + 2, DB_ROW = TN + 4;
+    constexpr int STAGE = TM * DA_ROW + DK * DB_ROW;  // doubles
+    constexpr int CA = DK / 2, CB = TN / 2;           // 16-byte chunks per A row / B row
+    constexpr int A_LD = TM * CA / kBlock, B_LD = DK * CB / kBlock;
+    constexpr int RT = 2 * FM, CT = 2 * FN;           // 16x16 MFMA tiles per wave along m and n
+    __shared__ __attribute__((aligned(16))) double lds[2 * STAGE];
+    int64_t bid = blockIdx.x;
+    const int tn = (int)(bid % tiles_n); bid /= tiles_n;
+    const int tm = (int)(bid % tiles_m); bid /= tiles_m;
+    A += bid * (int64_t)M * K;
+    B += bid * (int64_t)K * N;
+    C += bid * (int64_t)M * N;
+    const int m0 = tm * TM, n0 = tn * TN;
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
+
+    f64x2 ra[A_LD], rb[B_LD];
+    auto load_global = [&](int k0) __attribute__((always_inline)) {
+        static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i, row = id / CA, kk = k0 + (id % CA) * 2, gm = m0 + row;
+            if constexpr (VEC) {
+                const double *p = A + (int64_t)(gm < M ? gm : M - 1) * K + (kk < K ? kk : 0);
+                f64x2 v = *reinterpret_cast<const f64x2 *>(p);
+                ra[i] = (kk < K) ? v : f64x2{0.0, 0.0};
+            } else {
+                f64x2 v;
+#pragma unroll
+                for (int e = 0; e < 2; ++e) v[e] = (gm < M && kk + e < K) ? A[(int64_t)gm * K + kk + e] : 0.0;
+                ra[i] = v;
+            }
+        });
+        static_for<B_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i, krow = id / CB, gk = k0 + krow, gn = n0 + (id % CB) * 2;
+            if constexpr (VEC) {
+                const double *p = B + (int64_t)(gk < K ? gk : 0) * N + (gn < N ? gn : N - 2);
+                f64x2 v = *reinterpret_cast<const f64x2 *>(p);
+                rb[i] = (gk < K) ? v : f64x2{0.0, 0.0};
+            } else {
+                f64x2 v;
+#pragma unroll
+                for (int e = 0; e < 2; ++e) v[e] = (gk < K && gn + e < N) ? B[(int64_t)gk * N + gn + e] : 0.0;
+                rb[i] = v;
+            }
+        });
+    };
+    auto store_lds = [&](int stage) __attribute__((always_inline)) {
+        double *As = lds + stage * STAGE, *Bs = As + TM * DA_ROW;
+        static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i;
+            *reinterpret_cast<f64x2 *>(As + (id / CA) * DA_ROW + (id % CA) * 2) = ra[i];
+        });
+        static_for<B_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i;
+            *reinterpret_cast<f64x2 *>(Bs + (id / CB) * DB_ROW + (id % CB) * 2) = rb[i];
+        });
+    };
+
+    f64x4 acc[RT][CT];
+    static_for<RT>([&](auto i) __attribute__((always_inline)) {
+        static_for<CT>([&](auto j) __attribute__((always_inline)) { acc[i][j] = f64x4{0.0, 0.0, 0.0, 0.0}; });
+    });
+    const int q = lane >> 4, l16 = lane & 15;
+    auto compute = [&](int stage) __attribute__((always_inline)) {
+        const double *As = lds + stage * STAGE, *Bs = As + TM * DA_ROW;
+        f64x2 fa[RT][2];
+        double fb[CT][4];
+        static_for<RT>([&](auto i) __attribute__((always_inline)) {
+            const double *p = As + (wm * 32 * FM + 16 * i + l16) * DA_ROW + 4 * q;
+            fa[i][0] = *reinterpret_cast<const f64x2 *>(p);
+            fa[i][1] = *reinterpret_cast<const f64x2 *>(p + 2);
+        });
+        static_for<CT>([&](auto j) __attribute__((always_inline)) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) fb[j][e] = Bs[(4 * q + e) * DB_ROW + wn * 32 * FN + 16 * j + l16];
+        });
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            static_for<RT>([&](auto i) __attribute__((always_inline)) {
+                static_for<CT>([&](auto j) __attribute__((always_inline)) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[i][e >> 1][e & 1], fb[j][e], acc[i][j], 0, 0, 0);
+                });
+            });
+    };
+
+    const int KT = (K + DK - 1) / DK;
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const bool more = kt + 1 < KT;
+        if (more) load_global((kt + 1) * DK);
+        compute(kt & 1);
+        if (more) store_lds((kt + 1) & 1);
+        __syncthreads();
+    }
+
+    static_for<RT>([&](auto i) __attribute__((always_inline)) {
+        static_for<CT>([&](auto j) __attribute__((always_inline)) {
+            const int gn = n0 + wn * 32 * FN + 16 * j + l16;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int gm = m0 + wm * 32 * FM + 16 * i + 4 * v + q;
+                if (gm < M && gn < N) __builtin_nontemporal_store(acc[i][j][v], C + (int64_t)gm * N + gn);
+            }
+        });
+    });
+}
+
 // ---- generic tiled kernel (f32, f64, integers) ------------------------------------------
 constexpr int GT = 64, GK = 16;
 template <typename T>
@@ -678,6 +799,39 @@ inline int launch_f32(const void *a, const void *b, void *c, int64_t batch, int6
     }
 }
 
+template <int FM, int FN>
+int launch_f64_tile(const double *a, const double *b, double *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, hipStream_t st) {
+    const int64_t tiles_m = (m + 64 * FM - 1) / (64 * FM), tiles_n = (n + 64 * FN - 1) / (64 * FN), blocks = batch * tiles_m * tiles_n;
+    if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
+    if (vec) matmul_mfma_f64_kernel<FM, FN, true><<<(unsigned)blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
+    else matmul_mfma_f64_kernel<FM, FN, false><<<(unsigned)blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
+    return launch_status();
+}
+
+// fp64 on the matrix pipe; tile chosen for CU balance like fp32 (efficiencies measured on 4096^3)
+inline int launch_f64(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    const bool vec = k % 2 == 0 && n % 2 == 0 && n >= 2 && aligned(a, kVecBytes) && aligned(b, kVecBytes);
+    const int64_t cus = compute_units();
+    auto cost = [&](int tm, int tn, double eff) {
+        const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn);
+        const int64_t full = tiles / (2 * cus), rem = tiles % (2 * cus);
+        const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.6 : 0.0);
+        return rounds * (double)tm * (double)tn / eff;
+    };
+    const double *af = (const double *)a, *bf = (const double *)b;
+    double *cf = (double *)c;
+    int64_t choice = tuning().matmul_tile;
+    if (choice == 0) {
+        const double c1 = cost(128, 128, 1.0), c2 = cost(128, 64, 0.86), c3 = cost(64, 64, 0.95);
+        choice = (c1 <= c2 && c1 <= c3) ? 1 : (c2 <= c3) ? 2 : 3;
+    }
+    switch (choice) {
+    case 1: return launch_f64_tile<2, 2>(af, bf, cf, batch, m, k, n, vec, st);
+    case 2: return launch_f64_tile<2, 1>(af, bf, cf, batch, m, k, n, vec, st);
+    default: return launch_f64_tile<1, 1>(af, bf, cf, batch, m, k, n, vec, st);
+    }
+}
+
 }  // namespace dxh
 
 using namespace dxh;
@@ -701,7 +855,7 @@ extern "C" int dxh_matmul(int dtype, const void *a, const void *b, void *c, int6
     case DXH_BF16: return launch_mfma<bf16_t>(a, b, c, batch, m, k, n, st);
     case DXH_F16: return launch_mfma<f16_t>(a, b, c, batch, m, k, n, st);
     case DXH_F32: return launch_f32(a, b, c, batch, m, k, n, st);
-    case DXH_F64: return launch_tiled<double>(a, b, c, batch, m, k, n, st);
+    case DXH_F64: return launch_f64(a, b, c, batch, m, k, n, st);
     case DXH_I64: return launch_tiled<int64_t>(a, b, c, batch, m, k, n, st);
     case DXH_I32: return launch_tiled<int32_t>(a, b, c, batch, m, k, n, st);
     case DXH_I16: return launch_tiled<int16_t>(a, b, c, batch, m, k, n, st);

@@ -156,3 +156,31 @@ def test_matmul_f32_tile_configs(dxh, tile):
         assert np.array_equal(dC.get().reshape(m, n), (Ai @ Bi).astype(np.float32))
     finally:
         dx.check(dxh.dxh_tune(TILE_KNOB, 0))
+
+
+@pytest.mark.parametrize("tile", [1, 2, 3])
+def test_matmul_f64_tile_configs(dxh, tile):
+    """Every tile of the fp64 matrix-pipe kernel: vector path (even K, N), element-wise path (odd
+    K / N), ragged edges, batches, K not a multiple of the K step.  Bar: rel 1e-13*sqrt(K) of
+    sum_k |a||b| against numpy's float64 product (a different summation order), and exact on
+    small integers."""
+    rng = np.random.default_rng(600 + tile)
+    dx.check(dxh.dxh_tune(TILE_KNOB, tile))
+    try:
+        for batch, m, k, n in [(2, 300, 128, 264), (1, 130, 100, 68), (3, 70, 33, 9), (1, 257, 64, 1030), (1, 1, 2, 2),
+                               (1, 520, 1000, 260), (2, 65, 7, 129)]:
+            A = rng.standard_normal(batch * m * k)
+            B = rng.standard_normal(batch * k * n)
+            dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, np.float64)
+            dx.check(dxh.dxh_matmul(dx.F64, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+            got = dC.get().reshape(batch, m, n)
+            Af, Bf = A.reshape(batch, m, k), B.reshape(batch, k, n)
+            ref, mag = np.matmul(Af, Bf), np.matmul(np.abs(Af), np.abs(Bf))
+            assert np.all(np.abs(got - ref) <= 1e-13 * np.sqrt(k) * np.maximum(mag, 1e-300)), (tile, batch, m, k, n)
+        m, k, n = 200, 96, 132
+        Ai, Bi = rng.integers(-1000, 1001, (m, k)), rng.integers(-1000, 1001, (k, n))
+        dA, dB, dC = Dev(Ai.astype(np.float64).reshape(-1)), Dev(Bi.astype(np.float64).reshape(-1)), Dev.empty(m * n, np.float64)
+        dx.check(dxh.dxh_matmul(dx.F64, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+        assert np.array_equal(dC.get().reshape(m, n), (Ai @ Bi).astype(np.float64))
+    finally:
+        dx.check(dxh.dxh_tune(TILE_KNOB, 0))

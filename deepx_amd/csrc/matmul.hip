@@ -122,6 +122,40 @@ __global__ __launch_bounds__(kBlock) void matmul_mfma_kernel(const T *__restrict
 constexpr int PK = 64;  // K step of the MFMA tile kernel
 __device__ inline int swz(int row, int chunk) { return chunk ^ ((row ^ (row >> 3)) & 7); }
 
+// ---- XCD-aware workgroup -> tile map (shared by the MFMA kernels) ---------------------------
+// Workgroups are dealt round-robin to the 8 XCDs, each with a private L2.  XCD x takes the
+// contiguous range [x*chunk, (x+1)*chunk) of a grouped tile order (group_m tile rows at a time,
+// column-major inside a group), i.e. a compact, roughly square patch of C whose A and B panels
+// fit its L2.  The grid is 8*chunk workgroups; those past the last tile exit at once.
+struct TileMap { int tiles_m, tiles_n, total, chunk, group_m; };
+struct TileCoord { int batch, tm, tn; bool valid; };
+inline bool make_tile_map(int64_t batch, int64_t m, int64_t n, int tm, int tn, TileMap &map) {
+    const int64_t tiles_m = (m + tm - 1) / tm, tiles_n = (n + tn - 1) / tn, total = batch * tiles_m * tiles_n;
+    if (total > 0x0fffffff) return false;
+    map.tiles_m = (int)tiles_m; map.tiles_n = (int)tiles_n; map.total = (int)total;
+    map.chunk = (int)((total + 7) / 8);
+    int group_m = 1;  // tile rows per group: the chunk of one XCD should cover a roughly square patch of C
+    while ((int64_t)(group_m + 1) * (group_m + 1) * tm <= (int64_t)map.chunk * tn && group_m + 1 <= tiles_m) ++group_m;
+    map.group_m = group_m;
+    return true;
+}
+__device__ __forceinline__ TileCoord tile_of_block(const TileMap &map) {
+    TileCoord c;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    int logical = xcd * map.chunk + slot;
+    c.valid = logical < map.total;
+    const int per_batch = map.tiles_m * map.tiles_n;
+    c.batch = logical / per_batch;
+    logical -= c.batch * per_batch;
+    const int in_group = map.group_m * map.tiles_n;
+    const int first_m = (logical / in_group) * map.group_m;
+    const int size_m = (map.tiles_m - first_m < map.group_m) ? map.tiles_m - first_m : map.group_m;
+    const int within = logical % in_group;
+    c.tm = first_m + within % size_m;
+    c.tn = within / size_m;
+    return c;
+}
+
 // ---- MFMA kernel with the B transposition done by the LDS read ------------------------------
 // Workgroup tile TM x TN (64, 128 or 256 each), K step 64, 4 waves in a 2x2 grid, each wave a
 // (TM/2) x (TN/2) patch of 32x32x16 MFMAs.  Requirements (checked by the launcher): K % 64 == 0,
@@ -135,9 +169,7 @@ __device__ inline int swz(int row, int chunk) { return chunk ^ ((row ^ (row >> 3
 //          into the next stage and the global loads are spread over the four k-substeps.
 //   roles  the MFMA runs on (B^T, A^T): a lane of the result then holds 4 consecutive n of one row
 //          m, which packs into 8-byte LDS stores for the epilogue.
-//   map    blockIdx -> tile is XCD-aware: workgroups are dealt round-robin to the 8 XCDs, so XCD x
-//          takes the contiguous tile range [x*chunk, (x+1)*chunk) of a grouped (group_m tile rows
-//          at a time) ordering and its private L2 sees a compact set of A and B panels.
+//   map    blockIdx -> tile through tile_of_block (XCD-aware, above).
 template <typename F, int... I>
 __device__ __forceinline__ void static_for_impl(F &f, std::integer_sequence<int, I...>) { (f(std::integral_constant<int, I>{}), ...); }
 template <int N, typename F> __device__ __forceinline__ void static_for(F f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
@@ -166,8 +198,7 @@ constexpr int part_count(int count, int part) { return count * (part + 1) / 4 - 
 
 template <typename T, int TM, int TN, int PD>
 __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul_mfma_tile_kernel(
-    const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int K, int N, int tiles_m, int tiles_n,
-    int total_tiles, int chunk, int group_m) {
+    const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int K, int N, TileMap map) {
     static_assert(TM % 64 == 0 && (TN == 64 || TN == 128 || TN == 256), "B rows must split evenly over the 256 lanes");
     constexpr int FM = TM / 64, FN = TN / 64;      // 32x32 MFMA tiles per wave along m and n
     constexpr int A_LD = TM / 32, B_LD = TN / 32;  // 16-byte global loads per lane per K step
@@ -179,17 +210,9 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
     constexpr int LDS_ELEMS = (2 * STAGE > TM * LDC) ? 2 * STAGE : TM * LDC;
     __shared__ __attribute__((aligned(16))) uint16_t lds[LDS_ELEMS];
 
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    int logical = xcd * chunk + slot;
-    if (logical >= total_tiles) return;
-    const int per_batch = tiles_m * tiles_n;
-    const int batch = logical / per_batch;
-    logical -= batch * per_batch;
-    const int in_group = group_m * tiles_n;
-    const int first_m = (logical / in_group) * group_m;
-    const int size_m = (tiles_m - first_m < group_m) ? tiles_m - first_m : group_m;
-    const int within = logical % in_group;
-    const int tm = first_m + within % size_m, tn = within / size_m;
+    const TileCoord tc = tile_of_block(map);
+    if (!tc.valid) return;
+    const int batch = tc.batch, tm = tc.tm, tn = tc.tn;
     const int m0 = tm * TM, n0 = tn * TN;
 
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
@@ -364,8 +387,7 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
 //          clamped rows/columns; otherwise element-wise accesses with bounds checks.
 template <int FM, int FN, int FK, int PD, bool VEC>
 __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float *__restrict__ A, const float *__restrict__ B,
-                                                                    float *__restrict__ C, int M, int K, int N, int tiles_m,
-                                                                    int tiles_n) {
+                                                                    float *__restrict__ C, int M, int K, int N, TileMap map) {
     constexpr int TM = 64 * FM, TN = 64 * FN, FA_ROW = FK + 4, FB_ROW = TN + 4;
     constexpr int STAGE = TM * FA_ROW + FK * FB_ROW;  // floats
     constexpr int CA = FK / 4, CB = TN / 4;           // 16-byte chunks per A row / B row
@@ -373,12 +395,12 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
     constexpr int HK = FK / 2;                        // k values per lane half
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     __shared__ __attribute__((aligned(16))) float lds[2 * STAGE];
-    int64_t bid = blockIdx.x;
-    const int tn = (int)(bid % tiles_n); bid /= tiles_n;
-    const int tm = (int)(bid % tiles_m); bid /= tiles_m;
-    A += bid * (int64_t)M * K;
-    B += bid * (int64_t)K * N;
-    C += bid * (int64_t)M * N;
+    const TileCoord tc = tile_of_block(map);
+    if (!tc.valid) return;
+    const int tm = tc.tm, tn = tc.tn;
+    A += tc.batch * (int64_t)M * K;
+    B += tc.batch * (int64_t)K * N;
+    C += tc.batch * (int64_t)M * N;
     const int m0 = tm * TM, n0 = tn * TN;
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
 
@@ -511,20 +533,19 @@ typedef double f64x4 __attribute__((ext_vector_type(4)));
 typedef double f64x2 __attribute__((ext_vector_type(2)));
 template <int FM, int FN, bool VEC>
 __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double *__restrict__ A, const double *__restrict__ B,
-                                                                    double *__restrict__ C, int M, int K, int N, int tiles_m,
-                                                                    int tiles_n) {
+                                                                    double *__restrict__ C, int M, int K, int N, TileMap map) {
     constexpr int DK = 16, TM = 64 * FM, TN = 64 * FN, DA_ROW = DK + 2, DB_ROW = TN + 4;
     constexpr int STAGE = TM * DA_ROW + DK * DB_ROW;  // doubles
     constexpr int CA = DK / 2, CB = TN / 2;           // 16-byte chunks per A row / B row
     constexpr int A_LD = TM * CA / kBlock, B_LD = DK * CB / kBlock;
     constexpr int RT = 2 * FM, CT = 2 * FN;           // 16x16 MFMA tiles per wave along m and n
     __shared__ __attribute__((aligned(16))) double lds[2 * STAGE];
-    int64_t bid = blockIdx.x;
-    const int tn = (int)(bid % tiles_n); bid /= tiles_n;
-    const int tm = (int)(bid % tiles_m); bid /= tiles_m;
-    A += bid * (int64_t)M * K;
-    B += bid * (int64_t)K * N;
-    C += bid * (int64_t)M * N;
+    const TileCoord tc = tile_of_block(map);
+    if (!tc.valid) return;
+    const int tm = tc.tm, tn = tc.tn;
+    A += tc.batch * (int64_t)M * K;
+    B += tc.batch * (int64_t)K * N;
+    C += tc.batch * (int64_t)M * N;
     const int m0 = tm * TM, n0 = tn * TN;
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
 
@@ -688,14 +709,9 @@ __global__ __launch_bounds__(kBlock) void matmul_tiled_kernel(const T *__restric
 
 template <typename T, int TM, int TN, int PD>
 int launch_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    const int64_t tiles_m = (m + TM - 1) / TM, tiles_n = (n + TN - 1) / TN, total = batch * tiles_m * tiles_n;
-    if (total > 0x0fffffff) return DXH_ERR_SHAPE;
-    const int chunk = (int)((total + 7) / 8);  // tiles per XCD
-    // tile rows per group: the chunk of one XCD should cover a roughly square patch of C
-    int group_m = 1;
-    while ((int64_t)(group_m + 1) * (group_m + 1) * TM <= (int64_t)chunk * TN && group_m + 1 <= tiles_m) ++group_m;
-    matmul_mfma_tile_kernel<T, TM, TN, PD><<<(unsigned)(8 * chunk), kBlock, 0, st>>>(
-        (const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n, (int)total, chunk, group_m);
+    TileMap map;
+    if (!make_tile_map(batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
+    matmul_mfma_tile_kernel<T, TM, TN, PD><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map);
     return launch_status();
 }
 
@@ -761,10 +777,11 @@ int launch_tiled(const void *a, const void *b, void *c, int64_t batch, int64_t m
 
 template <int FM, int FN, int FK, int PD>
 int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, hipStream_t st) {
-    const int64_t tiles_m = (m + 64 * FM - 1) / (64 * FM), tiles_n = (n + 64 * FN - 1) / (64 * FN), blocks = batch * tiles_m * tiles_n;
-    if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
-    if (vec) matmul_mfma_f32_kernel<FM, FN, FK, PD, true><<<(unsigned)blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
-    else matmul_mfma_f32_kernel<FM, FN, FK, PD, false><<<(unsigned)blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
+    TileMap map;
+    if (!make_tile_map(batch, m, n, 64 * FM, 64 * FN, map)) return DXH_ERR_SHAPE;
+    const unsigned blocks = (unsigned)(8 * map.chunk);
+    if (vec) matmul_mfma_f32_kernel<FM, FN, FK, PD, true><<<blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, map);
+    else matmul_mfma_f32_kernel<FM, FN, FK, PD, false><<<blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, map);
     return launch_status();
 }
 
@@ -801,10 +818,11 @@ inline int launch_f32(const void *a, const void *b, void *c, int64_t batch, int6
 
 template <int FM, int FN>
 int launch_f64_tile(const double *a, const double *b, double *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, hipStream_t st) {
-    const int64_t tiles_m = (m + 64 * FM - 1) / (64 * FM), tiles_n = (n + 64 * FN - 1) / (64 * FN), blocks = batch * tiles_m * tiles_n;
-    if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
-    if (vec) matmul_mfma_f64_kernel<FM, FN, true><<<(unsigned)blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
-    else matmul_mfma_f64_kernel<FM, FN, false><<<(unsigned)blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n);
+    TileMap map;
+    if (!make_tile_map(batch, m, n, 64 * FM, 64 * FN, map)) return DXH_ERR_SHAPE;
+    const unsigned blocks = (unsigned)(8 * map.chunk);
+    if (vec) matmul_mfma_f64_kernel<FM, FN, true><<<blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, map);
+    else matmul_mfma_f64_kernel<FM, FN, false><<<blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, map);
     return launch_status();
 }
 

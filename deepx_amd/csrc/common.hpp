@@ -93,6 +93,7 @@ struct Tuning {
                                                   // walking its rows with software-pipelined loads
     int64_t reduce_col_min_rows = 16;             // DXH_TUNE_REDUCE_COL_MIN_ROWS
     int64_t reduce_col_max_lanes = 128;           // DXH_TUNE_REDUCE_COL_MAX_LANES
+    int64_t reduce_row_loads = 4;                 // DXH_TUNE_REDUCE_ROW_LOADS: vectors per lane a row group aims for
     int64_t matmul_tile = 0;                      // DXH_TUNE_MATMUL_TILE: 0 = chosen per shape
 };
 Tuning &tuning();  // runtime.hip

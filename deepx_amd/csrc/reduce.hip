@@ -339,7 +339,13 @@ inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, cons
         if (st.row) {
             // lanes per row: one 16-byte vector per lane per trip, up to the whole workgroup
             int64_t vecs = (R + vfull - 1) / vfull;
-            int G = vecs >= 2 * kWave ? kBlock : (int)std::min<int64_t>(kWave, pow2_ceil(vecs));
+            // each lane should have several independent 16-byte loads of its own: the whole
+            // workgroup on one row only when that still leaves `loads` vectors per lane, else a
+            // sub-wave group of lanes per row and 256/G rows per workgroup
+            const int64_t loads = tuning().reduce_row_loads;
+            int G = vecs >= (int64_t)kBlock * loads ? kBlock : (int)std::min<int64_t>(kWave, pow2_ceil((vecs + loads - 1) / loads));
+            // very short rows: at least 4 lanes (64 contiguous bytes) per row keep a wave's loads coalesced
+            G = std::max<int>(G, (int)std::min<int64_t>(4, pow2_ceil(vecs)));
             int64_t blocks0 = (pre + (kBlock / G) - 1) / (kBlock / G);
             if (G == kBlock && blocks0 < kTarget) {
                 int64_t min_chunk = 8192;  // elements: 8+ vector trips per lane

@@ -28,6 +28,7 @@ int dxh_tune(int knob, int64_t value) {
         if (value != 4 && value != 8 && value != 16 && value != 32 && value != 64 && value != 128 && value != 256) return DXH_ERR_ARG;
         t.reduce_col_max_lanes = value;
         return DXH_OK;
+    case DXH_TUNE_REDUCE_ROW_LOADS: if (value < 1 || value > 64) return DXH_ERR_ARG; t.reduce_row_loads = value; return DXH_OK;
     case DXH_TUNE_MATMUL_TILE: if (value < 0 || value > 5) return DXH_ERR_ARG; t.matmul_tile = value; return DXH_OK;
     default: return DXH_ERR_ARG;
     }

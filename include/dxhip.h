@@ -89,6 +89,7 @@ enum dxh_tune_knob {
     DXH_TUNE_REDUCE_TARGET_BLOCKS = 1, /* workgroups a reduction stage aims for before it stops splitting R */
     DXH_TUNE_REDUCE_COL_MIN_ROWS = 2,  /* strided-axis stage: fewest rows per lane when R is split */
     DXH_TUNE_REDUCE_COL_MAX_LANES = 3, /* strided-axis stage: widest column-lane count (16..256) */
+    DXH_TUNE_REDUCE_ROW_LOADS = 5,     /* contiguous-axis stage: 16-byte loads per lane a row's lane group aims for */
     DXH_TUNE_MATMUL_TILE = 4           /* matmul workgroup tile, 0 = chosen per shape; bf16/f16: 1 128x128, 2 128x64, 3 64x128,
                                           4 256x256, 5 64x64; f32: 1 128x128, 2 128x64, 3 64x64, 4 128x128 with K step 16 */
 };

@@ -217,6 +217,95 @@ __global__ __launch_bounds__(kBlock) void tile_transpose_kernel(const E *__restr
     }
 }
 
+// ---- tile_transpose, 16-byte version ----------------------------------------------------
+// Same (A, C) view, for elements of ES bytes with V = 16/ES of them per 16-byte vector; needs nA,
+// nC and every stride to be multiples of V and 16-byte aligned bases.  Tile = (16 V) x (16 V)
+// elements, so that both the input rows (along C) and the output rows (along A) are touched in
+// 256-byte runs by 16 lanes.  Each lane owns one V x V block: it loads V input rows of 16 bytes,
+// transposes the block in registers (relabelling for 4/8-byte elements, v_perm_b32 for 2/1-byte
+// ones) into V output vectors, and passes them through LDS to the lane that stores them, so all
+// global and LDS traffic is in 16-byte units.  The LDS slot of an a-block is XORed with the
+// c-block, which keeps both the stores (16 lanes, same a-block) and the loads conflict free.
+typedef uint32_t tt_u32x4 __attribute__((ext_vector_type(4)));
+
+template <int ES> __device__ __forceinline__ void transpose_block(const tt_u32x4 (&rows)[16 / ES], tt_u32x4 (&cols)[16 / ES]) {
+    constexpr int V = 16 / ES;
+    if constexpr (ES == 16) {
+        cols[0] = rows[0];
+    } else if constexpr (ES == 8) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) cols[j] = tt_u32x4{rows[0][2 * j], rows[0][2 * j + 1], rows[1][2 * j], rows[1][2 * j + 1]};
+    } else if constexpr (ES == 4) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) cols[j] = tt_u32x4{rows[0][j], rows[1][j], rows[2][j], rows[3][j]};
+    } else if constexpr (ES == 2) {
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                cols[j][d] = __builtin_amdgcn_perm(rows[2 * d + 1][j / 2], rows[2 * d][j / 2], (j & 1) ? 0x07060302u : 0x05040100u);
+    } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const uint32_t sel = 0x0c0c0000u | (uint32_t)((4 + (j & 3)) << 8) | (uint32_t)(j & 3);  // byte j%4 of two rows
+                const uint32_t t0 = __builtin_amdgcn_perm(rows[4 * d + 1][j / 4], rows[4 * d][j / 4], sel);
+                const uint32_t t1 = __builtin_amdgcn_perm(rows[4 * d + 3][j / 4], rows[4 * d + 2][j / 4], sel);
+                cols[j][d] = __builtin_amdgcn_perm(t1, t0, 0x05040100u);
+            }
+    }
+}
+
+template <int ES>
+__global__ __launch_bounds__(kBlock) void tile_transpose_vec_kernel(const char *__restrict__ in, char *__restrict__ out, int64_t nA,
+                                                                     int64_t sA, int64_t nC, int64_t oC, int tilesA, int tilesC,
+                                                                     BatchDims bd) {
+    constexpr int V = 16 / ES, T = 16 * V;
+    __shared__ tt_u32x4 lds[kBlock * V];  // [c in tile][a-block ^ c-block]
+    // Diagonal order: consecutive workgroups step along C and along A together, so that neither
+    // the reads (tile rows sA apart) nor the writes (tile rows oC apart) of the workgroups in
+    // flight fall on addresses that differ only in high bits (power-of-two pitches otherwise pile
+    // onto a few memory channels).
+    int64_t b = blockIdx.x;
+    const int tc = (int)(b % tilesC); b /= tilesC;
+    const int ta = (int)((b % tilesA + tc) % tilesA); b /= tilesA;
+    int64_t ioff = 0, ooff = 0;
+    for (int d = bd.n - 1; d >= 0; --d) {
+        int64_t q = b / bd.size[d];
+        int64_t r = b - q * bd.size[d];
+        ioff += r * bd.istride[d];
+        ooff += r * bd.ostride[d];
+        b = q;
+    }
+    const int l = threadIdx.x;
+    {   // lanes along C: V input rows of one V x V block each
+        const int cblk = l & 15, ablk = l >> 4;
+        const int64_t a0 = (int64_t)ta * T + ablk * V, c0 = (int64_t)tc * T + cblk * V;
+        if (a0 < nA && c0 < nC) {
+            tt_u32x4 rows[V], cols[V];
+#pragma unroll
+            for (int r = 0; r < V; ++r)
+                rows[r] = __builtin_nontemporal_load(reinterpret_cast<const tt_u32x4 *>(in + (ioff + (a0 + r) * sA + c0) * ES));
+            transpose_block<ES>(rows, cols);
+#pragma unroll
+            for (int j = 0; j < V; ++j) lds[(cblk * V + j) * 16 + (ablk ^ cblk)] = cols[j];
+        }
+    }
+    __syncthreads();
+    {   // lanes along A: 16 output rows (values of c) per pass, 256 contiguous bytes each
+        const int ablk = l & 15, crow = l >> 4;
+        const int64_t a0 = (int64_t)ta * T + ablk * V;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            const int c = crow + 16 * i;
+            const int64_t gc = (int64_t)tc * T + c;
+            if (gc < nC && a0 < nA)
+                __builtin_nontemporal_store(lds[c * 16 + (ablk ^ ((c / V) & 15))], reinterpret_cast<tt_u32x4 *>(out + (ooff + gc * oC + a0) * ES));
+        }
+    }
+}
+
 // ---- concat --------------------------------------------------------------------------------
 constexpr int kConcatMax = 8;
 struct ConcatSrcs {
@@ -356,13 +445,26 @@ int dxh_transpose(int dtype, const void *in, const int32_t *shape, int ndim, con
         return (int)hipMemcpyAsync(out, in, (size_t)n * es, hipMemcpyDeviceToDevice, st);
     }
     for (int i = 0; i < nd; ++i) if (osz[i] > 0xffffffffLL) return DXH_ERR_SHAPE;
+    int es_eff = es;  // element size the kernels move
+    if (ost[nd - 1] == 1 && nd >= 3) {
+        // A short innermost run (2..16 bytes, a power of two) that stays innermost is better moved
+        // as one wide element by the tiled transpose than gathered 16 bytes at a time from
+        // scattered rows: fold it into the element size.
+        const int64_t run_bytes = osz[nd - 1] * es;
+        const bool pow2 = (run_bytes & (run_bytes - 1)) == 0;
+        if (pow2 && run_bytes <= 16 && run_bytes > es && aligned(in, (size_t)run_bytes) && aligned(out, (size_t)run_bytes)) {
+            for (int i = 0; i < nd - 1; ++i) ost[i] /= osz[nd - 1];  // every other input stride is a multiple of the innermost size
+            es_eff = (int)run_bytes;
+            --nd;
+        }
+    }
     if (ost[nd - 1] == 1) {
         // the innermost output run is contiguous in the input too
         OuterDims od{};
         od.n = nd - 1;
         int64_t rows = 1;
         for (int i = 0; i < nd - 1; ++i) { od.size[i] = (uint32_t)osz[i]; od.stride[i] = ost[i]; rows *= osz[i]; }
-        return launch_gather(in, out, rows, osz[nd - 1], es, od, st);
+        return launch_gather(in, out, rows, osz[nd - 1], es_eff, od, st);
     }
     // the last axis moves: tile over (A = output-last axis, C = input-last axis)
     int64_t ostr[DXH_MAX_DIMS];
@@ -378,10 +480,29 @@ int dxh_transpose(int dtype, const void *in, const int32_t *shape, int ndim, con
         bd.size[bd.n] = (uint32_t)osz[i]; bd.istride[bd.n] = ost[i]; bd.ostride[bd.n] = ostr[i]; ++bd.n;
         batch *= osz[i];
     }
+    const int V = 16 / es_eff;
+    bool vec = aligned(in, kVecBytes) && aligned(out, kVecBytes) && nA % V == 0 && nC % V == 0 && sA % V == 0 && oC % V == 0;
+    for (int i = 0; i < bd.n; ++i) vec = vec && bd.istride[i] % V == 0 && bd.ostride[i] % V == 0;
+    if (vec) {
+        const int T = 16 * V;
+        const int64_t tilesA = (nA + T - 1) / T, tilesC = (nC + T - 1) / T, blocks = batch * tilesA * tilesC;
+        if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
+#define DXH_TT(ES) tile_transpose_vec_kernel<ES><<<(unsigned)blocks, kBlock, 0, st>>>((const char *)in, (char *)out, nA, sA, nC, oC, (int)tilesA, (int)tilesC, bd)
+        switch (es_eff) {
+        case 16: DXH_TT(16); break;
+        case 8: DXH_TT(8); break;
+        case 4: DXH_TT(4); break;
+        case 2: DXH_TT(2); break;
+        default: DXH_TT(1); break;
+        }
+#undef DXH_TT
+        return launch_status();
+    }
     const int64_t tilesA = (nA + kTile - 1) / kTile, tilesC = (nC + kTile - 1) / kTile;
     const int64_t blocks = batch * tilesA * tilesC;
     if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
-    switch (es) {
+    switch (es_eff) {
+    case 16: tile_transpose_kernel<uint4><<<(unsigned)blocks, kBlock, 0, st>>>((const uint4 *)in, (uint4 *)out, nA, sA, nC, oC, (int)tilesA, (int)tilesC, bd); break;
     case 8: tile_transpose_kernel<uint64_t><<<(unsigned)blocks, kBlock, 0, st>>>((const uint64_t *)in, (uint64_t *)out, nA, sA, nC, oC, (int)tilesA, (int)tilesC, bd); break;
     case 4: tile_transpose_kernel<uint32_t><<<(unsigned)blocks, kBlock, 0, st>>>((const uint32_t *)in, (uint32_t *)out, nA, sA, nC, oC, (int)tilesA, (int)tilesC, bd); break;
     case 2: tile_transpose_kernel<uint16_t><<<(unsigned)blocks, kBlock, 0, st>>>((const uint16_t *)in, (uint16_t *)out, nA, sA, nC, oC, (int)tilesA, (int)tilesC, bd); break;

@@ -408,6 +408,41 @@ inline bool valid_shape(const int32_t *shape, int ndim, int64_t *size) {
     return true;
 }
 
+// Output axes given as (extent, input stride in elements; 0 = broadcast): drop extent-1 axes,
+// merge neighbours that are both broadcast or adjacent in the input, then copy rows with the
+// gather kernel (innermost run dense) or splat one element per row (innermost axis broadcast).
+// Returns kTooManyAxes when more axes survive the merge than the kernels index.
+constexpr int kTooManyAxes = -1000;
+inline int launch_broadcast(const void *in, void *out, int es, int n_axes, const int64_t *extent, const int64_t *stride,
+                            int64_t nout, hipStream_t st) {
+    int64_t sz[2 * DXH_MAX_DIMS], sd[2 * DXH_MAX_DIMS];
+    int nd = 0;
+    for (int i = 0; i < n_axes; ++i) {
+        if (extent[i] == 1) continue;
+        if (nd > 0 && ((sd[nd - 1] == 0 && stride[i] == 0) || (stride[i] != 0 && sd[nd - 1] == stride[i] * extent[i]))) {
+            sz[nd - 1] *= extent[i];
+            sd[nd - 1] = stride[i];
+        } else { sz[nd] = extent[i]; sd[nd] = stride[i]; ++nd; }
+    }
+    if (nd == 0 || (nd == 1 && sd[0] == 1)) {
+        if (in == out) return DXH_OK;
+        return (int)hipMemcpyAsync(out, in, (size_t)nout * es, hipMemcpyDeviceToDevice, st);
+    }
+    if (nd - 1 > kMaxOuter) return kTooManyAxes;
+    for (int i = 0; i < nd; ++i) if (sz[i] > 0xffffffffLL) return DXH_ERR_SHAPE;
+    OuterDims od{};
+    od.n = nd - 1;
+    int64_t rows = 1;
+    for (int i = 0; i < nd - 1; ++i) { od.size[i] = (uint32_t)sz[i]; od.stride[i] = sd[i]; rows *= sz[i]; }
+    if (sd[nd - 1] == 1) return launch_gather(in, out, rows, sz[nd - 1], es, od, st, /*reuse=*/true);
+    switch (es) {  // innermost axis is broadcast: splat one element per row position
+    case 8: return launch_splat<uint64_t>(in, out, rows, sz[nd - 1], od, st);
+    case 4: return launch_splat<uint32_t>(in, out, rows, sz[nd - 1], od, st);
+    case 2: return launch_splat<uint16_t>(in, out, rows, sz[nd - 1], od, st);
+    default: return launch_splat<uint8_t>(in, out, rows, sz[nd - 1], od, st);
+    }
+}
+
 }  // namespace dxh
 
 using namespace dxh;
@@ -585,43 +620,20 @@ int dxh_broadcastTo(int dtype, const void *in, const int32_t *in_shape, int in_n
     int64_t istr[DXH_MAX_DIMS];
     { int64_t s = 1; for (int i = in_ndim - 1; i >= 0; --i) { istr[i] = s; s *= in_shape[i]; } }
     // per output axis: input stride, 0 where the axis is broadcast (broadcastMap, shape_changeshape.cpp:79-104)
-    int64_t sz[DXH_MAX_DIMS], sd[DXH_MAX_DIMS];
-    int nd = 0;
+    int64_t extent[DXH_MAX_DIMS], stride[DXH_MAX_DIMS];
     for (int i = 0; i < out_ndim; ++i) {
-        int64_t stride = 0;
+        extent[i] = out_shape[i];
+        stride[i] = 0;
         if (i >= shift) {
-            if (in_shape[i - shift] == out_shape[i]) stride = istr[i - shift];
-            else if (in_shape[i - shift] == 1) stride = 0;
-            else return DXH_ERR_SHAPE;
+            if (in_shape[i - shift] == out_shape[i]) stride[i] = istr[i - shift];
+            else if (in_shape[i - shift] != 1) return DXH_ERR_SHAPE;
         }
-        if (out_shape[i] == 1) continue;
-        // merge: both broadcast, or both dense and adjacent in the input
-        if (nd > 0 && ((sd[nd - 1] == 0 && stride == 0) || (stride != 0 && sd[nd - 1] == stride * out_shape[i]))) {
-            sz[nd - 1] *= out_shape[i];
-            sd[nd - 1] = stride;
-        } else { sz[nd] = out_shape[i]; sd[nd] = stride; ++nd; }
     }
     if (nout == 0) return DXH_OK;
     if (!in || !out) return DXH_ERR_ARG;
     if (!aligned(in, es) || !aligned(out, es)) return DXH_ERR_ALIGN;
-    hipStream_t st = as_stream(stream);
-    if (nd == 0 || (nd == 1 && sd[0] == 1)) {
-        if (in == out) return DXH_OK;
-        return (int)hipMemcpyAsync(out, in, (size_t)nout * es, hipMemcpyDeviceToDevice, st);
-    }
-    for (int i = 0; i < nd; ++i) if (sz[i] > 0xffffffffLL) return DXH_ERR_SHAPE;
-    OuterDims od{};
-    od.n = nd - 1;
-    int64_t rows = 1;
-    for (int i = 0; i < nd - 1; ++i) { od.size[i] = (uint32_t)sz[i]; od.stride[i] = sd[i]; rows *= sz[i]; }
-    if (sd[nd - 1] == 1) return launch_gather(in, out, rows, sz[nd - 1], es, od, st, /*reuse=*/true);
-    // innermost axis is broadcast: splat one element per row position
-    switch (es) {
-    case 8: return launch_splat<uint64_t>(in, out, rows, sz[nd - 1], od, st);
-    case 4: return launch_splat<uint32_t>(in, out, rows, sz[nd - 1], od, st);
-    case 2: return launch_splat<uint16_t>(in, out, rows, sz[nd - 1], od, st);
-    default: return launch_splat<uint8_t>(in, out, rows, sz[nd - 1], od, st);
-    }
+    const int rc = launch_broadcast(in, out, es, out_ndim, extent, stride, nout, as_stream(stream));
+    return rc == kTooManyAxes ? DXH_ERR_SHAPE : rc;
 }
 
 int dxh_indexselect(int dtype, const void *in, const int32_t *in_shape, int in_ndim, int index_dtype, const void *index,
@@ -684,6 +696,15 @@ int dxh_repeat(int dtype, const void *in, const int32_t *shape, int ndim, const 
     if (!in || !out) return DXH_ERR_ARG;
     if (!aligned(in, es) || !aligned(out, es)) return DXH_ERR_ALIGN;
     hipStream_t st = as_stream(stream);
+    {   // repeat = broadcast of the input seen as [d0, 1, d1, 1, ...] to [d0, r0, d1, r1, ...]
+        int64_t extent[2 * DXH_MAX_DIMS], stride[2 * DXH_MAX_DIMS];
+        for (int i = 0; i < ndim; ++i) {
+            extent[2 * i] = shape[i]; stride[2 * i] = rd.istride[i];
+            extent[2 * i + 1] = repeats[i]; stride[2 * i + 1] = 0;
+        }
+        const int rc = launch_broadcast(in, out, es, 2 * ndim, extent, stride, total, st);
+        if (rc != kTooManyAxes) return rc;
+    }
     unsigned grid = stream_grid(total, kBlock, 16);
     switch (es) {
     case 8: repeat_kernel<uint64_t><<<grid, kBlock, 0, st>>>((const uint64_t *)in, (uint64_t *)out, total, rd); break;

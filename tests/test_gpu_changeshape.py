@@ -46,6 +46,55 @@ def test_transpose(dxh, orc, es):
         assert np.array_equal(got, np.transpose(a, order).reshape(-1))
 
 
+# shapes whose extents are multiples of 16 elements in the two moving axes: the 16-byte tiled
+# kernel for every element size (tiles of 16..256 elements per side), with ragged tile edges,
+# batch axes before / between / after the moving axes, and short innermost runs (2..16 bytes)
+# that are folded into the element
+VEC_TRANSPOSES = [
+    ((256, 512), [1, 0]),
+    ((272, 48), [1, 0]),            # partial tiles on both sides
+    ((3, 64, 96), [0, 2, 1]),
+    ((32, 5, 48), [2, 1, 0]),
+    ((16, 7, 32, 3), [2, 1, 0, 3]),   # batch axis between, innermost run of 3 elements stays
+    ((48, 64, 4), [1, 0, 2]),       # innermost run of 4 elements: folded for 1/2/4-byte elements
+    ((48, 64, 2), [1, 0, 2]),
+    ((2, 48, 16, 8), [0, 2, 1, 3]),
+    ((5, 16, 2, 32), [0, 3, 2, 1]),
+    ((512, 16), [1, 0]),
+    ((16, 1024), [1, 0]),
+]
+
+
+@pytest.mark.parametrize("es", [1, 2, 4, 8])
+def test_transpose_vector_tiles(dxh, es):
+    rng = np.random.default_rng(140 + es)
+    dtype = RAW[es][0]
+    for shape, order in VEC_TRANSPOSES:
+        a = rnd(rng, shape, es)
+        da, out = Dev(a), Dev.empty(a.size, a.dtype)
+        dx.check(dxh.dxh_transpose(dtype, da.ptr, dx.i32arr(shape), len(shape), dx.i32arr(order), out.ptr, None), "transpose")
+        assert np.array_equal(out.get(), np.transpose(a, order).reshape(-1)), (es, shape, order)
+
+
+def test_transpose_unaligned_base_takes_the_elementwise_tiles(dxh):
+    """Same shapes from a base address that is only element-aligned: the 16-byte kernel must not be
+    chosen (it would fault or read the wrong bytes)."""
+    rng = np.random.default_rng(150)
+    for es in (1, 2, 4):
+        dtype = RAW[es][0]
+        for shape, order in [((256, 512), [1, 0]), ((48, 64, 4), [1, 0, 2])]:
+            a = rnd(rng, shape, es)
+            n = a.size
+            buf_in, buf_out = Dev.empty(n + 16, a.dtype), Dev.empty(n + 16, a.dtype)
+            import torch
+            buf_in.t[es:es + n * es].copy_(torch.from_numpy(a.reshape(-1).view(np.uint8).copy()))
+            pin, pout = buf_in.t.data_ptr() + es, buf_out.t.data_ptr() + es
+            dx.check(dxh.dxh_transpose(dtype, pin, dx.i32arr(shape), len(shape), dx.i32arr(order), pout, None), "transpose")
+            torch.cuda.synchronize()
+            got = buf_out.t[es:es + n * es].cpu().numpy().view(a.dtype)
+            assert np.array_equal(got, np.transpose(a, order).reshape(-1)), (es, shape, order)
+
+
 def test_transpose_bad_order(dxh):
     a = Dev(np.zeros(24, dtype=np.float32))
     assert dxh.dxh_transpose(dx.F32, a.ptr, dx.i32arr([2, 3, 4]), 3, dx.i32arr([0, 0, 1]), a.ptr, None) == -2

@@ -1,0 +1,351 @@
+// matmul_fp.hip — fp32 and fp64 GEMM on the matrix pipe: v_mfma_f32_32x32x2_f32 and
+// v_mfma_f64_16x16x4_f64, operands and accumulators in the storage type.
+#include "matmul_common.hpp"
+
+namespace dxh {
+
+// ---- fp32 MFMA kernel ------------------------------------------------------------------------
+// v_mfma_f32_32x32x2_f32 (fp32 operands, fp32 accumulate: 157 TFLOP/s peak, 64 cycles each).  A
+// fp32 GEMM on the matrix pipe is compute bound by a wide margin (8x fewer flops per operand
+// byte than bf16 at 1/16 of the rate), so this kernel is a plain double-buffered one: workgroup
+// tile (64 FM) x (64 FN), K step FK, 4 waves 2x2, each wave FM x FN MFMA tiles, PD K steps held
+// in registers ahead of the LDS stage being multiplied.
+//   A      LDS [m][FK k] with rows padded by 4 floats; a lane reads the FK/2 consecutive k of its
+//          row half with ds_read_b128 (the k order inside a K step is a free permutation as
+//          long as both operands use it: MFMA e of lane half h multiplies k = (FK/2) h + e).
+//   B      LDS [FK k][n] as loaded, rows padded by 4 floats; one ds_read_b32 per lane and k.
+//   roles  MFMA on (B^T, A^T): a result lane holds 4 consecutive n of one row m -> 16-byte stores.
+//   VEC    K % 4 == 0, N % 4 == 0 and 16-byte aligned pointers: 16-byte loads and stores with
+//          clamped rows/columns; otherwise element-wise accesses with bounds checks.
+template <int FM, int FN, int FK, int PD, bool VEC>
+__global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float *__restrict__ A, const float *__restrict__ B,
+                                                                    float *__restrict__ C, int M, int K, int N, TileMap map) {
+    constexpr int TM = 64 * FM, TN = 64 * FN, FA_ROW = FK + 4, FB_ROW = TN + 4;
+    constexpr int STAGE = TM * FA_ROW + FK * FB_ROW;  // floats
+    constexpr int CA = FK / 4, CB = TN / 4;           // 16-byte chunks per A row / B row
+    constexpr int A_LD = TM * CA / kBlock, B_LD = FK * CB / kBlock;
+    constexpr int HK = FK / 2;                        // k values per lane half
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    __shared__ __attribute__((aligned(16))) float lds[2 * STAGE];
+    const TileCoord tc = tile_of_block(map);
+    if (!tc.valid) return;
+    const int tm = tc.tm, tn = tc.tn;
+    A += tc.batch * (int64_t)M * K;
+    B += tc.batch * (int64_t)K * N;
+    C += tc.batch * (int64_t)M * N;
+    const int m0 = tm * TM, n0 = tn * TN;
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
+
+    // per-lane chunks: A (row = id / CA, c = id % CA), B (krow = id / CB, c = id % CB), id = t + 256 i
+    f32x4 ra[PD][A_LD], rb[PD][B_LD];
+    auto load_global = [&](auto set, int k0) __attribute__((always_inline)) {
+        static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i, row = id / CA, kk = k0 + (id % CA) * 4, gm = m0 + row;
+            if constexpr (VEC) {
+                const float *p = A + (int64_t)(gm < M ? gm : M - 1) * K + (kk < K ? kk : 0);
+                f32x4 v = *reinterpret_cast<const f32x4 *>(p);
+                ra[set][i] = (kk < K) ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+            } else {
+                f32x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = (gm < M && kk + e < K) ? A[(int64_t)gm * K + kk + e] : 0.f;
+                ra[set][i] = v;
+            }
+        });
+        static_for<B_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i, krow = id / CB, gk = k0 + krow, gn = n0 + (id % CB) * 4;
+            if constexpr (VEC) {
+                const float *p = B + (int64_t)(gk < K ? gk : 0) * N + (gn < N ? gn : N - 4);
+                f32x4 v = *reinterpret_cast<const f32x4 *>(p);
+                rb[set][i] = (gk < K) ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+            } else {
+                f32x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = (gk < K && gn + e < N) ? B[(int64_t)gk * N + gn + e] : 0.f;
+                rb[set][i] = v;
+            }
+        });
+    };
+    auto store_lds = [&](auto set, auto stage) __attribute__((always_inline)) {
+        float *As = lds + decltype(stage)::value * STAGE, *Bs = As + TM * FA_ROW;
+        static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i;
+            *reinterpret_cast<f32x4 *>(As + (id / CA) * FA_ROW + (id % CA) * 4) = ra[set][i];
+        });
+        static_for<B_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i;
+            *reinterpret_cast<f32x4 *>(Bs + (id / CB) * FB_ROW + (id % CB) * 4) = rb[set][i];
+        });
+    };
+
+    f32x16 acc[FM][FN];
+    static_for<FM>([&](auto i) __attribute__((always_inline)) {
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        });
+    });
+    const int h = lane >> 5, l32 = lane & 31;
+    // MFMA e of lane half h multiplies k = HK*h + e of the K step (both operands use this order)
+    auto compute = [&](auto stage) __attribute__((always_inline)) {
+        const float *As = lds + decltype(stage)::value * STAGE, *Bs = As + TM * FA_ROW;
+        static_for<HK / 8>([&](auto q) __attribute__((always_inline)) {  // 8 k per lane half at a time
+            f32x4 fa[FM][2];
+            float fb[FN][8];
+            static_for<FM>([&](auto i) __attribute__((always_inline)) {
+                const float *p = As + (wm * 32 * FM + 32 * i + l32) * FA_ROW + HK * h + 8 * decltype(q)::value;
+                fa[i][0] = *reinterpret_cast<const f32x4 *>(p);
+                fa[i][1] = *reinterpret_cast<const f32x4 *>(p + 4);
+            });
+            static_for<FN>([&](auto j) __attribute__((always_inline)) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) fb[j][e] = Bs[(HK * h + 8 * decltype(q)::value + e) * FB_ROW + wn * 32 * FN + 32 * j + l32];
+            });
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                static_for<FM>([&](auto i) __attribute__((always_inline)) {
+                    static_for<FN>([&](auto j) __attribute__((always_inline)) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][e], fa[i][e >> 2][e & 3], acc[i][j], 0, 0, 0);
+                    });
+                });
+        });
+    };
+
+    // LDS stage (kt & 1) holds K step kt, register set (kt + 1) % PD holds step kt + 1 and is
+    // refilled with step kt + 1 + PD once it has moved to LDS.  Steps past the end are clamped
+    // onto the last one (loaded, never multiplied).
+    const int KT = (K + FK - 1) / FK;
+    auto k_of = [&](int stepno) { return (stepno < KT ? stepno : KT - 1) * FK; };
+    auto step = [&](auto S, auto R, int k_load) __attribute__((always_inline)) {
+        compute(S);
+        store_lds(R, ic<decltype(S)::value ^ 1>{});
+        load_global(R, k_load);
+        __syncthreads();
+    };
+    load_global(ic<0>{}, 0);
+    store_lds(ic<0>{}, ic<0>{});
+    static_for<PD>([&](auto d) __attribute__((always_inline)) { load_global(ic<(decltype(d)::value + 1) % PD>{}, k_of(decltype(d)::value + 1)); });
+    __syncthreads();
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+        step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1 + PD));
+        step(ic<1>{}, ic<2 % PD>{}, k_of(kt + 2 + PD));
+    }
+    if (kt < KT) compute(ic<0>{});
+
+    // result lane: row m = lane%32 of its MFMA tile; register group g holds columns 8g + 4h .. +3
+    static_for<FM>([&](auto i) __attribute__((always_inline)) {
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
+            const int gm = m0 + wm * 32 * FM + 32 * i + l32;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int gn = n0 + wn * 32 * FN + 32 * j + 8 * g + 4 * h;
+                if constexpr (VEC) {
+                    if (gm < M && gn < N)
+                        __builtin_nontemporal_store(f32x4{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]},
+                                                    reinterpret_cast<f32x4 *>(C + (int64_t)gm * N + gn));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (gm < M && gn + e < N) C[(int64_t)gm * N + gn + e] = acc[i][j][4 * g + e];
+                }
+            }
+        });
+    });
+}
+
+// ---- fp64 MFMA kernel ------------------------------------------------------------------------
+// v_mfma_f64_16x16x4_f64 (78.6 TFLOP/s peak, 64 cycles each): lane L supplies A[row L%16][k L/16]
+// and B[k L/16][col L%16]; the result lane holds D[4v + L/16][L%16] in register v.  Same plan as
+// the fp32 kernel: workgroup tile (64 FM) x (64 FN), K step 16, 4 waves 2x2, each wave
+// (2 FM) x (2 FN) MFMA tiles, double-buffered LDS with one K step prefetched in registers.  MFMA e
+// of lane class q = L/16 multiplies k = 4q + e, so a lane reads its four A values of a K step as
+// two 16-byte LDS loads.  Result rows are contiguous over 16 lanes: plain 8-byte stores coalesce.
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+template <int FM, int FN, bool VEC>
+__global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double *__restrict__ A, const double *__restrict__ B,
+                                                                    double *__restrict__ C, int M, int K, int N, TileMap map) {
+    constexpr int DK = 16, TM = 64 * FM, TN = 64 * FN, DA_ROW = DK + 2, DB_ROW = TN + 4;
+    constexpr int STAGE = TM * DA_ROW + DK * DB_ROW;  // doubles
+    constexpr int CA = DK / 2, CB = TN / 2;           // 16-byte chunks per A row / B row
+    constexpr int A_LD = TM * CA / kBlock, B_LD = DK * CB / kBlock;
+    constexpr int RT = 2 * FM, CT = 2 * FN;           // 16x16 MFMA tiles per wave along m and n
+    __shared__ __attribute__((aligned(16))) double lds[2 * STAGE];
+    const TileCoord tc = tile_of_block(map);
+    if (!tc.valid) return;
+    const int tm = tc.tm, tn = tc.tn;
+    A += tc.batch * (int64_t)M * K;
+    B += tc.batch * (int64_t)K * N;
+    C += tc.batch * (int64_t)M * N;
+    const int m0 = tm * TM, n0 = tn * TN;
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
+
+    f64x2 ra[A_LD], rb[B_LD];
+    auto load_global = [&](int k0) __attribute__((always_inline)) {
+        static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i, row = id / CA, kk = k0 + (id % CA) * 2, gm = m0 + row;
+            if constexpr (VEC) {
+                const double *p = A + (int64_t)(gm < M ? gm : M - 1) * K + (kk < K ? kk : 0);
+                f64x2 v = *reinterpret_cast<const f64x2 *>(p);
+                ra[i] = (kk < K) ? v : f64x2{0.0, 0.0};
+            } else {
+                f64x2 v;
+#pragma unroll
+                for (int e = 0; e < 2; ++e) v[e] = (gm < M && kk + e < K) ? A[(int64_t)gm * K + kk + e] : 0.0;
+                ra[i] = v;
+            }
+        });
+        static_for<B_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i, krow = id / CB, gk = k0 + krow, gn = n0 + (id % CB) * 2;
+            if constexpr (VEC) {
+                const double *p = B + (int64_t)(gk < K ? gk : 0) * N + (gn < N ? gn : N - 2);
+                f64x2 v = *reinterpret_cast<const f64x2 *>(p);
+                rb[i] = (gk < K) ? v : f64x2{0.0, 0.0};
+            } else {
+                f64x2 v;
+#pragma unroll
+                for (int e = 0; e < 2; ++e) v[e] = (gk < K && gn + e < N) ? B[(int64_t)gk * N + gn + e] : 0.0;
+                rb[i] = v;
+            }
+        });
+    };
+    auto store_lds = [&](int stage) __attribute__((always_inline)) {
+        double *As = lds + stage * STAGE, *Bs = As + TM * DA_ROW;
+        static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i;
+            *reinterpret_cast<f64x2 *>(As + (id / CA) * DA_ROW + (id % CA) * 2) = ra[i];
+        });
+        static_for<B_LD>([&](auto i) __attribute__((always_inline)) {
+            const int id = t + kBlock * i;
+            *reinterpret_cast<f64x2 *>(Bs + (id / CB) * DB_ROW + (id % CB) * 2) = rb[i];
+        });
+    };
+
+    f64x4 acc[RT][CT];
+    static_for<RT>([&](auto i) __attribute__((always_inline)) {
+        static_for<CT>([&](auto j) __attribute__((always_inline)) { acc[i][j] = f64x4{0.0, 0.0, 0.0, 0.0}; });
+    });
+    const int q = lane >> 4, l16 = lane & 15;
+    auto compute = [&](int stage) __attribute__((always_inline)) {
+        const double *As = lds + stage * STAGE, *Bs = As + TM * DA_ROW;
+        f64x2 fa[RT][2];
+        double fb[CT][4];
+        static_for<RT>([&](auto i) __attribute__((always_inline)) {
+            const double *p = As + (wm * 32 * FM + 16 * i + l16) * DA_ROW + 4 * q;
+            fa[i][0] = *reinterpret_cast<const f64x2 *>(p);
+            fa[i][1] = *reinterpret_cast<const f64x2 *>(p + 2);
+        });
+        static_for<CT>([&](auto j) __attribute__((always_inline)) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) fb[j][e] = Bs[(4 * q + e) * DB_ROW + wn * 32 * FN + 16 * j + l16];
+        });
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            static_for<RT>([&](auto i) __attribute__((always_inline)) {
+                static_for<CT>([&](auto j) __attribute__((always_inline)) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[i][e >> 1][e & 1], fb[j][e], acc[i][j], 0, 0, 0);
+                });
+            });
+    };
+
+    const int KT = (K + DK - 1) / DK;
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const bool more = kt + 1 < KT;
+        if (more) load_global((kt + 1) * DK);
+        compute(kt & 1);
+        if (more) store_lds((kt + 1) & 1);
+        __syncthreads();
+    }
+
+    static_for<RT>([&](auto i) __attribute__((always_inline)) {
+        static_for<CT>([&](auto j) __attribute__((always_inline)) {
+            const int gn = n0 + wn * 32 * FN + 16 * j + l16;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int gm = m0 + wm * 32 * FM + 16 * i + 4 * v + q;
+                if (gm < M && gn < N) __builtin_nontemporal_store(acc[i][j][v], C + (int64_t)gm * N + gn);
+            }
+        });
+    });
+}
+
+template <int FM, int FN, int FK, int PD>
+int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, hipStream_t st) {
+    TileMap map;
+    if (!make_tile_map(batch, m, n, 64 * FM, 64 * FN, map)) return DXH_ERR_SHAPE;
+    const unsigned blocks = (unsigned)(8 * map.chunk);
+    if (vec) matmul_mfma_f32_kernel<FM, FN, FK, PD, true><<<blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, map);
+    else matmul_mfma_f32_kernel<FM, FN, FK, PD, false><<<blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, map);
+    return launch_status();
+}
+
+// fp32: the matrix pipe is the bound, so the tile is chosen for CU balance.  Cost model per tile
+// shape: two workgroups share a CU; a CU's time is (rounds of two tiles) x tile flops / efficiency,
+// where a last round that leaves at most one workgroup per CU counts 0.6 (a lone workgroup runs
+// faster than two that share the pipe) and the efficiencies are the measured large-square rates
+// relative to the 128x128 tile.  Small tiles take longer K steps and a deeper prefetch: with few
+// MFMAs per step only that hides the global-load latency.
+int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    const bool vec = k % 4 == 0 && n % 4 == 0 && n >= 4 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes);
+    const int64_t cus = compute_units();
+    auto cost = [&](int tm, int tn, double eff) {
+        const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn);
+        const int64_t full = tiles / (2 * cus), rem = tiles % (2 * cus);
+        const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.6 : 0.0);
+        return rounds * (double)tm * (double)tn / eff;
+    };
+    const float *af = (const float *)a, *bf = (const float *)b;
+    float *cf = (float *)c;
+    int64_t choice = tuning().matmul_tile;
+    if (choice == 0) {
+        const double c1 = cost(128, 128, 1.0), c2 = cost(128, 64, 0.95), c3 = cost(64, 64, 0.86);
+        choice = (c1 <= c2 && c1 <= c3) ? 1 : (c2 <= c3) ? 2 : 3;
+    }
+    switch (choice) {
+    case 1: return launch_f32_tile<2, 2, 32, 1>(af, bf, cf, batch, m, k, n, vec, st);
+    case 2: return launch_f32_tile<2, 1, 32, 2>(af, bf, cf, batch, m, k, n, vec, st);
+    case 3: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, st);
+    case 4: return launch_f32_tile<2, 2, 16, 1>(af, bf, cf, batch, m, k, n, vec, st);
+    default: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, st);
+    }
+}
+
+template <int FM, int FN>
+int launch_f64_tile(const double *a, const double *b, double *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, hipStream_t st) {
+    TileMap map;
+    if (!make_tile_map(batch, m, n, 64 * FM, 64 * FN, map)) return DXH_ERR_SHAPE;
+    const unsigned blocks = (unsigned)(8 * map.chunk);
+    if (vec) matmul_mfma_f64_kernel<FM, FN, true><<<blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, map);
+    else matmul_mfma_f64_kernel<FM, FN, false><<<blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, map);
+    return launch_status();
+}
+
+// fp64 on the matrix pipe; tile chosen for CU balance like fp32 (efficiencies measured on 4096^3)
+int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    const bool vec = k % 2 == 0 && n % 2 == 0 && n >= 2 && aligned(a, kVecBytes) && aligned(b, kVecBytes);
+    const int64_t cus = compute_units();
+    auto cost = [&](int tm, int tn, double eff) {
+        const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn);
+        const int64_t full = tiles / (2 * cus), rem = tiles % (2 * cus);
+        const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.6 : 0.0);
+        return rounds * (double)tm * (double)tn / eff;
+    };
+    const double *af = (const double *)a, *bf = (const double *)b;
+    double *cf = (double *)c;
+    int64_t choice = tuning().matmul_tile;
+    if (choice == 0) {
+        const double c1 = cost(128, 128, 1.0), c2 = cost(128, 64, 0.86), c3 = cost(64, 64, 0.95);
+        choice = (c1 <= c2 && c1 <= c3) ? 1 : (c2 <= c3) ? 2 : 3;
+    }
+    switch (choice) {
+    case 1: return launch_f64_tile<2, 2>(af, bf, cf, batch, m, k, n, vec, st);
+    case 2: return launch_f64_tile<2, 1>(af, bf, cf, batch, m, k, n, vec, st);
+    default: return launch_f64_tile<1, 1>(af, bf, cf, batch, m, k, n, vec, st);
+    }
+}
+
+}  // namespace dxh

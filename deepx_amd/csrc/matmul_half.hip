@@ -1,0 +1,372 @@
+// matmul_half.hip — bf16 / f16 GEMM on the matrix pipe (v_mfma_f32_32x32x16_{bf16,f16}, fp32
+// accumulate, one RNE rounding of C).  Aligned shapes (K % 64 == 0, N % 8 == 0) take
+// matmul_mfma_tile_kernel, 64x64 to 256x256 workgroup tiles, software-pipelined over K; anything
+// else takes matmul_mfma_kernel, a plain 128x128x32 tile with element-wise edge handling.
+#include "matmul_common.hpp"
+
+namespace dxh {
+
+constexpr int BM = 128, BN = 128, BK = 32;
+constexpr int LDK = BK + 8;  // padded k-stride (elements) of both LDS tiles: 80 bytes, keeps 16-byte alignment
+
+
+template <typename T, typename V> __device__ inline f32x16 mfma32(V a, V b, f32x16 c) {
+    if constexpr (std::is_same_v<T, bf16_t>)
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+// VEC_A: rows of A are 16-byte aligned (K % 8 == 0, base aligned); VEC_B likewise for B (N % 8 == 0).
+template <typename T, bool VEC_A, bool VEC_B>
+__global__ __launch_bounds__(kBlock) void matmul_mfma_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C,
+                                                              int M, int K, int N, int tiles_m, int tiles_n) {
+    __shared__ __attribute__((aligned(16))) uint16_t As[BM * LDK];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[BN * LDK];  // transposed: [n][k]
+    int64_t bid = blockIdx.x;
+    const int tn = (int)(bid % tiles_n); bid /= tiles_n;
+    const int tm = (int)(bid % tiles_m); bid /= tiles_m;
+    const int64_t batch = bid;
+    A += batch * (int64_t)M * K;
+    B += batch * (int64_t)K * N;
+    C += batch * (int64_t)M * N;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+    const int wm = w >> 1, wn = w & 1;
+    const uint16_t *Ar = reinterpret_cast<const uint16_t *>(A);
+    const uint16_t *Br = reinterpret_cast<const uint16_t *>(B);
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        // ---- A tile: 128 rows x 32 k, 16 bytes (8 k) per lane, two rows per lane
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int r = (t >> 2) + h * 64, kc = (t & 3) * 8;
+            const int gm = m0 + r, gk = k0 + kc;
+            vec_t<uint16_t, 8> x;
+            if (VEC_A && gm < M && gk + 8 <= K) {
+                x = *reinterpret_cast<const vec_t<uint16_t, 8> *>(Ar + (int64_t)gm * K + gk);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) x.v[j] = (gm < M && gk + j < K) ? Ar[(int64_t)gm * K + gk + j] : (uint16_t)0;
+            }
+            *reinterpret_cast<vec_t<uint16_t, 8> *>(&As[r * LDK + kc]) = x;
+        }
+        // ---- B tile: 32 k x 128 n, 16 bytes (8 n) per lane, transposed into Bs[n][k]
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int kr = (t >> 4) + h * 16, nc = (t & 15) * 8;
+            const int gk = k0 + kr, gn = n0 + nc;
+            vec_t<uint16_t, 8> x;
+            if (VEC_B && gk < K && gn + 8 <= N) {
+                x = *reinterpret_cast<const vec_t<uint16_t, 8> *>(Br + (int64_t)gk * N + gn);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) x.v[j] = (gk < K && gn + j < N) ? Br[(int64_t)gk * N + gn + j] : (uint16_t)0;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) Bs[(nc + j) * LDK + kr] = x.v[j];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 16) {
+            uint4 af[2], bf[2];
+            const int ko = kk + (lane >> 5) * 8;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) af[i] = *reinterpret_cast<const uint4 *>(&As[(wm * 64 + i * 32 + (lane & 31)) * LDK + ko]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) bf[j] = *reinterpret_cast<const uint4 *>(&Bs[(wn * 64 + j * 32 + (lane & 31)) * LDK + ko]);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = mfma32<T>(af[i], bf[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+    // ---- epilogue: D[row][col], col = lane%32, row = 8*(v/4) + 4*(lane/32) + v%4
+    uint16_t *Cr = reinterpret_cast<uint16_t *>(C);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = m0 + wm * 64 + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+                if (row < M && col < N) Cr[(int64_t)row * N + col] = store_acc<T>(acc[i][j][v]).bits;
+            }
+}
+
+constexpr int PK = 64;  // K step of the MFMA tile kernel
+__device__ inline int swz(int row, int chunk) { return chunk ^ ((row ^ (row >> 3)) & 7); }
+
+// ---- MFMA kernel with the B transposition done by the LDS read ------------------------------
+// Workgroup tile TM x TN (64, 128 or 256 each), K step 64, 4 waves in a 2x2 grid, each wave a
+// (TM/2) x (TN/2) patch of 32x32x16 MFMAs.  Requirements (checked by the launcher): K % 64 == 0,
+// N % 8 == 0, 16-byte aligned A, B, C.
+//   loads  every global load is 16 bytes per lane (a wave instruction occupies the vector cache for
+//          the same 16 cycles whatever its width, so 8-byte loads halve its throughput).
+//   A      [TM m][64 k] in LDS, 128-byte rows, 16-byte chunk c of row r at chunk c ^ swizzle(r).
+//   B      stays n-contiguous in LDS, [64 k][TN n] with rows padded by 64 bytes; the MFMA operand
+//          (8 consecutive k of one column per lane) is assembled by two ds_read_b64_tr_b16.
+//   pipe   PD K steps in flight in registers, two LDS stages, one barrier per K step; the stores
+//          into the next stage and the global loads are spread over the four k-substeps.
+//   roles  the MFMA runs on (B^T, A^T): a lane of the result then holds 4 consecutive n of one row
+//          m, which packs into 8-byte LDS stores for the epilogue.
+//   map    blockIdx -> tile through tile_of_block (XCD-aware, above).
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+// two fp32 accumulators -> one dword of two bf16/f16, round to nearest even (v_cvt_pk_bf16_f32 /
+// v_cvt_pk_f16_f32); element a in the low half
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    if constexpr (std::is_same_v<T, bf16_t>) return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+    else return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, f16x2));
+}
+// Within each group of 16 lanes, lane i passes the address of 4 consecutive 16-bit elements
+// ("row i") and receives element i%4 of rows i/4, 4 + i/4, 8 + i/4, 12 + i/4.
+__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t *p) {
+    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p);
+    return __builtin_bit_cast(u32x2, v);
+}
+
+// the `count` loads of a K step are dealt out over its four k-substeps
+constexpr int part_first(int count, int part) { return count * part / 4; }
+constexpr int part_count(int count, int part) { return count * (part + 1) / 4 - count * part / 4; }
+
+template <typename T, int TM, int TN, int PD>
+__global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul_mfma_tile_kernel(
+    const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int K, int N, TileMap map) {
+    static_assert(TM % 64 == 0 && (TN == 64 || TN == 128 || TN == 256), "B rows must split evenly over the 256 lanes");
+    constexpr int FM = TM / 64, FN = TN / 64;      // 32x32 MFMA tiles per wave along m and n
+    constexpr int A_LD = TM / 32, B_LD = TN / 32;  // 16-byte global loads per lane per K step
+    constexpr int CB = TN / 8;                     // 16-byte chunks per B row
+    constexpr int KR = kBlock / CB;                // B rows covered by one load of the workgroup
+    constexpr int B_ROW = TN + 32;                 // elements per k-row of the B stage (64-byte pad)
+    constexpr int A_STAGE = TM * PK, STAGE = A_STAGE + PK * B_ROW;
+    constexpr int LDC = TN + 8;
+    constexpr int LDS_ELEMS = (2 * STAGE > TM * LDC) ? 2 * STAGE : TM * LDC;
+    __shared__ __attribute__((aligned(16))) uint16_t lds[LDS_ELEMS];
+
+    const TileCoord tc = tile_of_block(map);
+    if (!tc.valid) return;
+    const int batch = tc.batch, tm = tc.tm, tn = tc.tn;
+    const int m0 = tm * TM, n0 = tn * TN;
+
+    const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
+    const uint16_t *Ab = reinterpret_cast<const uint16_t *>(A) + ((int64_t)batch * M + m0) * K;
+    const uint16_t *Bb = reinterpret_cast<const uint16_t *>(B) + (int64_t)batch * K * N + n0;
+
+    // Branch-free loads: rows past M and columns past N are clamped onto valid memory; their
+    // products land in accumulator rows/columns that the epilogue never stores.
+    const int arow = t >> 3, ach = t & 7;
+    int a_off[A_LD], a_lds[A_LD];
+    static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
+        const int r = arow + 32 * i;
+        a_off[i] = (m0 + r < M ? r : M - 1 - m0) * K + ach * 8;
+        a_lds[i] = r * PK + swz(r, ach) * 8;
+    });
+    const int brow = t / CB, bch = t % CB;
+    const int b_off = brow * N + (n0 + bch * 8 < N ? bch * 8 : N - 8 - n0);
+    const int b_lds = brow * B_ROW + bch * 8;
+
+    u32x4 ra[PD][A_LD], rb[PD][B_LD];
+    auto load_part = [&](auto set, auto part, int k0) __attribute__((always_inline)) {
+        static_for<part_count(A_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
+            constexpr int i = part_first(A_LD, decltype(part)::value) + decltype(q)::value;
+            ra[set][i] = *reinterpret_cast<const u32x4 *>(Ab + a_off[i] + k0);
+        });
+        static_for<part_count(B_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
+            constexpr int i = part_first(B_LD, decltype(part)::value) + decltype(q)::value;
+            rb[set][i] = *reinterpret_cast<const u32x4 *>(Bb + (int64_t)(k0 + i * KR) * N + b_off);
+        });
+    };
+    auto store_part = [&](auto set, auto part, auto stage) __attribute__((always_inline)) {
+        uint16_t *As = lds + decltype(stage)::value * STAGE, *Bs = As + A_STAGE;
+        static_for<part_count(A_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
+            constexpr int i = part_first(A_LD, decltype(part)::value) + decltype(q)::value;
+            *reinterpret_cast<u32x4 *>(As + a_lds[i]) = ra[set][i];
+        });
+        static_for<part_count(B_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
+            constexpr int i = part_first(B_LD, decltype(part)::value) + decltype(q)::value;
+            *reinterpret_cast<u32x4 *>(Bs + b_lds + i * KR * B_ROW) = rb[set][i];
+        });
+    };
+
+    // fragment registers, double-buffered over the k-substeps
+    u32x4 fa[2][FM], fb[2][FN];
+    const int fa_row = wm * (TM / 2) + (lane & 31), fch = lane >> 5;
+    const int fb_off = (8 * fch + ((lane & 15) >> 2)) * B_ROW + wn * (TN / 2) + (lane & 16) + 4 * (lane & 3);
+    auto read_frags = [&](auto buf, auto stage, auto ks) __attribute__((always_inline)) {
+        const uint16_t *As = lds + decltype(stage)::value * STAGE, *Bs = As + A_STAGE;
+        static_for<FM>([&](auto i) __attribute__((always_inline)) {
+            const int row = fa_row + 32 * i, ch = decltype(ks)::value * 2 + fch;
+            fa[buf][i] = *reinterpret_cast<const u32x4 *>(As + row * PK + swz(row, ch) * 8);
+        });
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
+            const uint16_t *p = Bs + fb_off + decltype(ks)::value * 16 * B_ROW + 32 * j;
+            const u32x2 lo = lds_read_tr16(p), hi = lds_read_tr16(p + 4 * B_ROW);
+            fb[buf][j] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        });
+    };
+
+    f32x16 acc[FM][FN];
+    static_for<FM>([&](auto i) __attribute__((always_inline)) {
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        });
+    });
+    constexpr int NM = FM * FN;                                 // MFMAs per k-substep
+    constexpr int ND = FM + 2 * FN;                             // LDS fragment reads per substep
+    auto mma = [&](auto buf, auto lo, auto hi) __attribute__((always_inline)) {
+        static_for<decltype(hi)::value - decltype(lo)::value>([&](auto x) __attribute__((always_inline)) {
+            constexpr int idx = decltype(lo)::value + decltype(x)::value, i = idx / FN, j = idx % FN;
+            acc[i][j] = mfma32<T>(fb[buf][j], fa[buf][i], acc[i][j]);
+        });
+    };
+    // Issue order inside a scheduling region: after each of `mfmas` MFMAs an even share of the
+    // region's LDS reads, LDS writes and global loads, so that the matrix pipe always has the next
+    // MFMA queued while the memory instructions are issued underneath it.
+    auto interleave = [&](auto mfmas, auto reads, auto writes, auto loads) __attribute__((always_inline)) {
+        constexpr int nm = decltype(mfmas)::value, nr = decltype(reads)::value, nw = decltype(writes)::value, nl = decltype(loads)::value;
+        static_for<nm>([&](auto x) __attribute__((always_inline)) {
+            constexpr int m = decltype(x)::value;
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            constexpr int r = nr * (m + 1) / nm - nr * m / nm, wr = nw * (m + 1) / nm - nw * m / nm, l = nl * (m + 1) / nm - nl * m / nm;
+            if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+            if constexpr (wr > 0) __builtin_amdgcn_sched_group_barrier(0x200, wr, 0);
+            if constexpr (l > 0) __builtin_amdgcn_sched_group_barrier(0x020, l, 0);
+        });
+    };
+
+    // One K step: LDS stage S is multiplied; register set R (the next K step) moves into stage
+    // S^1 and is refilled with the K step PD further on.  Fragment buffer 0 holds substep 0 on
+    // entry.  The last substep straddles the barrier: half of its MFMAs are queued before it and
+    // the other half runs under the first fragment reads of stage S^1.
+    auto step = [&](auto S, auto R, int k_load) __attribute__((always_inline)) {
+        constexpr int s = decltype(S)::value;
+        static_for<4>([&](auto ks) __attribute__((always_inline)) {
+            constexpr int cur = decltype(ks)::value & 1;
+            constexpr int NW = part_count(A_LD, decltype(ks)::value) + part_count(B_LD, decltype(ks)::value);  // LDS writes = global loads
+            if constexpr (decltype(ks)::value < 3) {
+                read_frags(ic<cur ^ 1>{}, S, ic<decltype(ks)::value + 1>{});
+                store_part(R, ks, ic<s ^ 1>{});
+                load_part(R, ks, k_load);
+                mma(ic<cur>{}, ic<0>{}, ic<NM>{});
+                interleave(ic<NM>{}, ic<ND>{}, ic<NW>{}, ic<NW>{});
+            } else {
+                store_part(R, ks, ic<s ^ 1>{});
+                load_part(R, ks, k_load);
+                mma(ic<cur>{}, ic<0>{}, ic<NM / 2>{});
+                interleave(ic<NM / 2>{}, ic<0>{}, ic<NW>{}, ic<NW>{});
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();
+                read_frags(ic<cur ^ 1>{}, ic<s ^ 1>{}, ic<0>{});
+                mma(ic<cur>{}, ic<NM / 2>{}, ic<NM>{});
+                interleave(ic<NM - NM / 2>{}, ic<ND>{}, ic<0>{}, ic<0>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+
+    const int KT = K / PK;
+    auto k_of = [&](int stepno) __attribute__((always_inline)) { return (stepno < KT ? stepno : KT - 1) * PK; };
+    static_for<4>([&](auto part) __attribute__((always_inline)) { load_part(ic<0>{}, part, k_of(0)); });
+    static_for<4>([&](auto part) __attribute__((always_inline)) { store_part(ic<0>{}, part, ic<0>{}); });
+    static_for<PD>([&](auto d) __attribute__((always_inline)) { static_for<4>([&](auto part) __attribute__((always_inline)) { load_part(ic<(decltype(d)::value + 1) % PD>{}, part, k_of(decltype(d)::value + 1)); }); });
+    __syncthreads();
+    read_frags(ic<0>{}, ic<0>{}, ic<0>{});
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+        step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1 + PD));
+        step(ic<1>{}, ic<2 % PD>{}, k_of(kt + 2 + PD));
+    }
+    if (kt < KT) step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1 + PD));
+    __syncthreads();
+
+    // ---- epilogue: result lane holds row m = lane%32 of its MFMA tile and, per group g of 4
+    // registers, columns 8g + 4*(lane/32) .. +3: one 8-byte LDS store each, then 16-byte row stores
+    uint16_t *Cs = lds;
+    static_for<FM>([&](auto i) __attribute__((always_inline)) {
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int row = wm * (TM / 2) + 32 * i + (lane & 31);
+                const int col = wn * (TN / 2) + 32 * j + 8 * g + 4 * (lane >> 5);
+                *reinterpret_cast<u32x2 *>(Cs + row * LDC + col) =
+                    u32x2{pack2<T>(acc[i][j][4 * g], acc[i][j][4 * g + 1]), pack2<T>(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3])};
+            }
+        });
+    });
+    __syncthreads();
+    uint16_t *Cr = reinterpret_cast<uint16_t *>(C) + (int64_t)batch * M * N;
+#pragma unroll
+    for (int i = 0; i < TM * CB / kBlock; ++i) {
+        const int c = t + i * kBlock, row = c / CB, ch = c % CB;
+        const int gm = m0 + row, gn = n0 + ch * 8;
+        if (gm < M && gn < N)  // N % 8 == 0: a chunk is either fully inside or fully outside
+            st_nt(reinterpret_cast<uint4 *>(Cr + (int64_t)gm * N + gn), *reinterpret_cast<const uint4 *>(Cs + row * LDC + ch * 8));
+    }
+}
+
+template <typename T, int TM, int TN, int PD>
+int launch_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    TileMap map;
+    if (!make_tile_map(batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
+    matmul_mfma_tile_kernel<T, TM, TN, PD><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map);
+    return launch_status();
+}
+
+template <typename T>
+int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    const bool fast = k % PK == 0 && n % 8 == 0 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes) &&
+                      k <= (1 << 22) && n <= (1 << 24);
+    int64_t choice = tuning().matmul_tile;
+    if (fast && choice == 0) {
+        // 256x256 tiles halve the bytes every CU pulls through its vector cache per flop, but need
+        // about one tile per CU to pay off.  Below that, 128x128 tiles (two workgroups per CU) as
+        // long as they still give every CU a workgroup and a half; skinny outputs go to 128x64 or
+        // 64x64 tiles so that all CUs (and their vector caches) take part.
+        const int64_t cus = compute_units();
+        auto tiles = [&](int tm, int tn) { return batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn); };
+        if (tiles(256, 256) * 10 >= cus * 9) choice = 4;
+        else if (tiles(128, 128) * 2 >= cus * 3) choice = 1;
+        else if (tiles(128, 64) * 2 >= cus) choice = 2;
+        else choice = 5;
+    }
+    if (fast) {
+        switch (choice) {
+        case 2: return launch_tile<T, 128, 64, 1>(a, b, c, batch, m, k, n, st);
+        case 3: return launch_tile<T, 64, 128, 1>(a, b, c, batch, m, k, n, st);
+        case 4: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, st);
+        case 5: return launch_tile<T, 64, 64, 1>(a, b, c, batch, m, k, n, st);
+        default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, st);
+        }
+    }
+    const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
+    const int64_t blocks = batch * tiles_m * tiles_n;
+    if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
+    const bool va = (k % 8 == 0) && aligned(a, kVecBytes);
+    const bool vb = (n % 8 == 0) && aligned(b, kVecBytes);
+#define DXH_MM(VA, VB) matmul_mfma_kernel<T, VA, VB><<<(unsigned)blocks, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, (int)tiles_m, (int)tiles_n)
+    if (va && vb) DXH_MM(true, true);
+    else if (va) DXH_MM(true, false);
+    else if (vb) DXH_MM(false, true);
+    else DXH_MM(false, false);
+#undef DXH_MM
+    return launch_status();
+}
+int launch_matmul_half(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    return dtype == DXH_BF16 ? launch_mfma<bf16_t>(a, b, c, batch, m, k, n, st) : launch_mfma<f16_t>(a, b, c, batch, m, k, n, st);
+}
+
+}  // namespace dxh

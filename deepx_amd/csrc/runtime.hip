@@ -127,6 +127,24 @@ int dxh_event_elapsed_ms(void *start, void *stop, float *ms) {
     return (int)hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop);
 }
 
+static_assert(sizeof(hipIpcMemHandle_t) == DXH_IPC_HANDLE_BYTES, "handle size is part of the ABI");
+int dxh_ipc_export(const void *ptr, void *handle) {
+    if (!ptr || !handle) return DXH_ERR_ARG;
+    hipIpcMemHandle_t h;
+    hipError_t e = hipIpcGetMemHandle(&h, const_cast<void *>(ptr));
+    if (e != hipSuccess) return (int)e;
+    std::memcpy(handle, &h, sizeof h);
+    return DXH_OK;
+}
+int dxh_ipc_open(const void *handle, void **ptr) {
+    if (!handle || !ptr) return DXH_ERR_ARG;
+    *ptr = nullptr;
+    hipIpcMemHandle_t h;
+    std::memcpy(&h, handle, sizeof h);
+    return (int)hipIpcOpenMemHandle(ptr, h, hipIpcMemLazyEnablePeerAccess);
+}
+int dxh_ipc_close(void *ptr) { return ptr ? (int)hipIpcCloseMemHandle(ptr) : DXH_OK; }
+
 int dxh_graph_begin_capture(void *stream) {
     if (!stream) return DXH_ERR_ARG;  // the NULL stream cannot be captured
     return (int)hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal);

@@ -67,6 +67,9 @@ SIGNATURES = {
     "dxh_event_record": ([_p, _p], _i),
     "dxh_event_sync": ([_p], _i),
     "dxh_event_elapsed_ms": ([_p, _p, C.POINTER(_f)], _i),
+    "dxh_ipc_export": ([_p, _p], _i),
+    "dxh_ipc_open": ([_p, C.POINTER(_p)], _i),
+    "dxh_ipc_close": ([_p], _i),
     "dxh_graph_begin_capture": ([_p], _i),
     "dxh_graph_end_capture": ([_p, C.POINTER(_p)], _i),
     "dxh_graph_launch": ([_p, _p], _i),

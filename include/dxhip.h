@@ -113,6 +113,17 @@ DXH_API int dxh_event_record(void *event, void *stream);
 DXH_API int dxh_event_sync(void *event);
 DXH_API int dxh_event_elapsed_ms(void *start, void *stop, float *ms);
 
+/* ---- sharing one allocation between processes on the same GPU (heap tensors).
+ * The reference plans this for its heap-tensor store (cudaIpcGetMemHandle / cudaIpcOpenMemHandle,
+ * executor/heapmem-cuda/README.md:36-40); its tree holds no IPC code yet.  `handle` is an opaque
+ * DXH_IPC_HANDLE_BYTES buffer that may be sent to another process as bytes.  `ptr` must be the
+ * start of a dxh_malloc allocation (keep shared allocations under 2 GiB); a pointer obtained with
+ * dxh_ipc_open is released with dxh_ipc_close, never dxh_free. */
+#define DXH_IPC_HANDLE_BYTES 64
+DXH_API int dxh_ipc_export(const void *ptr, void *handle);
+DXH_API int dxh_ipc_open(const void *handle, void **ptr);
+DXH_API int dxh_ipc_close(void *ptr);
+
 /* ---- HIP graphs: record the kernels a sequence of dxh_* calls launches on `stream` once, replay
  * them with one launch.  No counterpart in the reference (it launches op by op on the default
  * stream); used by the executor for datagrams that carry several deepxIR lines

@@ -174,7 +174,9 @@ def test_indexselect_out_of_range_is_clamped(dxh):
 def test_repeat(dxh, orc, es):
     rng = np.random.default_rng(80 + es)
     dtype = RAW[es][0]
-    for shape, reps in [((3, 4), (2, 3)), ((2, 3, 4), (1, 2, 1)), ((5,), (4,))]:
+    for shape, reps in [((3, 4), (2, 3)), ((2, 3, 4), (1, 2, 1)), ((5,), (4,)), ((64, 48), (3, 2)), ((16, 1, 32), (1, 5, 1)), ((4096,), (7,)),
+                        ((2, 3, 2, 3, 2, 3, 2, 3), (2, 2, 2, 2, 2, 2, 2, 2)),   # 16 interleaved axes: more than the row kernels index
+                        ((3, 2, 2, 2, 2, 2, 2), (1, 2, 1, 2, 1, 2, 3))]:
         a = rnd(rng, shape, es)
         want_np = a
         for ax, r in enumerate(reps):

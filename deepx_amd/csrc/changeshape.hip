@@ -189,9 +189,9 @@ __global__ __launch_bounds__(kBlock) void tile_transpose_kernel(const E *__restr
                                                                  int64_t sA, int64_t nC, int64_t oC, int tilesA, int tilesC,
                                                                  BatchDims bd) {
     __shared__ E tile[kTile][kTile + 1];
-    int64_t b = blockIdx.x;
+    int64_t b = blockIdx.x;  // diagonal order over the tile grid, see tile_transpose_vec_kernel
     const int tc = (int)(b % tilesC); b /= tilesC;
-    const int ta = (int)(b % tilesA); b /= tilesA;
+    const int ta = (int)((b % tilesA + tc) % tilesA); b /= tilesA;
     int64_t ioff = 0, ooff = 0;
     for (int d = bd.n - 1; d >= 0; --d) {
         int64_t q = b / bd.size[d];

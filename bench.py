@@ -322,16 +322,19 @@ def cpu_baseline(np, dx):
     out = np.empty(8192, dtype=np.float32)
     shX, shP = dx.i32arr([rows, 8192]), dx.i32arr([8192, 64])
     plan = [(0, X, shX, [1]), (0, X, shX, [0]), (2, X, shX, [1]), (3, X, shX, [1]), (1, P, shP, [1])]
-    nbytes = 0
-    # one untimed pass to fault the pages in, then one timed pass of the 5 distinct ops x 2 keepdims
+    # one untimed pass to fault the pages in, then 5 timed passes of the 5 distinct ops x 2 keepdims; median
     for op, arr, sh, ax in plan:
         orc.orc_faithful_reduce_f32(op, H.hp(arr), sh, 2, dx.i32arr(ax), 1, 0, H.hp(out))
-    t0 = time.perf_counter()
-    for kd in (1, 0):
-        for op, arr, sh, ax in plan:
-            assert orc.orc_faithful_reduce_f32(op, H.hp(arr), sh, 2, dx.i32arr(ax), 1, kd, H.hp(out)) == 0
-            nbytes += arr.nbytes + 8192 * 4
-    dt = time.perf_counter() - t0
+    times = []
+    for _ in range(5):
+        nbytes = 0
+        t0 = time.perf_counter()
+        for kd in (1, 0):
+            for op, arr, sh, ax in plan:
+                assert orc.orc_faithful_reduce_f32(op, H.hp(arr), sh, 2, dx.i32arr(ax), 1, kd, H.hp(out)) == 0
+                nbytes += arr.nbytes + 8192 * 4
+        times.append(time.perf_counter() - t0)
+    dt = sorted(times)[len(times) // 2]
     model = ""
     try:
         with open("/proc/cpuinfo") as f:
@@ -342,7 +345,7 @@ def cpu_baseline(np, dx):
     except OSError:
         pass
     return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": f"one full config-2 step (10 ops, {nbytes} bytes) in {dt:.2f} s; OMP threads={cores}; cpu='{model}'; -O2, AVX2 auto-vectorisation"}
+            "sample": f"full config-2 step (10 ops, {nbytes} bytes), median of 5 timed passes after 1 warm-up: {dt:.2f} s; OMP threads={cores}; cpu='{model}'; -O2, AVX2 auto-vectorisation"}
 
 
 if __name__ == "__main__":

@@ -289,8 +289,97 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
         c5[label] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_matmul(dx.F32, ptr(Am), ptr(Bm), ptr(Cm), 1, mm, kk, nn, None)),
                           flops=2 * mm * kk * nn, peak_tf=MFMA_F32_PEAK_TF, peak_name="frac_mfma_f32")
         c5[label]["hipblaslt_TFLOP/s"] = vendor_gemm_tflops(torch, Am.view(mm, kk), Bm.view(kk, nn), Cm.view(mm, nn))
+    del Am, Bm, Cm
+    torch.cuda.empty_cache()
+    c5["mlp_block_over_deepxIR"] = config5_block_over_ir()
     res["config5"] = c5
     return res
+
+
+def config5_block_over_ir(rows=2048, hidden=896, inter=4864, iters=30):
+    """The whole config-5 block (RMSNorm + gated MLP, 22 deepxIR compute ops on [2048,896] activations)
+    through the executor's dispatch core in this process (libdxexec.so, the code behind the UDP
+    server): wall time per block when the lines are executed one by one, as one batch, and as a
+    recorded HIP graph."""
+    import ctypes as C
+    lib = os.path.join(ROOT, "deepx_amd", "executor", "libdxexec.so")
+    if not os.path.exists(lib):
+        raise RuntimeError("libdxexec.so is not built: run `python __graft_entry__.py build`")
+    E = C.CDLL(lib)
+    E.dxe_create.restype = C.c_void_p
+    E.dxe_destroy.argtypes = [C.c_void_p]
+    E.dxe_execute.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_size_t]
+    E.dxe_execute_batch.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_size_t]
+    E.dxe_set_graphs.argtypes = [C.c_void_p, C.c_int]
+    ex = E.dxe_create()
+    buf = C.create_string_buffer(1 << 16)
+
+    def run(line):
+        E.dxe_execute(ex, line.encode(), buf, len(buf))
+        reply = buf.value.decode()
+        if " ok" not in reply.split("//")[0]:
+            raise RuntimeError(f"{line}: {reply}")
+
+    S, Hd, I = rows, hidden, inter
+    b16, f32 = "bfloat16", "float32"
+    T = lambda n, dt=f32: f"tensor<{dt}>:{n}"
+    V = lambda v: "vector<int32>:[" + " ".join(str(x) for x in v) + "]"
+    tensors = [("x", [S, Hd], b16), ("w", [1, Hd], b16), ("Wg", [Hd, I], b16), ("Wu", [Hd, I], b16), ("Wd", [I, Hd], b16),
+               ("xf", [S, Hd], f32), ("sq", [S, Hd], f32), ("var", [S, 1], f32), ("rs", [S, Hd], f32), ("xn", [S, Hd], f32),
+               ("wf1", [1, Hd], f32), ("wf", [S, Hd], f32), ("h", [S, Hd], b16), ("g", [S, I], b16), ("u", [S, I], b16),
+               ("sg", [S, I], b16), ("y", [S, Hd], b16)]
+    for name, shape, dt in tensors:
+        run(f"newtensor({V(shape)})->({T('b5_' + name, dt)})")
+    run(f"normal(var<float32>:0, var<float32>:1, var<int32>:14)->({T('b5_x', b16)}) // author=miaobyte")
+    run(f"constant(var<float32>:1)->({T('b5_w', b16)}) // author=miaobyte")
+    for name, seed in (("Wg", 15), ("Wu", 16), ("Wd", 17)):
+        run(f"normal(var<float32>:0, var<float32>:0.02, var<int32>:{seed})->({T('b5_' + name, b16)}) // author=miaobyte")
+    n = lambda name, dt=f32: T("b5_" + name, dt)
+    block = [f"todtype({n('x', b16)})->({n('xf')})",
+             f"powscalar({n('xf')}, var<float32>:2)->({n('sq')})",
+             f"sum({n('sq')}, {V([-1])}, var<bool>:True)->({n('var')})",
+             f"divscalar({n('var')}, var<float32>:{Hd})->({n('var')})",
+             f"addscalar({n('var')}, var<float32>:1e-06)->({n('var')})",
+             f"sqrt({n('var')})->({n('var')})",
+             f"rdivscalar(var<float32>:1, {n('var')})->({n('var')})",
+             f"broadcastTo({n('var')}, {V([S, Hd])})->({n('rs')})",
+             f"mul({n('xf')}, {n('rs')})->({n('xn')})",
+             f"todtype({n('w', b16)})->({n('wf1')})",
+             f"broadcastTo({n('wf1')}, {V([S, Hd])})->({n('wf')})",
+             f"mul({n('wf')}, {n('xn')})->({n('xn')})",
+             f"todtype({n('xn')})->({n('h', b16)})",
+             f"matmul({n('h', b16)}, {n('Wg', b16)})->({n('g', b16)})",
+             f"matmul({n('h', b16)}, {n('Wu', b16)})->({n('u', b16)})",
+             f"mulscalar({n('g', b16)}, var<float32>:-1)->({n('sg', b16)})",
+             f"exp({n('sg', b16)})->({n('sg', b16)})",
+             f"addscalar({n('sg', b16)}, var<float32>:1)->({n('sg', b16)})",
+             f"rdivscalar(var<float32>:1, {n('sg', b16)})->({n('sg', b16)})",
+             f"mul({n('g', b16)}, {n('sg', b16)})->({n('sg', b16)})",
+             f"mul({n('sg', b16)}, {n('u', b16)})->({n('sg', b16)})",
+             f"matmul({n('sg', b16)}, {n('Wd', b16)})->({n('y', b16)})"]
+    lines = [f"{l} // author=miaobyte id={i + 1}" for i, l in enumerate(block)]
+    text = "\n".join(lines).encode()
+
+    def one_by_one():
+        for l in lines:
+            E.dxe_execute(ex, l.encode(), buf, len(buf))
+
+    def batched():
+        E.dxe_execute_batch(ex, text, buf, len(buf))
+
+    out = {"ops": len(lines), "rows": S}
+    for label, fn, graphs in (("line_by_line_us", one_by_one, 0), ("one_batch_us", batched, 0), ("recorded_graph_us", batched, 1)):
+        E.dxe_set_graphs(ex, graphs)
+        for _ in range(4):
+            fn()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        out[label] = round((time.perf_counter() - t0) / iters * 1e6, 1)
+        if any(" ok" not in r.split("//")[0] for r in buf.value.decode().split("\n")):
+            raise RuntimeError("config-5 block failed: " + buf.value.decode())
+    E.dxe_destroy(ex)
+    return out
 
 
 def vendor_gemm_tflops(torch, A, B, C, reps=20, warm=5):

@@ -29,7 +29,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 MFMA_F32_PEAK_TF = 157.3
 MFMA_BF16_PEAK_TF = 2500.0  # dense bf16
-REDUCE_ROW_TRAFFIC_BYTES = 268646182  # measured, see profiles/bench_pmc_hbm_traffic.md
+REDUCE_ROW_TRAFFIC_BYTES = 268609587  # measured, see profiles/bench_pmc_hbm_traffic.md
 
 
 def main():

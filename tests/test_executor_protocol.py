@@ -191,3 +191,36 @@ def test_inproc_batch_replies_in_order(ex):
     # a batch of one line is the plain path
     assert ex.execute_batch(["argset(var<int32>:9)->(var<int32>:bz) // id=206"])[0].startswith("206 ok//")
     assert ex.stats()["batches"] == before + 1
+
+
+def test_mutated_instructions_never_take_the_process_down(ex):
+    """Seeded mutations (deletions, insertions, substitutions of separator and digit characters) of
+    valid instructions and short random strings: every one gets a reply line and the process lives
+    (the reference unwinds out of its receiver thread on the first malformed line)."""
+    import random
+    rng = random.Random(1234)
+    seeds = ["add(tensor<float32>:a, tensor<float32>:b)->(tensor<float32>:c) // author=miaobyte id=1 created_at=1.5 sent_at=2.5",
+             "sum(tensor<float32>:x, vector<int32>:[0 1], var<bool>:true)->(tensor<float32>:y) // id=2",
+             "argset(var<int32>:5)->(var<int32>:n) // id=4", "vecset(vector<int32>:[1 2 3])->(vector<int32>:v) // id=5",
+             "concat(listtensor<float32>:[a b c], var<int32>:1)->(tensor<float32>:o) // id=6",
+             "transpose(tensor<any>:a, vector<int32>:[1 0])->(tensor<any>:b) // benchmark.repeat=3 id=7",
+             "load(var<string>:/nonexistent/path)->() // id=8", "print(tensor<any>:zzz, var<string>:%f)->() // id=9"]
+    alphabet = "()<>[],:->/= \t|abcxyz0123456789.-+eE%\"'\\"
+    for _ in range(3000):
+        if rng.randrange(4) == 0:
+            s = "".join(rng.choice(alphabet) for _ in range(rng.randrange(0, 80)))
+        else:
+            chars = list(rng.choice(seeds))
+            for _ in range(rng.randrange(1, 6)):
+                pos = rng.randrange(len(chars)) if chars else 0
+                kind = rng.randrange(3)
+                if kind == 0 and chars:
+                    del chars[pos]
+                elif kind == 1:
+                    chars.insert(pos, rng.choice(alphabet))
+                elif chars:
+                    chars[pos] = rng.choice(alphabet)
+            s = "".join(chars)
+        reply = ex.execute(s)
+        assert " ok//" in reply or " error//" in reply, (s, reply)
+    assert ex.execute("argset(var<int32>:1)->(var<int32>:alive) // id=99").startswith("99 ok//")

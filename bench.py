@@ -291,6 +291,32 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
         c5[label]["hipblaslt_TFLOP/s"] = vendor_gemm_tflops(torch, Am.view(mm, kk), Bm.view(kk, nn), Cm.view(mm, nn))
     del Am, Bm, Cm
     torch.cuda.empty_cache()
+    # the glue ops of the block at their own sizes (7-20 MB tensors: they fit the 256 MiB Infinity
+    # Cache, so the rates are cache rates and say little about HBM; 6 buffer sets are rotated anyway)
+    S, Hd, I, R6 = 2048, 896, 4864, 6
+    g16 = [torch.randn(S * I, device=dev).to(torch.bfloat16) for _ in range(R6)]
+    u16 = [torch.randn(S * I, device=dev).to(torch.bfloat16) for _ in range(R6)]
+    o16 = [torch.empty(S * I, device=dev, dtype=torch.bfloat16) for _ in range(R6)]
+    x16 = [torch.randn(S * Hd, device=dev).to(torch.bfloat16) for _ in range(R6)]
+    x32 = [torch.randn(S * Hd, device=dev) for _ in range(R6)]
+    o32 = [torch.empty(S * Hd, device=dev) for _ in range(R6)]
+    col = [torch.rand(S, device=dev) + 0.5 for _ in range(R6)]
+    n16, n32 = S * I, S * Hd
+    one, two, neg = dx.scalar(1.0), dx.scalar(2.0), dx.scalar(-1.0)
+    shx, ax1, shc, shb = dx.i32arr([S, Hd]), dx.i32arr([1]), dx.i32arr([S, 1]), dx.i32arr([S, Hd])
+    glue = {
+        "mulscalar_bf16_2048x4864": (lambda i: L.dxh_mulscalar(dx.BF16, ptr(g16[i % R6]), neg, ptr(o16[i % R6]), n16, None), 2 * n16 * 2),
+        "exp_bf16_2048x4864": (lambda i: L.dxh_exp(dx.BF16, ptr(g16[i % R6]), ptr(o16[i % R6]), n16, None), 2 * n16 * 2),
+        "rdivscalar_bf16_2048x4864": (lambda i: L.dxh_rdivscalar(dx.BF16, one, ptr(g16[i % R6]), ptr(o16[i % R6]), n16, None), 2 * n16 * 2),
+        "mul_bf16_2048x4864": (lambda i: L.dxh_mul(dx.BF16, ptr(g16[i % R6]), ptr(u16[i % R6]), ptr(o16[i % R6]), n16, None), 3 * n16 * 2),
+        "todtype_bf16_to_f32_2048x896": (lambda i: L.dxh_todtype(dx.BF16, ptr(x16[i % R6]), dx.F32, ptr(o32[i % R6]), n32, None), n32 * 6),
+        "powscalar_f32_2048x896": (lambda i: L.dxh_powscalar(dx.F32, ptr(x32[i % R6]), two, ptr(o32[i % R6]), n32, None), 2 * n32 * 4),
+        "sum_f32_2048x896_axis1_keepdims": (lambda i: L.dxh_sum(dx.F32, ptr(x32[i % R6]), shx, 2, ax1, 1, ptr(col[i % R6]), None, 0, None), n32 * 4 + S * 4),
+        "broadcastTo_f32_2048x1_to_2048x896": (lambda i: L.dxh_broadcastTo(dx.F32, ptr(col[i % R6]), shc, 2, shb, 2, ptr(o32[i % R6]), None), n32 * 4 + S * 4),
+    }
+    c5["glue_ops(cache-resident sizes)"] = {k: entry(time_op(L, dx, torch, Events, ev, fn), nb) for k, (fn, nb) in glue.items()}
+    del g16, u16, o16, x16, x32, o32, col
+    torch.cuda.empty_cache()
     c5["mlp_block_over_deepxIR"] = config5_block_over_ir()
     res["config5"] = c5
     return res

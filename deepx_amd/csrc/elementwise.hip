@@ -40,6 +40,8 @@ struct OpPow {
     __device__ static double f(double a, double b) { return pow(a, b); }
 };
 struct OpRPow { template <typename A> __device__ static A f(A a, A b) { return OpPow::f(b, a); } };
+// pow(x, 2): the correctly rounded value is x*x (one rounding), including signed zeros, infinities and NaN
+struct OpSquare { template <typename A> __device__ static A f(A a) { return a * a; } };
 
 struct OpSqrt { __device__ static float f(float a) { return sqrtf(a); } __device__ static double f(double a) { return sqrt(a); } };
 struct OpExp { __device__ static float f(float a) { return expf(a); } __device__ static double f(double a) { return exp(a); } };
@@ -295,7 +297,12 @@ int dxh_divscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, vo
 int dxh_rdivscalar(int dtype, dxh_scalar s, const void *a, void *c, int64_t n, void *stream) { return scalar_all<OpRDiv>(dtype, a, s, c, n, stream); }
 int dxh_maxscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) { return scalar_all<OpMax>(dtype, a, s, c, n, stream); }
 int dxh_minscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) { return scalar_all<OpMin>(dtype, a, s, c, n, stream); }
-int dxh_powscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) { return scalar_f32f64<OpPow>(dtype, a, s, c, n, stream); }
+int dxh_powscalar(int dtype, const void *a, dxh_scalar s, void *c, int64_t n, void *stream) {
+    // the square (RMSNorm's powscalar(x, 2)) skips the general powf/pow expansion: 1.8 M floats took
+    // 11.5 us through it, a launch-bound 4 us as x*x
+    if (s.f == 2.0 && (dtype == DXH_F32 || dtype == DXH_F64)) return unary_float<OpSquare, false>(dtype, a, c, n, stream);
+    return scalar_f32f64<OpPow>(dtype, a, s, c, n, stream);
+}
 int dxh_rpowscalar(int dtype, dxh_scalar s, const void *a, void *c, int64_t n, void *stream) { return scalar_f32f64<OpRPow>(dtype, a, s, c, n, stream); }
 
 int dxh_sqrt(int dtype, const void *a, void *c, int64_t n, void *stream) { return unary_float<OpSqrt, true>(dtype, a, c, n, stream); }

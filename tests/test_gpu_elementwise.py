@@ -101,6 +101,12 @@ def test_powscalar(dxh, orc, dtype):
     # x**2 must equal x*x to 1 ulp (closed form)
     got, _ = run_scalar(dxh, orc, "powscalar", dtype, a, 2.0)
     assert H.ulp_diff(got, (a * a).astype(a.dtype), dtype) <= 1
+    # the square has its own kernel: special values must come out as pow(x, 2) gives them
+    sp = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, -3.0, 1e-30, -1e30, 1e30, np.finfo(a.dtype).tiny], dtype=a.dtype)
+    got, want = run_scalar(dxh, orc, "powscalar", dtype, sp, 2.0)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(got[ok], want[ok]) and np.array_equal(np.signbit(got[ok]), np.signbit(want[ok])), (got, want)
 
 
 def run_unary(dxh, orc, name, dtype, a):

@@ -95,6 +95,7 @@ struct Tuning {
     int64_t reduce_col_max_lanes = 128;           // DXH_TUNE_REDUCE_COL_MAX_LANES
     int64_t reduce_row_loads = 4;                 // DXH_TUNE_REDUCE_ROW_LOADS: vectors per lane a row group aims for
     int64_t matmul_tile = 0;                      // DXH_TUNE_MATMUL_TILE: 0 = chosen per shape
+    int64_t matmul_splitk = 0;                    // DXH_TUNE_MATMUL_SPLITK: 0 = chosen per shape, 1 = never, n = n slices
 };
 Tuning &tuning();  // runtime.hip
 inline bool use_nt_store(size_t out_bytes) { return (int64_t)out_bytes > tuning().nt_store_bytes; }

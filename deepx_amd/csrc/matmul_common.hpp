@@ -65,6 +65,68 @@ inline int compute_units() {
 }
 
 
+// ---- split-K -------------------------------------------------------------------------------
+// A product with few output tiles and a long K leaves most CUs idle.  Such a product is cut along
+// K into `splits` slices of `ksub` (a multiple of the kernel's K step): the slice of workgroup
+// batch index x is x % splits of batch x / splits, its partial tile goes to a workspace in the
+// accumulator type, laid out [batch][split][M][N], and splitk_reduce_kernel adds the slices in
+// slice order (same result on every run) and rounds once to the output type.  The workspace
+// (splitk_workspace, runtime.hip) is a grow-only buffer owned by the library, one per stream, so
+// calls on different streams do not share it; a stream under graph capture never splits, because
+// a recorded pointer would not survive the buffer growing.  Cutting pays for a second launch
+// only when the uncut K loop is long: K >= min_k, slices of at least min_k / 4.
+struct KSplit { int splits, ksub; };
+void *splitk_workspace(hipStream_t st, size_t bytes);  // nullptr when the allocation fails
+void splitk_release(hipStream_t st);
+inline KSplit choose_ksplit(int64_t tiles, int64_t k, int kstep, int64_t min_k, int64_t partial_bytes, hipStream_t st) {
+    KSplit r{1, (int)k};
+    const int64_t cus = compute_units(), ksteps = (k + kstep - 1) / kstep, knob = tuning().matmul_splitk;
+    int64_t want;
+    if (knob == 1) return r;
+    if (knob >= 2) {
+        want = knob;
+    } else {
+        if (tiles * 2 > cus || k < min_k) return r;
+        want = (2 * cus + tiles - 1) / tiles;  // two workgroups per CU
+        if (want > 4 * k / min_k) want = 4 * k / min_k;
+    }
+    if (want > ksteps) want = ksteps;
+    if (want > 1024) want = 1024;
+    if (want < 2 || want * partial_bytes > ((int64_t)1 << 28)) return r;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess) { (void)hipGetLastError(); return r; }
+    if (cap != hipStreamCaptureStatusNone) return r;
+    const int64_t per = (ksteps + want - 1) / want;
+    r.ksub = (int)(per * kstep);
+    r.splits = (int)((k + r.ksub - 1) / r.ksub);
+    if (r.splits < 2) return KSplit{1, (int)k};
+    return r;
+}
+
+template <typename TA, typename TO> __device__ __forceinline__ TO splitk_round(TA v) {
+    if constexpr (std::is_same_v<TA, TO>) return v;
+    else return store_acc<TO>(v);
+}
+// out[b][e] = sum over s (ascending) of ws[b][s][e]; one element per lane and trip (coalesced)
+template <typename TA, typename TO>
+__global__ __launch_bounds__(kBlock) void splitk_reduce_kernel(const TA *__restrict__ ws, TO *__restrict__ out, int splits, int64_t mn, int64_t total) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t b = i / mn, e = i - b * mn;
+        const TA *p = ws + b * splits * mn + e;
+        TA acc = p[0];
+        for (int s = 1; s < splits; ++s) acc += p[(int64_t)s * mn];
+        out[i] = splitk_round<TA, TO>(acc);
+    }
+}
+template <typename TA, typename TO>
+int launch_splitk_reduce(const TA *ws, TO *out, int64_t batch, int64_t mn, int splits, hipStream_t st) {
+    const int64_t total = batch * mn;
+    int64_t blocks = (total + kBlock - 1) / kBlock;
+    if (blocks > 8192) blocks = 8192;
+    splitk_reduce_kernel<TA, TO><<<(unsigned)blocks, kBlock, 0, st>>>(ws, out, splits, mn, total);
+    return launch_status();
+}
+
 // entry points of the per-dtype translation units (matmul_half.hip, matmul_fp.hip)
 int launch_matmul_half(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
 int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);

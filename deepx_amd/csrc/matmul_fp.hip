@@ -19,19 +19,22 @@ namespace dxh {
 //          clamped rows/columns; otherwise element-wise accesses with bounds checks.
 template <int FM, int FN, int FK, int PD, bool VEC>
 __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float *__restrict__ A, const float *__restrict__ B,
-                                                                    float *__restrict__ C, int M, int K, int N, TileMap map) {
+                                                                    float *__restrict__ C, int M, int lda, int N, TileMap map, KSplit ks) {
     constexpr int TM = 64 * FM, TN = 64 * FN, FA_ROW = FK + 4, FB_ROW = TN + 4;
     constexpr int STAGE = TM * FA_ROW + FK * FB_ROW;  // floats
     constexpr int CA = FK / 4, CB = TN / 4;           // 16-byte chunks per A row / B row
     constexpr int A_LD = TM * CA / kBlock, B_LD = FK * CB / kBlock;
     constexpr int HK = FK / 2;                        // k values per lane half
     typedef float f32x4 __attribute__((ext_vector_type(4)));
-    __shared__ __attribute__((aligned(16))) float lds[2 * STAGE];
+    constexpr int LDS_FLOATS = 2 * STAGE > TM * (TN + 4) ? 2 * STAGE : TM * (TN + 4);  // K-loop stages, then the result tile
+    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     const TileCoord tc = tile_of_block(map);
     if (!tc.valid) return;
     const int tm = tc.tm, tn = tc.tn;
-    A += tc.batch * (int64_t)M * K;
-    B += tc.batch * (int64_t)K * N;
+    // K slice of this workgroup: rows of A keep their pitch lda, K is the length of the slice
+    const int slice = tc.batch % ks.splits, kbase = slice * ks.ksub, K = lda - kbase < ks.ksub ? lda - kbase : ks.ksub;
+    A += (tc.batch / ks.splits) * (int64_t)M * lda + kbase;
+    B += ((tc.batch / ks.splits) * (int64_t)lda + kbase) * N;
     C += tc.batch * (int64_t)M * N;
     const int m0 = tm * TM, n0 = tn * TN;
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
@@ -42,13 +45,13 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
         static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
             const int id = t + kBlock * i, row = id / CA, kk = k0 + (id % CA) * 4, gm = m0 + row;
             if constexpr (VEC) {
-                const float *p = A + (int64_t)(gm < M ? gm : M - 1) * K + (kk < K ? kk : 0);
+                const float *p = A + (int64_t)(gm < M ? gm : M - 1) * lda + (kk < K ? kk : 0);
                 f32x4 v = *reinterpret_cast<const f32x4 *>(p);
                 ra[set][i] = (kk < K) ? v : f32x4{0.f, 0.f, 0.f, 0.f};
             } else {
                 f32x4 v;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = (gm < M && kk + e < K) ? A[(int64_t)gm * K + kk + e] : 0.f;
+                for (int e = 0; e < 4; ++e) v[e] = (gm < M && kk + e < K) ? A[(int64_t)gm * lda + kk + e] : 0.f;
                 ra[set][i] = v;
             }
         });
@@ -133,25 +136,36 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
     }
     if (kt < KT) compute(ic<0>{});
 
-    // result lane: row m = lane%32 of its MFMA tile; register group g holds columns 8g + 4h .. +3
+    // Result lane: row m = lane%32 of its MFMA tile; register group g holds columns 8g + 4h .. +3.
+    // The tile goes through LDS (rows padded by 4 floats: the 16 lanes of a ds_write_b128 phase
+    // hit 16 different bank quads) so that every global store instruction writes whole rows of
+    // the tile: a short-K product is bound by this store stream.
+    constexpr int LDC = TN + 4;
+    __syncthreads();
     static_for<FM>([&](auto i) __attribute__((always_inline)) {
         static_for<FN>([&](auto j) __attribute__((always_inline)) {
-            const int gm = m0 + wm * 32 * FM + 32 * i + l32;
+            float *p = lds + (wm * 32 * FM + 32 * i + l32) * LDC + wn * 32 * FN + 32 * j + 4 * h;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int gn = n0 + wn * 32 * FN + 32 * j + 8 * g + 4 * h;
-                if constexpr (VEC) {
-                    if (gm < M && gn < N)
-                        __builtin_nontemporal_store(f32x4{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]},
-                                                    reinterpret_cast<f32x4 *>(C + (int64_t)gm * N + gn));
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (gm < M && gn + e < N) C[(int64_t)gm * N + gn + e] = acc[i][j][4 * g + e];
-                }
-            }
+            for (int g = 0; g < 4; ++g)
+                *reinterpret_cast<f32x4 *>(p + 8 * g) = f32x4{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
         });
     });
+    __syncthreads();
+    if constexpr (VEC) {
+#pragma unroll
+        for (int i = 0; i < TM * CB / kBlock; ++i) {
+            const int id = t + kBlock * i, row = id / CB, col = (id % CB) * 4, gm = m0 + row, gn = n0 + col;
+            if (gm < M && gn < N)
+                __builtin_nontemporal_store(*reinterpret_cast<const f32x4 *>(lds + row * LDC + col),
+                                            reinterpret_cast<f32x4 *>(C + (int64_t)gm * N + gn));
+        }
+    } else {
+#pragma unroll 4
+        for (int i = 0; i < TM * TN / kBlock; ++i) {
+            const int id = t + kBlock * i, row = id / TN, col = id % TN, gm = m0 + row, gn = n0 + col;
+            if (gm < M && gn < N) C[(int64_t)gm * N + gn] = lds[row * LDC + col];
+        }
+    }
 }
 
 // ---- fp64 MFMA kernel ------------------------------------------------------------------------
@@ -165,7 +179,7 @@ typedef double f64x4 __attribute__((ext_vector_type(4)));
 typedef double f64x2 __attribute__((ext_vector_type(2)));
 template <int FM, int FN, bool VEC>
 __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double *__restrict__ A, const double *__restrict__ B,
-                                                                    double *__restrict__ C, int M, int K, int N, TileMap map) {
+                                                                    double *__restrict__ C, int M, int lda, int N, TileMap map, KSplit ks) {
     constexpr int DK = 16, TM = 64 * FM, TN = 64 * FN, DA_ROW = DK + 2, DB_ROW = TN + 4;
     constexpr int STAGE = TM * DA_ROW + DK * DB_ROW;  // doubles
     constexpr int CA = DK / 2, CB = TN / 2;           // 16-byte chunks per A row / B row
@@ -175,8 +189,9 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double
     const TileCoord tc = tile_of_block(map);
     if (!tc.valid) return;
     const int tm = tc.tm, tn = tc.tn;
-    A += tc.batch * (int64_t)M * K;
-    B += tc.batch * (int64_t)K * N;
+    const int slice = tc.batch % ks.splits, kbase = slice * ks.ksub, K = lda - kbase < ks.ksub ? lda - kbase : ks.ksub;  // K slice, as in the fp32 kernel
+    A += (tc.batch / ks.splits) * (int64_t)M * lda + kbase;
+    B += ((tc.batch / ks.splits) * (int64_t)lda + kbase) * N;
     C += tc.batch * (int64_t)M * N;
     const int m0 = tm * TM, n0 = tn * TN;
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
@@ -186,13 +201,13 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double
         static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
             const int id = t + kBlock * i, row = id / CA, kk = k0 + (id % CA) * 2, gm = m0 + row;
             if constexpr (VEC) {
-                const double *p = A + (int64_t)(gm < M ? gm : M - 1) * K + (kk < K ? kk : 0);
+                const double *p = A + (int64_t)(gm < M ? gm : M - 1) * lda + (kk < K ? kk : 0);
                 f64x2 v = *reinterpret_cast<const f64x2 *>(p);
                 ra[i] = (kk < K) ? v : f64x2{0.0, 0.0};
             } else {
                 f64x2 v;
 #pragma unroll
-                for (int e = 0; e < 2; ++e) v[e] = (gm < M && kk + e < K) ? A[(int64_t)gm * K + kk + e] : 0.0;
+                for (int e = 0; e < 2; ++e) v[e] = (gm < M && kk + e < K) ? A[(int64_t)gm * lda + kk + e] : 0.0;
                 ra[i] = v;
             }
         });
@@ -273,14 +288,37 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double
     });
 }
 
+// Launch of one tile shape, cut along K when choose_ksplit says so: the slices then write fp32 /
+// fp64 partial tiles into the stream's workspace and splitk_reduce_kernel adds them up.
+template <typename T, typename Launch>
+int launch_fp_tile(Launch launch, int tm, int tn, int kstep, int64_t min_k, T *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn), partial = batch * m * n * (int64_t)sizeof(T);
+    const KSplit ks = choose_ksplit(tiles, k, kstep, min_k, partial, st);
+    TileMap map;
+    if (!make_tile_map(batch * ks.splits, m, n, tm, tn, map)) return DXH_ERR_SHAPE;
+    const unsigned blocks = (unsigned)(8 * map.chunk);
+    if (ks.splits == 1) {
+        launch(blocks, c, map, ks);
+        return launch_status();
+    }
+    T *ws = (T *)splitk_workspace(st, (size_t)(partial * ks.splits));
+    if (!ws) {  // no workspace: one slice
+        const KSplit one{1, (int)k};
+        if (!make_tile_map(batch, m, n, tm, tn, map)) return DXH_ERR_SHAPE;
+        launch((unsigned)(8 * map.chunk), c, map, one);
+        return launch_status();
+    }
+    launch(blocks, ws, map, ks);
+    const int rc = launch_status();
+    return rc != DXH_OK ? rc : launch_splitk_reduce<T, T>(ws, c, batch, m * n, ks.splits, st);
+}
+
 template <int FM, int FN, int FK, int PD>
 int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, hipStream_t st) {
-    TileMap map;
-    if (!make_tile_map(batch, m, n, 64 * FM, 64 * FN, map)) return DXH_ERR_SHAPE;
-    const unsigned blocks = (unsigned)(8 * map.chunk);
-    if (vec) matmul_mfma_f32_kernel<FM, FN, FK, PD, true><<<blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, map);
-    else matmul_mfma_f32_kernel<FM, FN, FK, PD, false><<<blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, map);
-    return launch_status();
+    return launch_fp_tile<float>([&](unsigned blocks, float *out, const TileMap &map, KSplit ks) {
+        if (vec) matmul_mfma_f32_kernel<FM, FN, FK, PD, true><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks);
+        else matmul_mfma_f32_kernel<FM, FN, FK, PD, false><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks);
+    }, 64 * FM, 64 * FN, FK, 1024, c, batch, m, k, n, st);
 }
 
 // fp32: the matrix pipe is the bound, so the tile is chosen for CU balance.  Cost model per tile
@@ -316,12 +354,10 @@ int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int6
 
 template <int FM, int FN>
 int launch_f64_tile(const double *a, const double *b, double *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, hipStream_t st) {
-    TileMap map;
-    if (!make_tile_map(batch, m, n, 64 * FM, 64 * FN, map)) return DXH_ERR_SHAPE;
-    const unsigned blocks = (unsigned)(8 * map.chunk);
-    if (vec) matmul_mfma_f64_kernel<FM, FN, true><<<blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, map);
-    else matmul_mfma_f64_kernel<FM, FN, false><<<blocks, kBlock, 0, st>>>(a, b, c, (int)m, (int)k, (int)n, map);
-    return launch_status();
+    return launch_fp_tile<double>([&](unsigned blocks, double *out, const TileMap &map, KSplit ks) {
+        if (vec) matmul_mfma_f64_kernel<FM, FN, true><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks);
+        else matmul_mfma_f64_kernel<FM, FN, false><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks);
+    }, 64 * FM, 64 * FN, 16, 512, c, batch, m, k, n, st);
 }
 
 // fp64 on the matrix pipe; tile chosen for CU balance like fp32 (efficiencies measured on 4096^3)

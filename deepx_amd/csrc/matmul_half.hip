@@ -1,5 +1,5 @@
 // matmul_half.hip — bf16 / f16 GEMM on the matrix pipe (v_mfma_f32_32x32x16_{bf16,f16}, fp32
-// accumulate, one RNE rounding of C).  Aligned shapes (K % 64 == 0, N % 8 == 0) take
+// accumulate, one RNE rounding of C).  Aligned shapes (K % 8 == 0, N % 8 == 0) take
 // matmul_mfma_tile_kernel, 64x64 to 256x256 workgroup tiles, software-pipelined over K; anything
 // else takes matmul_mfma_kernel, a plain 128x128x32 tile with element-wise edge handling.
 #include "matmul_common.hpp"
@@ -109,8 +109,9 @@ __device__ inline int swz(int row, int chunk) { return chunk ^ ((row ^ (row >> 3
 
 // ---- MFMA kernel with the B transposition done by the LDS read ------------------------------
 // Workgroup tile TM x TN (64, 128 or 256 each), K step 64, 4 waves in a 2x2 grid, each wave a
-// (TM/2) x (TN/2) patch of 32x32x16 MFMAs.  Requirements (checked by the launcher): K % 64 == 0,
-// N % 8 == 0, 16-byte aligned A, B, C.
+// (TM/2) x (TN/2) patch of 32x32x16 MFMAs.  Requirements (checked by the launcher): K % 8 == 0,
+// N % 8 == 0, 16-byte aligned A, B, C.  KTAIL (K % 64 != 0): chunks of A and rows of B at k >= K
+// are read from clamped addresses and replaced by zeros.
 //   loads  every global load is 16 bytes per lane (a wave instruction occupies the vector cache for
 //          the same 16 cycles whatever its width, so 8-byte loads halve its throughput).
 //   A      [TM m][64 k] in LDS, 128-byte rows, 16-byte chunk c of row r at chunk c ^ swizzle(r).
@@ -142,9 +143,9 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t *p) {
 constexpr int part_first(int count, int part) { return count * part / 4; }
 constexpr int part_count(int count, int part) { return count * (part + 1) / 4 - count * part / 4; }
 
-template <typename T, int TM, int TN, int PD>
+template <typename T, int TM, int TN, int PD, bool KTAIL, bool SPLIT>
 __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul_mfma_tile_kernel(
-    const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int K, int N, TileMap map) {
+    const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, float *__restrict__ partial, int M, int lda, int N, TileMap map, KSplit ks) {
     static_assert(TM % 64 == 0 && (TN == 64 || TN == 128 || TN == 256), "B rows must split evenly over the 256 lanes");
     constexpr int FM = TM / 64, FN = TN / 64;      // 32x32 MFMA tiles per wave along m and n
     constexpr int A_LD = TM / 32, B_LD = TN / 32;  // 16-byte global loads per lane per K step
@@ -158,12 +159,15 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
 
     const TileCoord tc = tile_of_block(map);
     if (!tc.valid) return;
-    const int batch = tc.batch, tm = tc.tm, tn = tc.tn;
+    // SPLIT: the workgroup multiplies K slice tc.batch % splits of batch tc.batch / splits (rows of
+    // A keep their pitch lda, K is the slice length) and stores an fp32 partial tile.
+    const int batch = SPLIT ? tc.batch / ks.splits : tc.batch, tm = tc.tm, tn = tc.tn;
+    const int kbase = SPLIT ? (tc.batch % ks.splits) * ks.ksub : 0, K = SPLIT ? (lda - kbase < ks.ksub ? lda - kbase : ks.ksub) : lda;
     const int m0 = tm * TM, n0 = tn * TN;
 
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
-    const uint16_t *Ab = reinterpret_cast<const uint16_t *>(A) + ((int64_t)batch * M + m0) * K;
-    const uint16_t *Bb = reinterpret_cast<const uint16_t *>(B) + (int64_t)batch * K * N + n0;
+    const uint16_t *Ab = reinterpret_cast<const uint16_t *>(A) + ((int64_t)batch * M + m0) * lda + kbase;
+    const uint16_t *Bb = reinterpret_cast<const uint16_t *>(B) + ((int64_t)batch * lda + kbase) * N + n0;
 
     // Branch-free loads: rows past M and columns past N are clamped onto valid memory; their
     // products land in accumulator rows/columns that the epilogue never stores.
@@ -171,33 +175,50 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
     int a_off[A_LD], a_lds[A_LD];
     static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
         const int r = arow + 32 * i;
-        a_off[i] = (m0 + r < M ? r : M - 1 - m0) * K + ach * 8;
+        a_off[i] = (m0 + r < M ? r : M - 1 - m0) * lda + ach * 8;
         a_lds[i] = r * PK + swz(r, ach) * 8;
     });
     const int brow = t / CB, bch = t % CB;
-    const int b_off = brow * N + (n0 + bch * 8 < N ? bch * 8 : N - 8 - n0);
+    const int b_col = n0 + bch * 8 < N ? bch * 8 : N - 8 - n0, b_off = brow * N + b_col;
     const int b_lds = brow * B_ROW + bch * 8;
 
     u32x4 ra[PD][A_LD], rb[PD][B_LD];
     auto load_part = [&](auto set, auto part, int k0) __attribute__((always_inline)) {
         static_for<part_count(A_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
             constexpr int i = part_first(A_LD, decltype(part)::value) + decltype(q)::value;
-            ra[set][i] = *reinterpret_cast<const u32x4 *>(Ab + a_off[i] + k0);
+            if constexpr (KTAIL) {
+                ra[set][i] = *reinterpret_cast<const u32x4 *>(Ab + a_off[i] + (k0 + ach * 8 < K ? k0 : K - 8 - ach * 8));
+            } else {
+                ra[set][i] = *reinterpret_cast<const u32x4 *>(Ab + a_off[i] + k0);
+            }
         });
         static_for<part_count(B_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
             constexpr int i = part_first(B_LD, decltype(part)::value) + decltype(q)::value;
-            rb[set][i] = *reinterpret_cast<const u32x4 *>(Bb + (int64_t)(k0 + i * KR) * N + b_off);
+            if constexpr (KTAIL) {
+                const int gk = k0 + brow + i * KR;
+                rb[set][i] = *reinterpret_cast<const u32x4 *>(Bb + (int64_t)(gk < K ? gk : K - 1) * N + b_col);
+            } else {
+                rb[set][i] = *reinterpret_cast<const u32x4 *>(Bb + (int64_t)(k0 + i * KR) * N + b_off);
+            }
         });
     };
-    auto store_part = [&](auto set, auto part, auto stage) __attribute__((always_inline)) {
+    // k0: the K step that register set `set` holds.  The zero fill of a partial K step happens
+    // here and not at the load, so that nothing waits for a load right after issuing it.
+    auto store_part = [&](auto set, auto part, auto stage, int k0) __attribute__((always_inline)) {
         uint16_t *As = lds + decltype(stage)::value * STAGE, *Bs = As + A_STAGE;
         static_for<part_count(A_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
             constexpr int i = part_first(A_LD, decltype(part)::value) + decltype(q)::value;
-            *reinterpret_cast<u32x4 *>(As + a_lds[i]) = ra[set][i];
+            if constexpr (KTAIL)
+                *reinterpret_cast<u32x4 *>(As + a_lds[i]) = k0 + ach * 8 < K ? ra[set][i] : u32x4{0u, 0u, 0u, 0u};
+            else
+                *reinterpret_cast<u32x4 *>(As + a_lds[i]) = ra[set][i];
         });
         static_for<part_count(B_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
             constexpr int i = part_first(B_LD, decltype(part)::value) + decltype(q)::value;
-            *reinterpret_cast<u32x4 *>(Bs + b_lds + i * KR * B_ROW) = rb[set][i];
+            if constexpr (KTAIL)
+                *reinterpret_cast<u32x4 *>(Bs + b_lds + i * KR * B_ROW) = k0 + brow + i * KR < K ? rb[set][i] : u32x4{0u, 0u, 0u, 0u};
+            else
+                *reinterpret_cast<u32x4 *>(Bs + b_lds + i * KR * B_ROW) = rb[set][i];
         });
     };
 
@@ -252,19 +273,19 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
     // S^1 and is refilled with the K step PD further on.  Fragment buffer 0 holds substep 0 on
     // entry.  The last substep straddles the barrier: half of its MFMAs are queued before it and
     // the other half runs under the first fragment reads of stage S^1.
-    auto step = [&](auto S, auto R, int k_load) __attribute__((always_inline)) {
+    auto step = [&](auto S, auto R, int k_store, int k_load) __attribute__((always_inline)) {
         constexpr int s = decltype(S)::value;
         static_for<4>([&](auto ks) __attribute__((always_inline)) {
             constexpr int cur = decltype(ks)::value & 1;
             constexpr int NW = part_count(A_LD, decltype(ks)::value) + part_count(B_LD, decltype(ks)::value);  // LDS writes = global loads
             if constexpr (decltype(ks)::value < 3) {
                 read_frags(ic<cur ^ 1>{}, S, ic<decltype(ks)::value + 1>{});
-                store_part(R, ks, ic<s ^ 1>{});
+                store_part(R, ks, ic<s ^ 1>{}, k_store);
                 load_part(R, ks, k_load);
                 mma(ic<cur>{}, ic<0>{}, ic<NM>{});
                 interleave(ic<NM>{}, ic<ND>{}, ic<NW>{}, ic<NW>{});
             } else {
-                store_part(R, ks, ic<s ^ 1>{});
+                store_part(R, ks, ic<s ^ 1>{}, k_store);
                 load_part(R, ks, k_load);
                 mma(ic<cur>{}, ic<0>{}, ic<NM / 2>{});
                 interleave(ic<NM / 2>{}, ic<0>{}, ic<NW>{}, ic<NW>{});
@@ -278,19 +299,36 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
         });
     };
 
-    const int KT = K / PK;
+    const int KT = (K + PK - 1) / PK;
     auto k_of = [&](int stepno) __attribute__((always_inline)) { return (stepno < KT ? stepno : KT - 1) * PK; };
     static_for<4>([&](auto part) __attribute__((always_inline)) { load_part(ic<0>{}, part, k_of(0)); });
-    static_for<4>([&](auto part) __attribute__((always_inline)) { store_part(ic<0>{}, part, ic<0>{}); });
+    static_for<4>([&](auto part) __attribute__((always_inline)) { store_part(ic<0>{}, part, ic<0>{}, 0); });
     static_for<PD>([&](auto d) __attribute__((always_inline)) { static_for<4>([&](auto part) __attribute__((always_inline)) { load_part(ic<(decltype(d)::value + 1) % PD>{}, part, k_of(decltype(d)::value + 1)); }); });
     __syncthreads();
     read_frags(ic<0>{}, ic<0>{}, ic<0>{});
     int kt = 0;
     for (; kt + 1 < KT; kt += 2) {
-        step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1 + PD));
-        step(ic<1>{}, ic<2 % PD>{}, k_of(kt + 2 + PD));
+        step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1), k_of(kt + 1 + PD));
+        step(ic<1>{}, ic<2 % PD>{}, k_of(kt + 2), k_of(kt + 2 + PD));
     }
-    if (kt < KT) step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1 + PD));
+    if (kt < KT) step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1), k_of(kt + 1 + PD));
+    if constexpr (SPLIT) {
+        // fp32 partial tile straight from the accumulators: 16 bytes (4 consecutive n) per store
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+        float *P = partial + (int64_t)tc.batch * M * N;
+        static_for<FM>([&](auto i) __attribute__((always_inline)) {
+            static_for<FN>([&](auto j) __attribute__((always_inline)) {
+                const int gm = m0 + wm * (TM / 2) + 32 * i + (lane & 31);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int gn = n0 + wn * (TN / 2) + 32 * j + 8 * g + 4 * (lane >> 5);
+                    if (gm < M && gn < N)  // N % 8 == 0: four columns are inside or outside together
+                        *reinterpret_cast<f32x4 *>(P + (int64_t)gm * N + gn) = f32x4{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                }
+            });
+        });
+        return;
+    }
     __syncthreads();
 
     // ---- epilogue: result lane holds row m = lane%32 of its MFMA tile and, per group g of 4
@@ -322,15 +360,44 @@ template <typename T, int TM, int TN, int PD>
 int launch_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     TileMap map;
     if (!make_tile_map(batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
-    matmul_mfma_tile_kernel<T, TM, TN, PD><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map);
+    const KSplit one{1, (int)k};
+    if (k % PK == 0)
+        matmul_mfma_tile_kernel<T, TM, TN, PD, false, false><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one);
+    else
+        matmul_mfma_tile_kernel<T, TM, TN, PD, true, false><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one);
     return launch_status();
+}
+
+// Few output tiles and a long K: 64x64 tiles over K slices, fp32 partial tiles in the stream's
+// workspace, then one pass that adds the slices in order and rounds once.  Returns kNoSplit when the
+// product should not be cut (the caller then launches the ordinary way).
+constexpr int kNoSplit = -1001;  // not a DXH_ERR_* value
+template <typename T>
+int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    constexpr int TM = 64, TN = 64;
+    const int64_t tiles = batch * ((m + TM - 1) / TM) * ((n + TN - 1) / TN), partial = batch * m * n * (int64_t)sizeof(float);
+    const KSplit ks = choose_ksplit(tiles, k, PK, 2048, partial, st);
+    TileMap map;
+    if (ks.splits < 2 || !make_tile_map(batch * ks.splits, m, n, TM, TN, map)) return kNoSplit;
+    float *ws = (float *)splitk_workspace(st, (size_t)(partial * ks.splits));
+    if (!ws) return kNoSplit;
+    if (k % PK == 0)
+        matmul_mfma_tile_kernel<T, TM, TN, 1, false, true><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks);
+    else
+        matmul_mfma_tile_kernel<T, TM, TN, 1, true, true><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks);
+    const int rc = launch_status();
+    return rc != DXH_OK ? rc : launch_splitk_reduce<float, T>(ws, (T *)c, batch, m * n, ks.splits, st);
 }
 
 template <typename T>
 int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    const bool fast = k % PK == 0 && n % 8 == 0 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes) &&
+    const bool fast = k % 8 == 0 && n % 8 == 0 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes) &&
                       k <= (1 << 22) && n <= (1 << 24);
     int64_t choice = tuning().matmul_tile;
+    if (fast && (choice == 0 || choice == 5)) {
+        const int rc = launch_split<T>(a, b, c, batch, m, k, n, st);
+        if (rc != kNoSplit) return rc;
+    }
     if (fast && choice == 0) {
         // 256x256 tiles halve the bytes every CU pulls through its vector cache per flop, but need
         // about one tile per CU to pay off.  Below that, 128x128 tiles (two workgroups per CU) as

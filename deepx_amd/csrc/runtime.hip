@@ -1,7 +1,9 @@
 // runtime.hip — device memory, copies, streams and events behind the C ABI.
 // Replaces the cudaMalloc/cudaFree/cudaMemcpy calls of
 // executor/op-cuda/src/deepx/tensorfunc/tensorlife_miaobyte.hpp:16-68.
-#include "common.hpp"
+#include "matmul_common.hpp"
+#include <map>
+#include <mutex>
 #include <cstdio>
 #include <cstring>
 
@@ -11,6 +13,39 @@ namespace dxh {
 Tuning &tuning() {
     static Tuning t;
     return t;
+}
+}  // namespace dxh
+
+namespace dxh {
+// One grow-only split-K workspace per (device, stream): kernels of one stream run in order, so a
+// buffer per stream is never shared by two products in flight.  Growing frees the old buffer with
+// hipFree, which waits for the device, so work still reading it has finished.
+namespace {
+struct Workspace { void *ptr; size_t bytes; };
+std::mutex g_ws_mutex;
+std::map<std::pair<int, hipStream_t>, Workspace> g_ws;
+}  // namespace
+void *splitk_workspace(hipStream_t st, size_t bytes) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    Workspace &w = g_ws[{dev, st}];
+    if (w.bytes >= bytes) return w.ptr;
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    if (w.ptr) (void)hipFree(w.ptr);
+    w.ptr = p;
+    w.bytes = bytes;
+    return p;
+}
+void splitk_release(hipStream_t st) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return; }
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    auto it = g_ws.find({dev, st});
+    if (it == g_ws.end()) return;
+    if (it->second.ptr) (void)hipFree(it->second.ptr);
+    g_ws.erase(it);
 }
 }  // namespace dxh
 
@@ -30,6 +65,7 @@ int dxh_tune(int knob, int64_t value) {
         return DXH_OK;
     case DXH_TUNE_REDUCE_ROW_LOADS: if (value < 1 || value > 64) return DXH_ERR_ARG; t.reduce_row_loads = value; return DXH_OK;
     case DXH_TUNE_MATMUL_TILE: if (value < 0 || value > 5) return DXH_ERR_ARG; t.matmul_tile = value; return DXH_OK;
+    case DXH_TUNE_MATMUL_SPLITK: if (value < 0 || value > 1024) return DXH_ERR_ARG; t.matmul_splitk = value; return DXH_OK;
     default: return DXH_ERR_ARG;
     }
 }
@@ -102,7 +138,11 @@ int dxh_stream_create(void **stream) {
     *stream = (void *)s;
     return (int)e;
 }
-int dxh_stream_destroy(void *stream) { return stream ? (int)hipStreamDestroy(as_stream(stream)) : DXH_OK; }
+int dxh_stream_destroy(void *stream) {
+    if (!stream) return DXH_OK;
+    dxh::splitk_release(as_stream(stream));
+    return (int)hipStreamDestroy(as_stream(stream));
+}
 int dxh_stream_sync(void *stream) { return (int)hipStreamSynchronize(as_stream(stream)); }
 int dxh_device_sync(void) { return (int)hipDeviceSynchronize(); }
 

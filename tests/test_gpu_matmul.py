@@ -89,12 +89,13 @@ TILE_KNOB = 4  # DXH_TUNE_MATMUL_TILE
 def test_matmul_tile_configs(dxh, dtype, tile):
     """Every workgroup tile of the MFMA kernel (forced through the tuning knob) on aligned shapes
     with ragged tile edges, more than one batch and M, N below one tile; float64 numpy is the
-    reference, bar rel 1e-2 of sum_k |a||b| as above."""
+    reference, bar rel 1e-2 of sum_k |a||b| as above.  K = 72, 8, 1000, 56 end in a partial K step
+    (zero-filled in the kernel)."""
     rng = np.random.default_rng(300 + tile + dtype)
     dx.check(dxh.dxh_tune(TILE_KNOB, tile))
     try:
         for batch, m, k, n in [(2, 300, 128, 264), (1, 520, 192, 520), (3, 70, 64, 8), (1, 257, 64, 1032), (1, 1, 64, 16),
-                               (1, 1024, 448, 768)]:
+                               (1, 1024, 448, 768), (1, 300, 72, 264), (2, 130, 8, 16), (1, 257, 1000, 520), (1, 64, 56, 64)]:
             A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
             B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
             dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, A.dtype)
@@ -113,21 +114,21 @@ def test_matmul_tiles_exact_on_small_integers(dxh):
     summation order: every tile must return the exact product rounded once (RNE) to bf16.  A wrong
     fragment, k-permutation or edge clamp changes an integer and fails bit-exactly."""
     rng = np.random.default_rng(77)
-    m, k, n = 384, 256, 520
-    Ai, Bi = rng.integers(-4, 5, (m, k)), rng.integers(-4, 5, (k, n))
-    A = H.to_storage(Ai.astype(np.float64).reshape(-1), dx.BF16)
-    B = H.to_storage(Bi.astype(np.float64).reshape(-1), dx.BF16)
-    want = (Ai @ Bi).astype(np.float64)  # |sum| <= 16*256 = 4096: exact in fp32
-    dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, np.uint16)
-    for tile in (0, 1, 2, 3, 4, 5):
-        dx.check(dxh.dxh_tune(TILE_KNOB, tile))
-        try:
-            dx.check(dxh.dxh_matmul(dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
-            got = H.to_float(dC.get(), dx.BF16).astype(np.float64).reshape(m, n)
-        finally:
-            dx.check(dxh.dxh_tune(TILE_KNOB, 0))
-        # one RNE rounding of the exact integer to bf16
-        assert np.array_equal(got, H.to_float(H.to_storage(want.reshape(-1), dx.BF16), dx.BF16).astype(np.float64).reshape(m, n)), tile
+    for m, k, n in [(384, 256, 520), (200, 200, 136)]:  # the second K ends in a partial K step
+        Ai, Bi = rng.integers(-4, 5, (m, k)), rng.integers(-4, 5, (k, n))
+        A = H.to_storage(Ai.astype(np.float64).reshape(-1), dx.BF16)
+        B = H.to_storage(Bi.astype(np.float64).reshape(-1), dx.BF16)
+        want = (Ai @ Bi).astype(np.float64)  # |sum| <= 16*256 = 4096: exact in fp32
+        dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, np.uint16)
+        for tile in (0, 1, 2, 3, 4, 5):
+            dx.check(dxh.dxh_tune(TILE_KNOB, tile))
+            try:
+                dx.check(dxh.dxh_matmul(dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+                got = H.to_float(dC.get(), dx.BF16).astype(np.float64).reshape(m, n)
+            finally:
+                dx.check(dxh.dxh_tune(TILE_KNOB, 0))
+            # one RNE rounding of the exact integer to bf16
+            assert np.array_equal(got, H.to_float(H.to_storage(want.reshape(-1), dx.BF16), dx.BF16).astype(np.float64).reshape(m, n)), (tile, k)
 
 
 @pytest.mark.parametrize("tile", [1, 2, 3, 4])
@@ -184,3 +185,100 @@ def test_matmul_f64_tile_configs(dxh, tile):
         assert np.array_equal(dC.get().reshape(m, n), (Ai @ Bi).astype(np.float64))
     finally:
         dx.check(dxh.dxh_tune(TILE_KNOB, 0))
+
+
+SPLITK_KNOB = 6  # DXH_TUNE_MATMUL_SPLITK
+
+
+def _ref_product(A, B, dtype, batch, m, k, n):
+    Af = H.to_float(A, dtype).astype(np.float64).reshape(batch, m, k)
+    Bf = H.to_float(B, dtype).astype(np.float64).reshape(batch, k, n)
+    return np.matmul(Af, Bf), np.matmul(np.abs(Af), np.abs(Bf))
+
+
+@pytest.mark.parametrize("dtype", [dx.BF16, dx.F16, dx.F32, dx.F64])
+@pytest.mark.parametrize("splits", [2, 3, 7])
+def test_matmul_split_k_forced(dxh, dtype, splits):
+    """A product cut into K slices (forced through the tuning knob) against float64 numpy, on
+    batches, ragged tiles, a K that ends in a partial K step and a K shorter than `splits` K steps;
+    same bars as the unsplit kernels.  Small-integer operands must come out exact, and a second
+    run bit-identical (the slices are added in a fixed order)."""
+    rng = np.random.default_rng(700 + dtype + splits)
+    rel = {dx.F32: 1e-5, dx.F64: 1e-13, dx.BF16: 1e-2, dx.F16: 1e-2}[dtype]
+    dx.check(dxh.dxh_tune(SPLITK_KNOB, splits))
+    try:
+        for batch, m, k, n in [(1, 64, 1024, 64), (2, 70, 520, 72), (1, 16, 4096, 136), (3, 1, 200, 8), (1, 130, 64, 64), (1, 33, 1000, 264)]:
+            A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
+            B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
+            dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, A.dtype)
+            dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+            first = dC.get()
+            got = H.to_float(first, dtype).astype(np.float64).reshape(batch, m, n)
+            ref, mag = _ref_product(A, B, dtype, batch, m, k, n)
+            scale = np.sqrt(k) if dtype in (dx.F32, dx.F64) else 1.0
+            assert np.all(np.abs(got - ref) <= rel * scale * np.maximum(mag, 1e-300)), (dtype, splits, batch, m, k, n)
+            dC2 = Dev.empty(batch * m * n, A.dtype)
+            dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC2.ptr, batch, m, k, n, None), "matmul")
+            assert np.array_equal(first, dC2.get()), "split-K result varies between runs"
+        m, k, n = 96, 456, 72
+        Ai, Bi = rng.integers(-4, 5, (m, k)), rng.integers(-4, 5, (k, n))
+        A = H.to_storage(Ai.astype(np.float64).reshape(-1), dtype)
+        B = H.to_storage(Bi.astype(np.float64).reshape(-1), dtype)
+        dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, A.dtype)
+        dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+        want = H.to_float(H.to_storage((Ai @ Bi).astype(np.float64).reshape(-1), dtype), dtype)  # one rounding of the exact integer
+        assert np.array_equal(H.to_float(dC.get(), dtype), want)
+    finally:
+        dx.check(dxh.dxh_tune(SPLITK_KNOB, 0))
+
+
+@pytest.mark.parametrize("dtype", [dx.BF16, dx.F32, dx.F64])
+def test_matmul_skinny_shapes_auto_split(dxh, dtype):
+    """Shapes that the launcher cuts along K by itself (few output tiles, long K), and the same
+    shapes with the knob at 1 (never cut): both within the bar of float64 numpy."""
+    rng = np.random.default_rng(800 + dtype)
+    rel = {dx.F32: 1e-5, dx.F64: 1e-13, dx.BF16: 1e-2}[dtype]
+    for knob in (0, 1):
+        dx.check(dxh.dxh_tune(SPLITK_KNOB, knob))
+        try:
+            for batch, m, k, n in [(1, 1, 4096, 512), (1, 16, 2048, 1024), (1, 64, 20000, 64), (2, 300, 1024, 8)]:
+                A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
+                B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
+                dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, A.dtype)
+                dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+                got = H.to_float(dC.get(), dtype).astype(np.float64).reshape(batch, m, n)
+                ref, mag = _ref_product(A, B, dtype, batch, m, k, n)
+                scale = np.sqrt(k) if dtype in (dx.F32, dx.F64) else 1.0
+                assert np.all(np.abs(got - ref) <= rel * scale * np.maximum(mag, 1e-300)), (dtype, knob, batch, m, k, n)
+        finally:
+            dx.check(dxh.dxh_tune(SPLITK_KNOB, 0))
+
+
+def test_matmul_under_capture_does_not_split(dxh):
+    """A stream under graph capture may not allocate: a matmul that would be cut along K is
+    recorded as one unsplit kernel, and the replayed graph gives the eager result."""
+    import ctypes as C
+    rng = np.random.default_rng(900)
+    m, k, n = 16, 4096, 256
+    A = rng.standard_normal(m * k).astype(np.float32)
+    B = rng.standard_normal(k * n).astype(np.float32)
+    dA, dB, dC, dG = Dev(A), Dev(B), Dev.empty(m * n, np.float32), Dev.empty(m * n, np.float32)
+    dx.check(dxh.dxh_tune(SPLITK_KNOB, 1))
+    try:
+        dx.check(dxh.dxh_matmul(dx.F32, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))  # unsplit, eager
+    finally:
+        dx.check(dxh.dxh_tune(SPLITK_KNOB, 0))
+    want = dC.get()
+    st = C.c_void_p()
+    dx.check(dxh.dxh_stream_create(C.byref(st)))
+    graph = C.c_void_p()
+    dx.check(dxh.dxh_graph_begin_capture(st))
+    rc = dxh.dxh_matmul(dx.F32, dA.ptr, dB.ptr, dG.ptr, 1, m, k, n, st)
+    dx.check(dxh.dxh_graph_end_capture(st, C.byref(graph)))
+    dx.check(rc, "matmul under capture")
+    for _ in range(3):
+        dx.check(dxh.dxh_graph_launch(graph, st))
+        dx.check(dxh.dxh_stream_sync(st))
+        assert np.array_equal(dG.get(), want)
+    dx.check(dxh.dxh_graph_destroy(graph))
+    dx.check(dxh.dxh_stream_destroy(st))

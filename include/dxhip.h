@@ -272,7 +272,11 @@ DXH_API int dxh_dropout(int dtype, void *inout, int64_t n, float p, uint32_t see
  * cblas_sgemm executor/op-ompsimd/src/deepx/tensorfunc/matmul_cblas.hpp:11-60.
  * C[b,m,n] = sum_k A[b,m,k] * B[b,k,n], row-major, alpha=1 beta=0, `batch` = product of
  * the leading dims.  f16/bf16: MFMA with fp32 accumulate, one RNE rounding of the
- * result; f32/f64 accumulate in their own type; integers wrap. */
+ * result; f32/f64 accumulate in their own type; integers wrap.  A float product with few
+ * output tiles and a long K is cut along K (DXH_TUNE_MATMUL_SPLITK) into partial products that
+ * are added in a fixed order; their buffer (at most 256 MiB) belongs to the library, one per
+ * stream, allocated on first need and released by dxh_stream_destroy.  On a stream under
+ * graph capture the product is never cut. */
 DXH_API int dxh_matmul(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m,
                        int64_t k, int64_t n, void *stream);
 

@@ -71,13 +71,20 @@ inline int compute_units() {
 // batch index x is x % splits of batch x / splits, its partial tile goes to a workspace in the
 // accumulator type, laid out [batch][split][M][N], and splitk_reduce_kernel adds the slices in
 // slice order (same result on every run) and rounds once to the output type.  The workspace
-// (splitk_workspace, runtime.hip) is a grow-only buffer owned by the library, one per stream, so
+// (stream_workspace, runtime.hip) is a grow-only buffer owned by the library, one per stream, so
 // calls on different streams do not share it; a stream under graph capture never splits, because
 // a recorded pointer would not survive the buffer growing.  Cutting pays for a second launch
 // only when the uncut K loop is long: K >= min_k, slices of at least min_k / 4.
 struct KSplit { int splits, ksub; };
-void *splitk_workspace(hipStream_t st, size_t bytes);  // nullptr when the allocation fails
-void splitk_release(hipStream_t st);
+constexpr int kWorkspaceSplitK = 0, kWorkspacePadded = 1, kWorkspaceKinds = 2;
+constexpr int64_t kWorkspaceMaxBytes = (int64_t)1 << 28;
+void *stream_workspace(hipStream_t st, int kind, size_t bytes);  // nullptr when the allocation fails
+void stream_workspace_release(hipStream_t st);
+inline bool stream_is_capturing(hipStream_t st) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess) { (void)hipGetLastError(); return true; }  // unknown: assume the worst
+    return cap != hipStreamCaptureStatusNone;
+}
 inline KSplit choose_ksplit(int64_t tiles, int64_t k, int kstep, int64_t min_k, int64_t partial_bytes, hipStream_t st) {
     KSplit r{1, (int)k};
     const int64_t cus = compute_units(), ksteps = (k + kstep - 1) / kstep, knob = tuning().matmul_splitk;
@@ -92,10 +99,7 @@ inline KSplit choose_ksplit(int64_t tiles, int64_t k, int kstep, int64_t min_k, 
     }
     if (want > ksteps) want = ksteps;
     if (want > 1024) want = 1024;
-    if (want < 2 || want * partial_bytes > ((int64_t)1 << 28)) return r;
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &cap) != hipSuccess) { (void)hipGetLastError(); return r; }
-    if (cap != hipStreamCaptureStatusNone) return r;
+    if (want < 2 || want * partial_bytes > kWorkspaceMaxBytes || stream_is_capturing(st)) return r;
     const int64_t per = (ksteps + want - 1) / want;
     r.ksub = (int)(per * kstep);
     r.splits = (int)((k + r.ksub - 1) / r.ksub);

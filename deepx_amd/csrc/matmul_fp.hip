@@ -301,7 +301,7 @@ int launch_fp_tile(Launch launch, int tm, int tn, int kstep, int64_t min_k, T *c
         launch(blocks, c, map, ks);
         return launch_status();
     }
-    T *ws = (T *)splitk_workspace(st, (size_t)(partial * ks.splits));
+    T *ws = (T *)stream_workspace(st, kWorkspaceSplitK, (size_t)(partial * ks.splits));
     if (!ws) {  // no workspace: one slice
         const KSplit one{1, (int)k};
         if (!make_tile_map(batch, m, n, tm, tn, map)) return DXH_ERR_SHAPE;

@@ -1,7 +1,9 @@
 // matmul_half.hip — bf16 / f16 GEMM on the matrix pipe (v_mfma_f32_32x32x16_{bf16,f16}, fp32
 // accumulate, one RNE rounding of C).  Aligned shapes (K % 8 == 0, N % 8 == 0) take
-// matmul_mfma_tile_kernel, 64x64 to 256x256 workgroup tiles, software-pipelined over K; anything
-// else takes matmul_mfma_kernel, a plain 128x128x32 tile with element-wise edge handling.
+// matmul_mfma_tile_kernel, 64x64 to 256x256 workgroup tiles, software-pipelined over K, cut along
+// K when the output has few tiles; other shapes run the same kernel on zero-padded copies, or,
+// when no workspace may be used, matmul_mfma_kernel, a plain 128x128x32 tile with element-wise
+// edge handling.
 #include "matmul_common.hpp"
 
 namespace dxh {
@@ -379,7 +381,7 @@ int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m
     const KSplit ks = choose_ksplit(tiles, k, PK, 2048, partial, st);
     TileMap map;
     if (ks.splits < 2 || !make_tile_map(batch * ks.splits, m, n, TM, TN, map)) return kNoSplit;
-    float *ws = (float *)splitk_workspace(st, (size_t)(partial * ks.splits));
+    float *ws = (float *)stream_workspace(st, kWorkspaceSplitK, (size_t)(partial * ks.splits));
     if (!ws) return kNoSplit;
     if (k % PK == 0)
         matmul_mfma_tile_kernel<T, TM, TN, 1, false, true><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks);
@@ -387,6 +389,64 @@ int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m
         matmul_mfma_tile_kernel<T, TM, TN, 1, true, true><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks);
     const int rc = launch_status();
     return rc != DXH_OK ? rc : launch_splitk_reduce<float, T>(ws, (T *)c, batch, m * n, ks.splits, st);
+}
+
+// ---- rows that are not 16-byte aligned (odd K or N, unaligned bases) ---------------------------
+// The tile kernel needs 16-byte rows.  Such a product runs on zero-padded copies instead: A to
+// [M][K8], B to [K8][N8] (K8, N8 the next multiples of 8), the tile kernel on those, and the first
+// N columns of its [M][N8] result copied out.  The three copies move each operand once more
+// through HBM, a fraction of what the element-wise fallback kernel loses.
+// out[b][r][c] = (r < rows_in && c < cols_in) ? in[b][r][c] : 0, 8 columns (16 bytes out) per lane
+__global__ __launch_bounds__(kBlock) void pad_rows_kernel(const uint16_t *__restrict__ in, uint16_t *__restrict__ out, int64_t rows_in, int64_t cols_in,
+                                                          int64_t rows_out, int64_t chunks_out, int64_t total) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t ch = i % chunks_out, r = (i / chunks_out) % rows_out, b = i / (chunks_out * rows_out);
+        const uint16_t *p = in + (b * rows_in + r) * cols_in + ch * 8;
+        vec_t<uint16_t, 8> x;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x.v[e] = (r < rows_in && ch * 8 + e < cols_in) ? p[e] : (uint16_t)0;
+        *reinterpret_cast<vec_t<uint16_t, 8> *>(out + i * 8) = x;
+    }
+}
+// out[r][c] = in[r][c] for c < cols (in rows hold chunks_in * 8 columns)
+__global__ __launch_bounds__(kBlock) void unpad_rows_kernel(const uint16_t *__restrict__ in, uint16_t *__restrict__ out, int64_t cols, int64_t chunks_in, int64_t total) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t ch = i % chunks_in, r = i / chunks_in;
+        const vec_t<uint16_t, 8> x = *reinterpret_cast<const vec_t<uint16_t, 8> *>(in + i * 8);
+        uint16_t *p = out + r * cols + ch * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (ch * 8 + e < cols) p[e] = x.v[e];
+    }
+}
+inline unsigned copy_blocks(int64_t total) {
+    const int64_t blocks = (total + kBlock - 1) / kBlock;
+    return (unsigned)(blocks > 16384 ? 16384 : blocks);
+}
+
+template <typename T> int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
+
+template <typename T>
+int launch_padded(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    const int64_t k8 = (k + 7) / 8 * 8, n8 = (n + 7) / 8 * 8;
+    const int64_t a_elems = (batch * m * k8 + 7) / 8 * 8, b_elems = batch * k8 * n8, c_elems = batch * m * n8;  // each part starts 16-byte aligned
+    const int64_t bytes = (a_elems + b_elems + c_elems) * 2;
+    if (bytes > kWorkspaceMaxBytes || m * n * k < (1 << 16) || stream_is_capturing(st)) return kNoSplit;
+    uint16_t *ws = (uint16_t *)stream_workspace(st, kWorkspacePadded, (size_t)bytes);
+    if (!ws) return kNoSplit;
+    uint16_t *ap = ws, *bp = ap + a_elems, *cp = bp + b_elems;
+    int64_t total = batch * m * (k8 / 8);
+    const bool a_as_is = k == k8 && aligned(a, kVecBytes);  // only B and C have short rows
+    if (!a_as_is) pad_rows_kernel<<<copy_blocks(total), kBlock, 0, st>>>((const uint16_t *)a, ap, m, k, m, k8 / 8, total);
+    total = batch * k8 * (n8 / 8);
+    pad_rows_kernel<<<copy_blocks(total), kBlock, 0, st>>>((const uint16_t *)b, bp, k, n, k8, n8 / 8, total);
+    int rc = launch_status();
+    if (rc != DXH_OK) return rc;
+    rc = launch_mfma<T>(a_as_is ? a : ap, bp, cp, batch, m, k8, n8, st);
+    if (rc != DXH_OK) return rc;
+    total = batch * m * (n8 / 8);
+    unpad_rows_kernel<<<copy_blocks(total), kBlock, 0, st>>>(cp, (uint16_t *)c, n, n8 / 8, total);
+    return launch_status();
 }
 
 template <typename T>
@@ -418,6 +478,10 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
         case 5: return launch_tile<T, 64, 64, 1>(a, b, c, batch, m, k, n, st);
         default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, st);
         }
+    }
+    if (!fast && tuning().matmul_tile == 0 && k <= (1 << 22) && n <= (1 << 24)) {
+        const int rc = launch_padded<T>(a, b, c, batch, m, k, n, st);
+        if (rc != kNoSplit) return rc;
     }
     const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     const int64_t blocks = batch * tiles_m * tiles_n;

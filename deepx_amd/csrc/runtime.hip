@@ -4,6 +4,7 @@
 #include "matmul_common.hpp"
 #include <map>
 #include <mutex>
+#include <tuple>
 #include <cstdio>
 #include <cstring>
 
@@ -17,19 +18,19 @@ Tuning &tuning() {
 }  // namespace dxh
 
 namespace dxh {
-// One grow-only split-K workspace per (device, stream): kernels of one stream run in order, so a
-// buffer per stream is never shared by two products in flight.  Growing frees the old buffer with
+// Grow-only matmul workspaces, one per (device, stream, kind): kernels of one stream run in order,
+// so a buffer per stream is never shared by two products in flight.  Growing frees the old buffer with
 // hipFree, which waits for the device, so work still reading it has finished.
 namespace {
 struct Workspace { void *ptr; size_t bytes; };
 std::mutex g_ws_mutex;
-std::map<std::pair<int, hipStream_t>, Workspace> g_ws;
+std::map<std::tuple<int, hipStream_t, int>, Workspace> g_ws;
 }  // namespace
-void *splitk_workspace(hipStream_t st, size_t bytes) {
+void *stream_workspace(hipStream_t st, int kind, size_t bytes) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    Workspace &w = g_ws[{dev, st}];
+    Workspace &w = g_ws[std::make_tuple(dev, st, kind)];
     if (w.bytes >= bytes) return w.ptr;
     void *p = nullptr;
     if (hipMalloc(&p, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
@@ -38,14 +39,16 @@ void *splitk_workspace(hipStream_t st, size_t bytes) {
     w.bytes = bytes;
     return p;
 }
-void splitk_release(hipStream_t st) {
+void stream_workspace_release(hipStream_t st) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return; }
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    auto it = g_ws.find({dev, st});
-    if (it == g_ws.end()) return;
-    if (it->second.ptr) (void)hipFree(it->second.ptr);
-    g_ws.erase(it);
+    for (int kind = 0; kind < kWorkspaceKinds; ++kind) {
+        auto it = g_ws.find(std::make_tuple(dev, st, kind));
+        if (it == g_ws.end()) continue;
+        if (it->second.ptr) (void)hipFree(it->second.ptr);
+        g_ws.erase(it);
+    }
 }
 }  // namespace dxh
 
@@ -140,7 +143,7 @@ int dxh_stream_create(void **stream) {
 }
 int dxh_stream_destroy(void *stream) {
     if (!stream) return DXH_OK;
-    dxh::splitk_release(as_stream(stream));
+    dxh::stream_workspace_release(as_stream(stream));
     return (int)hipStreamDestroy(as_stream(stream));
 }
 int dxh_stream_sync(void *stream) { return (int)hipStreamSynchronize(as_stream(stream)); }

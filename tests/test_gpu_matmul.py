@@ -282,3 +282,34 @@ def test_matmul_under_capture_does_not_split(dxh):
         assert np.array_equal(dG.get(), want)
     dx.check(dxh.dxh_graph_destroy(graph))
     dx.check(dxh.dxh_stream_destroy(st))
+
+
+@pytest.mark.parametrize("dtype", [dx.BF16, dx.F16])
+@pytest.mark.parametrize("tile", [0, 1])
+def test_matmul_half_rows_not_16_byte_aligned(dxh, dtype, tile):
+    """Odd K / N and bases that are only 2-byte aligned: with the tile knob at 0 the product runs on
+    zero-padded copies of the operands, with the knob set it stays on the element-wise fallback
+    kernel; both against float64 numpy (rel 1e-2 of sum_k |a||b|) and exact on small integers."""
+    rng = np.random.default_rng(1000 + dtype + tile)
+    dx.check(dxh.dxh_tune(TILE_KNOB, tile))
+    try:
+        for batch, m, k, n, off in [(1, 333, 777, 555, 0), (2, 130, 71, 150, 0), (1, 257, 129, 65, 0), (3, 31, 200, 17, 0),
+                                    (1, 64, 72, 61, 0), (1, 200, 63, 64, 0), (1, 128, 64, 128, 1), (2, 65, 96, 72, 3)]:
+            A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
+            B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
+            # `off` elements of slack in front: the operands then start 2 * off bytes past a 256-byte boundary
+            dA, dB, dC = Dev(np.concatenate([np.zeros(off, A.dtype), A])), Dev(np.concatenate([np.zeros(off, B.dtype), B])), Dev.empty(batch * m * n + off, A.dtype)
+            dx.check(dxh.dxh_matmul(dtype, dA.ptr.value + 2 * off, dB.ptr.value + 2 * off, dC.ptr.value + 2 * off, batch, m, k, n, None), "matmul")
+            got = H.to_float(dC.get()[off:], dtype).astype(np.float64).reshape(batch, m, n)
+            ref, mag = _ref_product(A, B, dtype, batch, m, k, n)
+            assert np.all(np.abs(got - ref) <= 1e-2 * np.maximum(mag, 1e-30)), (dtype, tile, batch, m, k, n, off)
+        m, k, n = 131, 203, 77
+        Ai, Bi = rng.integers(-4, 5, (m, k)), rng.integers(-4, 5, (k, n))
+        A = H.to_storage(Ai.astype(np.float64).reshape(-1), dtype)
+        B = H.to_storage(Bi.astype(np.float64).reshape(-1), dtype)
+        dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, A.dtype)
+        dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+        want = H.to_float(H.to_storage((Ai @ Bi).astype(np.float64).reshape(-1), dtype), dtype)
+        assert np.array_equal(H.to_float(dC.get(), dtype), want)
+    finally:
+        dx.check(dxh.dxh_tune(TILE_KNOB, 0))

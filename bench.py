@@ -28,6 +28,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 MFMA_F32_PEAK_TF = 157.3
+MFMA_F64_PEAK_TF = 78.6
 MFMA_BF16_PEAK_TF = 2500.0  # dense bf16
 REDUCE_ROW_TRAFFIC_BYTES = 268609587  # measured, see profiles/bench_pmc_hbm_traffic.md
 
@@ -37,6 +38,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--ramp-ms", type=float, default=100.0,
+                    help="untimed steps run for this long before the warmup steps: from idle the GPU takes "
+                         "about 30 ms of load to reach its steady clocks")
     ap.add_argument("--no-per-op", action="store_true", help="skip the per-op table of the other configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -122,6 +126,10 @@ def main():
 
     ev = Events()
     step_events = [[ev.pair() for _ in groups] for _ in range(args.steps)]
+    ramp_t0 = time.perf_counter()
+    while (time.perf_counter() - ramp_t0) * 1e3 < args.ramp_ms:  # untimed: clocks settle
+        run_step()
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         run_step()
     torch.cuda.synchronize()
@@ -169,7 +177,8 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "config2: reductions on fp32 [8192,8192] (sum axis1/axis0, reducemax, reducemin) + prod [8192,64], keepdims true+false, 10 ops/step",
-                   "bytes_per_step": step_bytes, "input_copies_rotated": NX, "device": name.value.decode()},
+                   "bytes_per_step": step_bytes, "input_copies_rotated": NX, "clock_ramp_ms_before_warmup": args.ramp_ms,
+                   "device": name.value.decode()},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "per_op": per_op,
@@ -177,12 +186,19 @@ def main():
     print(json.dumps(line))
 
 
+RAMP_MS = 40.0  # untimed launches before every measurement: from idle the clocks take ~30 ms of load to settle
+
+
 def time_op(L, dx, torch, Events, ev, launch, reps=20, warm=3):
     """average time (ms) of `launch(i)`: one hipEvent pair on the NULL stream around `reps`
     back-to-back launches (callers rotate buffers through `i` so inputs come from HBM)"""
-    for i in range(warm):
-        launch(i)
-    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while True:
+        for i in range(warm):
+            launch(i)
+        torch.cuda.synchronize()
+        if (time.perf_counter() - t0) * 1e3 >= RAMP_MS:
+            break
     a, b = ev.pair()
     L.dxh_event_record(a, None)
     for i in range(reps):
@@ -288,6 +304,14 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
         Cm = torch.empty(mm * nn, device=dev)
         c5[label] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_matmul(dx.F32, ptr(Am), ptr(Bm), ptr(Cm), 1, mm, kk, nn, None)),
                           flops=2 * mm * kk * nn, peak_tf=MFMA_F32_PEAK_TF, peak_name="frac_mfma_f32")
+        c5[label]["hipblaslt_TFLOP/s"] = vendor_gemm_tflops(torch, Am.view(mm, kk), Bm.view(kk, nn), Cm.view(mm, nn))
+    # and in fp64, which the reference's dispatch also accepts (v_mfma_f64_16x16x4_f64)
+    for label, (mm, kk, nn) in [("matmul_f64_2048x896x4864", (2048, 896, 4864)), ("matmul_f64_2048x4864x896", (2048, 4864, 896))]:
+        Am = torch.randn(mm * kk, device=dev, dtype=torch.float64)
+        Bm = torch.randn(kk * nn, device=dev, dtype=torch.float64) * 0.02
+        Cm = torch.empty(mm * nn, device=dev, dtype=torch.float64)
+        c5[label] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_matmul(dx.F64, ptr(Am), ptr(Bm), ptr(Cm), 1, mm, kk, nn, None)),
+                          flops=2 * mm * kk * nn, peak_tf=MFMA_F64_PEAK_TF, peak_name="frac_mfma_f64")
         c5[label]["hipblaslt_TFLOP/s"] = vendor_gemm_tflops(torch, Am.view(mm, kk), Bm.view(kk, nn), Cm.view(mm, nn))
     del Am, Bm, Cm
     torch.cuda.empty_cache()
@@ -411,9 +435,13 @@ def config5_block_over_ir(rows=2048, hidden=896, inter=4864, iters=30):
 def vendor_gemm_tflops(torch, A, B, C, reps=20, warm=5):
     """torch.matmul (hipBLASLt / rocBLAS) on the same operands, for context next to our kernel's rate.
     Timed with torch's own events on torch's current stream, which is where torch launches it."""
-    for _ in range(warm):
-        torch.matmul(A, B, out=C)
-    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while True:
+        for _ in range(warm):
+            torch.matmul(A, B, out=C)
+        torch.cuda.synchronize()
+        if (time.perf_counter() - t0) * 1e3 >= RAMP_MS:
+            break
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(reps):

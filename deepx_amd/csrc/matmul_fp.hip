@@ -7,9 +7,12 @@ namespace dxh {
 // ---- fp32 MFMA kernel ------------------------------------------------------------------------
 // v_mfma_f32_32x32x2_f32 (fp32 operands, fp32 accumulate: 157 TFLOP/s peak, 64 cycles each).  A
 // fp32 GEMM on the matrix pipe is compute bound by a wide margin (8x fewer flops per operand
-// byte than bf16 at 1/16 of the rate), so this kernel is a plain double-buffered one: workgroup
-// tile (64 FM) x (64 FN), K step FK, 4 waves 2x2, each wave FM x FN MFMA tiles, PD K steps held
-// in registers ahead of the LDS stage being multiplied.
+// byte than bf16 at 1/16 of the rate): workgroup tile (64 FM) x (64 FN), K step FK, 4 waves 2x2,
+// each wave FM x FN MFMA tiles, two LDS stages, PD K steps held in registers ahead of the stage
+// being multiplied.  What keeps the pipe full is the issue order: MFMA operands are read from LDS
+// one group (8 k) ahead into a second register buffer, and LDS stores, global loads and those
+// reads are pinned between the MFMAs (sched_group_barrier); left alone the compiler reads each
+// operand right before its MFMA and the pipe idles for an LDS latency every fourth MFMA.
 //   A      LDS [m][FK k] with rows padded by 4 floats; a lane reads the FK/2 consecutive k of its
 //          row half with ds_read_b128 (the k order inside a K step is a free permutation as
 //          long as both operands use it: MFMA e of lane half h multiplies k = (FK/2) h + e).
@@ -45,9 +48,7 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
         static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
             const int id = t + kBlock * i, row = id / CA, kk = k0 + (id % CA) * 4, gm = m0 + row;
             if constexpr (VEC) {
-                const float *p = A + (int64_t)(gm < M ? gm : M - 1) * lda + (kk < K ? kk : 0);
-                f32x4 v = *reinterpret_cast<const f32x4 *>(p);
-                ra[set][i] = (kk < K) ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+                ra[set][i] = *reinterpret_cast<const f32x4 *>(A + (int64_t)(gm < M ? gm : M - 1) * lda + (kk < K ? kk : 0));
             } else {
                 f32x4 v;
 #pragma unroll
@@ -58,9 +59,7 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
         static_for<B_LD>([&](auto i) __attribute__((always_inline)) {
             const int id = t + kBlock * i, krow = id / CB, gk = k0 + krow, gn = n0 + (id % CB) * 4;
             if constexpr (VEC) {
-                const float *p = B + (int64_t)(gk < K ? gk : 0) * N + (gn < N ? gn : N - 4);
-                f32x4 v = *reinterpret_cast<const f32x4 *>(p);
-                rb[set][i] = (gk < K) ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+                rb[set][i] = *reinterpret_cast<const f32x4 *>(B + (int64_t)(gk < K ? gk : 0) * N + (gn < N ? gn : N - 4));
             } else {
                 f32x4 v;
 #pragma unroll
@@ -69,15 +68,21 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
             }
         });
     };
-    auto store_lds = [&](auto set, auto stage) __attribute__((always_inline)) {
+    // k0: the K step that register set `set` holds.  MASKED (only the store of a partial last K
+    // step): chunks past K were loaded from a clamped address and are zeroed here.  The common
+    // path has no select on loaded values: the scheduler would move it to the top of the K step
+    // and every step would wait out the full latency of its own prefetch.
+    auto store_lds = [&](auto set, auto stage, auto masked, int k0) __attribute__((always_inline)) {
         float *As = lds + decltype(stage)::value * STAGE, *Bs = As + TM * FA_ROW;
         static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
             const int id = t + kBlock * i;
-            *reinterpret_cast<f32x4 *>(As + (id / CA) * FA_ROW + (id % CA) * 4) = ra[set][i];
+            const bool keep = !decltype(masked)::value || k0 + (id % CA) * 4 < K;
+            *reinterpret_cast<f32x4 *>(As + (id / CA) * FA_ROW + (id % CA) * 4) = keep ? ra[set][i] : f32x4{0.f, 0.f, 0.f, 0.f};
         });
         static_for<B_LD>([&](auto i) __attribute__((always_inline)) {
             const int id = t + kBlock * i;
-            *reinterpret_cast<f32x4 *>(Bs + (id / CB) * FB_ROW + (id % CB) * 4) = rb[set][i];
+            const bool keep = !decltype(masked)::value || k0 + id / CB < K;
+            *reinterpret_cast<f32x4 *>(Bs + (id / CB) * FB_ROW + (id % CB) * 4) = keep ? rb[set][i] : f32x4{0.f, 0.f, 0.f, 0.f};
         });
     };
 
@@ -89,52 +94,115 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
         });
     });
     const int h = lane >> 5, l32 = lane & 31;
-    // MFMA e of lane half h multiplies k = HK*h + e of the K step (both operands use this order)
-    auto compute = [&](auto stage) __attribute__((always_inline)) {
+    // A K step is multiplied in Q groups of 8 k per lane half (MFMA e of lane half h multiplies
+    // k = HK*h + 8q + e; both operands use this order).  The operands of a group sit in one of
+    // two register buffers, read from LDS while the previous group is being multiplied.
+    constexpr int Q = HK / 8, NMG = FM * FN * 8, NRG = 2 * FM + 8 * FN, NLD = A_LD + B_LD;
+    f32x4 fa[2][FM][2];
+    float fb[2][FN][8];
+    auto read_frags = [&](auto buf, auto stage, auto q) __attribute__((always_inline)) {
         const float *As = lds + decltype(stage)::value * STAGE, *Bs = As + TM * FA_ROW;
-        static_for<HK / 8>([&](auto q) __attribute__((always_inline)) {  // 8 k per lane half at a time
-            f32x4 fa[FM][2];
-            float fb[FN][8];
-            static_for<FM>([&](auto i) __attribute__((always_inline)) {
-                const float *p = As + (wm * 32 * FM + 32 * i + l32) * FA_ROW + HK * h + 8 * decltype(q)::value;
-                fa[i][0] = *reinterpret_cast<const f32x4 *>(p);
-                fa[i][1] = *reinterpret_cast<const f32x4 *>(p + 4);
-            });
-            static_for<FN>([&](auto j) __attribute__((always_inline)) {
+        static_for<FM>([&](auto i) __attribute__((always_inline)) {
+            const float *p = As + (wm * 32 * FM + 32 * i + l32) * FA_ROW + HK * h + 8 * decltype(q)::value;
+            fa[buf][i][0] = *reinterpret_cast<const f32x4 *>(p);
+            fa[buf][i][1] = *reinterpret_cast<const f32x4 *>(p + 4);
+        });
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) fb[j][e] = Bs[(HK * h + 8 * decltype(q)::value + e) * FB_ROW + wn * 32 * FN + 32 * j + l32];
-            });
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                static_for<FM>([&](auto i) __attribute__((always_inline)) {
-                    static_for<FN>([&](auto j) __attribute__((always_inline)) {
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][e], fa[i][e >> 2][e & 3], acc[i][j], 0, 0, 0);
-                    });
-                });
+            for (int e = 0; e < 8; ++e) fb[buf][j][e] = Bs[(HK * h + 8 * decltype(q)::value + e) * FB_ROW + wn * 32 * FN + 32 * j + l32];
+        });
+    };
+    auto mma = [&](auto buf, auto lo, auto hi) __attribute__((always_inline)) {
+        static_for<decltype(hi)::value - decltype(lo)::value>([&](auto x) __attribute__((always_inline)) {
+            constexpr int idx = decltype(lo)::value + decltype(x)::value, e = idx / (FM * FN), i = idx % (FM * FN) / FN, j = idx % FN;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[buf][j][e], fa[buf][i][e >> 2][e & 3], acc[i][j], 0, 0, 0);
+        });
+    };
+    // Issue order inside a scheduling region: after each MFMA an even share of the region's LDS
+    // reads, LDS writes and global loads (counts are upper bounds: paired ds_read2 count once).
+    auto interleave = [&](auto mfmas, auto reads, auto writes, auto loads) __attribute__((always_inline)) {
+        constexpr int nm = decltype(mfmas)::value, nr = decltype(reads)::value, nw = decltype(writes)::value, nl = decltype(loads)::value;
+        static_for<nm>([&](auto x) __attribute__((always_inline)) {
+            constexpr int m = decltype(x)::value;
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            constexpr int r = nr * (m + 1) / nm - nr * m / nm, wr = nw * (m + 1) / nm - nw * m / nm, l = nl * (m + 1) / nm - nl * m / nm;
+            if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+            if constexpr (wr > 0) __builtin_amdgcn_sched_group_barrier(0x200, wr, 0);
+            if constexpr (l > 0) __builtin_amdgcn_sched_group_barrier(0x020, l, 0);
+        });
+    };
+
+    // One K step: LDS stage S is multiplied (its group 0 is already in a fragment buffer); register
+    // set R (K step k_store) moves into stage S^1 and is refilled with K step k_load.  The LDS
+    // stores and global loads are dealt out between the first half of the last group's MFMAs; the
+    // second half runs after the barrier, under the reads of the next stage's group 0.
+    auto step = [&](auto S, auto masked, int k_store, int k_load) __attribute__((always_inline)) {
+        constexpr int sv = decltype(S)::value;
+        const auto R = ic<(PD == 1) ? 0 : sv ^ 1>{};  // register set (kt + 1) % PD
+        static_for<Q>([&](auto q) __attribute__((always_inline)) {
+            constexpr int qv = decltype(q)::value, cur = (sv * Q + qv) & 1;
+            if constexpr (qv + 1 < Q) {
+                read_frags(ic<cur ^ 1>{}, S, ic<qv + 1>{});
+                mma(ic<cur>{}, ic<0>{}, ic<NMG>{});
+                interleave(ic<NMG>{}, ic<NRG>{}, ic<0>{}, ic<0>{});
+            } else {
+                store_lds(R, ic<sv ^ 1>{}, masked, k_store);
+                load_global(R, k_load);
+                mma(ic<cur>{}, ic<0>{}, ic<NMG / 2>{});
+                interleave(ic<NMG / 2>{}, ic<0>{}, ic<NLD>{}, ic<NLD>{});
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();
+                read_frags(ic<cur ^ 1>{}, ic<sv ^ 1>{}, ic<0>{});
+                mma(ic<cur>{}, ic<NMG / 2>{}, ic<NMG>{});
+                interleave(ic<NMG - NMG / 2>{}, ic<NRG>{}, ic<0>{}, ic<0>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    auto last_step = [&](auto S) __attribute__((always_inline)) {  // nothing left to load
+        constexpr int sv = decltype(S)::value;
+        static_for<Q>([&](auto q) __attribute__((always_inline)) {
+            constexpr int qv = decltype(q)::value, cur = (sv * Q + qv) & 1;
+            if constexpr (qv + 1 < Q) {
+                read_frags(ic<cur ^ 1>{}, S, ic<qv + 1>{});
+                mma(ic<cur>{}, ic<0>{}, ic<NMG>{});
+                interleave(ic<NMG>{}, ic<NRG>{}, ic<0>{}, ic<0>{});
+            } else {
+                mma(ic<cur>{}, ic<0>{}, ic<NMG>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
         });
     };
 
     // LDS stage (kt & 1) holds K step kt, register set (kt + 1) % PD holds step kt + 1 and is
     // refilled with step kt + 1 + PD once it has moved to LDS.  Steps past the end are clamped
-    // onto the last one (loaded, never multiplied).
+    // onto the last one (loaded, never stored).  Only the store of a partial last K step is masked.
     const int KT = (K + FK - 1) / FK;
+    const bool tail = VEC && K % FK != 0;
     auto k_of = [&](int stepno) { return (stepno < KT ? stepno : KT - 1) * FK; };
-    auto step = [&](auto S, auto R, int k_load) __attribute__((always_inline)) {
-        compute(S);
-        store_lds(R, ic<decltype(S)::value ^ 1>{});
-        load_global(R, k_load);
-        __syncthreads();
-    };
     load_global(ic<0>{}, 0);
-    store_lds(ic<0>{}, ic<0>{});
+    if (tail && KT == 1) store_lds(ic<0>{}, ic<0>{}, std::true_type{}, 0);
+    else store_lds(ic<0>{}, ic<0>{}, std::false_type{}, 0);
     static_for<PD>([&](auto d) __attribute__((always_inline)) { load_global(ic<(decltype(d)::value + 1) % PD>{}, k_of(decltype(d)::value + 1)); });
     __syncthreads();
+    read_frags(ic<0>{}, ic<0>{}, ic<0>{});
+    const int plain = tail ? KT - 2 : KT - 1;  // steps kt < plain store a full K step
     int kt = 0;
-    for (; kt + 1 < KT; kt += 2) {
-        step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1 + PD));
-        step(ic<1>{}, ic<2 % PD>{}, k_of(kt + 2 + PD));
+    for (; kt + 1 < plain; kt += 2) {
+        step(ic<0>{}, std::false_type{}, (kt + 1) * FK, k_of(kt + 1 + PD));
+        step(ic<1>{}, std::false_type{}, (kt + 2) * FK, k_of(kt + 2 + PD));
     }
-    if (kt < KT) compute(ic<0>{});
+    if (kt < plain) {
+        step(ic<0>{}, std::false_type{}, (kt + 1) * FK, k_of(kt + 1 + PD));
+        ++kt;
+    }
+    if (tail && KT >= 2) {
+        if (kt & 1) step(ic<1>{}, std::true_type{}, (kt + 1) * FK, k_of(kt + 1 + PD));
+        else step(ic<0>{}, std::true_type{}, (kt + 1) * FK, k_of(kt + 1 + PD));
+        ++kt;
+    }
+    if (kt & 1) last_step(ic<1>{});
+    else last_step(ic<0>{});
 
     // Result lane: row m = lane%32 of its MFMA tile; register group g holds columns 8g + 4h .. +3.
     // The tile goes through LDS (rows padded by 4 floats: the 16 lanes of a ds_write_b128 phase
@@ -201,9 +269,7 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double
         static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
             const int id = t + kBlock * i, row = id / CA, kk = k0 + (id % CA) * 2, gm = m0 + row;
             if constexpr (VEC) {
-                const double *p = A + (int64_t)(gm < M ? gm : M - 1) * lda + (kk < K ? kk : 0);
-                f64x2 v = *reinterpret_cast<const f64x2 *>(p);
-                ra[i] = (kk < K) ? v : f64x2{0.0, 0.0};
+                ra[i] = *reinterpret_cast<const f64x2 *>(A + (int64_t)(gm < M ? gm : M - 1) * lda + (kk < K ? kk : 0));
             } else {
                 f64x2 v;
 #pragma unroll
@@ -214,9 +280,7 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double
         static_for<B_LD>([&](auto i) __attribute__((always_inline)) {
             const int id = t + kBlock * i, krow = id / CB, gk = k0 + krow, gn = n0 + (id % CB) * 2;
             if constexpr (VEC) {
-                const double *p = B + (int64_t)(gk < K ? gk : 0) * N + (gn < N ? gn : N - 2);
-                f64x2 v = *reinterpret_cast<const f64x2 *>(p);
-                rb[i] = (gk < K) ? v : f64x2{0.0, 0.0};
+                rb[i] = *reinterpret_cast<const f64x2 *>(B + (int64_t)(gk < K ? gk : 0) * N + (gn < N ? gn : N - 2));
             } else {
                 f64x2 v;
 #pragma unroll
@@ -225,15 +289,18 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double
             }
         });
     };
-    auto store_lds = [&](int stage) __attribute__((always_inline)) {
-        double *As = lds + stage * STAGE, *Bs = As + TM * DA_ROW;
+    // MASKED (only the store of a partial last K step): chunks past K are zeroed (see the fp32 kernel)
+    auto store_lds = [&](auto stage, auto masked, int k0) __attribute__((always_inline)) {
+        double *As = lds + decltype(stage)::value * STAGE, *Bs = As + TM * DA_ROW;
         static_for<A_LD>([&](auto i) __attribute__((always_inline)) {
             const int id = t + kBlock * i;
-            *reinterpret_cast<f64x2 *>(As + (id / CA) * DA_ROW + (id % CA) * 2) = ra[i];
+            const bool keep = !decltype(masked)::value || k0 + (id % CA) * 2 < K;
+            *reinterpret_cast<f64x2 *>(As + (id / CA) * DA_ROW + (id % CA) * 2) = keep ? ra[i] : f64x2{0.0, 0.0};
         });
         static_for<B_LD>([&](auto i) __attribute__((always_inline)) {
             const int id = t + kBlock * i;
-            *reinterpret_cast<f64x2 *>(Bs + (id / CB) * DB_ROW + (id % CB) * 2) = rb[i];
+            const bool keep = !decltype(masked)::value || k0 + id / CB < K;
+            *reinterpret_cast<f64x2 *>(Bs + (id / CB) * DB_ROW + (id % CB) * 2) = keep ? rb[i] : f64x2{0.0, 0.0};
         });
     };
 
@@ -242,39 +309,115 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double
         static_for<CT>([&](auto j) __attribute__((always_inline)) { acc[i][j] = f64x4{0.0, 0.0, 0.0, 0.0}; });
     });
     const int q = lane >> 4, l16 = lane & 15;
-    auto compute = [&](int stage) __attribute__((always_inline)) {
-        const double *As = lds + stage * STAGE, *Bs = As + TM * DA_ROW;
-        f64x2 fa[RT][2];
-        double fb[CT][4];
+    // MFMA e of lane quarter q multiplies k = 4q + e.  A K step is multiplied in Q groups of GE
+    // e (one e for the 128x128 tile, whose 128 accumulator registers leave room for no more);
+    // the operands of a group are read from LDS into one of two register buffers while the
+    // previous group is multiplied, and LDS stores / global loads are pinned between the MFMAs, as
+    // in the fp32 kernel.
+    constexpr int GE = (FM * FN == 4) ? 1 : 2, Q = 4 / GE;
+    constexpr int NMG = RT * CT * GE, NRG = RT + GE * CT, NLD = A_LD + B_LD;
+    double fa[2][RT][GE], fb[2][CT][GE];
+    auto read_frags = [&](auto buf, auto stage, auto g) __attribute__((always_inline)) {
+        const double *As = lds + decltype(stage)::value * STAGE, *Bs = As + TM * DA_ROW;
         static_for<RT>([&](auto i) __attribute__((always_inline)) {
-            const double *p = As + (wm * 32 * FM + 16 * i + l16) * DA_ROW + 4 * q;
-            fa[i][0] = *reinterpret_cast<const f64x2 *>(p);
-            fa[i][1] = *reinterpret_cast<const f64x2 *>(p + 2);
+            const double *p = As + (wm * 32 * FM + 16 * i + l16) * DA_ROW + 4 * q + GE * decltype(g)::value;
+            if constexpr (GE == 2) {
+                const f64x2 v = *reinterpret_cast<const f64x2 *>(p);
+                fa[buf][i][0] = v[0];
+                fa[buf][i][GE - 1] = v[1];
+            } else {
+                fa[buf][i][0] = *p;
+            }
         });
         static_for<CT>([&](auto j) __attribute__((always_inline)) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) fb[j][e] = Bs[(4 * q + e) * DB_ROW + wn * 32 * FN + 16 * j + l16];
+            for (int e = 0; e < GE; ++e) fb[buf][j][e] = Bs[(4 * q + GE * decltype(g)::value + e) * DB_ROW + wn * 32 * FN + 16 * j + l16];
         });
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            static_for<RT>([&](auto i) __attribute__((always_inline)) {
-                static_for<CT>([&](auto j) __attribute__((always_inline)) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[i][e >> 1][e & 1], fb[j][e], acc[i][j], 0, 0, 0);
-                });
-            });
+    };
+    auto mma = [&](auto buf, auto lo, auto hi) __attribute__((always_inline)) {
+        static_for<decltype(hi)::value - decltype(lo)::value>([&](auto x) __attribute__((always_inline)) {
+            constexpr int idx = decltype(lo)::value + decltype(x)::value, e = idx / (RT * CT), i = idx % (RT * CT) / CT, j = idx % CT;
+            acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[buf][i][e], fb[buf][j][e], acc[i][j], 0, 0, 0);
+        });
+    };
+    auto interleave = [&](auto mfmas, auto reads, auto writes, auto loads) __attribute__((always_inline)) {
+        constexpr int nm = decltype(mfmas)::value, nr = decltype(reads)::value, nw = decltype(writes)::value, nl = decltype(loads)::value;
+        static_for<nm>([&](auto x) __attribute__((always_inline)) {
+            constexpr int m = decltype(x)::value;
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            constexpr int r = nr * (m + 1) / nm - nr * m / nm, wr = nw * (m + 1) / nm - nw * m / nm, l = nl * (m + 1) / nm - nl * m / nm;
+            if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+            if constexpr (wr > 0) __builtin_amdgcn_sched_group_barrier(0x200, wr, 0);
+            if constexpr (l > 0) __builtin_amdgcn_sched_group_barrier(0x020, l, 0);
+        });
+    };
+    // One K step: stage S is multiplied (its group 0 already sits in fragment buffer 0); the
+    // register set (K step k_store) moves into stage S^1 and is refilled with K step k_load.
+    auto step = [&](auto S, auto masked, int k_store, int k_load) __attribute__((always_inline)) {
+        constexpr int sv = decltype(S)::value;
+        static_for<Q>([&](auto g) __attribute__((always_inline)) {
+            constexpr int gv = decltype(g)::value, cur = gv & 1;  // Q is even
+            if constexpr (gv + 1 < Q) {
+                read_frags(ic<cur ^ 1>{}, S, ic<gv + 1>{});
+                mma(ic<cur>{}, ic<0>{}, ic<NMG>{});
+                interleave(ic<NMG>{}, ic<NRG>{}, ic<0>{}, ic<0>{});
+            } else {
+                store_lds(ic<sv ^ 1>{}, masked, k_store);
+                load_global(k_load);
+                mma(ic<cur>{}, ic<0>{}, ic<NMG / 2>{});
+                interleave(ic<NMG / 2>{}, ic<0>{}, ic<NLD>{}, ic<NLD>{});
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();
+                read_frags(ic<cur ^ 1>{}, ic<sv ^ 1>{}, ic<0>{});
+                mma(ic<cur>{}, ic<NMG / 2>{}, ic<NMG>{});
+                interleave(ic<NMG - NMG / 2>{}, ic<NRG>{}, ic<0>{}, ic<0>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    auto last_step = [&](auto S) __attribute__((always_inline)) {
+        static_for<Q>([&](auto g) __attribute__((always_inline)) {
+            constexpr int gv = decltype(g)::value, cur = gv & 1;
+            if constexpr (gv + 1 < Q) {
+                read_frags(ic<cur ^ 1>{}, S, ic<gv + 1>{});
+                mma(ic<cur>{}, ic<0>{}, ic<NMG>{});
+                interleave(ic<NMG>{}, ic<NRG>{}, ic<0>{}, ic<0>{});
+            } else {
+                mma(ic<cur>{}, ic<0>{}, ic<NMG>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
     };
 
+    // Stage (kt & 1) holds K step kt and the register set holds step kt + 1, refilled with step
+    // kt + 2 once it has moved to LDS (steps past the end are clamped onto the last one: loaded,
+    // never stored).  Only the store of a partial last K step is masked.
     const int KT = (K + DK - 1) / DK;
+    const bool tail = VEC && K % DK != 0;
+    auto k_of = [&](int stepno) { return (stepno < KT ? stepno : KT - 1) * DK; };
     load_global(0);
-    store_lds(0);
+    if (tail && KT == 1) store_lds(ic<0>{}, std::true_type{}, 0);
+    else store_lds(ic<0>{}, std::false_type{}, 0);
+    load_global(k_of(1));
     __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-        const bool more = kt + 1 < KT;
-        if (more) load_global((kt + 1) * DK);
-        compute(kt & 1);
-        if (more) store_lds((kt + 1) & 1);
-        __syncthreads();
+    read_frags(ic<0>{}, ic<0>{}, ic<0>{});
+    const int plain = tail ? KT - 2 : KT - 1;  // steps kt < plain store a full K step
+    int kt = 0;
+    for (; kt + 1 < plain; kt += 2) {
+        step(ic<0>{}, std::false_type{}, (kt + 1) * DK, k_of(kt + 2));
+        step(ic<1>{}, std::false_type{}, (kt + 2) * DK, k_of(kt + 3));
     }
+    if (kt < plain) {
+        step(ic<0>{}, std::false_type{}, (kt + 1) * DK, k_of(kt + 2));
+        ++kt;
+    }
+    if (tail && KT >= 2) {
+        if (kt & 1) step(ic<1>{}, std::true_type{}, (kt + 1) * DK, k_of(kt + 2));
+        else step(ic<0>{}, std::true_type{}, (kt + 1) * DK, k_of(kt + 2));
+        ++kt;
+    }
+    if (kt & 1) last_step(ic<1>{});
+    else last_step(ic<0>{});
 
     static_for<RT>([&](auto i) __attribute__((always_inline)) {
         static_for<CT>([&](auto j) __attribute__((always_inline)) {
@@ -322,25 +465,26 @@ int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int
 }
 
 // fp32: the matrix pipe is the bound, so the tile is chosen for CU balance.  Cost model per tile
-// shape: two workgroups share a CU; a CU's time is (rounds of two tiles) x tile flops / efficiency,
-// where a last round that leaves at most one workgroup per CU counts 0.6 (a lone workgroup runs
-// faster than two that share the pipe) and the efficiencies are the measured large-square rates
-// relative to the 128x128 tile.  Small tiles take longer K steps and a deeper prefetch: with few
-// MFMAs per step only that hides the global-load latency.
+// shape, in microseconds: two workgroups share a CU, a round of two workgroups per CU takes a fixed
+// 3 us (first loads, result stores) plus K times the tile's time per k (0.118 us for 128x128 on
+// 4096^3; 128x64 and 64x64 run at 0.96 and 0.90 of that rate per flop), and a last round that
+// leaves at most one workgroup per CU counts 0.55 (a lone workgroup has the matrix pipe to itself).
+// Small tiles take longer K steps and a deeper prefetch: with few MFMAs per step only that hides
+// the global-load latency.
 int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     const bool vec = k % 4 == 0 && n % 4 == 0 && n >= 4 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes);
     const int64_t cus = compute_units();
     auto cost = [&](int tm, int tn, double eff) {
         const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn);
         const int64_t full = tiles / (2 * cus), rem = tiles % (2 * cus);
-        const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.6 : 0.0);
-        return rounds * (double)tm * (double)tn / eff;
+        const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.55 : 0.0);
+        return rounds * (3.0 + (double)k * 0.1183 * (double)(tm * tn) / (128.0 * 128.0) / eff);
     };
     const float *af = (const float *)a, *bf = (const float *)b;
     float *cf = (float *)c;
     int64_t choice = tuning().matmul_tile;
     if (choice == 0) {
-        const double c1 = cost(128, 128, 1.0), c2 = cost(128, 64, 0.95), c3 = cost(64, 64, 0.86);
+        const double c1 = cost(128, 128, 1.0), c2 = cost(128, 64, 0.957), c3 = cost(64, 64, 0.897);
         choice = (c1 <= c2 && c1 <= c3) ? 1 : (c2 <= c3) ? 2 : 3;
     }
     switch (choice) {
@@ -360,22 +504,24 @@ int launch_f64_tile(const double *a, const double *b, double *c, int64_t batch, 
     }, 64 * FM, 64 * FN, 16, 512, c, batch, m, k, n, st);
 }
 
-// fp64 on the matrix pipe; tile chosen for CU balance like fp32 (efficiencies measured on 4096^3)
+// fp64 on the matrix pipe; tile chosen for CU balance with the fp32 cost model (0.116 us per k for
+// a round of 128x64 tiles on 4096^3, 64x64 at 0.94 of that rate per flop).  The 128x128 tile is
+// not chosen: its 128 accumulator registers leave too few for the operand buffers and it runs
+// behind 128x64 on every shape tried; the tuning knob still selects it.
 int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     const bool vec = k % 2 == 0 && n % 2 == 0 && n >= 2 && aligned(a, kVecBytes) && aligned(b, kVecBytes);
     const int64_t cus = compute_units();
     auto cost = [&](int tm, int tn, double eff) {
         const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn);
         const int64_t full = tiles / (2 * cus), rem = tiles % (2 * cus);
-        const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.6 : 0.0);
-        return rounds * (double)tm * (double)tn / eff;
+        const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.55 : 0.0);
+        return rounds * (3.0 + (double)k * 0.1163 * (double)(tm * tn) / (128.0 * 64.0) / eff);
     };
     const double *af = (const double *)a, *bf = (const double *)b;
     double *cf = (double *)c;
     int64_t choice = tuning().matmul_tile;
     if (choice == 0) {
-        const double c1 = cost(128, 128, 1.0), c2 = cost(128, 64, 0.86), c3 = cost(64, 64, 0.95);
-        choice = (c1 <= c2 && c1 <= c3) ? 1 : (c2 <= c3) ? 2 : 3;
+        choice = cost(128, 64, 1.0) <= cost(64, 64, 0.941) ? 2 : 3;
     }
     switch (choice) {
     case 1: return launch_f64_tile<2, 2>(af, bf, cf, batch, m, k, n, vec, st);

@@ -206,18 +206,18 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
     };
     // k0: the K step that register set `set` holds.  The zero fill of a partial K step happens
     // here and not at the load, so that nothing waits for a load right after issuing it.
-    auto store_part = [&](auto set, auto part, auto stage, int k0) __attribute__((always_inline)) {
+    auto store_part = [&](auto set, auto part, auto stage, auto masked, int k0) __attribute__((always_inline)) {
         uint16_t *As = lds + decltype(stage)::value * STAGE, *Bs = As + A_STAGE;
         static_for<part_count(A_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
             constexpr int i = part_first(A_LD, decltype(part)::value) + decltype(q)::value;
-            if constexpr (KTAIL)
+            if constexpr (KTAIL && decltype(masked)::value)
                 *reinterpret_cast<u32x4 *>(As + a_lds[i]) = k0 + ach * 8 < K ? ra[set][i] : u32x4{0u, 0u, 0u, 0u};
             else
                 *reinterpret_cast<u32x4 *>(As + a_lds[i]) = ra[set][i];
         });
         static_for<part_count(B_LD, decltype(part)::value)>([&](auto q) __attribute__((always_inline)) {
             constexpr int i = part_first(B_LD, decltype(part)::value) + decltype(q)::value;
-            if constexpr (KTAIL)
+            if constexpr (KTAIL && decltype(masked)::value)
                 *reinterpret_cast<u32x4 *>(Bs + b_lds + i * KR * B_ROW) = k0 + brow + i * KR < K ? rb[set][i] : u32x4{0u, 0u, 0u, 0u};
             else
                 *reinterpret_cast<u32x4 *>(Bs + b_lds + i * KR * B_ROW) = rb[set][i];
@@ -275,19 +275,20 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
     // S^1 and is refilled with the K step PD further on.  Fragment buffer 0 holds substep 0 on
     // entry.  The last substep straddles the barrier: half of its MFMAs are queued before it and
     // the other half runs under the first fragment reads of stage S^1.
-    auto step = [&](auto S, auto R, int k_store, int k_load) __attribute__((always_inline)) {
+    auto step = [&](auto S, auto masked, int k_store, int k_load) __attribute__((always_inline)) {
         constexpr int s = decltype(S)::value;
+        const auto R = ic<(PD == 1) ? 0 : s ^ 1>{};  // register set (kt + 1) % PD
         static_for<4>([&](auto ks) __attribute__((always_inline)) {
             constexpr int cur = decltype(ks)::value & 1;
             constexpr int NW = part_count(A_LD, decltype(ks)::value) + part_count(B_LD, decltype(ks)::value);  // LDS writes = global loads
             if constexpr (decltype(ks)::value < 3) {
                 read_frags(ic<cur ^ 1>{}, S, ic<decltype(ks)::value + 1>{});
-                store_part(R, ks, ic<s ^ 1>{}, k_store);
+                store_part(R, ks, ic<s ^ 1>{}, masked, k_store);
                 load_part(R, ks, k_load);
                 mma(ic<cur>{}, ic<0>{}, ic<NM>{});
                 interleave(ic<NM>{}, ic<ND>{}, ic<NW>{}, ic<NW>{});
             } else {
-                store_part(R, ks, ic<s ^ 1>{}, k_store);
+                store_part(R, ks, ic<s ^ 1>{}, masked, k_store);
                 load_part(R, ks, k_load);
                 mma(ic<cur>{}, ic<0>{}, ic<NM / 2>{});
                 interleave(ic<NM / 2>{}, ic<0>{}, ic<NW>{}, ic<NW>{});
@@ -304,16 +305,19 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
     const int KT = (K + PK - 1) / PK;
     auto k_of = [&](int stepno) __attribute__((always_inline)) { return (stepno < KT ? stepno : KT - 1) * PK; };
     static_for<4>([&](auto part) __attribute__((always_inline)) { load_part(ic<0>{}, part, k_of(0)); });
-    static_for<4>([&](auto part) __attribute__((always_inline)) { store_part(ic<0>{}, part, ic<0>{}, 0); });
+    static_for<4>([&](auto part) __attribute__((always_inline)) { store_part(ic<0>{}, part, ic<0>{}, std::true_type{}, 0); });
     static_for<PD>([&](auto d) __attribute__((always_inline)) { static_for<4>([&](auto part) __attribute__((always_inline)) { load_part(ic<(decltype(d)::value + 1) % PD>{}, part, k_of(decltype(d)::value + 1)); }); });
     __syncthreads();
     read_frags(ic<0>{}, ic<0>{}, ic<0>{});
+    // KTAIL kernels mask every store: peeling the two steps that need it costs more registers
+    // than the tile sizes with 128 and more accumulator registers have left.
+    const auto masked = std::integral_constant<bool, KTAIL>{};
     int kt = 0;
     for (; kt + 1 < KT; kt += 2) {
-        step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1), k_of(kt + 1 + PD));
-        step(ic<1>{}, ic<2 % PD>{}, k_of(kt + 2), k_of(kt + 2 + PD));
+        step(ic<0>{}, masked, k_of(kt + 1), k_of(kt + 1 + PD));
+        step(ic<1>{}, masked, k_of(kt + 2), k_of(kt + 2 + PD));
     }
-    if (kt < KT) step(ic<0>{}, ic<1 % PD>{}, k_of(kt + 1), k_of(kt + 1 + PD));
+    if (kt < KT) step(ic<0>{}, masked, k_of(kt + 1), k_of(kt + 1 + PD));
     if constexpr (SPLIT) {
         // fp32 partial tile straight from the accumulators: 16 bytes (4 consecutive n) per store
         typedef float f32x4 __attribute__((ext_vector_type(4)));

@@ -1,6 +1,7 @@
 // matmul_common.hpp — pieces shared by the matrix-pipe GEMM kernels: vector typedefs, compile-time
 // loops, the XCD-aware workgroup -> tile map and the launch-side helpers.
 #pragma once
+#include <mutex>
 #include <utility>
 #include "common.hpp"
 
@@ -79,6 +80,9 @@ struct KSplit { int splits, ksub; };
 constexpr int kWorkspaceSplitK = 0, kWorkspacePadded = 1, kWorkspaceKinds = 2;
 constexpr int64_t kWorkspaceMaxBytes = (int64_t)1 << 28;
 void *stream_workspace(hipStream_t st, int kind, size_t bytes);  // nullptr when the allocation fails
+// Held from the workspace request to the last launch that uses it: two host threads that launch on
+// one stream must not interleave their (fill workspace, consume workspace) launch pairs.
+std::recursive_mutex &workspace_launch_mutex();
 void stream_workspace_release(hipStream_t st);
 inline bool stream_is_capturing(hipStream_t st) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;

@@ -444,6 +444,7 @@ int launch_fp_tile(Launch launch, int tm, int tn, int kstep, int64_t min_k, T *c
         launch(blocks, c, map, ks);
         return launch_status();
     }
+    std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
     T *ws = (T *)stream_workspace(st, kWorkspaceSplitK, (size_t)(partial * ks.splits));
     if (!ws) {  // no workspace: one slice
         const KSplit one{1, (int)k};
@@ -468,7 +469,7 @@ int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int
 // shape, in microseconds: two workgroups share a CU, a round of two workgroups per CU takes a fixed
 // 3 us (first loads, result stores) plus K times the tile's time per k (0.118 us for 128x128 on
 // 4096^3; 128x64 and 64x64 run at 0.96 and 0.90 of that rate per flop), and a last round that
-// leaves at most one workgroup per CU counts 0.55 (a lone workgroup has the matrix pipe to itself).
+// leaves at most one workgroup per CU counts 0.5 (a lone workgroup has the matrix pipe to itself).
 // Small tiles take longer K steps and a deeper prefetch: with few MFMAs per step only that hides
 // the global-load latency.
 int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
@@ -477,7 +478,7 @@ int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int6
     auto cost = [&](int tm, int tn, double eff) {
         const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn);
         const int64_t full = tiles / (2 * cus), rem = tiles % (2 * cus);
-        const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.55 : 0.0);
+        const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.5 : 0.0);
         return rounds * (3.0 + (double)k * 0.1183 * (double)(tm * tn) / (128.0 * 128.0) / eff);
     };
     const float *af = (const float *)a, *bf = (const float *)b;
@@ -514,7 +515,7 @@ int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int6
     auto cost = [&](int tm, int tn, double eff) {
         const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn);
         const int64_t full = tiles / (2 * cus), rem = tiles % (2 * cus);
-        const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.55 : 0.0);
+        const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.5 : 0.0);
         return rounds * (3.0 + (double)k * 0.1163 * (double)(tm * tn) / (128.0 * 64.0) / eff);
     };
     const double *af = (const double *)a, *bf = (const double *)b;

@@ -385,6 +385,7 @@ int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m
     const KSplit ks = choose_ksplit(tiles, k, PK, 2048, partial, st);
     TileMap map;
     if (ks.splits < 2 || !make_tile_map(batch * ks.splits, m, n, TM, TN, map)) return kNoSplit;
+    std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
     float *ws = (float *)stream_workspace(st, kWorkspaceSplitK, (size_t)(partial * ks.splits));
     if (!ws) return kNoSplit;
     if (k % PK == 0)
@@ -436,6 +437,7 @@ int launch_padded(const void *a, const void *b, void *c, int64_t batch, int64_t 
     const int64_t a_elems = (batch * m * k8 + 7) / 8 * 8, b_elems = batch * k8 * n8, c_elems = batch * m * n8;  // each part starts 16-byte aligned
     const int64_t bytes = (a_elems + b_elems + c_elems) * 2;
     if (bytes > kWorkspaceMaxBytes || m * n * k < (1 << 16) || stream_is_capturing(st)) return kNoSplit;
+    std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
     uint16_t *ws = (uint16_t *)stream_workspace(st, kWorkspacePadded, (size_t)bytes);
     if (!ws) return kNoSplit;
     uint16_t *ap = ws, *bp = ap + a_elems, *cp = bp + b_elems;

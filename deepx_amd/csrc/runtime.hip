@@ -26,6 +26,10 @@ struct Workspace { void *ptr; size_t bytes; };
 std::mutex g_ws_mutex;
 std::map<std::tuple<int, hipStream_t, int>, Workspace> g_ws;
 }  // namespace
+std::recursive_mutex &workspace_launch_mutex() {
+    static std::recursive_mutex m;
+    return m;
+}
 void *stream_workspace(hipStream_t st, int kind, size_t bytes) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }

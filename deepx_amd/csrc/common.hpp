@@ -84,6 +84,11 @@ template <typename VT> __device__ inline void st_nt(VT *p, const VT &v) {
     __builtin_nontemporal_store(__builtin_bit_cast(R, v), reinterpret_cast<R *>(p));
 }
 
+template <bool NTL, typename VT> __device__ inline VT ld_sel(const VT *p) {
+    if constexpr (NTL) return ld_nt(p);
+    else return *p;
+}
+
 // Stores carry the nt hint too.  A/B runs in one process on random data (the knob below): 64 MiB
 // add 6.28 vs 6.10 TB/s, bf16 broadcast 5.9 vs 4.9 TB/s in favour of nt, at every size tried.
 struct Tuning {
@@ -96,8 +101,24 @@ struct Tuning {
     int64_t reduce_row_loads = 4;                 // DXH_TUNE_REDUCE_ROW_LOADS: vectors per lane a row group aims for
     int64_t matmul_tile = 0;                      // DXH_TUNE_MATMUL_TILE: 0 = chosen per shape
     int64_t matmul_splitk = 0;                    // DXH_TUNE_MATMUL_SPLITK: 0 = chosen per shape, 1 = never, n = n slices
+    int64_t nt_load = 0;                          // DXH_TUNE_NT_LOAD: 0 = by op class and size, 1 = always, 2 = never
 };
 Tuning &tuning();  // runtime.hip
+
+// Whether the loads of a streaming kernel carry the nt hint.  Measured on MI355X with buffers
+// rotated through 768 MB (fp32, GB/s with nt / without):
+//   one read per write (scalar, unary)   16 MiB 4671/5528   64 MiB 5907/6657   128 MiB 6238/6898   256 MiB 6340/5905
+//   two reads per write (binary)          4 MiB 2783/3209   16 MiB 5339/5174    64 MiB 6368/5878   256 MiB 6499/5832
+//   read only (row reduction)            16 MiB 3263/3460   64 MiB 5751/5937   128 MiB 6577/6655   256 MiB 6834/5991
+// i.e. plain loads win while the tensors of one launch fit the 256 MiB last-level cache, except
+// for read-dominated streams of more than a few MiB.
+inline bool nt_load_forced(bool by_rule) {
+    const int64_t knob = tuning().nt_load;
+    return knob == 1 ? true : knob == 2 ? false : by_rule;
+}
+inline bool nt_load_1r1w(size_t in_bytes, size_t out_bytes) { return nt_load_forced(in_bytes + out_bytes > ((size_t)256 << 20)); }
+inline bool nt_load_2r1w(size_t total_bytes) { return nt_load_forced(total_bytes > ((size_t)24 << 20)); }
+inline bool nt_load_reduce(size_t in_bytes) { return nt_load_forced(in_bytes > ((size_t)128 << 20)); }
 inline bool use_nt_store(size_t out_bytes) { return (int64_t)out_bytes > tuning().nt_store_bytes; }
 template <bool NT, typename VT> __device__ inline void st_sel(VT *p, const VT &v) {
     if constexpr (NT) st_nt(p, v); else *p = v;

@@ -51,8 +51,8 @@ template <int K, typename A> __device__ inline uint8_t cmp_one(A a, A b, float e
 }
 
 // SCALAR=true compares against `s`, otherwise against b[i].
-template <typename T, int V, int K, bool SCALAR>
-__global__ __launch_bounds__(kBlock) void compare_kernel(const T *__restrict__ a, const T *__restrict__ b, const T s,
+template <typename T, int V, int K, bool SCALAR, bool NTL>
+__device__ __forceinline__ void compare_body(const T *__restrict__ a, const T *__restrict__ b, const T s,
                                                           float eps, uint8_t *__restrict__ m, int64_t n) {
     using VT = vec_t<T, V>;
     using MT = vec_t<uint8_t, V>;
@@ -68,8 +68,8 @@ __global__ __launch_bounds__(kBlock) void compare_kernel(const T *__restrict__ a
         for (int u = 0; u < kUnrollC; ++u) {
             int64_t j = i + u * kBlock;
             if (decltype(full)::value || j < nv) {
-                x[u] = ld_nt(&va[j]);
-                if constexpr (!SCALAR) y[u] = ld_nt(&vb[j]);
+                x[u] = ld_sel<NTL>(&va[j]);
+                if constexpr (!SCALAR) y[u] = ld_sel<NTL>(&vb[j]);
             }
         }
 #pragma unroll
@@ -96,18 +96,25 @@ __global__ __launch_bounds__(kBlock) void compare_kernel(const T *__restrict__ a
         }
     }
 }
+template <typename T, int V, int K, bool SCALAR>
+__global__ __launch_bounds__(kBlock) void compare_kernel(const T *__restrict__ a, const T *__restrict__ b, const T s, float eps, uint8_t *__restrict__ m, int64_t n, int ntl) {
+    if (ntl) compare_body<T, V, K, SCALAR, true>(a, b, s, eps, m, n);
+    else compare_body<T, V, K, SCALAR, false>(a, b, s, eps, m, n);
+}
 
 template <typename T, int K, bool SCALAR>
 int launch_compare(const void *a, const void *b, dxh_scalar s, float eps, void *m, int64_t n, hipStream_t st) {
     if (!aligned(a, sizeof(T)) || (!SCALAR && !aligned(b, sizeof(T)))) return DXH_ERR_ALIGN;
     constexpr int V = vec_len<T>;
     const T sv = SCALAR ? scalar_to<T>(s) : T{};
+    // a comparison reads 4..16 bytes per mask byte: a read-dominated stream
+    const int ntl = SCALAR ? nt_load_reduce((size_t)n * sizeof(T)) : nt_load_2r1w((size_t)n * (2 * sizeof(T) + 1));
     if (aligned(a, kVecBytes) && (SCALAR || aligned(b, kVecBytes)) && aligned(m, V)) {
         unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
-        compare_kernel<T, V, K, SCALAR><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, sv, eps, (uint8_t *)m, n);
+        compare_kernel<T, V, K, SCALAR><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, sv, eps, (uint8_t *)m, n, ntl);
     } else {
         unsigned g = stream_grid(n, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
-        compare_kernel<T, 1, K, SCALAR><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, sv, eps, (uint8_t *)m, n);
+        compare_kernel<T, 1, K, SCALAR><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, sv, eps, (uint8_t *)m, n, ntl);
     }
     return launch_status();
 }
@@ -135,8 +142,8 @@ int compare_all(int dtype, const void *a, const void *b, dxh_scalar s, float eps
 struct SwitchPtrs { const void *p[DXH_SWITCH_MAX]; };
 
 // bool cases, two tensors: C[i] = cases[i] ? t1[i] : t0[i]; both sources stream.
-template <typename R, int V, bool NTS>
-__global__ __launch_bounds__(kBlock) void switch_bool_kernel(const R *__restrict__ t0, const R *__restrict__ t1,
+template <typename R, int V, bool NTS, bool NTL>
+__device__ __forceinline__ void switch_bool_body(const R *__restrict__ t0, const R *__restrict__ t1,
                                                               const uint8_t *__restrict__ cases, R *__restrict__ c, int64_t n) {
     using VT = vec_t<R, V>;
     using MT = vec_t<uint8_t, V>;
@@ -151,7 +158,7 @@ __global__ __launch_bounds__(kBlock) void switch_bool_kernel(const R *__restrict
 #pragma unroll
         for (int u = 0; u < kUnrollC; ++u) {
             int64_t j = i + u * kBlock;
-            if (decltype(full)::value || j < nv) { x[u] = ld_nt(&v0[j]); y[u] = ld_nt(&v1[j]); w[u] = ld_nt(&vm[j]); }
+            if (decltype(full)::value || j < nv) { x[u] = ld_sel<NTL>(&v0[j]); y[u] = ld_sel<NTL>(&v1[j]); w[u] = ld_sel<NTL>(&vm[j]); }
         }
 #pragma unroll
         for (int u = 0; u < kUnrollC; ++u) {
@@ -168,6 +175,11 @@ __global__ __launch_bounds__(kBlock) void switch_bool_kernel(const R *__restrict
         int64_t j = nv * V + threadIdx.x;
         if (j < n) c[j] = cases[j] ? t1[j] : t0[j];
     }
+}
+template <typename R, int V, bool NTS>
+__global__ __launch_bounds__(kBlock) void switch_bool_kernel(const R *__restrict__ t0, const R *__restrict__ t1, const uint8_t *__restrict__ cases, R *__restrict__ c, int64_t n, int ntl) {
+    if (ntl) switch_bool_body<R, V, NTS, true>(t0, t1, cases, c, n);
+    else switch_bool_body<R, V, NTS, false>(t0, t1, cases, c, n);
 }
 
 // int32 cases, up to DXH_SWITCH_MAX tensors: only the selected source is read.
@@ -192,13 +204,14 @@ int launch_switch(const void *const *tensors, int nt, int cases_dtype, const voi
     if (cases_dtype == DXH_BOOL) {
         if (nt != 2) return DXH_ERR_ARG;
         constexpr int V = kVecBytes / (int)sizeof(R);
+        const int ntl = nt_load_2r1w((size_t)n * (3 * sizeof(R) + 1));
         if (aligned(tensors[0], kVecBytes) && aligned(tensors[1], kVecBytes) && aligned(c, kVecBytes) && aligned(cases, V)) {
             unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
-            if (use_nt_store((size_t)n * sizeof(R))) switch_bool_kernel<R, V, true><<<g, kBlock, 0, st>>>((const R *)tensors[0], (const R *)tensors[1], (const uint8_t *)cases, (R *)c, n);
-            else switch_bool_kernel<R, V, false><<<g, kBlock, 0, st>>>((const R *)tensors[0], (const R *)tensors[1], (const uint8_t *)cases, (R *)c, n);
+            if (use_nt_store((size_t)n * sizeof(R))) switch_bool_kernel<R, V, true><<<g, kBlock, 0, st>>>((const R *)tensors[0], (const R *)tensors[1], (const uint8_t *)cases, (R *)c, n, ntl);
+            else switch_bool_kernel<R, V, false><<<g, kBlock, 0, st>>>((const R *)tensors[0], (const R *)tensors[1], (const uint8_t *)cases, (R *)c, n, ntl);
         } else {
             unsigned g = stream_grid(n, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
-            switch_bool_kernel<R, 1, false><<<g, kBlock, 0, st>>>((const R *)tensors[0], (const R *)tensors[1], (const uint8_t *)cases, (R *)c, n);
+            switch_bool_kernel<R, 1, false><<<g, kBlock, 0, st>>>((const R *)tensors[0], (const R *)tensors[1], (const uint8_t *)cases, (R *)c, n, ntl);
         }
     } else if (cases_dtype == DXH_I32) {
         if (!aligned(cases, 4)) return DXH_ERR_ALIGN;
@@ -241,8 +254,8 @@ template <typename D, typename S> __device__ inline D cast_elem(S v) {
     }
 }
 
-template <typename S, typename D, int V, bool NTS>
-__global__ __launch_bounds__(kBlock) void cast_kernel(const S *__restrict__ a, D *__restrict__ c, int64_t n) {
+template <typename S, typename D, int V, bool NTS, bool NTL>
+__device__ __forceinline__ void cast_body(const S *__restrict__ a, D *__restrict__ c, int64_t n) {
     using VS = vec_t<S, V>;
     using VD = vec_t<D, V>;
     const int64_t nv = n / V;
@@ -253,7 +266,7 @@ __global__ __launch_bounds__(kBlock) void cast_kernel(const S *__restrict__ a, D
 #pragma unroll
         for (int u = 0; u < kUnrollC; ++u) {
             int64_t j = i + u * kBlock;
-            if (decltype(full)::value || j < nv) x[u] = ld_nt(&va[j]);
+            if (decltype(full)::value || j < nv) x[u] = ld_sel<NTL>(&va[j]);
         }
 #pragma unroll
         for (int u = 0; u < kUnrollC; ++u) {
@@ -271,18 +284,24 @@ __global__ __launch_bounds__(kBlock) void cast_kernel(const S *__restrict__ a, D
         if (j < n) c[j] = cast_elem<D, S>(a[j]);
     }
 }
+template <typename S, typename D, int V, bool NTS>
+__global__ __launch_bounds__(kBlock) void cast_kernel(const S *__restrict__ a, D *__restrict__ c, int64_t n, int ntl) {
+    if (ntl) cast_body<S, D, V, NTS, true>(a, c, n);
+    else cast_body<S, D, V, NTS, false>(a, c, n);
+}
 
 template <typename S, typename D> int launch_cast(const void *a, void *c, int64_t n, hipStream_t st) {
     if (!aligned(a, sizeof(S)) || !aligned(c, sizeof(D))) return DXH_ERR_ALIGN;
     constexpr int W = sizeof(S) > sizeof(D) ? sizeof(S) : sizeof(D);
     constexpr int V = kVecBytes / W;  // the wider side moves 16 bytes per lane
+    const int ntl = nt_load_1r1w((size_t)n * sizeof(S), (size_t)n * sizeof(D));
     if (aligned(a, V * sizeof(S)) && aligned(c, V * sizeof(D))) {
         unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
-        if (use_nt_store((size_t)n * sizeof(D))) cast_kernel<S, D, V, true><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n);
-        else cast_kernel<S, D, V, false><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n);
+        if (use_nt_store((size_t)n * sizeof(D))) cast_kernel<S, D, V, true><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n, ntl);
+        else cast_kernel<S, D, V, false><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n, ntl);
     } else {
         unsigned g = stream_grid(n, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
-        cast_kernel<S, D, 1, false><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n);
+        cast_kernel<S, D, 1, false><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n, ntl);
     }
     return launch_status();
 }

@@ -71,8 +71,8 @@ template <int U, typename Body> __device__ inline void tile_loop(int64_t nv, Bod
     }
 }
 
-template <typename T, int V, typename Op, bool NTS>
-__global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a, const T *__restrict__ b,
+template <typename T, int V, typename Op, bool NTS, bool NTL>
+__device__ __forceinline__ void binary_body(const T *__restrict__ a, const T *__restrict__ b,
                                                          T *__restrict__ c, int64_t n) {
     using VT = vec_t<T, V>;
     using A = acc_t<T>;
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a,
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             int64_t j = i + u * kBlock;
-            if (decltype(full)::value || j < nv) { x[u] = ld_nt(&va[j]); y[u] = ld_nt(&vb[j]); }
+            if (decltype(full)::value || j < nv) { x[u] = ld_sel<NTL>(&va[j]); y[u] = ld_sel<NTL>(&vb[j]); }
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -104,9 +104,15 @@ __global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a,
         if (j < n) c[j] = store_acc<T>(Op::f(A(load_acc(a[j])), A(load_acc(b[j]))));
     }
 }
-
+// ntl: loads carry the nt hint (chosen per launch, see nt_load_* in common.hpp)
 template <typename T, int V, typename Op, bool NTS>
-__global__ __launch_bounds__(kBlock) void scalar_kernel(const T *__restrict__ a, const T s, T *__restrict__ c, int64_t n) {
+__global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ c, int64_t n, int ntl) {
+    if (ntl) binary_body<T, V, Op, NTS, true>(a, b, c, n);
+    else binary_body<T, V, Op, NTS, false>(a, b, c, n);
+}
+
+template <typename T, int V, typename Op, bool NTS, bool NTL>
+__device__ __forceinline__ void scalar_body(const T *__restrict__ a, const T s, T *__restrict__ c, int64_t n) {
     using VT = vec_t<T, V>;
     using A = acc_t<T>;
     const int64_t nv = n / V;
@@ -118,7 +124,7 @@ __global__ __launch_bounds__(kBlock) void scalar_kernel(const T *__restrict__ a,
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             int64_t j = i + u * kBlock;
-            if (decltype(full)::value || j < nv) x[u] = ld_nt(&va[j]);
+            if (decltype(full)::value || j < nv) x[u] = ld_sel<NTL>(&va[j]);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -136,9 +142,15 @@ __global__ __launch_bounds__(kBlock) void scalar_kernel(const T *__restrict__ a,
         if (j < n) c[j] = store_acc<T>(Op::f(A(load_acc(a[j])), sv));
     }
 }
-
+// ntl: loads carry the nt hint (chosen per launch, see nt_load_* in common.hpp)
 template <typename T, int V, typename Op, bool NTS>
-__global__ __launch_bounds__(kBlock) void unary_kernel(const T *__restrict__ a, T *__restrict__ c, int64_t n) {
+__global__ __launch_bounds__(kBlock) void scalar_kernel(const T *__restrict__ a, const T s, T *__restrict__ c, int64_t n, int ntl) {
+    if (ntl) scalar_body<T, V, Op, NTS, true>(a, s, c, n);
+    else scalar_body<T, V, Op, NTS, false>(a, s, c, n);
+}
+
+template <typename T, int V, typename Op, bool NTS, bool NTL>
+__device__ __forceinline__ void unary_body(const T *__restrict__ a, T *__restrict__ c, int64_t n) {
     using VT = vec_t<T, V>;
     const int64_t nv = n / V;
     const VT *va = reinterpret_cast<const VT *>(a);
@@ -148,7 +160,7 @@ __global__ __launch_bounds__(kBlock) void unary_kernel(const T *__restrict__ a, 
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             int64_t j = i + u * kBlock;
-            if (decltype(full)::value || j < nv) x[u] = ld_nt(&va[j]);
+            if (decltype(full)::value || j < nv) x[u] = ld_sel<NTL>(&va[j]);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -166,19 +178,26 @@ __global__ __launch_bounds__(kBlock) void unary_kernel(const T *__restrict__ a, 
         if (j < n) c[j] = store_acc<T>(Op::f(load_acc(a[j])));
     }
 }
+// ntl: loads carry the nt hint (chosen per launch, see nt_load_* in common.hpp)
+template <typename T, int V, typename Op, bool NTS>
+__global__ __launch_bounds__(kBlock) void unary_kernel(const T *__restrict__ a, T *__restrict__ c, int64_t n, int ntl) {
+    if (ntl) unary_body<T, V, Op, NTS, true>(a, c, n);
+    else unary_body<T, V, Op, NTS, false>(a, c, n);
+}
 
 // ---- host launchers ---------------------------------------------------------------------
 template <typename T, typename Op>
 int launch_binary(const void *a, const void *b, void *c, int64_t n, hipStream_t st) {
     if (!aligned(a, sizeof(T)) || !aligned(b, sizeof(T)) || !aligned(c, sizeof(T))) return DXH_ERR_ALIGN;
     constexpr int V = vec_len<T>;
+    const int ntl = nt_load_2r1w((size_t)n * sizeof(T) * 3);
     if (aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes)) {
         unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnroll, kBlocksPerCU);
-        if (use_nt_store((size_t)n * sizeof(T))) binary_kernel<T, V, Op, true><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n);
-        else binary_kernel<T, V, Op, false><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n);
+        if (use_nt_store((size_t)n * sizeof(T))) binary_kernel<T, V, Op, true><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n, ntl);
+        else binary_kernel<T, V, Op, false><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n, ntl);
     } else {
         unsigned g = stream_grid(n, (int64_t)kBlock * kUnroll, kBlocksPerCU);
-        binary_kernel<T, 1, Op, false><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n);
+        binary_kernel<T, 1, Op, false><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n, ntl);
     }
     return launch_status();
 }
@@ -187,13 +206,14 @@ int launch_scalar(const void *a, dxh_scalar s, void *c, int64_t n, hipStream_t s
     if (!aligned(a, sizeof(T)) || !aligned(c, sizeof(T))) return DXH_ERR_ALIGN;
     constexpr int V = vec_len<T>;
     const T sv = scalar_to<T>(s);
+    const int ntl = nt_load_1r1w((size_t)n * sizeof(T), (size_t)n * sizeof(T));
     if (aligned(a, kVecBytes) && aligned(c, kVecBytes)) {
         unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnroll, kBlocksPerCU);
-        if (use_nt_store((size_t)n * sizeof(T))) scalar_kernel<T, V, Op, true><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n);
-        else scalar_kernel<T, V, Op, false><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n);
+        if (use_nt_store((size_t)n * sizeof(T))) scalar_kernel<T, V, Op, true><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n, ntl);
+        else scalar_kernel<T, V, Op, false><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n, ntl);
     } else {
         unsigned g = stream_grid(n, (int64_t)kBlock * kUnroll, kBlocksPerCU);
-        scalar_kernel<T, 1, Op, false><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n);
+        scalar_kernel<T, 1, Op, false><<<g, kBlock, 0, st>>>((const T *)a, sv, (T *)c, n, ntl);
     }
     return launch_status();
 }
@@ -201,13 +221,14 @@ template <typename T, typename Op>
 int launch_unary(const void *a, void *c, int64_t n, hipStream_t st) {
     if (!aligned(a, sizeof(T)) || !aligned(c, sizeof(T))) return DXH_ERR_ALIGN;
     constexpr int V = vec_len<T>;
+    const int ntl = nt_load_1r1w((size_t)n * sizeof(T), (size_t)n * sizeof(T));
     if (aligned(a, kVecBytes) && aligned(c, kVecBytes)) {
         unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnroll, kBlocksPerCU);
-        if (use_nt_store((size_t)n * sizeof(T))) unary_kernel<T, V, Op, true><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n);
-        else unary_kernel<T, V, Op, false><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n);
+        if (use_nt_store((size_t)n * sizeof(T))) unary_kernel<T, V, Op, true><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n, ntl);
+        else unary_kernel<T, V, Op, false><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n, ntl);
     } else {
         unsigned g = stream_grid(n, (int64_t)kBlock * kUnroll, kBlocksPerCU);
-        unary_kernel<T, 1, Op, false><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n);
+        unary_kernel<T, 1, Op, false><<<g, kBlock, 0, st>>>((const T *)a, (T *)c, n, ntl);
     }
     return launch_status();
 }

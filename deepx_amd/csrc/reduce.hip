@@ -78,12 +78,11 @@ template <typename A> __device__ inline A shfl_xor_any(A v, int off) {
 // in [pre, R] (R contiguous) -> out [pre, S]; chunk s covers r in [s*chunk, min(R,(s+1)*chunk)).
 // G lanes cooperate on one (row, chunk); G in {1,2,..,64} packs 256/G rows per workgroup,
 // G == 256 gives the whole workgroup to one row.
-template <int K, typename Tin, typename Tout, typename TS, int V>
-__global__ __launch_bounds__(kBlock) void reduce_row_kernel(const Tin *__restrict__ in, Tout *__restrict__ out,
+template <int K, typename Tin, typename Tout, typename TS, int V, bool NTL>
+__device__ __forceinline__ void reduce_row_body(racc_t<TS> *lds, const Tin *__restrict__ in, Tout *__restrict__ out,
                                                              int64_t pre, int64_t R, int S, int64_t chunk, int G) {
     using A = racc_t<TS>;
     using VT = vec_t<Tin, V>;
-    __shared__ A lds[kBlock / kWave];
     const int rows_per_block = kBlock / G;
     const int lane = threadIdx.x % G;
     const int64_t row = (int64_t)blockIdx.x * rows_per_block + threadIdx.x / G;
@@ -104,7 +103,7 @@ __global__ __launch_bounds__(kBlock) void reduce_row_kernel(const Tin *__restric
         for (; i + 7 * (int64_t)G < lv; i += 8 * (int64_t)G) {
             VT x[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) x[u] = ld_nt(&pv[i + u * (int64_t)G]);
+            for (int u = 0; u < 8; ++u) x[u] = ld_sel<NTL>(&pv[i + u * (int64_t)G]);
 #pragma unroll
             for (int k = 0; k < V; ++k) {
                 A t0 = rop<K, A>(rop<K, A>(rload<A>(x[0].v[k]), rload<A>(x[1].v[k])), rop<K, A>(rload<A>(x[2].v[k]), rload<A>(x[3].v[k])));
@@ -113,7 +112,7 @@ __global__ __launch_bounds__(kBlock) void reduce_row_kernel(const Tin *__restric
             }
         }
         for (; i + 3 * (int64_t)G < lv; i += 4 * (int64_t)G) {
-            VT x0 = ld_nt(&pv[i]), x1 = ld_nt(&pv[i + G]), x2 = ld_nt(&pv[i + 2 * (int64_t)G]), x3 = ld_nt(&pv[i + 3 * (int64_t)G]);
+            VT x0 = ld_sel<NTL>(&pv[i]), x1 = ld_sel<NTL>(&pv[i + G]), x2 = ld_sel<NTL>(&pv[i + 2 * (int64_t)G]), x3 = ld_sel<NTL>(&pv[i + 3 * (int64_t)G]);
 #pragma unroll
             for (int k = 0; k < V; ++k) {
                 A t0 = rop<K, A>(rload<A>(x0.v[k]), rload<A>(x1.v[k]));
@@ -122,7 +121,7 @@ __global__ __launch_bounds__(kBlock) void reduce_row_kernel(const Tin *__restric
             }
         }
         for (; i < lv; i += G) {
-            VT x = ld_nt(&pv[i]);
+            VT x = ld_sel<NTL>(&pv[i]);
 #pragma unroll
             for (int k = 0; k < V; ++k) acc[k] = rop<K, A>(acc[k], rload<A>(x.v[k]));
         }
@@ -147,17 +146,24 @@ __global__ __launch_bounds__(kBlock) void reduce_row_kernel(const Tin *__restric
         out[row * S + s] = rstore<Tout, A>(v);
     }
 }
+// ntl: loads carry the nt hint (chosen per launch, see nt_load_reduce in common.hpp)
+template <int K, typename Tin, typename Tout, typename TS, int V>
+__global__ __launch_bounds__(kBlock) void reduce_row_kernel(const Tin *__restrict__ in, Tout *__restrict__ out, int64_t pre, int64_t R, int S, int64_t chunk, int G, int ntl) {
+    using A = racc_t<TS>;
+    __shared__ A lds[kBlock / kWave];
+    if (ntl) reduce_row_body<K, Tin, Tout, TS, V, true>(lds, in, out, pre, R, S, chunk, G);
+    else reduce_row_body<K, Tin, Tout, TS, V, false>(lds, in, out, pre, R, S, chunk, G);
+}
 
 // ---- col stage ---------------------------------------------------------------------------
 // in [pre, R, post] -> out [pre, S, post].  Workgroup = TX column-lanes x TY row-lanes
 // (TX*TY == 256); a column-lane owns V adjacent columns.  Linear block id -> (p, s, ctile).
-template <int K, typename Tin, typename Tout, typename TS, int V>
-__global__ __launch_bounds__(kBlock) void reduce_col_kernel(const Tin *__restrict__ in, Tout *__restrict__ out,
+template <int K, typename Tin, typename Tout, typename TS, int V, bool NTL>
+__device__ __forceinline__ void reduce_col_body(racc_t<TS> *lds, const Tin *__restrict__ in, Tout *__restrict__ out,
                                                              int64_t pre, int64_t R, int64_t post, int S, int64_t chunk,
                                                              int TX, int ctiles) {
     using A = racc_t<TS>;
     using VT = vec_t<Tin, V>;
-    __shared__ A lds[kBlock * V];
     const int TY = kBlock / TX;
     const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
     int64_t b = blockIdx.x;
@@ -180,7 +186,7 @@ __global__ __launch_bounds__(kBlock) void reduce_col_kernel(const Tin *__restric
         if (r + 7 * (int64_t)TY < r1) {
             VT x[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) x[u] = ld_nt(&base[(r + u * (int64_t)TY) * postv]);
+            for (int u = 0; u < 8; ++u) x[u] = ld_sel<NTL>(&base[(r + u * (int64_t)TY) * postv]);
             r += 8 * (int64_t)TY;
             auto fold = [&](const VT(&b)[8]) __attribute__((always_inline)) {
 #pragma unroll
@@ -193,7 +199,7 @@ __global__ __launch_bounds__(kBlock) void reduce_col_kernel(const Tin *__restric
             for (; r + 7 * (int64_t)TY < r1; r += 8 * (int64_t)TY) {
                 VT y[8];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) y[u] = ld_nt(&base[(r + u * (int64_t)TY) * postv]);
+                for (int u = 0; u < 8; ++u) y[u] = ld_sel<NTL>(&base[(r + u * (int64_t)TY) * postv]);
                 fold(x);
 #pragma unroll
                 for (int u = 0; u < 8; ++u) x[u] = y[u];
@@ -201,7 +207,7 @@ __global__ __launch_bounds__(kBlock) void reduce_col_kernel(const Tin *__restric
             fold(x);
         }
         for (; r < r1; r += TY) {
-            VT x = ld_nt(&base[r * postv]);
+            VT x = ld_sel<NTL>(&base[r * postv]);
 #pragma unroll
             for (int k = 0; k < V; ++k) acc[k] = rop<K, A>(acc[k], rload<A>(x.v[k]));
         }
@@ -222,6 +228,14 @@ __global__ __launch_bounds__(kBlock) void reduce_col_kernel(const Tin *__restric
 #pragma unroll
         for (int k = 0; k < V; ++k) o[k] = rstore<Tout, A>(lds[(k * TY) * TX + tx]);
     }
+}
+// ntl: loads carry the nt hint (chosen per launch, see nt_load_reduce in common.hpp)
+template <int K, typename Tin, typename Tout, typename TS, int V>
+__global__ __launch_bounds__(kBlock) void reduce_col_kernel(const Tin *__restrict__ in, Tout *__restrict__ out, int64_t pre, int64_t R, int64_t post, int S, int64_t chunk, int TX, int ctiles, int ntl) {
+    using A = racc_t<TS>;
+    __shared__ A lds[kBlock * V];
+    if (ntl) reduce_col_body<K, Tin, Tout, TS, V, true>(lds, in, out, pre, R, post, S, chunk, TX, ctiles);
+    else reduce_col_body<K, Tin, Tout, TS, V, false>(lds, in, out, pre, R, post, S, chunk, TX, ctiles);
 }
 
 // fill `n` outputs with the identity (a reduced axis of size 0), or copy (nothing to reduce)
@@ -395,15 +409,16 @@ inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, cons
 template <int K, typename Tin, typename Tout, typename TS>
 int launch_stage(const Stage &st, const void *in, void *out, hipStream_t stream) {
     constexpr int VF = kVecBytes / (int)sizeof(Tin);
+    const int ntl = nt_load_reduce((size_t)(st.pre * st.R * st.post) * sizeof(Tin));
     if (st.row) {
         const int rows_per_block = kBlock / st.G;
         int64_t gx = (st.pre + rows_per_block - 1) / rows_per_block;
         if (gx > 0x7fffffff || st.S > 65535) return DXH_ERR_SHAPE;
         dim3 grid((unsigned)gx, (unsigned)st.S);
         if (st.V == VF && aligned(in, kVecBytes))
-            reduce_row_kernel<K, Tin, Tout, TS, VF><<<grid, kBlock, 0, stream>>>((const Tin *)in, (Tout *)out, st.pre, st.R, st.S, st.chunk, st.G);
+            reduce_row_kernel<K, Tin, Tout, TS, VF><<<grid, kBlock, 0, stream>>>((const Tin *)in, (Tout *)out, st.pre, st.R, st.S, st.chunk, st.G, ntl);
         else
-            reduce_row_kernel<K, Tin, Tout, TS, 1><<<grid, kBlock, 0, stream>>>((const Tin *)in, (Tout *)out, st.pre, st.R, st.S, st.chunk, st.G);
+            reduce_row_kernel<K, Tin, Tout, TS, 1><<<grid, kBlock, 0, stream>>>((const Tin *)in, (Tout *)out, st.pre, st.R, st.S, st.chunk, st.G, ntl);
     } else {
         bool vec = st.V == VF && aligned(in, kVecBytes);
         int TX = st.TX, ctiles = st.ctiles;
@@ -414,9 +429,9 @@ int launch_stage(const Stage &st, const void *in, void *out, hipStream_t stream)
         int64_t gx = st.pre * st.S * ctiles;
         if (gx > 0x7fffffff) return DXH_ERR_SHAPE;
         if (vec)
-            reduce_col_kernel<K, Tin, Tout, TS, VF><<<(unsigned)gx, kBlock, 0, stream>>>((const Tin *)in, (Tout *)out, st.pre, st.R, st.post, st.S, st.chunk, TX, ctiles);
+            reduce_col_kernel<K, Tin, Tout, TS, VF><<<(unsigned)gx, kBlock, 0, stream>>>((const Tin *)in, (Tout *)out, st.pre, st.R, st.post, st.S, st.chunk, TX, ctiles, ntl);
         else
-            reduce_col_kernel<K, Tin, Tout, TS, 1><<<(unsigned)gx, kBlock, 0, stream>>>((const Tin *)in, (Tout *)out, st.pre, st.R, st.post, st.S, st.chunk, TX, ctiles);
+            reduce_col_kernel<K, Tin, Tout, TS, 1><<<(unsigned)gx, kBlock, 0, stream>>>((const Tin *)in, (Tout *)out, st.pre, st.R, st.post, st.S, st.chunk, TX, ctiles, ntl);
     }
     return launch_status();
 }

@@ -312,3 +312,37 @@ def test_config1_chain_full_size(dxh, orc):
     den = np.abs(B) + np.float32(1.0)
     assert np.array_equal(d["d"].get(), den)
     assert np.array_equal(d["G"].get(), Fg / den)  # div is exact on the device's own F
+
+
+def test_nt_load_knob_gives_identical_results(dxh):
+    """The non-temporal hint on loads is a cache policy, chosen per launch by op class and size:
+    forcing it on (1) or off (2) through the tuning knob must not change a single bit of an
+    elementwise, compare, cast or reduce result."""
+    NT_LOAD_KNOB = 7  # DXH_TUNE_NT_LOAD
+    rng = np.random.default_rng(4242)
+    n = 300_001
+    A = rng.standard_normal(n).astype(np.float32)
+    B = rng.standard_normal(n).astype(np.float32)
+    dA, dB = Dev(A), Dev(B)
+    results = {}
+    for knob in (0, 1, 2):
+        dx.check(dxh.dxh_tune(NT_LOAD_KNOB, knob))
+        try:
+            dC, dS, dU, dM, dH = Dev.empty(n, np.float32), Dev.empty(n, np.float32), Dev.empty(n, np.float32), Dev.empty(n, np.uint8), Dev.empty(n, np.uint16)
+            dx.check(dxh.dxh_add(dx.F32, dA.ptr, dB.ptr, dC.ptr, n, None))
+            dx.check(dxh.dxh_mulscalar(dx.F32, dA.ptr, dx.scalar(1.5), dS.ptr, n, None))
+            dx.check(dxh.dxh_exp(dx.F32, dA.ptr, dU.ptr, n, None))
+            dx.check(dxh.dxh_less(dx.F32, dA.ptr, dB.ptr, dM.ptr, n, None))
+            dx.check(dxh.dxh_todtype(dx.F32, dA.ptr, dx.BF16, dH.ptr, n, None))
+            rows, cols = 300, 1000
+            dR, dK = Dev.empty(rows, np.float32), Dev.empty(cols, np.float32)
+            ws = Dev.empty(1 << 20, np.uint8)
+            sh = dx.i32arr([rows, cols])
+            dx.check(dxh.dxh_sum(dx.F32, dA.ptr, sh, 2, dx.i32arr([1]), 1, dR.ptr, ws.ptr, 1 << 20, None))
+            dx.check(dxh.dxh_reducemax(dx.F32, dA.ptr, sh, 2, dx.i32arr([0]), 1, dK.ptr, ws.ptr, 1 << 20, None))
+            results[knob] = [d.get().copy() for d in (dC, dS, dU, dM, dH, dR, dK)]
+        finally:
+            dx.check(dxh.dxh_tune(NT_LOAD_KNOB, 0))
+    for knob in (1, 2):
+        for got, want in zip(results[knob], results[0]):
+            assert np.array_equal(got, want), knob

@@ -84,6 +84,21 @@ template <typename VT> __device__ inline void st_nt(VT *p, const VT &v) {
     __builtin_nontemporal_store(__builtin_bit_cast(R, v), reinterpret_cast<R *>(p));
 }
 
+// Store policy of a streaming kernel: 0 plain, 1 nt, 2 write-through at system scope (sc0 sc1;
+// 16-byte stores only, narrower ones fall back to nt).  The last is the fastest partner of nt
+// loads when two tensors are read per tensor written (see stream_policy_2r1w).
+template <int ST, typename VT> __device__ inline void st_mode(VT *p, const VT &v) {
+    if constexpr (ST == 0) {
+        *p = v;
+    } else if constexpr (ST == 2 && sizeof(VT) == 16) {
+        const u32x4_t r = __builtin_bit_cast(u32x4_t, v);
+        // s_nop: a VALU write to the data registers of a 16-byte store needs a wait state after the
+        // store, which the compiler inserts for its own stores but not behind inline assembly
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(r) : "memory");
+    } else {
+        st_nt(p, v);
+    }
+}
 template <bool NTL, typename VT> __device__ inline VT ld_sel(const VT *p) {
     if constexpr (NTL) return ld_nt(p);
     else return *p;
@@ -118,6 +133,14 @@ inline bool nt_load_forced(bool by_rule) {
 }
 inline bool nt_load_1r1w(size_t in_bytes, size_t out_bytes) { return nt_load_forced(in_bytes + out_bytes > ((size_t)256 << 20)); }
 inline bool nt_load_2r1w(size_t total_bytes) { return nt_load_forced(total_bytes > ((size_t)24 << 20)); }
+// Two reads per write, loads and stores together (fp32 add, GB/s, MiB per tensor):
+//   loads nt, stores nt       32: 5869   64: 6367   128: 6593   256: 6451
+//   loads nt, stores sc0 sc1  32: 6197   64: 6758   128: 7138   256: 6264
+// 0 = plain loads + nt stores, 1 = nt loads + nt stores, 2 = nt loads + sc0 sc1 stores
+inline int stream_policy_2r1w(size_t total_bytes) {
+    if (!nt_load_2r1w(total_bytes)) return 0;
+    return total_bytes <= ((size_t)512 << 20) ? 2 : 1;
+}
 inline bool nt_load_reduce(size_t in_bytes) { return nt_load_forced(in_bytes > ((size_t)128 << 20)); }
 inline bool use_nt_store(size_t out_bytes) { return (int64_t)out_bytes > tuning().nt_store_bytes; }
 template <bool NT, typename VT> __device__ inline void st_sel(VT *p, const VT &v) {

@@ -71,7 +71,7 @@ template <int U, typename Body> __device__ inline void tile_loop(int64_t nv, Bod
     }
 }
 
-template <typename T, int V, typename Op, bool NTS, bool NTL>
+template <typename T, int V, typename Op, int ST, bool NTL>
 __device__ __forceinline__ void binary_body(const T *__restrict__ a, const T *__restrict__ b,
                                                          T *__restrict__ c, int64_t n) {
     using VT = vec_t<T, V>;
@@ -94,7 +94,7 @@ __device__ __forceinline__ void binary_body(const T *__restrict__ a, const T *__
                 VT r;
 #pragma unroll
                 for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(A(load_acc(x[u].v[k])), A(load_acc(y[u].v[k]))));
-                st_sel<NTS>(&vc[j], r);
+                st_mode<ST>(&vc[j], r);
             }
         }
     });
@@ -107,8 +107,14 @@ __device__ __forceinline__ void binary_body(const T *__restrict__ a, const T *__
 // ntl: loads carry the nt hint (chosen per launch, see nt_load_* in common.hpp)
 template <typename T, int V, typename Op, bool NTS>
 __global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ c, int64_t n, int ntl) {
-    if (ntl) binary_body<T, V, Op, NTS, true>(a, b, c, n);
-    else binary_body<T, V, Op, NTS, false>(a, b, c, n);
+    if constexpr (NTS) {  // ntl here: a stream_policy_2r1w value
+        if (ntl == 2) binary_body<T, V, Op, 2, true>(a, b, c, n);
+        else if (ntl == 1) binary_body<T, V, Op, 1, true>(a, b, c, n);
+        else binary_body<T, V, Op, 1, false>(a, b, c, n);
+    } else {
+        if (ntl) binary_body<T, V, Op, 0, true>(a, b, c, n);
+        else binary_body<T, V, Op, 0, false>(a, b, c, n);
+    }
 }
 
 template <typename T, int V, typename Op, bool NTS, bool NTL>
@@ -190,7 +196,7 @@ template <typename T, typename Op>
 int launch_binary(const void *a, const void *b, void *c, int64_t n, hipStream_t st) {
     if (!aligned(a, sizeof(T)) || !aligned(b, sizeof(T)) || !aligned(c, sizeof(T))) return DXH_ERR_ALIGN;
     constexpr int V = vec_len<T>;
-    const int ntl = nt_load_2r1w((size_t)n * sizeof(T) * 3);
+    const int ntl = stream_policy_2r1w((size_t)n * sizeof(T) * 3);
     if (aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes)) {
         unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnroll, kBlocksPerCU);
         if (use_nt_store((size_t)n * sizeof(T))) binary_kernel<T, V, Op, true><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, n, ntl);

@@ -102,7 +102,7 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const void *__restr
         }
 #pragma unroll
         for (int u = 0; u < kGatherUnroll; ++u)
-            if (g[u] < total) st_sel<NTS>(&out[g[u]], x[u]);
+            if (g[u] < total) st_mode<NTS ? 3 : 0>(&out[g[u]], x[u]);
     }
 }
 
@@ -301,7 +301,7 @@ __global__ __launch_bounds__(kBlock) void tile_transpose_vec_kernel(const char *
             const int c = crow + 16 * i;
             const int64_t gc = (int64_t)tc * T + c;
             if (gc < nC && a0 < nA)
-                __builtin_nontemporal_store(lds[c * 16 + (ablk ^ ((c / V) & 15))], reinterpret_cast<tt_u32x4 *>(out + (ooff + gc * oC + a0) * ES));
+                st_mode<3>(reinterpret_cast<tt_u32x4 *>(out + (ooff + gc * oC + a0) * ES), lds[c * 16 + (ablk ^ ((c / V) & 15))]);
         }
     }
 }
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(kBlock) void concat_kernel(ConcatSrcs s, U *__restr
             o = g / run;
             v = g - o * run;
         }
-        st_nt(&out[o * out_row + pref + v], ld_nt(&src[g]));
+        st_mode<3>(&out[o * out_row + pref + v], ld_nt(&src[g]));
     }
 }
 
@@ -374,7 +374,7 @@ __global__ __launch_bounds__(kBlock) void indexselect_kernel(const U *__restrict
         }
 #pragma unroll
         for (int u = 0; u < kGatherUnroll; ++u)
-            if (g[u] < total) st_nt(&out[g[u]], x[u]);
+            if (g[u] < total) st_mode<3>(&out[g[u]], x[u]);
     }
 }
 

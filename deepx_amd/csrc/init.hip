@@ -14,7 +14,7 @@ __global__ __launch_bounds__(kBlock) void constant_kernel(T *__restrict__ out, i
     for (int k = 0; k < V; ++k) r.v[k] = value;
     VT *vo = reinterpret_cast<VT *>(out);
     const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nv; i += stride) st_nt(&vo[i], r);
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nv; i += stride) st_mode<3>(&vo[i], r);
     if (blockIdx.x == 0) {
         int64_t j = nv * V + threadIdx.x;
         if (j < n) out[j] = value;

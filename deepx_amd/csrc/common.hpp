@@ -66,8 +66,9 @@ template <> struct raw_of<8> { using type = uint64_t; };
 template <> struct raw_of<16> { using type = uint4; };
 
 // ---- streaming (non-temporal) global access ------------------------------------------------
-// Every tensor of an elementwise / changeshape / reduce op is touched exactly once, so loads and
-// stores carry the `nt` hint: on MI355X this lifted a streaming add from ~5.0 to ~6.5 TB/s.
+// Every tensor of an elementwise / changeshape / reduce op is touched exactly once.  The `nt`
+// hint lifted a streaming add from ~5.0 to ~6.5 TB/s on MI355X; which loads and stores carry it
+// (or one of the scope bits) is decided per launch: nt_load_*, stream_policy_2r1w, st_mode below.
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 template <int BYTES> struct nt_raw;
 template <> struct nt_raw<1> { using type = uint8_t; };

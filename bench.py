@@ -111,14 +111,14 @@ def main():
     n_ops = sum(len(ops) for _, ops in groups)
     rot = [0]
 
-    def run_step(events=None):
+    def run_step(events=None, stream=None):
         for gi, (kern, ops) in enumerate(groups):
             if events is not None:
                 L.dxh_event_record(events[gi][0], None)
             for (label, fn, sh, ax, bufs, nbytes) in ops:
                 buf = bufs[rot[0] % NX]
                 rot[0] += 1
-                rc = fn(dx.F32, ptr(buf), sh, 2, ax, 1, ptr(out), ptr(ws), wsb.value, None)
+                rc = fn(dx.F32, ptr(buf), sh, 2, ax, 1, ptr(out), ptr(ws), wsb.value, stream)
                 if rc != 0:
                     dx.check(rc, label)
             if events is not None:
@@ -149,6 +149,29 @@ def main():
         nb = ops[0][5]
         c2[kern] = {"ops": [o[0] for o in ops], "avg_launch_ms": round(ms, 5), "GB/s": round(nb / ms / 1e6, 1),
                     "frac_hbm": round(nb / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes_per_launch": nb}
+    # For information, not `value`: the same step recorded once into a HIP graph (dxh_graph_*, what
+    # the executor does for repeated multi-line datagrams) and replayed; NX steps per graph so the
+    # rotation of the input copies is the same as above.
+    gst, gexec = C.c_void_p(), C.c_void_p()
+    dx.check(L.dxh_stream_create(C.byref(gst)))
+    rot[0] = 0
+    dx.check(L.dxh_graph_begin_capture(gst))
+    for _ in range(NX):
+        run_step(stream=gst)
+    dx.check(L.dxh_graph_end_capture(gst, C.byref(gexec)))
+    for _ in range(40):
+        dx.check(L.dxh_graph_launch(gexec, gst))
+    dx.check(L.dxh_stream_sync(gst))
+    g_t0 = time.perf_counter()
+    g_reps = max(1, args.steps // NX + 1)
+    for _ in range(g_reps):
+        dx.check(L.dxh_graph_launch(gexec, gst))
+    dx.check(L.dxh_stream_sync(gst))
+    graph_ms_per_step = (time.perf_counter() - g_t0) * 1e3 / (g_reps * NX)
+    dx.check(L.dxh_graph_destroy(gexec))
+    dx.check(L.dxh_stream_destroy(gst))
+    c2["step_as_recorded_hip_graph"] = {"ms_per_step": round(graph_ms_per_step, 4), "GB/s": round(step_bytes / graph_ms_per_step / 1e6, 1),
+                                        "frac_hbm": round(step_bytes / graph_ms_per_step / 1e6 / HBM_PEAK_GBS, 4), "bytes": step_bytes}
     dom_ms = group_ms["reduce_row_kernel"]
     achieved = XB / dom_ms / 1e6
     roofline = {"bound": "hbm", "kernel": "reduce_row_kernel<sum|max|min,f32> [8192,8192] axis 1 (6 of 10 launches per step)",

@@ -113,7 +113,7 @@ def main():
 
     def run_step(events=None, stream=None):
         for gi, (kern, ops) in enumerate(groups):
-            if events is not None:
+            if events is not None and events[gi] is not None:
                 L.dxh_event_record(events[gi][0], None)
             for (label, fn, sh, ax, bufs, nbytes) in ops:
                 buf = bufs[rot[0] % NX]
@@ -121,11 +121,15 @@ def main():
                 rc = fn(dx.F32, ptr(buf), sh, 2, ax, 1, ptr(out), ptr(ws), wsb.value, stream)
                 if rc != 0:
                     dx.check(rc, label)
-            if events is not None:
+            if events is not None and events[gi] is not None:
                 L.dxh_event_record(events[gi][1], None)
 
+    # Inside the timed region only the dominant kernel's group carries an event pair (an event
+    # record is a barrier packet of its own and costs the step about a microsecond); the other
+    # groups are timed the same way in a pass of their own after it.
     ev = Events()
-    step_events = [[ev.pair() for _ in groups] for _ in range(args.steps)]
+    step_events = [[ev.pair() if gi == 0 else None for gi, _ in enumerate(groups)] for _ in range(args.steps)]
+    info_events = [[ev.pair() for _ in groups] for _ in range(args.steps)]
     ramp_t0 = time.perf_counter()
     while (time.perf_counter() - ramp_t0) * 1e3 < args.ramp_ms:  # untimed: clocks settle
         run_step()
@@ -141,10 +145,14 @@ def main():
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
+    for s in range(args.steps):  # untimed pass: every group with its own event pair
+        run_step(info_events[s])
+    torch.cuda.synchronize()
     c2 = {}
     group_ms = {}
     for gi, (kern, ops) in enumerate(groups):
-        ms = float(np.mean([Events.ms(*step_events[s][gi]) for s in range(args.steps)])) / len(ops)
+        src = step_events if gi == 0 else info_events
+        ms = float(np.mean([Events.ms(*src[s][gi]) for s in range(args.steps)])) / len(ops)
         group_ms[kern] = ms
         nb = ops[0][5]
         c2[kern] = {"ops": [o[0] for o in ops], "avg_launch_ms": round(ms, 5), "GB/s": round(nb / ms / 1e6, 1),

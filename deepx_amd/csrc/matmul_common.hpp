@@ -18,6 +18,24 @@ __device__ __forceinline__ void static_for_impl(F &f, std::integer_sequence<int,
 template <int N, typename F> __device__ __forceinline__ void static_for(F f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
 template <int V> using ic = std::integral_constant<int, V>;
 
+// Issue order inside a scheduling region of a matrix-pipe kernel: after each of `mfmas` MFMAs an
+// even share of the region's LDS reads, LDS writes and global loads (counts are upper bounds: a
+// paired ds_read2 counts once), so that the matrix pipe always has the next MFMA queued while the
+// memory instructions are issued underneath it.  Left alone, the compiler reads each operand
+// right before the MFMA that uses it and the pipe idles for an LDS latency every few MFMAs.
+template <typename M, typename R, typename W, typename L>
+__device__ __forceinline__ void interleave(M, R, W, L) {
+    constexpr int nm = M::value, nr = R::value, nw = W::value, nl = L::value;
+    static_for<nm>([&](auto x) __attribute__((always_inline)) {
+        constexpr int m = decltype(x)::value;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        constexpr int r = nr * (m + 1) / nm - nr * m / nm, wr = nw * (m + 1) / nm - nw * m / nm, l = nl * (m + 1) / nm - nl * m / nm;
+        if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);   // LDS reads
+        if constexpr (wr > 0) __builtin_amdgcn_sched_group_barrier(0x200, wr, 0);  // LDS writes
+        if constexpr (l > 0) __builtin_amdgcn_sched_group_barrier(0x020, l, 0);   // global loads
+    });
+}
+
 
 // ---- XCD-aware workgroup -> tile map (shared by the MFMA kernels) ---------------------------
 // Workgroups are dealt round-robin to the 8 XCDs, each with a private L2.  XCD x takes the

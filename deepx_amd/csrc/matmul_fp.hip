@@ -118,19 +118,6 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[buf][j][e], fa[buf][i][e >> 2][e & 3], acc[i][j], 0, 0, 0);
         });
     };
-    // Issue order inside a scheduling region: after each MFMA an even share of the region's LDS
-    // reads, LDS writes and global loads (counts are upper bounds: paired ds_read2 count once).
-    auto interleave = [&](auto mfmas, auto reads, auto writes, auto loads) __attribute__((always_inline)) {
-        constexpr int nm = decltype(mfmas)::value, nr = decltype(reads)::value, nw = decltype(writes)::value, nl = decltype(loads)::value;
-        static_for<nm>([&](auto x) __attribute__((always_inline)) {
-            constexpr int m = decltype(x)::value;
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            constexpr int r = nr * (m + 1) / nm - nr * m / nm, wr = nw * (m + 1) / nm - nw * m / nm, l = nl * (m + 1) / nm - nl * m / nm;
-            if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
-            if constexpr (wr > 0) __builtin_amdgcn_sched_group_barrier(0x200, wr, 0);
-            if constexpr (l > 0) __builtin_amdgcn_sched_group_barrier(0x020, l, 0);
-        });
-    };
 
     // One K step: LDS stage S is multiplied (its group 0 is already in a fragment buffer); register
     // set R (K step k_store) moves into stage S^1 and is refilled with K step k_load.  The LDS
@@ -338,17 +325,6 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double
         static_for<decltype(hi)::value - decltype(lo)::value>([&](auto x) __attribute__((always_inline)) {
             constexpr int idx = decltype(lo)::value + decltype(x)::value, e = idx / (RT * CT), i = idx % (RT * CT) / CT, j = idx % CT;
             acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[buf][i][e], fb[buf][j][e], acc[i][j], 0, 0, 0);
-        });
-    };
-    auto interleave = [&](auto mfmas, auto reads, auto writes, auto loads) __attribute__((always_inline)) {
-        constexpr int nm = decltype(mfmas)::value, nr = decltype(reads)::value, nw = decltype(writes)::value, nl = decltype(loads)::value;
-        static_for<nm>([&](auto x) __attribute__((always_inline)) {
-            constexpr int m = decltype(x)::value;
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            constexpr int r = nr * (m + 1) / nm - nr * m / nm, wr = nw * (m + 1) / nm - nw * m / nm, l = nl * (m + 1) / nm - nl * m / nm;
-            if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
-            if constexpr (wr > 0) __builtin_amdgcn_sched_group_barrier(0x200, wr, 0);
-            if constexpr (l > 0) __builtin_amdgcn_sched_group_barrier(0x020, l, 0);
         });
     };
     // One K step: stage S is multiplied (its group 0 already sits in fragment buffer 0); the

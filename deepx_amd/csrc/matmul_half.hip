@@ -256,20 +256,6 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
             acc[i][j] = mfma32<T>(fb[buf][j], fa[buf][i], acc[i][j]);
         });
     };
-    // Issue order inside a scheduling region: after each of `mfmas` MFMAs an even share of the
-    // region's LDS reads, LDS writes and global loads, so that the matrix pipe always has the next
-    // MFMA queued while the memory instructions are issued underneath it.
-    auto interleave = [&](auto mfmas, auto reads, auto writes, auto loads) __attribute__((always_inline)) {
-        constexpr int nm = decltype(mfmas)::value, nr = decltype(reads)::value, nw = decltype(writes)::value, nl = decltype(loads)::value;
-        static_for<nm>([&](auto x) __attribute__((always_inline)) {
-            constexpr int m = decltype(x)::value;
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            constexpr int r = nr * (m + 1) / nm - nr * m / nm, wr = nw * (m + 1) / nm - nw * m / nm, l = nl * (m + 1) / nm - nl * m / nm;
-            if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
-            if constexpr (wr > 0) __builtin_amdgcn_sched_group_barrier(0x200, wr, 0);
-            if constexpr (l > 0) __builtin_amdgcn_sched_group_barrier(0x020, l, 0);
-        });
-    };
 
     // One K step: LDS stage S is multiplied; register set R (the next K step) moves into stage
     // S^1 and is refilled with the K step PD further on.  Fragment buffer 0 holds substep 0 on

@@ -278,7 +278,9 @@ DXH_API int dxh_dropout(int dtype, void *inout, int64_t n, float p, uint32_t see
  * output tiles and a long K is cut along K (DXH_TUNE_MATMUL_SPLITK) into partial products that
  * are added in a fixed order; their buffer (at most 256 MiB) belongs to the library, one per
  * stream, allocated on first need and released by dxh_stream_destroy.  On a stream under
- * graph capture the product is never cut. */
+ * graph capture no workspace is used (the product is not cut, and bf16/f16 operands with odd K
+ * or N take the element-wise kernel instead of padded copies): a recorded float matmul of such a
+ * shape can differ from the eager one in summation order, within the same error bound. */
 DXH_API int dxh_matmul(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m,
                        int64_t k, int64_t n, void *stream);
 

@@ -313,3 +313,20 @@ def test_matmul_half_rows_not_16_byte_aligned(dxh, dtype, tile):
         assert np.array_equal(H.to_float(dC.get(), dtype), want)
     finally:
         dx.check(dxh.dxh_tune(TILE_KNOB, 0))
+
+
+def test_matmul_int8_matrix_pipe_wraps_like_the_reference(dxh):
+    """int8 products large enough for the matrix-pipe kernel (int32 accumulate, low 8 bits
+    stored), full-range operands: the result must equal the exact integer product reduced modulo
+    2^8, which is what accumulating in int8 (the reference's arithmetic) gives.  Aligned and
+    ragged shapes, batches, a K long enough for the int32 accumulators to wrap as well."""
+    rng = np.random.default_rng(1234)
+    for batch, m, k, n in [(1, 512, 256, 512), (2, 300, 200, 520), (1, 1000, 77, 333), (8, 128, 64, 128), (1, 129, 1000, 1040),
+                           (1, 256, 140000, 512)]:
+        A = rng.integers(-128, 128, (batch, m, k), dtype=np.int8)
+        B = rng.integers(-128, 128, (batch, k, n), dtype=np.int8)
+        dA, dB, dC = Dev(A.reshape(-1)), Dev(B.reshape(-1)), Dev.empty(batch * m * n, np.int8)
+        dx.check(dxh.dxh_matmul(dx.I8, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+        # float64 BLAS matmul is exact here: |sum| <= 140000 * 2^14 < 2^53
+        want = np.matmul(A.astype(np.float64), B.astype(np.float64)).astype(np.int64).astype(np.int8)
+        assert np.array_equal(dC.get().reshape(batch, m, n), want), (batch, m, k, n)

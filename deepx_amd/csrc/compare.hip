@@ -51,21 +51,27 @@ template <int K, typename A> __device__ inline uint8_t cmp_one(A a, A b, float e
 }
 
 // SCALAR=true compares against `s`, otherwise against b[i].
+// Vectors per lane and trip: a comparison with a scalar has one load stream, and a single 16-byte
+// load per lane does not keep it busy (fp32 equalscalar, 64 / 256 MiB: 4.8 / 5.7 TB/s with one
+// vector per lane, 5.6 / 6.0 with four); with two load streams, and for 1-byte elements, one
+// vector per lane measured the same or better.
+template <typename T, bool SCALAR> constexpr int compare_unroll = (SCALAR && sizeof(T) > 1) ? 4 : 1;
 template <typename T, int V, int K, bool SCALAR, bool NTL>
 __device__ __forceinline__ void compare_body(const T *__restrict__ a, const T *__restrict__ b, const T s,
                                                           float eps, uint8_t *__restrict__ m, int64_t n) {
     using VT = vec_t<T, V>;
     using MT = vec_t<uint8_t, V>;
     using A = acc_t<T>;
+    constexpr int UC = compare_unroll<T, SCALAR>;
     const int64_t nv = n / V;
     const A sv = load_acc(s);
     const VT *va = reinterpret_cast<const VT *>(a);
     const VT *vb = reinterpret_cast<const VT *>(b);
     MT *vm = reinterpret_cast<MT *>(m);
-    tile_loop_c<kUnrollC>(nv, [&](int64_t i, auto full) {
-        VT x[kUnrollC], y[kUnrollC];
+    tile_loop_c<UC>(nv, [&](int64_t i, auto full) {
+        VT x[UC], y[UC];
 #pragma unroll
-        for (int u = 0; u < kUnrollC; ++u) {
+        for (int u = 0; u < UC; ++u) {
             int64_t j = i + u * kBlock;
             if (decltype(full)::value || j < nv) {
                 x[u] = ld_sel<NTL>(&va[j]);
@@ -73,7 +79,7 @@ __device__ __forceinline__ void compare_body(const T *__restrict__ a, const T *_
             }
         }
 #pragma unroll
-        for (int u = 0; u < kUnrollC; ++u) {
+        for (int u = 0; u < UC; ++u) {
             int64_t j = i + u * kBlock;
             if (decltype(full)::value || j < nv) {
                 MT r;
@@ -107,13 +113,14 @@ int launch_compare(const void *a, const void *b, dxh_scalar s, float eps, void *
     if (!aligned(a, sizeof(T)) || (!SCALAR && !aligned(b, sizeof(T)))) return DXH_ERR_ALIGN;
     constexpr int V = vec_len<T>;
     const T sv = SCALAR ? scalar_to<T>(s) : T{};
-    // a comparison reads 4..16 bytes per mask byte: a read-dominated stream
-    const int ntl = SCALAR ? nt_load_reduce((size_t)n * sizeof(T)) : nt_load_2r1w((size_t)n * (2 * sizeof(T) + 1));
+    // a comparison reads 1..16 bytes per mask byte, a read-dominated stream: nt loads from 16 MiB up
+    // (fp32 / bf16 equalscalar at 64 MiB: 4742 / 4764 GB/s with nt loads, 4658 / 3898 without)
+    const int ntl = SCALAR ? nt_load_forced((size_t)n * sizeof(T) > ((size_t)16 << 20)) : nt_load_2r1w((size_t)n * (2 * sizeof(T) + 1));
     if (aligned(a, kVecBytes) && (SCALAR || aligned(b, kVecBytes)) && aligned(m, V)) {
-        unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
+        unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * compare_unroll<T, SCALAR>, kBlocksPerCUC);
         compare_kernel<T, V, K, SCALAR><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, sv, eps, (uint8_t *)m, n, ntl);
     } else {
-        unsigned g = stream_grid(n, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
+        unsigned g = stream_grid(n, (int64_t)kBlock * compare_unroll<T, SCALAR>, kBlocksPerCUC);
         compare_kernel<T, 1, K, SCALAR><<<g, kBlock, 0, st>>>((const T *)a, (const T *)b, sv, eps, (uint8_t *)m, n, ntl);
     }
     return launch_status();
@@ -254,6 +261,10 @@ template <typename D, typename S> __device__ inline D cast_elem(S v) {
     }
 }
 
+// Vectors per lane and trip: a narrowing cast is read-dominated and wants several loads in flight
+// per lane (int32 -> int8 at 256 MiB: 5.1 TB/s with one vector per lane, 6.9 with four); a widening
+// or same-size one is write-dominated and measured 5-8 % faster with one.
+template <typename S, typename D> constexpr int cast_unroll = sizeof(D) < sizeof(S) ? 4 : 1;
 template <typename S, typename D, int V, bool NTS, bool NTL>
 __device__ __forceinline__ void cast_body(const S *__restrict__ a, D *__restrict__ c, int64_t n) {
     using VS = vec_t<S, V>;
@@ -261,15 +272,15 @@ __device__ __forceinline__ void cast_body(const S *__restrict__ a, D *__restrict
     const int64_t nv = n / V;
     const VS *va = reinterpret_cast<const VS *>(a);
     VD *vc = reinterpret_cast<VD *>(c);
-    tile_loop_c<kUnrollC>(nv, [&](int64_t i, auto full) {
-        VS x[kUnrollC];
+    tile_loop_c<cast_unroll<S, D>>(nv, [&](int64_t i, auto full) {
+        VS x[cast_unroll<S, D>];
 #pragma unroll
-        for (int u = 0; u < kUnrollC; ++u) {
+        for (int u = 0; u < cast_unroll<S, D>; ++u) {
             int64_t j = i + u * kBlock;
             if (decltype(full)::value || j < nv) x[u] = ld_sel<NTL>(&va[j]);
         }
 #pragma unroll
-        for (int u = 0; u < kUnrollC; ++u) {
+        for (int u = 0; u < cast_unroll<S, D>; ++u) {
             int64_t j = i + u * kBlock;
             if (decltype(full)::value || j < nv) {
                 VD r;
@@ -296,11 +307,11 @@ template <typename S, typename D> int launch_cast(const void *a, void *c, int64_
     constexpr int V = kVecBytes / W;  // the wider side moves 16 bytes per lane
     const int ntl = nt_load_1r1w((size_t)n * sizeof(S), (size_t)n * sizeof(D));
     if (aligned(a, V * sizeof(S)) && aligned(c, V * sizeof(D))) {
-        unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
+        unsigned g = stream_grid(n / V + 1, (int64_t)kBlock * cast_unroll<S, D>, kBlocksPerCUC);
         if (use_nt_store((size_t)n * sizeof(D))) cast_kernel<S, D, V, true><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n, ntl);
         else cast_kernel<S, D, V, false><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n, ntl);
     } else {
-        unsigned g = stream_grid(n, (int64_t)kBlock * kUnrollC, kBlocksPerCUC);
+        unsigned g = stream_grid(n, (int64_t)kBlock * cast_unroll<S, D>, kBlocksPerCUC);
         cast_kernel<S, D, 1, false><<<g, kBlock, 0, st>>>((const S *)a, (D *)c, n, ntl);
     }
     return launch_status();

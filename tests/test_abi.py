@@ -43,3 +43,33 @@ def test_argument_errors_need_no_gpu():
     assert L.dxh_reduce_workspace_bytes(dx.F32, dx.i32arr([8192, 8192]), 2, dx.i32arr([0]), 1, C.byref(n)) == 0 and n.value > 0
     assert L.dxh_reduce_workspace_bytes(dx.F32, dx.i32arr([8192, 8192]), 2, dx.i32arr([2]), 1, C.byref(n)) == -2
     assert L.dxh_matmul(dx.BOOL, None, None, None, 1, 2, 2, 2, None) == -1
+
+
+def test_tuning_knobs_validate_their_values():
+    """dxh_tune is host state only: every knob of the header accepts its documented range and
+    rejects values outside it (and unknown knobs) with DXH_ERR_ARG."""
+    L = dx.load()
+    text = open(os.path.join(ROOT, "include", "dxhip.h")).read()
+    knobs = {name: int(val) for name, val in re.findall(r"(DXH_TUNE_\w+)\s*=\s*(\d+)", text)}
+    assert sorted(knobs.values()) == list(range(len(knobs))), knobs  # dense numbering, no duplicates
+    good = {"DXH_TUNE_NT_STORE_BYTES": [0, 1 << 20], "DXH_TUNE_REDUCE_TARGET_BLOCKS": [256, 1024], "DXH_TUNE_REDUCE_COL_MIN_ROWS": [1, 16],
+            "DXH_TUNE_REDUCE_COL_MAX_LANES": [4, 32, 128, 256], "DXH_TUNE_MATMUL_TILE": [1, 5, 0], "DXH_TUNE_REDUCE_ROW_LOADS": [1, 4],
+            "DXH_TUNE_MATMUL_SPLITK": [1, 7, 1024, 0], "DXH_TUNE_NT_LOAD": [1, 2, 0]}
+    bad = {"DXH_TUNE_REDUCE_TARGET_BLOCKS": [0], "DXH_TUNE_REDUCE_COL_MIN_ROWS": [0], "DXH_TUNE_REDUCE_COL_MAX_LANES": [3, 512],
+           "DXH_TUNE_MATMUL_TILE": [-1, 6], "DXH_TUNE_REDUCE_ROW_LOADS": [0, 65], "DXH_TUNE_MATMUL_SPLITK": [-1, 1025], "DXH_TUNE_NT_LOAD": [-1, 3]}
+    assert set(good) == set(knobs), set(good) ^ set(knobs)
+    defaults = {"DXH_TUNE_NT_STORE_BYTES": 0, "DXH_TUNE_REDUCE_TARGET_BLOCKS": 1024, "DXH_TUNE_REDUCE_COL_MIN_ROWS": 16,
+                "DXH_TUNE_REDUCE_COL_MAX_LANES": 128, "DXH_TUNE_MATMUL_TILE": 0, "DXH_TUNE_REDUCE_ROW_LOADS": 4,
+                "DXH_TUNE_MATMUL_SPLITK": 0, "DXH_TUNE_NT_LOAD": 0}
+    try:
+        for name, values in good.items():
+            for v in values:
+                assert L.dxh_tune(knobs[name], v) == 0, (name, v)
+        for name, values in bad.items():
+            for v in values:
+                assert L.dxh_tune(knobs[name], v) == -2, (name, v)
+        assert L.dxh_tune(len(knobs), 0) == -2
+        assert L.dxh_tune(-1, 0) == -2
+    finally:
+        for name, v in defaults.items():
+            assert L.dxh_tune(knobs[name], v) == 0

@@ -6,6 +6,7 @@
 //   bf16 / f16   matmul_half.hip: MFMA v_mfma_f32_32x32x16_{bf16,f16}, fp32 accumulate, one RNE
 //                rounding of C.
 //   f32 / f64    matmul_fp.hip: MFMA v_mfma_f32_32x32x2_f32 / v_mfma_f64_16x16x4_f64.
+//   M <= 8       matmul_skinny.hip (floats): vector-ALU stream over B, K cut into slices.
 //   integers     here: LDS-tiled 64x64x16 multiply-add kernel, 4x4 outputs per lane; accumulate in
 //                the storage type (integers wrap).  int8 with at least 8 output tiles of 128x128:
 //                v_mfma_i32_32x32x16_i8, int32 accumulate, low 8 bits stored (the same value).
@@ -211,6 +212,10 @@ extern "C" int dxh_matmul(int dtype, const void *a, const void *b, void *c, int6
     }
     if (!a || !b) return DXH_ERR_ARG;
     if (!aligned(a, es) || !aligned(b, es) || !aligned(c, es)) return DXH_ERR_ALIGN;
+    if (m <= 8) {  // a few rows of A: a stream over B, not matrix-pipe work
+        const int rc = launch_matmul_skinny(dtype, a, b, c, batch, m, k, n, st);
+        if (rc != kNoSkinny) return rc;
+    }
     switch (dtype) {
     case DXH_BF16:
     case DXH_F16: return launch_matmul_half(dtype, a, b, c, batch, m, k, n, st);

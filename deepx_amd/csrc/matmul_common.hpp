@@ -153,7 +153,10 @@ int launch_splitk_reduce(const TA *ws, TO *out, int64_t batch, int64_t mn, int s
     return launch_status();
 }
 
-// entry points of the per-dtype translation units (matmul_half.hip, matmul_fp.hip)
+// entry points of the per-dtype translation units (matmul_half.hip, matmul_fp.hip) and of the
+// few-rows kernel (matmul_skinny.hip; kNoSkinny = not a shape for it)
+constexpr int kNoSkinny = -1002;  // not a DXH_ERR_* value
+int launch_matmul_skinny(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
 int launch_matmul_half(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
 int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
 int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);

@@ -457,7 +457,8 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
         // 64x64 tiles so that all CUs (and their vector caches) take part.
         const int64_t cus = compute_units();
         auto tiles = [&](int tm, int tn) { return batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn); };
-        if (tiles(256, 256) * 10 >= cus * 9) choice = 4;
+        if (m <= 64) choice = 5;  // one tile row: anything taller multiplies padding (bf16 [1,896]x[896,151936]: 53 vs 75 us)
+        else if (tiles(256, 256) * 10 >= cus * 9) choice = 4;
         else if (tiles(128, 128) * 2 >= cus * 3) choice = 1;
         else if (tiles(128, 64) * 2 >= cus) choice = 2;
         else choice = 5;

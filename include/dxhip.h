@@ -95,8 +95,13 @@ enum dxh_tune_knob {
     DXH_TUNE_MATMUL_SPLITK = 6,        /* slices along K of a float matmul: 0 = chosen per shape (few output tiles and a long
                                           K are cut so that every CU has work), 1 = never, n <= 1024 = n slices.  Slices are
                                           added in slice order, so results do not vary from run to run. */
-    DXH_TUNE_NT_LOAD = 7               /* non-temporal hint on the loads of elementwise / compare / reduce kernels:
+    DXH_TUNE_NT_LOAD = 7,              /* non-temporal hint on the loads of elementwise / compare / reduce kernels:
                                           0 = by op class and tensor size, 1 = always, 2 = never */
+    DXH_TUNE_SKINNY_PER_CU = 8,        /* matmul with at most 8 rows of A (streaming kernel): workgroups per CU that the
+                                          cut of K aims for (default 2) */
+    DXH_TUNE_SKINNY_MIN_ROWS = 9,      /* ... and the fewest rows of B per K slice (default 256, at least 8) */
+    DXH_TUNE_SKINNY_HALF = 10          /* 1 = that kernel also for bf16 / f16 (default 0: they stay on the matrix pipe,
+                                          which is as fast or faster for them) */
 };
 DXH_API int dxh_tune(int knob, int64_t value);
 DXH_API int dxh_device_count(int *count);

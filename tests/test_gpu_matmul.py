@@ -330,3 +330,42 @@ def test_matmul_int8_matrix_pipe_wraps_like_the_reference(dxh):
         # float64 BLAS matmul is exact here: |sum| <= 140000 * 2^14 < 2^53
         want = np.matmul(A.astype(np.float64), B.astype(np.float64)).astype(np.int64).astype(np.int8)
         assert np.array_equal(dC.get().reshape(batch, m, n), want), (batch, m, k, n)
+
+
+@pytest.mark.parametrize("dtype", [dx.BF16, dx.F16, dx.F32, dx.F64])
+def test_matmul_few_rows(dxh, dtype):
+    """At most 8 rows of A with K >= 256 take the streaming kernel (vector ALU, K in slices, fp32 /
+    fp64 sums; by default for fp32 and fp64 only, here forced for the 16-bit types too): every row-count template, batches, odd K, a K of several slices and sub-chunks, N
+    down to one vector; float64 numpy is the reference (same bars as the matrix-pipe kernels),
+    small-integer operands must be exact and a second run bit-identical."""
+    rng = np.random.default_rng(1100 + dtype)
+    rel = {dx.F32: 1e-5, dx.F64: 1e-13, dx.BF16: 1e-2, dx.F16: 1e-2}[dtype]
+    dx.check(dxh.dxh_tune(10, 1))  # DXH_TUNE_SKINNY_HALF: by default the kernel serves fp32 / fp64 only
+    try:
+        _few_rows_cases(dxh, dtype, rng, rel)
+    finally:
+        dx.check(dxh.dxh_tune(10, 0))
+
+
+def _few_rows_cases(dxh, dtype, rng, rel):
+    for batch, m, k, n in [(1, 1, 4096, 512), (2, 3, 1000, 264), (1, 8, 300, 8), (1, 5, 257, 1040), (1, 4, 70000, 64), (3, 2, 256, 4096),
+                           (1, 7, 2048, 4864), (1, 1, 896, 151936 // 8)]:
+        A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
+        B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
+        dA, dB, dC, dC2 = Dev(A), Dev(B), Dev.empty(batch * m * n, A.dtype), Dev.empty(batch * m * n, A.dtype)
+        dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+        dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC2.ptr, batch, m, k, n, None), "matmul")
+        first = dC.get()
+        assert np.array_equal(first, dC2.get()), "result varies between runs"
+        got = H.to_float(first, dtype).astype(np.float64).reshape(batch, m, n)
+        ref, mag = _ref_product(A, B, dtype, batch, m, k, n)
+        scale = np.sqrt(k) if dtype in (dx.F32, dx.F64) else 1.0
+        assert np.all(np.abs(got - ref) <= rel * scale * np.maximum(mag, 1e-300)), (dtype, batch, m, k, n)
+    m, k, n = 6, 1500, 136
+    Ai, Bi = rng.integers(-4, 5, (m, k)), rng.integers(-4, 5, (k, n))
+    A = H.to_storage(Ai.astype(np.float64).reshape(-1), dtype)
+    B = H.to_storage(Bi.astype(np.float64).reshape(-1), dtype)
+    dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, A.dtype)
+    dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+    want = H.to_float(H.to_storage((Ai @ Bi).astype(np.float64).reshape(-1), dtype), dtype)
+    assert np.array_equal(H.to_float(dC.get(), dtype), want)

@@ -153,6 +153,71 @@ int launch_splitk_reduce(const TA *ws, TO *out, int64_t batch, int64_t mn, int s
     return launch_status();
 }
 
+// ---- rows that are not 16-byte aligned (odd K or N, unaligned bases) ---------------------------
+// The matrix-pipe kernels want 16-byte rows.  Such a product runs on zero-padded copies instead: A
+// to [M][Kp], B to [Kp][Np] (Kp, Np the next multiples of 16 bytes), the kernel on those, and the
+// first N columns of its [M][Np] result copied out.  The three copies move each operand once more
+// through HBM, a fraction of what element-wise loads lose (bf16 2047x895x4863: 197 -> 56 us).
+// E: unsigned integer of the element size.  kNoSplit: not done (no workspace under graph
+// capture, operands over the workspace limit, tiny products), the caller takes its other path.
+constexpr int kNoSplit = -1001;  // not a DXH_ERR_* value
+// out[b][r][c] = (r < rows_in && c < cols_in) ? in[b][r][c] : 0, one 16-byte chunk of out per lane
+template <typename E>
+__global__ __launch_bounds__(kBlock) void pad_rows_kernel(const E *__restrict__ in, E *__restrict__ out, int64_t rows_in, int64_t cols_in,
+                                                          int64_t rows_out, int64_t chunks_out, int64_t total) {
+    constexpr int V = kVecBytes / (int)sizeof(E);
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t ch = i % chunks_out, r = (i / chunks_out) % rows_out, b = i / (chunks_out * rows_out);
+        const E *p = in + (b * rows_in + r) * cols_in + ch * V;
+        vec_t<E, V> x;
+#pragma unroll
+        for (int e = 0; e < V; ++e) x.v[e] = (r < rows_in && ch * V + e < cols_in) ? p[e] : (E)0;
+        *reinterpret_cast<vec_t<E, V> *>(out + i * V) = x;
+    }
+}
+// out[r][c] = in[r][c] for c < cols (rows of in hold chunks_in 16-byte chunks)
+template <typename E>
+__global__ __launch_bounds__(kBlock) void unpad_rows_kernel(const E *__restrict__ in, E *__restrict__ out, int64_t cols, int64_t chunks_in, int64_t total) {
+    constexpr int V = kVecBytes / (int)sizeof(E);
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t ch = i % chunks_in, r = i / chunks_in;
+        const vec_t<E, V> x = *reinterpret_cast<const vec_t<E, V> *>(in + i * V);
+        E *p = out + r * cols + ch * V;
+#pragma unroll
+        for (int e = 0; e < V; ++e)
+            if (ch * V + e < cols) p[e] = x.v[e];
+    }
+}
+inline unsigned copy_blocks(int64_t total) {
+    const int64_t blocks = (total + kBlock - 1) / kBlock;
+    return (unsigned)(blocks > 16384 ? 16384 : blocks);
+}
+// inner(a, b, c, k_padded, n_padded) launches the aligned product on the copies
+template <typename E, typename Inner>
+int launch_on_padded_copies(Inner inner, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    constexpr int V = kVecBytes / (int)sizeof(E);
+    const int64_t kp = (k + V - 1) / V * V, np = (n + V - 1) / V * V;
+    const int64_t a_elems = (batch * m * kp + V - 1) / V * V, b_elems = batch * kp * np, c_elems = batch * m * np;  // each part starts 16-byte aligned
+    const int64_t bytes = (a_elems + b_elems + c_elems) * (int64_t)sizeof(E);
+    if (bytes > kWorkspaceMaxBytes || m * n * k < (1 << 16) || stream_is_capturing(st)) return kNoSplit;
+    std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
+    E *ws = (E *)stream_workspace(st, kWorkspacePadded, (size_t)bytes);
+    if (!ws) return kNoSplit;
+    E *ap = ws, *bp = ap + a_elems, *cp = bp + b_elems;
+    int64_t total = batch * m * (kp / V);
+    const bool a_as_is = k == kp && ((uintptr_t)a % kVecBytes) == 0;  // only B and C have short rows
+    if (!a_as_is) pad_rows_kernel<E><<<copy_blocks(total), kBlock, 0, st>>>((const E *)a, ap, m, k, m, kp / V, total);
+    total = batch * kp * (np / V);
+    pad_rows_kernel<E><<<copy_blocks(total), kBlock, 0, st>>>((const E *)b, bp, k, n, kp, np / V, total);
+    int rc = launch_status();
+    if (rc != DXH_OK) return rc;
+    rc = inner(a_as_is ? a : (const void *)ap, (const void *)bp, (void *)cp, kp, np);
+    if (rc != DXH_OK) return rc;
+    total = batch * m * (np / V);
+    unpad_rows_kernel<E><<<copy_blocks(total), kBlock, 0, st>>>(cp, (E *)c, n, np / V, total);
+    return launch_status();
+}
+
 // entry points of the per-dtype translation units (matmul_half.hip, matmul_fp.hip) and of the
 // few-rows kernel (matmul_skinny.hip; kNoSkinny = not a shape for it)
 constexpr int kNoSkinny = -1002;  // not a DXH_ERR_* value

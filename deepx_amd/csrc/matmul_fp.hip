@@ -457,6 +457,11 @@ int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int6
         const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.5 : 0.0);
         return rounds * (3.0 + (double)k * 0.1183 * (double)(tm * tn) / (128.0 * 128.0) / eff);
     };
+    if (!vec && tuning().matmul_tile == 0) {  // odd K / N or unaligned bases: the vector path on zero-padded copies
+        const int rc = launch_on_padded_copies<uint32_t>(
+            [&](const void *pa, const void *pb, void *pc, int64_t pk, int64_t pn) { return launch_matmul_f32(pa, pb, pc, batch, m, pk, pn, st); }, a, b, c, batch, m, k, n, st);
+        if (rc != kNoSplit) return rc;
+    }
     const float *af = (const float *)a, *bf = (const float *)b;
     float *cf = (float *)c;
     int64_t choice = tuning().matmul_tile;
@@ -494,6 +499,11 @@ int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int6
         const double rounds = (double)full + (rem > cus ? 1.0 : rem > 0 ? 0.5 : 0.0);
         return rounds * (3.0 + (double)k * 0.1163 * (double)(tm * tn) / (128.0 * 64.0) / eff);
     };
+    if (!vec && tuning().matmul_tile == 0) {  // odd K / N or unaligned bases: the vector path on zero-padded copies
+        const int rc = launch_on_padded_copies<uint64_t>(
+            [&](const void *pa, const void *pb, void *pc, int64_t pk, int64_t pn) { return launch_matmul_f64(pa, pb, pc, batch, m, pk, pn, st); }, a, b, c, batch, m, k, n, st);
+        if (rc != kNoSplit) return rc;
+    }
     const double *af = (const double *)a, *bf = (const double *)b;
     double *cf = (double *)c;
     int64_t choice = tuning().matmul_tile;

@@ -363,7 +363,6 @@ int launch_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m,
 // Few output tiles and a long K: 64x64 tiles over K slices, fp32 partial tiles in the stream's
 // workspace, then one pass that adds the slices in order and rounds once.  Returns kNoSplit when the
 // product should not be cut (the caller then launches the ordinary way).
-constexpr int kNoSplit = -1001;  // not a DXH_ERR_* value
 template <typename T>
 int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     constexpr int TM = 64, TN = 64;
@@ -382,63 +381,13 @@ int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m
     return rc != DXH_OK ? rc : launch_splitk_reduce<float, T>(ws, (T *)c, batch, m * n, ks.splits, st);
 }
 
-// ---- rows that are not 16-byte aligned (odd K or N, unaligned bases) ---------------------------
-// The tile kernel needs 16-byte rows.  Such a product runs on zero-padded copies instead: A to
-// [M][K8], B to [K8][N8] (K8, N8 the next multiples of 8), the tile kernel on those, and the first
-// N columns of its [M][N8] result copied out.  The three copies move each operand once more
-// through HBM, a fraction of what the element-wise fallback kernel loses.
-// out[b][r][c] = (r < rows_in && c < cols_in) ? in[b][r][c] : 0, 8 columns (16 bytes out) per lane
-__global__ __launch_bounds__(kBlock) void pad_rows_kernel(const uint16_t *__restrict__ in, uint16_t *__restrict__ out, int64_t rows_in, int64_t cols_in,
-                                                          int64_t rows_out, int64_t chunks_out, int64_t total) {
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
-        const int64_t ch = i % chunks_out, r = (i / chunks_out) % rows_out, b = i / (chunks_out * rows_out);
-        const uint16_t *p = in + (b * rows_in + r) * cols_in + ch * 8;
-        vec_t<uint16_t, 8> x;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) x.v[e] = (r < rows_in && ch * 8 + e < cols_in) ? p[e] : (uint16_t)0;
-        *reinterpret_cast<vec_t<uint16_t, 8> *>(out + i * 8) = x;
-    }
-}
-// out[r][c] = in[r][c] for c < cols (in rows hold chunks_in * 8 columns)
-__global__ __launch_bounds__(kBlock) void unpad_rows_kernel(const uint16_t *__restrict__ in, uint16_t *__restrict__ out, int64_t cols, int64_t chunks_in, int64_t total) {
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
-        const int64_t ch = i % chunks_in, r = i / chunks_in;
-        const vec_t<uint16_t, 8> x = *reinterpret_cast<const vec_t<uint16_t, 8> *>(in + i * 8);
-        uint16_t *p = out + r * cols + ch * 8;
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-            if (ch * 8 + e < cols) p[e] = x.v[e];
-    }
-}
-inline unsigned copy_blocks(int64_t total) {
-    const int64_t blocks = (total + kBlock - 1) / kBlock;
-    return (unsigned)(blocks > 16384 ? 16384 : blocks);
-}
-
+// rows that are not 16-byte aligned (odd K or N, unaligned bases): the tile kernel on zero-padded
+// copies, see launch_on_padded_copies
 template <typename T> int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
-
 template <typename T>
 int launch_padded(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    const int64_t k8 = (k + 7) / 8 * 8, n8 = (n + 7) / 8 * 8;
-    const int64_t a_elems = (batch * m * k8 + 7) / 8 * 8, b_elems = batch * k8 * n8, c_elems = batch * m * n8;  // each part starts 16-byte aligned
-    const int64_t bytes = (a_elems + b_elems + c_elems) * 2;
-    if (bytes > kWorkspaceMaxBytes || m * n * k < (1 << 16) || stream_is_capturing(st)) return kNoSplit;
-    std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
-    uint16_t *ws = (uint16_t *)stream_workspace(st, kWorkspacePadded, (size_t)bytes);
-    if (!ws) return kNoSplit;
-    uint16_t *ap = ws, *bp = ap + a_elems, *cp = bp + b_elems;
-    int64_t total = batch * m * (k8 / 8);
-    const bool a_as_is = k == k8 && aligned(a, kVecBytes);  // only B and C have short rows
-    if (!a_as_is) pad_rows_kernel<<<copy_blocks(total), kBlock, 0, st>>>((const uint16_t *)a, ap, m, k, m, k8 / 8, total);
-    total = batch * k8 * (n8 / 8);
-    pad_rows_kernel<<<copy_blocks(total), kBlock, 0, st>>>((const uint16_t *)b, bp, k, n, k8, n8 / 8, total);
-    int rc = launch_status();
-    if (rc != DXH_OK) return rc;
-    rc = launch_mfma<T>(a_as_is ? a : ap, bp, cp, batch, m, k8, n8, st);
-    if (rc != DXH_OK) return rc;
-    total = batch * m * (n8 / 8);
-    unpad_rows_kernel<<<copy_blocks(total), kBlock, 0, st>>>(cp, (uint16_t *)c, n, n8 / 8, total);
-    return launch_status();
+    return launch_on_padded_copies<uint16_t>(
+        [&](const void *pa, const void *pb, void *pc, int64_t pk, int64_t pn) { return launch_mfma<T>(pa, pb, pc, batch, m, pk, pn, st); }, a, b, c, batch, m, k, n, st);
 }
 
 template <typename T>

@@ -96,7 +96,7 @@ inline int compute_units() {
 // only when the uncut K loop is long: K >= min_k, slices of at least min_k / 4.
 struct KSplit { int splits, ksub; };
 constexpr int kWorkspaceSplitK = 0, kWorkspacePadded = 1, kWorkspaceKinds = 2;
-constexpr int64_t kWorkspaceMaxBytes = (int64_t)1 << 28;
+constexpr int64_t kWorkspaceMaxBytes = (int64_t)1 << 30;  // 1 GiB of 288: padded copies of a [2048,768]x[768,50257] bf16 product need 283 MB
 void *stream_workspace(hipStream_t st, int kind, size_t bytes);  // nullptr when the allocation fails
 // Held from the workspace request to the last launch that uses it: two host threads that launch on
 // one stream must not interleave their (fill workspace, consume workspace) launch pairs.

@@ -281,7 +281,7 @@ DXH_API int dxh_dropout(int dtype, void *inout, int64_t n, float p, uint32_t see
  * the leading dims.  f16/bf16: MFMA with fp32 accumulate, one RNE rounding of the
  * result; f32/f64 accumulate in their own type; integers wrap.  A float product with few
  * output tiles and a long K is cut along K (DXH_TUNE_MATMUL_SPLITK) into partial products that
- * are added in a fixed order; their buffer (at most 256 MiB) belongs to the library, one per
+ * are added in a fixed order; their buffer (at most 1 GiB) belongs to the library, one per
  * stream, allocated on first need and released by dxh_stream_destroy.  On a stream under
  * graph capture no workspace is used (the product is not cut, and bf16/f16 operands with odd K
  * or N take the element-wise kernel instead of padded copies): a recorded float matmul of such a

@@ -145,9 +145,14 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t *p) {
 constexpr int part_first(int count, int part) { return count * part / 4; }
 constexpr int part_count(int count, int part) { return count * (part + 1) / 4 - count * part / 4; }
 
-template <typename T, int TM, int TN, int PD, bool KTAIL, bool SPLIT>
+template <typename T, int TM, int TN, int PD, bool KTAIL, int MODE>
 __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul_mfma_tile_kernel(
-    const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, float *__restrict__ partial, int M, int lda, int N, TileMap map, KSplit ks) {
+    const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, float *__restrict__ partial, int M, int lda, int N, TileMap map, KSplit ks,
+    int ldc, int n_store) {
+    // MODE 0: C[M][N] in 16-byte row pieces.  1 (SPLIT): fp32 partial tile of a K slice.  2 (EDGE): C has
+    // its own pitch ldc and n_store <= N columns (B was zero-padded to N columns): rows of C are not
+    // 16-byte aligned, so the tile is stored element by element.
+    constexpr bool SPLIT = MODE == 1, EDGE = MODE == 2;
     static_assert(TM % 64 == 0 && (TN == 64 || TN == 128 || TN == 256), "B rows must split evenly over the 256 lanes");
     constexpr int FM = TM / 64, FN = TN / 64;      // 32x32 MFMA tiles per wave along m and n
     constexpr int A_LD = TM / 32, B_LD = TN / 32;  // 16-byte global loads per lane per K step
@@ -338,25 +343,39 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
         });
     });
     __syncthreads();
-    uint16_t *Cr = reinterpret_cast<uint16_t *>(C) + (int64_t)batch * M * N;
+    uint16_t *Cr = reinterpret_cast<uint16_t *>(C) + (int64_t)batch * M * (EDGE ? ldc : N);
+    if constexpr (EDGE) {
+        // consecutive lanes along a row, one element each: every store instruction writes runs of
+        // contiguous bytes whatever the alignment of the row
+#pragma unroll 8
+        for (int i = 0; i < TM * TN / kBlock; ++i) {
+            const int c = t + i * kBlock, row = c / TN, col = c % TN;
+            const int gm = m0 + row, gn = n0 + col;
+            if (gm < M && gn < n_store) Cr[(int64_t)gm * ldc + gn] = Cs[row * LDC + col];
+        }
+    } else {
 #pragma unroll
-    for (int i = 0; i < TM * CB / kBlock; ++i) {
-        const int c = t + i * kBlock, row = c / CB, ch = c % CB;
-        const int gm = m0 + row, gn = n0 + ch * 8;
-        if (gm < M && gn < N)  // N % 8 == 0: a chunk is either fully inside or fully outside
-            st_nt(reinterpret_cast<uint4 *>(Cr + (int64_t)gm * N + gn), *reinterpret_cast<const uint4 *>(Cs + row * LDC + ch * 8));
+        for (int i = 0; i < TM * CB / kBlock; ++i) {
+            const int c = t + i * kBlock, row = c / CB, ch = c % CB;
+            const int gm = m0 + row, gn = n0 + ch * 8;
+            if (gm < M && gn < N)  // N % 8 == 0: a chunk is either fully inside or fully outside
+                st_nt(reinterpret_cast<uint4 *>(Cr + (int64_t)gm * N + gn), *reinterpret_cast<const uint4 *>(Cs + row * LDC + ch * 8));
+        }
     }
 }
 
+// ldc < 0: C is [M][N] and 16-byte aligned.  ldc >= 0 (needs K % 64 == 0): C has pitch ldc and ldc columns.
 template <typename T, int TM, int TN, int PD>
-int launch_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+int launch_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st) {
     TileMap map;
     if (!make_tile_map(batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
     const KSplit one{1, (int)k};
-    if (k % PK == 0)
-        matmul_mfma_tile_kernel<T, TM, TN, PD, false, false><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one);
+    if (ldc >= 0)
+        matmul_mfma_tile_kernel<T, TM, TN, PD, false, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one, (int)ldc, (int)ldc);
+    else if (k % PK == 0)
+        matmul_mfma_tile_kernel<T, TM, TN, PD, false, 0><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one, (int)n, (int)n);
     else
-        matmul_mfma_tile_kernel<T, TM, TN, PD, true, false><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one);
+        matmul_mfma_tile_kernel<T, TM, TN, PD, true, 0><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one, (int)n, (int)n);
     return launch_status();
 }
 
@@ -374,28 +393,47 @@ int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m
     float *ws = (float *)stream_workspace(st, kWorkspaceSplitK, (size_t)(partial * ks.splits));
     if (!ws) return kNoSplit;
     if (k % PK == 0)
-        matmul_mfma_tile_kernel<T, TM, TN, 1, false, true><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks);
+        matmul_mfma_tile_kernel<T, TM, TN, 1, false, 1><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
     else
-        matmul_mfma_tile_kernel<T, TM, TN, 1, true, true><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks);
+        matmul_mfma_tile_kernel<T, TM, TN, 1, true, 1><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
     const int rc = launch_status();
     return rc != DXH_OK ? rc : launch_splitk_reduce<float, T>(ws, (T *)c, batch, m * n, ks.splits, st);
 }
 
-// rows that are not 16-byte aligned (odd K or N, unaligned bases): the tile kernel on zero-padded
-// copies, see launch_on_padded_copies
-template <typename T> int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
+// Rows that are not 16-byte aligned (odd K or N, unaligned bases): A and B are copied, zero-padded
+// to K64 (next multiple of 64) and N8 columns, into the stream's workspace, the tile kernel runs on
+// the copies and stores C directly at its own pitch, element by element (EDGE).  Returns kNoSplit
+// when that is not possible (graph capture, operands over the workspace limit, tiny products).
+template <typename T> int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, int64_t ldc = -1);
 template <typename T>
 int launch_padded(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    return launch_on_padded_copies<uint16_t>(
-        [&](const void *pa, const void *pb, void *pc, int64_t pk, int64_t pn) { return launch_mfma<T>(pa, pb, pc, batch, m, pk, pn, st); }, a, b, c, batch, m, k, n, st);
+    const int64_t kp = (k + PK - 1) / PK * PK, np = (n + 7) / 8 * 8;
+    const bool a_as_is = k == kp && aligned(a, kVecBytes);
+    const int64_t a_elems = a_as_is ? 0 : (batch * m * kp + 7) / 8 * 8, b_elems = batch * kp * np;
+    const int64_t bytes = (a_elems + b_elems) * 2;
+    if (bytes > kWorkspaceMaxBytes || m * n * k < (1 << 16) || kp > (1 << 22) || np > (1 << 24) || stream_is_capturing(st)) return kNoSplit;
+    std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
+    uint16_t *ws = (uint16_t *)stream_workspace(st, kWorkspacePadded, (size_t)bytes);
+    if (!ws) return kNoSplit;
+    uint16_t *ap = ws, *bp = ws + a_elems;
+    if (!a_as_is) {
+        const int64_t total = batch * m * (kp / 8);
+        pad_rows_kernel<uint16_t><<<copy_blocks(total), kBlock, 0, st>>>((const uint16_t *)a, ap, m, k, m, kp / 8, total);
+    }
+    const int64_t total = batch * kp * (np / 8);
+    pad_rows_kernel<uint16_t><<<copy_blocks(total), kBlock, 0, st>>>((const uint16_t *)b, bp, k, n, kp, np / 8, total);
+    const int rc = launch_status();
+    return rc != DXH_OK ? rc : launch_mfma<T>(a_as_is ? a : (const void *)ap, bp, c, batch, m, kp, np, st, n);
 }
 
+// ldc >= 0: called by launch_padded on its copies; C then has ldc columns at pitch ldc
 template <typename T>
-int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    const bool fast = k % 8 == 0 && n % 8 == 0 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes) &&
+int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, int64_t ldc) {
+    const bool fast = k % 8 == 0 && n % 8 == 0 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && (ldc >= 0 || aligned(c, kVecBytes)) &&
                       k <= (1 << 22) && n <= (1 << 24);
     int64_t choice = tuning().matmul_tile;
-    if (fast && (choice == 0 || choice == 5)) {
+    if (ldc >= 0 && (!fast || k % PK != 0)) return DXH_ERR_ALIGN;  // launch_padded hands over aligned copies only
+    if (fast && ldc < 0 && (choice == 0 || choice == 5)) {
         const int rc = launch_split<T>(a, b, c, batch, m, k, n, st);
         if (rc != kNoSplit) return rc;
     }
@@ -414,11 +452,11 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
     }
     if (fast) {
         switch (choice) {
-        case 2: return launch_tile<T, 128, 64, 1>(a, b, c, batch, m, k, n, st);
-        case 3: return launch_tile<T, 64, 128, 1>(a, b, c, batch, m, k, n, st);
-        case 4: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, st);
-        case 5: return launch_tile<T, 64, 64, 1>(a, b, c, batch, m, k, n, st);
-        default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, st);
+        case 2: return launch_tile<T, 128, 64, 1>(a, b, c, batch, m, k, n, ldc, st);
+        case 3: return launch_tile<T, 64, 128, 1>(a, b, c, batch, m, k, n, ldc, st);
+        case 4: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st);
+        case 5: return launch_tile<T, 64, 64, 1>(a, b, c, batch, m, k, n, ldc, st);
+        default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, ldc, st);
         }
     }
     if (!fast && tuning().matmul_tile == 0 && k <= (1 << 22) && n <= (1 << 24)) {

@@ -127,8 +127,16 @@ struct Tuning {
     int64_t skinny_per_cu = 2;                    // DXH_TUNE_SKINNY_PER_CU
     int64_t skinny_min_rows = 256;                // DXH_TUNE_SKINNY_MIN_ROWS
     int64_t skinny_half = 0;                      // DXH_TUNE_SKINNY_HALF
+    int64_t reduce_fused_finish = 1;              // DXH_TUNE_REDUCE_FUSED_FINISH
 };
 Tuning &tuning();  // runtime.hip
+
+inline bool stream_is_capturing(hipStream_t st) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess) { (void)hipGetLastError(); return true; }  // unknown: assume the worst
+    return cap != hipStreamCaptureStatusNone;
+}
+void reduce_stream_release(hipStream_t st);  // reduce.hip: gives back the stream's slice of finish counters
 
 // Whether the loads of a streaming kernel carry the nt hint.  Measured on MI355X with buffers
 // rotated through 768 MB (fp32, GB/s with nt / without):
@@ -152,6 +160,10 @@ inline int stream_policy_2r1w(size_t total_bytes) {
     return total_bytes <= ((size_t)512 << 20) ? 2 : 1;
 }
 inline bool nt_load_reduce(size_t in_bytes) { return nt_load_forced(in_bytes > ((size_t)128 << 20)); }
+// Strided-axis stage: its rows are a pitch apart, and nt loads won at every size tried (fp32 [R,8192],
+// nt / plain GB/s: 32 MiB 3174/3067, 128 MiB 5520/5270, 256 MiB 6190/5894; bf16 [8192,8192] 4574/2964,
+// bf16 [64,512,2048] axis 1 5794/3239) except within noise at 7 MiB.
+inline bool nt_load_reduce_col(size_t in_bytes) { return nt_load_forced(in_bytes >= ((size_t)8 << 20)); }
 inline bool use_nt_store(size_t out_bytes) { return (int64_t)out_bytes > tuning().nt_store_bytes; }
 template <bool NT, typename VT> __device__ inline void st_sel(VT *p, const VT &v) {
     if constexpr (NT) st_nt(p, v); else *p = v;

@@ -102,11 +102,6 @@ void *stream_workspace(hipStream_t st, int kind, size_t bytes);  // nullptr when
 // one stream must not interleave their (fill workspace, consume workspace) launch pairs.
 std::recursive_mutex &workspace_launch_mutex();
 void stream_workspace_release(hipStream_t st);
-inline bool stream_is_capturing(hipStream_t st) {
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &cap) != hipSuccess) { (void)hipGetLastError(); return true; }  // unknown: assume the worst
-    return cap != hipStreamCaptureStatusNone;
-}
 inline KSplit choose_ksplit(int64_t tiles, int64_t k, int kstep, int64_t min_k, int64_t partial_bytes, hipStream_t st) {
     KSplit r{1, (int)k};
     const int64_t cus = compute_units(), ksteps = (k + kstep - 1) / kstep, knob = tuning().matmul_splitk;

@@ -16,10 +16,16 @@
 //
 // When a stage has too few workgroups to fill 256 CUs, R is split into S chunks whose
 // partials ([pre, S, post], accumulate type) go to the caller's workspace and are reduced
-// by one more stage; results are deterministic (no atomics).  Both stage kinds are
-// HBM-bound: algorithmic bytes = input once + output once.
+// by one more stage; results are deterministic (no atomic accumulation).  A split col
+// stage over the caller's input normally finishes inside the same launch: every workgroup
+// stores its partial tile and counts itself in on the tile's counter, and the one that
+// arrives last adds the S partials in a fixed order (reduce_col_fused_kernel; the counters
+// live in a file-scope device array and return to zero, see finish_counters).  Both stage
+// kinds are HBM-bound: algorithmic bytes = input once + output once.
 #include "common.hpp"
 #include <limits>
+#include <map>
+#include <mutex>
 #include <vector>
 
 namespace dxh {
@@ -158,7 +164,9 @@ __global__ __launch_bounds__(kBlock) void reduce_row_kernel(const Tin *__restric
 // ---- col stage ---------------------------------------------------------------------------
 // in [pre, R, post] -> out [pre, S, post].  Workgroup = TX column-lanes x TY row-lanes
 // (TX*TY == 256); a column-lane owns V adjacent columns.  Linear block id -> (p, s, ctile).
-template <int K, typename Tin, typename Tout, typename TS, int V, bool NTL>
+// COH: the partial tile is written through to memory (device-scope stores), for a reader in another
+// workgroup of the same launch.
+template <int K, typename Tin, typename Tout, typename TS, int V, bool NTL, bool COH = false>
 __device__ __forceinline__ void reduce_col_body(racc_t<TS> *lds, const Tin *__restrict__ in, Tout *__restrict__ out,
                                                              int64_t pre, int64_t R, int64_t post, int S, int64_t chunk,
                                                              int TX, int ctiles) {
@@ -226,7 +234,10 @@ __device__ __forceinline__ void reduce_col_body(racc_t<TS> *lds, const Tin *__re
     if (ty == 0 && active) {
         Tout *o = out + (p * S + s) * post + cv * V;
 #pragma unroll
-        for (int k = 0; k < V; ++k) o[k] = rstore<Tout, A>(lds[(k * TY) * TX + tx]);
+        for (int k = 0; k < V; ++k) {
+            if constexpr (COH) __hip_atomic_store(o + k, rstore<Tout, A>(lds[(k * TY) * TX + tx]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else o[k] = rstore<Tout, A>(lds[(k * TY) * TX + tx]);
+        }
     }
 }
 // ntl: loads carry the nt hint (chosen per launch, see nt_load_reduce in common.hpp)
@@ -236,6 +247,146 @@ __global__ __launch_bounds__(kBlock) void reduce_col_kernel(const Tin *__restric
     __shared__ A lds[kBlock * V];
     if (ntl) reduce_col_body<K, Tin, Tout, TS, V, true>(lds, in, out, pre, R, post, S, chunk, TX, ctiles);
     else reduce_col_body<K, Tin, Tout, TS, V, false>(lds, in, out, pre, R, post, S, chunk, TX, ctiles);
+}
+
+// Split col stage and its second pass in one launch.  `part` [pre, S, post] takes the partial
+// tiles as before; `cnt[p * ctiles + ct]` counts the workgroups of output tile (p, ct) that have
+// stored theirs.  The partials are stored and loaded with device-scope accesses (written through
+// to memory, read past the reader's own L2: the workgroups of a tile run on different XCDs), and
+// the barrier before the count waits until this workgroup's stores have completed.  A release /
+// acquire pair on the counter would do the same by writing back and invalidating whole L2s once
+// per workgroup, which cost 30 us of 45 on [8192,8192].  The workgroup that arrives last adds the
+// partials in an order fixed by the launch shape, so the result does not depend on which one it
+// was, and puts the counter back to zero for the next launch.
+template <int K, typename Tin, typename Tfin, typename TS, int V>
+__global__ __launch_bounds__(kBlock) void reduce_col_fused_kernel(const Tin *__restrict__ in, racc_t<TS> *part, Tfin *__restrict__ fout, unsigned *cnt,
+                                                                    int64_t pre, int64_t R, int64_t post, int S, int64_t chunk, int TX, int ctiles, int ntl) {
+    using A = racc_t<TS>;
+    __shared__ A lds[kBlock * V];
+    __shared__ int is_last;
+    if (ntl) reduce_col_body<K, Tin, A, TS, V, true, true>(lds, in, part, pre, R, post, S, chunk, TX, ctiles);
+    else reduce_col_body<K, Tin, A, TS, V, false, true>(lds, in, part, pre, R, post, S, chunk, TX, ctiles);
+    __syncthreads();  // every store of this workgroup has been acknowledged (the barrier waits on vmcnt)
+    const int ct = (int)(blockIdx.x % ctiles);
+    const int64_t p = blockIdx.x / ctiles / S;
+    if (threadIdx.x == 0) {
+        unsigned *c = cnt + p * ctiles + ct;
+        const unsigned old = __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int last = old == (unsigned)(S - 1);
+        if (last) __hip_atomic_store(c, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = last;
+    }
+    __syncthreads();
+    if (!is_last) return;
+    // The S partial tiles are folded like S rows of a col stage: row-lane ty takes slices ty, ty + TY,
+    // ... (independent loads, a few in flight), then the same LDS tree across the row-lanes.
+    const int TY = kBlock / TX, tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+    const int64_t cv = (int64_t)ct * TX + tx;
+    const bool active = cv < post / V;
+    A acc[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) acc[k] = rinit<K, A, TS>();
+    if (active) {
+        const A *q = part + p * S * post + cv * V;
+        auto ld = [&](int s, int k) __attribute__((always_inline)) { return __hip_atomic_load(q + (int64_t)s * post + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+        int s = ty;
+        for (; s + 3 * TY < S; s += 4 * TY) {
+            A x[4][V];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int k = 0; k < V; ++k) x[u][k] = ld(s + u * TY, k);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int k = 0; k < V; ++k) acc[k] = rop<K, A>(acc[k], x[u][k]);
+        }
+        for (; s < S; s += TY) {
+#pragma unroll
+            for (int k = 0; k < V; ++k) acc[k] = rop<K, A>(acc[k], ld(s, k));
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < V; ++k) lds[(k * TY + ty) * TX + tx] = acc[k];
+    __syncthreads();
+    for (int h = TY >> 1; h > 0; h >>= 1) {
+        if (ty < h) {
+#pragma unroll
+            for (int k = 0; k < V; ++k)
+                lds[(k * TY + ty) * TX + tx] = rop<K, A>(lds[(k * TY + ty) * TX + tx], lds[(k * TY + ty + h) * TX + tx]);
+        }
+        __syncthreads();
+    }
+    if (ty == 0 && active) {
+        Tfin *o = fout + p * post + cv * V;
+#pragma unroll
+        for (int k = 0; k < V; ++k) o[k] = rstore<Tfin, A>(lds[(k * TY) * TX + tx]);
+    }
+}
+
+// Counters of reduce_col_fused_kernel: zero at module load, and every launch leaves them zero.
+// Kernels of one stream run in order, so an eager stream owns one slice for as long as it is
+// known here (dxh_stream_destroy gives it back).  A launch recorded under stream capture may
+// later replay on any stream next to eager work, so it takes counters of its own from the
+// second half of the array, never handed out twice; when either half is used up the caller
+// falls back to two launches.
+constexpr int kFinishSlice = 1024, kFinishSlices = 32, kFinishCounters = 2 * kFinishSlice * kFinishSlices;
+static __device__ __align__(256) unsigned g_finish_counters[kFinishCounters];
+namespace {
+struct FinishState {
+    unsigned *base = nullptr;
+    bool resolved = false;
+    std::map<hipStream_t, int> slice;
+    std::vector<int> free_slices;
+    int slices_used = 0;
+    int64_t capture_next = (int64_t)kFinishSlice * kFinishSlices;
+};
+std::mutex g_finish_mutex;
+std::map<int, FinishState> g_finish;  // by device
+}  // namespace
+
+unsigned *finish_counters(hipStream_t st, int64_t need) {
+    if (need > kFinishSlice || !tuning().reduce_fused_finish) return nullptr;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    const bool capturing = stream_is_capturing(st);
+    std::lock_guard<std::mutex> lock(g_finish_mutex);
+    FinishState &f = g_finish[dev];
+    if (!f.resolved) {
+        if (capturing) return nullptr;  // nothing but launches while a capture is open
+        f.resolved = true;
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_finish_counters)) != hipSuccess) { (void)hipGetLastError(); ptr = nullptr; }
+        f.base = (unsigned *)ptr;
+    }
+    if (!f.base) return nullptr;
+    if (capturing) {
+        if (f.capture_next + need > kFinishCounters) return nullptr;
+        unsigned *r = f.base + f.capture_next;
+        f.capture_next += need;
+        return r;
+    }
+    auto it = f.slice.find(st);
+    if (it == f.slice.end()) {
+        int idx;
+        if (!f.free_slices.empty()) { idx = f.free_slices.back(); f.free_slices.pop_back(); }
+        else if (f.slices_used < kFinishSlices) idx = f.slices_used++;
+        else return nullptr;
+        it = f.slice.emplace(st, idx).first;
+    }
+    return f.base + (int64_t)it->second * kFinishSlice;
+}
+
+void reduce_stream_release(hipStream_t st) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return; }
+    std::lock_guard<std::mutex> lock(g_finish_mutex);
+    auto d = g_finish.find(dev);
+    if (d == g_finish.end()) return;
+    auto it = d->second.slice.find(st);
+    if (it == d->second.slice.end()) return;
+    d->second.free_slices.push_back(it->second);
+    d->second.slice.erase(it);
 }
 
 // fill `n` outputs with the identity (a reduced axis of size 0), or copy (nothing to reduce)
@@ -409,7 +560,8 @@ inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, cons
 template <int K, typename Tin, typename Tout, typename TS>
 int launch_stage(const Stage &st, const void *in, void *out, hipStream_t stream) {
     constexpr int VF = kVecBytes / (int)sizeof(Tin);
-    const int ntl = nt_load_reduce((size_t)(st.pre * st.R * st.post) * sizeof(Tin));
+    const size_t in_bytes = (size_t)(st.pre * st.R * st.post) * sizeof(Tin);
+    const int ntl = st.row ? nt_load_reduce(in_bytes) : nt_load_reduce_col(in_bytes);
     if (st.row) {
         const int rows_per_block = kBlock / st.G;
         int64_t gx = (st.pre + rows_per_block - 1) / rows_per_block;
@@ -436,6 +588,23 @@ int launch_stage(const Stage &st, const void *in, void *out, hipStream_t stream)
     return launch_status();
 }
 
+// Split col stage `st` over the caller's input together with its second pass `s2`: one launch
+// when counters are to be had.  Returns kNotFused when the pair has to run as two launches.
+constexpr int kNotFused = -1003;
+template <int K, typename Tfin, typename TS>
+int launch_fused_col(const Stage &st, const void *in, void *part, void *fout, hipStream_t stream) {
+    using A = racc_t<TS>;
+    constexpr int VF = kVecBytes / (int)sizeof(TS);
+    if (st.V != VF || !aligned(in, kVecBytes)) return kNotFused;
+    const int64_t gx = st.pre * st.S * st.ctiles;
+    if (gx > 0x7fffffff) return kNotFused;
+    unsigned *cnt = finish_counters(stream, st.pre * st.ctiles);
+    if (!cnt) return kNotFused;
+    const int ntl = nt_load_reduce_col((size_t)(st.pre * st.R * st.post) * sizeof(TS));
+    reduce_col_fused_kernel<K, TS, Tfin, TS, VF><<<(unsigned)gx, kBlock, 0, stream>>>((const TS *)in, (A *)part, (Tfin *)fout, cnt, st.pre, st.R, st.post, st.S, st.chunk, st.TX, st.ctiles, ntl);
+    return launch_status();
+}
+
 template <int K, typename TS>
 int reduce_typed(const void *in, const int32_t *shape, int ndim, const int32_t *dims, int ndims, void *out,
                  void *workspace, size_t workspace_bytes, hipStream_t stream) {
@@ -458,8 +627,20 @@ int reduce_typed(const void *in, const int32_t *shape, int ndim, const int32_t *
     }
     if (pl.ws_bytes > 0 && (!workspace || workspace_bytes < pl.ws_bytes || !aligned(workspace, 256))) return DXH_ERR_WORKSPACE;
     const void *cur = in;
-    for (const Stage &st : pl.stages) {
+    for (size_t i = 0; i < pl.stages.size(); ++i) {
+        const Stage &st = pl.stages[i];
         void *dst = st.out_is_acc ? (void *)((char *)workspace + st.out_off) : out;
+        if (!st.row && st.S > 1 && !st.in_is_acc && i + 1 < pl.stages.size()) {
+            const Stage &s2 = pl.stages[i + 1];  // the pass over this stage's S partials
+            void *fin = s2.out_is_acc ? (void *)((char *)workspace + s2.out_off) : out;
+            rc = s2.out_is_acc ? launch_fused_col<K, A, TS>(st, cur, dst, fin, stream) : launch_fused_col<K, TS, TS>(st, cur, dst, fin, stream);
+            if (rc != kNotFused) {
+                if (rc != DXH_OK) return rc;
+                cur = fin;
+                ++i;
+                continue;
+            }
+        }
         if (!st.in_is_acc && !st.out_is_acc) rc = launch_stage<K, TS, TS, TS>(st, cur, dst, stream);
         else if (!st.in_is_acc && st.out_is_acc) rc = launch_stage<K, TS, A, TS>(st, cur, dst, stream);
         else if (st.in_is_acc && st.out_is_acc) rc = launch_stage<K, A, A, TS>(st, cur, dst, stream);

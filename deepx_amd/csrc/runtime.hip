@@ -77,6 +77,7 @@ int dxh_tune(int knob, int64_t value) {
     case DXH_TUNE_SKINNY_PER_CU: if (value < 1 || value > 64) return DXH_ERR_ARG; t.skinny_per_cu = value; return DXH_OK;
     case DXH_TUNE_SKINNY_MIN_ROWS: if (value < 8) return DXH_ERR_ARG; t.skinny_min_rows = value; return DXH_OK;
     case DXH_TUNE_SKINNY_HALF: if (value < 0 || value > 1) return DXH_ERR_ARG; t.skinny_half = value; return DXH_OK;
+    case DXH_TUNE_REDUCE_FUSED_FINISH: if (value < 0 || value > 1) return DXH_ERR_ARG; t.reduce_fused_finish = value; return DXH_OK;
     default: return DXH_ERR_ARG;
     }
 }
@@ -152,6 +153,7 @@ int dxh_stream_create(void **stream) {
 int dxh_stream_destroy(void *stream) {
     if (!stream) return DXH_OK;
     dxh::stream_workspace_release(as_stream(stream));
+    dxh::reduce_stream_release(as_stream(stream));
     return (int)hipStreamDestroy(as_stream(stream));
 }
 int dxh_stream_sync(void *stream) { return (int)hipStreamSynchronize(as_stream(stream)); }

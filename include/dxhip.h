@@ -100,8 +100,13 @@ enum dxh_tune_knob {
     DXH_TUNE_SKINNY_PER_CU = 8,        /* matmul with at most 8 rows of A (streaming kernel): workgroups per CU that the
                                           cut of K aims for (default 2) */
     DXH_TUNE_SKINNY_MIN_ROWS = 9,      /* ... and the fewest rows of B per K slice (default 256, at least 8) */
-    DXH_TUNE_SKINNY_HALF = 10          /* 1 = that kernel also for bf16 / f16 (default 0: they stay on the matrix pipe,
+    DXH_TUNE_SKINNY_HALF = 10,         /* 1 = that kernel also for bf16 / f16 (default 0: they stay on the matrix pipe,
                                           which is as fast or faster for them) */
+    DXH_TUNE_REDUCE_FUSED_FINISH = 11  /* strided-axis reduction whose reduced axis is cut into slices: 1 (default) = the
+                                          workgroup that finishes a tile last adds the slices, in a fixed order, inside the
+                                          same launch, 0 = a second launch does (also the fallback when the library's
+                                          completion counters are used up).  The two differ in the last bits of a
+                                          floating-point sum or product (different, each fixed, order of addition). */
 };
 DXH_API int dxh_tune(int knob, int64_t value);
 DXH_API int dxh_device_count(int *count);

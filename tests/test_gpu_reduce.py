@@ -140,3 +140,84 @@ def test_config2_full_size(dxh, orc):
     ref = P.astype(np.float64).prod(axis=1)
     assert np.all(np.abs(got - ref) <= 1e-5 * 8 * np.abs(ref))
     assert np.all(np.abs(want - ref) <= 1e-5 * 8 * np.abs(ref))
+
+
+FUSED_KNOB = 11  # DXH_TUNE_REDUCE_FUSED_FINISH
+
+
+def _reduce_on(dxh, name, dtype, da, shape, dims, out, ws, ws_bytes, stream):
+    dx.check(getattr(dxh, "dxh_" + name)(dtype, da.ptr, dx.i32arr(shape), len(shape), dx.i32arr(dims), len(dims), out.ptr, ws.ptr, ws_bytes, stream), name)
+
+
+@pytest.mark.parametrize("dtype", [dx.F32, dx.F64, dx.BF16, dx.I32, dx.I8])
+def test_split_strided_axis_finishes_in_one_launch(dxh, orc, dtype):
+    """A strided axis cut into slices: the last workgroup of a tile adds the slices inside the same
+    launch (knob 11 = 1, default) or a second launch does (0).  Both against the oracle to the
+    file's bars; integers and max / min bit-equal between the two; the one-launch path called
+    three times in a row (its completion counters must be back at zero) gives the same bits."""
+    rng = np.random.default_rng(500 + dtype)
+    for shape, dims in [((4096, 512), [0]), ((3, 2048, 256), [1]), ((8, 4096), [0]), ((5000, 1000), [0]), ((2, 3000, 40), [1]), ((7, 1024, 64), [0, 1])]:
+        a = H.rand(rng, dtype, int(np.prod(shape)), 0.5, 1.5) if dtype not in H.INTS else H.rand(rng, dtype, int(np.prod(shape)))
+        for name in OPS:
+            if name == "prod" and dtype not in H.INTS:
+                a = H.rand(rng, dtype, int(np.prod(shape)), 0.999, 1.001)
+            res = {}
+            for knob in (1, 0):
+                dx.check(dxh.dxh_tune(FUSED_KNOB, knob))
+                try:
+                    runs = [gpu_reduce(dxh, name, dtype, a, shape, dims) for _ in range(3 if knob else 1)]
+                finally:
+                    dx.check(dxh.dxh_tune(FUSED_KNOB, 1))
+                got, nout = runs[0]
+                for other, _ in runs[1:]:
+                    assert np.array_equal(got.view(np.uint8), other.view(np.uint8)), (name, shape, dims)
+                res[knob] = got
+                nred = int(np.prod(shape)) // nout
+                check(name, dtype, got, cpu_reduce(orc, name, dtype, a, shape, dims, nout), nred)
+            if dtype in H.INTS or name in ("reducemax", "reducemin"):
+                assert np.array_equal(res[0], res[1]), (name, shape, dims)
+
+
+def test_one_launch_finish_on_two_streams_and_under_capture(dxh):
+    """Two streams reduce different tensors at the same time (each owns its completion counters), and
+    a reduction recorded under stream capture replays three times next to eager calls on the
+    capture stream; every result equals the eager one-launch result on the default stream."""
+    rng = np.random.default_rng(77)
+    shape, dims = (4096, 2048), [0]
+    sh, dm = dx.i32arr(shape), dx.i32arr(dims)
+    n, nout = shape[0] * shape[1], shape[1]
+    X = [rng.standard_normal(n).astype(np.float32) for _ in range(2)]
+    want = [gpu_reduce(dxh, "sum", dx.F32, x, shape, dims)[0] for x in X]
+    wsb = C.c_size_t(0)
+    dx.check(dxh.dxh_reduce_workspace_bytes(dx.F32, sh, 2, dm, 1, C.byref(wsb)))
+    assert wsb.value > 0  # the axis is cut
+    streams = [C.c_void_p(), C.c_void_p()]
+    for s in streams:
+        dx.check(dxh.dxh_stream_create(C.byref(s)))
+    dev = [Dev(x) for x in X]
+    outs = [Dev.empty(nout, np.float32) for _ in range(2)]
+    wss = [Dev.empty(wsb.value, np.uint8) for _ in range(2)]
+    for _ in range(20):
+        for i in range(2):
+            _reduce_on(dxh, "sum", dx.F32, dev[i], shape, dims, outs[i], wss[i], wsb.value, streams[i])
+    for i in range(2):
+        dx.check(dxh.dxh_stream_sync(streams[i]))
+        assert np.array_equal(outs[i].get(), want[i])
+    # capture on stream 0, replay on stream 1 while stream 0 keeps reducing eagerly
+    gout, gws = Dev.empty(nout, np.float32), Dev.empty(wsb.value, np.uint8)
+    graph = C.c_void_p()
+    dx.check(dxh.dxh_graph_begin_capture(streams[0]))
+    rc = dxh.dxh_sum(dx.F32, dev[1].ptr, sh, 2, dm, 1, gout.ptr, gws.ptr, wsb.value, streams[0])
+    dx.check(dxh.dxh_graph_end_capture(streams[0], C.byref(graph)))
+    dx.check(rc, "sum under capture")
+    for _ in range(3):
+        dx.check(dxh.dxh_graph_launch(graph, streams[1]))
+        for _ in range(5):
+            _reduce_on(dxh, "sum", dx.F32, dev[0], shape, dims, outs[0], wss[0], wsb.value, streams[0])
+        dx.check(dxh.dxh_stream_sync(streams[1]))
+        dx.check(dxh.dxh_stream_sync(streams[0]))
+        assert np.array_equal(gout.get(), want[1])
+        assert np.array_equal(outs[0].get(), want[0])
+    dx.check(dxh.dxh_graph_destroy(graph))
+    for s in streams:
+        dx.check(dxh.dxh_stream_destroy(s))

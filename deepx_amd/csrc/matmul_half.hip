@@ -110,7 +110,7 @@ constexpr int PK = 64;  // K step of the MFMA tile kernel
 __device__ inline int swz(int row, int chunk) { return chunk ^ ((row ^ (row >> 3)) & 7); }
 
 // ---- MFMA kernel with the B transposition done by the LDS read ------------------------------
-// Workgroup tile TM x TN (64, 128 or 256 each), K step 64, 4 waves in a 2x2 grid, each wave a
+// Workgroup tile TM x TN (TM a multiple of 64, TN 64, 128 or 256), K step 64, 4 waves in a 2x2 grid, each wave a
 // (TM/2) x (TN/2) patch of 32x32x16 MFMAs.  Requirements (checked by the launcher): K % 8 == 0,
 // N % 8 == 0, 16-byte aligned A, B, C.  KTAIL (K % 64 != 0): chunks of A and rows of B at k >= K
 // are read from clamped addresses and replaced by zeros.
@@ -119,7 +119,7 @@ __device__ inline int swz(int row, int chunk) { return chunk ^ ((row ^ (row >> 3
 //   A      [TM m][64 k] in LDS, 128-byte rows, 16-byte chunk c of row r at chunk c ^ swizzle(r).
 //   B      stays n-contiguous in LDS, [64 k][TN n] with rows padded by 64 bytes; the MFMA operand
 //          (8 consecutive k of one column per lane) is assembled by two ds_read_b64_tr_b16.
-//   pipe   PD K steps in flight in registers, two LDS stages, one barrier per K step; the stores
+//   pipe   PD (1 or 2) K steps in flight in registers, two LDS stages, one barrier per K step; the stores
 //          into the next stage and the global loads are spread over the four k-substeps.
 //   roles  the MFMA runs on (B^T, A^T): a lane of the result then holds 4 consecutive n of one row
 //          m, which packs into 8-byte LDS stores for the epilogue.
@@ -384,7 +384,7 @@ int launch_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m,
 // product should not be cut (the caller then launches the ordinary way).
 template <typename T>
 int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    constexpr int TM = 64, TN = 64;
+    constexpr int TM = 64, TN = 64, SPD = 1;  // two K steps in flight were measured slower here (64x8192x4096: 21.4 vs 19.0 us)
     const int64_t tiles = batch * ((m + TM - 1) / TM) * ((n + TN - 1) / TN), partial = batch * m * n * (int64_t)sizeof(float);
     const KSplit ks = choose_ksplit(tiles, k, PK, 2048, partial, st);
     TileMap map;
@@ -393,9 +393,9 @@ int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m
     float *ws = (float *)stream_workspace(st, kWorkspaceSplitK, (size_t)(partial * ks.splits));
     if (!ws) return kNoSplit;
     if (k % PK == 0)
-        matmul_mfma_tile_kernel<T, TM, TN, 1, false, 1><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
+        matmul_mfma_tile_kernel<T, TM, TN, SPD, false, 1><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
     else
-        matmul_mfma_tile_kernel<T, TM, TN, 1, true, 1><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
+        matmul_mfma_tile_kernel<T, TM, TN, SPD, true, 1><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
     const int rc = launch_status();
     return rc != DXH_OK ? rc : launch_splitk_reduce<float, T>(ws, (T *)c, batch, m * n, ks.splits, st);
 }
@@ -445,17 +445,34 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
         const int64_t cus = compute_units();
         auto tiles = [&](int tm, int tn) { return batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn); };
         if (m <= 64) choice = 5;  // one tile row: anything taller multiplies padding (bf16 [1,896]x[896,151936]: 53 vs 75 us)
-        else if (tiles(256, 256) * 10 >= cus * 9) choice = 4;
-        else if (tiles(128, 128) * 2 >= cus * 3) choice = 1;
-        else if (tiles(128, 64) * 2 >= cus) choice = 2;
+        else if (tiles(128, 128) * 2 >= cus * 3) {
+            // Enough output for the large tiles: estimated time in us of the three candidates.  The two
+            // one-workgroup-per-CU tiles run in rounds of `cus` tiles, each round paying its own
+            // prologue and its own burst of C stores (nothing else runs on the CU to hide them); K
+            // steps get faster when only part of the CUs is busy.  128x128 tiles run two to a CU: a
+            // pair of tiles takes 1.08 us per K step, a tile that has the CU to itself 0.6 us.
+            const double ksteps = (double)((k + PK - 1) / PK);
+            auto one_per_cu = [&](int tm, int tn, double step, double overhead) {
+                const int64_t t = tiles(tm, tn), rounds = (t + cus - 1) / cus;
+                const double busy = rounds > 1 ? 1.0 : (double)t / (double)cus;
+                return (double)rounds * (ksteps * step * (0.65 + 0.35 * busy) + overhead);
+            };
+            const int64_t t1 = tiles(128, 128), full = t1 / (2 * cus), rem = t1 % (2 * cus);
+            const double c1 = ksteps * (1.08 * (double)full + (rem == 0 ? 0.0 : rem <= cus ? 0.6 : 1.08)) + 2.0;
+            const double edge = ldc >= 0 ? 5.0 : 0.0;  // element-wise C stores make the burst at the end of a round longer
+            const double c4 = one_per_cu(256, 256, 1.645, 3.5 + edge), c6 = one_per_cu(192, 256, 1.21, 6.0 + edge);
+            choice = (c1 <= c4 && c1 <= c6) ? 1 : (c4 <= c6) ? 4 : 6;
+        }
+        else if (tiles(128, 64) * 4 >= cus * 3) choice = 2;  // 1024x8192x1024 (128 such tiles): 38 us, 31 us with 256 64x64 tiles
         else choice = 5;
     }
     if (fast) {
         switch (choice) {
-        case 2: return launch_tile<T, 128, 64, 1>(a, b, c, batch, m, k, n, ldc, st);
-        case 3: return launch_tile<T, 64, 128, 1>(a, b, c, batch, m, k, n, ldc, st);
+        case 2: return launch_tile<T, 128, 64, 2>(a, b, c, batch, m, k, n, ldc, st);
+        case 3: return launch_tile<T, 64, 128, 2>(a, b, c, batch, m, k, n, ldc, st);
         case 4: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st);
-        case 5: return launch_tile<T, 64, 64, 1>(a, b, c, batch, m, k, n, ldc, st);
+        case 5: return launch_tile<T, 64, 64, 2>(a, b, c, batch, m, k, n, ldc, st);
+        case 6: return launch_tile<T, 192, 256, 1>(a, b, c, batch, m, k, n, ldc, st);
         default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, ldc, st);
         }
     }

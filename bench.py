@@ -373,15 +373,12 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
     del g16, u16, o16, x16, x32, o32, col
     torch.cuda.empty_cache()
     c5["mlp_block_over_deepxIR"] = config5_block_over_ir()
+    res["config1"]["chain_over_deepxIR"] = config1_chain_over_ir()
     res["config5"] = c5
     return res
 
 
-def config5_block_over_ir(rows=2048, hidden=896, inter=4864, iters=30):
-    """The whole config-5 block (RMSNorm + gated MLP, 22 deepxIR compute ops on [2048,896] activations)
-    through the executor's dispatch core in this process (libdxexec.so, the code behind the UDP
-    server): wall time per block when the lines are executed one by one, as one batch, and as a
-    recorded HIP graph."""
+def _executor_lib():
     import ctypes as C
     lib = os.path.join(ROOT, "deepx_amd", "executor", "libdxexec.so")
     if not os.path.exists(lib):
@@ -392,15 +389,67 @@ def config5_block_over_ir(rows=2048, hidden=896, inter=4864, iters=30):
     E.dxe_execute.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_size_t]
     E.dxe_execute_batch.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_size_t]
     E.dxe_set_graphs.argtypes = [C.c_void_p, C.c_int]
-    ex = E.dxe_create()
-    buf = C.create_string_buffer(1 << 16)
+    E.dxe_set_fusion.argtypes = [C.c_void_p, C.c_int]
+    return E
 
-    def run(line):
-        E.dxe_execute(ex, line.encode(), buf, len(buf))
-        reply = buf.value.decode()
-        if " ok" not in reply.split("//")[0]:
-            raise RuntimeError(f"{line}: {reply}")
 
+def lines_over_ir(setup, block, iters=30):
+    """`block` (deepxIR lines) through the executor's dispatch core in this process (libdxexec.so, the
+    code behind the UDP server): wall time per pass when the lines are executed one by one, as one
+    batch, as one batch with runs of float elementwise lines fused into single launches, and as a
+    recorded HIP graph without and with those fused runs.  Every mode gets a fresh executor (a
+    recorded graph is keyed by the text of the batch)."""
+    import ctypes as C
+    E = _executor_lib()
+    lines = [f"{l} // author=miaobyte id={i + 1}" for i, l in enumerate(block)]
+    text = "\n".join(lines).encode()
+    out = {"ops": len(lines)}
+    for label, batched, fused, graphs in (("line_by_line_us", 0, 0, 0), ("one_batch_us", 1, 0, 0), ("one_batch_fused_us", 1, 1, 0),
+                                          ("recorded_graph_us", 1, 0, 1), ("recorded_graph_fused_us", 1, 1, 1)):
+        ex = E.dxe_create()
+        buf = C.create_string_buffer(1 << 16)
+        for line in setup:
+            E.dxe_execute(ex, line.encode(), buf, len(buf))
+            reply = buf.value.decode()
+            if " ok" not in reply.split("//")[0]:
+                raise RuntimeError(f"{line}: {reply}")
+        E.dxe_set_graphs(ex, graphs)
+        E.dxe_set_fusion(ex, fused)
+
+        def once():
+            if batched:
+                E.dxe_execute_batch(ex, text, buf, len(buf))
+            else:
+                for l in lines:
+                    E.dxe_execute(ex, l.encode(), buf, len(buf))
+
+        for _ in range(4):
+            once()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            once()
+        out[label] = round((time.perf_counter() - t0) / iters * 1e6, 1)
+        if any(" ok" not in r.split("//")[0] for r in buf.value.decode().split("\n")):
+            raise RuntimeError("block failed: " + buf.value.decode())
+        E.dxe_destroy(ex)
+    return out
+
+
+def config1_chain_over_ir(side=4096):
+    """The 8-op elementwise chain of config 1 on [4096,4096] fp32 as deepxIR lines."""
+    T = lambda n: f"tensor<float32>:c1_{n}"
+    V = f"vector<int32>:[{side} {side}]"
+    names = ["A", "B", "C", "D", "E", "F", "nB", "absB", "den", "G"]
+    setup = [f"newtensor({V})->({T(n)})" for n in names]
+    setup += [f"uniform(var<float32>:-1, var<float32>:1, var<int32>:{seed})->({T(n)}) // author=miaobyte" for n, seed in (("A", 1), ("B", 2))]
+    block = [f"add({T('A')}, {T('B')})->({T('C')})", f"mul({T('C')}, {T('B')})->({T('D')})", f"addscalar({T('D')}, var<float32>:0.5)->({T('E')})",
+             f"exp({T('E')})->({T('F')})", f"mulscalar({T('B')}, var<float32>:-1)->({T('nB')})", f"max({T('B')}, {T('nB')})->({T('absB')})",
+             f"addscalar({T('absB')}, var<float32>:1)->({T('den')})", f"div({T('F')}, {T('den')})->({T('G')})"]
+    return lines_over_ir(setup, block)
+
+
+def config5_block_over_ir(rows=2048, hidden=896, inter=4864):
+    """The whole config-5 block (RMSNorm + gated MLP, 22 deepxIR compute ops on [2048,896] activations)."""
     S, Hd, I = rows, hidden, inter
     b16, f32 = "bfloat16", "float32"
     T = lambda n, dt=f32: f"tensor<{dt}>:{n}"
@@ -409,12 +458,11 @@ def config5_block_over_ir(rows=2048, hidden=896, inter=4864, iters=30):
                ("xf", [S, Hd], f32), ("sq", [S, Hd], f32), ("var", [S, 1], f32), ("rs", [S, Hd], f32), ("xn", [S, Hd], f32),
                ("wf1", [1, Hd], f32), ("wf", [S, Hd], f32), ("h", [S, Hd], b16), ("g", [S, I], b16), ("u", [S, I], b16),
                ("sg", [S, I], b16), ("y", [S, Hd], b16)]
-    for name, shape, dt in tensors:
-        run(f"newtensor({V(shape)})->({T('b5_' + name, dt)})")
-    run(f"normal(var<float32>:0, var<float32>:1, var<int32>:14)->({T('b5_x', b16)}) // author=miaobyte")
-    run(f"constant(var<float32>:1)->({T('b5_w', b16)}) // author=miaobyte")
+    setup = [f"newtensor({V(shape)})->({T('b5_' + name, dt)})" for name, shape, dt in tensors]
+    setup.append(f"normal(var<float32>:0, var<float32>:1, var<int32>:14)->({T('b5_x', b16)}) // author=miaobyte")
+    setup.append(f"constant(var<float32>:1)->({T('b5_w', b16)}) // author=miaobyte")
     for name, seed in (("Wg", 15), ("Wu", 16), ("Wd", 17)):
-        run(f"normal(var<float32>:0, var<float32>:0.02, var<int32>:{seed})->({T('b5_' + name, b16)}) // author=miaobyte")
+        setup.append(f"normal(var<float32>:0, var<float32>:0.02, var<int32>:{seed})->({T('b5_' + name, b16)}) // author=miaobyte")
     n = lambda name, dt=f32: T("b5_" + name, dt)
     block = [f"todtype({n('x', b16)})->({n('xf')})",
              f"powscalar({n('xf')}, var<float32>:2)->({n('sq')})",
@@ -438,28 +486,8 @@ def config5_block_over_ir(rows=2048, hidden=896, inter=4864, iters=30):
              f"mul({n('g', b16)}, {n('sg', b16)})->({n('sg', b16)})",
              f"mul({n('sg', b16)}, {n('u', b16)})->({n('sg', b16)})",
              f"matmul({n('sg', b16)}, {n('Wd', b16)})->({n('y', b16)})"]
-    lines = [f"{l} // author=miaobyte id={i + 1}" for i, l in enumerate(block)]
-    text = "\n".join(lines).encode()
-
-    def one_by_one():
-        for l in lines:
-            E.dxe_execute(ex, l.encode(), buf, len(buf))
-
-    def batched():
-        E.dxe_execute_batch(ex, text, buf, len(buf))
-
-    out = {"ops": len(lines), "rows": S}
-    for label, fn, graphs in (("line_by_line_us", one_by_one, 0), ("one_batch_us", batched, 0), ("recorded_graph_us", batched, 1)):
-        E.dxe_set_graphs(ex, graphs)
-        for _ in range(4):
-            fn()
-        t0 = time.perf_counter()
-        for _ in range(iters):
-            fn()
-        out[label] = round((time.perf_counter() - t0) / iters * 1e6, 1)
-        if any(" ok" not in r.split("//")[0] for r in buf.value.decode().split("\n")):
-            raise RuntimeError("config-5 block failed: " + buf.value.decode())
-    E.dxe_destroy(ex)
+    out = lines_over_ir(setup, block)
+    out["rows"] = S
     return out
 
 

@@ -302,6 +302,112 @@ template <typename Op, bool HALF> int unary_float(int dtype, const void *a, void
     }
 }
 
+
+// ---- a run of elementwise ops in one launch ---------------------------------------------------
+// Same arithmetic as the kernels above, op after op, each result rounded to T and stored before
+// the next op uses it, so every output has the bits the separate launches give.  What is saved is
+// the traffic: an operand that an earlier op of the run produced (or that was loaded for an
+// earlier op) is not read from memory again.  A lane handles one 16-byte vector index: it loads
+// that vector of every input up front (all loads in flight together) and walks the op list.  The
+// result of the op before is at hand in registers; inputs, and results that a later op other
+// than the next one uses, sit in LDS slots of the lane's own, addressed by operand number at run
+// time (no barriers: no lane reads another lane's slots).  The launch asks for as many slots as
+// the run needs (4 KiB each), so short runs keep the CU full of waves.
+constexpr int kChainOps = DXH_CHAIN_MAX_OPS, kChainInputs = DXH_CHAIN_MAX_INPUTS;
+struct ChainArgs {
+    const void *in[kChainInputs];
+    void *out[kChainOps];
+    double scalar[kChainOps];  // already rounded to T on the host
+    int8_t code[kChainOps], lhs[kChainOps], rhs[kChainOps];  // operand: LDS slot, or kChainPrev = result of the op before
+    int8_t save[kChainOps];                                  // LDS slot that keeps the result for later ops, or -1
+    int n_in, n_ops;                                         // inputs occupy slots 0 .. n_in - 1
+};
+constexpr int kChainPrev = -1;
+template <typename T>
+__global__ __launch_bounds__(kBlock) void chain_kernel(const ChainArgs p, int64_t nv) {
+    constexpr int V = vec_len<T>;
+    using VT = vec_t<T, V>;
+    using A = acc_t<T>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char chain_lds[];
+    const int t = threadIdx.x;
+    // The op table is indexed by a loop counter.  Out of the kernel argument that would make the
+    // compiler copy the whole table into per-lane scratch memory; out of LDS (filled once, with
+    // constant indices) it is a broadcast read.
+    __shared__ int s_code[kChainOps], s_lhs[kChainOps], s_rhs[kChainOps], s_save[kChainOps];
+    __shared__ double s_scalar[kChainOps];
+    __shared__ void *s_out[kChainOps];
+    if (t == 0) {
+#pragma unroll
+        for (int k = 0; k < kChainOps; ++k) {
+            s_code[k] = p.code[k]; s_lhs[k] = p.lhs[k]; s_rhs[k] = p.rhs[k]; s_save[k] = p.save[k];
+            s_scalar[k] = p.scalar[k]; s_out[k] = p.out[k];
+        }
+    }
+    __syncthreads();
+    // registers and LDS hold raw 16-byte vectors (a select between two of them stays in registers)
+    u32x4_t *raw = reinterpret_cast<u32x4_t *>(chain_lds);
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + t; i < nv; i += (int64_t)gridDim.x * kBlock) {
+        u32x4_t x0 = {0u, 0u, 0u, 0u}, x1 = x0, x2 = x0, x3 = x0, x4 = x0, x5 = x0, x6 = x0, x7 = x0;
+#define DXH_CH_LOAD(j) if (j < p.n_in) x##j = reinterpret_cast<const u32x4_t *>(p.in[j])[i]
+        DXH_CH_LOAD(0); DXH_CH_LOAD(1); DXH_CH_LOAD(2); DXH_CH_LOAD(3); DXH_CH_LOAD(4); DXH_CH_LOAD(5); DXH_CH_LOAD(6); DXH_CH_LOAD(7);
+#undef DXH_CH_LOAD
+#define DXH_CH_KEEP(j) if (j < p.n_in) raw[j * kBlock + t] = x##j
+        DXH_CH_KEEP(0); DXH_CH_KEEP(1); DXH_CH_KEEP(2); DXH_CH_KEEP(3); DXH_CH_KEEP(4); DXH_CH_KEEP(5); DXH_CH_KEEP(6); DXH_CH_KEEP(7);
+#undef DXH_CH_KEEP
+        u32x4_t prev = x0;
+        for (int k = 0; k < p.n_ops; ++k) {
+            const int code = __builtin_amdgcn_readfirstlane(s_code[k]), l = __builtin_amdgcn_readfirstlane(s_lhs[k]);
+            const int q = __builtin_amdgcn_readfirstlane(s_rhs[k]), save = __builtin_amdgcn_readfirstlane(s_save[k]);
+            u32x4_t ra = prev, rb = prev;
+            if (l != kChainPrev) ra = raw[l * kBlock + t];
+            if (q != kChainPrev) rb = raw[q * kBlock + t];
+            const VT a = __builtin_bit_cast(VT, ra), b = __builtin_bit_cast(VT, rb);
+            const A s = A(s_scalar[k]);
+            VT r;
+#define DXH_CH_BIN(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) r.v[v] = store_acc<T>(Op::f(A(load_acc(a.v[v])), A(load_acc(b.v[v])))); break
+#define DXH_CH_SCALAR(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) r.v[v] = store_acc<T>(Op::f(A(load_acc(a.v[v])), s)); break
+#define DXH_CH_UNARY(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) r.v[v] = store_acc<T>(Op::f(load_acc(a.v[v]))); break
+            switch (code) {
+            case DXH_CHAIN_ADD: DXH_CH_BIN(OpAdd);
+            case DXH_CHAIN_SUB: DXH_CH_BIN(OpSub);
+            case DXH_CHAIN_MUL: DXH_CH_BIN(OpMul);
+            case DXH_CHAIN_DIV: DXH_CH_BIN(OpDiv);
+            case DXH_CHAIN_MAX: DXH_CH_BIN(OpMax);
+            case DXH_CHAIN_MIN: DXH_CH_BIN(OpMin);
+            case DXH_CHAIN_ADDSCALAR: DXH_CH_SCALAR(OpAdd);
+            case DXH_CHAIN_SUBSCALAR: DXH_CH_SCALAR(OpSub);
+            case DXH_CHAIN_RSUBSCALAR: DXH_CH_SCALAR(OpRSub);
+            case DXH_CHAIN_MULSCALAR: DXH_CH_SCALAR(OpMul);
+            case DXH_CHAIN_DIVSCALAR: DXH_CH_SCALAR(OpDiv);
+            case DXH_CHAIN_RDIVSCALAR: DXH_CH_SCALAR(OpRDiv);
+            case DXH_CHAIN_MAXSCALAR: DXH_CH_SCALAR(OpMax);
+            case DXH_CHAIN_MINSCALAR: DXH_CH_SCALAR(OpMin);
+            case DXH_CHAIN_SQRT: DXH_CH_UNARY(OpSqrt);
+            case DXH_CHAIN_EXP: DXH_CH_UNARY(OpExp);
+            default: DXH_CH_UNARY(OpLog);
+            }
+#undef DXH_CH_BIN
+#undef DXH_CH_SCALAR
+#undef DXH_CH_UNARY
+            prev = __builtin_bit_cast(u32x4_t, r);
+            if (save >= 0) raw[save * kBlock + t] = prev;
+            if (s_out[k]) __builtin_nontemporal_store(prev, &reinterpret_cast<u32x4_t *>(s_out[k])[i]);
+        }
+    }
+}
+
+template <typename T>
+int launch_chain(ChainArgs &p, const dxh_chain_op *ops, int64_t n, hipStream_t st) {
+    constexpr int V = vec_len<T>;
+    if (n % V != 0) return DXH_ERR_ALIGN;
+    for (int k = 0; k < p.n_ops; ++k) p.scalar[k] = (double)load_acc(scalar_to<T>(ops[k].scalar));
+    const int64_t nv = n / V, blocks = (nv + kBlock - 1) / kBlock;
+    int slots = p.n_in;
+    for (int k = 0; k < p.n_ops; ++k) slots = std::max(slots, p.save[k] + 1);
+    chain_kernel<T><<<(unsigned)std::min<int64_t>(blocks, 1 << 22), kBlock, (size_t)slots * kBlock * kVecBytes, st>>>(p, nv);
+    return launch_status();
+}
+
 }  // namespace dxh
 
 using namespace dxh;
@@ -349,6 +455,49 @@ int dxh_invert(int dtype, const void *a, void *c, int64_t n, void *stream) {
     case DXH_I16: return launch_unary<int16_t, OpInvert>(a, c, n, st);
     case DXH_I8: return launch_unary<int8_t, OpInvert>(a, c, n, st);
     case DXH_BOOL: return launch_unary<bool_t, OpInvert>(a, c, n, st);
+    default: return DXH_ERR_DTYPE;
+    }
+}
+
+int dxh_chain(int dtype, const void *const *inputs, int n_inputs, const dxh_chain_op *ops, int n_ops, int64_t n, void *stream) {
+    DXH_CHECK_N(n);
+    if (n_ops < 1 || n_ops > kChainOps || n_inputs < 0 || n_inputs > kChainInputs || !ops || (n_inputs > 0 && !inputs)) return DXH_ERR_ARG;
+    ChainArgs p{};
+    p.n_in = n_inputs;
+    p.n_ops = n_ops;
+    for (int j = 0; j < n_inputs; ++j) {
+        if (!inputs[j]) return DXH_ERR_ARG;
+        if (!aligned(inputs[j], kVecBytes)) return DXH_ERR_ALIGN;
+        p.in[j] = inputs[j];
+    }
+    // operand of op k: an input's slot, the registers (result of op k - 1), or the slot that the
+    // producing op saves into (handed out here, on first use)
+    int next_slot = n_inputs;
+    for (int k = 0; k < n_ops; ++k) p.save[k] = -1;
+    constexpr int kBad = -2;
+    auto operand = [&](int ref, int k) {
+        if (ref >= 0 && ref < n_inputs) return ref;
+        if (ref < DXH_CHAIN_RESULT || ref >= DXH_CHAIN_RESULT + k) return kBad;
+        const int j = ref - DXH_CHAIN_RESULT;
+        if (j == k - 1) return kChainPrev;
+        if (p.save[j] < 0) p.save[j] = (int8_t)next_slot++;
+        return (int)p.save[j];
+    };
+    for (int k = 0; k < n_ops; ++k) {
+        const dxh_chain_op &o = ops[k];
+        if (o.code < DXH_CHAIN_ADD || o.code > DXH_CHAIN_LOG || (!o.out && k == n_ops - 1)) return DXH_ERR_ARG;
+        if (o.out && !aligned(o.out, kVecBytes)) return DXH_ERR_ALIGN;
+        const int l = operand(o.lhs, k), r = o.code <= DXH_CHAIN_MIN ? operand(o.rhs, k) : l;
+        if (l == kBad || r == kBad) return DXH_ERR_ARG;
+        p.code[k] = (int8_t)o.code; p.lhs[k] = (int8_t)l; p.rhs[k] = (int8_t)r; p.out[k] = o.out;
+    }
+    if (n == 0) return DXH_OK;
+    hipStream_t st = as_stream(stream);
+    switch (dtype) {
+    case DXH_F64: return launch_chain<double>(p, ops, n, st);
+    case DXH_F32: return launch_chain<float>(p, ops, n, st);
+    case DXH_F16: return launch_chain<f16_t>(p, ops, n, st);
+    case DXH_BF16: return launch_chain<bf16_t>(p, ops, n, st);
     default: return DXH_ERR_DTYPE;
     }
 }

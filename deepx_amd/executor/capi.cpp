@@ -39,6 +39,12 @@ DXE_API size_t dxe_execute_batch(void *ex, const char *text, char *reply, size_t
 }
 // graph recording on/off (the DEEPX_GRAPH switch) and the batch counters: "batches captures replays rejects"
 DXE_API void dxe_set_graphs(void *ex, int on) { static_cast<Executor *>(ex)->use_graphs = on != 0; }
+// one launch for runs of float elementwise lines inside a batch (the DEEPX_FUSE switch), and its counters: "runs lines"
+DXE_API void dxe_set_fusion(void *ex, int on) { static_cast<Executor *>(ex)->use_fusion = on != 0; }
+DXE_API size_t dxe_fusion_stats(void *ex, char *out, size_t buflen) {
+    const auto &s = static_cast<Executor *>(ex)->stats;
+    return copy_out(std::to_string(s.fused_runs) + " " + std::to_string(s.fused_lines), out, buflen);
+}
 DXE_API size_t dxe_stats(void *ex, char *out, size_t buflen) {
     const auto &s = static_cast<Executor *>(ex)->stats;
     return copy_out(std::to_string(s.batches) + " " + std::to_string(s.graph_captures) + " " + std::to_string(s.graph_replays) + " " +

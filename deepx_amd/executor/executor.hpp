@@ -31,7 +31,11 @@ public:
     // DEEPX_GRAPH=1: a datagram of several graph-safe lines that arrives a second time is recorded
     // into a HIP graph and replayed from then on (one launch instead of one per kernel)
     bool use_graphs = false;
-    struct Stats { uint64_t batches = 0, graph_captures = 0, graph_replays = 0, graph_rejects = 0; } stats;
+    // Inside a batch, consecutive float elementwise lines over tensors of one dtype and size run as
+    // one launch (dxh_chain): same bits in every output, operands that the run itself produced are
+    // not read back from memory.  DEEPX_FUSE=0 turns it off.
+    bool use_fusion = true;
+    struct Stats { uint64_t batches = 0, graph_captures = 0, graph_replays = 0, graph_rejects = 0, fused_runs = 0, fused_lines = 0; } stats;
 
     Executor() {
         register_all(factory);
@@ -43,6 +47,8 @@ public:
         has_device = dxh_device_count(&count) == DXH_OK && count > 0;
         const char *g = std::getenv("DEEPX_GRAPH");
         use_graphs = g && !std::strcmp(g, "1");
+        const char *fuse = std::getenv("DEEPX_FUSE");
+        if (fuse && !std::strcmp(fuse, "0")) use_fusion = false;
     }
     ~Executor() {
         for (auto &kv : graphs_) dxh_graph_destroy(kv.second.exec);
@@ -171,26 +177,55 @@ public:
             it.tf->returns = it.call.returns;
             graphable = graphable && it.tf->graph_safe && it.tf->metadata.benchmark_repeat <= 1 && !uses_named_arg(it.call);
         }
+        std::vector<std::shared_ptr<TF>> tfs(items.size());
+        for (size_t i = 0; i < items.size(); ++i) if (!items[i].failed) tfs[i] = items[i].tf;
+        // Runs line i, or a run of lines that starts at i as one launch; returns how many lines that were.
+        // A run that cannot be launched after all falls back to its first line alone.
+        auto run_next = [&](size_t i, std::string &message, int &rc) -> size_t {
+            if (use_fusion && has_device) {
+                const size_t len = chain_length(tfs, i, mem);
+                if (len >= 2) {
+                    rc = run_chain(tfs, i, len, mem, message);
+                    if (rc == 0) { ++stats.fused_runs; stats.fused_lines += len; return len; }
+                    message.clear();
+                }
+            }
+            const int repeat = items[i].tf->metadata.benchmark_repeat > 1 ? items[i].tf->metadata.benchmark_repeat : 1;
+            rc = 0;
+            for (int r = 0; r < repeat && rc == 0; ++r) rc = items[i].tf->run(mem, message);
+            return 1;
+        };
         bool done = false;
         if (graphable) {
-            if (run_as_graph(key, items.size(), [&](size_t i, std::string &msg) { return items[i].tf->run(mem, msg); }, [&](size_t i) -> const TF & { return items[i].call; })) {
+            auto run_all = [&]() {
+                for (size_t i = 0; i < items.size();) {
+                    std::string message;
+                    int rc = 0;
+                    const size_t used = run_next(i, message, rc);
+                    if (rc != 0) return false;
+                    i += used;
+                }
+                return true;
+            };
+            if (run_as_graph(key, items.size(), run_all, [&](size_t i) -> const TF & { return items[i].call; })) {
                 for (Item &it : items) { it.resp.start_at = recv_at; it.resp.finish(""); }
                 done = true;
             }
         }
         if (!done) {
-            for (Item &it : items) {
-                if (it.failed) continue;
-                it.resp.start_at = std::chrono::system_clock::now();
+            for (size_t i = 0; i < items.size();) {
+                if (items[i].failed) { ++i; continue; }
+                const TimePoint started = std::chrono::system_clock::now();
                 int rc = 0;
                 std::string message;
-                const int repeat = it.tf->metadata.benchmark_repeat > 1 ? it.tf->metadata.benchmark_repeat : 1;
-                for (int r = 0; r < repeat && rc == 0; ++r) rc = it.tf->run(mem, message);
+                const size_t used = run_next(i, message, rc);
+                for (size_t j = i; j < i + used; ++j) items[j].resp.start_at = started;
                 if (rc != 0) {
                     std::cerr << message << std::endl;
-                    it.resp.error(message);
-                    it.failed = true;
+                    items[i].resp.error(message);
+                    items[i].failed = true;
                 }
+                i += used;
             }
             std::string sync_error;
             if (sync_each && has_device) {
@@ -273,7 +308,7 @@ private:
     // recorded on its second arrival (the first, eager, pass also sizes the reduction workspace),
     // and replayed only while every tensor it names still has the address, size and dtype it was
     // recorded with.
-    bool run_as_graph(const std::string &key, size_t n, const std::function<int(size_t, std::string &)> &run_at,
+    bool run_as_graph(const std::string &key, size_t n, const std::function<bool()> &run_all,
                       const std::function<const TF &(size_t)> &call_at) {
         if (rejected_.count(key)) return false;
         Graph now;
@@ -295,11 +330,7 @@ private:
             if (dxh_graph_begin_capture(graph_stream_) != DXH_OK) return false;
             mem.stream = graph_stream_;
             mem.recording = true;
-            bool ok = true;
-            for (size_t i = 0; i < n && ok; ++i) {
-                std::string message;
-                ok = run_at(i, message) == 0;
-            }
+            const bool ok = run_all();
             mem.stream = nullptr;
             mem.recording = false;
             void *exec = nullptr;

@@ -102,5 +102,10 @@ public:
 };
 
 int register_all(TfFactory &factory);  // ops.cpp
+// ops.cpp: how many of the calls tfs[first], tfs[first + 1], ... (nullptr = a line that failed
+// earlier) can run as one dxh_chain launch right now (tensors present, one float dtype and size,
+// 16-byte aligned whole vectors); 0 or 1 = none.  run_chain launches exactly that run.
+size_t chain_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem);
+int run_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, size_t count, Mem &mem, std::string &error);
 
 }  // namespace deepx

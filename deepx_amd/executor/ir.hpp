@@ -125,6 +125,9 @@ public:
     // true for ops that only launch kernels on Mem's stream (no allocation, host copy, file I/O or
     // fresh random seed): those may be recorded into a HIP graph by the batch path
     bool graph_safe = false;
+    // float elementwise ops that dxh_chain can run as part of one launch: its op code, and where the
+    // operands sit (1: args 0 and 1 are tensors, 2: tensor then scalar, 3: scalar then tensor, 4: one tensor)
+    int chain_code = -1, chain_kind = 0;
 
     TF() = default;
     explicit TF(const std::string &text) { parse(text); }

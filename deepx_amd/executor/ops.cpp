@@ -67,6 +67,16 @@ void reg(TfFactory &f, const char *name, const char *author, const char *tftype,
     for (const char *r : returns) tf->returns.push_back(registered(r));
     tf->fn = std::move(fn);
     const std::string kind = tftype, op = name;
+    static const struct { const char *name; int code, kind; } chainable[] = {
+        {"add", DXH_CHAIN_ADD, 1}, {"sub", DXH_CHAIN_SUB, 1}, {"mul", DXH_CHAIN_MUL, 1}, {"div", DXH_CHAIN_DIV, 1},
+        {"max", DXH_CHAIN_MAX, 1}, {"min", DXH_CHAIN_MIN, 1},
+        {"addscalar", DXH_CHAIN_ADDSCALAR, 2}, {"subscalar", DXH_CHAIN_SUBSCALAR, 2}, {"rsubscalar", DXH_CHAIN_RSUBSCALAR, 3},
+        {"mulscalar", DXH_CHAIN_MULSCALAR, 2}, {"divscalar", DXH_CHAIN_DIVSCALAR, 2}, {"rdivscalar", DXH_CHAIN_RDIVSCALAR, 3},
+        {"maxscalar", DXH_CHAIN_MAXSCALAR, 2}, {"minscalar", DXH_CHAIN_MINSCALAR, 2},
+        {"sqrt", DXH_CHAIN_SQRT, 4}, {"exp", DXH_CHAIN_EXP, 4}, {"log", DXH_CHAIN_LOG, 4}};
+    if (kind == "elementwise")
+        for (const auto &c : chainable)
+            if (op == c.name) { tf->chain_code = c.code; tf->chain_kind = c.kind; }
     tf->graph_safe = kind == "elementwise" || kind == "reduce" || kind == "changeshape" || op == "matmul" ||
                      op == "constant" || op == "arange";
     if (op == "reshape") tf->graph_safe = false;  // rewrites the tensor's shape on the host
@@ -539,6 +549,103 @@ int register_all(TfFactory &f) {
         reg(f, "matmul", author, "matmul", "T3=T1 @ T2", {T_ANY ":A", T_ANY ":B"}, {T_ANY ":C"}, matmul);
 #undef T_ANY
     return 0;
+}
+
+// ---- several elementwise lines as one launch --------------------------------------------------
+namespace {
+struct ChainPlan {
+    int dtype = 0;
+    int64_t n = 0;
+    std::vector<const void *> inputs;
+    std::vector<dxh_chain_op> ops;
+};
+// Builds the longest run starting at tfs[first].  A tensor operand is the latest result of the run
+// with that name, else an input of the run (read before the run writes anything, which is what a
+// line-by-line execution sees as long as no earlier line of the run has written it — and those are
+// taken as results).  A tensor that several lines of the run write is stored by the last of them
+// only: nothing reads memory in between.  The run ends before a line that is not a chainable float
+// op, has another dtype or size, needs a ninth input, or whose operands are missing (the ordinary
+// path then reports the error for that line).
+size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem, ChainPlan &plan) {
+    std::vector<std::string> input_names, output_names;
+    size_t count = 0;
+    for (size_t i = first; i < tfs.size() && plan.ops.size() < DXH_CHAIN_MAX_OPS; ++i) {
+        const TF *tf = tfs[i].get();
+        if (!tf || tf->chain_kind == 0 || tf->metadata.benchmark_repeat > 1 || tf->returns.size() != 1) break;
+        const size_t nargs = tf->chain_kind == 4 ? 1 : 2;
+        if (tf->args.size() != nargs) break;
+        const Param *tensors[2] = {nullptr, nullptr};
+        const Param *scalar = nullptr;
+        switch (tf->chain_kind) {
+        case 1: tensors[0] = &tf->args[0]; tensors[1] = &tf->args[1]; break;
+        case 2: tensors[0] = &tf->args[0]; scalar = &tf->args[1]; break;
+        case 3: scalar = &tf->args[0]; tensors[0] = &tf->args[1]; break;
+        default: tensors[0] = &tf->args[0]; break;
+        }
+        auto out = mem.findtensor(tf->returns[0].textvalue);
+        if (!out) break;
+        const int dtype = out->dtype();
+        if (dtype != DXH_F64 && dtype != DXH_F32 && dtype != DXH_F16 && dtype != DXH_BF16) break;
+        if (plan.ops.empty()) { plan.dtype = dtype; plan.n = out->shape.size; }
+        if (dtype != plan.dtype || out->shape.size != plan.n) break;
+        dxh_chain_op op{};
+        op.code = tf->chain_code;
+        op.out = out->data;
+        std::vector<std::string> new_inputs;
+        std::vector<const void *> new_ptrs;
+        bool ok = true;
+        for (int side = 0; side < 2 && ok; ++side) {
+            if (!tensors[side]) continue;
+            const std::string &name = tensors[side]->textvalue;
+            auto t = mem.findtensor(name);
+            if (!t || t->dtype() != plan.dtype || t->shape.size != plan.n) { ok = false; break; }
+            int ref = -1;
+            for (size_t j = output_names.size(); j-- > 0;)
+                if (output_names[j] == name) { ref = DXH_CHAIN_RESULT + (int)j; break; }
+            if (ref < 0) {
+                for (size_t j = 0; j < input_names.size() && ref < 0; ++j) if (input_names[j] == name) ref = (int)j;
+                for (size_t j = 0; j < new_inputs.size() && ref < 0; ++j) if (new_inputs[j] == name) ref = (int)(input_names.size() + j);
+                if (ref < 0) {
+                    if (input_names.size() + new_inputs.size() >= DXH_CHAIN_MAX_INPUTS) { ok = false; break; }
+                    ref = (int)(input_names.size() + new_inputs.size());
+                    new_inputs.push_back(name);
+                    new_ptrs.push_back(t->data);
+                }
+            }
+            (side == 0 ? op.lhs : op.rhs) = ref;
+        }
+        if (!ok) break;
+        if (scalar) {
+            try { op.scalar = scalar_of(*scalar, mem); } catch (const std::exception &) { break; }
+        }
+        input_names.insert(input_names.end(), new_inputs.begin(), new_inputs.end());
+        plan.inputs.insert(plan.inputs.end(), new_ptrs.begin(), new_ptrs.end());
+        output_names.push_back(tf->returns[0].textvalue);
+        plan.ops.push_back(op);
+        ++count;
+    }
+    if (count < 2) return count;
+    for (size_t j = 0; j < output_names.size(); ++j)
+        for (size_t m = j + 1; m < output_names.size(); ++m)
+            if (output_names[m] == output_names[j]) plan.ops[j].out = nullptr;  // overwritten by line m of the run
+    // whole 16-byte vectors at 16-byte aligned addresses, or the separate calls take it
+    const int64_t vec = 16 / precision_bytes((Precision)plan.dtype);
+    bool aligned = plan.n % vec == 0;
+    for (const void *p : plan.inputs) aligned = aligned && ((uintptr_t)p & 15) == 0;
+    for (const dxh_chain_op &o : plan.ops) aligned = aligned && ((uintptr_t)o.out & 15) == 0;  // NULL passes
+    return aligned ? count : 0;
+}
+}  // namespace
+
+size_t chain_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem) {
+    ChainPlan plan;
+    return plan_chain(tfs, first, mem, plan);
+}
+int run_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, size_t count, Mem &mem, std::string &error) {
+    ChainPlan plan;
+    if (plan_chain(tfs, first, mem, plan) != count || count < 2) return fail(error, "chain: the run changed between planning and launch");
+    return hip_result(dxh_chain(plan.dtype, plan.inputs.data(), (int)plan.inputs.size(), plan.ops.data(), (int)plan.ops.size(), plan.n, mem.stream),
+                      "chain", error);
 }
 
 }  // namespace deepx

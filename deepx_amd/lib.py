@@ -26,6 +26,17 @@ class Scalar(C.Structure):
     _fields_ = [("f", C.c_double), ("i", C.c_int64)]
 
 
+class ChainOp(C.Structure):
+    """dxh_chain_op: one op of a dxh_chain run."""
+    _fields_ = [("code", C.c_int32), ("lhs", C.c_int32), ("rhs", C.c_int32), ("scalar", Scalar), ("out", C.c_void_p)]
+
+
+# enum dxh_chain_code, in the header's order
+CHAIN_CODES = ["add", "sub", "mul", "div", "max", "min", "addscalar", "subscalar", "rsubscalar", "mulscalar",
+               "divscalar", "rdivscalar", "maxscalar", "minscalar", "sqrt", "exp", "log"]
+CHAIN_RESULT = 16
+
+
 def scalar(v):
     """Both views of one scalar, as the executor fills them from T(std::stof(text))."""
     f = float(v)
@@ -82,6 +93,7 @@ SIGNATURES = {
     "dxh_powscalar": (_SCL, _i), "dxh_rpowscalar": (_RSCL, _i),
     "dxh_sqrt": (_UN, _i), "dxh_exp": (_UN, _i), "dxh_log": (_UN, _i),
     "dxh_sin": (_UN, _i), "dxh_cos": (_UN, _i), "dxh_tan": (_UN, _i), "dxh_invert": (_UN, _i),
+    "dxh_chain": ([_i, _pp, _i, C.POINTER(ChainOp), _i, _i64, _p], _i),
     "dxh_todtype": ([_i, _p, _i, _p, _i64, _p], _i),
     "dxh_equal": ([_i, _p, _p, _f, _p, _i64, _p], _i),
     "dxh_notequal": ([_i, _p, _p, _f, _p, _i64, _p], _i),

@@ -193,6 +193,36 @@ DXH_API int dxh_cos(int dtype, const void *a, void *c, int64_t n, void *stream);
 DXH_API int dxh_tan(int dtype, const void *a, void *c, int64_t n, void *stream);
 DXH_API int dxh_invert(int dtype, const void *a, void *c, int64_t n, void *stream);
 
+/* ---- a run of elementwise ops in one launch
+ * No counterpart in the reference, which launches op by op; for a caller that holds several
+ * instructions at once (a datagram of deepxIR lines, udpserver.cpp:49-58).  Op k of the run is one of
+ * the float ops above over tensors of `n` elements of `dtype` (f64 f32 f16 bf16); its tensor
+ * operands are inputs[ref] or, as DXH_CHAIN_RESULT + j, the result of op j < k of the same run; its
+ * result is rounded to `dtype` and stored to `out` before a later op uses it, so every `out` holds
+ * exactly what the separate calls would have stored.  Inputs are read before any result is written:
+ * an `out` may be one of the inputs (in-place ops), but a later op that is to see such a result must
+ * name it as DXH_CHAIN_RESULT + j.  An op other than the last may have out = NULL: its result then only
+ * feeds later ops of the run (for a tensor that a later op of the run overwrites anyway).
+ * All pointers 16-byte aligned and n a multiple of 16 / sizeof(dtype),
+ * else DXH_ERR_ALIGN (use the separate calls then).  Scalar forms take `scalar` and `lhs`; unary
+ * forms `lhs` only. */
+enum dxh_chain_code {
+    DXH_CHAIN_ADD = 0, DXH_CHAIN_SUB, DXH_CHAIN_MUL, DXH_CHAIN_DIV, DXH_CHAIN_MAX, DXH_CHAIN_MIN,      /* lhs op rhs */
+    DXH_CHAIN_ADDSCALAR, DXH_CHAIN_SUBSCALAR, DXH_CHAIN_RSUBSCALAR, DXH_CHAIN_MULSCALAR,               /* lhs op scalar; R: scalar op lhs */
+    DXH_CHAIN_DIVSCALAR, DXH_CHAIN_RDIVSCALAR, DXH_CHAIN_MAXSCALAR, DXH_CHAIN_MINSCALAR,
+    DXH_CHAIN_SQRT, DXH_CHAIN_EXP, DXH_CHAIN_LOG                                                       /* f(lhs) */
+};
+#define DXH_CHAIN_MAX_OPS 8
+#define DXH_CHAIN_MAX_INPUTS 8
+#define DXH_CHAIN_RESULT 16
+typedef struct dxh_chain_op {
+    int32_t code;      /* enum dxh_chain_code */
+    int32_t lhs, rhs;  /* operand references */
+    dxh_scalar scalar;
+    void *out;         /* NULL: not stored */
+} dxh_chain_op;
+DXH_API int dxh_chain(int dtype, const void *const *inputs, int n_inputs, const dxh_chain_op *ops, int n_ops, int64_t n, void *stream);
+
 /* ---- cast: launch_todtype elementwise_miaobyte_basic.cuh:11-16.
  * C[i] = static_cast<dst>(A[i]) (float->int truncates toward zero, saturating at
  * the integer range; float->f16/bf16 rounds RNE).  Same dtype = device copy. */

@@ -23,6 +23,7 @@ class InProc:
         L.dxe_create.restype = C.c_void_p
         L.dxe_destroy.argtypes = [C.c_void_p]
         for name, args in [("dxe_execute", [C.c_void_p, C.c_char_p]), ("dxe_execute_batch", [C.c_void_p, C.c_char_p]), ("dxe_stats", [C.c_void_p]),
+                           ("dxe_fusion_stats", [C.c_void_p]),
                            ("dxe_parse", [C.c_char_p]), ("dxe_match", [C.c_void_p, C.c_char_p]),
                            ("dxe_op_table", [C.c_void_p, C.c_char_p]), ("dxe_typedef_roundtrip", [C.c_char_p]),
                            ("dxe_tensor_yaml", [C.c_void_p, C.c_char_p]), ("dxe_shape_yaml_roundtrip", [C.c_char_p])]:
@@ -32,6 +33,7 @@ class InProc:
         L.dxe_infer_shape.argtypes = [C.c_char_p, C.POINTER(C.c_int), C.c_int, C.POINTER(C.c_int), C.c_int, C.c_int, C.c_char_p, C.c_size_t]
         L.dxe_infer_shape.restype = C.c_size_t
         L.dxe_set_graphs.argtypes = [C.c_void_p, C.c_int]
+        L.dxe_set_fusion.argtypes = [C.c_void_p, C.c_int]
         self.L = L
         self.ex = L.dxe_create()
         assert self.ex
@@ -44,6 +46,11 @@ class InProc:
     def execute(self, line): return self._call(self.L.dxe_execute, self.ex, line.encode())
     def execute_batch(self, lines): return self._call(self.L.dxe_execute_batch, self.ex, "\n".join(lines).encode()).split("\n")
     def set_graphs(self, on): self.L.dxe_set_graphs(self.ex, int(on))
+    def set_fusion(self, on): self.L.dxe_set_fusion(self.ex, int(on))
+
+    def fusion_stats(self):
+        runs, lines = (int(x) for x in self._call(self.L.dxe_fusion_stats, self.ex).split())
+        return {"runs": runs, "lines": lines}
 
     def stats(self):
         b, c, r, j = (int(x) for x in self._call(self.L.dxe_stats, self.ex).split())

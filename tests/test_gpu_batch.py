@@ -5,6 +5,8 @@ synchronisations between the replays."""
 import numpy as np
 import pytest
 
+from deepx_amd import lib as dx
+from tests import helpers as H
 from tests.executor_client import InProc, UdpExecutor, read_tensor, write_tensor
 
 pytestmark = pytest.mark.gpu
@@ -80,6 +82,7 @@ def test_batch_equals_line_by_line(tmp_path):
     for n in NAMES[2:]:
         assert np.array_equal(h.get("s_" + n).view(np.uint32), want[n].view(np.uint32)), n
     assert ex.stats()["captures"] == 0  # graphs are off unless asked for
+    assert ex.fusion_stats() == {"runs": 0, "lines": 0}  # 257 * 129 floats are not a whole number of 16-byte vectors
 
 
 def test_graph_replays_track_new_inputs(tmp_path):
@@ -192,3 +195,125 @@ def test_graphs_over_udp(tmp_path):
     finally:
         srv.close()
     assert srv.proc.returncode == 0
+
+
+def test_fused_runs_equal_line_by_line(tmp_path):
+    """Inside a batch, runs of float elementwise lines over one dtype and size are launched as one
+    kernel.  Bit for bit the tensors of a line-by-line execution, for: a run that is cut by a
+    reduction and by an integer op, an in-place line whose old value an earlier line reads and whose
+    new value a later line reads, bfloat16, a size that is not a whole number of vectors (not
+    fused), a line that fails in the middle (its neighbours still run), and the same batch with
+    fusion switched off."""
+    rng = np.random.default_rng(91)
+    shape = [64, 136]
+    lines = [
+        "add({a}, {b})->({c})", "mulscalar({c}, var<float32>:0.25)->({d})", "sub({d}, {a})->({a})",   # in place: a changes here
+        "mul({a}, {c})->({e})", "exp({e})->({f})",
+        "sum({f}, vector<int32>:[1], var<bool>:true)->({s})",                                          # not elementwise: cuts the run
+        "rdivscalar(var<float32>:1, {s})->({t})", "sqrt({t})->({u})", "log({u})->({v})",               # [64,1] tensors: a run of their own
+        "max({f}, {e})->({g})", "minscalar({g}, var<float32>:1.5)->({h})",
+        "add({i1}, {i2})->({i3})",                                                                     # int32: never fused
+        "div({h}, {b})->({k})", "rsubscalar(var<float32>:2, {k})->({m})",
+    ]
+    big = ["a", "b", "c", "d", "e", "f", "g", "h", "k", "m"]
+    small = ["s", "t", "u", "v"]
+    ints = ["i1", "i2", "i3"]
+
+    def build(ex, prefix, dt):
+        h = Host(ex, tmp_path)
+        for n in big[2:]:
+            h.run(f"newtensor({V(shape)})->({T(prefix + n, dt)})")
+        for n in small:
+            h.run(f"newtensor({V([shape[0], 1])})->({T(prefix + n, dt)})")
+        h.run(f"newtensor({V(shape)})->({T(prefix + 'i3', 'int32')})")
+        return h
+
+    def fill(h, prefix, dt, data):
+        stored = lambda x: x if dt == "float32" else H.to_storage(x.reshape(-1).astype(np.float64), dx.BF16).reshape(x.shape)
+        h.put(prefix + "a", stored(data["a"]), dt)
+        h.put(prefix + "b", stored(data["b"]), dt)
+        h.put(prefix + "i1", data["i1"], "int32")
+        h.put(prefix + "i2", data["i2"], "int32")
+
+    for dt in ("float32", "bfloat16"):
+        data = {"a": rng.uniform(0.5, 1.5, shape).astype(np.float32), "b": rng.uniform(0.5, 1.5, shape).astype(np.float32),
+                "i1": rng.integers(-9, 9, shape).astype(np.int32), "i2": rng.integers(-9, 9, shape).astype(np.int32)}
+        results = {}
+        for mode in ("lines", "fused", "unfused"):
+            ex = InProc()
+            ex.set_fusion(mode == "fused")
+            prefix = f"{mode}_{dt}_"
+            h = build(ex, prefix, dt)
+            fill(h, prefix, dt, data)
+            names = {n: T(prefix + n, "int32" if n in ints else dt) for n in big + small + ints}
+            text = [line.format(**names) + f" // author=miaobyte id={500 + i}" for i, line in enumerate(lines)]
+            if mode == "lines":
+                rs = [ex.execute(t) for t in text]
+            else:
+                rs = ex.execute_batch(text)
+            assert all(r.split(" ")[1].startswith("ok") for r in rs), rs
+            results[mode] = {n: h.get(prefix + n) for n in big + small + ["i3"]}
+            if mode == "fused":
+                # [add mulscalar sub mul exp] [rdivscalar sqrt log] [max minscalar] [div rsubscalar]
+                assert ex.fusion_stats() == {"runs": 4, "lines": 12}, ex.fusion_stats()
+            else:
+                assert ex.fusion_stats() == {"runs": 0, "lines": 0}
+        for n in big + small + ["i3"]:
+            want = results["lines"][n]
+            for mode in ("fused", "unfused"):
+                got = results[mode][n]
+                assert got.dtype == want.dtype and np.array_equal(got.view(np.uint8), want.view(np.uint8)), (dt, mode, n)
+
+    # a length that is not a whole number of 16-byte vectors is left to the separate kernels
+    ex = InProc()
+    h = Host(ex, tmp_path)
+    for n in ("y", "z"):
+        h.run(f"newtensor({V([3, 5])})->({T('odd_' + n)})")
+    x = rng.uniform(-1, 1, [3, 5]).astype(np.float32)
+    h.put("odd_x", x)
+    rs = ex.execute_batch([f"mulscalar({T('odd_x')}, var<float32>:2)->({T('odd_y')}) // id=1", f"exp({T('odd_y')})->({T('odd_z')}) // id=2"])
+    assert all(r.split(" ")[1].startswith("ok") for r in rs) and ex.fusion_stats()["runs"] == 0
+    assert np.array_equal(h.get("odd_z"), np.exp((x * np.float32(2)).astype(np.float32)).astype(np.float32)) or np.allclose(h.get("odd_z"), np.exp(x * 2), rtol=1e-6)
+
+    # a failing line (unknown tensor) between fusable ones: reported on its own, the rest runs
+    ex = InProc()
+    h = Host(ex, tmp_path)
+    for n in ("p", "q", "r"):
+        h.run(f"newtensor({V([8, 16])})->({T('e_' + n)})")
+    x = rng.uniform(-1, 1, [8, 16]).astype(np.float32)
+    h.put("e_x", x)
+    rs = ex.execute_batch([f"addscalar({T('e_x')}, var<float32>:1)->({T('e_p')}) // id=1", f"mulscalar({T('e_p')}, var<float32>:3)->({T('e_q')}) // id=2",
+                           f"add({T('e_q')}, {T('e_missing')})->({T('e_r')}) // id=3", f"sqrt({T('e_q')})->({T('e_r')}) // id=4"])
+    assert [r.split(" ")[1][:2] for r in rs] == ["ok", "ok", "er", "ok"], rs
+    assert np.array_equal(h.get("e_q"), (x + np.float32(1)) * np.float32(3))
+
+
+def test_fused_in_place_run(tmp_path):
+    """The SiLU gate as the front emits it for an in-place activation: five lines rewrite one tensor.
+    As one launch only the last of them stores it; the result equals the line-by-line bits, and the
+    tensors that the run only reads are untouched."""
+    rng = np.random.default_rng(92)
+    shape = [32, 264]
+    g = H.to_storage(rng.standard_normal(shape[0] * shape[1]), dx.BF16).reshape(shape)
+    u = H.to_storage(rng.standard_normal(shape[0] * shape[1]), dx.BF16).reshape(shape)
+    b16 = "bfloat16"
+    outs = {}
+    for mode in ("lines", "fused"):
+        ex = InProc()
+        h = Host(ex, tmp_path)
+        p = mode + "_"
+        h.run(f"newtensor({V(shape)})->({T(p + 'sg', b16)})")
+        h.put(p + "g", g, b16)
+        h.put(p + "u", u, b16)
+        n = lambda name: T(p + name, b16)
+        text = [f"mulscalar({n('g')}, var<float32>:-1)->({n('sg')})", f"exp({n('sg')})->({n('sg')})", f"addscalar({n('sg')}, var<float32>:1)->({n('sg')})",
+                f"rdivscalar(var<float32>:1, {n('sg')})->({n('sg')})", f"mul({n('g')}, {n('sg')})->({n('sg')})", f"mul({n('sg')}, {n('u')})->({n('sg')})"]
+        text = [t + f" // author=miaobyte id={i + 1}" for i, t in enumerate(text)]
+        rs = [ex.execute(t) for t in text] if mode == "lines" else ex.execute_batch(text)
+        assert all(r.split(" ")[1].startswith("ok") for r in rs), rs
+        if mode == "fused":
+            assert ex.fusion_stats() == {"runs": 1, "lines": 6}
+        outs[mode] = {k: h.get(p + k) for k in ("sg", "g", "u")}
+    for k in ("sg", "g", "u"):
+        assert np.array_equal(outs["fused"][k], outs["lines"][k]), k
+    assert np.array_equal(outs["fused"]["g"], g) and np.array_equal(outs["fused"]["u"], u)

@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 MFMA_F32_PEAK_TF = 157.3
 MFMA_F64_PEAK_TF = 78.6
 MFMA_BF16_PEAK_TF = 2500.0  # dense bf16
-REDUCE_ROW_TRAFFIC_BYTES = 268558100
+REDUCE_ROW_TRAFFIC_BYTES = 268585444
 
 
 def main():

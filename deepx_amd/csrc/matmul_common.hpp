@@ -170,6 +170,53 @@ __global__ __launch_bounds__(kBlock) void pad_rows_kernel(const E *__restrict__ 
         *reinterpret_cast<vec_t<E, V> *>(out + i * V) = x;
     }
 }
+// The same for 2-byte elements, whose source chunks start on any 2-byte boundary: a lane reads
+// the aligned dwords that cover its 8 elements (one 16-byte load that only needs 4-byte alignment,
+// plus one dword when the chunk starts in the upper half of a dword) and shifts, instead of eight
+// 2-byte loads.  Only dwords that hold at least one wanted element are read, so no load leaves
+// the pages of the source.
+inline unsigned copy_blocks(int64_t total);
+typedef uint32_t u32x4_a4_t __attribute__((ext_vector_type(4), aligned(4)));
+template <int UNUSED = 0>  // a template only so that the header can define it
+__global__ __launch_bounds__(kBlock) void pad_rows16_kernel(const uint16_t *__restrict__ in, uint16_t *__restrict__ out, int64_t rows_in, int64_t cols_in,
+                                                            int64_t rows_out, int64_t chunks_out, int64_t total) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t ch = i % chunks_out, r = (i / chunks_out) % rows_out, b = i / (chunks_out * rows_out);
+        const int64_t left = cols_in - ch * 8;  // elements of the source row from this chunk on
+        u32x4_t x = {0u, 0u, 0u, 0u};
+        if (r < rows_in && left > 0) {
+            const uint16_t *p = in + (b * rows_in + r) * cols_in + ch * 8;
+            const bool odd = (reinterpret_cast<uintptr_t>(p) & 2) != 0;
+            const uint32_t *q = reinterpret_cast<const uint32_t *>(p - (odd ? 1 : 0));  // the dword that holds p[0]
+            uint32_t d[5] = {0u, 0u, 0u, 0u, 0u};
+            if (left >= 8) {
+                const u32x4_t v = *reinterpret_cast<const u32x4_a4_t *>(q);
+                d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+                if (odd) d[4] = q[4];
+            } else {
+                const int dwords = ((odd ? 1 : 0) + (int)left + 1) / 2;
+#pragma unroll
+                for (int j = 0; j < 5; ++j)
+                    if (j < dwords) d[j] = q[j];
+            }
+            uint32_t o[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                o[j] = odd ? (d[j] >> 16) | (d[j + 1] << 16) : d[j];
+                if (left < 8) o[j] &= (2 * j < left ? 0xffffu : 0u) | (2 * j + 1 < left ? 0xffff0000u : 0u);
+            }
+            x = u32x4_t{o[0], o[1], o[2], o[3]};
+        }
+        *reinterpret_cast<u32x4_t *>(out + i * 8) = x;
+    }
+}
+template <typename E>
+inline void launch_pad_rows(const E *in, E *out, int64_t rows_in, int64_t cols_in, int64_t rows_out, int64_t chunks_out, int64_t total, hipStream_t st) {
+    if constexpr (sizeof(E) == 2)
+        pad_rows16_kernel<0><<<copy_blocks(total), kBlock, 0, st>>>((const uint16_t *)in, (uint16_t *)out, rows_in, cols_in, rows_out, chunks_out, total);
+    else
+        pad_rows_kernel<E><<<copy_blocks(total), kBlock, 0, st>>>(in, out, rows_in, cols_in, rows_out, chunks_out, total);
+}
 // out[r][c] = in[r][c] for c < cols (rows of in hold chunks_in 16-byte chunks)
 template <typename E>
 __global__ __launch_bounds__(kBlock) void unpad_rows_kernel(const E *__restrict__ in, E *__restrict__ out, int64_t cols, int64_t chunks_in, int64_t total) {

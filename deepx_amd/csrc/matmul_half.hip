@@ -418,10 +418,10 @@ int launch_padded(const void *a, const void *b, void *c, int64_t batch, int64_t 
     uint16_t *ap = ws, *bp = ws + a_elems;
     if (!a_as_is) {
         const int64_t total = batch * m * (kp / 8);
-        pad_rows_kernel<uint16_t><<<copy_blocks(total), kBlock, 0, st>>>((const uint16_t *)a, ap, m, k, m, kp / 8, total);
+        launch_pad_rows<uint16_t>((const uint16_t *)a, ap, m, k, m, kp / 8, total, st);
     }
     const int64_t total = batch * kp * (np / 8);
-    pad_rows_kernel<uint16_t><<<copy_blocks(total), kBlock, 0, st>>>((const uint16_t *)b, bp, k, n, kp, np / 8, total);
+    launch_pad_rows<uint16_t>((const uint16_t *)b, bp, k, n, kp, np / 8, total, st);
     const int rc = launch_status();
     return rc != DXH_OK ? rc : launch_mfma<T>(a_as_is ? a : (const void *)ap, bp, c, batch, m, kp, np, st, n);
 }

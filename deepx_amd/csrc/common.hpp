@@ -124,7 +124,7 @@ struct Tuning {
     int64_t matmul_tile = 0;                      // DXH_TUNE_MATMUL_TILE: 0 = chosen per shape
     int64_t matmul_splitk = 0;                    // DXH_TUNE_MATMUL_SPLITK: 0 = chosen per shape, 1 = never, n = n slices
     int64_t nt_load = 0;                          // DXH_TUNE_NT_LOAD: 0 = by op class and size, 1 = always, 2 = never
-    int64_t skinny_per_cu = 2;                    // DXH_TUNE_SKINNY_PER_CU
+    int64_t skinny_per_cu = 1;                    // DXH_TUNE_SKINNY_PER_CU
     int64_t skinny_min_rows = 256;                // DXH_TUNE_SKINNY_MIN_ROWS
     int64_t skinny_half = 0;                      // DXH_TUNE_SKINNY_HALF
     int64_t reduce_fused_finish = 1;              // DXH_TUNE_REDUCE_FUSED_FINISH

@@ -22,7 +22,18 @@ template <> struct skinny_acc<double> { using type = double; };
 __device__ __forceinline__ float fma_acc(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ double fma_acc(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
-template <typename T, int MB, typename TO>
+// AL: N is a multiple of V and B is 16-byte aligned, so row r of B splits into aligned 16-byte
+// pieces that start at the same columns for every r.  Otherwise (any N, B aligned to its element
+// size) the 16-byte grid of row r starts phase(r) = (address of B[r][0] / sizeof(T)) % V elements
+// before column 0, and the loads follow that grid instead of the columns: a k-lane visits rows
+// r = ty + 8 i, whose phase is the same for every i (8 N elements are a whole number of 16-byte
+// pieces), so lane (tx, ty) owns the V columns from c0 - phase(ty) + V tx on, all its loads are
+// aligned, and its accumulators stay with the same columns.  A workgroup then loads 32 pieces per
+// row but answers for 31 V columns, the ones every k-lane covers whatever its phase; the sums over
+// the k-lanes pick each column out of LDS at the k-lane's own offset.  Pieces that stick out of a
+// row (before column 0, past N) bring in neighbouring elements, or bytes just outside the buffer
+// within the same aligned 16 bytes; their sums belong to columns that are never stored.
+template <typename T, int MB, typename TO, bool AL>
 __global__ __launch_bounds__(kBlock) void matmul_skinny_kernel(const T *__restrict__ A, const T *__restrict__ B, TO *__restrict__ out,
                                                                 int M, int K, int N, int S, int chunk) {
     using AT = typename skinny_acc<T>::type;
@@ -33,18 +44,26 @@ __global__ __launch_bounds__(kBlock) void matmul_skinny_kernel(const T *__restri
     const int tx = threadIdx.x % kSkinnyTX, ty = threadIdx.x / kSkinnyTX;
     const int64_t batch = blockIdx.z;
     const int s = blockIdx.y;
-    const int nv = N / V;                       // launcher guarantees N % V == 0
-    const int cv = blockIdx.x * kSkinnyTX + tx;  // vector column of this lane
-    const bool active = cv < nv;
+    const int nv = N / V;                        // AL only
+    const int cv = blockIdx.x * kSkinnyTX + tx;  // AL: vector column of this lane
     A += batch * (int64_t)M * K;
     B += batch * (int64_t)K * N;
     const int k0 = s * chunk, k1 = (k0 + chunk < K) ? k0 + chunk : K;
+    constexpr int kCols = (AL ? kSkinnyTX : kSkinnyTX - 1) * V;  // columns a workgroup answers for
+    auto phase = [&](int y) __attribute__((always_inline)) { return AL ? 0 : (int)((reinterpret_cast<uintptr_t>(B + (int64_t)(k0 + y) * N) / sizeof(T)) % V); };
+    const int c0 = blockIdx.x * kCols;               // !AL: first column of the workgroup
+    const int col0 = c0 - phase(ty) + V * tx;        // !AL: first column of this lane (may be -V + 1 .. -1)
+    const bool active = AL ? cv < nv : col0 < N;
     AT acc[MB][V];
 #pragma unroll
     for (int m = 0; m < MB; ++m)
 #pragma unroll
         for (int v = 0; v < V; ++v) acc[m][v] = AT(0);
     const VT *Bv = reinterpret_cast<const VT *>(B) + cv;
+    auto load_b = [&](int64_t row) __attribute__((always_inline)) -> VT {
+        if constexpr (AL) return Bv[row * nv];
+        else return *reinterpret_cast<const VT *>(B + row * N + col0);
+    };
     for (int kb = k0; kb < k1; kb += kSub) {
         const int len = (kb + kSub < k1) ? kSub : k1 - kb;
         // The first four rows of B are requested before A is staged, so that their latency runs
@@ -54,7 +73,7 @@ __global__ __launch_bounds__(kBlock) void matmul_skinny_kernel(const T *__restri
         const bool batched = active && ty + (U - 1) * kSkinnyTY < len;
         if (batched) {
 #pragma unroll
-            for (int u = 0; u < U; ++u) x[u] = Bv[(int64_t)(kb + ty + u * kSkinnyTY) * nv];
+            for (int u = 0; u < U; ++u) x[u] = load_b(kb + ty + u * kSkinnyTY);
         }
         __syncthreads();  // the previous sub-chunk's A values are no longer read
 #pragma unroll
@@ -77,7 +96,7 @@ __global__ __launch_bounds__(kBlock) void matmul_skinny_kernel(const T *__restri
                 for (; r + STEP + (U - 1) * kSkinnyTY < len; r += STEP) {
                     VT y[U];
 #pragma unroll
-                    for (int u = 0; u < U; ++u) y[u] = Bv[(int64_t)(kb + r + STEP + u * kSkinnyTY) * nv];
+                    for (int u = 0; u < U; ++u) y[u] = load_b(kb + r + STEP + u * kSkinnyTY);
                     use(x, r);
 #pragma unroll
                     for (int u = 0; u < U; ++u) x[u] = y[u];
@@ -86,7 +105,7 @@ __global__ __launch_bounds__(kBlock) void matmul_skinny_kernel(const T *__restri
                 r += STEP;
             }
             for (; r < len; r += kSkinnyTY) {
-                const VT b = Bv[(int64_t)(kb + r) * nv];
+                const VT b = load_b(kb + r);
 #pragma unroll
                 for (int m = 0; m < MB; ++m) {
                     const AT a = a_lds[m * kSub + r];
@@ -101,6 +120,21 @@ __global__ __launch_bounds__(kBlock) void matmul_skinny_kernel(const T *__restri
 #pragma unroll
     for (int m = 0; m < MB; ++m) {
         __syncthreads();
+        if constexpr (!AL) {
+            // red[y][q]: what k-lane y summed for column c0 - phase(y) + q
+#pragma unroll
+            for (int v = 0; v < V; ++v) red[ty * (kSkinnyTX * V) + V * tx + v] = active ? acc[m][v] : AT(0);
+            __syncthreads();
+            const int col = c0 + (int)threadIdx.x;
+            if ((int)threadIdx.x < kCols && col < N && m < M) {
+                AT t = red[threadIdx.x + phase(0)];
+#pragma unroll
+                for (int y = 1; y < kSkinnyTY; ++y) t += red[y * (kSkinnyTX * V) + threadIdx.x + phase(y)];
+                if constexpr (std::is_same_v<TO, AT>) o[(int64_t)m * N + col] = t;
+                else o[(int64_t)m * N + col] = store_acc<TO>(t);
+            }
+            continue;
+        }
 #pragma unroll
         for (int v = 0; v < V; ++v) red[(v * kSkinnyTY + ty) * kSkinnyTX + tx] = acc[m][v];
         __syncthreads();
@@ -117,11 +151,11 @@ __global__ __launch_bounds__(kBlock) void matmul_skinny_kernel(const T *__restri
     }
 }
 
-template <typename T, int MB>
+template <typename T, int MB, bool AL>
 int launch_skinny_mb(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     using AT = typename skinny_acc<T>::type;
     constexpr int V = kVecBytes / (int)sizeof(T);
-    const int64_t ctiles = (n / V + kSkinnyTX - 1) / kSkinnyTX;
+    const int64_t cols = (AL ? kSkinnyTX : kSkinnyTX - 1) * V, ctiles = (n + cols - 1) / cols;
     // slices of K: about `per_cu` workgroups per CU, at least `min_rows` rows per slice, none under capture
     const int64_t per_cu = tuning().skinny_per_cu, min_rows = tuning().skinny_min_rows;
     int64_t S = (per_cu * (int64_t)compute_units() + batch * ctiles - 1) / (batch * ctiles);
@@ -135,13 +169,13 @@ int launch_skinny_mb(const void *a, const void *b, void *c, int64_t batch, int64
     if (ctiles > 0x7fffffff || S > 65535 || batch > 65535) return kNoSkinny;
     const dim3 grid((unsigned)ctiles, (unsigned)S, (unsigned)batch);
     if (S == 1) {
-        matmul_skinny_kernel<T, MB, T><<<grid, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, 1, (int)chunk);
+        matmul_skinny_kernel<T, MB, T, AL><<<grid, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, 1, (int)chunk);
         return launch_status();
     }
     std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
     AT *ws = (AT *)stream_workspace(st, kWorkspaceSplitK, (size_t)(partial * S));
     if (!ws) return kNoSkinny;
-    matmul_skinny_kernel<T, MB, AT><<<grid, kBlock, 0, st>>>((const T *)a, (const T *)b, ws, (int)m, (int)k, (int)n, (int)S, (int)chunk);
+    matmul_skinny_kernel<T, MB, AT, AL><<<grid, kBlock, 0, st>>>((const T *)a, (const T *)b, ws, (int)m, (int)k, (int)n, (int)S, (int)chunk);
     const int rc = launch_status();
     return rc != DXH_OK ? rc : launch_splitk_reduce<AT, T>(ws, (T *)c, batch, m * n, (int)S, st);
 }
@@ -150,11 +184,18 @@ int launch_skinny_mb(const void *a, const void *b, void *c, int64_t batch, int64
 template <typename T>
 int launch_skinny_t(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     constexpr int V = kVecBytes / (int)sizeof(T);
-    if (m > 8 || k < 256 || n % V != 0 || !aligned(b, kVecBytes) || k > 0x7fffffff / 2 || tuning().matmul_tile != 0) return kNoSkinny;
-    if (m == 1) return launch_skinny_mb<T, 1>(a, b, c, batch, m, k, n, st);
-    if (m == 2) return launch_skinny_mb<T, 2>(a, b, c, batch, m, k, n, st);
-    if (m <= 4) return launch_skinny_mb<T, 4>(a, b, c, batch, m, k, n, st);
-    return launch_skinny_mb<T, 8>(a, b, c, batch, m, k, n, st);
+    if (m > 8 || k < 256 || k > 0x7fffffff / 2 || n > 0x7fffffff / 2 || tuning().matmul_tile != 0) return kNoSkinny;
+    if (n % V == 0 && aligned(b, kVecBytes)) {
+        if (m == 1) return launch_skinny_mb<T, 1, true>(a, b, c, batch, m, k, n, st);
+        if (m == 2) return launch_skinny_mb<T, 2, true>(a, b, c, batch, m, k, n, st);
+        if (m <= 4) return launch_skinny_mb<T, 4, true>(a, b, c, batch, m, k, n, st);
+        return launch_skinny_mb<T, 8, true>(a, b, c, batch, m, k, n, st);
+    }
+    if (!aligned(b, sizeof(T))) return kNoSkinny;
+    if (m == 1) return launch_skinny_mb<T, 1, false>(a, b, c, batch, m, k, n, st);
+    if (m == 2) return launch_skinny_mb<T, 2, false>(a, b, c, batch, m, k, n, st);
+    if (m <= 4) return launch_skinny_mb<T, 4, false>(a, b, c, batch, m, k, n, st);
+    return launch_skinny_mb<T, 8, false>(a, b, c, batch, m, k, n, st);
 }
 
 // fp32 and fp64 by default.  The kernel is correct for bf16 / f16 as well (DXH_TUNE_SKINNY_HALF),
@@ -164,8 +205,9 @@ int launch_skinny_t(const void *a, const void *b, void *c, int64_t batch, int64_
 // 19.3 against 28.6 us for one row of [4096,4096], 93 against 153 us for [896,151936] (5.9 TB/s).
 int launch_matmul_skinny(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     switch (dtype) {
-    case DXH_BF16: return tuning().skinny_half ? launch_skinny_t<bf16_t>(a, b, c, batch, m, k, n, st) : kNoSkinny;
-    case DXH_F16: return tuning().skinny_half ? launch_skinny_t<f16_t>(a, b, c, batch, m, k, n, st) : kNoSkinny;
+    // 16-bit types: only where the matrix pipe would first have to copy B into 16-byte rows (or when asked for)
+    case DXH_BF16: return (tuning().skinny_half || n % 8 != 0 || !aligned(b, kVecBytes)) ? launch_skinny_t<bf16_t>(a, b, c, batch, m, k, n, st) : kNoSkinny;
+    case DXH_F16: return (tuning().skinny_half || n % 8 != 0 || !aligned(b, kVecBytes)) ? launch_skinny_t<f16_t>(a, b, c, batch, m, k, n, st) : kNoSkinny;
     case DXH_F32: return launch_skinny_t<float>(a, b, c, batch, m, k, n, st);
     case DXH_F64: return launch_skinny_t<double>(a, b, c, batch, m, k, n, st);
     default: return kNoSkinny;

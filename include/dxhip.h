@@ -98,7 +98,7 @@ enum dxh_tune_knob {
     DXH_TUNE_NT_LOAD = 7,              /* non-temporal hint on the loads of elementwise / compare / reduce kernels:
                                           0 = by op class and tensor size, 1 = always, 2 = never */
     DXH_TUNE_SKINNY_PER_CU = 8,        /* matmul with at most 8 rows of A (streaming kernel): workgroups per CU that the
-                                          cut of K aims for (default 2) */
+                                          cut of K aims for (default 1) */
     DXH_TUNE_SKINNY_MIN_ROWS = 9,      /* ... and the fewest rows of B per K slice (default 256, at least 8) */
     DXH_TUNE_SKINNY_HALF = 10,         /* 1 = that kernel also for bf16 / f16 (default 0: they stay on the matrix pipe,
                                           which is as fast or faster for them) */

@@ -369,3 +369,42 @@ def _few_rows_cases(dxh, dtype, rng, rel):
     dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
     want = H.to_float(H.to_storage((Ai @ Bi).astype(np.float64).reshape(-1), dtype), dtype)
     assert np.array_equal(H.to_float(dC.get(), dtype), want)
+
+
+@pytest.mark.parametrize("dtype", [dx.F32, dx.F64, dx.BF16, dx.F16])
+def test_matmul_few_rows_any_n(dxh, dtype):
+    """At most 8 rows and an N that is not a multiple of the 16-byte vector (rows of B then start
+    on any element boundary), bases off a 16-byte boundary, N below one workgroup's width and a K
+    of several slices: float64 numpy reference, exact on small integers, runs bit-identical, and
+    nothing written past the end of C."""
+    rng = np.random.default_rng(1200 + dtype)
+    rel = {dx.F32: 1e-5, dx.F64: 1e-13, dx.BF16: 1e-2, dx.F16: 1e-2}[dtype]
+    npd = H.NP[dtype]
+    for batch, m, k, n, off in [(1, 1, 768, 50257, 0), (2, 3, 1000, 263, 0), (1, 8, 300, 9, 0), (1, 5, 257, 1041, 1), (1, 4, 70000, 67, 0),
+                                (3, 2, 256, 4097, 3), (1, 7, 2048, 4863, 0), (1, 1, 4096, 5, 1)]:
+        A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
+        B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
+        guard = 64
+        dA = Dev(np.concatenate([np.zeros(off, npd), A]))
+        dB = Dev(np.concatenate([np.zeros(off, npd), B]))
+        outs = []
+        seven = H.to_storage(np.full(1, 7.0), dtype)[0]
+        for _ in range(2):
+            dC = Dev(np.full(off + batch * m * n + guard, seven, npd))
+            es = np.dtype(npd).itemsize
+            dx.check(dxh.dxh_matmul(dtype, dA.ptr.value + es * off, dB.ptr.value + es * off, dC.ptr.value + es * off, batch, m, k, n, None), "matmul")
+            outs.append(dC.get())
+        assert np.array_equal(outs[0], outs[1]), "result varies between runs"
+        assert np.all(outs[0][:off] == seven) and np.all(outs[0][off + batch * m * n:] == seven), "wrote outside C"
+        got = H.to_float(outs[0][off:off + batch * m * n], dtype).astype(np.float64).reshape(batch, m, n)
+        ref, mag = _ref_product(A, B, dtype, batch, m, k, n)
+        scale = np.sqrt(k) if dtype in (dx.F32, dx.F64) else 1.0
+        assert np.all(np.abs(got - ref) <= rel * scale * np.maximum(mag, 1e-300)), (dtype, batch, m, k, n, off)
+    m, k, n = 6, 1500, 137
+    Ai, Bi = rng.integers(-4, 5, (m, k)), rng.integers(-4, 5, (k, n))
+    A = H.to_storage(Ai.astype(np.float64).reshape(-1), dtype)
+    B = H.to_storage(Bi.astype(np.float64).reshape(-1), dtype)
+    dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, npd)
+    dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+    want = H.to_float(H.to_storage((Ai @ Bi).astype(np.float64).reshape(-1), dtype), dtype)
+    assert np.array_equal(H.to_float(dC.get(), dtype), want)

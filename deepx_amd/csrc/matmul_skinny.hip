@@ -5,7 +5,7 @@
 //   C[m][n] = sum_k A[m][k] B[k][n],  m < MB <= 8
 //   workgroup  32 column-lanes x 8 k-lanes; a column-lane owns V = 16 / sizeof(T) adjacent columns
 //              (one 16-byte load per row of B), so a workgroup reads 512 contiguous bytes per row
-//   K          cut into S slices (grid.y) so that a few workgroups per CU exist; a slice is
+//   K          cut into S slices (grid.y) while there is less than a workgroup per CU; a slice is
 //              walked in sub-chunks of kSub rows whose A values are staged in LDS (every lane of a
 //              k-lane reads the same A[m][k]: an LDS broadcast)
 //   sums       fp32 (fp64 for fp64) fused multiply-adds per lane, the 8 k-lanes are added through
@@ -198,11 +198,12 @@ int launch_skinny_t(const void *a, const void *b, void *c, int64_t batch, int64_
     return launch_skinny_mb<T, 8, false>(a, b, c, batch, m, k, n, st);
 }
 
-// fp32 and fp64 by default.  The kernel is correct for bf16 / f16 as well (DXH_TUNE_SKINNY_HALF),
-// but there the 64x64 matrix-pipe tiles over K slices are as
-// fast or faster: one row of [4096,4096] takes 12.3 us against 14.2 here, eight rows 12.7 against
-// 24.4 (eight conversions and multiply-adds per 2-byte element are vector-ALU-bound).  fp32:
-// 19.3 against 28.6 us for one row of [4096,4096], 93 against 153 us for [896,151936] (5.9 TB/s).
+// fp32 and fp64 always.  For bf16 / f16 with 16-byte rows of B the 64x64 matrix-pipe tiles over K
+// slices are as fast or faster (one row of [4096,4096] takes 12.3 us against 14.2 here, eight rows
+// 12.7 against 24.4: eight conversions and multiply-adds per 2-byte element are vector-ALU-bound),
+// so they come here only when the matrix pipe would need a padded copy of B first (one row of
+// [768,50257]: 18.5 us against 39.7) or when DXH_TUNE_SKINNY_HALF asks for it.  fp32: 15 against
+// 28.6 us for one row of [4096,4096], 93 against 153 us for [896,151936] (5.9 TB/s).
 int launch_matmul_skinny(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     switch (dtype) {
     // 16-bit types: only where the matrix pipe would first have to copy B into 16-byte rows (or when asked for)

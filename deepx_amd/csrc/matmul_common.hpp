@@ -234,12 +234,16 @@ inline unsigned copy_blocks(int64_t total) {
     const int64_t blocks = (total + kBlock - 1) / kBlock;
     return (unsigned)(blocks > 16384 ? 16384 : blocks);
 }
-// inner(a, b, c, k_padded, n_padded) launches the aligned product on the copies
+// inner(a, b, c, k_padded, n_padded, ldc) launches the aligned product on the copies.  With enough
+// output tiles that the product is never cut along K, C is written straight at its own pitch
+// (ldc = n) and no copy of C exists; a product that may be cut (its partial tiles assume [M][Np])
+// goes through a padded C' (ldc = -1) that is copied out afterwards.
 template <typename E, typename Inner>
 int launch_on_padded_copies(Inner inner, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     constexpr int V = kVecBytes / (int)sizeof(E);
     const int64_t kp = (k + V - 1) / V * V, np = (n + V - 1) / V * V;
-    const int64_t a_elems = (batch * m * kp + V - 1) / V * V, b_elems = batch * kp * np, c_elems = batch * m * np;  // each part starts 16-byte aligned
+    const bool direct = batch * ((m + 127) / 128) * ((np + 127) / 128) * 2 > compute_units() && tuning().matmul_splitk <= 1;
+    const int64_t a_elems = (batch * m * kp + V - 1) / V * V, b_elems = batch * kp * np, c_elems = direct ? 0 : batch * m * np;  // each part starts 16-byte aligned
     const int64_t bytes = (a_elems + b_elems + c_elems) * (int64_t)sizeof(E);
     if (bytes > kWorkspaceMaxBytes || m * n * k < (1 << 16) || stream_is_capturing(st)) return kNoSplit;
     std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
@@ -248,12 +252,13 @@ int launch_on_padded_copies(Inner inner, const void *a, const void *b, void *c, 
     E *ap = ws, *bp = ap + a_elems, *cp = bp + b_elems;
     int64_t total = batch * m * (kp / V);
     const bool a_as_is = k == kp && ((uintptr_t)a % kVecBytes) == 0;  // only B and C have short rows
-    if (!a_as_is) pad_rows_kernel<E><<<copy_blocks(total), kBlock, 0, st>>>((const E *)a, ap, m, k, m, kp / V, total);
+    if (!a_as_is) launch_pad_rows<E>((const E *)a, ap, m, k, m, kp / V, total, st);
     total = batch * kp * (np / V);
-    pad_rows_kernel<E><<<copy_blocks(total), kBlock, 0, st>>>((const E *)b, bp, k, n, kp, np / V, total);
+    launch_pad_rows<E>((const E *)b, bp, k, n, kp, np / V, total, st);
     int rc = launch_status();
     if (rc != DXH_OK) return rc;
-    rc = inner(a_as_is ? a : (const void *)ap, (const void *)bp, (void *)cp, kp, np);
+    if (direct) return inner(a_as_is ? a : (const void *)ap, (const void *)bp, c, kp, np, n);
+    rc = inner(a_as_is ? a : (const void *)ap, (const void *)bp, (void *)cp, kp, np, (int64_t)-1);
     if (rc != DXH_OK) return rc;
     total = batch * m * (np / V);
     unpad_rows_kernel<E><<<copy_blocks(total), kBlock, 0, st>>>(cp, (E *)c, n, np / V, total);

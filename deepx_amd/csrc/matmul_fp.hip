@@ -18,11 +18,15 @@ namespace dxh {
 //          long as both operands use it: MFMA e of lane half h multiplies k = (FK/2) h + e).
 //   B      LDS [FK k][n] as loaded, rows padded by 4 floats; one ds_read_b32 per lane and k.
 //   roles  MFMA on (B^T, A^T): a result lane holds 4 consecutive n of one row m -> 16-byte stores.
+//   MODE   0: element-wise accesses with bounds checks.  1 (VEC): K % 4 == 0, N % 4 == 0 and 16-byte
+//          aligned pointers.  2: A and B as in 1, but C has its own pitch ldc and n_store <= N columns
+//          (B was zero-padded to N columns) and is stored element by element.
 //   VEC    K % 4 == 0, N % 4 == 0 and 16-byte aligned pointers: 16-byte loads and stores with
 //          clamped rows/columns; otherwise element-wise accesses with bounds checks.
-template <int FM, int FN, int FK, int PD, bool VEC>
+template <int FM, int FN, int FK, int PD, int MODE>
 __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float *__restrict__ A, const float *__restrict__ B,
-                                                                    float *__restrict__ C, int M, int lda, int N, TileMap map, KSplit ks) {
+                                                                    float *__restrict__ C, int M, int lda, int N, TileMap map, KSplit ks, int ldc, int n_store) {
+    constexpr bool VEC = MODE != 0, EDGE = MODE == 2;
     constexpr int TM = 64 * FM, TN = 64 * FN, FA_ROW = FK + 4, FB_ROW = TN + 4;
     constexpr int STAGE = TM * FA_ROW + FK * FB_ROW;  // floats
     constexpr int CA = FK / 4, CB = TN / 4;           // 16-byte chunks per A row / B row
@@ -38,7 +42,7 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
     const int slice = tc.batch % ks.splits, kbase = slice * ks.ksub, K = lda - kbase < ks.ksub ? lda - kbase : ks.ksub;
     A += (tc.batch / ks.splits) * (int64_t)M * lda + kbase;
     B += ((tc.batch / ks.splits) * (int64_t)lda + kbase) * N;
-    C += tc.batch * (int64_t)M * N;
+    C += tc.batch * (int64_t)M * ldc;
     const int m0 = tm * TM, n0 = tn * TN;
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
 
@@ -206,7 +210,7 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
         });
     });
     __syncthreads();
-    if constexpr (VEC) {
+    if constexpr (VEC && !EDGE) {
 #pragma unroll
         for (int i = 0; i < TM * CB / kBlock; ++i) {
             const int id = t + kBlock * i, row = id / CB, col = (id % CB) * 4, gm = m0 + row, gn = n0 + col;
@@ -218,7 +222,7 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f32_kernel(const float 
 #pragma unroll 4
         for (int i = 0; i < TM * TN / kBlock; ++i) {
             const int id = t + kBlock * i, row = id / TN, col = id % TN, gm = m0 + row, gn = n0 + col;
-            if (gm < M && gn < N) C[(int64_t)gm * N + gn] = lds[row * LDC + col];
+            if (gm < M && gn < n_store) C[(int64_t)gm * ldc + gn] = lds[row * LDC + col];
         }
     }
 }
@@ -234,7 +238,7 @@ typedef double f64x4 __attribute__((ext_vector_type(4)));
 typedef double f64x2 __attribute__((ext_vector_type(2)));
 template <int FM, int FN, bool VEC>
 __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double *__restrict__ A, const double *__restrict__ B,
-                                                                    double *__restrict__ C, int M, int lda, int N, TileMap map, KSplit ks) {
+                                                                    double *__restrict__ C, int M, int lda, int N, TileMap map, KSplit ks, int ldc, int n_store) {
     constexpr int DK = 16, TM = 64 * FM, TN = 64 * FN, DA_ROW = DK + 2, DB_ROW = TN + 4;
     constexpr int STAGE = TM * DA_ROW + DK * DB_ROW;  // doubles
     constexpr int CA = DK / 2, CB = TN / 2;           // 16-byte chunks per A row / B row
@@ -247,7 +251,7 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double
     const int slice = tc.batch % ks.splits, kbase = slice * ks.ksub, K = lda - kbase < ks.ksub ? lda - kbase : ks.ksub;  // K slice, as in the fp32 kernel
     A += (tc.batch / ks.splits) * (int64_t)M * lda + kbase;
     B += ((tc.batch / ks.splits) * (int64_t)lda + kbase) * N;
-    C += tc.batch * (int64_t)M * N;
+    C += tc.batch * (int64_t)M * ldc;  // ldc = N, n_store = N unless B was zero-padded to N columns for a C of n_store columns
     const int m0 = tm * TM, n0 = tn * TN;
     const int t = threadIdx.x, lane = t & 63, w = t >> 6, wm = w >> 1, wn = w & 1;
 
@@ -401,7 +405,7 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int gm = m0 + wm * 32 * FM + 16 * i + 4 * v + q;
-                if (gm < M && gn < N) __builtin_nontemporal_store(acc[i][j][v], C + (int64_t)gm * N + gn);
+                if (gm < M && gn < n_store) __builtin_nontemporal_store(acc[i][j][v], C + (int64_t)gm * ldc + gn);
             }
         });
     });
@@ -409,10 +413,11 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double
 
 // Launch of one tile shape, cut along K when choose_ksplit says so: the slices then write fp32 /
 // fp64 partial tiles into the stream's workspace and splitk_reduce_kernel adds them up.
+// may_split = false: C has a pitch of its own (the slices' partial tiles and their sum assume [M][N]).
 template <typename T, typename Launch>
-int launch_fp_tile(Launch launch, int tm, int tn, int kstep, int64_t min_k, T *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+int launch_fp_tile(Launch launch, int tm, int tn, int kstep, int64_t min_k, T *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool may_split, hipStream_t st) {
     const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn), partial = batch * m * n * (int64_t)sizeof(T);
-    const KSplit ks = choose_ksplit(tiles, k, kstep, min_k, partial, st);
+    const KSplit ks = may_split ? choose_ksplit(tiles, k, kstep, min_k, partial, st) : KSplit{1, (int)k};
     TileMap map;
     if (!make_tile_map(batch * ks.splits, m, n, tm, tn, map)) return DXH_ERR_SHAPE;
     const unsigned blocks = (unsigned)(8 * map.chunk);
@@ -433,12 +438,14 @@ int launch_fp_tile(Launch launch, int tm, int tn, int kstep, int64_t min_k, T *c
     return rc != DXH_OK ? rc : launch_splitk_reduce<T, T>(ws, c, batch, m * n, ks.splits, st);
 }
 
+// ldc < 0: C is [M][N].  ldc >= 0 (vec only): C has ldc columns at pitch ldc, B was zero-padded to N columns.
 template <int FM, int FN, int FK, int PD>
-int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, hipStream_t st) {
+int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, int64_t ldc, hipStream_t st) {
     return launch_fp_tile<float>([&](unsigned blocks, float *out, const TileMap &map, KSplit ks) {
-        if (vec) matmul_mfma_f32_kernel<FM, FN, FK, PD, true><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks);
-        else matmul_mfma_f32_kernel<FM, FN, FK, PD, false><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks);
-    }, 64 * FM, 64 * FN, FK, 1024, c, batch, m, k, n, st);
+        if (ldc >= 0) matmul_mfma_f32_kernel<FM, FN, FK, PD, 2><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks, (int)ldc, (int)ldc);
+        else if (vec) matmul_mfma_f32_kernel<FM, FN, FK, PD, 1><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
+        else matmul_mfma_f32_kernel<FM, FN, FK, PD, 0><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
+    }, 64 * FM, 64 * FN, FK, 1024, c, batch, m, k, n, ldc < 0, st);
 }
 
 // fp32: the matrix pipe is the bound, so the tile is chosen for CU balance.  Cost model per tile
@@ -448,8 +455,14 @@ int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int
 // leaves at most one workgroup per CU counts 0.5 (a lone workgroup has the matrix pipe to itself).
 // Small tiles take longer K steps and a deeper prefetch: with few MFMAs per step only that hides
 // the global-load latency.
+static int launch_matmul_f32_at(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st);
 int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    const bool vec = k % 4 == 0 && n % 4 == 0 && n >= 4 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && aligned(c, kVecBytes);
+    return launch_matmul_f32_at(a, b, c, batch, m, k, n, -1, st);
+}
+// ldc >= 0: called on zero-padded copies of A and B; C then has ldc columns at pitch ldc
+static int launch_matmul_f32_at(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st) {
+    const bool vec = k % 4 == 0 && n % 4 == 0 && n >= 4 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && (ldc >= 0 || aligned(c, kVecBytes));
+    if (ldc >= 0 && !vec) return DXH_ERR_ALIGN;
     const int64_t cus = compute_units();
     auto cost = [&](int tm, int tn, double eff) {
         const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn);
@@ -459,7 +472,8 @@ int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int6
     };
     if (!vec && tuning().matmul_tile == 0) {  // odd K / N or unaligned bases: the vector path on zero-padded copies
         const int rc = launch_on_padded_copies<uint32_t>(
-            [&](const void *pa, const void *pb, void *pc, int64_t pk, int64_t pn) { return launch_matmul_f32(pa, pb, pc, batch, m, pk, pn, st); }, a, b, c, batch, m, k, n, st);
+            [&](const void *pa, const void *pb, void *pc, int64_t pk, int64_t pn, int64_t pitch) { return launch_matmul_f32_at(pa, pb, pc, batch, m, pk, pn, pitch, st); },
+            a, b, c, batch, m, k, n, st);
         if (rc != kNoSplit) return rc;
     }
     const float *af = (const float *)a, *bf = (const float *)b;
@@ -470,28 +484,34 @@ int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int6
         choice = (c1 <= c2 && c1 <= c3) ? 1 : (c2 <= c3) ? 2 : 3;
     }
     switch (choice) {
-    case 1: return launch_f32_tile<2, 2, 32, 1>(af, bf, cf, batch, m, k, n, vec, st);
-    case 2: return launch_f32_tile<2, 1, 32, 2>(af, bf, cf, batch, m, k, n, vec, st);
-    case 3: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, st);
-    case 4: return launch_f32_tile<2, 2, 16, 1>(af, bf, cf, batch, m, k, n, vec, st);
-    default: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, st);
+    case 1: return launch_f32_tile<2, 2, 32, 1>(af, bf, cf, batch, m, k, n, vec, ldc, st);
+    case 2: return launch_f32_tile<2, 1, 32, 2>(af, bf, cf, batch, m, k, n, vec, ldc, st);
+    case 3: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, ldc, st);
+    case 4: return launch_f32_tile<2, 2, 16, 1>(af, bf, cf, batch, m, k, n, vec, ldc, st);
+    default: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, ldc, st);
     }
 }
 
 template <int FM, int FN>
-int launch_f64_tile(const double *a, const double *b, double *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, hipStream_t st) {
+int launch_f64_tile(const double *a, const double *b, double *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, int64_t ldc, hipStream_t st) {
+    const int pitch = (int)(ldc >= 0 ? ldc : n);
     return launch_fp_tile<double>([&](unsigned blocks, double *out, const TileMap &map, KSplit ks) {
-        if (vec) matmul_mfma_f64_kernel<FM, FN, true><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks);
-        else matmul_mfma_f64_kernel<FM, FN, false><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks);
-    }, 64 * FM, 64 * FN, 16, 512, c, batch, m, k, n, st);
+        if (vec) matmul_mfma_f64_kernel<FM, FN, true><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks, pitch, pitch);
+        else matmul_mfma_f64_kernel<FM, FN, false><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks, pitch, pitch);
+    }, 64 * FM, 64 * FN, 16, 512, c, batch, m, k, n, ldc < 0, st);
 }
 
 // fp64 on the matrix pipe; tile chosen for CU balance with the fp32 cost model (0.116 us per k for
 // a round of 128x64 tiles on 4096^3, 64x64 at 0.94 of that rate per flop).  The 128x128 tile is
 // not chosen: its 128 accumulator registers leave too few for the operand buffers and it runs
 // behind 128x64 on every shape tried; the tuning knob still selects it.
+static int launch_matmul_f64_at(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st);
 int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    return launch_matmul_f64_at(a, b, c, batch, m, k, n, -1, st);
+}
+static int launch_matmul_f64_at(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st) {
     const bool vec = k % 2 == 0 && n % 2 == 0 && n >= 2 && aligned(a, kVecBytes) && aligned(b, kVecBytes);
+    if (ldc >= 0 && !vec) return DXH_ERR_ALIGN;
     const int64_t cus = compute_units();
     auto cost = [&](int tm, int tn, double eff) {
         const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn);
@@ -501,7 +521,8 @@ int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int6
     };
     if (!vec && tuning().matmul_tile == 0) {  // odd K / N or unaligned bases: the vector path on zero-padded copies
         const int rc = launch_on_padded_copies<uint64_t>(
-            [&](const void *pa, const void *pb, void *pc, int64_t pk, int64_t pn) { return launch_matmul_f64(pa, pb, pc, batch, m, pk, pn, st); }, a, b, c, batch, m, k, n, st);
+            [&](const void *pa, const void *pb, void *pc, int64_t pk, int64_t pn, int64_t pitch) { return launch_matmul_f64_at(pa, pb, pc, batch, m, pk, pn, pitch, st); },
+            a, b, c, batch, m, k, n, st);
         if (rc != kNoSplit) return rc;
     }
     const double *af = (const double *)a, *bf = (const double *)b;
@@ -511,9 +532,9 @@ int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int6
         choice = cost(128, 64, 1.0) <= cost(64, 64, 0.941) ? 2 : 3;
     }
     switch (choice) {
-    case 1: return launch_f64_tile<2, 2>(af, bf, cf, batch, m, k, n, vec, st);
-    case 2: return launch_f64_tile<2, 1>(af, bf, cf, batch, m, k, n, vec, st);
-    default: return launch_f64_tile<1, 1>(af, bf, cf, batch, m, k, n, vec, st);
+    case 1: return launch_f64_tile<2, 2>(af, bf, cf, batch, m, k, n, vec, ldc, st);
+    case 2: return launch_f64_tile<2, 1>(af, bf, cf, batch, m, k, n, vec, ldc, st);
+    default: return launch_f64_tile<1, 1>(af, bf, cf, batch, m, k, n, vec, ldc, st);
     }
 }
 

@@ -150,9 +150,9 @@ int launch_splitk_reduce(const TA *ws, TO *out, int64_t batch, int64_t mn, int s
 
 // ---- rows that are not 16-byte aligned (odd K or N, unaligned bases) ---------------------------
 // The matrix-pipe kernels want 16-byte rows.  Such a product runs on zero-padded copies instead: A
-// to [M][Kp], B to [Kp][Np] (Kp, Np the next multiples of 16 bytes), the kernel on those, and the
-// first N columns of its [M][Np] result copied out.  The three copies move each operand once more
-// through HBM, a fraction of what element-wise loads lose (bf16 2047x895x4863: 197 -> 56 us).
+// to [M][Kp], B to [Kp][Np] (Kp, Np the next multiples of 16 bytes) and the kernel on those, which
+// writes its [M][N] result element by element at C's own pitch.  The copies move A and B once more
+// through HBM, a fraction of what element-wise loads lose (bf16 2047x895x4863: 197 -> 42 us).
 // E: unsigned integer of the element size.  kNoSplit: not done (no workspace under graph
 // capture, operands over the workspace limit, tiny products), the caller takes its other path.
 constexpr int kNoSplit = -1001;  // not a DXH_ERR_* value

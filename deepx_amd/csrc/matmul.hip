@@ -212,7 +212,7 @@ extern "C" int dxh_matmul(int dtype, const void *a, const void *b, void *c, int6
     }
     if (!a || !b) return DXH_ERR_ARG;
     if (!aligned(a, es) || !aligned(b, es) || !aligned(c, es)) return DXH_ERR_ALIGN;
-    if (m <= 8) {  // a few rows of A: a stream over B, not matrix-pipe work
+    if (m <= 16) {  // a few rows of A: a stream over B, not matrix-pipe work
         const int rc = launch_matmul_skinny(dtype, a, b, c, batch, m, k, n, st);
         if (rc != kNoSkinny) return rc;
     }

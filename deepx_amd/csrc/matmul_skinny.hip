@@ -39,7 +39,7 @@ __global__ __launch_bounds__(kBlock) void matmul_skinny_kernel(const T *__restri
     using AT = typename skinny_acc<T>::type;
     constexpr int V = kVecBytes / (int)sizeof(T);
     using VT = vec_t<T, V>;
-    __shared__ AT a_lds[MB * kSub];
+    __shared__ __attribute__((aligned(16))) AT a_lds[MB * kSub];  // [row of the sub-chunk][m]: the MB values of a row are one or a few 16-byte reads
     __shared__ AT red[kBlock * V];
     const int tx = threadIdx.x % kSkinnyTX, ty = threadIdx.x / kSkinnyTX;
     const int64_t batch = blockIdx.z;
@@ -78,18 +78,20 @@ __global__ __launch_bounds__(kBlock) void matmul_skinny_kernel(const T *__restri
         __syncthreads();  // the previous sub-chunk's A values are no longer read
 #pragma unroll
         for (int m = 0; m < MB; ++m)
-            for (int r = threadIdx.x; r < len; r += kBlock) a_lds[m * kSub + r] = (m < M) ? AT(load_acc(A[(int64_t)m * K + kb + r])) : AT(0);
+            for (int r = threadIdx.x; r < len; r += kBlock) a_lds[r * MB + m] = (m < M) ? AT(load_acc(A[(int64_t)m * K + kb + r])) : AT(0);
         __syncthreads();
         if (active) {
             auto use = [&](const VT(&b)[U], int r) __attribute__((always_inline)) {
 #pragma unroll
-                for (int u = 0; u < U; ++u)
+                for (int u = 0; u < U; ++u) {
+                    AT a[MB];
 #pragma unroll
-                    for (int m = 0; m < MB; ++m) {
-                        const AT a = a_lds[m * kSub + r + u * kSkinnyTY];
+                    for (int m = 0; m < MB; ++m) a[m] = a_lds[(r + u * kSkinnyTY) * MB + m];
 #pragma unroll
-                        for (int v = 0; v < V; ++v) acc[m][v] = fma_acc(a, AT(load_acc(b[u].v[v])), acc[m][v]);
-                    }
+                    for (int m = 0; m < MB; ++m)
+#pragma unroll
+                        for (int v = 0; v < V; ++v) acc[m][v] = fma_acc(a[m], AT(load_acc(b[u].v[v])), acc[m][v]);
+                }
             };
             int r = ty;
             if (batched) {
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(kBlock) void matmul_skinny_kernel(const T *__restri
                 const VT b = load_b(kb + r);
 #pragma unroll
                 for (int m = 0; m < MB; ++m) {
-                    const AT a = a_lds[m * kSub + r];
+                    const AT a = a_lds[r * MB + m];
 #pragma unroll
                     for (int v = 0; v < V; ++v) acc[m][v] = fma_acc(a, AT(load_acc(b.v[v])), acc[m][v]);
                 }
@@ -184,18 +186,24 @@ int launch_skinny_mb(const void *a, const void *b, void *c, int64_t batch, int64
 template <typename T>
 int launch_skinny_t(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     constexpr int V = kVecBytes / (int)sizeof(T);
-    if (m > 8 || k < 256 || k > 0x7fffffff / 2 || n > 0x7fffffff / 2 || tuning().matmul_tile != 0) return kNoSkinny;
+    // 9..16 rows only for fp32 / fp64 whose rows of B are not 16-byte pieces, where the matrix pipe would need a
+    // padded copy of B first (fp32 12x4096x4097: 43 us there, 30 here); 16-bit types: the conversions make that many rows vector-ALU-bound
+    constexpr int kMaxRows = sizeof(T) >= 4 ? 16 : 8;
+    if (m > kMaxRows || k < 256 || k > 0x7fffffff / 2 || n > 0x7fffffff / 2 || tuning().matmul_tile != 0) return kNoSkinny;
     if (n % V == 0 && aligned(b, kVecBytes)) {
         if (m == 1) return launch_skinny_mb<T, 1, true>(a, b, c, batch, m, k, n, st);
         if (m == 2) return launch_skinny_mb<T, 2, true>(a, b, c, batch, m, k, n, st);
         if (m <= 4) return launch_skinny_mb<T, 4, true>(a, b, c, batch, m, k, n, st);
-        return launch_skinny_mb<T, 8, true>(a, b, c, batch, m, k, n, st);
+        if (m <= 8) return launch_skinny_mb<T, 8, true>(a, b, c, batch, m, k, n, st);
+        return kNoSkinny;  // 9..16 rows of 16-byte rows: the matrix pipe is as fast (fp32 16x4096x4096: 29.8 us there, 33.8 here)
     }
     if (!aligned(b, sizeof(T))) return kNoSkinny;
     if (m == 1) return launch_skinny_mb<T, 1, false>(a, b, c, batch, m, k, n, st);
     if (m == 2) return launch_skinny_mb<T, 2, false>(a, b, c, batch, m, k, n, st);
     if (m <= 4) return launch_skinny_mb<T, 4, false>(a, b, c, batch, m, k, n, st);
-    return launch_skinny_mb<T, 8, false>(a, b, c, batch, m, k, n, st);
+    if (m <= 8) return launch_skinny_mb<T, 8, false>(a, b, c, batch, m, k, n, st);
+    if constexpr (kMaxRows == 16) return launch_skinny_mb<T, 16, false>(a, b, c, batch, m, k, n, st);
+    return kNoSkinny;
 }
 
 // fp32 and fp64 always.  For bf16 / f16 with 16-byte rows of B the 64x64 matrix-pipe tiles over K

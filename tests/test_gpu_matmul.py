@@ -381,7 +381,7 @@ def test_matmul_few_rows_any_n(dxh, dtype):
     rel = {dx.F32: 1e-5, dx.F64: 1e-13, dx.BF16: 1e-2, dx.F16: 1e-2}[dtype]
     npd = H.NP[dtype]
     for batch, m, k, n, off in [(1, 1, 768, 50257, 0), (2, 3, 1000, 263, 0), (1, 8, 300, 9, 0), (1, 5, 257, 1041, 1), (1, 4, 70000, 67, 0),
-                                (3, 2, 256, 4097, 3), (1, 7, 2048, 4863, 0), (1, 1, 4096, 5, 1)]:
+                                (3, 2, 256, 4097, 3), (1, 7, 2048, 4863, 0), (1, 1, 4096, 5, 1), (1, 13, 1024, 1001, 0), (2, 16, 512, 127, 1)]:
         A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
         B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
         guard = 64

@@ -43,6 +43,21 @@ def test_argument_errors_need_no_gpu():
     assert L.dxh_reduce_workspace_bytes(dx.F32, dx.i32arr([8192, 8192]), 2, dx.i32arr([0]), 1, C.byref(n)) == 0 and n.value > 0
     assert L.dxh_reduce_workspace_bytes(dx.F32, dx.i32arr([8192, 8192]), 2, dx.i32arr([2]), 1, C.byref(n)) == -2
     assert L.dxh_matmul(dx.BOOL, None, None, None, 1, 2, 2, 2, None) == -1
+    # dxh_chain: operand references, op codes, counts, alignment and dtype are checked on the host
+    ins = (C.c_void_p * 2)(16, 32)
+    op = lambda code, lhs, rhs, out: dx.ChainOp(code, lhs, rhs, dx.scalar(1.0), out)
+    one = (dx.ChainOp * 1)(op(0, 0, 1, 48))
+    assert L.dxh_chain(dx.F32, ins, 2, one, 1, 0, None) == 0            # nothing to do
+    assert L.dxh_chain(dx.F32, ins, 2, one, 0, 8, None) == -2           # no ops
+    assert L.dxh_chain(dx.F32, ins, 2, one, 9, 8, None) == -2           # too many ops
+    assert L.dxh_chain(dx.I32, ins, 2, one, 1, 8, None) == -1           # float dtypes only
+    assert L.dxh_chain(dx.F32, ins, 2, one, 1, 7, None) == -5           # not a whole number of vectors
+    assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(0, 0, 2, 48)), 1, 8, None) == -2    # input 2 does not exist
+    assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(0, 0, dx.CHAIN_RESULT, 48)), 1, 8, None) == -2  # its own result
+    assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(17, 0, 1, 48)), 1, 8, None) == -2   # unknown op code
+    assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(0, 0, 1, 50)), 1, 8, None) == -5    # output off a 16-byte boundary
+    assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(0, 0, 1, None)), 1, 8, None) == -2  # the last op must store
+    assert len(dx.CHAIN_CODES) == 17 and dx.CHAIN_CODES[16] == "log"
 
 
 def test_tuning_knobs_validate_their_values():

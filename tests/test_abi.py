@@ -91,3 +91,13 @@ def test_tuning_knobs_validate_their_values():
     finally:
         for name, v in defaults.items():
             assert L.dxh_tune(knobs[name], v) == 0
+
+
+def test_chain_codes_follow_the_header():
+    """The op codes of dxh_chain are positional: the binding's list must be the header's enum, in order."""
+    text = open(os.path.join(ROOT, "include", "dxhip.h")).read()
+    body = text[text.index("enum dxh_chain_code {"):]
+    body = re.sub(r"/\*.*?\*/", "", body[:body.index("};")], flags=re.S)
+    names = re.findall(r"DXH_CHAIN_(\w+)", body)
+    assert [n.lower() for n in names] == dx.CHAIN_CODES
+    assert int(re.search(r"#define DXH_CHAIN_RESULT (\d+)", text).group(1)) == dx.CHAIN_RESULT

@@ -253,7 +253,8 @@ __global__ __launch_bounds__(kBlock) void reduce_col_kernel(const Tin *__restric
 // tiles as before; `cnt[p * ctiles + ct]` counts the workgroups of output tile (p, ct) that have
 // stored theirs.  The partials are stored and loaded with device-scope accesses (written through
 // to memory, read past the reader's own L2: the workgroups of a tile run on different XCDs), and
-// the barrier before the count waits until this workgroup's stores have completed.  A release /
+// every lane waits for the acknowledgement of its stores (s_waitcnt vmcnt(0)) before the barrier
+// that precedes the count.  A release /
 // acquire pair on the counter would do the same by writing back and invalidating whole L2s once
 // per workgroup, which cost 30 us of 45 on [8192,8192].  The workgroup that arrives last adds the
 // partials in an order fixed by the launch shape, so the result does not depend on which one it
@@ -266,7 +267,13 @@ __global__ __launch_bounds__(kBlock) void reduce_col_fused_kernel(const Tin *__r
     __shared__ int is_last;
     if (ntl) reduce_col_body<K, Tin, A, TS, V, true, true>(lds, in, part, pre, R, post, S, chunk, TX, ctiles);
     else reduce_col_body<K, Tin, A, TS, V, false, true>(lds, in, part, pre, R, post, S, chunk, TX, ctiles);
-    __syncthreads();  // every store of this workgroup has been acknowledged (the barrier waits on vmcnt)
+    // Every lane waits until its own partial-tile stores have been acknowledged before it enters the
+    // barrier.  They are write-through stores (sc1), whose acknowledgement comes from memory, past
+    // this XCD's L2: once all lanes are through the barrier the whole tile is in memory, so the count
+    // below cannot become visible before the data it announces.  This is the wait an agent-scope
+    // release fence would insert, without that fence's write-back of the whole L2.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
     const int ct = (int)(blockIdx.x % ctiles);
     const int64_t p = blockIdx.x / ctiles / S;
     if (threadIdx.x == 0) {
@@ -278,6 +285,10 @@ __global__ __launch_bounds__(kBlock) void reduce_col_fused_kernel(const Tin *__r
     }
     __syncthreads();
     if (!is_last) return;
+    // The partial tiles are read with device-scope loads (sc1: served from memory, never from a stale
+    // line of this XCD's L2) that are issued after the count was seen; the compiler may not move
+    // them above this point either.
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
     // The S partial tiles are folded like S rows of a col stage: row-lane ty takes slices ty, ty + TY,
     // ... (independent loads, a few in flight), then the same LDS tree across the row-lanes.
     const int TY = kBlock / TX, tx = threadIdx.x % TX, ty = threadIdx.x / TX;

@@ -221,3 +221,30 @@ def test_one_launch_finish_on_two_streams_and_under_capture(dxh):
     dx.check(dxh.dxh_graph_destroy(graph))
     for s in streams:
         dx.check(dxh.dxh_stream_destroy(s))
+
+
+def test_one_launch_finish_many_launches(dxh):
+    """The workgroup that stores a tile's last slice must see every other slice: 2000 launches of the
+    one-launch finish over four shapes and max / min / integer sum (order-independent, so the
+    two-launch path gives the same bits), compared after every launch; stops at the first mismatch."""
+    rng = np.random.default_rng(4242)
+    cases = [("reducemax", dx.F32, (4096, 512), [0]), ("reducemin", dx.F32, (3, 2048, 256), [1]),
+             ("sum", dx.I32, (5000, 1000), [0]), ("reducemax", dx.BF16, (8192, 2048), [0])]
+    prepared = []
+    for name, dtype, shape, dims in cases:
+        a = H.rand(rng, dtype, int(np.prod(shape)))
+        dx.check(dxh.dxh_tune(FUSED_KNOB, 0))
+        try:
+            want, nout = gpu_reduce(dxh, name, dtype, a, shape, dims)
+        finally:
+            dx.check(dxh.dxh_tune(FUSED_KNOB, 1))
+        sh, dm = dx.i32arr(shape), dx.i32arr(dims)
+        wsb = C.c_size_t(0)
+        dx.check(dxh.dxh_reduce_workspace_bytes(dtype, sh, len(shape), dm, len(dims), C.byref(wsb)))
+        assert wsb.value > 0, "the axis must be cut for this test to mean anything"
+        prepared.append((name, dtype, shape, dims, Dev(a), Dev.empty(nout, a.dtype), Dev.empty(wsb.value, np.uint8), wsb.value, want))
+    for it in range(500):
+        for name, dtype, shape, dims, da, out, ws, wsb, want in prepared:
+            _reduce_on(dxh, name, dtype, da, shape, dims, out, ws, wsb, None)
+            got = out.get()
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (it, name, shape)

@@ -197,8 +197,9 @@ int launch_tiled(const void *a, const void *b, void *c, int64_t batch, int64_t m
 
 using namespace dxh;
 
-extern "C" int dxh_matmul(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n,
-                          void *stream) {
+// One dispatcher for the real call and for the workspace query (sc.planning).
+static int matmul_dispatch(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n,
+                           void *stream, Scratch &sc) {
     if (batch < 0 || m < 0 || k < 0 || n < 0) return DXH_ERR_ARG;
     if (m > 0x7fffffff || k > 0x7fffffff || n > 0x7fffffff) return DXH_ERR_SHAPE;
     const int es = dtype_size(dtype);
@@ -207,20 +208,25 @@ extern "C" int dxh_matmul(int dtype, const void *a, const void *b, void *c, int6
     if (!c) return DXH_ERR_ARG;
     hipStream_t st = as_stream(stream);
     if (k == 0) {  // empty sum: a fill kernel rather than a memset node, so the call stays graph-capturable
+        if (sc.planning) return DXH_OK;
         dxh_scalar zero = {0.0, 0};
         return dxh_constant(dtype, c, batch * m * n, zero, stream);
     }
     if (!a || !b) return DXH_ERR_ARG;
     if (!aligned(a, es) || !aligned(b, es) || !aligned(c, es)) return DXH_ERR_ALIGN;
     if (m <= 16) {  // a few rows of A: a stream over B, not matrix-pipe work
-        const int rc = launch_matmul_skinny(dtype, a, b, c, batch, m, k, n, st);
+        const int rc = launch_matmul_skinny(dtype, a, b, c, batch, m, k, n, st, sc);
         if (rc != kNoSkinny) return rc;
     }
     switch (dtype) {
     case DXH_BF16:
-    case DXH_F16: return launch_matmul_half(dtype, a, b, c, batch, m, k, n, st);
-    case DXH_F32: return launch_matmul_f32(a, b, c, batch, m, k, n, st);
-    case DXH_F64: return launch_matmul_f64(a, b, c, batch, m, k, n, st);
+    case DXH_F16: return launch_matmul_half(dtype, a, b, c, batch, m, k, n, st, sc);
+    case DXH_F32: return launch_matmul_f32(a, b, c, batch, m, k, n, st, sc);
+    case DXH_F64: return launch_matmul_f64(a, b, c, batch, m, k, n, st, sc);
+    default: break;
+    }
+    if (sc.planning) return DXH_OK;  // the integer kernels need no scratch
+    switch (dtype) {
     case DXH_I64: return launch_tiled<int64_t>(a, b, c, batch, m, k, n, st);
     case DXH_I32: return launch_tiled<int32_t>(a, b, c, batch, m, k, n, st);
     case DXH_I16: return launch_tiled<int16_t>(a, b, c, batch, m, k, n, st);
@@ -231,3 +237,22 @@ extern "C" int dxh_matmul(int dtype, const void *a, const void *b, void *c, int6
     }
 }
 
+extern "C" int dxh_matmul_workspace_bytes(int dtype, const void *a, const void *b, const void *c, int64_t batch, int64_t m,
+                                          int64_t k, int64_t n, size_t *bytes) {
+    if (!bytes) return DXH_ERR_ARG;
+    *bytes = 0;
+    Scratch sc;
+    sc.planning = true;
+    const int rc = matmul_dispatch(dtype, a, b, const_cast<void *>(c), batch, m, k, n, nullptr, sc);
+    if (rc == DXH_OK) *bytes = sc.used;
+    return rc;
+}
+
+extern "C" int dxh_matmul(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n,
+                          void *workspace, size_t workspace_bytes, void *stream) {
+    if (workspace && !aligned(workspace, 256)) return DXH_ERR_WORKSPACE;
+    Scratch sc;
+    sc.base = (char *)workspace;
+    sc.bytes = workspace ? workspace_bytes : 0;
+    return matmul_dispatch(dtype, a, b, c, batch, m, k, n, stream, sc);
+}

@@ -1,7 +1,6 @@
 // matmul_common.hpp — pieces shared by the matrix-pipe GEMM kernels: vector typedefs, compile-time
 // loops, the XCD-aware workgroup -> tile map and the launch-side helpers.
 #pragma once
-#include <mutex>
 #include <utility>
 #include "common.hpp"
 
@@ -84,25 +83,37 @@ inline int compute_units() {
 }
 
 
+// ---- device scratch of one matmul call ---------------------------------------------------------
+// Partial tiles of a product cut along K and zero-padded operand copies live in the caller's
+// workspace (dxh_matmul's `workspace` argument); nothing here allocates.  The launchers carve what
+// they need from it with take().  dxh_matmul_workspace_bytes runs the same launchers in planning
+// mode: every decision is taken as for a real call, take() only adds up, and no kernel is launched.
+struct Scratch {
+    char *base = nullptr;
+    size_t bytes = 0, used = 0;
+    bool planning = false;
+    void *take(size_t n) {
+        n = (n + 255) & ~(size_t)255;
+        const size_t off = used;
+        used += n;
+        if (planning) return reinterpret_cast<void *>((uintptr_t)256);  // aligned, never dereferenced
+        return (base && used <= bytes) ? base + off : nullptr;
+    }
+};
+
 // ---- split-K -------------------------------------------------------------------------------
 // A product with few output tiles and a long K leaves most CUs idle.  Such a product is cut along
 // K into `splits` slices of `ksub` (a multiple of the kernel's K step): the slice of workgroup
-// batch index x is x % splits of batch x / splits, its partial tile goes to a workspace in the
-// accumulator type, laid out [batch][split][M][N], and splitk_reduce_kernel adds the slices in
-// slice order (same result on every run) and rounds once to the output type.  The workspace
-// (stream_workspace, runtime.hip) is a grow-only buffer owned by the library, one per stream, so
-// calls on different streams do not share it; a stream under graph capture never splits, because
-// a recorded pointer would not survive the buffer growing.  Cutting pays for a second launch
-// only when the uncut K loop is long: K >= min_k, slices of at least min_k / 4.
+// batch index x is x % splits of batch x / splits, its partial tile goes to the call's scratch in
+// the accumulator type, laid out [batch][split][M][N], and splitk_reduce_kernel adds the slices in
+// slice order (same result on every run, eager or replayed from a graph) and rounds once to the
+// output type.  Cutting pays for a second launch only when the uncut K loop is long: K >= min_k,
+// slices of at least min_k / 4.
 struct KSplit { int splits, ksub; };
-constexpr int kWorkspaceSplitK = 0, kWorkspacePadded = 1, kWorkspaceKinds = 2;
-constexpr int64_t kWorkspaceMaxBytes = (int64_t)1 << 30;  // 1 GiB of 288: padded copies of a [2048,768]x[768,50257] bf16 product need 283 MB
-void *stream_workspace(hipStream_t st, int kind, size_t bytes);  // nullptr when the allocation fails
-// Held from the workspace request to the last launch that uses it: two host threads that launch on
-// one stream must not interleave their (fill workspace, consume workspace) launch pairs.
-std::recursive_mutex &workspace_launch_mutex();
-void stream_workspace_release(hipStream_t st);
-inline KSplit choose_ksplit(int64_t tiles, int64_t k, int kstep, int64_t min_k, int64_t partial_bytes, hipStream_t st) {
+// No plan asks for more scratch than this: 1 GiB of 288 (padded copies of a [2048,768]x[768,50257]
+// bf16 product need 283 MB); beyond it a product stays uncut / takes the element-wise kernel.
+constexpr int64_t kWorkspaceMaxBytes = (int64_t)1 << 30;
+inline KSplit choose_ksplit(int64_t tiles, int64_t k, int kstep, int64_t min_k, int64_t partial_bytes) {
     KSplit r{1, (int)k};
     const int64_t cus = compute_units(), ksteps = (k + kstep - 1) / kstep, knob = tuning().matmul_splitk;
     int64_t want;
@@ -116,7 +127,7 @@ inline KSplit choose_ksplit(int64_t tiles, int64_t k, int kstep, int64_t min_k, 
     }
     if (want > ksteps) want = ksteps;
     if (want > 1024) want = 1024;
-    if (want < 2 || want * partial_bytes > kWorkspaceMaxBytes || stream_is_capturing(st)) return r;
+    if (want < 2 || want * partial_bytes > kWorkspaceMaxBytes) return r;
     const int64_t per = (ksteps + want - 1) / want;
     r.ksub = (int)(per * kstep);
     r.splits = (int)((k + r.ksub - 1) / r.ksub);
@@ -153,8 +164,8 @@ int launch_splitk_reduce(const TA *ws, TO *out, int64_t batch, int64_t mn, int s
 // to [M][Kp], B to [Kp][Np] (Kp, Np the next multiples of 16 bytes) and the kernel on those, which
 // writes its [M][N] result element by element at C's own pitch.  The copies move A and B once more
 // through HBM, a fraction of what element-wise loads lose (bf16 2047x895x4863: 197 -> 42 us).
-// E: unsigned integer of the element size.  kNoSplit: not done (no workspace under graph
-// capture, operands over the workspace limit, tiny products), the caller takes its other path.
+// E: unsigned integer of the element size.  kNoSplit: not done (operands over the scratch
+// limit, tiny products), the caller takes its other path.
 constexpr int kNoSplit = -1001;  // not a DXH_ERR_* value
 // out[b][r][c] = (r < rows_in && c < cols_in) ? in[b][r][c] : 0, one 16-byte chunk of out per lane
 template <typename E>
@@ -239,27 +250,29 @@ inline unsigned copy_blocks(int64_t total) {
 // (ldc = n) and no copy of C exists; a product that may be cut (its partial tiles assume [M][Np])
 // goes through a padded C' (ldc = -1) that is copied out afterwards.
 template <typename E, typename Inner>
-int launch_on_padded_copies(Inner inner, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+int launch_on_padded_copies(Inner inner, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc) {
     constexpr int V = kVecBytes / (int)sizeof(E);
     const int64_t kp = (k + V - 1) / V * V, np = (n + V - 1) / V * V;
     const bool direct = batch * ((m + 127) / 128) * ((np + 127) / 128) * 2 > compute_units() && tuning().matmul_splitk <= 1;
     const int64_t a_elems = (batch * m * kp + V - 1) / V * V, b_elems = batch * kp * np, c_elems = direct ? 0 : batch * m * np;  // each part starts 16-byte aligned
     const int64_t bytes = (a_elems + b_elems + c_elems) * (int64_t)sizeof(E);
-    if (bytes > kWorkspaceMaxBytes || m * n * k < (1 << 16) || stream_is_capturing(st)) return kNoSplit;
-    std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
-    E *ws = (E *)stream_workspace(st, kWorkspacePadded, (size_t)bytes);
-    if (!ws) return kNoSplit;
+    if (bytes > kWorkspaceMaxBytes || m * n * k < (1 << 16)) return kNoSplit;
+    E *ws = (E *)sc.take((size_t)bytes);
+    if (!ws) return DXH_ERR_WORKSPACE;
     E *ap = ws, *bp = ap + a_elems, *cp = bp + b_elems;
     int64_t total = batch * m * (kp / V);
     const bool a_as_is = k == kp && ((uintptr_t)a % kVecBytes) == 0;  // only B and C have short rows
-    if (!a_as_is) launch_pad_rows<E>((const E *)a, ap, m, k, m, kp / V, total, st);
-    total = batch * kp * (np / V);
-    launch_pad_rows<E>((const E *)b, bp, k, n, kp, np / V, total, st);
-    int rc = launch_status();
-    if (rc != DXH_OK) return rc;
+    int rc = DXH_OK;
+    if (!sc.planning) {
+        if (!a_as_is) launch_pad_rows<E>((const E *)a, ap, m, k, m, kp / V, total, st);
+        total = batch * kp * (np / V);
+        launch_pad_rows<E>((const E *)b, bp, k, n, kp, np / V, total, st);
+        rc = launch_status();
+        if (rc != DXH_OK) return rc;
+    }
     if (direct) return inner(a_as_is ? a : (const void *)ap, (const void *)bp, c, kp, np, n);
     rc = inner(a_as_is ? a : (const void *)ap, (const void *)bp, (void *)cp, kp, np, (int64_t)-1);
-    if (rc != DXH_OK) return rc;
+    if (rc != DXH_OK || sc.planning) return rc;
     total = batch * m * (np / V);
     unpad_rows_kernel<E><<<copy_blocks(total), kBlock, 0, st>>>(cp, (E *)c, n, np / V, total);
     return launch_status();
@@ -268,9 +281,9 @@ int launch_on_padded_copies(Inner inner, const void *a, const void *b, void *c, 
 // entry points of the per-dtype translation units (matmul_half.hip, matmul_fp.hip) and of the
 // few-rows kernel (matmul_skinny.hip; kNoSkinny = not a shape for it)
 constexpr int kNoSkinny = -1002;  // not a DXH_ERR_* value
-int launch_matmul_skinny(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
-int launch_matmul_half(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
-int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
-int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
+int launch_matmul_skinny(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc);
+int launch_matmul_half(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc);
+int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc);
+int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc);
 
 }  // namespace dxh

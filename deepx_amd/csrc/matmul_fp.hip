@@ -412,27 +412,23 @@ __global__ __launch_bounds__(kBlock, 2) void matmul_mfma_f64_kernel(const double
 }
 
 // Launch of one tile shape, cut along K when choose_ksplit says so: the slices then write fp32 /
-// fp64 partial tiles into the stream's workspace and splitk_reduce_kernel adds them up.
+// fp64 partial tiles into the call's scratch and splitk_reduce_kernel adds them up.
 // may_split = false: C has a pitch of its own (the slices' partial tiles and their sum assume [M][N]).
 template <typename T, typename Launch>
-int launch_fp_tile(Launch launch, int tm, int tn, int kstep, int64_t min_k, T *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool may_split, hipStream_t st) {
+int launch_fp_tile(Launch launch, int tm, int tn, int kstep, int64_t min_k, T *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool may_split, hipStream_t st, Scratch &sc) {
     const int64_t tiles = batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn), partial = batch * m * n * (int64_t)sizeof(T);
-    const KSplit ks = may_split ? choose_ksplit(tiles, k, kstep, min_k, partial, st) : KSplit{1, (int)k};
+    const KSplit ks = may_split ? choose_ksplit(tiles, k, kstep, min_k, partial) : KSplit{1, (int)k};
     TileMap map;
     if (!make_tile_map(batch * ks.splits, m, n, tm, tn, map)) return DXH_ERR_SHAPE;
     const unsigned blocks = (unsigned)(8 * map.chunk);
     if (ks.splits == 1) {
+        if (sc.planning) return DXH_OK;
         launch(blocks, c, map, ks);
         return launch_status();
     }
-    std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
-    T *ws = (T *)stream_workspace(st, kWorkspaceSplitK, (size_t)(partial * ks.splits));
-    if (!ws) {  // no workspace: one slice
-        const KSplit one{1, (int)k};
-        if (!make_tile_map(batch, m, n, tm, tn, map)) return DXH_ERR_SHAPE;
-        launch((unsigned)(8 * map.chunk), c, map, one);
-        return launch_status();
-    }
+    T *ws = (T *)sc.take((size_t)(partial * ks.splits));
+    if (!ws) return DXH_ERR_WORKSPACE;
+    if (sc.planning) return DXH_OK;
     launch(blocks, ws, map, ks);
     const int rc = launch_status();
     return rc != DXH_OK ? rc : launch_splitk_reduce<T, T>(ws, c, batch, m * n, ks.splits, st);
@@ -440,12 +436,12 @@ int launch_fp_tile(Launch launch, int tm, int tn, int kstep, int64_t min_k, T *c
 
 // ldc < 0: C is [M][N].  ldc >= 0 (vec only): C has ldc columns at pitch ldc, B was zero-padded to N columns.
 template <int FM, int FN, int FK, int PD>
-int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, int64_t ldc, hipStream_t st) {
+int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, int64_t ldc, hipStream_t st, Scratch &sc) {
     return launch_fp_tile<float>([&](unsigned blocks, float *out, const TileMap &map, KSplit ks) {
         if (ldc >= 0) matmul_mfma_f32_kernel<FM, FN, FK, PD, 2><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks, (int)ldc, (int)ldc);
         else if (vec) matmul_mfma_f32_kernel<FM, FN, FK, PD, 1><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
         else matmul_mfma_f32_kernel<FM, FN, FK, PD, 0><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
-    }, 64 * FM, 64 * FN, FK, 1024, c, batch, m, k, n, ldc < 0, st);
+    }, 64 * FM, 64 * FN, FK, 1024, c, batch, m, k, n, ldc < 0, st, sc);
 }
 
 // fp32: the matrix pipe is the bound, so the tile is chosen for CU balance.  Cost model per tile
@@ -455,12 +451,12 @@ int launch_f32_tile(const float *a, const float *b, float *c, int64_t batch, int
 // leaves at most one workgroup per CU counts 0.5 (a lone workgroup has the matrix pipe to itself).
 // Small tiles take longer K steps and a deeper prefetch: with few MFMAs per step only that hides
 // the global-load latency.
-static int launch_matmul_f32_at(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st);
-int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    return launch_matmul_f32_at(a, b, c, batch, m, k, n, -1, st);
+static int launch_matmul_f32_at(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st, Scratch &sc);
+int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc) {
+    return launch_matmul_f32_at(a, b, c, batch, m, k, n, -1, st, sc);
 }
 // ldc >= 0: called on zero-padded copies of A and B; C then has ldc columns at pitch ldc
-static int launch_matmul_f32_at(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st) {
+static int launch_matmul_f32_at(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st, Scratch &sc) {
     const bool vec = k % 4 == 0 && n % 4 == 0 && n >= 4 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && (ldc >= 0 || aligned(c, kVecBytes));
     if (ldc >= 0 && !vec) return DXH_ERR_ALIGN;
     const int64_t cus = compute_units();
@@ -472,8 +468,8 @@ static int launch_matmul_f32_at(const void *a, const void *b, void *c, int64_t b
     };
     if (!vec && tuning().matmul_tile == 0) {  // odd K / N or unaligned bases: the vector path on zero-padded copies
         const int rc = launch_on_padded_copies<uint32_t>(
-            [&](const void *pa, const void *pb, void *pc, int64_t pk, int64_t pn, int64_t pitch) { return launch_matmul_f32_at(pa, pb, pc, batch, m, pk, pn, pitch, st); },
-            a, b, c, batch, m, k, n, st);
+            [&](const void *pa, const void *pb, void *pc, int64_t pk, int64_t pn, int64_t pitch) { return launch_matmul_f32_at(pa, pb, pc, batch, m, pk, pn, pitch, st, sc); },
+            a, b, c, batch, m, k, n, st, sc);
         if (rc != kNoSplit) return rc;
     }
     const float *af = (const float *)a, *bf = (const float *)b;
@@ -484,32 +480,32 @@ static int launch_matmul_f32_at(const void *a, const void *b, void *c, int64_t b
         choice = (c1 <= c2 && c1 <= c3) ? 1 : (c2 <= c3) ? 2 : 3;
     }
     switch (choice) {
-    case 1: return launch_f32_tile<2, 2, 32, 1>(af, bf, cf, batch, m, k, n, vec, ldc, st);
-    case 2: return launch_f32_tile<2, 1, 32, 2>(af, bf, cf, batch, m, k, n, vec, ldc, st);
-    case 3: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, ldc, st);
-    case 4: return launch_f32_tile<2, 2, 16, 1>(af, bf, cf, batch, m, k, n, vec, ldc, st);
-    default: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, ldc, st);
+    case 1: return launch_f32_tile<2, 2, 32, 1>(af, bf, cf, batch, m, k, n, vec, ldc, st, sc);
+    case 2: return launch_f32_tile<2, 1, 32, 2>(af, bf, cf, batch, m, k, n, vec, ldc, st, sc);
+    case 3: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, ldc, st, sc);
+    case 4: return launch_f32_tile<2, 2, 16, 1>(af, bf, cf, batch, m, k, n, vec, ldc, st, sc);
+    default: return launch_f32_tile<1, 1, 64, 2>(af, bf, cf, batch, m, k, n, vec, ldc, st, sc);
     }
 }
 
 template <int FM, int FN>
-int launch_f64_tile(const double *a, const double *b, double *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, int64_t ldc, hipStream_t st) {
+int launch_f64_tile(const double *a, const double *b, double *c, int64_t batch, int64_t m, int64_t k, int64_t n, bool vec, int64_t ldc, hipStream_t st, Scratch &sc) {
     const int pitch = (int)(ldc >= 0 ? ldc : n);
     return launch_fp_tile<double>([&](unsigned blocks, double *out, const TileMap &map, KSplit ks) {
         if (vec) matmul_mfma_f64_kernel<FM, FN, true><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks, pitch, pitch);
         else matmul_mfma_f64_kernel<FM, FN, false><<<blocks, kBlock, 0, st>>>(a, b, out, (int)m, (int)k, (int)n, map, ks, pitch, pitch);
-    }, 64 * FM, 64 * FN, 16, 512, c, batch, m, k, n, ldc < 0, st);
+    }, 64 * FM, 64 * FN, 16, 512, c, batch, m, k, n, ldc < 0, st, sc);
 }
 
 // fp64 on the matrix pipe; tile chosen for CU balance with the fp32 cost model (0.116 us per k for
 // a round of 128x64 tiles on 4096^3, 64x64 at 0.94 of that rate per flop).  The 128x128 tile is
 // not chosen: its 128 accumulator registers leave too few for the operand buffers and it runs
 // behind 128x64 on every shape tried; the tuning knob still selects it.
-static int launch_matmul_f64_at(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st);
-int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    return launch_matmul_f64_at(a, b, c, batch, m, k, n, -1, st);
+static int launch_matmul_f64_at(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st, Scratch &sc);
+int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc) {
+    return launch_matmul_f64_at(a, b, c, batch, m, k, n, -1, st, sc);
 }
-static int launch_matmul_f64_at(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st) {
+static int launch_matmul_f64_at(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st, Scratch &sc) {
     const bool vec = k % 2 == 0 && n % 2 == 0 && n >= 2 && aligned(a, kVecBytes) && aligned(b, kVecBytes);
     if (ldc >= 0 && !vec) return DXH_ERR_ALIGN;
     const int64_t cus = compute_units();
@@ -521,8 +517,8 @@ static int launch_matmul_f64_at(const void *a, const void *b, void *c, int64_t b
     };
     if (!vec && tuning().matmul_tile == 0) {  // odd K / N or unaligned bases: the vector path on zero-padded copies
         const int rc = launch_on_padded_copies<uint64_t>(
-            [&](const void *pa, const void *pb, void *pc, int64_t pk, int64_t pn, int64_t pitch) { return launch_matmul_f64_at(pa, pb, pc, batch, m, pk, pn, pitch, st); },
-            a, b, c, batch, m, k, n, st);
+            [&](const void *pa, const void *pb, void *pc, int64_t pk, int64_t pn, int64_t pitch) { return launch_matmul_f64_at(pa, pb, pc, batch, m, pk, pn, pitch, st, sc); },
+            a, b, c, batch, m, k, n, st, sc);
         if (rc != kNoSplit) return rc;
     }
     const double *af = (const double *)a, *bf = (const double *)b;
@@ -532,9 +528,9 @@ static int launch_matmul_f64_at(const void *a, const void *b, void *c, int64_t b
         choice = cost(128, 64, 1.0) <= cost(64, 64, 0.941) ? 2 : 3;
     }
     switch (choice) {
-    case 1: return launch_f64_tile<2, 2>(af, bf, cf, batch, m, k, n, vec, ldc, st);
-    case 2: return launch_f64_tile<2, 1>(af, bf, cf, batch, m, k, n, vec, ldc, st);
-    default: return launch_f64_tile<1, 1>(af, bf, cf, batch, m, k, n, vec, ldc, st);
+    case 1: return launch_f64_tile<2, 2>(af, bf, cf, batch, m, k, n, vec, ldc, st, sc);
+    case 2: return launch_f64_tile<2, 1>(af, bf, cf, batch, m, k, n, vec, ldc, st, sc);
+    default: return launch_f64_tile<1, 1>(af, bf, cf, batch, m, k, n, vec, ldc, st, sc);
     }
 }
 

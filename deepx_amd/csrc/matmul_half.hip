@@ -2,8 +2,8 @@
 // accumulate, one RNE rounding of C).  Aligned shapes (K % 8 == 0, N % 8 == 0) take
 // matmul_mfma_tile_kernel, 64x64 to 256x256 workgroup tiles, software-pipelined over K, cut along
 // K when the output has few tiles; other shapes run the same kernel on zero-padded copies, or,
-// when no workspace may be used, matmul_mfma_kernel, a plain 128x128x32 tile with element-wise
-// edge handling.
+// when those would not fit the scratch limit, matmul_mfma_kernel, a plain 128x128x32 tile with
+// element-wise edge handling.
 #include "matmul_common.hpp"
 
 namespace dxh {
@@ -366,7 +366,8 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
 
 // ldc < 0: C is [M][N] and 16-byte aligned.  ldc >= 0 (needs K % 64 == 0): C has pitch ldc and ldc columns.
 template <typename T, int TM, int TN, int PD>
-int launch_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st) {
+int launch_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, hipStream_t st, Scratch &sc) {
+    if (sc.planning) return DXH_OK;  // needs no scratch
     TileMap map;
     if (!make_tile_map(batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
     const KSplit one{1, (int)k};
@@ -379,19 +380,19 @@ int launch_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m,
     return launch_status();
 }
 
-// Few output tiles and a long K: 64x64 tiles over K slices, fp32 partial tiles in the stream's
-// workspace, then one pass that adds the slices in order and rounds once.  Returns kNoSplit when the
+// Few output tiles and a long K: 64x64 tiles over K slices, fp32 partial tiles in the call's
+// scratch, then one pass that adds the slices in order and rounds once.  Returns kNoSplit when the
 // product should not be cut (the caller then launches the ordinary way).
 template <typename T>
-int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc) {
     constexpr int TM = 64, TN = 64, SPD = 1;  // two K steps in flight were measured slower here (64x8192x4096: 21.4 vs 19.0 us)
     const int64_t tiles = batch * ((m + TM - 1) / TM) * ((n + TN - 1) / TN), partial = batch * m * n * (int64_t)sizeof(float);
-    const KSplit ks = choose_ksplit(tiles, k, PK, 2048, partial, st);
+    const KSplit ks = choose_ksplit(tiles, k, PK, 2048, partial);
     TileMap map;
     if (ks.splits < 2 || !make_tile_map(batch * ks.splits, m, n, TM, TN, map)) return kNoSplit;
-    std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
-    float *ws = (float *)stream_workspace(st, kWorkspaceSplitK, (size_t)(partial * ks.splits));
-    if (!ws) return kNoSplit;
+    float *ws = (float *)sc.take((size_t)(partial * ks.splits));
+    if (!ws) return DXH_ERR_WORKSPACE;
+    if (sc.planning) return DXH_OK;
     if (k % PK == 0)
         matmul_mfma_tile_kernel<T, TM, TN, SPD, false, 1><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
     else
@@ -401,20 +402,20 @@ int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m
 }
 
 // Rows that are not 16-byte aligned (odd K or N, unaligned bases): A and B are copied, zero-padded
-// to K64 (next multiple of 64) and N8 columns, into the stream's workspace, the tile kernel runs on
+// to K64 (next multiple of 64) and N8 columns, into the call's scratch, the tile kernel runs on
 // the copies and stores C directly at its own pitch, element by element (EDGE).  Returns kNoSplit
-// when that is not possible (graph capture, operands over the workspace limit, tiny products).
-template <typename T> int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, int64_t ldc = -1);
+// when that is not possible (operands over the scratch limit, tiny products).
+template <typename T> int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc, int64_t ldc = -1);
 template <typename T>
-int launch_padded(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+int launch_padded(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc) {
     const int64_t kp = (k + PK - 1) / PK * PK, np = (n + 7) / 8 * 8;
     const bool a_as_is = k == kp && aligned(a, kVecBytes);
     const int64_t a_elems = a_as_is ? 0 : (batch * m * kp + 7) / 8 * 8, b_elems = batch * kp * np;
     const int64_t bytes = (a_elems + b_elems) * 2;
-    if (bytes > kWorkspaceMaxBytes || m * n * k < (1 << 16) || kp > (1 << 22) || np > (1 << 24) || stream_is_capturing(st)) return kNoSplit;
-    std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
-    uint16_t *ws = (uint16_t *)stream_workspace(st, kWorkspacePadded, (size_t)bytes);
-    if (!ws) return kNoSplit;
+    if (bytes > kWorkspaceMaxBytes || m * n * k < (1 << 16) || kp > (1 << 22) || np > (1 << 24)) return kNoSplit;
+    uint16_t *ws = (uint16_t *)sc.take((size_t)bytes);
+    if (!ws) return DXH_ERR_WORKSPACE;
+    if (sc.planning) return DXH_OK;  // the tile kernel on the copies needs no more
     uint16_t *ap = ws, *bp = ws + a_elems;
     if (!a_as_is) {
         const int64_t total = batch * m * (kp / 8);
@@ -423,18 +424,18 @@ int launch_padded(const void *a, const void *b, void *c, int64_t batch, int64_t 
     const int64_t total = batch * kp * (np / 8);
     launch_pad_rows<uint16_t>((const uint16_t *)b, bp, k, n, kp, np / 8, total, st);
     const int rc = launch_status();
-    return rc != DXH_OK ? rc : launch_mfma<T>(a_as_is ? a : (const void *)ap, bp, c, batch, m, kp, np, st, n);
+    return rc != DXH_OK ? rc : launch_mfma<T>(a_as_is ? a : (const void *)ap, bp, c, batch, m, kp, np, st, sc, n);
 }
 
 // ldc >= 0: called by launch_padded on its copies; C then has ldc columns at pitch ldc
 template <typename T>
-int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, int64_t ldc) {
+int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc, int64_t ldc) {
     const bool fast = k % 8 == 0 && n % 8 == 0 && aligned(a, kVecBytes) && aligned(b, kVecBytes) && (ldc >= 0 || aligned(c, kVecBytes)) &&
                       k <= (1 << 22) && n <= (1 << 24);
     int64_t choice = tuning().matmul_tile;
     if (ldc >= 0 && (!fast || k % PK != 0)) return DXH_ERR_ALIGN;  // launch_padded hands over aligned copies only
     if (fast && ldc < 0 && (choice == 0 || choice == 5)) {
-        const int rc = launch_split<T>(a, b, c, batch, m, k, n, st);
+        const int rc = launch_split<T>(a, b, c, batch, m, k, n, st, sc);
         if (rc != kNoSplit) return rc;
     }
     if (fast && choice == 0) {
@@ -468,18 +469,19 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
     }
     if (fast) {
         switch (choice) {
-        case 2: return launch_tile<T, 128, 64, 2>(a, b, c, batch, m, k, n, ldc, st);
-        case 3: return launch_tile<T, 64, 128, 2>(a, b, c, batch, m, k, n, ldc, st);
-        case 4: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st);
-        case 5: return launch_tile<T, 64, 64, 2>(a, b, c, batch, m, k, n, ldc, st);
-        case 6: return launch_tile<T, 192, 256, 1>(a, b, c, batch, m, k, n, ldc, st);
-        default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, ldc, st);
+        case 2: return launch_tile<T, 128, 64, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
+        case 3: return launch_tile<T, 64, 128, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
+        case 4: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
+        case 5: return launch_tile<T, 64, 64, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
+        case 6: return launch_tile<T, 192, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
+        default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         }
     }
     if (!fast && tuning().matmul_tile == 0 && k <= (1 << 22) && n <= (1 << 24)) {
-        const int rc = launch_padded<T>(a, b, c, batch, m, k, n, st);
+        const int rc = launch_padded<T>(a, b, c, batch, m, k, n, st, sc);
         if (rc != kNoSplit) return rc;
     }
+    if (sc.planning) return DXH_OK;
     const int64_t tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
     const int64_t blocks = batch * tiles_m * tiles_n;
     if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
@@ -493,8 +495,8 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
 #undef DXH_MM
     return launch_status();
 }
-int launch_matmul_half(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    return dtype == DXH_BF16 ? launch_mfma<bf16_t>(a, b, c, batch, m, k, n, st) : launch_mfma<f16_t>(a, b, c, batch, m, k, n, st);
+int launch_matmul_half(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc) {
+    return dtype == DXH_BF16 ? launch_mfma<bf16_t>(a, b, c, batch, m, k, n, st, sc) : launch_mfma<f16_t>(a, b, c, batch, m, k, n, st, sc);
 }
 
 }  // namespace dxh

@@ -154,29 +154,30 @@ __global__ __launch_bounds__(kBlock) void matmul_skinny_kernel(const T *__restri
 }
 
 template <typename T, int MB, bool AL>
-int launch_skinny_mb(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+int launch_skinny_mb(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc) {
     using AT = typename skinny_acc<T>::type;
     constexpr int V = kVecBytes / (int)sizeof(T);
     const int64_t cols = (AL ? kSkinnyTX : kSkinnyTX - 1) * V, ctiles = (n + cols - 1) / cols;
-    // slices of K: about `per_cu` workgroups per CU, at least `min_rows` rows per slice, none under capture
+    // slices of K: about `per_cu` workgroups per CU, at least `min_rows` rows per slice
     const int64_t per_cu = tuning().skinny_per_cu, min_rows = tuning().skinny_min_rows;
     int64_t S = (per_cu * (int64_t)compute_units() + batch * ctiles - 1) / (batch * ctiles);
     if (S > k / min_rows) S = k / min_rows;
     if (S < 1 || tuning().matmul_splitk == 1) S = 1;
     const int64_t partial = batch * m * n * (int64_t)sizeof(AT);
-    if (S > 1 && (S * partial > kWorkspaceMaxBytes || stream_is_capturing(st))) S = 1;
+    if (S > 1 && S * partial > kWorkspaceMaxBytes) S = 1;
     int64_t chunk = (k + S - 1) / S;
     chunk = (chunk + kSkinnyTY - 1) / kSkinnyTY * kSkinnyTY;
     S = (k + chunk - 1) / chunk;
     if (ctiles > 0x7fffffff || S > 65535 || batch > 65535) return kNoSkinny;
     const dim3 grid((unsigned)ctiles, (unsigned)S, (unsigned)batch);
     if (S == 1) {
+        if (sc.planning) return DXH_OK;
         matmul_skinny_kernel<T, MB, T, AL><<<grid, kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, 1, (int)chunk);
         return launch_status();
     }
-    std::lock_guard<std::recursive_mutex> hold(workspace_launch_mutex());
-    AT *ws = (AT *)stream_workspace(st, kWorkspaceSplitK, (size_t)(partial * S));
-    if (!ws) return kNoSkinny;
+    AT *ws = (AT *)sc.take((size_t)(partial * S));
+    if (!ws) return DXH_ERR_WORKSPACE;
+    if (sc.planning) return DXH_OK;
     matmul_skinny_kernel<T, MB, AT, AL><<<grid, kBlock, 0, st>>>((const T *)a, (const T *)b, ws, (int)m, (int)k, (int)n, (int)S, (int)chunk);
     const int rc = launch_status();
     return rc != DXH_OK ? rc : launch_splitk_reduce<AT, T>(ws, (T *)c, batch, m * n, (int)S, st);
@@ -184,25 +185,25 @@ int launch_skinny_mb(const void *a, const void *b, void *c, int64_t batch, int64
 
 // Returns kNoSkinny when the shape is not one for this kernel (the caller goes on to the matrix pipe).
 template <typename T>
-int launch_skinny_t(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+int launch_skinny_t(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc) {
     constexpr int V = kVecBytes / (int)sizeof(T);
     // 9..16 rows only for fp32 / fp64 whose rows of B are not 16-byte pieces, where the matrix pipe would need a
     // padded copy of B first (fp32 12x4096x4097: 43 us there, 30 here); 16-bit types: the conversions make that many rows vector-ALU-bound
     constexpr int kMaxRows = sizeof(T) >= 4 ? 16 : 8;
     if (m > kMaxRows || k < 256 || k > 0x7fffffff / 2 || n > 0x7fffffff / 2 || tuning().matmul_tile != 0) return kNoSkinny;
     if (n % V == 0 && aligned(b, kVecBytes)) {
-        if (m == 1) return launch_skinny_mb<T, 1, true>(a, b, c, batch, m, k, n, st);
-        if (m == 2) return launch_skinny_mb<T, 2, true>(a, b, c, batch, m, k, n, st);
-        if (m <= 4) return launch_skinny_mb<T, 4, true>(a, b, c, batch, m, k, n, st);
-        if (m <= 8) return launch_skinny_mb<T, 8, true>(a, b, c, batch, m, k, n, st);
+        if (m == 1) return launch_skinny_mb<T, 1, true>(a, b, c, batch, m, k, n, st, sc);
+        if (m == 2) return launch_skinny_mb<T, 2, true>(a, b, c, batch, m, k, n, st, sc);
+        if (m <= 4) return launch_skinny_mb<T, 4, true>(a, b, c, batch, m, k, n, st, sc);
+        if (m <= 8) return launch_skinny_mb<T, 8, true>(a, b, c, batch, m, k, n, st, sc);
         return kNoSkinny;  // 9..16 rows of 16-byte rows: the matrix pipe is as fast (fp32 16x4096x4096: 29.8 us there, 33.8 here)
     }
     if (!aligned(b, sizeof(T))) return kNoSkinny;
-    if (m == 1) return launch_skinny_mb<T, 1, false>(a, b, c, batch, m, k, n, st);
-    if (m == 2) return launch_skinny_mb<T, 2, false>(a, b, c, batch, m, k, n, st);
-    if (m <= 4) return launch_skinny_mb<T, 4, false>(a, b, c, batch, m, k, n, st);
-    if (m <= 8) return launch_skinny_mb<T, 8, false>(a, b, c, batch, m, k, n, st);
-    if constexpr (kMaxRows == 16) return launch_skinny_mb<T, 16, false>(a, b, c, batch, m, k, n, st);
+    if (m == 1) return launch_skinny_mb<T, 1, false>(a, b, c, batch, m, k, n, st, sc);
+    if (m == 2) return launch_skinny_mb<T, 2, false>(a, b, c, batch, m, k, n, st, sc);
+    if (m <= 4) return launch_skinny_mb<T, 4, false>(a, b, c, batch, m, k, n, st, sc);
+    if (m <= 8) return launch_skinny_mb<T, 8, false>(a, b, c, batch, m, k, n, st, sc);
+    if constexpr (kMaxRows == 16) return launch_skinny_mb<T, 16, false>(a, b, c, batch, m, k, n, st, sc);
     return kNoSkinny;
 }
 
@@ -212,13 +213,13 @@ int launch_skinny_t(const void *a, const void *b, void *c, int64_t batch, int64_
 // so they come here only when the matrix pipe would need a padded copy of B first (one row of
 // [768,50257]: 18.5 us against 39.7) or when DXH_TUNE_SKINNY_HALF asks for it.  fp32: 15 against
 // 28.6 us for one row of [4096,4096], 93 against 153 us for [896,151936] (5.9 TB/s).
-int launch_matmul_skinny(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+int launch_matmul_skinny(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc) {
     switch (dtype) {
     // 16-bit types: only where the matrix pipe would first have to copy B into 16-byte rows (or when asked for)
-    case DXH_BF16: return (tuning().skinny_half || n % 8 != 0 || !aligned(b, kVecBytes)) ? launch_skinny_t<bf16_t>(a, b, c, batch, m, k, n, st) : kNoSkinny;
-    case DXH_F16: return (tuning().skinny_half || n % 8 != 0 || !aligned(b, kVecBytes)) ? launch_skinny_t<f16_t>(a, b, c, batch, m, k, n, st) : kNoSkinny;
-    case DXH_F32: return launch_skinny_t<float>(a, b, c, batch, m, k, n, st);
-    case DXH_F64: return launch_skinny_t<double>(a, b, c, batch, m, k, n, st);
+    case DXH_BF16: return (tuning().skinny_half || n % 8 != 0 || !aligned(b, kVecBytes)) ? launch_skinny_t<bf16_t>(a, b, c, batch, m, k, n, st, sc) : kNoSkinny;
+    case DXH_F16: return (tuning().skinny_half || n % 8 != 0 || !aligned(b, kVecBytes)) ? launch_skinny_t<f16_t>(a, b, c, batch, m, k, n, st, sc) : kNoSkinny;
+    case DXH_F32: return launch_skinny_t<float>(a, b, c, batch, m, k, n, st, sc);
+    case DXH_F64: return launch_skinny_t<double>(a, b, c, batch, m, k, n, st, sc);
     default: return kNoSkinny;
     }
 }

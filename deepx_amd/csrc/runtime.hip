@@ -2,9 +2,6 @@
 // Replaces the cudaMalloc/cudaFree/cudaMemcpy calls of
 // executor/op-cuda/src/deepx/tensorfunc/tensorlife_miaobyte.hpp:16-68.
 #include "matmul_common.hpp"
-#include <map>
-#include <mutex>
-#include <tuple>
 #include <cstdio>
 #include <cstring>
 
@@ -14,45 +11,6 @@ namespace dxh {
 Tuning &tuning() {
     static Tuning t;
     return t;
-}
-}  // namespace dxh
-
-namespace dxh {
-// Grow-only matmul workspaces, one per (device, stream, kind): kernels of one stream run in order,
-// so a buffer per stream is never shared by two products in flight.  Growing frees the old buffer with
-// hipFree, which waits for the device, so work still reading it has finished.
-namespace {
-struct Workspace { void *ptr; size_t bytes; };
-std::mutex g_ws_mutex;
-std::map<std::tuple<int, hipStream_t, int>, Workspace> g_ws;
-}  // namespace
-std::recursive_mutex &workspace_launch_mutex() {
-    static std::recursive_mutex m;
-    return m;
-}
-void *stream_workspace(hipStream_t st, int kind, size_t bytes) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    Workspace &w = g_ws[std::make_tuple(dev, st, kind)];
-    if (w.bytes >= bytes) return w.ptr;
-    void *p = nullptr;
-    if (hipMalloc(&p, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
-    if (w.ptr) (void)hipFree(w.ptr);
-    w.ptr = p;
-    w.bytes = bytes;
-    return p;
-}
-void stream_workspace_release(hipStream_t st) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return; }
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    for (int kind = 0; kind < kWorkspaceKinds; ++kind) {
-        auto it = g_ws.find(std::make_tuple(dev, st, kind));
-        if (it == g_ws.end()) continue;
-        if (it->second.ptr) (void)hipFree(it->second.ptr);
-        g_ws.erase(it);
-    }
 }
 }  // namespace dxh
 
@@ -152,7 +110,6 @@ int dxh_stream_create(void **stream) {
 }
 int dxh_stream_destroy(void *stream) {
     if (!stream) return DXH_OK;
-    dxh::stream_workspace_release(as_stream(stream));
     dxh::reduce_stream_release(as_stream(stream));
     return (int)hipStreamDestroy(as_stream(stream));
 }

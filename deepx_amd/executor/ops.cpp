@@ -543,7 +543,12 @@ int register_all(TfFactory &f) {
         if (want != C->shape.shape) return fail(error, "matmul: output shape " + dims_str(C->shape.shape) + " != " + dims_str(want));
         int64_t batch = 1;
         for (int i = 0; i + 2 < A->shape.dim(); ++i) batch *= A->shape.shape[i];
-        return hip_result(dxh_matmul(A->dtype(), A->data, B->data, C->data, batch, A->shape.at(-2), A->shape.at(-1), B->shape.at(-1), mem.stream), "matmul", error);
+        const int64_t m = A->shape.at(-2), k = A->shape.at(-1), n = B->shape.at(-1);
+        size_t need = 0;
+        int rc = dxh_matmul_workspace_bytes(A->dtype(), A->data, B->data, C->data, batch, m, k, n, &need);
+        if (rc != DXH_OK) return hip_result(rc, "matmul", error);
+        void *ws = need ? mem.workspace(need) : nullptr;
+        return hip_result(dxh_matmul(A->dtype(), A->data, B->data, C->data, batch, m, k, n, ws, need ? mem.workspace_bytes() : 0, mem.stream), "matmul", error);
     };
     for (const char *author : {"cublas", "cblas", "miaobyte"})
         reg(f, "matmul", author, "matmul", "T3=T1 @ T2", {T_ANY ":A", T_ANY ":B"}, {T_ANY ":C"}, matmul);

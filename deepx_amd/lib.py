@@ -115,7 +115,8 @@ SIGNATURES = {
     "dxh_uniform": ([_i, _p, _i64, Scalar, Scalar, C.c_uint32, _p], _i),
     "dxh_normal": ([_i, _p, _i64, Scalar, Scalar, C.c_uint32, _p], _i),
     "dxh_dropout": ([_i, _p, _i64, _f, C.c_uint32, _p], _i),
-    "dxh_matmul": ([_i, _p, _p, _p, _i64, _i64, _i64, _i64, _p], _i),
+    "dxh_matmul_workspace_bytes": ([_i, _p, _p, _p, _i64, _i64, _i64, _i64, C.POINTER(_sz)], _i),
+    "dxh_matmul": ([_i, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz, _p], _i),
 }
 
 _lib = None

@@ -30,9 +30,9 @@
  *    the convention of executor/op-cuda/src/deepx/tensorfunc/cuda_math.cuh:243-251.
  *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls
  *    are asynchronous: they return after enqueueing, like the reference's launches.
- *  - element counts are 64-bit; kernels never allocate.  Entry points that need
- *    device scratch take a caller-provided workspace (size from the matching
- *    *_workspace_bytes query).
+ *  - element counts are 64-bit; no entry point but dxh_malloc allocates device
+ *    memory.  Those that need device scratch (reductions, matmul) take a
+ *    caller-provided workspace, sized by the matching *_workspace_bytes query.
  */
 #ifndef DXHIP_H
 #define DXHIP_H
@@ -316,13 +316,18 @@ DXH_API int dxh_dropout(int dtype, void *inout, int64_t n, float p, uint32_t see
  * the leading dims.  f16/bf16: MFMA with fp32 accumulate, one RNE rounding of the
  * result; f32/f64 accumulate in their own type; integers wrap.  A float product with few
  * output tiles and a long K is cut along K (DXH_TUNE_MATMUL_SPLITK) into partial products that
- * are added in a fixed order; their buffer (at most 1 GiB) belongs to the library, one per
- * stream, allocated on first need and released by dxh_stream_destroy.  On a stream under
- * graph capture no workspace is used (the product is not cut, and bf16/f16 operands with odd K
- * or N take the element-wise kernel instead of padded copies): a recorded float matmul of such a
- * shape can differ from the eager one in summation order, within the same error bound. */
+ * are added in a fixed order, and one whose rows are not 16-byte aligned (odd K or N, unaligned
+ * bases) runs on zero-padded copies of A and B: both live in `workspace`, device memory of the
+ * caller of at least dxh_matmul_workspace_bytes(same arguments) bytes, 256-byte aligned, that
+ * no other call in flight uses; the library allocates nothing.  `workspace` may be NULL when the
+ * query reports 0 (most shapes); a workspace that is too small gives DXH_ERR_WORKSPACE.  The
+ * query only looks at the alignment of a, b, c, never at what they point to.  Which kernels run
+ * depends on the arguments and the tuning knobs alone, so a call recorded under stream capture
+ * gives the bits of the eager call. */
+DXH_API int dxh_matmul_workspace_bytes(int dtype, const void *a, const void *b, const void *c, int64_t batch,
+                                       int64_t m, int64_t k, int64_t n, size_t *bytes);
 DXH_API int dxh_matmul(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m,
-                       int64_t k, int64_t n, void *stream);
+                       int64_t k, int64_t n, void *workspace, size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -41,6 +41,8 @@ def oracle():
             at = list(argtypes)
             if name in ("dxh_sum", "dxh_prod", "dxh_reducemax", "dxh_reducemin"):
                 at = at[:7]
+            elif name == "dxh_matmul":
+                at = at[:8]  # no workspace, no stream
             else:
                 at = at[:-1]  # drop the stream
             fn = getattr(L, oname)
@@ -162,3 +164,25 @@ class Dev:
         torch.cuda.synchronize()
         nbytes = int(np.prod(self.shape)) * np.dtype(self.np_dtype).itemsize
         return self.t[:nbytes].cpu().numpy().view(self.np_dtype).reshape(self.shape).copy()
+
+
+_mm_ws = {}
+
+
+def matmul(dxh, dtype, a, b, c, batch, m, k, n, stream=None):
+    """dxh_matmul with the workspace its own query asks for (one grow-only device buffer per
+    stream, as a caller of the C ABI would keep).  Returns the entry point's return code."""
+    need = C.c_size_t(0)
+    rc = dxh.dxh_matmul_workspace_bytes(dtype, a, b, c, batch, m, k, n, C.byref(need))
+    if rc != 0:
+        return rc
+    ws_ptr, ws_bytes = None, 0
+    if need.value:
+        key = stream.value if isinstance(stream, C.c_void_p) else stream
+        ws = _mm_ws.get(key)
+        if ws is None or ws.shape[0] < need.value:
+            import torch
+            torch.cuda.synchronize()  # work that still uses the old buffer
+            ws = _mm_ws[key] = Dev.empty(max(need.value, 1 << 22), np.uint8)
+        ws_ptr, ws_bytes = ws.ptr, ws.shape[0]
+    return dxh.dxh_matmul(dtype, a, b, c, batch, m, k, n, ws_ptr, ws_bytes, stream)

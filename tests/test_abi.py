@@ -42,7 +42,16 @@ def test_argument_errors_need_no_gpu():
     assert L.dxh_reduce_workspace_bytes(dx.F32, dx.i32arr([8192, 8192]), 2, dx.i32arr([1]), 1, C.byref(n)) == 0 and n.value == 0
     assert L.dxh_reduce_workspace_bytes(dx.F32, dx.i32arr([8192, 8192]), 2, dx.i32arr([0]), 1, C.byref(n)) == 0 and n.value > 0
     assert L.dxh_reduce_workspace_bytes(dx.F32, dx.i32arr([8192, 8192]), 2, dx.i32arr([2]), 1, C.byref(n)) == -2
-    assert L.dxh_matmul(dx.BOOL, None, None, None, 1, 2, 2, 2, None) == -1
+    assert L.dxh_matmul(dx.BOOL, None, None, None, 1, 2, 2, 2, None, 0, None) == -1
+    # the matmul workspace query is host arithmetic: 0 for the BASELINE shapes' first GEMM, partial tiles
+    # for a product cut along K, padded copies for rows that are not 16-byte pieces; it needs no GPU
+    P = lambda v: C.c_void_p(v)
+    assert L.dxh_matmul_workspace_bytes(dx.BF16, P(256), P(512), P(1024), 1, 2048, 896, 4864, C.byref(n)) == 0 and n.value == 0
+    assert L.dxh_matmul_workspace_bytes(dx.F32, P(256), P(512), P(1024), 1, 16, 4096, 256, C.byref(n)) == 0 and n.value >= 2 * 16 * 256 * 4
+    assert L.dxh_matmul_workspace_bytes(dx.BF16, P(256), P(512), P(1024), 1, 333, 777, 555, C.byref(n)) == 0 and n.value >= 832 * 560 * 2
+    assert L.dxh_matmul_workspace_bytes(dx.I32, P(256), P(512), P(1024), 1, 64, 64, 64, C.byref(n)) == 0 and n.value == 0
+    assert L.dxh_matmul_workspace_bytes(dx.BOOL, P(256), P(512), P(1024), 1, 64, 64, 64, C.byref(n)) == -1
+    assert L.dxh_matmul(dx.F32, P(256), P(512), P(1024), 1, 16, 4096, 256, P(100), 1 << 20, None) == -4  # workspace not 256-byte aligned
     # dxh_chain: operand references, op codes, counts, alignment and dtype are checked on the host
     ins = (C.c_void_p * 2)(16, 32)
     op = lambda code, lhs, rhs, out: dx.ChainOp(code, lhs, rhs, dx.scalar(1.0), out)

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 def run(dxh, orc, dtype, A, B, batch, m, k, n):
     dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, A.dtype)
-    dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+    dx.check(H.matmul(dxh, dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
     want = np.empty(batch * m * n, dtype=A.dtype)
     assert orc.orc_matmul(dtype, hp(A), hp(B), hp(want), batch, m, k, n) == 0
     return dC.get(), want
@@ -56,7 +56,7 @@ def test_matmul_reference_known_answer(dxh):
     A = np.arange(24, dtype=np.float32)
     B = np.arange(40, dtype=np.float32)
     dA, dB, dC = Dev(A), Dev(B), Dev.empty(30, np.float32)
-    dx.check(dxh.dxh_matmul(dx.F32, dA.ptr, dB.ptr, dC.ptr, 2, 3, 4, 5, None))
+    dx.check(H.matmul(dxh, dx.F32, dA.ptr, dB.ptr, dC.ptr, 2, 3, 4, 5, None))
     want = np.array([[[70, 76, 82, 88, 94], [190, 212, 234, 256, 278], [310, 348, 386, 424, 462]],
                      [[1510, 1564, 1618, 1672, 1726], [1950, 2020, 2090, 2160, 2230], [2390, 2476, 2562, 2648, 2734]]],
                     dtype=np.float32)
@@ -71,7 +71,7 @@ def test_config5_gemm_shapes_bf16(dxh, orc):
         A = H.f32_to_bf16_bits(rng.standard_normal(m * k).astype(np.float32))
         B = H.f32_to_bf16_bits(np.random.default_rng(seed).standard_normal(k * n).astype(np.float32) * 0.02)
         dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, np.uint16)
-        dx.check(dxh.dxh_matmul(dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+        dx.check(H.matmul(dxh, dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
         got = H.bf16_bits_to_f32(dC.get()).reshape(m, n).astype(np.float64)
         rows = rng.choice(m, 64, replace=False)
         Af = H.bf16_bits_to_f32(A).reshape(m, k).astype(np.float64)[rows]
@@ -99,7 +99,7 @@ def test_matmul_tile_configs(dxh, dtype, tile):
             A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
             B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
             dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, A.dtype)
-            dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+            dx.check(H.matmul(dxh, dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
             got = H.to_float(dC.get(), dtype).astype(np.float64).reshape(batch, m, n)
             Af = H.to_float(A, dtype).astype(np.float64).reshape(batch, m, k)
             Bf = H.to_float(B, dtype).astype(np.float64).reshape(batch, k, n)
@@ -123,7 +123,7 @@ def test_matmul_tiles_exact_on_small_integers(dxh):
         for tile in (0, 1, 2, 3, 4, 5, 6):
             dx.check(dxh.dxh_tune(TILE_KNOB, tile))
             try:
-                dx.check(dxh.dxh_matmul(dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+                dx.check(H.matmul(dxh, dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
                 got = H.to_float(dC.get(), dx.BF16).astype(np.float64).reshape(m, n)
             finally:
                 dx.check(dxh.dxh_tune(TILE_KNOB, 0))
@@ -144,7 +144,7 @@ def test_matmul_f32_tile_configs(dxh, tile):
             A = rng.standard_normal(batch * m * k).astype(np.float32)
             B = rng.standard_normal(batch * k * n).astype(np.float32)
             dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, np.float32)
-            dx.check(dxh.dxh_matmul(dx.F32, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+            dx.check(H.matmul(dxh, dx.F32, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
             got = dC.get().astype(np.float64).reshape(batch, m, n)
             Af, Bf = A.astype(np.float64).reshape(batch, m, k), B.astype(np.float64).reshape(batch, k, n)
             ref, mag = np.matmul(Af, Bf), np.matmul(np.abs(Af), np.abs(Bf))
@@ -153,7 +153,7 @@ def test_matmul_f32_tile_configs(dxh, tile):
         m, k, n = 200, 96, 132
         Ai, Bi = rng.integers(-8, 9, (m, k)), rng.integers(-8, 9, (k, n))
         dA, dB, dC = Dev(Ai.astype(np.float32).reshape(-1)), Dev(Bi.astype(np.float32).reshape(-1)), Dev.empty(m * n, np.float32)
-        dx.check(dxh.dxh_matmul(dx.F32, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+        dx.check(H.matmul(dxh, dx.F32, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
         assert np.array_equal(dC.get().reshape(m, n), (Ai @ Bi).astype(np.float32))
     finally:
         dx.check(dxh.dxh_tune(TILE_KNOB, 0))
@@ -173,7 +173,7 @@ def test_matmul_f64_tile_configs(dxh, tile):
             A = rng.standard_normal(batch * m * k)
             B = rng.standard_normal(batch * k * n)
             dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, np.float64)
-            dx.check(dxh.dxh_matmul(dx.F64, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+            dx.check(H.matmul(dxh, dx.F64, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
             got = dC.get().reshape(batch, m, n)
             Af, Bf = A.reshape(batch, m, k), B.reshape(batch, k, n)
             ref, mag = np.matmul(Af, Bf), np.matmul(np.abs(Af), np.abs(Bf))
@@ -181,7 +181,7 @@ def test_matmul_f64_tile_configs(dxh, tile):
         m, k, n = 200, 96, 132
         Ai, Bi = rng.integers(-1000, 1001, (m, k)), rng.integers(-1000, 1001, (k, n))
         dA, dB, dC = Dev(Ai.astype(np.float64).reshape(-1)), Dev(Bi.astype(np.float64).reshape(-1)), Dev.empty(m * n, np.float64)
-        dx.check(dxh.dxh_matmul(dx.F64, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+        dx.check(H.matmul(dxh, dx.F64, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
         assert np.array_equal(dC.get().reshape(m, n), (Ai @ Bi).astype(np.float64))
     finally:
         dx.check(dxh.dxh_tune(TILE_KNOB, 0))
@@ -211,21 +211,21 @@ def test_matmul_split_k_forced(dxh, dtype, splits):
             A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
             B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
             dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, A.dtype)
-            dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+            dx.check(H.matmul(dxh, dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
             first = dC.get()
             got = H.to_float(first, dtype).astype(np.float64).reshape(batch, m, n)
             ref, mag = _ref_product(A, B, dtype, batch, m, k, n)
             scale = np.sqrt(k) if dtype in (dx.F32, dx.F64) else 1.0
             assert np.all(np.abs(got - ref) <= rel * scale * np.maximum(mag, 1e-300)), (dtype, splits, batch, m, k, n)
             dC2 = Dev.empty(batch * m * n, A.dtype)
-            dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC2.ptr, batch, m, k, n, None), "matmul")
+            dx.check(H.matmul(dxh, dtype, dA.ptr, dB.ptr, dC2.ptr, batch, m, k, n, None), "matmul")
             assert np.array_equal(first, dC2.get()), "split-K result varies between runs"
         m, k, n = 96, 456, 72
         Ai, Bi = rng.integers(-4, 5, (m, k)), rng.integers(-4, 5, (k, n))
         A = H.to_storage(Ai.astype(np.float64).reshape(-1), dtype)
         B = H.to_storage(Bi.astype(np.float64).reshape(-1), dtype)
         dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, A.dtype)
-        dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+        dx.check(H.matmul(dxh, dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
         want = H.to_float(H.to_storage((Ai @ Bi).astype(np.float64).reshape(-1), dtype), dtype)  # one rounding of the exact integer
         assert np.array_equal(H.to_float(dC.get(), dtype), want)
     finally:
@@ -245,7 +245,7 @@ def test_matmul_skinny_shapes_auto_split(dxh, dtype):
                 A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
                 B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
                 dA, dB, dC = Dev(A), Dev(B), Dev.empty(batch * m * n, A.dtype)
-                dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+                dx.check(H.matmul(dxh, dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
                 got = H.to_float(dC.get(), dtype).astype(np.float64).reshape(batch, m, n)
                 ref, mag = _ref_product(A, B, dtype, batch, m, k, n)
                 scale = np.sqrt(k) if dtype in (dx.F32, dx.F64) else 1.0
@@ -254,32 +254,42 @@ def test_matmul_skinny_shapes_auto_split(dxh, dtype):
             dx.check(dxh.dxh_tune(SPLITK_KNOB, 0))
 
 
-def test_matmul_under_capture_does_not_split(dxh):
-    """A stream under graph capture may not allocate: a matmul that would be cut along K is
-    recorded as one unsplit kernel, and the replayed graph gives the eager result."""
+@pytest.mark.parametrize("dtype,m,k,n", [(dx.F32, 16, 4096, 256), (dx.BF16, 64, 8192, 64), (dx.BF16, 333, 777, 555),
+                                         (dx.F32, 4, 4096, 1024), (dx.F64, 130, 515, 67)])
+def test_matmul_under_capture_equals_eager(dxh, dtype, m, k, n):
+    """Products that are cut along K or run on padded copies keep their partial results in the
+    caller's workspace, so the same kernels run under stream capture: a recorded matmul replays
+    the bits of the eager call (and neither allocates)."""
     import ctypes as C
-    rng = np.random.default_rng(900)
-    m, k, n = 16, 4096, 256
-    A = rng.standard_normal(m * k).astype(np.float32)
-    B = rng.standard_normal(k * n).astype(np.float32)
-    dA, dB, dC, dG = Dev(A), Dev(B), Dev.empty(m * n, np.float32), Dev.empty(m * n, np.float32)
-    dx.check(dxh.dxh_tune(SPLITK_KNOB, 1))
-    try:
-        dx.check(dxh.dxh_matmul(dx.F32, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))  # unsplit, eager
-    finally:
-        dx.check(dxh.dxh_tune(SPLITK_KNOB, 0))
+    rng = np.random.default_rng(900 + m)
+    A = H.to_storage(rng.standard_normal(m * k), dtype)
+    B = H.to_storage(rng.standard_normal(k * n), dtype)
+    dA, dB, dC, dG = Dev(A), Dev(B), Dev.empty(m * n, A.dtype), Dev.empty(m * n, A.dtype)
+    need = C.c_size_t(0)
+    dx.check(dxh.dxh_matmul_workspace_bytes(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, C.byref(need)))
+    assert need.value > 0, "shape chosen to need scratch"
+    ws = Dev.empty(need.value, np.uint8)
+    assert dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None, 0, None) == -4
+    assert dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, ws.ptr, need.value - 1, None) == -4
+    dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, ws.ptr, need.value, None))
     want = dC.get()
+    ref = H.to_float(A, dtype).reshape(m, k) @ H.to_float(B, dtype).reshape(k, n)
+    bound = np.abs(H.to_float(A, dtype).reshape(m, k)) @ np.abs(H.to_float(B, dtype).reshape(k, n))
+    tol = 1e-2 if dtype == dx.BF16 else (1e-5 if dtype == dx.F32 else 1e-13) * np.sqrt(k)
+    assert np.all(np.abs(H.to_float(want, dtype).reshape(m, n) - ref) <= tol * bound + 1e-30)
     st = C.c_void_p()
     dx.check(dxh.dxh_stream_create(C.byref(st)))
     graph = C.c_void_p()
     dx.check(dxh.dxh_graph_begin_capture(st))
-    rc = dxh.dxh_matmul(dx.F32, dA.ptr, dB.ptr, dG.ptr, 1, m, k, n, st)
+    rc = dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dG.ptr, 1, m, k, n, ws.ptr, need.value, st)
     dx.check(dxh.dxh_graph_end_capture(st, C.byref(graph)))
     dx.check(rc, "matmul under capture")
     for _ in range(3):
         dx.check(dxh.dxh_graph_launch(graph, st))
         dx.check(dxh.dxh_stream_sync(st))
-        assert np.array_equal(dG.get(), want)
+        assert np.array_equal(dG.get().view(np.uint8), want.view(np.uint8))
+        dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, ws.ptr, need.value, None))  # eager work between replays
+        dx.check(dxh.dxh_device_sync())
     dx.check(dxh.dxh_graph_destroy(graph))
     dx.check(dxh.dxh_stream_destroy(st))
 
@@ -299,7 +309,7 @@ def test_matmul_half_rows_not_16_byte_aligned(dxh, dtype, tile):
             B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
             # `off` elements of slack in front: the operands then start 2 * off bytes past a 256-byte boundary
             dA, dB, dC = Dev(np.concatenate([np.zeros(off, A.dtype), A])), Dev(np.concatenate([np.zeros(off, B.dtype), B])), Dev.empty(batch * m * n + off, A.dtype)
-            dx.check(dxh.dxh_matmul(dtype, dA.ptr.value + 2 * off, dB.ptr.value + 2 * off, dC.ptr.value + 2 * off, batch, m, k, n, None), "matmul")
+            dx.check(H.matmul(dxh, dtype, dA.ptr.value + 2 * off, dB.ptr.value + 2 * off, dC.ptr.value + 2 * off, batch, m, k, n, None), "matmul")
             got = H.to_float(dC.get()[off:], dtype).astype(np.float64).reshape(batch, m, n)
             ref, mag = _ref_product(A, B, dtype, batch, m, k, n)
             assert np.all(np.abs(got - ref) <= 1e-2 * np.maximum(mag, 1e-30)), (dtype, tile, batch, m, k, n, off)
@@ -308,7 +318,7 @@ def test_matmul_half_rows_not_16_byte_aligned(dxh, dtype, tile):
         A = H.to_storage(Ai.astype(np.float64).reshape(-1), dtype)
         B = H.to_storage(Bi.astype(np.float64).reshape(-1), dtype)
         dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, A.dtype)
-        dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+        dx.check(H.matmul(dxh, dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
         want = H.to_float(H.to_storage((Ai @ Bi).astype(np.float64).reshape(-1), dtype), dtype)
         assert np.array_equal(H.to_float(dC.get(), dtype), want)
     finally:
@@ -326,7 +336,7 @@ def test_matmul_int8_matrix_pipe_wraps_like_the_reference(dxh):
         A = rng.integers(-128, 128, (batch, m, k), dtype=np.int8)
         B = rng.integers(-128, 128, (batch, k, n), dtype=np.int8)
         dA, dB, dC = Dev(A.reshape(-1)), Dev(B.reshape(-1)), Dev.empty(batch * m * n, np.int8)
-        dx.check(dxh.dxh_matmul(dx.I8, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+        dx.check(H.matmul(dxh, dx.I8, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
         # float64 BLAS matmul is exact here: |sum| <= 140000 * 2^14 < 2^53
         want = np.matmul(A.astype(np.float64), B.astype(np.float64)).astype(np.int64).astype(np.int8)
         assert np.array_equal(dC.get().reshape(batch, m, n), want), (batch, m, k, n)
@@ -353,8 +363,8 @@ def _few_rows_cases(dxh, dtype, rng, rel):
         A = H.to_storage(rng.standard_normal(batch * m * k), dtype)
         B = H.to_storage(rng.standard_normal(batch * k * n), dtype)
         dA, dB, dC, dC2 = Dev(A), Dev(B), Dev.empty(batch * m * n, A.dtype), Dev.empty(batch * m * n, A.dtype)
-        dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
-        dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC2.ptr, batch, m, k, n, None), "matmul")
+        dx.check(H.matmul(dxh, dtype, dA.ptr, dB.ptr, dC.ptr, batch, m, k, n, None), "matmul")
+        dx.check(H.matmul(dxh, dtype, dA.ptr, dB.ptr, dC2.ptr, batch, m, k, n, None), "matmul")
         first = dC.get()
         assert np.array_equal(first, dC2.get()), "result varies between runs"
         got = H.to_float(first, dtype).astype(np.float64).reshape(batch, m, n)
@@ -366,7 +376,7 @@ def _few_rows_cases(dxh, dtype, rng, rel):
     A = H.to_storage(Ai.astype(np.float64).reshape(-1), dtype)
     B = H.to_storage(Bi.astype(np.float64).reshape(-1), dtype)
     dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, A.dtype)
-    dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+    dx.check(H.matmul(dxh, dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
     want = H.to_float(H.to_storage((Ai @ Bi).astype(np.float64).reshape(-1), dtype), dtype)
     assert np.array_equal(H.to_float(dC.get(), dtype), want)
 
@@ -392,7 +402,7 @@ def test_matmul_few_rows_any_n(dxh, dtype):
         for _ in range(2):
             dC = Dev(np.full(off + batch * m * n + guard, seven, npd))
             es = np.dtype(npd).itemsize
-            dx.check(dxh.dxh_matmul(dtype, dA.ptr.value + es * off, dB.ptr.value + es * off, dC.ptr.value + es * off, batch, m, k, n, None), "matmul")
+            dx.check(H.matmul(dxh, dtype, dA.ptr.value + es * off, dB.ptr.value + es * off, dC.ptr.value + es * off, batch, m, k, n, None), "matmul")
             outs.append(dC.get())
         assert np.array_equal(outs[0], outs[1]), "result varies between runs"
         assert np.all(outs[0][:off] == seven) and np.all(outs[0][off + batch * m * n:] == seven), "wrote outside C"
@@ -405,6 +415,6 @@ def test_matmul_few_rows_any_n(dxh, dtype):
     A = H.to_storage(Ai.astype(np.float64).reshape(-1), dtype)
     B = H.to_storage(Bi.astype(np.float64).reshape(-1), dtype)
     dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, npd)
-    dx.check(dxh.dxh_matmul(dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
+    dx.check(H.matmul(dxh, dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
     want = H.to_float(H.to_storage((Ai @ Bi).astype(np.float64).reshape(-1), dtype), dtype)
     assert np.array_equal(H.to_float(dC.get(), dtype), want)

@@ -5,6 +5,7 @@
 #include <string>
 #include <vector>
 #include "executor.hpp"
+#include "tensorio.hpp"
 
 using namespace deepx;
 
@@ -84,6 +85,8 @@ DXE_API size_t dxe_typedef_roundtrip(const char *text, char *out, size_t buflen)
     TypeDef t = typedef_from(text ? text : "");
     return copy_out(typedef_str(t) + " " + std::to_string((int)t.category) + " " + std::to_string((int)t.precision), out, buflen);
 }
+// whether `print` accepts a format for a floating (is_float != 0) or integer tensor: 1 or 0
+DXE_API int dxe_print_format_ok(const char *fmt, int is_float) { return print_format_ok(fmt ? fmt : "", is_float != 0) ? 1 : 0; }
 // tensor metadata as the reference's .shape YAML; "error: ..." if the tensor does not exist
 DXE_API size_t dxe_tensor_yaml(void *ex, const char *name, char *out, size_t buflen) {
     try {

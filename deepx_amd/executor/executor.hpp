@@ -245,7 +245,12 @@ public:
     }
 
 private:
-    struct Pinned { std::string name; const void *data; int64_t bytes; int dtype; };
+    // What a recorded graph froze about a tensor: the kernels' pointer arguments and every launch
+    // shape derived from its dims (an in-place reshape keeps address and size but not those).
+    struct Pinned {
+        std::string name; const void *data; int64_t bytes; int dtype; std::vector<int> dims;
+        bool same(const void *d, int64_t b, int t, const std::vector<int> &s) const { return data == d && bytes == b && dtype == t && dims == s; }
+    };
     struct Graph { void *exec = nullptr; std::vector<Pinned> tensors; const void *workspace = nullptr; };
 
     // every tensor a call names (bare names, typed params and [a b c] lists alike)
@@ -279,7 +284,7 @@ private:
         g.tensors.clear();
         for (const std::string &name : names) {
             auto t = mem.gettensor(name);
-            g.tensors.push_back({name, t->data, t->shape.bytes(), t->dtype()});
+            g.tensors.push_back({name, t->data, t->shape.bytes(), t->dtype(), t->shape.shape});
         }
         g.workspace = mem.workspace_ptr();
         return true;
@@ -288,7 +293,7 @@ private:
         if (g.workspace != mem.workspace_ptr()) return false;
         for (const Pinned &p : g.tensors) {
             auto t = mem.findtensor(p.name);
-            if (!t || t->data != p.data || t->shape.bytes() != p.bytes || t->dtype() != p.dtype) return false;
+            if (!t || !p.same(t->data, t->shape.bytes(), t->dtype(), t->shape.shape)) return false;
         }
         return true;
     }
@@ -298,16 +303,16 @@ private:
     static bool same_pins(const Graph &a, const Graph &b) {
         if (a.workspace != b.workspace || a.tensors.size() != b.tensors.size()) return false;
         for (size_t i = 0; i < a.tensors.size(); ++i)
-            if (a.tensors[i].name != b.tensors[i].name || a.tensors[i].data != b.tensors[i].data ||
-                a.tensors[i].bytes != b.tensors[i].bytes || a.tensors[i].dtype != b.tensors[i].dtype) return false;
+            if (a.tensors[i].name != b.tensors[i].name ||
+                !a.tensors[i].same(b.tensors[i].data, b.tensors[i].bytes, b.tensors[i].dtype, b.tensors[i].dims)) return false;
         return true;
     }
 
     // Returns true when the whole batch ran (was replayed or recorded and launched) as one graph.
     // false = nothing ran on the device: the caller executes the lines eagerly.  A batch is only
-    // recorded on its second arrival (the first, eager, pass also sizes the reduction workspace),
-    // and replayed only while every tensor it names still has the address, size and dtype it was
-    // recorded with.
+    // recorded on its second arrival (the first, eager, pass also sizes the reduction / matmul
+    // workspace), and replayed only while every tensor it names still has the address, size, dtype
+    // and dims it was recorded with.
     bool run_as_graph(const std::string &key, size_t n, const std::function<bool()> &run_all,
                       const std::function<const TF &(size_t)> &call_at) {
         if (rejected_.count(key)) return false;
@@ -324,6 +329,9 @@ private:
             it = graphs_.end();
         }
         if (it == graphs_.end()) {
+            // bounded memory in a long-lived server: forgetting a text only costs one more eager pass
+            if (seen_.size() >= kMaxRemembered) seen_.clear();
+            if (rejected_.size() >= kMaxRemembered) rejected_.clear();
             if (seen_.insert(key).second) return false;  // first arrival: run eagerly
             if (!graph_stream_ && dxh_stream_create(&graph_stream_) != DXH_OK) { graph_stream_ = nullptr; return false; }
             if (dxh_stream_sync(nullptr) != DXH_OK) return false;
@@ -363,6 +371,7 @@ private:
     std::mutex mu_;
     void *graph_stream_ = nullptr;
     std::unordered_map<std::string, Graph> graphs_;
+    static constexpr size_t kMaxRemembered = 1024;
     std::unordered_set<std::string> seen_, rejected_;
 };
 

@@ -8,7 +8,9 @@
 // The tensor's name on load is the file stem (shape.cpp:140-142).  Device data moves through
 // one staged host copy.  print follows executor/deepxcore/src/stdutil/print.hpp:80-129.
 #pragma once
+#include <cctype>
 #include <cstdio>
+#include <cstring>
 #include <fstream>
 #include <memory>
 #include <ostream>
@@ -102,20 +104,56 @@ inline void print_element(std::ostream &os, const char *data, int64_t i, Precisi
         std::snprintf(buf, sizeof buf, fmt.c_str(), (double)f);
         break;
     }
-    case Precision::Int64: std::snprintf(buf, sizeof buf, fmt.find('l') == std::string::npos ? "%lld" : fmt.c_str(), (long long)((const int64_t *)data)[i]); break;
-    case Precision::Int32: std::snprintf(buf, sizeof buf, fmt.c_str(), ((const int32_t *)data)[i]); break;
-    case Precision::Int16: std::snprintf(buf, sizeof buf, fmt.c_str(), (int)((const int16_t *)data)[i]); break;
-    case Precision::Int8: std::snprintf(buf, sizeof buf, fmt.c_str(), (int)((const int8_t *)data)[i]); break;
-    case Precision::Bool: std::snprintf(buf, sizeof buf, fmt.c_str(), (int)((const uint8_t *)data)[i]); break;
+    // integer formats reach here with their length modifier rewritten to "ll" (print_tensor)
+    case Precision::Int64: std::snprintf(buf, sizeof buf, fmt.c_str(), (long long)((const int64_t *)data)[i]); break;
+    case Precision::Int32: std::snprintf(buf, sizeof buf, fmt.c_str(), (long long)((const int32_t *)data)[i]); break;
+    case Precision::Int16: std::snprintf(buf, sizeof buf, fmt.c_str(), (long long)((const int16_t *)data)[i]); break;
+    case Precision::Int8: std::snprintf(buf, sizeof buf, fmt.c_str(), (long long)((const int8_t *)data)[i]); break;
+    case Precision::Bool: std::snprintf(buf, sizeof buf, fmt.c_str(), (long long)((const uint8_t *)data)[i]); break;
     default: buf[0] = '?'; buf[1] = 0;
     }
     os << buf;
+}
+
+// The format of `print` arrives from the wire and goes to snprintf with one value: it must hold
+// exactly one conversion, of the value's kind (floating: f e g a and capitals; integer: d i u x X o),
+// with optional flags, width, precision and length modifier (not L: the value is a double); no %n,
+// %s, %c, %p, no '*'.  "%%" is
+// literal text.  (The reference passes the text through unchecked, stdutil/print.hpp.)
+inline bool print_format_ok(const std::string &fmt, bool is_float) {
+    int conversions = 0;
+    for (size_t i = 0; i < fmt.size(); ++i) {
+        if (fmt[i] != '%') continue;
+        ++i;
+        if (i < fmt.size() && fmt[i] == '%') continue;
+        while (i < fmt.size() && std::strchr("-+ #0", fmt[i])) ++i;
+        while (i < fmt.size() && std::isdigit((unsigned char)fmt[i])) ++i;
+        if (i < fmt.size() && fmt[i] == '.') { ++i; while (i < fmt.size() && std::isdigit((unsigned char)fmt[i])) ++i; }
+        while (i < fmt.size() && std::strchr(is_float ? "l" : "hljzt", fmt[i])) ++i;
+        if (i >= fmt.size() || !std::strchr(is_float ? "fFeEgGaA" : "diuxXo", fmt[i])) return false;
+        ++conversions;
+    }
+    return conversions == 1 && fmt.size() <= 64;
 }
 
 inline void print_tensor(const Tensor &t, std::string fmt, std::ostream &os) {
     const Precision p = t.shape.dtype;
     const bool is_float = (uint16_t(p) & uint16_t(Precision::Float)) != 0;
     if (fmt.empty()) fmt = is_float ? "%.4f" : "%d";
+    if (!print_format_ok(fmt, is_float)) throw std::invalid_argument("print: format must hold one " + std::string(is_float ? "floating" : "integer") + " conversion: " + fmt);
+    if (!is_float) {  // every integer value is passed as long long, whatever width the format named
+        std::string ll;
+        for (size_t i = 0; i < fmt.size(); ++i) {
+            if (fmt[i] != '%') { ll += fmt[i]; continue; }
+            ll += '%';
+            if (i + 1 < fmt.size() && fmt[i + 1] == '%') { ll += '%'; ++i; continue; }
+            for (++i; i < fmt.size() && !std::strchr("diuxXo", fmt[i]); ++i)
+                if (!std::strchr("hljzt", fmt[i])) ll += fmt[i];
+            ll += "ll";
+            if (i < fmt.size()) ll += fmt[i];
+        }
+        fmt = ll;
+    }
     std::vector<char> host = to_host(t);
     const Shape &s = t.shape;
     os << "shape:[";

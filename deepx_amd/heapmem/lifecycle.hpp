@@ -56,18 +56,31 @@ inline int dtype_bytes(const std::string &d) {
     return 0;
 }
 // "[2,3,4]" or "[2 3 4]" -> element count; -1 when malformed
+// Element count of "[2,3]" / "[2 3]"; -1 = malformed, -2 = the product does not fit (a count beyond
+// kMaxElements is as good as overflow: no shared allocation may be that large).
+constexpr long long kMaxElements = 1LL << 40;
 inline long long shape_elements(const std::string &shape) {
     long long n = 1;
-    bool any = false, in_number = false;
+    bool any = false, in_number = false, too_big = false;
     long long cur = 0;
+    auto fold = [&]() {
+        if (cur != 0 && n > kMaxElements / cur) too_big = true; else n *= cur;
+        cur = 0; in_number = false; any = true;
+    };
     for (char c : shape) {
-        if (std::isdigit((unsigned char)c)) { cur = cur * 10 + (c - '0'); in_number = true; }
-        else if (c == ',' || c == ' ' || c == '[' || c == ']') { if (in_number) { n *= cur; cur = 0; in_number = false; any = true; } }
+        if (std::isdigit((unsigned char)c)) {
+            if (cur > kMaxElements) too_big = true; else cur = cur * 10 + (c - '0');
+            in_number = true;
+        }
+        else if (c == ',' || c == ' ' || c == '[' || c == ']') { if (in_number) fold(); }
         else return -1;
     }
-    if (in_number) { n *= cur; any = true; }
+    if (in_number) fold();
+    if (too_big) return n == 0 ? 0 : -2;  // a zero extent anywhere makes the tensor empty whatever the others say
     return any ? n : (shape.find('[') != std::string::npos ? 1 : -1);  // "[]" is a scalar
 }
+// A shared allocation stays under 2 GiB: larger IPC handles do not open on the target machines.
+constexpr long long kMaxSharedBytes = (2LL << 30) - 1;
 inline std::string to_hex(const unsigned char *bytes, size_t n) {
     static const char *digits = "0123456789abcdef";
     std::string s;
@@ -125,8 +138,11 @@ public:
             const int es = dtype_bytes(cmd.dtype);
             const long long elements = shape_elements(cmd.shape);
             if (es == 0) return "unknown dtype: " + cmd.dtype;
+            if (elements == -2 || (elements > 0 && elements > kMaxSharedBytes / es))
+                return "tensor too large to share: " + cmd.shape + " " + cmd.dtype + " exceeds " + std::to_string(kMaxSharedBytes) + " bytes";
             if (elements < 0) return "malformed shape: " + cmd.shape;
             const long long bytes = elements * es;
+            Release(cmd.name);  // memory of an earlier incarnation whose registry entry is gone
             void *ptr = nullptr;
             int rc = ops_.alloc(&ptr, (size_t)bytes);
             if (rc != 0 || !ptr) return std::string("allocation failed: ") + dxh_error_string(rc);

@@ -34,6 +34,7 @@ class InProc:
         L.dxe_infer_shape.restype = C.c_size_t
         L.dxe_set_graphs.argtypes = [C.c_void_p, C.c_int]
         L.dxe_set_fusion.argtypes = [C.c_void_p, C.c_int]
+        L.dxe_print_format_ok.argtypes = [C.c_char_p, C.c_int]
         self.L = L
         self.ex = L.dxe_create()
         assert self.ex
@@ -62,6 +63,8 @@ class InProc:
     def typedef(self, text): return self._call(self.L.dxe_typedef_roundtrip, text.encode())
     def tensor_yaml(self, name): return self._call(self.L.dxe_tensor_yaml, self.ex, name.encode())
     def shape_yaml(self, text): return self._call(self.L.dxe_shape_yaml_roundtrip, text.encode())
+
+    def print_format_ok(self, fmt, is_float): return bool(self.L.dxe_print_format_ok(fmt.encode(), int(is_float)))
 
     def infer(self, op, a, b=(), extra=0):
         A = (C.c_int * max(1, len(a)))(*a)

@@ -150,6 +150,19 @@ def test_inproc_error_replies(ex):
     assert "id" not in ex.execute("sum(tensor<float32>:x, vector<int32>:[], var<bool>:false)->(tensor<float32>:y) // id=x9")[:4]  # bad id is an error reply, not a crash
 
 
+def test_print_format_from_the_wire_is_validated(ex):
+    """`print(t, format)` hands its format to snprintf with one value: exactly one conversion of the
+    value's kind is accepted; %n, %s, '*', several conversions or none are refused (an error reply)."""
+    for fmt in ["%f", "%.4f", "%8.3e", "%g", "%-10.2F", "%+.1f", "x=%f;", "%lf", "100%% %f"]:
+        assert ex.print_format_ok(fmt, True), fmt
+    for fmt in ["%d", "%5d", "%x", "%lld", "%ld", "%hhd", "%08X", "%i", "%u", "[%o]"]:
+        assert ex.print_format_ok(fmt, False), fmt
+    for fmt in ["%s", "%n", "%f%f", "%*d", "%.*f", "%d %d", "", "plain", "%", "%5", "%c", "%p", "%f%n", "%ls", "%Lf", "%" + "9" * 80 + "f"]:
+        assert not ex.print_format_ok(fmt, True), fmt
+        assert not ex.print_format_ok(fmt, False), fmt
+    assert not ex.print_format_ok("%d", True) and not ex.print_format_ok("%f", False)
+
+
 def test_udp_server_error_paths_and_framing():
     srv = UdpExecutor()
     try:

@@ -71,6 +71,20 @@ def test_bad_commands_are_reported_not_fatal(store):
     assert store.meta("bad") is None and store.owned() == 1
 
 
+def test_create_refuses_what_cannot_be_shared(store):
+    """A shared allocation stays under 2 GiB (larger IPC handles do not open), and a shape whose
+    element count overflows is refused instead of wrapping into a small or huge request."""
+    assert store.command(cmd("create", "big", dtype="f32", shape=[1 << 29], node="n")) == -1 and "too large" in store.last_error()
+    assert store.command(cmd("create", "big", dtype="int8", shape=[1 << 31], node="n")) == -1 and "too large" in store.last_error()
+    assert store.command(cmd("create", "big", dtype="f64", shape=[1 << 20, 1 << 20, 1 << 20, 1 << 20], node="n")) == -1 and "too large" in store.last_error()
+    assert store.command('{"op":"create","name":"big","dtype":"f32","shape":"[99999999999999999999999]","node":"n"}') == -1
+    assert "too large" in store.last_error()
+    assert store.meta("big") is None and store.owned() == 0
+    assert store.command(cmd("create", "empty", dtype="f32", shape=[1 << 40, 0], node="n")) == 1   # empty whatever the other extent says
+    assert store.meta("empty")["bytes"] == "0"
+    assert store.command(cmd("create", "edge", dtype="int8", shape=[4096], node="n")) == 1 and store.owned() == 2
+
+
 def test_sweep_keeps_referenced_tensors_of_live_owners(store):
     for name in ("a", "b"):
         assert store.command(cmd("create", name, dtype="f32", shape=[8], node="here")) == 1

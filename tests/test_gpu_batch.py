@@ -317,3 +317,112 @@ def test_fused_in_place_run(tmp_path):
     for k in ("sg", "g", "u"):
         assert np.array_equal(outs["fused"][k], outs["lines"][k]), k
     assert np.array_equal(outs["fused"]["g"], g) and np.array_equal(outs["fused"]["u"], u)
+
+
+def test_recorded_graph_notices_an_in_place_reshape(tmp_path):
+    """A recorded batch freezes launch shapes.  An in-place reshape keeps a tensor's address, size and
+    dtype but changes its dims: the next arrival of the same text must run with the new dims (be
+    recorded again), not replay the old launch."""
+    ex = InProc()
+    ex.set_graphs(True)
+    h = Host(ex, tmp_path)
+    a = np.arange(32, dtype=np.float32).reshape(4, 8)
+    h.put("rs_A", a)
+    h.run(f"newtensor({V([32])})->({T('rs_C')})")
+    h.run(f"newtensor({V([32])})->({T('rs_D')})")
+    lines = [f"transpose({T('rs_A')}, {V([1, 0])})->({T('rs_C')}) // author=miaobyte id=7001",
+             f"addscalar({T('rs_C')}, var<float32>:1)->({T('rs_D')}) // author=miaobyte id=7002"]
+    for _ in range(3):  # eager, recorded, replayed
+        assert all(r.split(" ")[1].startswith("ok") for r in ex.execute_batch(lines))
+    assert np.array_equal(h.get("rs_C"), a.T.reshape(-1))
+    assert ex.stats()["captures"] == 1 and ex.stats()["replays"] == 1
+    h.run(f"reshape({T('rs_A')}, {V([8, 4])})->({T('rs_A')})")
+    for _ in range(3):
+        h.run(f"constant(var<float32>:0)->({T('rs_C')})")
+        assert all(r.split(" ")[1].startswith("ok") for r in ex.execute_batch(lines))
+        assert np.array_equal(h.get("rs_C"), a.reshape(8, 4).T.reshape(-1))
+        assert np.array_equal(h.get("rs_D"), a.reshape(8, 4).T.reshape(-1) + 1)
+    assert ex.stats()["captures"] == 2, ex.stats()
+
+
+def test_config5_block_at_full_size_in_every_mode(tmp_path):
+    """The whole BASELINE config-5 block (RMSNorm + gated MLP, 22 deepxIR ops) at its stated size,
+    2048 rows, through the executor line by line, as one batch, as one batch with fused elementwise
+    runs, and as a recorded graph without and with fused runs.  Every mode against a float64 numpy
+    model of the same op sequence with bf16 rounding where the graph stores bf16 (rel 1e-2 per bf16
+    rounding; 3e-2 of the output scale end to end, 1e-2 for the normalised activations), and every
+    mode bit-identical to the line-by-line execution."""
+    rng = np.random.default_rng(14)
+    S, Hd, I = 2048, 896, 4864
+    f2b, b2f = H.f32_to_bf16_bits, H.bf16_bits_to_f32
+    x = f2b(rng.standard_normal((S, Hd)).astype(np.float32))
+    w = f2b(np.ones(Hd, dtype=np.float32) + 0.1 * rng.standard_normal(Hd).astype(np.float32))
+    Wg = f2b((rng.standard_normal((Hd, I)) * 0.02).astype(np.float32))
+    Wu = f2b((rng.standard_normal((Hd, I)) * 0.02).astype(np.float32))
+    Wd = f2b((rng.standard_normal((I, Hd)) * 0.02).astype(np.float32))
+    # float64 model (front/py/deepx/nn/modules/norm/t5layernorm.py:17-22, mlp/gatedmlp.py:20-26)
+    rb = lambda a: b2f(f2b(a.astype(np.float32))).astype(np.float64)
+    xf = b2f(x).astype(np.float64)
+    xn = xf * (1.0 / np.sqrt((xf ** 2).sum(-1, keepdims=True) / Hd + 1e-6))
+    h_ref = rb(b2f(w).astype(np.float64) * xn)
+    g = rb(h_ref @ b2f(Wg).astype(np.float64)); u = rb(h_ref @ b2f(Wu).astype(np.float64))
+    act = rb(rb(g * rb(1.0 / rb(1.0 + rb(np.exp(rb(-g)))))) * u)
+    y_ref = act @ b2f(Wd).astype(np.float64)
+
+    b16, f32 = "bfloat16", "float32"
+    n = lambda name, dt=f32: T("f5_" + name, dt)
+    tensors = [("xf", [S, Hd], f32), ("sq", [S, Hd], f32), ("var", [S, 1], f32), ("rs", [S, Hd], f32), ("xn", [S, Hd], f32),
+               ("wf1", [1, Hd], f32), ("wf", [S, Hd], f32), ("h", [S, Hd], b16), ("g", [S, I], b16), ("u", [S, I], b16),
+               ("sg", [S, I], b16), ("y", [S, Hd], b16)]
+    block = [f"todtype({n('x', b16)})->({n('xf')})",
+             f"powscalar({n('xf')}, var<float32>:2)->({n('sq')})",
+             f"sum({n('sq')}, {V([-1])}, var<bool>:True)->({n('var')})",
+             f"divscalar({n('var')}, var<float32>:{Hd})->({n('var')})",
+             f"addscalar({n('var')}, var<float32>:1e-06)->({n('var')})",
+             f"sqrt({n('var')})->({n('var')})",
+             f"rdivscalar(var<float32>:1, {n('var')})->({n('var')})",
+             f"broadcastTo({n('var')}, {V([S, Hd])})->({n('rs')})",
+             f"mul({n('xf')}, {n('rs')})->({n('xn')})",
+             f"todtype({n('w', b16)})->({n('wf1')})",
+             f"broadcastTo({n('wf1')}, {V([S, Hd])})->({n('wf')})",
+             f"mul({n('wf')}, {n('xn')})->({n('xn')})",
+             f"todtype({n('xn')})->({n('h', b16)})",
+             f"matmul({n('h', b16)}, {n('Wg', b16)})->({n('g', b16)})",
+             f"matmul({n('h', b16)}, {n('Wu', b16)})->({n('u', b16)})",
+             f"mulscalar({n('g', b16)}, var<float32>:-1)->({n('sg', b16)})",
+             f"exp({n('sg', b16)})->({n('sg', b16)})",
+             f"addscalar({n('sg', b16)}, var<float32>:1)->({n('sg', b16)})",
+             f"rdivscalar(var<float32>:1, {n('sg', b16)})->({n('sg', b16)})",
+             f"mul({n('g', b16)}, {n('sg', b16)})->({n('sg', b16)})",
+             f"mul({n('sg', b16)}, {n('u', b16)})->({n('sg', b16)})",
+             f"matmul({n('sg', b16)}, {n('Wd', b16)})->({n('y', b16)})"]
+    text = [f"{line} // author=miaobyte id={100 + i}" for i, line in enumerate(block)]
+    kept = {}
+    for mode, batched, fused, graphs in (("lines", 0, 0, 0), ("batch", 1, 0, 0), ("batch_fused", 1, 1, 0), ("graph", 1, 0, 1), ("graph_fused", 1, 1, 1)):
+        ex = InProc()
+        ex.set_graphs(bool(graphs))
+        ex.set_fusion(bool(fused))
+        h = Host(ex, tmp_path)
+        for name, arr in (("x", x), ("w", w.reshape(1, Hd)), ("Wg", Wg), ("Wu", Wu), ("Wd", Wd)):
+            h.put("f5_" + name, arr, b16)
+        for name, shape, dt in tensors:
+            h.run(f"newtensor({V(shape)})->({T('f5_' + name, dt)})")
+        for rep in range(3 if graphs else 1):  # a graph is recorded on the second arrival and replayed on the third
+            if rep:
+                h.run(f"constant(var<float32>:0)->({n('y', b16)})")
+            rs = ex.execute_batch(text) if batched else [ex.execute(t) for t in text]
+            assert all(r.split(" ")[1].startswith("ok") for r in rs), (mode, rs)
+        if graphs:
+            st = ex.stats()
+            assert st["captures"] == 1 and st["replays"] == 1 and st["rejects"] == 0, (mode, st)
+        if fused:
+            assert ex.fusion_stats()["runs"] >= 2, (mode, ex.fusion_stats())
+        kept[mode] = {k: h.get("f5_" + k) for k in ("y", "h", "sg")}
+        y = b2f(kept[mode]["y"]).astype(np.float64)
+        hh = b2f(kept[mode]["h"]).astype(np.float64)
+        assert np.abs(y - y_ref).max() <= 3e-2 * np.abs(y_ref).max(), mode
+        assert np.abs(hh - h_ref).max() <= 1e-2 * np.abs(h_ref).max(), mode
+        del ex
+    for mode in ("batch", "batch_fused", "graph", "graph_fused"):
+        for k in ("y", "h", "sg"):
+            assert np.array_equal(kept[mode][k], kept["lines"][k]), (mode, k)

@@ -1,8 +1,12 @@
-"""GPU parity: dxh_chain (a run of elementwise ops in one launch) against the separate entry points.
+"""GPU parity: dxh_chain (a run of elementwise ops in one launch) against the CPU oracle and
+against the separate entry points.
 
-Bar: bit-identical outputs, op by op — the run must store exactly what add / mulscalar / exp ...
-store when called one after another (those are checked against the CPU oracle in
-test_gpu_elementwise.py).
+Bars: every output of a run is compared op by op with the oracle applied to the operands the
+device used for that op (so errors do not compound): bit-exact for add / sub / mul / div / max /
+min, their scalar forms and sqrt (correctly rounded on both sides), <= 4 ulp for exp and log
+(glibc on the host, ROCm's device libm here; 16-bit floats compute in fp32 and round once, which
+leaves at most 1 ulp of the storage type).  And bit-identical to what add / mulscalar / exp ...
+store when called one after another.
 """
 import ctypes as C
 
@@ -11,7 +15,7 @@ import pytest
 
 from deepx_amd import lib as dx
 from tests import helpers as H
-from tests.helpers import Dev
+from tests.helpers import Dev, hp
 
 pytestmark = pytest.mark.gpu
 
@@ -49,14 +53,44 @@ def run_chain(dxh, dtype, inputs, prog, n, outs=None):
     return dxh.dxh_chain(dtype, ptrs, len(inputs), ops, len(prog), n, None), outs
 
 
+def check_against_oracle(orc, dtype, inputs, prog, outs, n, what):
+    """Op k of the run on the oracle, fed with the device's own operands of that op."""
+    host_in = [d.get() for d in inputs]
+    host_out = [o.get() for o in outs]
+    for k, (name, lhs, rhs, s) in enumerate(prog):
+        src = lambda r: host_in[r] if r < dx.CHAIN_RESULT else host_out[r - dx.CHAIN_RESULT]
+        want = np.empty(n, dtype=H.NP[dtype])
+        fn = getattr(orc, "orc_" + name)
+        if name in BINARY:
+            rc = fn(dtype, hp(src(lhs)), hp(src(rhs)), hp(want), n)
+        elif name in ("rsubscalar", "rdivscalar"):
+            rc = fn(dtype, dx.scalar(s), hp(src(lhs)), hp(want), n)
+        elif name in SCALAR:
+            rc = fn(dtype, hp(src(lhs)), dx.scalar(s), hp(want), n)
+        else:
+            rc = fn(dtype, hp(src(lhs)), hp(want), n)
+        assert rc == 0, (name, rc)
+        if name in ("exp", "log"):
+            ulps = H.ulp_diff(host_out[k], want, dtype)
+            assert ulps <= (4 if dtype in (dx.F32, dx.F64) else 1), (what, dtype, k, name, ulps)
+        else:
+            same = (host_out[k].view(np.uint8) == want.view(np.uint8)).all() or \
+                np.array_equal(host_out[k], want, equal_nan=dtype in (dx.F32, dx.F64))
+            if not same and dtype in (dx.F16, dx.BF16):  # NaN payloads aside, the bits must agree
+                f, w = H.to_float(host_out[k], dtype), H.to_float(want, dtype)
+                same = np.array_equal(np.isnan(f), np.isnan(w)) and np.array_equal(host_out[k][~np.isnan(w)], want[~np.isnan(w)])
+            assert same, (what, dtype, k, name)
+
+
 def same_bits(a, b):
     return np.array_equal(a.get().view(np.uint8), b.get().view(np.uint8))
 
 
 @pytest.mark.parametrize("dtype", [dx.F32, dx.BF16, dx.F16, dx.F64])
-def test_config1_chain_in_one_launch(dxh, dtype):
+def test_config1_chain_in_one_launch(dxh, orc, dtype):
     """The 8-op elementwise chain of BASELINE config 1 (abs composed from mulscalar and max) and
-    the SiLU gate of config 5, each as one run; every intermediate tensor bit-identical."""
+    the SiLU gate of config 5, each as one run; every intermediate tensor against the oracle and
+    bit-identical to the separate kernels."""
     rng = np.random.default_rng(40 + dtype)
     n = 1 << 18
     A, B = Dev(H.rand(rng, dtype, n)), Dev(H.rand(rng, dtype, n))
@@ -69,12 +103,13 @@ def test_config1_chain_in_one_launch(dxh, dtype):
         want = run_separately(dxh, dtype, [A, B], prog, n)
         rc, got = run_chain(dxh, dtype, [A, B], prog, n)
         dx.check(rc, "chain")
+        check_against_oracle(orc, dtype, [A, B], prog, got, n, "config chain")
         for k, (g, w) in enumerate(zip(got, want)):
             assert same_bits(g, w), (dtype, prog[k][0], k)
 
 
 @pytest.mark.parametrize("dtype", [dx.F32, dx.BF16, dx.F16, dx.F64])
-def test_random_runs_match_separate_calls(dxh, dtype):
+def test_random_runs_match_separate_calls(dxh, orc, dtype):
     """Random runs of 1..8 ops over up to 8 inputs, every op code, operands drawn from inputs and
     earlier results; sizes from one vector to several workgroups."""
     rng = np.random.default_rng(700 + dtype)
@@ -91,6 +126,7 @@ def test_random_runs_match_separate_calls(dxh, dtype):
         want = run_separately(dxh, dtype, inputs, prog, n)
         rc, got = run_chain(dxh, dtype, inputs, prog, n)
         dx.check(rc, "chain")
+        check_against_oracle(orc, dtype, inputs, prog, got, n, ("random run", trial, n))
         for k, (g, w) in enumerate(zip(got, want)):
             assert same_bits(g, w), (dtype, trial, n, prog, k)
 

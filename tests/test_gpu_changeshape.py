@@ -101,6 +101,31 @@ def test_transpose_bad_order(dxh):
     assert dxh.dxh_transpose(dx.F32, a.ptr, dx.i32arr([2, 3, 4]), 3, dx.i32arr([0, 1, 3]), a.ptr, None) == -2
 
 
+def test_concat_reference_expectation_on_the_hip_path(dxh):
+    """The expectation the reference's own concat test holds
+    (executor/op-ompsimd/test/tensorfunc/8_tensor_concat.cpp:47-129: four constant-filled [2,3,4]
+    tensors joined along each axis), through dxh_concat."""
+    import json
+    import os
+    g = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "concat_kat.json")))
+    arrs = [np.full(t["shape"], t["fill"], dtype=np.float32) for t in g["inputs"]]
+    devs = [Dev(a) for a in arrs]
+    for axis_s, exp in g["expected"].items():
+        axis, shape = int(axis_s), exp["shape"]
+        out = Dev.empty(int(np.prod(shape)), np.float32)
+        dx.check(dxh.dxh_concat(dx.F32, dx.ptrarr([d.ptr.value for d in devs]), len(devs), dx.i32arr([a.shape[axis] for a in arrs]),
+                                dx.i32arr(shape), 3, axis, out.ptr, None), "concat")
+        got = out.get().reshape(shape)
+        if axis == 0:
+            for i, v in enumerate(exp["blocks"]):
+                assert np.all(got[i] == v)
+        elif axis == 1:
+            for i in range(2):
+                assert np.array_equal(got[i], np.repeat(np.array(exp["rows"], dtype=np.float32)[:, None], 4, axis=1))
+        else:
+            assert np.all(got == np.array(exp["row"], dtype=np.float32))
+
+
 @pytest.mark.parametrize("es", [1, 2, 4, 8])
 def test_concat(dxh, orc, es):
     rng = np.random.default_rng(50 + es)

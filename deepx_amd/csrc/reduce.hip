@@ -716,3 +716,62 @@ int dxh_reducemin(int dtype, const void *in, const int32_t *shape, int ndim, con
 }
 
 }  // extern "C"
+
+// ---- dxh_sum for callers that cannot allocate ---------------------------------------------
+// The partial results that dxh_sum keeps in the caller's workspace live here in a file-scope
+// device array instead: one copy per GPU, held until the process ends.  In host code the array's
+// name is only a stand-in for the symbol; its device address is looked up once per device with
+// hipGetSymbolAddress (that device current) and only that pointer is ever handed to a kernel.
+// Nothing in it has to start at zero: a stage writes every partial it later reads.  Calls that
+// overlap on one GPU (two streams, two threads) share the array and race.
+constexpr size_t kScratchBytes = (size_t)4 << 20;
+static_assert(kScratchBytes == DXH_SUM_NOALLOC_SCRATCH_BYTES, "the limit is part of the ABI");
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];
+bool g_scratch_resolved[kMaxDevices];
+}  // namespace
+
+namespace dxh {
+// Device address of `scratch` on the current device; looked up on the first call per device.
+// The lookup is not a stream operation and is refused while `st` is being captured.
+int scratch_pointer(hipStream_t st, bool may_be_capturing, void **ptr) {
+    *ptr = nullptr;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { (void)hipGetLastError(); return (int)e; }
+    if (dev < 0 || dev >= kMaxDevices) return DXH_ERR_ARG;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_resolved[dev]) {
+        if (may_be_capturing && stream_is_capturing(st)) return DXH_ERR_NOT_READY;
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) { (void)hipGetLastError(); return (int)e; }
+        g_scratch_ptr[dev] = p;
+        g_scratch_resolved[dev] = true;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return DXH_OK;
+}
+// dxh_set_device is the library's set-up call for a device: both file-scope arrays are resolved
+// there, so that a first reduction under stream capture finds them ready.
+void reduce_device_init() {
+    void *p = nullptr;
+    (void)scratch_pointer(nullptr, false, &p);
+    (void)finish_counters(nullptr, 1);
+}
+}  // namespace dxh
+
+extern "C" int dxh_sum_noalloc(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims, int ndims, void *out,
+                    void *stream) {
+    size_t need = 0;
+    int rc = dxh_reduce_workspace_bytes(dtype, shape, ndim, dims, ndims, &need);
+    if (rc != DXH_OK) return rc;
+    if (need > kScratchBytes) return DXH_ERR_TOO_LARGE;
+    void *ws = nullptr;
+    rc = scratch_pointer(as_stream(stream), true, &ws);
+    if (rc != DXH_OK) return rc;
+    return reduce_all<R_SUM>(dtype, in, shape, ndim, dims, ndims, out, ws, kScratchBytes, stream);
+}

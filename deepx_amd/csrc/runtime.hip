@@ -48,6 +48,8 @@ const char *dxh_error_string(int code) {
     case DXH_ERR_SHAPE: return "shape mismatch";
     case DXH_ERR_WORKSPACE: return "workspace missing or too small";
     case DXH_ERR_ALIGN: return "pointer not aligned to its element size";
+    case DXH_ERR_TOO_LARGE: return "input needs more scratch than this entry point's fixed buffer holds";
+    case DXH_ERR_NOT_READY: return "first use on this device is under stream capture: call dxh_set_device first";
     default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);
@@ -60,7 +62,11 @@ int dxh_device_count(int *count) {
     if (e != hipSuccess) { *count = 0; (void)hipGetLastError(); }
     return (int)e;
 }
-int dxh_set_device(int device) { return (int)hipSetDevice(device); }
+int dxh_set_device(int device) {
+    hipError_t e = hipSetDevice(device);
+    if (e == hipSuccess) dxh::reduce_device_init();
+    return (int)e;
+}
 int dxh_device_name(char *buf, size_t buflen) {
     if (!buf || buflen == 0) return DXH_ERR_ARG;
     int dev = 0;

@@ -105,6 +105,7 @@ SIGNATURES = {
     "dxh_reduce_workspace_bytes": ([_i, _pi32, _i, _pi32, _i, C.POINTER(_sz)], _i),
     "dxh_sum": (_RED, _i), "dxh_prod": (_RED, _i),
     "dxh_reducemax": (_RED, _i), "dxh_reducemin": (_RED, _i),
+    "dxh_sum_noalloc": ([_i, _p, _pi32, _i, _pi32, _i, _p, _p], _i),
     "dxh_transpose": ([_i, _p, _pi32, _i, _pi32, _p, _p], _i),
     "dxh_concat": ([_i, _pp, _i, _pi32, _pi32, _i, _i, _p, _p], _i),
     "dxh_broadcastTo": ([_i, _p, _pi32, _i, _pi32, _i, _p, _p], _i),

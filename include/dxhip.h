@@ -65,7 +65,9 @@ enum dxh_error {
     DXH_ERR_ARG = -2,        /* null pointer, negative size, bad axis ... */
     DXH_ERR_SHAPE = -3,      /* shapes inconsistent for this op */
     DXH_ERR_WORKSPACE = -4,  /* workspace missing or too small */
-    DXH_ERR_ALIGN = -5       /* pointer not aligned to its element size */
+    DXH_ERR_ALIGN = -5,      /* pointer not aligned to its element size */
+    DXH_ERR_TOO_LARGE = -6,  /* the input needs more scratch than the entry point's fixed buffer holds */
+    DXH_ERR_NOT_READY = -7   /* first use on this device is under stream capture: call dxh_set_device first */
 };
 
 /* A scalar operand.  Floating dtypes read `f`, integer and bool dtypes read `i`.
@@ -271,6 +273,19 @@ DXH_API int dxh_reducemax(int dtype, const void *in, const int32_t *shape, int n
 DXH_API int dxh_reducemin(int dtype, const void *in, const int32_t *shape, int ndim,
                           const int32_t *dims, int ndims, void *out, void *workspace,
                           size_t workspace_bytes, void *stream);
+
+/* dxh_sum for callers that cannot allocate or pass a workspace: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments
+ * and results (bit for bit) as dxh_sum; the partial results that dxh_sum keeps in `workspace` live in
+ * a device array of DXH_SUM_NOALLOC_SCRATCH_BYTES inside the library instead (one copy per GPU, held
+ * until the process ends), and the call allocates and frees nothing.  A reduction whose
+ * dxh_reduce_workspace_bytes exceeds that size is refused with DXH_ERR_TOO_LARGE.  Every call on one
+ * GPU shares the array: calls that overlap there (two streams, two threads) race.  The array's address
+ * is looked up on the first call on a device or by dxh_set_device; a first call under stream capture
+ * returns DXH_ERR_NOT_READY. */
+#define DXH_SUM_NOALLOC_SCRATCH_BYTES (4u << 20)
+DXH_API int dxh_sum_noalloc(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *dims,
+                            int ndims, void *out, void *stream);
 
 /* ---- changeshape: changeshape_miaobyte.cuh:16-79.  Pure data movement, bit-exact,
  * chosen by element size, so every dtype above (and bool) is accepted.

@@ -52,6 +52,11 @@ def test_argument_errors_need_no_gpu():
     assert L.dxh_matmul_workspace_bytes(dx.I32, P(256), P(512), P(1024), 1, 64, 64, 64, C.byref(n)) == 0 and n.value == 0
     assert L.dxh_matmul_workspace_bytes(dx.BOOL, P(256), P(512), P(1024), 1, 64, 64, 64, C.byref(n)) == -1
     assert L.dxh_matmul(dx.F32, P(256), P(512), P(1024), 1, 16, 4096, 256, P(100), 1 << 20, None) == -4  # workspace not 256-byte aligned
+    # the sum that allocates nothing refuses what its fixed scratch array cannot hold, before any HIP call
+    assert L.dxh_sum_noalloc(dx.F32, C.c_void_p(256), dx.i32arr([4096, 4096, 16]), 3, dx.i32arr([0, 2]), 2, C.c_void_p(512), None) == -6
+    assert L.dxh_sum_noalloc(dx.F32, C.c_void_p(256), dx.i32arr([64, 64]), 2, dx.i32arr([2]), 1, C.c_void_p(512), None) == -2
+    assert L.dxh_sum_noalloc(dx.BOOL, C.c_void_p(256), dx.i32arr([64, 64]), 2, dx.i32arr([1]), 1, C.c_void_p(512), None) == -1
+    assert L.dxh_error_string(-6).decode().startswith("input needs more scratch")
     # dxh_chain: operand references, op codes, counts, alignment and dtype are checked on the host
     ins = (C.c_void_p * 2)(16, 32)
     op = lambda code, lhs, rhs, out: dx.ChainOp(code, lhs, rhs, dx.scalar(1.0), out)

@@ -43,6 +43,9 @@ def main():
                          "about 30 ms of load to reach its steady clocks")
     ap.add_argument("--no-per-op", action="store_true", help="skip the per-op table of the other configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--matmul-only", metavar="MxKxN", default="",
+                    help="run only the bf16 matmul of that shape, --steps launches after a clock ramp "
+                         "(the program a counter collection wraps) and print its own JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this executor path runs on ONE GPU (no sharding, no collectives); "
@@ -81,6 +84,28 @@ def main():
 
     def ptr(t):
         return C.c_void_p(t.data_ptr())
+
+    if args.matmul_only:
+        mm, kk, nn = (int(x) for x in args.matmul_only.lower().split("x"))
+        Am = torch.randn(mm * kk, device=dev).to(torch.bfloat16)
+        Bm = (torch.randn(kk * nn, device=dev) * 0.02).to(torch.bfloat16)
+        Cm = torch.empty(mm * nn, device=dev, dtype=torch.bfloat16)
+        launch = matmul_call(L, dx, torch, dev, dx.BF16, Am, Bm, Cm, mm, kk, nn)
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < args.ramp_ms:
+            launch(0)
+            dx.check(L.dxh_device_sync())
+        a, b = Events().pair()
+        dx.check(L.dxh_event_record(a, None))
+        for i in range(args.steps):
+            dx.check(launch(i), "matmul")
+        dx.check(L.dxh_event_record(b, None))
+        dx.check(L.dxh_event_sync(b))
+        ms = Events.ms(a, b) / args.steps
+        print(json.dumps({"matmul_bf16": args.matmul_only, "launches": args.steps, "us_per_launch": round(ms * 1e3, 2),
+                          "TFLOP/s": round(2 * mm * kk * nn / ms / 1e9, 1), "frac_mfma_bf16": round(2 * mm * kk * nn / ms / 1e9 / MFMA_BF16_PEAK_TF, 4),
+                          "device": name.value.decode()}))
+        return
 
     # ---------------- config 2: the step --------------------------------------------------
     g = torch.Generator(device=dev)

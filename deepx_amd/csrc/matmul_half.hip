@@ -4,20 +4,13 @@
 // K when the output has few tiles; other shapes run the same kernel on zero-padded copies, or,
 // when those would not fit the scratch limit, matmul_mfma_kernel, a plain 128x128x32 tile with
 // element-wise edge handling.
-#include "matmul_common.hpp"
+#include "matmul_half_ops.hpp"
 
 namespace dxh {
 
 constexpr int BM = 128, BN = 128, BK = 32;
 constexpr int LDK = BK + 8;  // padded k-stride (elements) of both LDS tiles: 80 bytes, keeps 16-byte alignment
 
-
-template <typename T, typename V> __device__ inline f32x16 mfma32(V a, V b, f32x16 c) {
-    if constexpr (std::is_same_v<T, bf16_t>)
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    else
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-}
 
 // VEC_A: rows of A are 16-byte aligned (K % 8 == 0, base aligned); VEC_B likewise for B (N % 8 == 0).
 template <typename T, bool VEC_A, bool VEC_B>
@@ -124,23 +117,6 @@ __device__ inline int swz(int row, int chunk) { return chunk ^ ((row ^ (row >> 3
 //   roles  the MFMA runs on (B^T, A^T): a lane of the result then holds 4 consecutive n of one row
 //          m, which packs into 8-byte LDS stores for the epilogue.
 //   map    blockIdx -> tile through tile_of_block (XCD-aware, above).
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-// two fp32 accumulators -> one dword of two bf16/f16, round to nearest even (v_cvt_pk_bf16_f32 /
-// v_cvt_pk_f16_f32); element a in the low half
-template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b) {
-    if constexpr (std::is_same_v<T, bf16_t>) return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
-    else return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, f16x2));
-}
-// Within each group of 16 lanes, lane i passes the address of 4 consecutive 16-bit elements
-// ("row i") and receives element i%4 of rows i/4, 4 + i/4, 8 + i/4, 12 + i/4.
-__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t *p) {
-    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p);
-    return __builtin_bit_cast(u32x2, v);
-}
-
 // the `count` loads of a K step are dealt out over its four k-substeps
 constexpr int part_first(int count, int part) { return count * part / 4; }
 constexpr int part_count(int count, int part) { return count * (part + 1) / 4 - count * part / 4; }
@@ -467,13 +443,23 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
         else if (tiles(128, 64) * 4 >= cus * 3) choice = 2;  // 1024x8192x1024 (128 such tiles): 38 us, 31 us with 256 64x64 tiles
         else choice = 5;
     }
+    // The two one-workgroup-per-CU tiles have a twin whose operands travel straight into LDS
+    // (matmul_half_dma.hip: less power, no LDS store traffic, deeper prefetch; 8192^3 830 -> 785 us,
+    // 4096^3 109 -> 102 us); it needs whole K steps of 32 and C at its own [M][N].
+    const bool dma_ok = fast && ldc < 0 && k % 32 == 0;
+    if (dma_ok && tuning().matmul_tile == 0 && (choice == 4 || choice == 6)) choice = choice == 4 ? 7 : 8;
+    if (dma_ok && (choice == 7 || choice == 8)) {
+        if (sc.planning) return DXH_OK;
+        return launch_matmul_half_dma(std::is_same_v<T, bf16_t> ? DXH_BF16 : DXH_F16, choice == 7 ? 0 : 1, a, b, c, batch, m, k, n, st);
+    }
     if (fast) {
         switch (choice) {
         case 2: return launch_tile<T, 128, 64, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 3: return launch_tile<T, 64, 128, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 4: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 5: return launch_tile<T, 64, 64, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
-        case 6: return launch_tile<T, 192, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
+        case 6: case 8: return launch_tile<T, 192, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
+        case 7: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         }
     }

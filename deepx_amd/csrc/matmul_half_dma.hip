@@ -1,0 +1,230 @@
+// matmul_half_dma.hip — bf16 / f16 GEMM on the matrix pipe with operands that travel from global
+// memory straight into LDS (global_load_lds_dwordx4), never through vector registers.
+//
+// Same tiling idea as matmul_mfma_tile_kernel (matmul_half.hip): workgroup tile TM x TN, 4 waves in
+// a 2 x 2 grid, v_mfma_f32_32x32x16_{bf16,f16} on (B^T, A^T), B transposed by the LDS read.  What
+// differs is the pipeline.  A K step is 32 deep and the tile keeps NS of them in LDS; the loads of
+// K step t + NS - 1 are issued while step t is multiplied, so NS - 1 steps of global latency are
+// hidden (the register-staged kernel hides one step of 64 and spends a register and an LDS store
+// per 16 bytes to do it).  One workgroup barrier per K step.
+//
+// LDS-direct loads write lane L's 16 bytes to (M0 base) + 16 L, a contiguous KiB per wave
+// instruction, so the LDS image is chosen by which global address each lane fetches:
+//   A stage  [TM rows][32 k], 64-byte rows; 16-byte chunk c of row r sits at chunk c ^ ((r >> 2) & 3):
+//            the 16 lanes of one pass of a ds_read_b128 then cover 16 different bank groups.
+//   B stage  [32 k][TN n], rows of TN * 2 bytes; 64-byte group g of row k sits at group g ^ (k & 3):
+//            the transposing read (ds_read_b64_tr_b16) fetches 64 bytes of 4 consecutive rows per
+//            half wave, which then fall on different banks.
+// Requirements (checked by the launcher): K % 32 == 0, N % 8 == 0, 16-byte aligned A, B, C.
+#include "matmul_half_ops.hpp"
+
+namespace dxh {
+
+constexpr int DK = 32;  // K step
+
+// One LDS-direct load: lane's 16 bytes from `base + off` land at LDS byte address lds + 16 * lane.
+// M0 is reserved (the compiler never keeps a value in it across statements), so it is not listed
+// as a clobber.  No "memory" clobber either: ordering against the LDS reads comes from the
+// workgroup barriers around it, and the statement is volatile, so it stays between them.
+__device__ __forceinline__ void dma16(const void *base, uint32_t off, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds));
+}
+template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N)); }
+
+template <typename T, int TM, int TN, int NS>
+__global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int K, int N,
+                                                                TileMap map) {
+    static_assert(TM % 64 == 0 && (TN == 128 || TN == 256), "tile shape");
+    constexpr int FM = TM / 64, FN = TN / 64;       // 32x32 MFMA tiles per wave along m and n
+    constexpr int A_INS = TM / 64, B_INS = TN / 64;  // LDS-direct loads per lane and K step
+    constexpr int NLD = A_INS + B_INS;
+    constexpr int A_BYTES = TM * 64, B_ROWB = TN * 2, STAGE = A_BYTES + DK * B_ROWB;
+    constexpr int LDC = TN + 8;
+    constexpr int LDS_BYTES = (NS * STAGE > TM * LDC * 2) ? NS * STAGE : TM * LDC * 2;
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+    static_assert((NS - 2) * NLD <= 63, "vmcnt field");
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[LDS_BYTES];
+
+    const TileCoord tc = tile_of_block(map);
+    if (!tc.valid) return;
+    const int m0 = tc.tm * TM, n0 = tc.tn * TN;
+    const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6), wm = w >> 1, wn = w & 1;
+    const uint16_t *Ab = reinterpret_cast<const uint16_t *>(A) + ((int64_t)tc.batch * M + m0) * K;
+    const uint16_t *Bb = reinterpret_cast<const uint16_t *>(B) + (int64_t)tc.batch * K * N + n0;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
+
+    // ---- which 16 bytes each lane fetches (byte offsets from the tile's A / B origin at k = 0) ----
+    // Rows past M and columns past N are clamped onto valid memory; their products land in
+    // accumulator rows / columns that the epilogue never stores.
+    uint32_t a_off[A_INS], b_off[B_INS];
+    static_for<A_INS>([&](auto q) __attribute__((always_inline)) {
+        const int r = 16 * (4 * decltype(q)::value + w) + (lane >> 2), c = (lane & 3) ^ ((lane >> 4) & 3);
+        a_off[q] = ((uint32_t)(m0 + r < M ? r : M - 1 - m0) * (uint32_t)K + (uint32_t)c * 8u) * 2u;
+    });
+    constexpr int LPR = TN / 8, RPB = 64 / LPR;  // lanes per B row, B rows per wave instruction
+    static_for<B_INS>([&](auto q) __attribute__((always_inline)) {
+        const int r = RPB * (4 * decltype(q)::value + w) + lane / LPR, p = lane % LPR;
+        const int col = (((p >> 2) ^ (r & 3)) * 4 + (p & 3)) * 8;
+        b_off[q] = ((uint32_t)r * (uint32_t)N + (uint32_t)(n0 + col < N ? col : N - 8 - n0)) * 2u;
+    });
+    // load q of a K step: q < A_INS moves 16 rows of A, the others RPB rows of B
+    auto issue_one = [&](auto q, uint32_t sa, const uint16_t *ag, const uint16_t *bg) __attribute__((always_inline)) {
+        constexpr int i = decltype(q)::value;
+        if constexpr (i < A_INS) dma16(ag, a_off[i], sa + i * 4096);
+        else dma16(bg, b_off[i - A_INS], sa + A_BYTES + (i - A_INS) * 4096);
+    };
+    auto issue = [&](int stage, int kstep) __attribute__((always_inline)) {
+        const uint32_t sa = lds0 + stage * STAGE + w * 1024;
+        const uint16_t *ag = Ab + kstep * DK, *bg = Bb + (int64_t)kstep * DK * N;
+        static_for<NLD>([&](auto q) __attribute__((always_inline)) { issue_one(q, sa, ag, bg); });
+    };
+
+    // ---- fragment reads -----------------------------------------------------------------------
+    const int sw = (lane >> 2) & 3, fch = lane >> 5;
+    const int fa_base = (wm * (TM / 2) + (lane & 31)) * 64;
+    int fa_ch[2];  // byte offset of the lane's chunk in substep 0 / 1
+    fa_ch[0] = ((fch) ^ sw) * 16;
+    fa_ch[1] = ((2 + fch) ^ sw) * 16;
+    const int fb_base = A_BYTES + (8 * fch + sw) * B_ROWB + ((lane & 16) + 4 * (lane & 3)) * 2;
+    int fb_g[FN];
+    static_for<FN>([&](auto j) __attribute__((always_inline)) { fb_g[j] = ((wn * (TN / 64) + decltype(j)::value) ^ sw) * 64; });
+
+    // fragment read r of a substep: r < FM is the A fragment of MFMA row r, the others are the low
+    // and high half (k 0-3 and 4-7 of the lane's eight) of a B fragment
+    u32x4 fa[2][FM], fb[2][FN];
+    auto read_one = [&](auto buf, auto ks, const unsigned char *S, auto r) __attribute__((always_inline)) {
+        constexpr int i = decltype(r)::value;
+        if constexpr (i < FM) {
+            fa[buf][i] = *reinterpret_cast<const u32x4 *>(S + fa_base + fa_ch[decltype(ks)::value] + i * 32 * 64);
+        } else {
+            constexpr int j = (i - FM) / 2, h = (i - FM) % 2;
+            const uint16_t *p = reinterpret_cast<const uint16_t *>(S + fb_base + fb_g[j] + decltype(ks)::value * 16 * B_ROWB) + h * 4 * TN;
+            const u32x2 v = lds_read_tr16(p);
+            if constexpr (h == 0) { fb[buf][j].x = v.x; fb[buf][j].y = v.y; }
+            else { fb[buf][j].z = v.x; fb[buf][j].w = v.y; }
+        }
+    };
+
+    f32x16 acc[FM][FN];
+    static_for<FM>([&](auto i) __attribute__((always_inline)) {
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        });
+    });
+    constexpr int NM = FM * FN, ND = FM + 2 * FN;
+    auto mma = [&](auto buf, auto lo, auto hi) __attribute__((always_inline)) {
+        static_for<decltype(hi)::value - decltype(lo)::value>([&](auto x) __attribute__((always_inline)) {
+            constexpr int idx = decltype(lo)::value + decltype(x)::value, i = idx / FN, j = idx % FN;
+            acc[i][j] = mfma32<T>(fb[buf][j], fa[buf][i], acc[i][j]);
+        });
+    };
+
+    const int KT = K / DK;
+    auto k_of = [&](int s) __attribute__((always_inline)) { return s < KT ? s : KT - 1; };
+    // steps past the end fetch the last step again: the count of loads in flight stays the same
+    // on every trip, and the copies land in stages that nobody reads any more
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s) issue(s, k_of(s));
+
+    // K step t: its stage is complete once at most (NS - 2) steps' loads are still in flight; the
+    // barrier makes every wave's part of it visible and tells that all waves are done with stage
+    // t - 1, which the loads of step t + NS - 1 then overwrite.  Substep 1 of step t - 1 straddles
+    // the barrier: its second half of MFMAs runs under the first fragment reads of step t.
+    //
+    // A phase of the K step: `nm` MFMAs of fragment buffer `mb` starting at `m0`, `nr` fragment
+    // reads into buffer `rb` for substep `rks` starting at read `r0`, `nd` loads starting at load
+    // `d0`, cut into groups of (one load, a few MFMAs, their share of the reads) whose order is
+    // pinned.  Spreading the loads matters: four waves that issue all their loads at once right
+    // after the barrier wait on the vector memory queue instead of feeding the matrix pipe
+    // (8192^3: matrix pipe 62 % busy with the loads in one burst, 870 -> 785 us spread out).
+    int stage = 0, fill = NS - 1;
+    uint32_t sa_fill = 0;
+    const uint16_t *ag_fill = Ab, *bg_fill = Bb;
+    const unsigned char *S_cur = lds;
+    auto phase = [&](auto mb, auto m0_, auto nm_, auto rb, auto rks, auto r0_, auto nr_, auto d0_, auto nd_) __attribute__((always_inline)) {
+        constexpr int m0 = decltype(m0_)::value, nm = decltype(nm_)::value, r0 = decltype(r0_)::value, nr = decltype(nr_)::value;
+        constexpr int d0 = decltype(d0_)::value, nd = decltype(nd_)::value;
+        constexpr int G = nd > 0 ? nd : 1;  // groups
+        static_for<G>([&](auto g_) __attribute__((always_inline)) {
+            constexpr int g = decltype(g_)::value;
+            constexpr int ma = nm * g / G, mz = nm * (g + 1) / G, ra = nr * g / G, rz = nr * (g + 1) / G;
+            if constexpr (nd > 0) issue_one(ic<d0 + g>{}, sa_fill, ag_fill, bg_fill);
+            static_for<rz - ra>([&](auto x) __attribute__((always_inline)) { read_one(rb, rks, S_cur, ic<r0 + ra + decltype(x)::value>{}); });
+            mma(mb, ic<m0 + ma>{}, ic<m0 + mz>{});
+            if constexpr (mz > ma) interleave(ic<mz - ma>{}, ic<rz - ra>{}, ic<0>{}, ic<0>{});
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    constexpr int D1 = NLD / 4, D2 = NLD / 2, D3 = NLD - D1 - D2;  // loads in the three phases
+    auto enter = [&](int kt) __attribute__((always_inline)) {
+        wait_loads<(NS - 2) * NLD>();
+        __syncthreads();
+        const int ks = k_of(kt + NS - 1);
+        sa_fill = lds0 + fill * STAGE + w * 1024;
+        ag_fill = Ab + ks * DK;
+        bg_fill = Bb + (int64_t)ks * DK * N;
+        S_cur = lds + stage * STAGE;
+    };
+    auto rest = [&]() __attribute__((always_inline)) {
+        phase(ic<0>{}, ic<0>{}, ic<NM>{}, ic<1>{}, ic<1>{}, ic<0>{}, ic<ND>{}, ic<D1>{}, ic<D2>{});
+        phase(ic<1>{}, ic<0>{}, ic<NM / 2>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<D1 + D2>{}, ic<D3>{});
+        stage = stage + 1 == NS ? 0 : stage + 1;
+        fill = fill + 1 == NS ? 0 : fill + 1;
+    };
+    enter(0);
+    // first step: nothing to multiply yet under the first fragment reads
+    phase(ic<1>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<ND>{}, ic<0>{}, ic<D1>{});
+    rest();
+    for (int kt = 1; kt < KT; ++kt) {
+        enter(kt);
+        phase(ic<1>{}, ic<NM / 2>{}, ic<NM - NM / 2>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<ND>{}, ic<0>{}, ic<D1>{});
+        rest();
+    }
+    mma(ic<1>{}, ic<NM / 2>{}, ic<NM>{});
+    wait_loads<0>();  // the refetched tail steps must have landed before the C tile reuses the LDS
+    __syncthreads();
+
+    // ---- epilogue: result lane holds row m = lane%32 of its MFMA tile and, per group g of 4
+    // registers, columns 8g + 4*(lane/32) .. +3: one 8-byte LDS store each, then 16-byte row stores
+    uint16_t *Cs = reinterpret_cast<uint16_t *>(lds);
+    static_for<FM>([&](auto i) __attribute__((always_inline)) {
+        static_for<FN>([&](auto j) __attribute__((always_inline)) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int row = wm * (TM / 2) + 32 * i + (lane & 31);
+                const int col = wn * (TN / 2) + 32 * j + 8 * g + 4 * (lane >> 5);
+                *reinterpret_cast<u32x2 *>(Cs + row * LDC + col) =
+                    u32x2{pack2<T>(acc[i][j][4 * g], acc[i][j][4 * g + 1]), pack2<T>(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3])};
+            }
+        });
+    });
+    __syncthreads();
+    uint16_t *Cr = reinterpret_cast<uint16_t *>(C) + (int64_t)tc.batch * M * N;
+    constexpr int CB = TN / 8;
+#pragma unroll
+    for (int i = 0; i < TM * CB / kBlock; ++i) {
+        const int c = t + i * kBlock, row = c / CB, ch = c % CB;
+        const int gm = m0 + row, gn = n0 + ch * 8;
+        if (gm < M && gn < N)  // N % 8 == 0: a chunk is either fully inside or fully outside
+            st_nt(reinterpret_cast<uint4 *>(Cr + (int64_t)gm * N + gn), *reinterpret_cast<const uint4 *>(Cs + row * LDC + ch * 8));
+    }
+}
+
+template <typename T, int TM, int TN, int NS>
+static int launch_dma_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    TileMap map;
+    if (!make_tile_map(batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
+    matmul_dma_kernel<T, TM, TN, NS><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map);
+    return launch_status();
+}
+
+// shape: 0 = 256x256, 1 = 192x256.  The caller has checked K % 32 == 0, N % 8 == 0, the alignment
+// of a, b, c and that every byte offset inside a tile fits 32 bits.
+int launch_matmul_half_dma(int dtype, int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    if (dtype == DXH_BF16)
+        return shape == 0 ? launch_dma_tile<bf16_t, 256, 256, 4>(a, b, c, batch, m, k, n, st) : launch_dma_tile<bf16_t, 192, 256, 5>(a, b, c, batch, m, k, n, st);
+    return shape == 0 ? launch_dma_tile<f16_t, 256, 256, 4>(a, b, c, batch, m, k, n, st) : launch_dma_tile<f16_t, 192, 256, 5>(a, b, c, batch, m, k, n, st);
+}
+
+}  // namespace dxh

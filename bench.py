@@ -30,7 +30,18 @@ HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 MFMA_F32_PEAK_TF = 157.3
 MFMA_F64_PEAK_TF = 78.6
 MFMA_BF16_PEAK_TF = 2500.0  # dense bf16
-REDUCE_ROW_TRAFFIC_BYTES = 268585444
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")  # HBM bytes per launch from the counter runs
+
+
+def measured_traffic(kernel):
+    """HBM bytes per launch of `kernel` as the last counter collection found them (rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size; the summary beside the file
+    says how), or None when the file has no entry for it."""
+    try:
+        with open(TRAFFIC_JSON) as f:
+            return json.load(f)["kernels"][kernel]["hbm_bytes_per_launch"]
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def main():
@@ -213,7 +224,7 @@ def main():
                 "bytes_per_launch": XB,
                 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the
                 # reading of a plain copy kernel of known size (profiles/bench_pmc_hbm_traffic.md)
-                "traffic": REDUCE_ROW_TRAFFIC_BYTES}
+                "traffic": measured_traffic("reduce_row_kernel f32 [8192,8192] axis 1")}
 
     # ---------------- the other BASELINE configs, one op at a time ----------------------------
     per_op = {"config2": c2}
@@ -236,10 +247,26 @@ def main():
                    "bytes_per_step": step_bytes, "input_copies_rotated": NX, "clock_ramp_ms_before_warmup": args.ramp_ms,
                    "device": name.value.decode()},
         "roofline": roofline,
+        "roofline_matmul": roofline_matmul(per_op),
         "cpu_baseline": cpu,
         "per_op": per_op,
     }
     print(json.dumps(line))
+
+
+def roofline_matmul(per_op):
+    """The kernel furthest from its roofline, beside the headline one: the bf16 GEMMs of config 5
+    against the dense bf16 matrix-pipe peak, from the per-op pass (None when that pass was skipped)."""
+    c5 = per_op.get("config5")
+    if not c5:
+        return None
+    shapes = {k: v for k, v in c5.items() if k.startswith("matmul_bf16_")}
+    worst = min(shapes, key=lambda k: shapes[k]["TFLOP/s"])
+    return {"bound": "mfma", "kernel": "bf16 matmul, fp32 accumulate (config 5); `achieved` is the slower of the two shapes",
+            "achieved": shapes[worst]["TFLOP/s"], "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
+            "frac": round(shapes[worst]["TFLOP/s"] / MFMA_BF16_PEAK_TF, 4), "shape": worst,
+            "per_shape": {k: {"TFLOP/s": v["TFLOP/s"], "frac": v["frac_mfma_bf16"], "ms": v["ms"]} for k, v in shapes.items()},
+            "traffic": measured_traffic("matmul bf16 " + worst.split("_")[-1])}
 
 
 RAMP_MS = 40.0  # untimed launches before every measurement: from idle the clocks take ~30 ms of load to settle
@@ -276,6 +303,19 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
         if flops is not None:
             e.update({"TFLOP/s": round(flops / ms / 1e9, 2), peak_name: round(flops / ms / 1e9 / peak_tf, 4), "flops": flops})
         return e
+
+    # ---- the floor under every small op: one launch of a kernel with nothing to do (a fill of one
+    # element), timed like every op below (back-to-back launches between two events), and the round
+    # trip of launching it and waiting for it (what a caller that needs each result pays per op)
+    one = torch.empty(64, device=dev)
+    zero = dx.scalar(0.0)
+    floor_ms = time_op(L, dx, torch, Events, ev, lambda i: L.dxh_constant(dx.F32, ptr(one), 1, zero, None), reps=200)
+    t0 = time.perf_counter()
+    for _ in range(500):
+        L.dxh_constant(dx.F32, ptr(one), 1, zero, None)
+        L.dxh_stream_sync(None)
+    res["launch_floor"] = {"back_to_back_us": round(floor_ms * 1e3, 2), "launch_and_wait_us": round((time.perf_counter() - t0) / 500 * 1e6, 2),
+                           "note": "ops whose time is within a microsecond or two of back_to_back_us are launch-bound, not bandwidth-bound"}
 
     # ---- config 1: fp32 [4096,4096] elementwise chain; 4 rotating buffer sets (64 MiB tensors)
     n = 4096 * 4096
@@ -427,22 +467,28 @@ def _executor_lib():
     E.dxe_execute_batch.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_size_t]
     E.dxe_set_graphs.argtypes = [C.c_void_p, C.c_int]
     E.dxe_set_fusion.argtypes = [C.c_void_p, C.c_int]
+    E.dxe_set_sync.argtypes = [C.c_void_p, C.c_int]
     return E
 
 
 def lines_over_ir(setup, block, iters=30):
     """`block` (deepxIR lines) through the executor's dispatch core in this process (libdxexec.so, the
-    code behind the UDP server): wall time per pass when the lines are executed one by one, as one
+    code behind the UDP server): wall time per pass when the lines are executed one by one (replies
+    at launch, as op-cuda sends them, and with a wait for the device before every reply), as one
     batch, as one batch with runs of float elementwise lines fused into single launches, and as a
-    recorded HIP graph without and with those fused runs.  Every mode gets a fresh executor (a
-    recorded graph is keyed by the text of the batch)."""
+    recorded HIP graph without and with those fused runs.  The timed region of every mode ends with
+    a wait for the device.  Every mode gets a fresh executor (a recorded graph is keyed by the text
+    of the batch)."""
     import ctypes as C
+    from deepx_amd import lib as dx
+    L = dx.load()
     E = _executor_lib()
     lines = [f"{l} // author=miaobyte id={i + 1}" for i, l in enumerate(block)]
     text = "\n".join(lines).encode()
     out = {"ops": len(lines)}
-    for label, batched, fused, graphs in (("line_by_line_us", 0, 0, 0), ("one_batch_us", 1, 0, 0), ("one_batch_fused_us", 1, 1, 0),
-                                          ("recorded_graph_us", 1, 0, 1), ("recorded_graph_fused_us", 1, 1, 1)):
+    for label, batched, fused, graphs, wait in (("line_by_line_us", 0, 0, 0, 0), ("line_by_line_waiting_for_each_us", 0, 0, 0, 1),
+                                                ("one_batch_us", 1, 0, 0, 0), ("one_batch_fused_us", 1, 1, 0, 0),
+                                                ("recorded_graph_us", 1, 0, 1, 0), ("recorded_graph_fused_us", 1, 1, 1, 0)):
         ex = E.dxe_create()
         buf = C.create_string_buffer(1 << 16)
         for line in setup:
@@ -452,6 +498,7 @@ def lines_over_ir(setup, block, iters=30):
                 raise RuntimeError(f"{line}: {reply}")
         E.dxe_set_graphs(ex, graphs)
         E.dxe_set_fusion(ex, fused)
+        E.dxe_set_sync(ex, wait)
 
         def once():
             if batched:
@@ -462,9 +509,11 @@ def lines_over_ir(setup, block, iters=30):
 
         for _ in range(4):
             once()
+        dx.check(L.dxh_device_sync())
         t0 = time.perf_counter()
         for _ in range(iters):
             once()
+        dx.check(L.dxh_device_sync())
         out[label] = round((time.perf_counter() - t0) / iters * 1e6, 1)
         if any(" ok" not in r.split("//")[0] for r in buf.value.decode().split("\n")):
             raise RuntimeError("block failed: " + buf.value.decode())

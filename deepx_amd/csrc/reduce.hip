@@ -300,7 +300,21 @@ __global__ __launch_bounds__(kBlock) void reduce_col_fused_kernel(const Tin *__r
     if (active) {
         const A *q = part + p * S * post + cv * V;
         auto ld = [&](int s, int k) __attribute__((always_inline)) { return __hip_atomic_load(q + (int64_t)s * post + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+        // every load of a batch is issued before the first is used: the partials come from memory
+        // (past the L2), and a lane that waited for them one by one would add a memory round trip
+        // per slice to the end of the launch
         int s = ty;
+        for (; s + 7 * TY < S; s += 8 * TY) {
+            A x[8][V];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int k = 0; k < V; ++k) x[u][k] = ld(s + u * TY, k);
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int k = 0; k < V; ++k) acc[k] = rop<K, A>(acc[k], x[u][k]);
+        }
         for (; s + 3 * TY < S; s += 4 * TY) {
             A x[4][V];
 #pragma unroll
@@ -522,6 +536,9 @@ inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, cons
             int G = vecs >= (int64_t)kBlock * loads ? kBlock : (int)std::min<int64_t>(kWave, pow2_ceil((vecs + loads - 1) / loads));
             // very short rows: at least 4 lanes (64 contiguous bytes) per row keep a wave's loads coalesced
             G = std::max<int>(G, (int)std::min<int64_t>(4, pow2_ceil(vecs)));
+            // a small input: rather fewer vectors per lane than fewer workgroups than two per CU
+            // (fp32 [8192,64]: 4 lanes per row make 128 workgroups, 16 lanes per row 512)
+            while (G < kWave && G < pow2_ceil(vecs) && (pre + (kBlock / G) - 1) / (kBlock / G) < 2 * kCUs) G <<= 1;
             int64_t blocks0 = (pre + (kBlock / G) - 1) / (kBlock / G);
             if (G == kBlock && blocks0 < kTarget) {
                 int64_t min_chunk = 8192;  // elements: 8+ vector trips per lane
@@ -536,11 +553,20 @@ inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, cons
             int TX = col_lanes(pre, postv, true);
             int TY = kBlock / TX;
             int64_t blocks0 = pre * ((postv + TX - 1) / TX);
-            const int64_t col_target = tuning().reduce_col_target_blocks;
+            // One workgroup per CU is the fastest split when it comes out as a single full round
+            // (fp32 [8192,8192]: 64 column tiles x 4 slices = 256 workgroups, 44 us; 45 us with 1024).
+            // When the tiles do not divide the CUs like that, a few workgroups too many would run
+            // as a second, nearly empty round: then four times as many, smaller ones keep every CU
+            // busy to the end (fp32 [8192,8256]: 260 workgroups 60 us, 1040 workgroups 49 us).
+            int64_t col_target = tuning().reduce_col_target_blocks;
+            const int64_t min_rows = (int64_t)TY * tuning().reduce_col_min_rows;
+            const int64_t smax = std::max<int64_t>(1, R / min_rows);
             if (blocks0 < col_target) {
-                int64_t min_rows = (int64_t)TY * tuning().reduce_col_min_rows;
-                int64_t smax = std::max<int64_t>(1, R / min_rows);
                 S = (int)std::min<int64_t>((col_target + blocks0 - 1) / blocks0, smax);
+                if (blocks0 * S > col_target && col_target == kCUs) {
+                    col_target *= 4;
+                    S = (int)std::min<int64_t>((col_target + blocks0 - 1) / blocks0, smax);
+                }
             }
             if (S == 1) st.may_split = false;  // nothing to split: narrow TX for parallelism instead
         }

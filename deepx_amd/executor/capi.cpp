@@ -38,6 +38,8 @@ DXE_API size_t dxe_execute_batch(void *ex, const char *text, char *reply, size_t
     for (const std::string &r : static_cast<Executor *>(ex)->execute_batch(lines)) { if (!out.empty()) out += '\n'; out += r; }
     return copy_out(out, reply, buflen);
 }
+// wait for the device before every reply (the DEEPX_SYNC switch; default off = reply at launch, like op-cuda)
+DXE_API void dxe_set_sync(void *ex, int on) { static_cast<Executor *>(ex)->sync_each = on != 0; }
 // graph recording on/off (the DEEPX_GRAPH switch) and the batch counters: "batches captures replays rejects"
 DXE_API void dxe_set_graphs(void *ex, int on) { static_cast<Executor *>(ex)->use_graphs = on != 0; }
 // one launch for runs of float elementwise lines inside a batch (the DEEPX_FUSE switch), and its counters: "runs lines"
@@ -45,6 +47,15 @@ DXE_API void dxe_set_fusion(void *ex, int on) { static_cast<Executor *>(ex)->use
 DXE_API size_t dxe_fusion_stats(void *ex, char *out, size_t buflen) {
     const auto &s = static_cast<Executor *>(ex)->stats;
     return copy_out(std::to_string(s.fused_runs) + " " + std::to_string(s.fused_lines), out, buflen);
+}
+// host-time breakdown of execute() (see Executor::Profile): on/off, and "lines parse match run sync reply" in ns; reading resets
+DXE_API void dxe_set_profile(void *ex, int on) { static_cast<Executor *>(ex)->profile = on != 0; }
+DXE_API size_t dxe_profile(void *ex, char *out, size_t buflen) {
+    auto &p = static_cast<Executor *>(ex)->prof;
+    const std::string s = std::to_string(p.lines) + " " + std::to_string(p.parse_ns) + " " + std::to_string(p.match_ns) + " " +
+                          std::to_string(p.run_ns) + " " + std::to_string(p.sync_ns) + " " + std::to_string(p.reply_ns);
+    p = Executor::Profile{};
+    return copy_out(s, out, buflen);
 }
 DXE_API size_t dxe_stats(void *ex, char *out, size_t buflen) {
     const auto &s = static_cast<Executor *>(ex)->stats;

@@ -26,7 +26,13 @@ public:
     Mem mem;
     TfFactory factory;
     bool ir_log = false;    // DEEPX_IR_LOG=1|true echoes every instruction (main.cpp:17-21)
-    bool sync_each = true;  // wait for the kernels before stamping finish_at; DEEPX_SYNC=0 replies at launch like op-cuda
+    // Replies go out when the kernels of a line have been launched, as op-cuda's do (its main loop
+    // never waits for the device, executor/op-cuda/src/client/main.cpp:60-104): kernels of later
+    // lines queue up behind them on the same stream, and every op that hands data to the host
+    // (save, print) waits for the device itself.  One launch-and-wait round trip costs 11.5 us on
+    // this runtime whatever the kernel, 250 us of a 22-line block.  DEEPX_SYNC=1 waits for the
+    // device before every reply (finish_at is then the end of the kernels, as on op-ompsimd).
+    bool sync_each = false;
     bool has_device = false;
     // DEEPX_GRAPH=1: a datagram of several graph-safe lines that arrives a second time is recorded
     // into a HIP graph and replayed from then on (one launch instead of one per kernel)
@@ -36,27 +42,43 @@ public:
     // not read back from memory.  DEEPX_FUSE=0 turns it off.
     bool use_fusion = true;
     struct Stats { uint64_t batches = 0, graph_captures = 0, graph_replays = 0, graph_rejects = 0, fused_runs = 0, fused_lines = 0; } stats;
+    // Where the host time of a line goes (steady clock, nanoseconds summed over `lines` calls of
+    // execute()): parsing the text, finding and cloning the registered op, its wrapper up to the
+    // kernel launch, the wait for the device, formatting the reply.  Off unless DEEPX_PROFILE=1.
+    bool profile = false;
+    struct Profile { uint64_t lines = 0, parse_ns = 0, match_ns = 0, run_ns = 0, sync_ns = 0, reply_ns = 0; } prof;
 
     Executor() {
         register_all(factory);
         const char *e = std::getenv("DEEPX_IR_LOG");
         ir_log = e && (!std::strcmp(e, "1") || !strcasecmp(e, "true"));
         const char *s = std::getenv("DEEPX_SYNC");
-        if (s && !std::strcmp(s, "0")) sync_each = false;
+        if (s) sync_each = !std::strcmp(s, "1");
         int count = 0;
         has_device = dxh_device_count(&count) == DXH_OK && count > 0;
         const char *g = std::getenv("DEEPX_GRAPH");
         use_graphs = g && !std::strcmp(g, "1");
+        const char *pr = std::getenv("DEEPX_PROFILE");
+        profile = pr && !std::strcmp(pr, "1");
         const char *fuse = std::getenv("DEEPX_FUSE");
         if (fuse && !std::strcmp(fuse, "0")) use_fusion = false;
     }
     ~Executor() {
-        for (auto &kv : graphs_) dxh_graph_destroy(kv.second.exec);
+        for (auto &kv : graphs_) drop_graph(kv.second);
         if (graph_stream_) dxh_stream_destroy(graph_stream_);
     }
 
     std::string execute(const std::string &line, TimePoint recv_at = std::chrono::system_clock::now()) {
         std::lock_guard<std::mutex> lock(mu_);
+        using Clock = std::chrono::steady_clock;
+        Clock::time_point mark = profile ? Clock::now() : Clock::time_point();
+        auto lap = [&](uint64_t &slot) {
+            if (!profile) return;
+            const Clock::time_point now = Clock::now();
+            slot += (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(now - mark).count();
+            mark = now;
+        };
+        if (profile) ++prof.lines;
         OpResp resp;
         resp.recv_at = recv_at;
         resp.start_at = recv_at;
@@ -67,6 +89,7 @@ public:
             resp.error(e.what());
             return resp.to_string();
         }
+        lap(prof.parse_ns);
         call.metadata.recv_at = recv_at;
         resp.id = call.metadata.id;
         if (ir_log) std::cout << "~" << call.to_string(true) << std::endl;
@@ -80,22 +103,27 @@ public:
         tf->name = call.name;
         tf->args = call.args;
         tf->returns = call.returns;
+        lap(prof.match_ns);
         resp.start_at = std::chrono::system_clock::now();
         int rc = 0;
         std::string message;
         const int repeat = tf->metadata.benchmark_repeat > 1 ? tf->metadata.benchmark_repeat : 1;
         for (int i = 0; i < repeat && rc == 0; ++i) rc = tf->run(mem, message);
+        lap(prof.run_ns);
         if (rc == 0 && sync_each && has_device) {
             int s = dxh_stream_sync(nullptr);
             if (s != DXH_OK) { rc = 1; message = std::string("hip: ") + dxh_error_string(s); }
         }
+        lap(prof.sync_ns);
         if (rc != 0) {
             std::cerr << message << std::endl;
             resp.error(message);
         } else {
             resp.finish("");
         }
-        return resp.to_string();
+        std::string reply = resp.to_string();
+        lap(prof.reply_ns);
+        return reply;
     }
 
     // All lines of one datagram (udpserver.cpp:49-58 splits them the same way), one reply per line,
@@ -297,8 +325,14 @@ private:
         }
         return true;
     }
+    // a replay may still be running when replies are sent at launch: wait before its graph goes away
+    void drop_graph(Graph &g) {
+        if (graph_stream_) dxh_stream_sync(graph_stream_);
+        dxh_graph_destroy(g.exec);
+        g.exec = nullptr;
+    }
     bool launch_graph(const Graph &g) {
-        return dxh_graph_launch(g.exec, graph_stream_) == DXH_OK && dxh_stream_sync(graph_stream_) == DXH_OK;
+        return dxh_graph_launch(g.exec, graph_stream_) == DXH_OK && (!sync_each || dxh_stream_sync(graph_stream_) == DXH_OK);
     }
     static bool same_pins(const Graph &a, const Graph &b) {
         if (a.workspace != b.workspace || a.tensors.size() != b.tensors.size()) return false;
@@ -324,7 +358,7 @@ private:
         }
         auto it = graphs_.find(key);
         if (it != graphs_.end() && !same_pins(it->second, now)) {
-            dxh_graph_destroy(it->second.exec);
+            drop_graph(it->second);
             graphs_.erase(it);
             it = graphs_.end();
         }
@@ -350,7 +384,7 @@ private:
                 return false;
             }
             if (graphs_.size() >= 64) {  // bounded cache: start over rather than track recency
-                for (auto &kv : graphs_) dxh_graph_destroy(kv.second.exec);
+                for (auto &kv : graphs_) drop_graph(kv.second);
                 graphs_.clear();
             }
             now.exec = exec;
@@ -359,8 +393,8 @@ private:
         } else {
             ++stats.graph_replays;
         }
-        if (dxh_graph_launch(it->second.exec, graph_stream_) != DXH_OK || dxh_stream_sync(graph_stream_) != DXH_OK) {
-            dxh_graph_destroy(it->second.exec);
+        if (dxh_graph_launch(it->second.exec, graph_stream_) != DXH_OK || (sync_each && dxh_stream_sync(graph_stream_) != DXH_OK)) {
+            drop_graph(it->second);
             graphs_.erase(it);
             rejected_.insert(key);
             return false;

@@ -35,6 +35,7 @@ class InProc:
         L.dxe_set_graphs.argtypes = [C.c_void_p, C.c_int]
         L.dxe_set_fusion.argtypes = [C.c_void_p, C.c_int]
         L.dxe_print_format_ok.argtypes = [C.c_char_p, C.c_int]
+        L.dxe_set_sync.argtypes = [C.c_void_p, C.c_int]
         self.L = L
         self.ex = L.dxe_create()
         assert self.ex
@@ -48,6 +49,7 @@ class InProc:
     def execute_batch(self, lines): return self._call(self.L.dxe_execute_batch, self.ex, "\n".join(lines).encode()).split("\n")
     def set_graphs(self, on): self.L.dxe_set_graphs(self.ex, int(on))
     def set_fusion(self, on): self.L.dxe_set_fusion(self.ex, int(on))
+    def set_sync(self, on): self.L.dxe_set_sync(self.ex, int(on))
 
     def fusion_stats(self):
         runs, lines = (int(x) for x in self._call(self.L.dxe_fusion_stats, self.ex).split())

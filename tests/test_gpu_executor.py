@@ -291,3 +291,29 @@ def test_benchmark_repeat_and_timestamps(srv, tmp_path):
     r = srv.must("add", [T("ba"), T("ba")], [T("ba")], extra="benchmark.repeat=3")
     assert np.all(fetch(srv, tmp_path, "ba")[0] == 8.0)  # 1 -> 2 -> 4 -> 8
     assert r.times["recv_at"] <= r.times["start_at"] <= r.times["finish_at"]
+
+
+def test_waiting_for_the_device_before_each_reply(tmp_path):
+    """DEEPX_SYNC=1: every reply is sent after the kernels of its line have finished (the default
+    replies at launch, as op-cuda does).  Same results either way; with the wait, finish_at of a
+    long op lies after its start_at by at least the kernel's run time."""
+    rng = np.random.default_rng(5)
+    a = rng.uniform(-1, 1, (512, 512)).astype(np.float32)
+    want = None
+    for env in ({"DEEPX_SYNC": "1"}, {}):
+        s = UdpExecutor(env=env)
+        try:
+            load(s, tmp_path, "sy_a", a, "float32")
+            s.must("newtensor", [V([512, 512])], [T("sy_c")], author="")
+            s.must("matmul", [T("sy_a"), T("sy_a")], [T("sy_c")], author="cublas")
+            s.must("exp", [T("sy_c")], [T("sy_c")])
+            got = fetch(s, tmp_path, "sy_c")[0]
+        finally:
+            s.close()
+        assert s.proc.returncode == 0
+        if want is None:
+            want = got
+            ref = np.exp(a.astype(np.float64) @ a.astype(np.float64))
+            assert np.allclose(got, ref, rtol=1e-4)
+        else:
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32))

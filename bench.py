@@ -57,6 +57,7 @@ def main():
     ap.add_argument("--matmul-only", metavar="MxKxN", default="",
                     help="run only the bf16 matmul of that shape, --steps launches after a clock ramp "
                          "(the program a counter collection wraps) and print its own JSON line")
+    ap.add_argument("--matmul-tile", type=int, default=0, help="with --matmul-only: force a workgroup tile (DXH_TUNE_MATMUL_TILE), 0 = chosen per shape")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this executor path runs on ONE GPU (no sharding, no collectives); "
@@ -101,6 +102,7 @@ def main():
         Am = torch.randn(mm * kk, device=dev).to(torch.bfloat16)
         Bm = (torch.randn(kk * nn, device=dev) * 0.02).to(torch.bfloat16)
         Cm = torch.empty(mm * nn, device=dev, dtype=torch.bfloat16)
+        dx.check(L.dxh_tune(4, args.matmul_tile), "DXH_TUNE_MATMUL_TILE")
         launch = matmul_call(L, dx, torch, dev, dx.BF16, Am, Bm, Cm, mm, kk, nn)
         t0 = time.perf_counter()
         while (time.perf_counter() - t0) * 1e3 < args.ramp_ms:
@@ -113,7 +115,7 @@ def main():
         dx.check(L.dxh_event_record(b, None))
         dx.check(L.dxh_event_sync(b))
         ms = Events.ms(a, b) / args.steps
-        print(json.dumps({"matmul_bf16": args.matmul_only, "launches": args.steps, "us_per_launch": round(ms * 1e3, 2),
+        print(json.dumps({"matmul_bf16": args.matmul_only, "tile_knob": args.matmul_tile, "launches": args.steps, "us_per_launch": round(ms * 1e3, 2),
                           "TFLOP/s": round(2 * mm * kk * nn / ms / 1e9, 1), "frac_mfma_bf16": round(2 * mm * kk * nn / ms / 1e9 / MFMA_BF16_PEAK_TF, 4),
                           "device": name.value.decode()}))
         return

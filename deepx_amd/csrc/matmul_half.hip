@@ -444,22 +444,24 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
         else choice = 5;
     }
     // The two one-workgroup-per-CU tiles have a twin whose operands travel straight into LDS
-    // (matmul_half_dma.hip: less power, no LDS store traffic, deeper prefetch; 8192^3 830 -> 785 us,
-    // 4096^3 109 -> 102 us); it needs whole K steps of 32 and C at its own [M][N].
-    const bool dma_ok = fast && ldc < 0 && k % 32 == 0;
-    if (dma_ok && tuning().matmul_tile == 0 && (choice == 4 || choice == 6)) choice = choice == 4 ? 7 : 8;
-    if (dma_ok && (choice == 7 || choice == 8)) {
+    // (matmul_half_dma.hip: less power, no LDS store traffic, deeper prefetch; 8192^3 830 -> 782 us,
+    // 4096^3 109 -> 102 us); it needs whole K steps of 64 and C at its own [M][N].  Its 256x256 tile
+    // runs two LDS stages of K 64 when K is long (whole cache lines of A, half the barriers) and four
+    // of K 32 when it is short (2048x896x4864: 21.2 against 22.6 us with the shallow pipeline).
+    const bool dma_ok = fast && ldc < 0 && k % 64 == 0;
+    if (dma_ok && tuning().matmul_tile == 0 && (choice == 4 || choice == 6)) choice = choice == 6 ? 8 : k >= 2048 ? 10 : 7;
+    if (dma_ok && choice >= 7 && choice <= 10) {
         if (sc.planning) return DXH_OK;
-        return launch_matmul_half_dma(std::is_same_v<T, bf16_t> ? DXH_BF16 : DXH_F16, choice == 7 ? 0 : 1, a, b, c, batch, m, k, n, st);
+        return launch_matmul_half_dma(std::is_same_v<T, bf16_t> ? DXH_BF16 : DXH_F16, (int)choice - 7, a, b, c, batch, m, k, n, st);
     }
     if (fast) {
         switch (choice) {
-        case 2: return launch_tile<T, 128, 64, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
+        case 2: case 9: return launch_tile<T, 128, 64, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 3: return launch_tile<T, 64, 128, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 4: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 5: return launch_tile<T, 64, 64, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 6: case 8: return launch_tile<T, 192, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
-        case 7: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
+        case 7: case 10: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         }
     }

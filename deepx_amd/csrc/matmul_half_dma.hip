@@ -3,24 +3,28 @@
 //
 // Same tiling idea as matmul_mfma_tile_kernel (matmul_half.hip): workgroup tile TM x TN, 4 waves in
 // a 2 x 2 grid, v_mfma_f32_32x32x16_{bf16,f16} on (B^T, A^T), B transposed by the LDS read.  What
-// differs is the pipeline.  A K step is 32 deep and the tile keeps NS of them in LDS; the loads of
-// K step t + NS - 1 are issued while step t is multiplied, so NS - 1 steps of global latency are
-// hidden (the register-staged kernel hides one step of 64 and spends a register and an LDS store
-// per 16 bytes to do it).  One workgroup barrier per K step.
+// differs is the pipeline.  The tile keeps NS K steps of DK (32 or 64) in LDS; the loads of K step
+// t + NS - 1 are issued, one between every few MFMAs, while step t is multiplied, so NS - 1 steps
+// of global latency are hidden without a register or an LDS store per 16 bytes.  LDS-direct loads
+// fill LDS at the vector cache's 64 bytes per clock without taking read bandwidth from the
+// fragment reads (ds_write_b128 at that rate leaves them 93 of 132 bytes per clock), and the
+// kernel draws less power: 8192^3 ran at 1.97 GHz against 1.83 GHz for the register-staged one.
+// One workgroup barrier per K step.
 //
 // LDS-direct loads write lane L's 16 bytes to (M0 base) + 16 L, a contiguous KiB per wave
 // instruction, so the LDS image is chosen by which global address each lane fetches:
-//   A stage  [TM rows][32 k], 64-byte rows; 16-byte chunk c of row r sits at chunk c ^ ((r >> 2) & 3):
-//            the 16 lanes of one pass of a ds_read_b128 then cover 16 different bank groups.
-//   B stage  [32 k][TN n], rows of TN * 2 bytes; 64-byte group g of row k sits at group g ^ (k & 3):
-//            the transposing read (ds_read_b64_tr_b16) fetches 64 bytes of 4 consecutive rows per
-//            half wave, which then fall on different banks.
-// Requirements (checked by the launcher): K % 32 == 0, N % 8 == 0, 16-byte aligned A, B, C.
+//   A stage  [TM rows][DK k]; 16-byte chunk c of row r sits at chunk c ^ ((r >> 2) & 3) in 64-byte
+//            rows (DK 32) and at c ^ ((r >> 1) & 7) in 128-byte rows (DK 64): the 16 lanes of one
+//            pass of a ds_read_b128 then cover 16 different bank groups.  DK 64 fetches whole
+//            128-byte cache lines of A; DK 32 half lines, twice.
+//   B stage  [DK k][TN n], rows of TN * 2 bytes; 64-byte group g of row k sits at group g ^ (k & 3)
+//            (g ^ ((k >> 1) & 1) in the 128-byte rows of TN 64): the transposing read
+//            (ds_read_b64_tr_b16) fetches 64 bytes of 4 consecutive rows per half wave, which then
+//            fall on different banks.
+// Requirements (checked by the launcher): K % DK == 0, N % 8 == 0, 16-byte aligned A, B, C.
 #include "matmul_half_ops.hpp"
 
 namespace dxh {
-
-constexpr int DK = 32;  // K step
 
 // One LDS-direct load: lane's 16 bytes from `base + off` land at LDS byte address lds + 16 * lane.
 // M0 is reserved (the compiler never keeps a value in it across statements), so it is not listed
@@ -31,14 +35,16 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t off, uint32_t l
 }
 template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N)); }
 
-template <typename T, int TM, int TN, int NS>
+template <typename T, int TM, int TN, int DK, int NS>
 __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int K, int N,
                                                                 TileMap map) {
-    static_assert(TM % 64 == 0 && (TN == 128 || TN == 256), "tile shape");
-    constexpr int FM = TM / 64, FN = TN / 64;       // 32x32 MFMA tiles per wave along m and n
-    constexpr int A_INS = TM / 64, B_INS = TN / 64;  // LDS-direct loads per lane and K step
+    static_assert(TM % 64 == 0 && (TN == 64 || TN == 128 || TN == 256) && (DK == 32 || DK == 64), "tile shape");
+    constexpr int FM = TM / 64, FN = TN / 64;  // 32x32 MFMA tiles per wave along m and n
+    constexpr int KS = DK / 16;                // k-substeps (one MFMA depth each) per K step
+    constexpr int A_ROWB = DK * 2;             // bytes of an A row in LDS
+    constexpr int A_INS = TM * A_ROWB / 4096, B_INS = DK * TN * 2 / 4096;  // LDS-direct loads per lane and K step
     constexpr int NLD = A_INS + B_INS;
-    constexpr int A_BYTES = TM * 64, B_ROWB = TN * 2, STAGE = A_BYTES + DK * B_ROWB;
+    constexpr int A_BYTES = TM * A_ROWB, B_ROWB = TN * 2, STAGE = A_BYTES + DK * B_ROWB;
     constexpr int LDC = TN + 8;
     constexpr int LDS_BYTES = (NS * STAGE > TM * LDC * 2) ? NS * STAGE : TM * LDC * 2;
     static_assert(LDS_BYTES <= 160 * 1024, "LDS");
@@ -57,14 +63,24 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
     // Rows past M and columns past N are clamped onto valid memory; their products land in
     // accumulator rows / columns that the epilogue never stores.
     uint32_t a_off[A_INS], b_off[B_INS];
+    // A rows of 64 bytes (K step 32): a wave instruction covers 16 rows, chunk c of row r sits at
+    // c ^ ((r >> 2) & 3).  Rows of 128 bytes (K step 64): 8 rows, chunk c at c ^ ((r >> 1) & 7).
+    // Either way the 16 lanes of one pass of a ds_read_b128 fall on 16 different bank groups.
     static_for<A_INS>([&](auto q) __attribute__((always_inline)) {
-        const int r = 16 * (4 * decltype(q)::value + w) + (lane >> 2), c = (lane & 3) ^ ((lane >> 4) & 3);
+        constexpr int blk4 = 4 * decltype(q)::value;
+        int r, c;
+        if constexpr (DK == 32) { r = 16 * (blk4 + w) + (lane >> 2); c = (lane & 3) ^ ((r >> 2) & 3); }
+        else { r = 8 * (blk4 + w) + (lane >> 3); c = (lane & 7) ^ ((r >> 1) & 7); }
         a_off[q] = ((uint32_t)(m0 + r < M ? r : M - 1 - m0) * (uint32_t)K + (uint32_t)c * 8u) * 2u;
     });
     constexpr int LPR = TN / 8, RPB = 64 / LPR;  // lanes per B row, B rows per wave instruction
+    // B rows of 256 bytes and more hold four 64-byte groups or a multiple: group g of row k sits at
+    // g ^ (k & 3).  A 128-byte row (TN 64) has two: g ^ ((k >> 1) & 1), which still spreads the four
+    // rows of a transposing read over all banks (rows k and k + 2 are 256 bytes apart).
+    auto bswz = [](int k) __attribute__((always_inline)) { return TN >= 128 ? (k & 3) : ((k >> 1) & 1); };
     static_for<B_INS>([&](auto q) __attribute__((always_inline)) {
         const int r = RPB * (4 * decltype(q)::value + w) + lane / LPR, p = lane % LPR;
-        const int col = (((p >> 2) ^ (r & 3)) * 4 + (p & 3)) * 8;
+        const int col = (((p >> 2) ^ bswz(r)) * 4 + (p & 3)) * 8;
         b_off[q] = ((uint32_t)r * (uint32_t)N + (uint32_t)(n0 + col < N ? col : N - 8 - n0)) * 2u;
     });
     // load q of a K step: q < A_INS moves 16 rows of A, the others RPB rows of B
@@ -81,13 +97,13 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
 
     // ---- fragment reads -----------------------------------------------------------------------
     const int sw = (lane >> 2) & 3, fch = lane >> 5;
-    const int fa_base = (wm * (TM / 2) + (lane & 31)) * 64;
-    int fa_ch[2];  // byte offset of the lane's chunk in substep 0 / 1
-    fa_ch[0] = ((fch) ^ sw) * 16;
-    fa_ch[1] = ((2 + fch) ^ sw) * 16;
+    const int fa_base = (wm * (TM / 2) + (lane & 31)) * A_ROWB;
+    const int swa = DK == 32 ? sw : (lane >> 1) & 7;  // the A row's swizzle term: rows of a wave tile start at multiples of 32
+    int fa_ch[KS];  // byte offset of the lane's chunk in each substep
+    static_for<KS>([&](auto ks) __attribute__((always_inline)) { fa_ch[ks] = ((2 * decltype(ks)::value + fch) ^ swa) * 16; });
     const int fb_base = A_BYTES + (8 * fch + sw) * B_ROWB + ((lane & 16) + 4 * (lane & 3)) * 2;
     int fb_g[FN];
-    static_for<FN>([&](auto j) __attribute__((always_inline)) { fb_g[j] = ((wn * (TN / 64) + decltype(j)::value) ^ sw) * 64; });
+    static_for<FN>([&](auto j) __attribute__((always_inline)) { fb_g[j] = ((wn * (TN / 64) + decltype(j)::value) ^ bswz(sw)) * 64; });
 
     // fragment read r of a substep: r < FM is the A fragment of MFMA row r, the others are the low
     // and high half (k 0-3 and 4-7 of the lane's eight) of a B fragment
@@ -95,7 +111,7 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
     auto read_one = [&](auto buf, auto ks, const unsigned char *S, auto r) __attribute__((always_inline)) {
         constexpr int i = decltype(r)::value;
         if constexpr (i < FM) {
-            fa[buf][i] = *reinterpret_cast<const u32x4 *>(S + fa_base + fa_ch[decltype(ks)::value] + i * 32 * 64);
+            fa[buf][i] = *reinterpret_cast<const u32x4 *>(S + fa_base + fa_ch[decltype(ks)::value] + i * 32 * A_ROWB);
         } else {
             constexpr int j = (i - FM) / 2, h = (i - FM) % 2;
             const uint16_t *p = reinterpret_cast<const uint16_t *>(S + fb_base + fb_g[j] + decltype(ks)::value * 16 * B_ROWB) + h * 4 * TN;
@@ -156,7 +172,12 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
             __builtin_amdgcn_sched_barrier(0);
         });
     };
-    constexpr int D1 = NLD / 4, D2 = NLD / 2, D3 = NLD - D1 - D2;  // loads in the three phases
+    // The K step as phases: [second half of the previous step's last substep | first reads of this
+    // step], then one phase per substep but the last [its MFMAs | the next substep's reads], then
+    // [first half of the last substep].  Loads are dealt out in proportion to the MFMAs of a phase.
+    constexpr int TOTAL = KS * NM;                                      // MFMAs per K step
+    constexpr auto load_at = [](int mfmas_before) { return NLD * mfmas_before / TOTAL; };
+    constexpr int H = NM / 2;                                           // MFMAs after the barrier of the straddling substep
     auto enter = [&](int kt) __attribute__((always_inline)) {
         wait_loads<(NS - 2) * NLD>();
         __syncthreads();
@@ -167,21 +188,26 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
         S_cur = lds + stage * STAGE;
     };
     auto rest = [&]() __attribute__((always_inline)) {
-        phase(ic<0>{}, ic<0>{}, ic<NM>{}, ic<1>{}, ic<1>{}, ic<0>{}, ic<ND>{}, ic<D1>{}, ic<D2>{});
-        phase(ic<1>{}, ic<0>{}, ic<NM / 2>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<D1 + D2>{}, ic<D3>{});
+        static_for<KS - 1>([&](auto ks_) __attribute__((always_inline)) {
+            constexpr int ks = decltype(ks_)::value, before = (NM - H) + ks * NM;
+            phase(ic<ks & 1>{}, ic<0>{}, ic<NM>{}, ic<(ks + 1) & 1>{}, ic<ks + 1>{}, ic<0>{}, ic<ND>{}, ic<load_at(before)>{},
+                  ic<load_at(before + NM) - load_at(before)>{});
+        });
+        constexpr int before = (NM - H) + (KS - 1) * NM;
+        phase(ic<(KS - 1) & 1>{}, ic<0>{}, ic<H>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<load_at(before)>{}, ic<NLD - load_at(before)>{});
         stage = stage + 1 == NS ? 0 : stage + 1;
         fill = fill + 1 == NS ? 0 : fill + 1;
     };
     enter(0);
     // first step: nothing to multiply yet under the first fragment reads
-    phase(ic<1>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<ND>{}, ic<0>{}, ic<D1>{});
+    phase(ic<1>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<ND>{}, ic<0>{}, ic<load_at(NM - H)>{});
     rest();
     for (int kt = 1; kt < KT; ++kt) {
         enter(kt);
-        phase(ic<1>{}, ic<NM / 2>{}, ic<NM - NM / 2>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<ND>{}, ic<0>{}, ic<D1>{});
+        phase(ic<(KS - 1) & 1>{}, ic<H>{}, ic<NM - H>{}, ic<0>{}, ic<0>{}, ic<0>{}, ic<ND>{}, ic<0>{}, ic<load_at(NM - H)>{});
         rest();
     }
-    mma(ic<1>{}, ic<NM / 2>{}, ic<NM>{});
+    mma(ic<(KS - 1) & 1>{}, ic<H>{}, ic<NM>{});
     wait_loads<0>();  // the refetched tail steps must have landed before the C tile reuses the LDS
     __syncthreads();
 
@@ -211,20 +237,28 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
     }
 }
 
-template <typename T, int TM, int TN, int NS>
+template <typename T, int TM, int TN, int DK, int NS>
 static int launch_dma_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     TileMap map;
     if (!make_tile_map(batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
-    matmul_dma_kernel<T, TM, TN, NS><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map);
+    matmul_dma_kernel<T, TM, TN, DK, NS><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map);
     return launch_status();
 }
 
-// shape: 0 = 256x256, 1 = 192x256.  The caller has checked K % 32 == 0, N % 8 == 0, the alignment
-// of a, b, c and that every byte offset inside a tile fits 32 bits.
+// shape: 0 = 256x256 in K steps of 32, 1 = 192x256 / 32, 2 = 128x64 / 64, 3 = 256x256 / 64.  The caller has
+// checked K % 64 == 0, N % 8 == 0, the alignment of a, b, c and that every byte offset inside a tile
+// fits 32 bits.
+template <typename T>
+static int launch_dma_shape(int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+    switch (shape) {
+    case 0: return launch_dma_tile<T, 256, 256, 32, 4>(a, b, c, batch, m, k, n, st);
+    case 1: return launch_dma_tile<T, 192, 256, 32, 5>(a, b, c, batch, m, k, n, st);
+    case 3: return launch_dma_tile<T, 256, 256, 64, 2>(a, b, c, batch, m, k, n, st);
+    default: return launch_dma_tile<T, 128, 64, 64, 5>(a, b, c, batch, m, k, n, st);
+    }
+}
 int launch_matmul_half_dma(int dtype, int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    if (dtype == DXH_BF16)
-        return shape == 0 ? launch_dma_tile<bf16_t, 256, 256, 4>(a, b, c, batch, m, k, n, st) : launch_dma_tile<bf16_t, 192, 256, 5>(a, b, c, batch, m, k, n, st);
-    return shape == 0 ? launch_dma_tile<f16_t, 256, 256, 4>(a, b, c, batch, m, k, n, st) : launch_dma_tile<f16_t, 192, 256, 5>(a, b, c, batch, m, k, n, st);
+    return dtype == DXH_BF16 ? launch_dma_shape<bf16_t>(shape, a, b, c, batch, m, k, n, st) : launch_dma_shape<f16_t>(shape, a, b, c, batch, m, k, n, st);
 }
 
 }  // namespace dxh

@@ -84,7 +84,7 @@ def test_config5_gemm_shapes_bf16(dxh, orc):
 TILE_KNOB = 4  # DXH_TUNE_MATMUL_TILE
 
 
-@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10])
 @pytest.mark.parametrize("dtype", [dx.BF16, dx.F16])
 def test_matmul_tile_configs(dxh, dtype, tile):
     """Every workgroup tile of the MFMA kernel (forced through the tuning knob) on aligned shapes
@@ -123,7 +123,7 @@ def test_matmul_tiles_exact_on_small_integers(dxh):
         B = H.to_storage(Bi.astype(np.float64).reshape(-1), dx.BF16)
         want = (Ai @ Bi).astype(np.float64)  # |sum| <= 16*256 = 4096: exact in fp32
         dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, np.uint16)
-        for tile in (0, 1, 2, 3, 4, 5, 6, 7, 8):
+        for tile in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10):
             dx.check(dxh.dxh_tune(TILE_KNOB, tile))
             try:
                 dx.check(H.matmul(dxh, dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))

@@ -31,11 +31,21 @@ __host__ __device__ inline float load_acc(bf16_t x) { return bits_to_float(uint3
 __host__ __device__ inline float load_acc(f16_t x) { return float(__builtin_bit_cast(_Float16, x.bits)); }
 template <typename T> __host__ __device__ inline T load_acc(T x) { return x; }
 
+// fp32 -> bf16, round to nearest even, NaN kept quiet.  The device has an instruction for it
+// (v_cvt_pk_bf16_f32, two values at a time) whose result equals the arithmetic below for every one of
+// the 2^32 inputs, NaN payloads included (checked exhaustively on the GPU); the host computes it.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
 __host__ __device__ inline bf16_t to_bf16(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return bf16_t{uint16_t(__builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{f, f}, bf16x2_t)))};
+#else
     uint32_t u = float_to_bits(f);
     if ((u & 0x7fffffffu) > 0x7f800000u) return bf16_t{uint16_t((u >> 16) | 0x0040u)};
     u += 0x7fffu + ((u >> 16) & 1u);
     return bf16_t{uint16_t(u >> 16)};
+#endif
 }
 __host__ __device__ inline f16_t to_f16(float f) {
     return f16_t{__builtin_bit_cast(uint16_t, (_Float16)f)};  // v_cvt_f16_f32, RNE
@@ -45,6 +55,12 @@ template <typename T> __host__ __device__ inline T store_acc(acc_t<T> v) {
     else if constexpr (std::is_same_v<T, f16_t>) return to_f16(v);
     else return v;
 }
+
+// V results of an op -> one vector of the storage type.  16-bit floats are converted two at a time
+// (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32, both round to nearest even): one instruction per dword of
+// the vector instead of a conversion and a merge per element.
+template <typename T, int V> struct alignas(sizeof(T) * V) vec_t;
+template <typename T, int V> __device__ __forceinline__ void store_acc_vec(vec_t<T, V> &r, const acc_t<T> (&x)[V]);
 
 // scalar operand -> storage type, mirroring T(std::stof(text)) upstream of the ABI
 template <typename T> inline T scalar_to(const dxh_scalar &s) {
@@ -56,6 +72,19 @@ template <typename T> inline T scalar_to(const dxh_scalar &s) {
 
 // ---- 16-byte vectors -------------------------------------------------------------------
 template <typename T, int N> struct alignas(sizeof(T) * N) vec_t { T v[N]; };
+template <typename T, int V> __device__ __forceinline__ void store_acc_vec(vec_t<T, V> &r, const acc_t<T> (&x)[V]) {
+    if constexpr ((std::is_same_v<T, bf16_t> || std::is_same_v<T, f16_t>) && V % 2 == 0) {
+        uint32_t *w = reinterpret_cast<uint32_t *>(r.v);
+#pragma unroll
+        for (int k = 0; k < V / 2; ++k) {
+            if constexpr (std::is_same_v<T, bf16_t>) w[k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{x[2 * k], x[2 * k + 1]}, bf16x2_t));
+            else w[k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{x[2 * k], x[2 * k + 1]}, f16x2_t));
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(x[k]);
+    }
+}
 template <typename T> constexpr int vec_len = kVecBytes / (int)sizeof(T);
 
 template <int BYTES> struct raw_of;

@@ -92,8 +92,10 @@ __device__ __forceinline__ void binary_body(const T *__restrict__ a, const T *__
             int64_t j = i + u * kBlock;
             if (decltype(full)::value || j < nv) {
                 VT r;
+                A t[V];
 #pragma unroll
-                for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(A(load_acc(x[u].v[k])), A(load_acc(y[u].v[k]))));
+                for (int k = 0; k < V; ++k) t[k] = Op::f(A(load_acc(x[u].v[k])), A(load_acc(y[u].v[k])));
+                store_acc_vec<T, V>(r, t);
                 st_mode<ST>(&vc[j], r);
             }
         }
@@ -137,8 +139,10 @@ __device__ __forceinline__ void scalar_body(const T *__restrict__ a, const T s, 
             int64_t j = i + u * kBlock;
             if (decltype(full)::value || j < nv) {
                 VT r;
+                A t[V];
 #pragma unroll
-                for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(A(load_acc(x[u].v[k])), sv));
+                for (int k = 0; k < V; ++k) t[k] = Op::f(A(load_acc(x[u].v[k])), sv);
+                store_acc_vec<T, V>(r, t);
                 st_sel<NTS>(&vc[j], r);
             }
         }
@@ -173,8 +177,10 @@ __device__ __forceinline__ void unary_body(const T *__restrict__ a, T *__restric
             int64_t j = i + u * kBlock;
             if (decltype(full)::value || j < nv) {
                 VT r;
+                acc_t<T> t[V];
 #pragma unroll
-                for (int k = 0; k < V; ++k) r.v[k] = store_acc<T>(Op::f(load_acc(x[u].v[k])));
+                for (int k = 0; k < V; ++k) t[k] = Op::f(load_acc(x[u].v[k]));
+                store_acc_vec<T, V>(r, t);
                 st_sel<NTS>(&vc[j], r);
             }
         }
@@ -364,9 +370,10 @@ __global__ __launch_bounds__(kBlock) void chain_kernel(const ChainArgs p, int64_
             const VT a = __builtin_bit_cast(VT, ra), b = __builtin_bit_cast(VT, rb);
             const A s = A(s_scalar[k]);
             VT r;
-#define DXH_CH_BIN(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) r.v[v] = store_acc<T>(Op::f(A(load_acc(a.v[v])), A(load_acc(b.v[v])))); break
-#define DXH_CH_SCALAR(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) r.v[v] = store_acc<T>(Op::f(A(load_acc(a.v[v])), s)); break
-#define DXH_CH_UNARY(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) r.v[v] = store_acc<T>(Op::f(load_acc(a.v[v]))); break
+            A y[V];
+#define DXH_CH_BIN(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) y[v] = Op::f(A(load_acc(a.v[v])), A(load_acc(b.v[v]))); break
+#define DXH_CH_SCALAR(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) y[v] = Op::f(A(load_acc(a.v[v])), s); break
+#define DXH_CH_UNARY(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) y[v] = Op::f(load_acc(a.v[v])); break
             switch (code) {
             case DXH_CHAIN_ADD: DXH_CH_BIN(OpAdd);
             case DXH_CHAIN_SUB: DXH_CH_BIN(OpSub);
@@ -389,6 +396,7 @@ __global__ __launch_bounds__(kBlock) void chain_kernel(const ChainArgs p, int64_
 #undef DXH_CH_BIN
 #undef DXH_CH_SCALAR
 #undef DXH_CH_UNARY
+            store_acc_vec<T, V>(r, y);
             prev = __builtin_bit_cast(u32x4_t, r);
             if (save >= 0) raw[save * kBlock + t] = prev;
             if (s_out[k]) __builtin_nontemporal_store(prev, &reinterpret_cast<u32x4_t *>(s_out[k])[i]);

@@ -414,6 +414,7 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
         const int rc = launch_split<T>(a, b, c, batch, m, k, n, st, sc);
         if (rc != kNoSplit) return rc;
     }
+    const bool dma_ok = fast && ldc < 0 && k % 64 == 0;
     if (fast && choice == 0) {
         // 256x256 tiles halve the bytes every CU pulls through its vector cache per flop, but need
         // about one tile per CU to pay off.  Below that, 128x128 tiles (two workgroups per CU) as
@@ -439,6 +440,15 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
             const double edge = ldc >= 0 ? 5.0 : 0.0;  // element-wise C stores make the burst at the end of a round longer
             const double c4 = one_per_cu(256, 256, 1.645, 3.5 + edge), c6 = one_per_cu(192, 256, 1.21, 6.0 + edge);
             choice = (c1 <= c4 && c1 <= c6) ? 1 : (c4 <= c6) ? 4 : 6;
+            // Lower tiles of the same width, one wave per 64 columns (matmul_half_dma.hip only): when a
+            // lower tile still fits the output into one round, every CU's K loop gets shorter
+            // (2048x896x4864: 18.2 us with 160 rows, 19.8 with 192; 2048x4096x4096: 56.9 us with 128
+            // rows, 63.4 with 192, hipBLASLt 70.9).
+            if (dma_ok) {
+                const double c11 = one_per_cu(160, 256, 1.0, 5.5), c12 = one_per_cu(128, 256, 0.89, 5.0);
+                const double best = choice == 1 ? c1 : choice == 4 ? c4 : c6;
+                if (c11 < best || c12 < best) choice = c12 <= c11 ? 12 : 11;
+            }
         }
         else if (tiles(128, 64) * 4 >= cus * 3) choice = 2;  // 1024x8192x1024 (128 such tiles): 38 us, 31 us with 256 64x64 tiles
         else choice = 5;
@@ -448,9 +458,8 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
     // 4096^3 109 -> 102 us); it needs whole K steps of 64 and C at its own [M][N].  Its 256x256 tile
     // runs two LDS stages of K 64 when K is long (whole cache lines of A, half the barriers) and four
     // of K 32 when it is short (2048x896x4864: 21.2 against 22.6 us with the shallow pipeline).
-    const bool dma_ok = fast && ldc < 0 && k % 64 == 0;
     if (dma_ok && tuning().matmul_tile == 0 && (choice == 4 || choice == 6)) choice = choice == 6 ? 8 : k >= 2048 ? 10 : 7;
-    if (dma_ok && choice >= 7 && choice <= 10) {
+    if (dma_ok && choice >= 7 && choice <= 12) {
         if (sc.planning) return DXH_OK;
         return launch_matmul_half_dma(std::is_same_v<T, bf16_t> ? DXH_BF16 : DXH_F16, (int)choice - 7, a, b, c, batch, m, k, n, st);
     }
@@ -460,7 +469,7 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
         case 3: return launch_tile<T, 64, 128, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 4: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 5: return launch_tile<T, 64, 64, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
-        case 6: case 8: return launch_tile<T, 192, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
+        case 6: case 8: case 11: case 12: return launch_tile<T, 192, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 7: case 10: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         }

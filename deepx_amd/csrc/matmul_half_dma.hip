@@ -35,14 +35,20 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t off, uint32_t l
 }
 template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N)); }
 
-template <typename T, int TM, int TN, int DK, int NS>
+template <typename T, int TM, int TN, int DK, int NS, int WN = 2>
 __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int K, int N,
                                                                 TileMap map) {
-    static_assert(TM % 64 == 0 && (TN == 64 || TN == 128 || TN == 256) && (DK == 32 || DK == 64), "tile shape");
-    constexpr int FM = TM / 64, FN = TN / 64;  // 32x32 MFMA tiles per wave along m and n
-    constexpr int KS = DK / 16;                // k-substeps (one MFMA depth each) per K step
-    constexpr int A_ROWB = DK * 2;             // bytes of an A row in LDS
-    constexpr int A_INS = TM * A_ROWB / 4096, B_INS = DK * TN * 2 / 4096;  // LDS-direct loads per lane and K step
+    // the four waves form a WM x WN grid over the tile: 2 x 2, or 1 x 4 for a tile height that is
+    // a multiple of 32 but not of 64
+    constexpr int WM = 4 / WN, WTM = TM / WM, WTN = TN / WN;
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && (TN == 64 || TN == 128 || TN == 256) && (DK == 32 || DK == 64), "tile shape");
+    constexpr int FM = WTM / 32, FN = WTN / 32;  // 32x32 MFMA tiles per wave along m and n
+    constexpr int KS = DK / 16;                  // k-substeps (one MFMA depth each) per K step
+    constexpr int A_ROWB = DK * 2;               // bytes of an A row in LDS
+    // LDS-direct loads per lane and K step.  A tile whose KiB blocks do not divide by four waves is
+    // rounded up: the waves left over fetch the last block once more (same data to the same place),
+    // so that every wave has the same number of loads in flight and one vmcnt value fits all.
+    constexpr int A_BLOCKS = TM * A_ROWB / 1024, A_INS = (A_BLOCKS + 3) / 4, B_INS = DK * TN * 2 / 4096;
     constexpr int NLD = A_INS + B_INS;
     constexpr int A_BYTES = TM * A_ROWB, B_ROWB = TN * 2, STAGE = A_BYTES + DK * B_ROWB;
     constexpr int LDC = TN + 8;
@@ -54,7 +60,7 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
     const TileCoord tc = tile_of_block(map);
     if (!tc.valid) return;
     const int m0 = tc.tm * TM, n0 = tc.tn * TN;
-    const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6), wm = w >> 1, wn = w & 1;
+    const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6), wm = w / WN, wn = w % WN;
     const uint16_t *Ab = reinterpret_cast<const uint16_t *>(A) + ((int64_t)tc.batch * M + m0) * K;
     const uint16_t *Bb = reinterpret_cast<const uint16_t *>(B) + (int64_t)tc.batch * K * N + n0;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
@@ -66,12 +72,14 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
     // A rows of 64 bytes (K step 32): a wave instruction covers 16 rows, chunk c of row r sits at
     // c ^ ((r >> 2) & 3).  Rows of 128 bytes (K step 64): 8 rows, chunk c at c ^ ((r >> 1) & 7).
     // Either way the 16 lanes of one pass of a ds_read_b128 fall on 16 different bank groups.
+    uint32_t a_lds[A_INS];  // byte offset of the load's KiB block inside the A stage
     static_for<A_INS>([&](auto q) __attribute__((always_inline)) {
-        constexpr int blk4 = 4 * decltype(q)::value;
+        const int blk = 4 * decltype(q)::value + w < A_BLOCKS ? 4 * decltype(q)::value + w : A_BLOCKS - 1;
         int r, c;
-        if constexpr (DK == 32) { r = 16 * (blk4 + w) + (lane >> 2); c = (lane & 3) ^ ((r >> 2) & 3); }
-        else { r = 8 * (blk4 + w) + (lane >> 3); c = (lane & 7) ^ ((r >> 1) & 7); }
+        if constexpr (DK == 32) { r = 16 * blk + (lane >> 2); c = (lane & 3) ^ ((r >> 2) & 3); }
+        else { r = 8 * blk + (lane >> 3); c = (lane & 7) ^ ((r >> 1) & 7); }
         a_off[q] = ((uint32_t)(m0 + r < M ? r : M - 1 - m0) * (uint32_t)K + (uint32_t)c * 8u) * 2u;
+        a_lds[q] = (uint32_t)blk * 1024u;
     });
     constexpr int LPR = TN / 8, RPB = 64 / LPR;  // lanes per B row, B rows per wave instruction
     // B rows of 256 bytes and more hold four 64-byte groups or a multiple: group g of row k sits at
@@ -86,24 +94,24 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
     // load q of a K step: q < A_INS moves 16 rows of A, the others RPB rows of B
     auto issue_one = [&](auto q, uint32_t sa, const uint16_t *ag, const uint16_t *bg) __attribute__((always_inline)) {
         constexpr int i = decltype(q)::value;
-        if constexpr (i < A_INS) dma16(ag, a_off[i], sa + i * 4096);
-        else dma16(bg, b_off[i - A_INS], sa + A_BYTES + (i - A_INS) * 4096);
+        if constexpr (i < A_INS) dma16(ag, a_off[i], sa + a_lds[i]);
+        else dma16(bg, b_off[i - A_INS], sa + w * 1024 + A_BYTES + (i - A_INS) * 4096);
     };
     auto issue = [&](int stage, int kstep) __attribute__((always_inline)) {
-        const uint32_t sa = lds0 + stage * STAGE + w * 1024;
+        const uint32_t sa = lds0 + stage * STAGE;
         const uint16_t *ag = Ab + kstep * DK, *bg = Bb + (int64_t)kstep * DK * N;
         static_for<NLD>([&](auto q) __attribute__((always_inline)) { issue_one(q, sa, ag, bg); });
     };
 
     // ---- fragment reads -----------------------------------------------------------------------
     const int sw = (lane >> 2) & 3, fch = lane >> 5;
-    const int fa_base = (wm * (TM / 2) + (lane & 31)) * A_ROWB;
+    const int fa_base = (wm * WTM + (lane & 31)) * A_ROWB;
     const int swa = DK == 32 ? sw : (lane >> 1) & 7;  // the A row's swizzle term: rows of a wave tile start at multiples of 32
     int fa_ch[KS];  // byte offset of the lane's chunk in each substep
     static_for<KS>([&](auto ks) __attribute__((always_inline)) { fa_ch[ks] = ((2 * decltype(ks)::value + fch) ^ swa) * 16; });
     const int fb_base = A_BYTES + (8 * fch + sw) * B_ROWB + ((lane & 16) + 4 * (lane & 3)) * 2;
     int fb_g[FN];
-    static_for<FN>([&](auto j) __attribute__((always_inline)) { fb_g[j] = ((wn * (TN / 64) + decltype(j)::value) ^ bswz(sw)) * 64; });
+    static_for<FN>([&](auto j) __attribute__((always_inline)) { fb_g[j] = ((wn * (WTN / 32) + decltype(j)::value) ^ bswz(sw)) * 64; });
 
     // fragment read r of a substep: r < FM is the A fragment of MFMA row r, the others are the low
     // and high half (k 0-3 and 4-7 of the lane's eight) of a B fragment
@@ -182,7 +190,7 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
         wait_loads<(NS - 2) * NLD>();
         __syncthreads();
         const int ks = k_of(kt + NS - 1);
-        sa_fill = lds0 + fill * STAGE + w * 1024;
+        sa_fill = lds0 + fill * STAGE;
         ag_fill = Ab + ks * DK;
         bg_fill = Bb + (int64_t)ks * DK * N;
         S_cur = lds + stage * STAGE;
@@ -218,8 +226,8 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
         static_for<FN>([&](auto j) __attribute__((always_inline)) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const int row = wm * (TM / 2) + 32 * i + (lane & 31);
-                const int col = wn * (TN / 2) + 32 * j + 8 * g + 4 * (lane >> 5);
+                const int row = wm * WTM + 32 * i + (lane & 31);
+                const int col = wn * WTN + 32 * j + 8 * g + 4 * (lane >> 5);
                 *reinterpret_cast<u32x2 *>(Cs + row * LDC + col) =
                     u32x2{pack2<T>(acc[i][j][4 * g], acc[i][j][4 * g + 1]), pack2<T>(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3])};
             }
@@ -237,11 +245,11 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
     }
 }
 
-template <typename T, int TM, int TN, int DK, int NS>
+template <typename T, int TM, int TN, int DK, int NS, int WN = 2>
 static int launch_dma_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     TileMap map;
     if (!make_tile_map(batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
-    matmul_dma_kernel<T, TM, TN, DK, NS><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map);
+    matmul_dma_kernel<T, TM, TN, DK, NS, WN><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map);
     return launch_status();
 }
 
@@ -254,6 +262,8 @@ static int launch_dma_shape(int shape, const void *a, const void *b, void *c, in
     case 0: return launch_dma_tile<T, 256, 256, 32, 4>(a, b, c, batch, m, k, n, st);
     case 1: return launch_dma_tile<T, 192, 256, 32, 5>(a, b, c, batch, m, k, n, st);
     case 3: return launch_dma_tile<T, 256, 256, 64, 2>(a, b, c, batch, m, k, n, st);
+    case 4: return launch_dma_tile<T, 160, 256, 32, 5, 4>(a, b, c, batch, m, k, n, st);
+    case 5: return launch_dma_tile<T, 128, 256, 32, 5, 4>(a, b, c, batch, m, k, n, st);
     default: return launch_dma_tile<T, 128, 64, 64, 5>(a, b, c, batch, m, k, n, st);
     }
 }

@@ -416,6 +416,146 @@ int launch_chain(ChainArgs &p, const dxh_chain_op *ops, int64_t n, hipStream_t s
     return launch_status();
 }
 
+
+// ---- a run of elementwise ops over a [rows, cols] view, with row / column vectors and casts ------
+// The same interpreter for runs whose tensors differ in dtype (f32, bf16, f16) or in extent: besides
+// [rows, cols] tensors a run may read and write row vectors [1, cols] and column vectors [rows, 1],
+// and its ops include the cast (todtype) and the copy of a vector into every row or column
+// (broadcastTo).  A lane owns four adjacent columns of one row.  Every value is carried as fp32 (a
+// 16-bit float is exact in it) and every result is rounded to its op's dtype before anything uses
+// it, so the stored bits are those of the separate launches.  An op on vectors is computed by every
+// lane for its own row or columns and stored by the lanes of column 0 or row 0 only; a later op of
+// the run that reads the vector has the value at hand, no lane waits for another.  That is also why
+// a vector input must not be an output of the same run: lanes that read it race with the lane that
+// overwrites it.
+enum { kRowFull = 0, kRowVec = 1, kColVec = 2 };
+enum { kRcF32 = 0, kRcBF16 = 1, kRcF16 = 2 };
+struct RowChainArgs {
+    const void *in[kChainInputs];
+    void *out[kChainOps];
+    float scalar[kChainOps];  // already rounded to the op's dtype on the host
+    int8_t in_dtype[kChainInputs], in_kind[kChainInputs];
+    int8_t code[kChainOps], lhs[kChainOps], rhs[kChainOps], save[kChainOps], dtype[kChainOps], kind[kChainOps];
+    int n_in, n_ops;
+};
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x4_t rowchain_load(const void *p, int dt, int kind, int64_t row, int64_t c4, int64_t i) {
+    if (kind == kColVec) {
+        float v;
+        if (dt == kRcF32) v = reinterpret_cast<const float *>(p)[row];
+        else if (dt == kRcBF16) v = load_acc(reinterpret_cast<const bf16_t *>(p)[row]);
+        else v = load_acc(reinterpret_cast<const f16_t *>(p)[row]);
+        return f32x4_t{v, v, v, v};
+    }
+    const int64_t j = kind == kRowVec ? c4 : i;
+    if (dt == kRcF32) return reinterpret_cast<const f32x4_t *>(p)[j];
+    if (dt == kRcBF16) {
+        const vec_t<bf16_t, 4> x = reinterpret_cast<const vec_t<bf16_t, 4> *>(p)[j];
+        return f32x4_t{load_acc(x.v[0]), load_acc(x.v[1]), load_acc(x.v[2]), load_acc(x.v[3])};
+    }
+    const vec_t<f16_t, 4> x = reinterpret_cast<const vec_t<f16_t, 4> *>(p)[j];
+    return f32x4_t{load_acc(x.v[0]), load_acc(x.v[1]), load_acc(x.v[2]), load_acc(x.v[3])};
+}
+// rounds y to the op's dtype (in place, as fp32 again) and stores it where the op's extent says
+__device__ __forceinline__ void rowchain_round_store(float (&y)[4], void *out, int dt, int kind, int64_t row, int64_t c4, int64_t i) {
+    const bool mine = kind == kRowFull || (kind == kRowVec ? row == 0 : c4 == 0);
+    const int64_t j = kind == kRowVec ? c4 : i;
+    if (dt == kRcF32) {
+        if (out && mine) {
+            if (kind == kColVec) reinterpret_cast<float *>(out)[row] = y[0];
+            else reinterpret_cast<f32x4_t *>(out)[j] = f32x4_t{y[0], y[1], y[2], y[3]};
+        }
+    } else if (dt == kRcBF16) {
+        vec_t<bf16_t, 4> r;
+        store_acc_vec<bf16_t, 4>(r, y);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) y[v] = load_acc(r.v[v]);
+        if (out && mine) {
+            if (kind == kColVec) reinterpret_cast<bf16_t *>(out)[row] = r.v[0];
+            else reinterpret_cast<vec_t<bf16_t, 4> *>(out)[j] = r;
+        }
+    } else {
+        vec_t<f16_t, 4> r;
+        store_acc_vec<f16_t, 4>(r, y);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) y[v] = load_acc(r.v[v]);
+        if (out && mine) {
+            if (kind == kColVec) reinterpret_cast<f16_t *>(out)[row] = r.v[0];
+            else reinterpret_cast<vec_t<f16_t, 4> *>(out)[j] = r;
+        }
+    }
+}
+__global__ __launch_bounds__(kBlock) void chain_rows_kernel(const RowChainArgs p, int64_t rows, int64_t cq) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char chain_lds[];
+    const int t = threadIdx.x;
+    // op and input tables in LDS, for the reason given in chain_kernel
+    __shared__ int s_code[kChainOps], s_lhs[kChainOps], s_rhs[kChainOps], s_save[kChainOps], s_dtype[kChainOps], s_kind[kChainOps];
+    __shared__ int s_in_dtype[kChainInputs], s_in_kind[kChainInputs];
+    __shared__ float s_scalar[kChainOps];
+    __shared__ void *s_out[kChainOps];
+    __shared__ const void *s_in[kChainInputs];
+    if (t == 0) {
+#pragma unroll
+        for (int k = 0; k < kChainOps; ++k) {
+            s_code[k] = p.code[k]; s_lhs[k] = p.lhs[k]; s_rhs[k] = p.rhs[k]; s_save[k] = p.save[k];
+            s_dtype[k] = p.dtype[k]; s_kind[k] = p.kind[k]; s_scalar[k] = p.scalar[k]; s_out[k] = p.out[k];
+        }
+#pragma unroll
+        for (int j = 0; j < kChainInputs; ++j) { s_in[j] = p.in[j]; s_in_dtype[j] = p.in_dtype[j]; s_in_kind[j] = p.in_kind[j]; }
+    }
+    __syncthreads();
+    f32x4_t *slot = reinterpret_cast<f32x4_t *>(chain_lds);
+    const int64_t total = rows * cq;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + t; i < total; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t row = i / cq, c4 = i - row * cq;
+        f32x4_t prev = {0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < p.n_in; ++j) {
+            const int dt = __builtin_amdgcn_readfirstlane(s_in_dtype[j]), kind = __builtin_amdgcn_readfirstlane(s_in_kind[j]);
+            slot[j * kBlock + t] = rowchain_load(s_in[j], dt, kind, row, c4, i);
+        }
+        for (int k = 0; k < p.n_ops; ++k) {
+            const int code = __builtin_amdgcn_readfirstlane(s_code[k]), l = __builtin_amdgcn_readfirstlane(s_lhs[k]);
+            const int q = __builtin_amdgcn_readfirstlane(s_rhs[k]), save = __builtin_amdgcn_readfirstlane(s_save[k]);
+            const int dt = __builtin_amdgcn_readfirstlane(s_dtype[k]), kind = __builtin_amdgcn_readfirstlane(s_kind[k]);
+            f32x4_t a = prev, b = prev;
+            if (l != kChainPrev) a = slot[l * kBlock + t];
+            if (q != kChainPrev) b = slot[q * kBlock + t];
+            const float s = s_scalar[k];
+            float y[4];
+#define DXH_RC_BIN(Op) _Pragma("unroll") for (int v = 0; v < 4; ++v) y[v] = Op::f(a[v], b[v]); break
+#define DXH_RC_SCALAR(Op) _Pragma("unroll") for (int v = 0; v < 4; ++v) y[v] = Op::f(a[v], s); break
+#define DXH_RC_UNARY(Op) _Pragma("unroll") for (int v = 0; v < 4; ++v) y[v] = Op::f(a[v]); break
+            switch (code) {
+            case DXH_CHAIN_ADD: DXH_RC_BIN(OpAdd);
+            case DXH_CHAIN_SUB: DXH_RC_BIN(OpSub);
+            case DXH_CHAIN_MUL: DXH_RC_BIN(OpMul);
+            case DXH_CHAIN_DIV: DXH_RC_BIN(OpDiv);
+            case DXH_CHAIN_MAX: DXH_RC_BIN(OpMax);
+            case DXH_CHAIN_MIN: DXH_RC_BIN(OpMin);
+            case DXH_CHAIN_ADDSCALAR: DXH_RC_SCALAR(OpAdd);
+            case DXH_CHAIN_SUBSCALAR: DXH_RC_SCALAR(OpSub);
+            case DXH_CHAIN_RSUBSCALAR: DXH_RC_SCALAR(OpRSub);
+            case DXH_CHAIN_MULSCALAR: DXH_RC_SCALAR(OpMul);
+            case DXH_CHAIN_DIVSCALAR: DXH_RC_SCALAR(OpDiv);
+            case DXH_CHAIN_RDIVSCALAR: DXH_RC_SCALAR(OpRDiv);
+            case DXH_CHAIN_MAXSCALAR: DXH_RC_SCALAR(OpMax);
+            case DXH_CHAIN_MINSCALAR: DXH_RC_SCALAR(OpMin);
+            case DXH_CHAIN_SQRT: DXH_RC_UNARY(OpSqrt);
+            case DXH_CHAIN_EXP: DXH_RC_UNARY(OpExp);
+            case DXH_CHAIN_LOG: DXH_RC_UNARY(OpLog);
+            case DXH_CHAIN_SQUARE: DXH_RC_UNARY(OpSquare);
+            default: _Pragma("unroll") for (int v = 0; v < 4; ++v) y[v] = a[v]; break;  // DXH_CHAIN_COPY
+            }
+#undef DXH_RC_BIN
+#undef DXH_RC_SCALAR
+#undef DXH_RC_UNARY
+            rowchain_round_store(y, s_out[k], dt, kind, row, c4, i);
+            prev = f32x4_t{y[0], y[1], y[2], y[3]};
+            if (save >= 0) slot[save * kBlock + t] = prev;
+        }
+    }
+}
+
 }  // namespace dxh
 
 using namespace dxh;
@@ -508,6 +648,61 @@ int dxh_chain(int dtype, const void *const *inputs, int n_inputs, const dxh_chai
     case DXH_BF16: return launch_chain<bf16_t>(p, ops, n, st);
     default: return DXH_ERR_DTYPE;
     }
+}
+
+
+int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain_rows_op *ops, int n_ops, int64_t rows, int64_t cols, void *stream) {
+    if (rows < 0 || cols < 0 || n_ops < 1 || n_ops > kChainOps || n_inputs < 0 || n_inputs > kChainInputs || !ops || (n_inputs > 0 && !inputs)) return DXH_ERR_ARG;
+    if (cols % 4 != 0) return DXH_ERR_ALIGN;
+    if (rows > 0 && cols / 4 > INT64_MAX / rows) return DXH_ERR_SHAPE;
+    auto dtype_code = [](int dtype) { return dtype == DXH_F32 ? (int)kRcF32 : dtype == DXH_BF16 ? (int)kRcBF16 : dtype == DXH_F16 ? (int)kRcF16 : -1; };
+    // a [rows, cols] tensor or a row vector is touched four elements at a time, a column vector one
+    auto align_of = [](int dt, int kind) { return (size_t)(kind == kColVec ? 1 : 4) * (dt == kRcF32 ? 4 : 2); };
+    RowChainArgs p{};
+    p.n_in = n_inputs;
+    p.n_ops = n_ops;
+    for (int j = 0; j < n_inputs; ++j) {
+        const int dt = dtype_code(inputs[j].dtype);
+        if (dt < 0) return DXH_ERR_DTYPE;
+        if (!inputs[j].data || inputs[j].extent < DXH_CHAIN_FULL || inputs[j].extent > DXH_CHAIN_COLUMN) return DXH_ERR_ARG;
+        if (!aligned(inputs[j].data, align_of(dt, inputs[j].extent))) return DXH_ERR_ALIGN;
+        p.in[j] = inputs[j].data; p.in_dtype[j] = (int8_t)dt; p.in_kind[j] = (int8_t)inputs[j].extent;
+    }
+    int next_slot = n_inputs;
+    for (int k = 0; k < n_ops; ++k) p.save[k] = -1;
+    constexpr int kBad = -2;
+    // operand of op k (see dxh_chain); `want` is the op's extent: a [rows, cols] op takes anything, an op
+    // on vectors only vectors of its own kind
+    auto operand = [&](int ref, int k, int want) {
+        if (ref >= 0 && ref < n_inputs) return want == kRowFull || p.in_kind[ref] == want ? ref : kBad;
+        if (ref < DXH_CHAIN_RESULT || ref >= DXH_CHAIN_RESULT + k) return kBad;
+        const int j = ref - DXH_CHAIN_RESULT;
+        if (want != kRowFull && p.kind[j] != want) return kBad;
+        if (j == k - 1) return kChainPrev;
+        if (p.save[j] < 0) p.save[j] = (int8_t)next_slot++;
+        return (int)p.save[j];
+    };
+    for (int k = 0; k < n_ops; ++k) {
+        const dxh_chain_rows_op &o = ops[k];
+        const int dt = dtype_code(o.dtype);
+        if (dt < 0) return DXH_ERR_DTYPE;
+        if (o.code < DXH_CHAIN_ADD || o.code > DXH_CHAIN_COPY || o.extent < DXH_CHAIN_FULL || o.extent > DXH_CHAIN_COLUMN || (!o.out && k == n_ops - 1)) return DXH_ERR_ARG;
+        if (o.out && !aligned(o.out, align_of(dt, o.extent))) return DXH_ERR_ALIGN;
+        p.kind[k] = (int8_t)o.extent;  // before operand(): a later op asks for it
+        const int l = operand(o.lhs, k, o.extent), r = o.code <= DXH_CHAIN_MIN ? operand(o.rhs, k, o.extent) : l;
+        if (l == kBad || r == kBad) return DXH_ERR_ARG;
+        for (int j = 0; j < n_inputs; ++j)
+            if (o.out && o.out == inputs[j].data && inputs[j].extent != DXH_CHAIN_FULL) return DXH_ERR_ARG;  // lanes would race for it
+        p.code[k] = (int8_t)o.code; p.lhs[k] = (int8_t)l; p.rhs[k] = (int8_t)r; p.out[k] = o.out; p.dtype[k] = (int8_t)dt;
+        const float sf = (float)o.scalar.f;
+        p.scalar[k] = dt == kRcF32 ? sf : dt == kRcBF16 ? load_acc(to_bf16(sf)) : load_acc(to_f16(sf));
+    }
+    if (rows == 0 || cols == 0) return DXH_OK;
+    int slots = n_inputs;
+    for (int k = 0; k < n_ops; ++k) slots = std::max(slots, p.save[k] + 1);
+    const int64_t cq = cols / 4, total = rows * cq, blocks = (total + kBlock - 1) / kBlock;
+    chain_rows_kernel<<<(unsigned)std::min<int64_t>(blocks, 1 << 22), kBlock, (size_t)std::max(slots, 1) * kBlock * kVecBytes, as_stream(stream)>>>(p, rows, cq);
+    return launch_status();
 }
 
 }  // extern "C"

@@ -77,6 +77,10 @@ void reg(TfFactory &f, const char *name, const char *author, const char *tftype,
     if (kind == "elementwise")
         for (const auto &c : chainable)
             if (op == c.name) { tf->chain_code = c.code; tf->chain_kind = c.kind; }
+    // lines that only dxh_chain_rows takes: the cast, the square, a vector spread over rows or columns
+    if (op == "todtype") { tf->chain_code = DXH_CHAIN_COPY; tf->chain_kind = 5; }
+    if (op == "broadcastTo") { tf->chain_code = DXH_CHAIN_COPY; tf->chain_kind = 6; }
+    if (op == "powscalar") { tf->chain_code = DXH_CHAIN_SQUARE; tf->chain_kind = 7; }
     tf->graph_safe = kind == "elementwise" || kind == "reduce" || kind == "changeshape" || op == "matmul" ||
                      op == "constant" || op == "arange";
     if (op == "reshape") tf->graph_safe = false;  // rewrites the tensor's shape on the host
@@ -558,81 +562,148 @@ int register_all(TfFactory &f) {
 
 // ---- several elementwise lines as one launch --------------------------------------------------
 namespace {
+// A run goes out in one of two forms: tensors of one float dtype and one size through dxh_chain, or,
+// when the lines differ in dtype (todtype), square a tensor (powscalar by 2) or spread a [rows, 1] /
+// [1, cols] tensor over [rows, cols] (broadcastTo), through dxh_chain_rows.
 struct ChainPlan {
+    bool by_rows = false;
     int dtype = 0;
-    int64_t n = 0;
+    int64_t n = 0, rows = 0, cols = 0;
     std::vector<const void *> inputs;
     std::vector<dxh_chain_op> ops;
+    std::vector<dxh_chain_tensor> row_inputs;
+    std::vector<dxh_chain_rows_op> row_ops;
 };
+enum { kChainTodtype = 5, kChainBroadcast = 6, kChainPowscalar = 7 };
 // Builds the longest run starting at tfs[first].  A tensor operand is the latest result of the run
 // with that name, else an input of the run (read before the run writes anything, which is what a
 // line-by-line execution sees as long as no earlier line of the run has written it — and those are
 // taken as results).  A tensor that several lines of the run write is stored by the last of them
-// only: nothing reads memory in between.  The run ends before a line that is not a chainable float
-// op, has another dtype or size, needs a ninth input, or whose operands are missing (the ordinary
-// path then reports the error for that line).
+// only: nothing reads memory in between.  The first line's output fixes the [rows, cols] view (cols
+// = its last dim); later tensors are that size, or a row / column vector of it.  The run ends before
+// a line that is not a chainable float op, does not fit the view, needs a ninth input, would overwrite
+// a vector that the run reads from memory (lanes of other rows or columns may not have read it yet),
+// or whose operands are missing or mismatched (the ordinary path then reports the error for that line).
 size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem, ChainPlan &plan) {
-    std::vector<std::string> input_names, output_names;
-    size_t count = 0;
-    for (size_t i = first; i < tfs.size() && plan.ops.size() < DXH_CHAIN_MAX_OPS; ++i) {
+    struct Input { std::string name; const void *data; int dtype, extent; };
+    struct Op { dxh_chain_rows_op op; std::string out_name; };
+    std::vector<Input> inputs;
+    std::vector<Op> ops;
+    bool needs_rows = false, has_f64 = false;
+    int64_t rows = 0, cols = 0;
+    auto is_float = [](int dtype) { return dtype == DXH_F64 || dtype == DXH_F32 || dtype == DXH_F16 || dtype == DXH_BF16; };
+    // extent of a tensor in the run's view, or -1
+    auto extent_of = [&](const Tensor &t) {
+        if (t.shape.size == rows * cols) return (int)DXH_CHAIN_FULL;
+        if (rows > 1 && cols > 1 && t.shape.dim() >= 1) {
+            if (t.shape.size == cols && t.shape.at(-1) == cols) return (int)DXH_CHAIN_ROW;
+            if (t.shape.size == rows && t.shape.at(-1) == 1) return (int)DXH_CHAIN_COLUMN;
+        }
+        return -1;
+    };
+    for (size_t i = first; i < tfs.size() && ops.size() < DXH_CHAIN_MAX_OPS; ++i) {
         const TF *tf = tfs[i].get();
         if (!tf || tf->chain_kind == 0 || tf->metadata.benchmark_repeat > 1 || tf->returns.size() != 1) break;
-        const size_t nargs = tf->chain_kind == 4 ? 1 : 2;
+        const int kind = tf->chain_kind;
+        const size_t nargs = kind == 4 || kind == kChainTodtype ? 1 : 2;
         if (tf->args.size() != nargs) break;
         const Param *tensors[2] = {nullptr, nullptr};
         const Param *scalar = nullptr;
-        switch (tf->chain_kind) {
+        switch (kind) {
         case 1: tensors[0] = &tf->args[0]; tensors[1] = &tf->args[1]; break;
-        case 2: tensors[0] = &tf->args[0]; scalar = &tf->args[1]; break;
+        case 2: case kChainPowscalar: tensors[0] = &tf->args[0]; scalar = &tf->args[1]; break;
         case 3: scalar = &tf->args[0]; tensors[0] = &tf->args[1]; break;
-        default: tensors[0] = &tf->args[0]; break;
+        default: tensors[0] = &tf->args[0]; break;  // unary, todtype, broadcastTo (whose second argument is the shape)
         }
         auto out = mem.findtensor(tf->returns[0].textvalue);
-        if (!out) break;
-        const int dtype = out->dtype();
-        if (dtype != DXH_F64 && dtype != DXH_F32 && dtype != DXH_F16 && dtype != DXH_BF16) break;
-        if (plan.ops.empty()) { plan.dtype = dtype; plan.n = out->shape.size; }
-        if (dtype != plan.dtype || out->shape.size != plan.n) break;
-        dxh_chain_op op{};
-        op.code = tf->chain_code;
-        op.out = out->data;
-        std::vector<std::string> new_inputs;
-        std::vector<const void *> new_ptrs;
+        if (!out || !is_float(out->dtype()) || out->shape.size == 0) break;
+        if (ops.empty()) {
+            cols = out->shape.dim() >= 1 ? out->shape.at(-1) : 1;
+            rows = out->shape.size / std::max<int64_t>(cols, 1);
+        }
+        Op op{};
+        op.op.code = tf->chain_code;
+        op.op.out = out->data;
+        op.op.dtype = out->dtype();
+        op.op.extent = extent_of(*out);
+        op.out_name = tf->returns[0].textvalue;
+        if (op.op.extent < 0) break;
+        bool line_needs_rows = op.op.extent != DXH_CHAIN_FULL || kind >= kChainTodtype || (!ops.empty() && out->dtype() != ops[0].op.dtype);
+        if (scalar) {
+            try { op.op.scalar = scalar_of(*scalar, mem); } catch (const std::exception &) { break; }
+        }
+        if (kind == kChainPowscalar && (op.op.scalar.f != 2.0 || out->dtype() != DXH_F32)) break;  // only the square has a chain code
+        if (kind == kChainBroadcast) {
+            std::vector<int> ns;
+            try { ns = ints_of(tf->args[1], mem); } catch (const std::exception &) { break; }
+            if (ns != out->shape.shape || op.op.extent != DXH_CHAIN_FULL) break;
+        }
+        std::vector<Input> new_inputs;
         bool ok = true;
         for (int side = 0; side < 2 && ok; ++side) {
             if (!tensors[side]) continue;
             const std::string &name = tensors[side]->textvalue;
             auto t = mem.findtensor(name);
-            if (!t || t->dtype() != plan.dtype || t->shape.size != plan.n) { ok = false; break; }
+            if (!t || !is_float(t->dtype())) { ok = false; break; }
+            const int extent = extent_of(*t);
+            if (extent < 0) { ok = false; break; }
+            // what the line itself would refuse: another dtype (but for todtype), another size (but for broadcastTo)
+            if (kind != kChainTodtype && t->dtype() != out->dtype()) { ok = false; break; }
+            if (kind != kChainBroadcast && (extent != op.op.extent || t->shape.size != out->shape.size)) { ok = false; break; }
+            if (kind == kChainBroadcast && broadcast_shape(t->shape.shape, out->shape.shape) != out->shape.shape) { ok = false; break; }
+            line_needs_rows = line_needs_rows || extent != DXH_CHAIN_FULL || t->dtype() != out->dtype();
             int ref = -1;
-            for (size_t j = output_names.size(); j-- > 0;)
-                if (output_names[j] == name) { ref = DXH_CHAIN_RESULT + (int)j; break; }
+            for (size_t j = ops.size(); j-- > 0;)
+                if (ops[j].out_name == name) { ref = DXH_CHAIN_RESULT + (int)j; break; }
             if (ref < 0) {
-                for (size_t j = 0; j < input_names.size() && ref < 0; ++j) if (input_names[j] == name) ref = (int)j;
-                for (size_t j = 0; j < new_inputs.size() && ref < 0; ++j) if (new_inputs[j] == name) ref = (int)(input_names.size() + j);
+                for (size_t j = 0; j < inputs.size() && ref < 0; ++j) if (inputs[j].name == name) ref = (int)j;
+                for (size_t j = 0; j < new_inputs.size() && ref < 0; ++j) if (new_inputs[j].name == name) ref = (int)(inputs.size() + j);
                 if (ref < 0) {
-                    if (input_names.size() + new_inputs.size() >= DXH_CHAIN_MAX_INPUTS) { ok = false; break; }
-                    ref = (int)(input_names.size() + new_inputs.size());
-                    new_inputs.push_back(name);
-                    new_ptrs.push_back(t->data);
+                    if (inputs.size() + new_inputs.size() >= DXH_CHAIN_MAX_INPUTS) { ok = false; break; }
+                    ref = (int)(inputs.size() + new_inputs.size());
+                    new_inputs.push_back({name, t->data, t->dtype(), extent});
                 }
             }
-            (side == 0 ? op.lhs : op.rhs) = ref;
+            (side == 0 ? op.op.lhs : op.op.rhs) = ref;
         }
         if (!ok) break;
-        if (scalar) {
-            try { op.scalar = scalar_of(*scalar, mem); } catch (const std::exception &) { break; }
-        }
-        input_names.insert(input_names.end(), new_inputs.begin(), new_inputs.end());
-        plan.inputs.insert(plan.inputs.end(), new_ptrs.begin(), new_ptrs.end());
-        output_names.push_back(tf->returns[0].textvalue);
-        plan.ops.push_back(op);
-        ++count;
+        // this line's output is a vector that the run (this line included) reads from memory
+        bool overwrites_vector_input = false;
+        for (const Input &in : inputs) overwrites_vector_input |= in.extent != DXH_CHAIN_FULL && in.name == op.out_name;
+        for (const Input &in : new_inputs) overwrites_vector_input |= in.extent != DXH_CHAIN_FULL && in.name == op.out_name;
+        if (overwrites_vector_input) break;
+        const bool line_f64 = out->dtype() == DXH_F64;
+        if ((needs_rows || line_needs_rows) && (has_f64 || line_f64)) break;  // the row form has no fp64
+        needs_rows = needs_rows || line_needs_rows;
+        has_f64 = has_f64 || line_f64;
+        inputs.insert(inputs.end(), new_inputs.begin(), new_inputs.end());
+        ops.push_back(op);
     }
+    const size_t count = ops.size();
     if (count < 2) return count;
-    for (size_t j = 0; j < output_names.size(); ++j)
-        for (size_t m = j + 1; m < output_names.size(); ++m)
-            if (output_names[m] == output_names[j]) plan.ops[j].out = nullptr;  // overwritten by line m of the run
+    for (size_t j = 0; j < count; ++j)
+        for (size_t m = j + 1; m < count; ++m)
+            if (ops[m].out_name == ops[j].out_name) ops[j].op.out = nullptr;  // overwritten by line m of the run
+    plan.by_rows = needs_rows;
+    plan.rows = rows; plan.cols = cols;
+    if (needs_rows) {
+        // whole groups of four columns, tensors aligned to such a group, or the separate calls take it
+        bool aligned = cols % 4 == 0;
+        auto group_bytes = [](int dtype, int extent) { return (uintptr_t)(extent == DXH_CHAIN_COLUMN ? 1 : 4) * (dtype == DXH_F32 ? 4 : 2); };
+        for (const Input &in : inputs) {
+            aligned = aligned && (uintptr_t)in.data % group_bytes(in.dtype, in.extent) == 0;
+            plan.row_inputs.push_back({in.data, in.dtype, in.extent});
+        }
+        for (const Op &o : ops) {
+            aligned = aligned && (uintptr_t)o.op.out % group_bytes(o.op.dtype, o.op.extent) == 0;  // NULL passes
+            plan.row_ops.push_back(o.op);
+        }
+        return aligned ? count : 0;
+    }
+    plan.dtype = ops[0].op.dtype;
+    plan.n = rows * cols;
+    for (const Input &in : inputs) plan.inputs.push_back(in.data);
+    for (const Op &o : ops) plan.ops.push_back({o.op.code, o.op.lhs, o.op.rhs, o.op.scalar, o.op.out});
     // whole 16-byte vectors at 16-byte aligned addresses, or the separate calls take it
     const int64_t vec = 16 / precision_bytes((Precision)plan.dtype);
     bool aligned = plan.n % vec == 0;
@@ -649,6 +720,9 @@ size_t chain_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, M
 int run_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, size_t count, Mem &mem, std::string &error) {
     ChainPlan plan;
     if (plan_chain(tfs, first, mem, plan) != count || count < 2) return fail(error, "chain: the run changed between planning and launch");
+    if (plan.by_rows)
+        return hip_result(dxh_chain_rows(plan.row_inputs.data(), (int)plan.row_inputs.size(), plan.row_ops.data(), (int)plan.row_ops.size(), plan.rows, plan.cols, mem.stream),
+                          "chain", error);
     return hip_result(dxh_chain(plan.dtype, plan.inputs.data(), (int)plan.inputs.size(), plan.ops.data(), (int)plan.ops.size(), plan.n, mem.stream),
                       "chain", error);
 }

@@ -31,10 +31,22 @@ class ChainOp(C.Structure):
     _fields_ = [("code", C.c_int32), ("lhs", C.c_int32), ("rhs", C.c_int32), ("scalar", Scalar), ("out", C.c_void_p)]
 
 
-# enum dxh_chain_code, in the header's order
+class ChainTensor(C.Structure):
+    """dxh_chain_tensor: one input of a dxh_chain_rows run."""
+    _fields_ = [("data", C.c_void_p), ("dtype", C.c_int32), ("extent", C.c_int32)]
+
+
+class ChainRowsOp(C.Structure):
+    """dxh_chain_rows_op: one op of a dxh_chain_rows run."""
+    _fields_ = [("code", C.c_int32), ("lhs", C.c_int32), ("rhs", C.c_int32), ("scalar", Scalar), ("out", C.c_void_p),
+                ("dtype", C.c_int32), ("extent", C.c_int32)]
+
+
+# enum dxh_chain_code, in the header's order (the last two: dxh_chain_rows only)
 CHAIN_CODES = ["add", "sub", "mul", "div", "max", "min", "addscalar", "subscalar", "rsubscalar", "mulscalar",
-               "divscalar", "rdivscalar", "maxscalar", "minscalar", "sqrt", "exp", "log"]
+               "divscalar", "rdivscalar", "maxscalar", "minscalar", "sqrt", "exp", "log", "square", "copy"]
 CHAIN_RESULT = 16
+CHAIN_FULL, CHAIN_ROW, CHAIN_COLUMN = 0, 1, 2  # enum dxh_chain_extent
 
 
 def scalar(v):
@@ -94,6 +106,7 @@ SIGNATURES = {
     "dxh_sqrt": (_UN, _i), "dxh_exp": (_UN, _i), "dxh_log": (_UN, _i),
     "dxh_sin": (_UN, _i), "dxh_cos": (_UN, _i), "dxh_tan": (_UN, _i), "dxh_invert": (_UN, _i),
     "dxh_chain": ([_i, _pp, _i, C.POINTER(ChainOp), _i, _i64, _p], _i),
+    "dxh_chain_rows": ([C.POINTER(ChainTensor), _i, C.POINTER(ChainRowsOp), _i, _i64, _i64, _p], _i),
     "dxh_todtype": ([_i, _p, _i, _p, _i64, _p], _i),
     "dxh_equal": ([_i, _p, _p, _f, _p, _i64, _p], _i),
     "dxh_notequal": ([_i, _p, _p, _f, _p, _i64, _p], _i),

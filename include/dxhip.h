@@ -216,7 +216,8 @@ enum dxh_chain_code {
     DXH_CHAIN_ADD = 0, DXH_CHAIN_SUB, DXH_CHAIN_MUL, DXH_CHAIN_DIV, DXH_CHAIN_MAX, DXH_CHAIN_MIN,      /* lhs op rhs */
     DXH_CHAIN_ADDSCALAR, DXH_CHAIN_SUBSCALAR, DXH_CHAIN_RSUBSCALAR, DXH_CHAIN_MULSCALAR,               /* lhs op scalar; R: scalar op lhs */
     DXH_CHAIN_DIVSCALAR, DXH_CHAIN_RDIVSCALAR, DXH_CHAIN_MAXSCALAR, DXH_CHAIN_MINSCALAR,
-    DXH_CHAIN_SQRT, DXH_CHAIN_EXP, DXH_CHAIN_LOG                                                       /* f(lhs) */
+    DXH_CHAIN_SQRT, DXH_CHAIN_EXP, DXH_CHAIN_LOG,                                                      /* f(lhs) */
+    DXH_CHAIN_SQUARE, DXH_CHAIN_COPY                                                                   /* dxh_chain_rows only */
 };
 #define DXH_CHAIN_MAX_OPS 8
 #define DXH_CHAIN_MAX_INPUTS 8
@@ -228,6 +229,36 @@ typedef struct dxh_chain_op {
     void *out;         /* NULL: not stored */
 } dxh_chain_op;
 DXH_API int dxh_chain(int dtype, const void *const *inputs, int n_inputs, const dxh_chain_op *ops, int n_ops, int64_t n, void *stream);
+
+/* ---- the same over a [rows, cols] view, with row / column vectors and casts
+ * No counterpart in the reference either.  The tensors of this run may differ in dtype (f32 f16 bf16)
+ * and in extent: [rows, cols] (DXH_CHAIN_FULL), a row vector [1, cols] or a column vector [rows, 1].
+ * Op k is one of the ops of dxh_chain, DXH_CHAIN_SQUARE (lhs * lhs: powscalar with exponent 2 of
+ * elementwise_miaobyte_sqrt.cuh:30, whose correctly rounded value that is) or DXH_CHAIN_COPY
+ * (lhs as it is: with another dtype the cast of launch_todtype, elementwise_miaobyte_basic.cuh:11-16,
+ * with a vector operand and full extent launch_broadcastTo, changeshape_miaobyte.cuh:42-46).  It computes
+ * in fp32 on its operands' values and rounds the result to its own `dtype` before that is stored or
+ * used, which is what the separate calls do: every `out` holds their bits.  An op of full extent takes
+ * operands of any extent (a vector counts for every row or column); an op on row or column vectors takes
+ * vectors of its own kind only and stores `cols` or `rows` elements.  Operand references, in-place use
+ * of [rows, cols] tensors and out = NULL as for dxh_chain; a vector input must not be an `out` of the
+ * run (DXH_ERR_ARG: run the ops that update it in place on their own).  cols a multiple of 4 and
+ * [rows, cols] / row-vector pointers aligned to 4 elements, else DXH_ERR_ALIGN. */
+enum dxh_chain_extent { DXH_CHAIN_FULL = 0, DXH_CHAIN_ROW = 1, DXH_CHAIN_COLUMN = 2 };
+typedef struct dxh_chain_tensor {
+    const void *data;
+    int32_t dtype;     /* DXH_F32, DXH_F16 or DXH_BF16 */
+    int32_t extent;    /* enum dxh_chain_extent */
+} dxh_chain_tensor;
+typedef struct dxh_chain_rows_op {
+    int32_t code;      /* enum dxh_chain_code */
+    int32_t lhs, rhs;  /* index into inputs, or DXH_CHAIN_RESULT + j */
+    dxh_scalar scalar;
+    void *out;         /* NULL: not stored */
+    int32_t dtype;     /* of the result */
+    int32_t extent;    /* of the result */
+} dxh_chain_rows_op;
+DXH_API int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain_rows_op *ops, int n_ops, int64_t rows, int64_t cols, void *stream);
 
 /* ---- cast: launch_todtype elementwise_miaobyte_basic.cuh:11-16.
  * C[i] = static_cast<dst>(A[i]) (float->int truncates toward zero, saturating at

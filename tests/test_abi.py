@@ -71,7 +71,29 @@ def test_argument_errors_need_no_gpu():
     assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(17, 0, 1, 48)), 1, 8, None) == -2   # unknown op code
     assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(0, 0, 1, 50)), 1, 8, None) == -5    # output off a 16-byte boundary
     assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(0, 0, 1, None)), 1, 8, None) == -2  # the last op must store
-    assert len(dx.CHAIN_CODES) == 17 and dx.CHAIN_CODES[16] == "log"
+    assert len(dx.CHAIN_CODES) == 19 and dx.CHAIN_CODES[16] == "log" and dx.CHAIN_CODES[18] == "copy"
+    # dxh_chain_rows: the same checks, and those on extents: a [rows, cols] op takes any operand, an op on
+    # vectors only vectors of its kind; a vector input may not be an output of the run
+    T, R = dx.ChainTensor, dx.ChainRowsOp
+    FULL, ROW, COL = dx.CHAIN_FULL, dx.CHAIN_ROW, dx.CHAIN_COLUMN
+    tin = (T * 3)(T(64, dx.F32, FULL), T(128, dx.BF16, ROW), T(256, dx.F32, COL))
+    rop = lambda code, lhs, rhs, out, dtype=dx.F32, extent=FULL: R(code, lhs, rhs, dx.scalar(1.0), out, dtype, extent)
+    run = lambda *ops, n_in=3, rows=8, cols=16: L.dxh_chain_rows(tin, n_in, (R * len(ops))(*ops), len(ops), rows, cols, None)
+    assert run(rop(2, 0, 1, 512), rows=0) == 0                               # nothing to do
+    assert run(rop(2, 0, 1, 512), cols=18) == -5                             # cols not a multiple of 4
+    assert run(rop(2, 0, 1, 512, dx.F64)) == -1                              # no fp64 in this form
+    assert L.dxh_chain_rows((T * 1)(T(64, dx.I32, FULL)), 1, (R * 1)(rop(18, 0, 0, 512)), 1, 8, 16, None) == -1
+    assert run(rop(19, 0, 0, 512)) == -2                                     # unknown op code
+    assert run(rop(2, 0, 3, 512)) == -2                                      # input 3 does not exist
+    assert run(rop(2, 0, 1, 512, extent=3)) == -2                            # unknown extent
+    assert run(rop(2, 0, 1, None)) == -2                                     # the last op must store
+    assert run(rop(2, 0, 1, 520)) == -5                                      # fp32 output off a 16-byte boundary
+    assert run(rop(18, 1, 0, 516, dx.BF16, ROW)) == -5                       # bf16 row off an 8-byte boundary
+    assert run(rop(18, 2, 0, 516, dx.F32, COL), rop(2, 0, dx.CHAIN_RESULT, 512), rows=0) == 0  # a column needs its element size only
+    assert run(rop(9, 0, 0, 512, dx.F32, ROW)) == -2                         # an op on row vectors cannot read a [rows, cols] tensor
+    assert run(rop(9, 2, 0, 512, dx.F32, ROW)) == -2                         # ... nor a column vector
+    assert run(rop(18, 1, 0, 1024, dx.F32, ROW), rop(0, dx.CHAIN_RESULT, 2, 512, dx.F32, COL)) == -2  # a row result into a column op
+    assert run(rop(9, 2, 0, 256, dx.F32, COL), rop(2, 0, dx.CHAIN_RESULT, 512)) == -2  # overwrites the column vector it reads
 
 
 def test_tuning_knobs_validate_their_values():

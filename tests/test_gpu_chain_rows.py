@@ -1,0 +1,226 @@
+"""GPU parity: dxh_chain_rows (a run of elementwise ops over a [rows, cols] view whose tensors may
+differ in dtype and may be row or column vectors) against the separate entry points, the CPU
+oracle and a numpy model.
+
+Bars: bit-identical to what todtype / powscalar / broadcastTo / mul ... store when called one
+after another; each op of such a run bit-exact against the oracle fed with the device's own
+operands (casts, squares, copies and products are correctly rounded on both sides); random runs
+of exactly rounded ops bit-exact against numpy float32 arithmetic with one rounding to the op's
+dtype (NaN payloads aside).
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from deepx_amd import lib as dx
+from tests import helpers as H
+from tests.helpers import Dev, hp
+
+pytestmark = pytest.mark.gpu
+
+FULL, ROW, COL = dx.CHAIN_FULL, dx.CHAIN_ROW, dx.CHAIN_COLUMN
+R = dx.CHAIN_RESULT
+BINARY = ["add", "sub", "mul", "div", "max", "min"]
+SCALAR = ["addscalar", "subscalar", "rsubscalar", "mulscalar", "divscalar", "rdivscalar", "maxscalar", "minscalar"]
+
+
+def count(extent, rows, cols):
+    return rows * cols if extent == FULL else cols if extent == ROW else rows
+
+
+def run_rows(dxh, inputs, prog, rows, cols, outs=None):
+    """inputs: (Dev, dtype, extent); prog: (name, lhs, rhs, scalar, dtype, extent).  Returns rc and the outputs."""
+    if outs is None:
+        outs = [Dev.empty(count(e, rows, cols), H.NP[dt]) for (_, _, _, _, dt, e) in prog]
+    tin = (dx.ChainTensor * max(1, len(inputs)))(*[dx.ChainTensor(d.ptr, dt, e) for d, dt, e in inputs])
+    ops = (dx.ChainRowsOp * len(prog))()
+    for k, (name, lhs, rhs, s, dt, e) in enumerate(prog):
+        ops[k] = dx.ChainRowsOp(dx.CHAIN_CODES.index(name), lhs, rhs, dx.scalar(s), outs[k].ptr if outs[k] is not None else None, dt, e)
+    return dxh.dxh_chain_rows(tin, len(inputs), ops, len(prog), rows, cols, None), outs
+
+
+def shape_of(extent, rows, cols):
+    return [rows, cols] if extent == FULL else [1, cols] if extent == ROW else [rows, 1]
+
+
+def run_separately(dxh, orc, inputs, prog, rows, cols):
+    """The lines a front end would send, one entry point each, on the device; every result also
+    against the oracle applied to the device's operands of that op."""
+    outs = []
+    for k, (name, lhs, rhs, s, dt, e) in enumerate(prog):
+        src = lambda r: inputs[r] if r < R else (outs[r - R], prog[r - R][4], prog[r - R][5])
+        a, adt, ae = src(lhs)
+        n = count(e, rows, cols)
+        out = Dev.empty(n, H.NP[dt])
+        want = np.empty(n, dtype=H.NP[dt])
+        ah = a.get()
+        if name == "copy" and ae != e:
+            assert adt == dt and e == FULL
+            ish, osh = shape_of(ae, rows, cols), [rows, cols]
+            dx.check(dxh.dxh_broadcastTo(dt, a.ptr, dx.i32arr(ish), 2, dx.i32arr(osh), 2, out.ptr, None), "broadcastTo")
+            assert orc.orc_broadcastTo(dt, hp(ah), dx.i32arr(ish), 2, dx.i32arr(osh), 2, hp(want)) == 0
+        elif name == "copy":
+            dx.check(dxh.dxh_todtype(adt, a.ptr, dt, out.ptr, n, None), "todtype")
+            assert orc.orc_todtype(adt, hp(ah), dt, hp(want), n) == 0
+        elif name == "square":
+            assert adt == dt == dx.F32 and ae == e
+            dx.check(dxh.dxh_powscalar(dt, a.ptr, dx.scalar(2.0), out.ptr, n, None), "powscalar")
+            assert orc.orc_powscalar(dt, hp(ah), dx.scalar(2.0), hp(want), n) == 0
+        elif name in BINARY:
+            b, bdt, be = src(rhs)
+            assert adt == bdt == dt and ae == be == e
+            dx.check(getattr(dxh, "dxh_" + name)(dt, a.ptr, b.ptr, out.ptr, n, None), name)
+            assert getattr(orc, "orc_" + name)(dt, hp(ah), hp(b.get()), hp(want), n) == 0
+        elif name in ("rsubscalar", "rdivscalar"):
+            assert adt == dt and ae == e
+            dx.check(getattr(dxh, "dxh_" + name)(dt, dx.scalar(s), a.ptr, out.ptr, n, None), name)
+            assert getattr(orc, "orc_" + name)(dt, dx.scalar(s), hp(ah), hp(want), n) == 0
+        elif name in SCALAR:
+            assert adt == dt and ae == e
+            dx.check(getattr(dxh, "dxh_" + name)(dt, a.ptr, dx.scalar(s), out.ptr, n, None), name)
+            assert getattr(orc, "orc_" + name)(dt, hp(ah), dx.scalar(s), hp(want), n) == 0
+        else:
+            assert adt == dt and ae == e and name == "sqrt"
+            dx.check(dxh.dxh_sqrt(dt, a.ptr, out.ptr, n, None), name)
+            assert orc.orc_sqrt(dt, hp(ah), hp(want), n) == 0
+        got = out.get()
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), ("oracle", k, name, rows, cols)
+        outs.append(out)
+    return outs
+
+
+def same_bits(a, b):
+    return np.array_equal(a.get().view(np.uint8), b.get().view(np.uint8))
+
+
+@pytest.mark.parametrize("half", [dx.BF16, dx.F16])
+def test_rmsnorm_lines_as_runs(dxh, orc, half):
+    """The elementwise lines of an RMSNorm either side of its row sum (t5layernorm.py:17-22 as the
+    front end emits it): cast and square before the sum; after it the reciprocal root spread over
+    the columns, the product, the weight cast, spread over the rows and multiplied, and the cast of
+    the result.  Every tensor a line writes, bit for bit what the separate entry points store, and
+    each of those against the oracle."""
+    rng = np.random.default_rng(1200 + half)
+    for rows, cols in [(2048, 896), (5, 12), (2, 4), (257, 1000), (64, 4096)]:
+        x = Dev(H.rand(rng, half, rows * cols, -2.0, 2.0))
+        w = Dev(H.rand(rng, half, cols, 0.5, 1.5))
+        var = Dev(H.rand(rng, dx.F32, rows, 0.05, 3.0))  # stands for 1/sqrt(mean + eps) of each row
+        before = [("copy", 0, 0, 0, dx.F32, FULL), ("square", R + 0, 0, 2.0, dx.F32, FULL)]
+        ins = [(x, half, FULL)]
+        want = run_separately(dxh, orc, ins, before, rows, cols)
+        rc, got = run_rows(dxh, ins, before, rows, cols)
+        dx.check(rc, "chain_rows")
+        for k in range(len(before)):
+            assert same_bits(got[k], want[k]), ("before", rows, cols, k)
+        xf = got[0]
+        after = [("copy", 0, 0, 0, dx.F32, FULL),        # broadcastTo(var) -> rs
+                 ("mul", 1, R + 0, 0, dx.F32, FULL),      # xf * rs -> xn
+                 ("copy", 2, 0, 0, dx.F32, ROW),          # todtype(w) -> wf1
+                 ("copy", R + 2, 0, 0, dx.F32, FULL),     # broadcastTo(wf1) -> wf
+                 ("mul", R + 3, R + 1, 0, dx.F32, FULL),  # wf * xn -> xn
+                 ("copy", R + 4, 0, 0, half, FULL)]       # todtype(xn) -> h
+        ins = [(var, dx.F32, COL), (xf, dx.F32, FULL), (w, half, ROW)]
+        want = run_separately(dxh, orc, ins, after, rows, cols)
+        rc, got = run_rows(dxh, ins, after, rows, cols)
+        dx.check(rc, "chain_rows")
+        for k in range(len(after)):
+            assert same_bits(got[k], want[k]), ("after", rows, cols, k)
+        # the same with the first product not stored (the second overwrites xn in the IR)
+        outs = [Dev.empty(count(e, rows, cols), H.NP[dt]) for (_, _, _, _, dt, e) in after]
+        outs[1] = None
+        rc, got2 = run_rows(dxh, ins, after, rows, cols, outs=outs)
+        dx.check(rc, "chain_rows")
+        for k in (0, 2, 3, 4, 5):
+            assert same_bits(got2[k], want[k]), ("after, xn stored once", rows, cols, k)
+
+
+def model(inputs_host, prog, rows, cols):
+    """numpy float32 arithmetic on operands spread to [rows, cols], one rounding to the op's dtype."""
+    def spread(values, extent):
+        v = np.asarray(values, dtype=np.float32)
+        return v.reshape(rows, cols) if extent == FULL else np.broadcast_to(v.reshape(1, cols), (rows, cols)) if extent == ROW \
+            else np.broadcast_to(v.reshape(rows, 1), (rows, cols))
+    results = []
+    with np.errstate(all="ignore"):
+        for name, lhs, rhs, s, dt, e in prog:
+            src = lambda r: inputs_host[r] if r < R else results[r - R]
+            a, b = src(lhs), src(rhs)
+            sc = np.float32(H.to_float(H.to_storage(np.array([s]), dt), dt)[0])
+            if name == "add": y = a + b
+            elif name == "sub": y = a - b
+            elif name == "mul": y = a * b
+            elif name == "div": y = a / b
+            elif name == "max": y = np.where(a < b, b, a)
+            elif name == "min": y = np.where(b < a, b, a)
+            elif name == "addscalar": y = a + sc
+            elif name == "subscalar": y = a - sc
+            elif name == "rsubscalar": y = sc - a
+            elif name == "mulscalar": y = a * sc
+            elif name == "divscalar": y = a / sc
+            elif name == "rdivscalar": y = sc / a
+            elif name == "maxscalar": y = np.where(a < sc, sc, a)
+            elif name == "minscalar": y = np.where(sc < a, sc, a)
+            elif name == "sqrt": y = np.sqrt(a)
+            elif name == "square": y = a * a
+            else: y = a
+            y = np.asarray(y, dtype=np.float32)
+            results.append(H.to_float(H.to_storage(y.reshape(-1), dt), dt).astype(np.float32).reshape(rows, cols))
+    return results
+
+
+def test_random_mixed_runs_match_the_model(dxh):
+    """Random runs of 1..8 ops over up to 8 inputs of mixed dtype (f32, bf16, f16) and extent; ops of
+    full extent draw operands of any extent (a vector counts for every row or column), ops on vectors
+    only vectors of their kind.  Shapes from one group of four columns to several workgroups, row
+    counts that leave the last workgroup ragged."""
+    rng = np.random.default_rng(4242)
+    dtypes = [dx.F32, dx.BF16, dx.F16]
+    names = BINARY + SCALAR + ["sqrt", "square", "copy"]
+    for trial in range(40):
+        rows, cols = [(1, 4), (3, 8), (7, 36), (64, 256), (33, 1000), (300, 132)][trial % 6]
+        n_in = int(rng.integers(1, 9))
+        inputs, host = [], []
+        for j in range(n_in):
+            dt = dtypes[int(rng.integers(0, 3))]
+            e = FULL if rows == 1 or j == 0 else int(rng.integers(0, 3))
+            data = H.rand(rng, dt, count(e, rows, cols), 0.25, 2.0)
+            inputs.append((Dev(data), dt, e))
+            v = H.to_float(data, dt).astype(np.float32)
+            host.append(np.broadcast_to(v.reshape(shape_of(e, rows, cols)), (rows, cols)))
+        prog, extents = [], []
+        for k in range(int(rng.integers(1, 9))):
+            e = FULL if rows == 1 else int(rng.choice([FULL, FULL, ROW, COL]))
+            fits = [j for j in range(n_in) if e == FULL or inputs[j][2] == e] + [R + j for j in range(k) if e == FULL or extents[j] == e]
+            if not fits:
+                e = FULL
+                fits = list(range(n_in)) + [R + j for j in range(k)]
+            pick = lambda: int(fits[int(rng.integers(0, len(fits)))])
+            prog.append((str(rng.choice(names)), pick(), pick(), float(rng.choice([0.5, 1.0, 2.0, -1.0, 3.1])), dtypes[int(rng.integers(0, 3))], e))
+            extents.append(e)
+        rc, got = run_rows(dxh, inputs, prog, rows, cols)
+        dx.check(rc, "chain_rows")
+        want = model(host, prog, rows, cols)
+        for k, (name, _, _, _, dt, e) in enumerate(prog):
+            g = H.to_float(got[k].get(), dt).astype(np.float32)
+            w = want[k][0, :] if e == ROW else want[k][:, 0] if e == COL else want[k].reshape(-1)
+            assert np.array_equal(g, w, equal_nan=True), (trial, rows, cols, k, prog)
+
+
+def test_in_place_and_refusals(dxh):
+    """A [rows, cols] output may be one of the inputs (a lane reads its own elements before it writes
+    them); a vector input may not (DXH_ERR_ARG), nor may an op on vectors read a [rows, cols] tensor."""
+    rng = np.random.default_rng(5)
+    rows, cols = 48, 64
+    a, v = H.rand(rng, dx.F32, rows * cols), H.rand(rng, dx.F32, rows)
+    A, Vc = Dev(a), Dev(v)
+    prog = [("mul", 0, 1, 0, dx.F32, FULL), ("add", R + 0, 0, 0, dx.F32, FULL)]  # a *= v (per row); c = a_new + a_old
+    out2 = Dev.empty(rows * cols, np.float32)
+    rc, _ = run_rows(dxh, [(A, dx.F32, FULL), (Vc, dx.F32, COL)], prog, rows, cols, outs=[A, out2])
+    dx.check(rc, "chain_rows")
+    prod = (a.reshape(rows, cols) * v.reshape(rows, 1)).astype(np.float32)
+    assert np.array_equal(A.get().reshape(rows, cols), prod) and np.array_equal(out2.get().reshape(rows, cols), prod + a.reshape(rows, cols))
+    rc, _ = run_rows(dxh, [(A, dx.F32, FULL), (Vc, dx.F32, COL)], [("sqrt", 1, 0, 0, dx.F32, COL), ("mul", 0, R + 0, 0, dx.F32, FULL)], rows, cols, outs=[Vc, out2])
+    assert rc == -2
+    rc, _ = run_rows(dxh, [(A, dx.F32, FULL), (Vc, dx.F32, COL)], [("sqrt", 0, 0, 0, dx.F32, COL)], rows, cols)
+    assert rc == -2

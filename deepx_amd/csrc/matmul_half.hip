@@ -444,10 +444,14 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
             // lower tile still fits the output into one round, every CU's K loop gets shorter
             // (2048x896x4864: 18.2 us with 160 rows, 19.8 with 192; 2048x4096x4096: 56.9 us with 128
             // rows, 63.4 with 192, hipBLASLt 70.9).
+            // And a tile half as wide for an N that 256 columns divide badly (8192x4864x896, where 256-wide
+            // tiles compute 1024 columns: 58.5 us against 66.5 with 128 rows x 256).
             if (dma_ok) {
-                const double c11 = one_per_cu(160, 256, 1.0, 5.5), c12 = one_per_cu(128, 256, 0.89, 5.0);
-                const double best = choice == 1 ? c1 : choice == 4 ? c4 : c6;
-                if (c11 < best || c12 < best) choice = c12 <= c11 ? 12 : 11;
+                const double c11 = one_per_cu(160, 256, 1.0, 5.5), c12 = one_per_cu(128, 256, 0.89, 5.0), c13 = one_per_cu(256, 128, 0.76, 3.5) - (tiles(256, 128) <= cus / 2 ? ksteps * 0.09 : 0.0);  // 0.52 us per step up to half the CUs
+                double best = choice == 1 ? c1 : choice == 4 ? c4 : c6;
+                if (c11 < best) { best = c11; choice = 11; }
+                if (c12 < best) { best = c12; choice = 12; }
+                if (c13 < best) { best = c13; choice = 13; }
             }
         }
         else if (tiles(128, 64) * 4 >= cus * 3) choice = 2;  // 1024x8192x1024 (128 such tiles): 38 us, 31 us with 256 64x64 tiles
@@ -459,7 +463,7 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
     // runs two LDS stages of K 64 when K is long (whole cache lines of A, half the barriers) and four
     // of K 32 when it is short (2048x896x4864: 21.2 against 22.6 us with the shallow pipeline).
     if (dma_ok && tuning().matmul_tile == 0 && (choice == 4 || choice == 6)) choice = choice == 6 ? 8 : k >= 2048 ? 10 : 7;
-    if (dma_ok && choice >= 7 && choice <= 12) {
+    if (dma_ok && choice >= 7 && choice <= 13) {
         if (sc.planning) return DXH_OK;
         return launch_matmul_half_dma(std::is_same_v<T, bf16_t> ? DXH_BF16 : DXH_F16, (int)choice - 7, a, b, c, batch, m, k, n, st);
     }
@@ -470,7 +474,7 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
         case 4: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 5: return launch_tile<T, 64, 64, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 6: case 8: case 11: case 12: return launch_tile<T, 192, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
-        case 7: case 10: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
+        case 7: case 10: case 13: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         }
     }

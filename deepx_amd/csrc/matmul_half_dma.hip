@@ -264,6 +264,7 @@ static int launch_dma_shape(int shape, const void *a, const void *b, void *c, in
     case 3: return launch_dma_tile<T, 256, 256, 64, 2>(a, b, c, batch, m, k, n, st);
     case 4: return launch_dma_tile<T, 160, 256, 32, 5, 4>(a, b, c, batch, m, k, n, st);
     case 5: return launch_dma_tile<T, 128, 256, 32, 5, 4>(a, b, c, batch, m, k, n, st);
+    case 6: return launch_dma_tile<T, 256, 128, 64, 3>(a, b, c, batch, m, k, n, st);
     default: return launch_dma_tile<T, 128, 64, 64, 5>(a, b, c, batch, m, k, n, st);
     }
 }

@@ -84,13 +84,13 @@ def test_config5_gemm_shapes_bf16(dxh, orc):
 TILE_KNOB = 4  # DXH_TUNE_MATMUL_TILE
 
 
-@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12])
+@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13])
 @pytest.mark.parametrize("dtype", [dx.BF16, dx.F16])
 def test_matmul_tile_configs(dxh, dtype, tile):
     """Every workgroup tile of the MFMA kernel (forced through the tuning knob) on aligned shapes
     with ragged tile edges, more than one batch and M, N below one tile; float64 numpy is the
     reference, bar rel 1e-2 of sum_k |a||b| as above.  K = 72, 8, 1000, 56 end in a partial K step
-    (zero-filled in the kernel; tiles 7 to 12, whose operands go straight into LDS in whole K steps,
+    (zero-filled in the kernel; tiles 7 to 13, whose operands go straight into LDS in whole K steps,
     hand those to their register-staged twins); K = 32 and 64 are shorter than the LDS pipeline of
     those tiles, K = 192 and 448 wrap around its stages.  Tiles 11 and 12 (160 and 128 rows, four
     waves side by side) meet M below, at and above a tile, with a last tile of 1 to 159 rows."""
@@ -124,7 +124,7 @@ def test_matmul_tiles_exact_on_small_integers(dxh):
         B = H.to_storage(Bi.astype(np.float64).reshape(-1), dx.BF16)
         want = (Ai @ Bi).astype(np.float64)  # |sum| <= 16*256 = 4096: exact in fp32
         dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, np.uint16)
-        for tile in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12):
+        for tile in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13):
             dx.check(dxh.dxh_tune(TILE_KNOB, tile))
             try:
                 dx.check(H.matmul(dxh, dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))

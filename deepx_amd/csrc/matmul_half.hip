@@ -423,12 +423,12 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
         const int64_t cus = compute_units();
         auto tiles = [&](int tm, int tn) { return batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn); };
         if (m <= 64) choice = 5;  // one tile row: anything taller multiplies padding (bf16 [1,896]x[896,151936]: 53 vs 75 us)
-        else if (tiles(128, 128) * 2 >= cus * 3) {
-            // Enough output for the large tiles: estimated time in us of the three candidates.  The two
+        else if (tiles(128, 64) * 4 >= cus * 3) {
+            // Enough output for tiles of 128x64 and up: estimated time in us of the candidates.  The two
             // one-workgroup-per-CU tiles run in rounds of `cus` tiles, each round paying its own
             // prologue and its own burst of C stores (nothing else runs on the CU to hide them); K
             // steps get faster when only part of the CUs is busy.  128x128 tiles run two to a CU: a
-            // pair of tiles takes 1.08 us per K step, a tile that has the CU to itself 0.6 us.
+            // pair of tiles takes 1.08 us per K step, a tile that has the CU to itself 0.53 us.
             const double ksteps = (double)((k + PK - 1) / PK);
             auto one_per_cu = [&](int tm, int tn, double step, double overhead) {
                 const int64_t t = tiles(tm, tn), rounds = (t + cus - 1) / cus;
@@ -436,26 +436,30 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
                 return (double)rounds * (ksteps * step * (0.65 + 0.35 * busy) + overhead);
             };
             const int64_t t1 = tiles(128, 128), full = t1 / (2 * cus), rem = t1 % (2 * cus);
-            const double c1 = ksteps * (1.08 * (double)full + (rem == 0 ? 0.0 : rem <= cus ? 0.6 : 1.08)) + 2.0;
+            const double c1 = ksteps * (1.08 * (double)full + (rem == 0 ? 0.0 : rem <= cus ? 0.53 : 1.08)) + 2.0;
             const double edge = ldc >= 0 ? 5.0 : 0.0;  // element-wise C stores make the burst at the end of a round longer
             const double c4 = one_per_cu(256, 256, 1.645, 3.5 + edge), c6 = one_per_cu(192, 256, 1.21, 6.0 + edge);
+            // 128x64 tiles, two to a CU as well: 0.33 us per K step and tile (2048x4864x896: 224 tiles, 27 us)
+            const double c2 = ksteps * 0.33 * (double)((tiles(128, 64) + cus - 1) / cus) + 2.0;
             choice = (c1 <= c4 && c1 <= c6) ? 1 : (c4 <= c6) ? 4 : 6;
+            if (c2 < (choice == 1 ? c1 : choice == 4 ? c4 : c6)) choice = 2;
             // Lower tiles of the same width, one wave per 64 columns (matmul_half_dma.hip only): when a
             // lower tile still fits the output into one round, every CU's K loop gets shorter
             // (2048x896x4864: 18.2 us with 160 rows, 19.8 with 192; 2048x4096x4096: 56.9 us with 128
             // rows, 63.4 with 192, hipBLASLt 70.9).
             // And a tile half as wide for an N that 256 columns divide badly (8192x4864x896, where 256-wide
             // tiles compute 1024 columns: 58.5 us against 66.5 with 128 rows x 256).
+            // All three are taken for a single round only: over several rounds the square tile's lower
+            // traffic through L2 wins again (8192^3: 843 us with 256x128, 790 with 256x256).
             if (dma_ok) {
                 const double c11 = one_per_cu(160, 256, 1.0, 5.5), c12 = one_per_cu(128, 256, 0.89, 5.0), c13 = one_per_cu(256, 128, 0.76, 3.5) - (tiles(256, 128) <= cus / 2 ? ksteps * 0.09 : 0.0);  // 0.52 us per step up to half the CUs
-                double best = choice == 1 ? c1 : choice == 4 ? c4 : c6;
-                if (c11 < best) { best = c11; choice = 11; }
-                if (c12 < best) { best = c12; choice = 12; }
-                if (c13 < best) { best = c13; choice = 13; }
+                double best = choice == 1 ? c1 : choice == 2 ? c2 : choice == 4 ? c4 : c6;
+                if (c11 < best && tiles(160, 256) <= cus) { best = c11; choice = 11; }
+                if (c12 < best && tiles(128, 256) <= cus) { best = c12; choice = 12; }
+                if (c13 < best && tiles(256, 128) <= cus) { best = c13; choice = 13; }
             }
         }
-        else if (tiles(128, 64) * 4 >= cus * 3) choice = 2;  // 1024x8192x1024 (128 such tiles): 38 us, 31 us with 256 64x64 tiles
-        else choice = 5;
+        else choice = 5;  // 1024x8192x1024 as 128 tiles of 128x64: 38 us, 31 us with 256 64x64 tiles
     }
     // The two one-workgroup-per-CU tiles have a twin whose operands travel straight into LDS
     // (matmul_half_dma.hip: less power, no LDS store traffic, deeper prefetch; 8192^3 830 -> 782 us,

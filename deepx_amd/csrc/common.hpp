@@ -167,6 +167,7 @@ inline bool stream_is_capturing(hipStream_t st) {
 }
 void reduce_stream_release(hipStream_t st);  // reduce.hip: gives back the stream's slice of finish counters
 void reduce_device_init();  // reduce.hip: resolves the file-scope device arrays of the current device
+void chain_device_init();   // elementwise.hip: raises the dynamic-LDS limit of the row-form chain kernels on the current device
 
 // Whether the loads of a streaming kernel carry the nt hint.  Measured on MI355X with buffers
 // rotated through 768 MB (fp32, GB/s with nt / without):

@@ -6,7 +6,8 @@
 // against grid-stride variants that loop: 6.4 TB/s vs 5.0 TB/s for a 3-stream add).  Arithmetic follows executor/op-ompsimd's
 // tensorfunc/elementwise_miaobyte.hpp (cited per op in include/dxhip.h); 16-bit floats
 // compute in fp32 and round once.
-#include "common.hpp"
+#include "reduce_order.hpp"
+#include <mutex>
 
 namespace dxh {
 
@@ -420,22 +421,35 @@ int launch_chain(ChainArgs &p, const dxh_chain_op *ops, int64_t n, hipStream_t s
 // ---- a run of elementwise ops over a [rows, cols] view, with row / column vectors and casts ------
 // The same interpreter for runs whose tensors differ in dtype (f32, bf16, f16) or in extent: besides
 // [rows, cols] tensors a run may read and write row vectors [1, cols] and column vectors [rows, 1],
-// and its ops include the cast (todtype) and the copy of a vector into every row or column
-// (broadcastTo).  A lane owns four adjacent columns of one row.  Every value is carried as fp32 (a
-// 16-bit float is exact in it) and every result is rounded to its op's dtype before anything uses
-// it, so the stored bits are those of the separate launches.  An op on vectors is computed by every
-// lane for its own row or columns and stored by the lanes of column 0 or row 0 only; a later op of
-// the run that reads the vector has the value at hand, no lane waits for another.  That is also why
-// a vector input must not be an output of the same run: lanes that read it race with the lane that
-// overwrites it.
+// and its ops include the cast (todtype), the copy of a vector into every row or column
+// (broadcastTo) and the sum of every row (sum over the last axis).  A lane owns groups of four
+// adjacent columns of one row.  Every value is carried as fp32 (a 16-bit float is exact in it) and
+// every result is rounded to its op's dtype before anything uses it, so the stored bits are those
+// of the separate launches.  An op on vectors is computed by every lane for its own row or columns
+// and stored by the lanes of column 0 or row 0 only; a later op of the run that reads the vector
+// has the value at hand, no lane waits for another.  That is also why a vector input must not be
+// an output of the same run: lanes that read it race with the lane that overwrites it.
+//
+// Two lane layouts, one group of four columns per lane in both.  Without a row sum the groups are
+// dealt out in memory order.  With one (BYROW) a row has P adjacent lanes of its own (P a power of
+// two, lanes past the row's last group idle) and the sum is folded by the first G of them exactly as
+// the G lanes of dxh_sum's row stage fold it (same code, reduce_order.hpp; the operand is read back
+// from its LDS slot, where lane j of the row put group j), so it has the bits dxh_sum would store;
+// two workgroup barriers per sum hand the operand over and the result back.
+//
+// The op table is read from the kernel-argument segment itself, through the scalar cache, with the
+// op counter as index: indexing the by-value argument that way would make the compiler copy it to
+// per-lane scratch memory, and a copy in LDS costs a set-up phase longer than the ops of a small run.
 enum { kRowFull = 0, kRowVec = 1, kColVec = 2 };
 enum { kRcF32 = 0, kRcBF16 = 1, kRcF16 = 2 };
-struct RowChainArgs {
+constexpr int kRowOps = DXH_CHAIN_ROWS_MAX_OPS, kRowVecs = 4;
+constexpr size_t kRowLdsMax = 156 * 1024, kRowLdsDefault = 64 * 1024;  // dynamic LDS: what the CU has beside the static part, what a launch gets unasked
+struct RowChainArgs {  // first kernel argument: sits at offset 0 of the kernel-argument segment
+    uint64_t op[kRowOps];  // code | lhs << 8 | rhs << 16 | save << 24 | dtype << 32 | extent << 40; lhs, rhs, save as int8
+    float scalar[kRowOps];  // already rounded to the op's dtype on the host
+    void *out[kRowOps];
     const void *in[kChainInputs];
-    void *out[kChainOps];
-    float scalar[kChainOps];  // already rounded to the op's dtype on the host
-    int8_t in_dtype[kChainInputs], in_kind[kChainInputs];
-    int8_t code[kChainOps], lhs[kChainOps], rhs[kChainOps], save[kChainOps], dtype[kChainOps], kind[kChainOps];
+    uint8_t in_dtype[kChainInputs], in_kind[kChainInputs];
     int n_in, n_ops;
 };
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
@@ -456,12 +470,13 @@ __device__ __forceinline__ f32x4_t rowchain_load(const void *p, int dt, int kind
     const vec_t<f16_t, 4> x = reinterpret_cast<const vec_t<f16_t, 4> *>(p)[j];
     return f32x4_t{load_acc(x.v[0]), load_acc(x.v[1]), load_acc(x.v[2]), load_acc(x.v[3])};
 }
-// rounds y to the op's dtype (in place, as fp32 again) and stores it where the op's extent says
-__device__ __forceinline__ void rowchain_round_store(float (&y)[4], void *out, int dt, int kind, int64_t row, int64_t c4, int64_t i) {
-    const bool mine = kind == kRowFull || (kind == kRowVec ? row == 0 : c4 == 0);
+// rounds y to the op's dtype (in place, as fp32 again) and, if this lane is the one to store it
+// (`owner`: its group of columns exists), stores it where the op's extent says
+__device__ __forceinline__ void rowchain_round_store(float (&y)[4], void *out, int dt, int kind, bool owner, int64_t row, int64_t c4, int64_t i) {
+    const bool mine = out && owner && (kind == kRowFull || (kind == kRowVec ? row == 0 : c4 == 0));
     const int64_t j = kind == kRowVec ? c4 : i;
     if (dt == kRcF32) {
-        if (out && mine) {
+        if (mine) {
             if (kind == kColVec) reinterpret_cast<float *>(out)[row] = y[0];
             else reinterpret_cast<f32x4_t *>(out)[j] = f32x4_t{y[0], y[1], y[2], y[3]};
         }
@@ -470,7 +485,7 @@ __device__ __forceinline__ void rowchain_round_store(float (&y)[4], void *out, i
         store_acc_vec<bf16_t, 4>(r, y);
 #pragma unroll
         for (int v = 0; v < 4; ++v) y[v] = load_acc(r.v[v]);
-        if (out && mine) {
+        if (mine) {
             if (kind == kColVec) reinterpret_cast<bf16_t *>(out)[row] = r.v[0];
             else reinterpret_cast<vec_t<bf16_t, 4> *>(out)[j] = r;
         }
@@ -479,48 +494,69 @@ __device__ __forceinline__ void rowchain_round_store(float (&y)[4], void *out, i
         store_acc_vec<f16_t, 4>(r, y);
 #pragma unroll
         for (int v = 0; v < 4; ++v) y[v] = load_acc(r.v[v]);
-        if (out && mine) {
+        if (mine) {
             if (kind == kColVec) reinterpret_cast<f16_t *>(out)[row] = r.v[0];
             else reinterpret_cast<vec_t<f16_t, 4> *>(out)[j] = r;
         }
     }
 }
-__global__ __launch_bounds__(kBlock) void chain_rows_kernel(const RowChainArgs p, int64_t rows, int64_t cq) {
+template <bool BYROW>
+__global__ __launch_bounds__(kBlock) void chain_rows_kernel(const RowChainArgs p, int64_t rows, int64_t cq, int G, int P) {
     extern __shared__ __attribute__((aligned(16))) unsigned char chain_lds[];
+    __shared__ float row_sums[kBlock];  // BYROW: one per row of the workgroup
+    typedef const RowChainArgs __attribute__((address_space(4))) *ArgTable;
+    const ArgTable tab = (ArgTable)__builtin_amdgcn_kernarg_segment_ptr();
     const int t = threadIdx.x;
-    // op and input tables in LDS, for the reason given in chain_kernel
-    __shared__ int s_code[kChainOps], s_lhs[kChainOps], s_rhs[kChainOps], s_save[kChainOps], s_dtype[kChainOps], s_kind[kChainOps];
-    __shared__ int s_in_dtype[kChainInputs], s_in_kind[kChainInputs];
-    __shared__ float s_scalar[kChainOps];
-    __shared__ void *s_out[kChainOps];
-    __shared__ const void *s_in[kChainInputs];
-    if (t == 0) {
-#pragma unroll
-        for (int k = 0; k < kChainOps; ++k) {
-            s_code[k] = p.code[k]; s_lhs[k] = p.lhs[k]; s_rhs[k] = p.rhs[k]; s_save[k] = p.save[k];
-            s_dtype[k] = p.dtype[k]; s_kind[k] = p.kind[k]; s_scalar[k] = p.scalar[k]; s_out[k] = p.out[k];
-        }
-#pragma unroll
-        for (int j = 0; j < kChainInputs; ++j) { s_in[j] = p.in[j]; s_in_dtype[j] = p.in_dtype[j]; s_in_kind[j] = p.in_kind[j]; }
-    }
-    __syncthreads();
-    f32x4_t *slot = reinterpret_cast<f32x4_t *>(chain_lds);
+    f32x4_t *slot = reinterpret_cast<f32x4_t *>(chain_lds);  // slot s of this lane: slot[s * kBlock + t]
     const int64_t total = rows * cq;
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + t; i < total; i += (int64_t)gridDim.x * kBlock) {
-        const int64_t row = i / cq, c4 = i - row * cq;
-        f32x4_t prev = {0.f, 0.f, 0.f, 0.f};
-        for (int j = 0; j < p.n_in; ++j) {
-            const int dt = __builtin_amdgcn_readfirstlane(s_in_dtype[j]), kind = __builtin_amdgcn_readfirstlane(s_in_kind[j]);
-            slot[j * kBlock + t] = rowchain_load(s_in[j], dt, kind, row, c4, i);
+    const int64_t first = BYROW ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * kBlock + t;
+    const int64_t step = BYROW ? total : (int64_t)gridDim.x * kBlock;  // BYROW: one trip, the rows come from the block index
+    const int n_in = p.n_in, n_ops = p.n_ops;
+    for (int64_t i0 = first; i0 < total; i0 += step) {
+        int64_t row, c4, idx;
+        bool own = true;
+        int lane = 0, row_in_block = 0;
+        if constexpr (BYROW) {
+            lane = t & (P - 1);
+            row_in_block = t / P;
+            const int64_t r = (int64_t)blockIdx.x * (kBlock / P) + row_in_block;
+            // lanes past the last row or the row's last group go through the motions (barriers and shuffles
+            // need them) on a clamped position and store nothing
+            own = r < rows && lane < cq;
+            row = r < rows ? r : rows - 1;
+            c4 = lane < cq ? lane : cq - 1;
+            idx = row * cq + c4;
+        } else {
+            if (total <= 0x7fffffff) { const uint32_t r32 = (uint32_t)i0 / (uint32_t)cq; row = r32; c4 = (uint32_t)i0 - r32 * (uint32_t)cq; }
+            else { row = i0 / cq; c4 = i0 - row * cq; }
+            idx = i0;
         }
-        for (int k = 0; k < p.n_ops; ++k) {
-            const int code = __builtin_amdgcn_readfirstlane(s_code[k]), l = __builtin_amdgcn_readfirstlane(s_lhs[k]);
-            const int q = __builtin_amdgcn_readfirstlane(s_rhs[k]), save = __builtin_amdgcn_readfirstlane(s_save[k]);
-            const int dt = __builtin_amdgcn_readfirstlane(s_dtype[k]), kind = __builtin_amdgcn_readfirstlane(s_kind[k]);
+        f32x4_t prev = {0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < n_in; ++j) slot[j * kBlock + t] = rowchain_load(tab->in[j], tab->in_dtype[j], tab->in_kind[j], row, c4, idx);
+        for (int k = 0; k < n_ops; ++k) {
+            const uint64_t d = tab->op[k];
+            const int code = (int)(d & 0xff), l = (int)(int8_t)(d >> 8), q = (int)(int8_t)(d >> 16), save = (int)(int8_t)(d >> 24);
+            const int dt = (int)((d >> 32) & 0xff), kind = (int)((d >> 40) & 0xff);
+            const float s = tab->scalar[k];
+            void *out = tab->out[k];
             f32x4_t a = prev, b = prev;
             if (l != kChainPrev) a = slot[l * kBlock + t];
             if (q != kChainPrev) b = slot[q * kBlock + t];
-            const float s = s_scalar[k];
+            float rowsum = 0.f;
+            if constexpr (BYROW) {
+                if (code == DXH_CHAIN_ROWSUM) {  // the operand sits in slot l (the host sees to that), group j of the row at lane j
+                    __syncthreads();
+                    if (lane < G) {
+                        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+                        const f32x4_t *src = slot + l * kBlock + row_in_block * P;
+                        row_lane_fold<R_SUM, float, 4>(acc, lane, G, cq, [&](int64_t i) __attribute__((always_inline)) { return __builtin_bit_cast(vec_t<float, 4>, src[i]); });
+                        const float v = row_group_fold<R_SUM, float, 4>(acc, G);
+                        if (lane == 0) row_sums[row_in_block] = v;
+                    }
+                    __syncthreads();
+                    rowsum = row_sums[row_in_block];
+                }
+            }
             float y[4];
 #define DXH_RC_BIN(Op) _Pragma("unroll") for (int v = 0; v < 4; ++v) y[v] = Op::f(a[v], b[v]); break
 #define DXH_RC_SCALAR(Op) _Pragma("unroll") for (int v = 0; v < 4; ++v) y[v] = Op::f(a[v], s); break
@@ -544,17 +580,41 @@ __global__ __launch_bounds__(kBlock) void chain_rows_kernel(const RowChainArgs p
             case DXH_CHAIN_EXP: DXH_RC_UNARY(OpExp);
             case DXH_CHAIN_LOG: DXH_RC_UNARY(OpLog);
             case DXH_CHAIN_SQUARE: DXH_RC_UNARY(OpSquare);
+            case DXH_CHAIN_ROWSUM: _Pragma("unroll") for (int v = 0; v < 4; ++v) y[v] = rowsum; break;
             default: _Pragma("unroll") for (int v = 0; v < 4; ++v) y[v] = a[v]; break;  // DXH_CHAIN_COPY
             }
 #undef DXH_RC_BIN
 #undef DXH_RC_SCALAR
 #undef DXH_RC_UNARY
-            rowchain_round_store(y, s_out[k], dt, kind, row, c4, i);
+            rowchain_round_store(y, out, dt, kind, own, row, c4, idx);
             prev = f32x4_t{y[0], y[1], y[2], y[3]};
             if (save >= 0) slot[save * kBlock + t] = prev;
         }
     }
 }
+
+// Launches with more dynamic LDS than a kernel gets unasked need the limit raised once per device.
+// That is a call on the function, not on a stream: it is made at device set-up (dxh_set_device) or
+// by the first launch that needs it, unless that one is being captured.
+namespace {
+std::mutex g_rows_mutex;
+bool g_rows_lds_raised[64] = {};
+}
+int chain_rows_raise_lds(hipStream_t st, bool may_be_capturing) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { (void)hipGetLastError(); return (int)e; }
+    if (dev < 0 || dev >= 64) return DXH_ERR_ARG;
+    std::lock_guard<std::mutex> lock(g_rows_mutex);
+    if (g_rows_lds_raised[dev]) return DXH_OK;
+    if (may_be_capturing && stream_is_capturing(st)) return DXH_ERR_NOT_READY;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chain_rows_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRowLdsMax);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(&chain_rows_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRowLdsMax);
+    if (e != hipSuccess) { (void)hipGetLastError(); return (int)e; }
+    g_rows_lds_raised[dev] = true;
+    return DXH_OK;
+}
+void chain_device_init() { (void)chain_rows_raise_lds(nullptr, false); }
 
 }  // namespace dxh
 
@@ -651,8 +711,14 @@ int dxh_chain(int dtype, const void *const *inputs, int n_inputs, const dxh_chai
 }
 
 
+int dxh_chain_rows_can_sum(int64_t rows, int64_t cols) {
+    if (rows < 1 || cols < 4 || cols % 4 != 0) return 0;
+    const int g = sum_rows_group_f32(rows, cols);
+    return g > 0 && cols / 4 <= (int64_t)g * kRowVecs;
+}
+
 int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain_rows_op *ops, int n_ops, int64_t rows, int64_t cols, void *stream) {
-    if (rows < 0 || cols < 0 || n_ops < 1 || n_ops > kChainOps || n_inputs < 0 || n_inputs > kChainInputs || !ops || (n_inputs > 0 && !inputs)) return DXH_ERR_ARG;
+    if (rows < 0 || cols < 0 || n_ops < 1 || n_ops > kRowOps || n_inputs < 0 || n_inputs > kChainInputs || !ops || (n_inputs > 0 && !inputs)) return DXH_ERR_ARG;
     if (cols % 4 != 0) return DXH_ERR_ALIGN;
     if (rows > 0 && cols / 4 > INT64_MAX / rows) return DXH_ERR_SHAPE;
     auto dtype_code = [](int dtype) { return dtype == DXH_F32 ? (int)kRcF32 : dtype == DXH_BF16 ? (int)kRcBF16 : dtype == DXH_F16 ? (int)kRcF16 : -1; };
@@ -666,42 +732,85 @@ int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain
         if (dt < 0) return DXH_ERR_DTYPE;
         if (!inputs[j].data || inputs[j].extent < DXH_CHAIN_FULL || inputs[j].extent > DXH_CHAIN_COLUMN) return DXH_ERR_ARG;
         if (!aligned(inputs[j].data, align_of(dt, inputs[j].extent))) return DXH_ERR_ALIGN;
-        p.in[j] = inputs[j].data; p.in_dtype[j] = (int8_t)dt; p.in_kind[j] = (int8_t)inputs[j].extent;
+        p.in[j] = inputs[j].data; p.in_dtype[j] = (uint8_t)dt; p.in_kind[j] = (uint8_t)inputs[j].extent;
     }
     int next_slot = n_inputs;
-    for (int k = 0; k < n_ops; ++k) p.save[k] = -1;
+    bool by_row = false;
+    int save_of[kRowOps], kind_of[kRowOps], dtype_of[kRowOps], code_of[kRowOps], lhs_of[kRowOps], rhs_of[kRowOps];
+    for (int k = 0; k < n_ops; ++k) save_of[k] = -1;
     constexpr int kBad = -2;
-    // operand of op k (see dxh_chain); `want` is the op's extent: a [rows, cols] op takes anything, an op
-    // on vectors only vectors of its own kind
-    auto operand = [&](int ref, int k, int want) {
-        if (ref >= 0 && ref < n_inputs) return want == kRowFull || p.in_kind[ref] == want ? ref : kBad;
+    // operand of op k (see dxh_chain); `want` is the extent it must have, or -1 for any; `in_slot`: never
+    // the registers, even when it is the result of the op before
+    auto operand = [&](int ref, int k, int want, bool in_slot, int *dtype) {
+        if (ref >= 0 && ref < n_inputs) {
+            *dtype = p.in_dtype[ref];
+            return want < 0 || p.in_kind[ref] == want ? ref : kBad;
+        }
         if (ref < DXH_CHAIN_RESULT || ref >= DXH_CHAIN_RESULT + k) return kBad;
         const int j = ref - DXH_CHAIN_RESULT;
-        if (want != kRowFull && p.kind[j] != want) return kBad;
-        if (j == k - 1) return kChainPrev;
-        if (p.save[j] < 0) p.save[j] = (int8_t)next_slot++;
-        return (int)p.save[j];
+        *dtype = dtype_of[j];
+        if (want >= 0 && kind_of[j] != want) return kBad;
+        if (j == k - 1 && !in_slot) return kChainPrev;
+        if (save_of[j] < 0) save_of[j] = next_slot++;
+        return save_of[j];
     };
     for (int k = 0; k < n_ops; ++k) {
         const dxh_chain_rows_op &o = ops[k];
         const int dt = dtype_code(o.dtype);
         if (dt < 0) return DXH_ERR_DTYPE;
-        if (o.code < DXH_CHAIN_ADD || o.code > DXH_CHAIN_COPY || o.extent < DXH_CHAIN_FULL || o.extent > DXH_CHAIN_COLUMN || (!o.out && k == n_ops - 1)) return DXH_ERR_ARG;
+        if (o.code < DXH_CHAIN_ADD || o.code > DXH_CHAIN_ROWSUM || o.extent < DXH_CHAIN_FULL || o.extent > DXH_CHAIN_COLUMN || (!o.out && k == n_ops - 1)) return DXH_ERR_ARG;
         if (o.out && !aligned(o.out, align_of(dt, o.extent))) return DXH_ERR_ALIGN;
-        p.kind[k] = (int8_t)o.extent;  // before operand(): a later op asks for it
-        const int l = operand(o.lhs, k, o.extent), r = o.code <= DXH_CHAIN_MIN ? operand(o.rhs, k, o.extent) : l;
+        kind_of[k] = o.extent;  // before operand(): a later op asks for it
+        dtype_of[k] = dt;
+        const bool rowsum = o.code == DXH_CHAIN_ROWSUM;
+        // an op of full extent takes anything, an op on vectors only vectors of its own kind; the row sum
+        // turns an fp32 [rows, cols] operand into an fp32 column
+        const int want = rowsum ? (int)kRowFull : o.extent == DXH_CHAIN_FULL ? -1 : o.extent;
+        int ldt = 0, rdt = 0;
+        const int l = operand(o.lhs, k, want, rowsum, &ldt), r = o.code <= DXH_CHAIN_MIN ? operand(o.rhs, k, want, false, &rdt) : l;
         if (l == kBad || r == kBad) return DXH_ERR_ARG;
+        if (rowsum) {
+            if (o.extent != DXH_CHAIN_COLUMN) return DXH_ERR_ARG;
+            if (dt != kRcF32 || ldt != kRcF32) return DXH_ERR_DTYPE;
+            by_row = true;
+        }
         for (int j = 0; j < n_inputs; ++j)
             if (o.out && o.out == inputs[j].data && inputs[j].extent != DXH_CHAIN_FULL) return DXH_ERR_ARG;  // lanes would race for it
-        p.code[k] = (int8_t)o.code; p.lhs[k] = (int8_t)l; p.rhs[k] = (int8_t)r; p.out[k] = o.out; p.dtype[k] = (int8_t)dt;
+        code_of[k] = o.code; lhs_of[k] = l; rhs_of[k] = r; p.out[k] = o.out;
         const float sf = (float)o.scalar.f;
         p.scalar[k] = dt == kRcF32 ? sf : dt == kRcBF16 ? load_acc(to_bf16(sf)) : load_acc(to_f16(sf));
     }
+    int slots = std::max(n_inputs, 1);
+    for (int k = 0; k < n_ops; ++k) {  // save_of[k] is final only now: a later op may have asked for the slot
+        slots = std::max(slots, save_of[k] + 1);
+        p.op[k] = (uint64_t)(uint8_t)code_of[k] | (uint64_t)(uint8_t)(int8_t)lhs_of[k] << 8 | (uint64_t)(uint8_t)(int8_t)rhs_of[k] << 16 |
+                  (uint64_t)(uint8_t)(int8_t)save_of[k] << 24 | (uint64_t)(uint8_t)dtype_of[k] << 32 | (uint64_t)(uint8_t)kind_of[k] << 40;
+    }
+    const int64_t cq = cols / 4;
+    int group = 0, per_row = 1;
+    if (by_row) {  // the first lanes of a row fold it as dxh_sum's row stage would, or the sums would not be its sums
+        if (rows == 0 || cols == 0) return DXH_OK;
+        group = sum_rows_group_f32(rows, cols);
+        if (group <= 0 || cq > (int64_t)group * kRowVecs) return DXH_ERR_SHAPE;
+        per_row = group;
+        while (per_row < cq) per_row <<= 1;  // at most group * kRowVecs = kBlock lanes
+    }
+    const size_t lds = (size_t)slots * kBlock * kVecBytes;
+    if (lds > kRowLdsMax) return DXH_ERR_SHAPE;
     if (rows == 0 || cols == 0) return DXH_OK;
-    int slots = n_inputs;
-    for (int k = 0; k < n_ops; ++k) slots = std::max(slots, p.save[k] + 1);
-    const int64_t cq = cols / 4, total = rows * cq, blocks = (total + kBlock - 1) / kBlock;
-    chain_rows_kernel<<<(unsigned)std::min<int64_t>(blocks, 1 << 22), kBlock, (size_t)std::max(slots, 1) * kBlock * kVecBytes, as_stream(stream)>>>(p, rows, cq);
+    hipStream_t st = as_stream(stream);
+    if (lds > kRowLdsDefault) {
+        const int rc = chain_rows_raise_lds(st, true);
+        if (rc != DXH_OK) return rc;
+    }
+    if (by_row) {
+        const int64_t rows_per_block = kBlock / per_row, blocks = (rows + rows_per_block - 1) / rows_per_block;
+        if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
+        chain_rows_kernel<true><<<(unsigned)blocks, kBlock, lds, st>>>(p, rows, cq, group, per_row);
+    } else {
+        const int64_t blocks = (rows * cq + kBlock - 1) / kBlock;
+        chain_rows_kernel<false><<<(unsigned)std::min<int64_t>(blocks, 1 << 22), kBlock, lds, st>>>(p, rows, cq, 1, 1);
+    }
     return launch_status();
 }
 

@@ -22,63 +22,12 @@
 // arrives last adds the S partials in a fixed order (reduce_col_fused_kernel; the counters
 // live in a file-scope device array and return to zero, see finish_counters).  Both stage
 // kinds are HBM-bound: algorithmic bytes = input once + output once.
-#include "common.hpp"
-#include <limits>
+#include "reduce_order.hpp"
 #include <map>
 #include <mutex>
 #include <vector>
 
 namespace dxh {
-
-enum RedKind { R_SUM = 0, R_PROD = 1, R_MAX = 2, R_MIN = 3 };
-
-template <typename T> struct racc_of { using type = T; };
-template <> struct racc_of<bf16_t> { using type = float; };
-template <> struct racc_of<f16_t> { using type = float; };
-template <> struct racc_of<int16_t> { using type = int32_t; };
-template <> struct racc_of<int8_t> { using type = int32_t; };
-template <typename T> using racc_t = typename racc_of<T>::type;
-
-template <typename A, typename T> __device__ inline A rload(T x) {
-    if constexpr (std::is_same_v<T, bf16_t> || std::is_same_v<T, f16_t>) return load_acc(x);
-    else return A(x);
-}
-template <typename T, typename A> __device__ inline T rstore(A v) {
-    if constexpr (std::is_same_v<T, bf16_t>) return to_bf16(v);
-    else if constexpr (std::is_same_v<T, f16_t>) return to_f16(v);
-    else return T(v);  // integers truncate: wrap-around arithmetic is width independent
-}
-
-// identity element: 0 / 1 / lowest() / max() of the STORAGE type, as the reference
-// pre-fills the result (reduce_miaobyte.hpp:24,101,191,274)
-template <int K, typename A, typename TS> __host__ __device__ inline A rinit() {
-    if constexpr (K == R_SUM) return A(0);
-    else if constexpr (K == R_PROD) return A(1);
-    else if constexpr (std::is_same_v<TS, bf16_t>) return K == R_MAX ? -3.3895313892515355e38f : 3.3895313892515355e38f;
-    else if constexpr (std::is_same_v<TS, f16_t>) return K == R_MAX ? -65504.0f : 65504.0f;
-    else return K == R_MAX ? A(std::numeric_limits<TS>::lowest()) : A(std::numeric_limits<TS>::max());
-}
-template <int K, typename A> __device__ inline A rop(A a, A b) {
-    if constexpr (K == R_SUM) {
-        if constexpr (std::is_integral_v<A>) { using U = std::make_unsigned_t<A>; return A(U(a) + U(b)); }
-        else return a + b;
-    } else if constexpr (K == R_PROD) {
-        if constexpr (std::is_integral_v<A>) { using U = std::make_unsigned_t<A>; return A(U(a) * U(b)); }
-        else return a * b;
-    } else if constexpr (K == R_MAX) return (a < b) ? b : a;
-    else return (b < a) ? b : a;
-}
-
-template <typename A> __device__ inline A shfl_xor_any(A v, int off) {
-    if constexpr (sizeof(A) == 8) {
-        uint64_t u = __builtin_bit_cast(uint64_t, v);
-        uint32_t lo = __shfl_xor((int)(uint32_t)u, off, kWave);
-        uint32_t hi = __shfl_xor((int)(uint32_t)(u >> 32), off, kWave);
-        return __builtin_bit_cast(A, (uint64_t(hi) << 32) | lo);
-    } else {
-        return __builtin_bit_cast(A, __shfl_xor(__builtin_bit_cast(int, v), off, kWave));
-    }
-}
 
 // ---- row stage ---------------------------------------------------------------------------
 // in [pre, R] (R contiguous) -> out [pre, S]; chunk s covers r in [s*chunk, min(R,(s+1)*chunk)).
@@ -104,41 +53,12 @@ __device__ __forceinline__ void reduce_row_body(racc_t<TS> *lds, const Tin *__re
         const Tin *p = in + row * R + r0;
         const VT *pv = reinterpret_cast<const VT *>(p);
         const int64_t lv = len / V;
-        int64_t i = lane;
-        // 8 independent 16-byte non-temporal loads in flight per lane, then 4, then singles
-        for (; i + 7 * (int64_t)G < lv; i += 8 * (int64_t)G) {
-            VT x[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) x[u] = ld_sel<NTL>(&pv[i + u * (int64_t)G]);
-#pragma unroll
-            for (int k = 0; k < V; ++k) {
-                A t0 = rop<K, A>(rop<K, A>(rload<A>(x[0].v[k]), rload<A>(x[1].v[k])), rop<K, A>(rload<A>(x[2].v[k]), rload<A>(x[3].v[k])));
-                A t1 = rop<K, A>(rop<K, A>(rload<A>(x[4].v[k]), rload<A>(x[5].v[k])), rop<K, A>(rload<A>(x[6].v[k]), rload<A>(x[7].v[k])));
-                acc[k] = rop<K, A>(acc[k], rop<K, A>(t0, t1));
-            }
-        }
-        for (; i + 3 * (int64_t)G < lv; i += 4 * (int64_t)G) {
-            VT x0 = ld_sel<NTL>(&pv[i]), x1 = ld_sel<NTL>(&pv[i + G]), x2 = ld_sel<NTL>(&pv[i + 2 * (int64_t)G]), x3 = ld_sel<NTL>(&pv[i + 3 * (int64_t)G]);
-#pragma unroll
-            for (int k = 0; k < V; ++k) {
-                A t0 = rop<K, A>(rload<A>(x0.v[k]), rload<A>(x1.v[k]));
-                A t1 = rop<K, A>(rload<A>(x2.v[k]), rload<A>(x3.v[k]));
-                acc[k] = rop<K, A>(acc[k], rop<K, A>(t0, t1));
-            }
-        }
-        for (; i < lv; i += G) {
-            VT x = ld_sel<NTL>(&pv[i]);
-#pragma unroll
-            for (int k = 0; k < V; ++k) acc[k] = rop<K, A>(acc[k], rload<A>(x.v[k]));
-        }
+        // 8 independent 16-byte loads in flight per lane, then 4, then singles
+        row_lane_fold<K, A, V>(acc, lane, G, lv, [&](int64_t i) __attribute__((always_inline)) { return ld_sel<NTL>(&pv[i]); });
         for (int64_t j = lv * V + lane; j < len; j += G) acc[0] = rop<K, A>(acc[0], rload<A>(p[j]));
     }
-    A v = acc[0];
-#pragma unroll
-    for (int k = 1; k < V; ++k) v = rop<K, A>(v, acc[k]);
     // lanes of one group are adjacent, so xor-shuffles below G stay inside the group
-    const int gw = G < kWave ? G : kWave;
-    for (int off = gw >> 1; off > 0; off >>= 1) v = rop<K, A>(v, shfl_xor_any<A>(v, off));
+    const A v = row_group_fold<K, A, V>(acc, G);
     if (G == kBlock) {
         if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = v;
         __syncthreads();
@@ -592,6 +512,16 @@ inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, cons
     }
     pl.ws_bytes = off;
     return DXH_OK;
+}
+
+int sum_rows_group_f32(int64_t rows, int64_t cols) {
+    if (rows < 1 || cols < 1 || rows > INT32_MAX || cols > INT32_MAX) return 0;
+    const int32_t shape[2] = {(int32_t)rows, (int32_t)cols}, dims[1] = {1};
+    Plan pl;
+    if (build_plan(sizeof(float), sizeof(float), shape, 2, dims, 1, pl) != DXH_OK || pl.copy_only || pl.stages.size() != 1) return 0;
+    const Stage &st = pl.stages[0];
+    if (!st.row || st.S != 1 || st.V != kVecBytes / (int)sizeof(float) || st.G > kWave || st.pre != rows || st.R != cols) return 0;
+    return st.G;
 }
 
 template <int K, typename Tin, typename Tout, typename TS>

@@ -64,7 +64,7 @@ int dxh_device_count(int *count) {
 }
 int dxh_set_device(int device) {
     hipError_t e = hipSetDevice(device);
-    if (e == hipSuccess) dxh::reduce_device_init();
+    if (e == hipSuccess) { dxh::reduce_device_init(); dxh::chain_device_init(); }
     return (int)e;
 }
 int dxh_device_name(char *buf, size_t buflen) {

@@ -81,6 +81,7 @@ void reg(TfFactory &f, const char *name, const char *author, const char *tftype,
     if (op == "todtype") { tf->chain_code = DXH_CHAIN_COPY; tf->chain_kind = 5; }
     if (op == "broadcastTo") { tf->chain_code = DXH_CHAIN_COPY; tf->chain_kind = 6; }
     if (op == "powscalar") { tf->chain_code = DXH_CHAIN_SQUARE; tf->chain_kind = 7; }
+    if (op == "sum") { tf->chain_code = DXH_CHAIN_ROWSUM; tf->chain_kind = 8; }
     tf->graph_safe = kind == "elementwise" || kind == "reduce" || kind == "changeshape" || op == "matmul" ||
                      op == "constant" || op == "arange";
     if (op == "reshape") tf->graph_safe = false;  // rewrites the tensor's shape on the host
@@ -574,7 +575,7 @@ struct ChainPlan {
     std::vector<dxh_chain_tensor> row_inputs;
     std::vector<dxh_chain_rows_op> row_ops;
 };
-enum { kChainTodtype = 5, kChainBroadcast = 6, kChainPowscalar = 7 };
+enum { kChainTodtype = 5, kChainBroadcast = 6, kChainPowscalar = 7, kChainSum = 8 };
 // Builds the longest run starting at tfs[first].  A tensor operand is the latest result of the run
 // with that name, else an input of the run (read before the run writes anything, which is what a
 // line-by-line execution sees as long as no earlier line of the run has written it — and those are
@@ -584,7 +585,7 @@ enum { kChainTodtype = 5, kChainBroadcast = 6, kChainPowscalar = 7 };
 // a line that is not a chainable float op, does not fit the view, needs a ninth input, would overwrite
 // a vector that the run reads from memory (lanes of other rows or columns may not have read it yet),
 // or whose operands are missing or mismatched (the ordinary path then reports the error for that line).
-size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem, ChainPlan &plan) {
+size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem, ChainPlan &plan, size_t max_ops = DXH_CHAIN_ROWS_MAX_OPS) {
     struct Input { std::string name; const void *data; int dtype, extent; };
     struct Op { dxh_chain_rows_op op; std::string out_name; };
     std::vector<Input> inputs;
@@ -601,11 +602,11 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
         }
         return -1;
     };
-    for (size_t i = first; i < tfs.size() && ops.size() < DXH_CHAIN_MAX_OPS; ++i) {
+    for (size_t i = first; i < tfs.size() && ops.size() < max_ops; ++i) {
         const TF *tf = tfs[i].get();
         if (!tf || tf->chain_kind == 0 || tf->metadata.benchmark_repeat > 1 || tf->returns.size() != 1) break;
         const int kind = tf->chain_kind;
-        const size_t nargs = kind == 4 || kind == kChainTodtype ? 1 : 2;
+        const size_t nargs = kind == 4 || kind == kChainTodtype ? 1 : kind == kChainSum ? 3 : 2;
         if (tf->args.size() != nargs) break;
         const Param *tensors[2] = {nullptr, nullptr};
         const Param *scalar = nullptr;
@@ -627,6 +628,17 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
         op.op.dtype = out->dtype();
         op.op.extent = extent_of(*out);
         op.out_name = tf->returns[0].textvalue;
+        if (kind == kChainSum) {
+            // the sum of every row of an fp32 [rows, cols] tensor, when the row stage of dxh_sum would be one lane group per row
+            if (ops.empty() || rows < 2 || out->dtype() != DXH_F32 || out->shape.size != rows || !dxh_chain_rows_can_sum(rows, cols)) break;
+            auto in = mem.findtensor(tf->args[0].textvalue);
+            if (!in || in->shape.dim() < 1 || in->shape.at(-1) != cols) break;
+            try {
+                if (checked_dims(in->shape.shape, ints_of(tf->args[1], mem)) != std::vector<int>{in->shape.dim() - 1}) break;
+                (void)bool_of(tf->args[2]);
+            } catch (const std::exception &) { break; }
+            op.op.extent = DXH_CHAIN_COLUMN;
+        }
         if (op.op.extent < 0) break;
         bool line_needs_rows = op.op.extent != DXH_CHAIN_FULL || kind >= kChainTodtype || (!ops.empty() && out->dtype() != ops[0].op.dtype);
         if (scalar) {
@@ -649,7 +661,8 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
             if (extent < 0) { ok = false; break; }
             // what the line itself would refuse: another dtype (but for todtype), another size (but for broadcastTo)
             if (kind != kChainTodtype && t->dtype() != out->dtype()) { ok = false; break; }
-            if (kind != kChainBroadcast && (extent != op.op.extent || t->shape.size != out->shape.size)) { ok = false; break; }
+            if (kind == kChainSum && extent != DXH_CHAIN_FULL) { ok = false; break; }
+            if (kind != kChainBroadcast && kind != kChainSum && (extent != op.op.extent || t->shape.size != out->shape.size)) { ok = false; break; }
             if (kind == kChainBroadcast && broadcast_shape(t->shape.shape, out->shape.shape) != out->shape.shape) { ok = false; break; }
             line_needs_rows = line_needs_rows || extent != DXH_CHAIN_FULL || t->dtype() != out->dtype();
             int ref = -1;
@@ -681,6 +694,10 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
     }
     const size_t count = ops.size();
     if (count < 2) return count;
+    if (!needs_rows && count > DXH_CHAIN_MAX_OPS) {  // the one-dtype form takes fewer ops
+        plan = ChainPlan{};
+        return plan_chain(tfs, first, mem, plan, DXH_CHAIN_MAX_OPS);
+    }
     for (size_t j = 0; j < count; ++j)
         for (size_t m = j + 1; m < count; ++m)
             if (ops[m].out_name == ops[j].out_name) ops[j].op.out = nullptr;  // overwritten by line m of the run

@@ -217,9 +217,10 @@ enum dxh_chain_code {
     DXH_CHAIN_ADDSCALAR, DXH_CHAIN_SUBSCALAR, DXH_CHAIN_RSUBSCALAR, DXH_CHAIN_MULSCALAR,               /* lhs op scalar; R: scalar op lhs */
     DXH_CHAIN_DIVSCALAR, DXH_CHAIN_RDIVSCALAR, DXH_CHAIN_MAXSCALAR, DXH_CHAIN_MINSCALAR,
     DXH_CHAIN_SQRT, DXH_CHAIN_EXP, DXH_CHAIN_LOG,                                                      /* f(lhs) */
-    DXH_CHAIN_SQUARE, DXH_CHAIN_COPY                                                                   /* dxh_chain_rows only */
+    DXH_CHAIN_SQUARE, DXH_CHAIN_COPY, DXH_CHAIN_ROWSUM                                                 /* dxh_chain_rows only */
 };
 #define DXH_CHAIN_MAX_OPS 8
+#define DXH_CHAIN_ROWS_MAX_OPS 16
 #define DXH_CHAIN_MAX_INPUTS 8
 #define DXH_CHAIN_RESULT 16
 typedef struct dxh_chain_op {
@@ -243,7 +244,16 @@ DXH_API int dxh_chain(int dtype, const void *const *inputs, int n_inputs, const 
  * vectors of its own kind only and stores `cols` or `rows` elements.  Operand references, in-place use
  * of [rows, cols] tensors and out = NULL as for dxh_chain; a vector input must not be an `out` of the
  * run (DXH_ERR_ARG: run the ops that update it in place on their own).  cols a multiple of 4 and
- * [rows, cols] / row-vector pointers aligned to 4 elements, else DXH_ERR_ALIGN. */
+ * [rows, cols] / row-vector pointers aligned to 4 elements, else DXH_ERR_ALIGN.  Up to
+ * DXH_CHAIN_ROWS_MAX_OPS ops.
+ * DXH_CHAIN_ROWSUM (fp32 only) is launch_sum (reduce_miaobyte.cuh:16-21) over the last axis inside the
+ * run: lhs of full extent, the result a column vector with the bits dxh_sum stores for the same rows
+ * (the lanes share the rows as its kernel would and add in its order).  That needs rows short enough
+ * for one lane group: dxh_chain_rows_can_sum says whether a [rows, cols] view qualifies (1) or not (0),
+ * and a run with a row sum over one that does not is refused with DXH_ERR_SHAPE, as is a run that needs
+ * more LDS than a CU has.  A run whose LDS need exceeds 64 KiB raises the kernel's limit first: once
+ * per device, in dxh_set_device or on such a run's first launch, which must not be one under stream
+ * capture (DXH_ERR_NOT_READY then). */
 enum dxh_chain_extent { DXH_CHAIN_FULL = 0, DXH_CHAIN_ROW = 1, DXH_CHAIN_COLUMN = 2 };
 typedef struct dxh_chain_tensor {
     const void *data;
@@ -258,6 +268,7 @@ typedef struct dxh_chain_rows_op {
     int32_t dtype;     /* of the result */
     int32_t extent;    /* of the result */
 } dxh_chain_rows_op;
+DXH_API int dxh_chain_rows_can_sum(int64_t rows, int64_t cols);
 DXH_API int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain_rows_op *ops, int n_ops, int64_t rows, int64_t cols, void *stream);
 
 /* ---- cast: launch_todtype elementwise_miaobyte_basic.cuh:11-16.

@@ -71,7 +71,7 @@ def test_argument_errors_need_no_gpu():
     assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(17, 0, 1, 48)), 1, 8, None) == -2   # unknown op code
     assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(0, 0, 1, 50)), 1, 8, None) == -5    # output off a 16-byte boundary
     assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(0, 0, 1, None)), 1, 8, None) == -2  # the last op must store
-    assert len(dx.CHAIN_CODES) == 19 and dx.CHAIN_CODES[16] == "log" and dx.CHAIN_CODES[18] == "copy"
+    assert len(dx.CHAIN_CODES) == 20 and dx.CHAIN_CODES[16] == "log" and dx.CHAIN_CODES[18] == "copy"
     # dxh_chain_rows: the same checks, and those on extents: a [rows, cols] op takes any operand, an op on
     # vectors only vectors of its kind; a vector input may not be an output of the run
     T, R = dx.ChainTensor, dx.ChainRowsOp
@@ -83,7 +83,7 @@ def test_argument_errors_need_no_gpu():
     assert run(rop(2, 0, 1, 512), cols=18) == -5                             # cols not a multiple of 4
     assert run(rop(2, 0, 1, 512, dx.F64)) == -1                              # no fp64 in this form
     assert L.dxh_chain_rows((T * 1)(T(64, dx.I32, FULL)), 1, (R * 1)(rop(18, 0, 0, 512)), 1, 8, 16, None) == -1
-    assert run(rop(19, 0, 0, 512)) == -2                                     # unknown op code
+    assert run(rop(20, 0, 0, 512)) == -2                                     # unknown op code
     assert run(rop(2, 0, 3, 512)) == -2                                      # input 3 does not exist
     assert run(rop(2, 0, 1, 512, extent=3)) == -2                            # unknown extent
     assert run(rop(2, 0, 1, None)) == -2                                     # the last op must store
@@ -94,6 +94,16 @@ def test_argument_errors_need_no_gpu():
     assert run(rop(9, 2, 0, 512, dx.F32, ROW)) == -2                         # ... nor a column vector
     assert run(rop(18, 1, 0, 1024, dx.F32, ROW), rop(0, dx.CHAIN_RESULT, 2, 512, dx.F32, COL)) == -2  # a row result into a column op
     assert run(rop(9, 2, 0, 256, dx.F32, COL), rop(2, 0, dx.CHAIN_RESULT, 512)) == -2  # overwrites the column vector it reads
+    # the row sum: an fp32 [rows, cols] operand into an fp32 column, over views whose rows one lane group folds
+    assert run(rop(19, 0, 0, 512, dx.F32, FULL)) == -2                       # its result is a column
+    assert run(rop(19, 2, 0, 512, dx.F32, COL)) == -2                        # its operand is not
+    assert run(rop(19, 0, 0, 512, dx.BF16, COL)) == -1                       # fp32 only
+    assert L.dxh_chain_rows((T * 1)(T(64, dx.BF16, FULL)), 1, (R * 1)(rop(19, 0, 0, 512, dx.F32, COL)), 1, 8, 16, None) == -1
+    assert L.dxh_chain_rows_can_sum(2048, 896) == 1 and L.dxh_chain_rows_can_sum(8, 16) == 1
+    assert L.dxh_chain_rows_can_sum(8, 18) == 0 and L.dxh_chain_rows_can_sum(0, 16) == 0
+    assert L.dxh_chain_rows_can_sum(64, 1 << 20) == 0                        # a row that long is cut or takes the whole workgroup
+    assert run(rop(19, 0, 0, 512, dx.F32, COL), rows=64, cols=1 << 20) == -3
+    assert run(*([rop(2, 0, 0, 512)] * 17)) == -2                            # too many ops
 
 
 def test_tuning_knobs_validate_their_values():

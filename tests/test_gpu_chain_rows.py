@@ -80,12 +80,18 @@ def run_separately(dxh, orc, inputs, prog, rows, cols):
             assert adt == dt and ae == e
             dx.check(getattr(dxh, "dxh_" + name)(dt, a.ptr, dx.scalar(s), out.ptr, n, None), name)
             assert getattr(orc, "orc_" + name)(dt, hp(ah), dx.scalar(s), hp(want), n) == 0
+        elif name == "rowsum":
+            assert adt == dt == dx.F32 and ae == FULL and e == COL
+            dx.check(dxh.dxh_sum(dt, a.ptr, dx.i32arr([rows, cols]), 2, dx.i32arr([1]), 1, out.ptr, None, 0, None), "sum")
+            want = None  # the order of a float sum is the kernel's own: checked against float64 below
+            ref = ah.astype(np.float64).reshape(rows, cols)
+            assert np.all(np.abs(out.get().astype(np.float64) - ref.sum(1)) <= 1e-6 * np.abs(ref).sum(1) + 1e-30), ("sum", rows, cols)
         else:
             assert adt == dt and ae == e and name == "sqrt"
             dx.check(dxh.dxh_sqrt(dt, a.ptr, out.ptr, n, None), name)
             assert orc.orc_sqrt(dt, hp(ah), hp(want), n) == 0
         got = out.get()
-        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), ("oracle", k, name, rows, cols)
+        assert want is None or np.array_equal(got.view(np.uint8), want.view(np.uint8)), ("oracle", k, name, rows, cols)
         outs.append(out)
     return outs
 
@@ -133,6 +139,54 @@ def test_rmsnorm_lines_as_runs(dxh, orc, half):
         dx.check(rc, "chain_rows")
         for k in (0, 2, 3, 4, 5):
             assert same_bits(got2[k], want[k]), ("after, xn stored once", rows, cols, k)
+
+
+@pytest.mark.parametrize("half", [dx.BF16, dx.F16])
+def test_whole_rmsnorm_as_one_run(dxh, orc, half):
+    """All thirteen elementwise and reduce lines of the RMSNorm in one launch: the row sum sits in
+    the middle of the run (its operand produced by the run, its result a column vector that the
+    scalar lines then work on), with the lanes laid out as dxh_sum's own kernel has them, so every
+    tensor — the sums included — has the bits of the thirteen separate launches.  Shapes: rows of
+    one to four vector groups per lane, row counts that leave the last workgroup ragged, the
+    config-5 size; and shapes whose rows dxh_sum would not give to one lane group are refused."""
+    rng = np.random.default_rng(1300 + half)
+    for rows, cols in [(2048, 896), (5, 12), (2, 4), (257, 1000), (64, 1024), (1000, 256), (33, 64), (7, 520)]:
+        assert dxh.dxh_chain_rows_can_sum(rows, cols) == 1, (rows, cols)
+        x = Dev(H.rand(rng, half, rows * cols, -2.0, 2.0))
+        w = Dev(H.rand(rng, half, cols, 0.5, 1.5))
+        prog = [("copy", 0, 0, 0, dx.F32, FULL),             # todtype(x) -> xf
+                ("square", R + 0, 0, 2.0, dx.F32, FULL),      # powscalar(xf, 2) -> sq
+                ("rowsum", R + 1, 0, 0, dx.F32, COL),         # sum(sq, [-1], keepdims) -> var
+                ("divscalar", R + 2, 0, float(cols), dx.F32, COL),
+                ("addscalar", R + 3, 0, 1e-6, dx.F32, COL),
+                ("sqrt", R + 4, 0, 0, dx.F32, COL),
+                ("rdivscalar", R + 5, 0, 1.0, dx.F32, COL),
+                ("copy", R + 6, 0, 0, dx.F32, FULL),          # broadcastTo(var) -> rs
+                ("mul", R + 0, R + 7, 0, dx.F32, FULL),       # xf * rs -> xn
+                ("copy", 1, 0, 0, dx.F32, ROW),               # todtype(w) -> wf1
+                ("copy", R + 9, 0, 0, dx.F32, FULL),          # broadcastTo(wf1) -> wf
+                ("mul", R + 10, R + 8, 0, dx.F32, FULL),      # wf * xn -> xn
+                ("copy", R + 11, 0, 0, half, FULL)]           # todtype(xn) -> h
+        ins = [(x, half, FULL), (w, half, ROW)]
+        want = run_separately(dxh, orc, ins, prog, rows, cols)
+        rc, got = run_rows(dxh, ins, prog, rows, cols)
+        dx.check(rc, "chain_rows")
+        for k in range(len(prog)):
+            assert same_bits(got[k], want[k]), (rows, cols, k, prog[k][0])
+        # as the IR has it: var and xn written several times, stored once
+        outs = [Dev.empty(count(e, rows, cols), H.NP[dt]) for (_, _, _, _, dt, e) in prog]
+        for k in (2, 3, 4, 5, 8):
+            outs[k] = None
+        rc, got2 = run_rows(dxh, ins, prog, rows, cols, outs=outs)
+        dx.check(rc, "chain_rows")
+        for k in (0, 1, 6, 7, 9, 10, 11, 12):
+            assert same_bits(got2[k], want[k]), ("stored once", rows, cols, k)
+    # rows too long for one lane group: refused, the caller runs the lines one by one
+    for rows, cols in [(4, 8192), (2, 1 << 16)]:
+        assert dxh.dxh_chain_rows_can_sum(rows, cols) == 0
+        x = Dev(H.rand(rng, dx.F32, rows * cols))
+        rc, _ = run_rows(dxh, [(x, dx.F32, FULL)], [("rowsum", 0, 0, 0, dx.F32, COL)], rows, cols)
+        assert rc == -3
 
 
 def model(inputs_host, prog, rows, cols):

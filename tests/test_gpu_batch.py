@@ -430,3 +430,75 @@ def test_config5_block_at_full_size_in_every_mode(tmp_path):
     for mode in ("batch", "batch_fused", "graph", "graph_fused"):
         for k in kept["lines"]:
             assert np.array_equal(kept[mode][k], kept["lines"][k]), (mode, k)
+
+
+def test_random_batches_fused_equal_line_by_line(tmp_path):
+    """Random batches over a pool of [rows, cols], [rows, 1] and [1, cols] tensors in float32,
+    bfloat16 and float16: elementwise lines (in place or not), casts, squares, broadcastTo of the
+    vectors and sums over the last axis, in random order.  Whatever runs the planner forms — one
+    dtype, mixed, with row or column vectors, with a row sum inside, cut at a vector that would be
+    overwritten while other lanes still read it — every tensor must end up with the bits of the
+    line-by-line execution, and every line must get the reply it gets on its own."""
+    rng = np.random.default_rng(20251)
+    dts = ["float32", "bfloat16", "float16"]
+    code = {"float32": dx.F32, "bfloat16": dx.BF16, "float16": dx.F16}
+    fused_lines = 0
+    for trial in range(72):
+        rows, cols = [(16, 64), (5, 12), (64, 896), (3, 1000), (33, 260), (128, 32)][trial % 6]
+        shapes = {"F": [rows, cols], "C": [rows, 1], "R": [1, cols]}
+        pool = [(f"t{trial}_{k}{i}_{dt[:3]}{dt[-2:]}", k, dt) for k in shapes for i in range(3) for dt in dts]
+        data = {name: H.to_storage(rng.uniform(0.25, 2.0, int(np.prod(shapes[k]))), code[dt]).reshape(shapes[k]) if dt != "float32"
+                else rng.uniform(0.25, 2.0, shapes[k]).astype(np.float32) for name, k, dt in pool}
+        def pick(k, dt):
+            fits = [p for p in pool if p[1] == k and p[2] == dt]
+            return fits[int(rng.integers(0, len(fits)))]
+        lines = []
+        for _ in range(int(rng.integers(10, 22))):
+            kind = str(rng.choice(["bin", "bin", "scalar", "scalar", "sqrt", "todtype", "square", "broadcast", "sum"]))
+            k, dt = str(rng.choice(["F", "F", "F", "C", "R"])), str(rng.choice(dts))
+            a, b, c = pick(k, dt), pick(k, dt), pick(k, dt)
+            if kind == "bin":
+                lines.append(f"{rng.choice(['add', 'mul', 'sub', 'max', 'min', 'div'])}({T(a[0], dt)}, {T(b[0], dt)})->({T(c[0], dt)})")
+            elif kind == "scalar":
+                op = str(rng.choice(["addscalar", "mulscalar", "divscalar", "maxscalar", "rsubscalar", "rdivscalar"]))
+                s = float(rng.choice([0.5, 2.0, 1.25, 3.0]))
+                args = f"var<float32>:{s}, {T(a[0], dt)}" if op in ("rsubscalar", "rdivscalar") else f"{T(a[0], dt)}, var<float32>:{s}"
+                lines.append(f"{op}({args})->({T(c[0], dt)})")
+            elif kind == "sqrt":
+                lines.append(f"sqrt({T(a[0], dt)})->({T(c[0], dt)})")
+            elif kind == "todtype":
+                d2 = str(rng.choice(dts))
+                lines.append(f"todtype({T(a[0], dt)})->({T(pick(k, d2)[0], d2)})")
+            elif kind == "square":
+                a, c = pick(k, "float32"), pick(k, "float32")
+                lines.append(f"powscalar({T(a[0])}, var<float32>:2)->({T(c[0])})")
+            elif kind == "broadcast":
+                v = pick(str(rng.choice(["C", "R"])), dt)
+                lines.append(f"broadcastTo({T(v[0], dt)}, {V(shapes['F'])})->({T(pick('F', dt)[0], dt)})")
+            else:
+                dt = str(rng.choice(["float32", "float32", "bfloat16"]))
+                lines.append(f"sum({T(pick('F', dt)[0], dt)}, {V([-1])}, var<bool>:true)->({T(pick('C', dt)[0], dt)})")
+        text = [f"{line} // author=miaobyte id={900 + i}" for i, line in enumerate(lines)]
+        results, replies = {}, {}
+        for mode in ("lines", "fused"):
+            ex = InProc()
+            ex.set_fusion(mode == "fused")
+            h = Host(ex, tmp_path)
+            for name, k, dt in pool:
+                h.put(name, data[name], dt)
+            replies[mode] = [ex.execute(t) for t in text] if mode == "lines" else ex.execute_batch(text)
+            if mode == "fused":
+                fused_lines += ex.fusion_stats()["lines"]
+            results[mode] = {name: h.get(name) for name, _, _ in pool}
+            del ex
+        assert [r.split("//")[0] for r in replies["fused"]] == [r.split("//")[0] for r in replies["lines"]], (trial, lines)
+        for name, _, _ in pool:
+            a, b = results["lines"][name], results["fused"][name]
+            same = np.array_equal(a.view(np.uint8), b.view(np.uint8))
+            if not same and a.dtype.kind == "f":
+                same = np.array_equal(a, b, equal_nan=True)
+            if not same:  # 16-bit floats come back as raw bits: NaN payloads aside they must agree
+                fa, fb = H.to_float(a.reshape(-1), code[[p for p in pool if p[0] == name][0][2]]), H.to_float(b.reshape(-1), code[[p for p in pool if p[0] == name][0][2]])
+                same = np.array_equal(fa, fb, equal_nan=True)
+            assert same, (trial, name, lines)
+    assert fused_lines > 400  # the batches did form runs

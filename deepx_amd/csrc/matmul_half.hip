@@ -446,13 +446,14 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
             // Lower tiles of the same width, one wave per 64 columns (matmul_half_dma.hip only): when a
             // lower tile still fits the output into one round, every CU's K loop gets shorter
             // (2048x896x4864: 18.2 us with 160 rows, 19.8 with 192; 2048x4096x4096: 56.9 us with 128
-            // rows, 63.4 with 192, hipBLASLt 70.9).
+            // rows, 63.4 with 192, hipBLASLt 70.9).  Both run three LDS stages of K 64 (against five of
+            // K 32: 2048x4096x4096 58.4 -> 55.7 us, 3072^3 with 160 rows 51.6 -> 48.8 us).
             // And a tile half as wide for an N that 256 columns divide badly (8192x4864x896, where 256-wide
             // tiles compute 1024 columns: 58.5 us against 66.5 with 128 rows x 256).
             // All three are taken for a single round only: over several rounds the square tile's lower
             // traffic through L2 wins again (8192^3: 843 us with 256x128, 790 with 256x256).
             if (dma_ok) {
-                const double c11 = one_per_cu(160, 256, 1.0, 5.5), c12 = one_per_cu(128, 256, 0.89, 5.0), c13 = one_per_cu(256, 128, 0.76, 3.5) - (tiles(256, 128) <= cus / 2 ? ksteps * 0.09 : 0.0);  // 0.52 us per step up to half the CUs
+                const double c11 = one_per_cu(160, 256, 0.96, 5.5), c12 = one_per_cu(128, 256, 0.85, 5.0), c13 = one_per_cu(256, 128, 0.76, 3.5) - (tiles(256, 128) <= cus / 2 ? ksteps * 0.09 : 0.0);  // 0.52 us per step up to half the CUs
                 double best = choice == 1 ? c1 : choice == 2 ? c2 : choice == 4 ? c4 : c6;
                 if (c11 < best && tiles(160, 256) <= cus) { best = c11; choice = 11; }
                 if (c12 < best && tiles(128, 256) <= cus) { best = c12; choice = 12; }

@@ -253,7 +253,8 @@ static int launch_dma_tile(const void *a, const void *b, void *c, int64_t batch,
     return launch_status();
 }
 
-// shape: 0 = 256x256 in K steps of 32, 1 = 192x256 / 32, 2 = 128x64 / 64, 3 = 256x256 / 64.  The caller has
+// shape: 0 = 256x256 in K steps of 32, 1 = 192x256 / 32, 2 = 128x64 / 64, 3 = 256x256 / 64, 4 = 160x256 / 64 and
+// 5 = 128x256 / 64 with the waves side by side, 6 = 256x128 / 64.  The caller has
 // checked K % 64 == 0, N % 8 == 0, the alignment of a, b, c and that every byte offset inside a tile
 // fits 32 bits.
 template <typename T>
@@ -262,8 +263,8 @@ static int launch_dma_shape(int shape, const void *a, const void *b, void *c, in
     case 0: return launch_dma_tile<T, 256, 256, 32, 4>(a, b, c, batch, m, k, n, st);
     case 1: return launch_dma_tile<T, 192, 256, 32, 5>(a, b, c, batch, m, k, n, st);
     case 3: return launch_dma_tile<T, 256, 256, 64, 2>(a, b, c, batch, m, k, n, st);
-    case 4: return launch_dma_tile<T, 160, 256, 32, 5, 4>(a, b, c, batch, m, k, n, st);
-    case 5: return launch_dma_tile<T, 128, 256, 32, 5, 4>(a, b, c, batch, m, k, n, st);
+    case 4: return launch_dma_tile<T, 160, 256, 64, 3, 4>(a, b, c, batch, m, k, n, st);
+    case 5: return launch_dma_tile<T, 128, 256, 64, 3, 4>(a, b, c, batch, m, k, n, st);
     case 6: return launch_dma_tile<T, 256, 128, 64, 3>(a, b, c, batch, m, k, n, st);
     default: return launch_dma_tile<T, 128, 64, 64, 5>(a, b, c, batch, m, k, n, st);
     }

@@ -95,8 +95,8 @@ enum dxh_tune_knob {
     DXH_TUNE_MATMUL_TILE = 4,          /* matmul workgroup tile, 0 = chosen per shape; bf16/f16: 1 128x128, 2 128x64, 3 64x128,
                                           4 256x256, 5 64x64, 6 192x256; 7 / 8 / 9 / 10 = 256x256 / 192x256 / 128x64 / 256x256 with
                                           operands loaded straight into LDS in K steps of 32 / 32 / 64 / 64 (K a multiple of 64,
-                                          else the register-staged twin 4 / 6 / 2 / 4 runs); 11 / 12 = 160x256 / 128x256 of
-                                          the same kind, one wave per 64 columns (twin 6), 13 = 256x128 in K steps of 64 (twin 4);
+                                          else the register-staged twin 4 / 6 / 2 / 4 runs); 11 / 12 / 13 = 160x256 / 128x256 /
+                                          256x128 of the same kind in K steps of 64, the first two with one wave per 64 columns (twins 6 / 6 / 4);
                                           f32: 1 128x128, 2 128x64, 3 64x64, 4 128x128 with K step 16 */
     DXH_TUNE_MATMUL_SPLITK = 6,        /* slices along K of a float matmul: 0 = chosen per shape (few output tiles and a long
                                           K are cut so that every CU has work), 1 = never, n <= 1024 = n slices.  Slices are

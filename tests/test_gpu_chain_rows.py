@@ -108,7 +108,7 @@ def test_rmsnorm_lines_as_runs(dxh, orc, half):
     the result.  Every tensor a line writes, bit for bit what the separate entry points store, and
     each of those against the oracle."""
     rng = np.random.default_rng(1200 + half)
-    for rows, cols in [(2048, 896), (5, 12), (2, 4), (257, 1000), (64, 4096)]:
+    for rows, cols in [(2048, 896), (5, 12), (2, 4), (257, 1000), (64, 4096), (2100, 500), (4099, 260)]:
         x = Dev(H.rand(rng, half, rows * cols, -2.0, 2.0))
         w = Dev(H.rand(rng, half, cols, 0.5, 1.5))
         var = Dev(H.rand(rng, dx.F32, rows, 0.05, 3.0))  # stands for 1/sqrt(mean + eps) of each row
@@ -150,7 +150,7 @@ def test_whole_rmsnorm_as_one_run(dxh, orc, half):
     one to four vector groups per lane, row counts that leave the last workgroup ragged, the
     config-5 size; and shapes whose rows dxh_sum would not give to one lane group are refused."""
     rng = np.random.default_rng(1300 + half)
-    for rows, cols in [(2048, 896), (5, 12), (2, 4), (257, 1000), (64, 1024), (1000, 256), (33, 64), (7, 520)]:
+    for rows, cols in [(2048, 896), (5, 12), (2, 4), (257, 1000), (64, 1024), (1000, 256), (33, 64), (7, 520), (2100, 500), (4099, 260), (1029, 1024)]:
         assert dxh.dxh_chain_rows_can_sum(rows, cols) == 1, (rows, cols)
         x = Dev(H.rand(rng, half, rows * cols, -2.0, 2.0))
         w = Dev(H.rand(rng, half, cols, 0.5, 1.5))
@@ -232,7 +232,7 @@ def test_random_mixed_runs_match_the_model(dxh):
     dtypes = [dx.F32, dx.BF16, dx.F16]
     names = BINARY + SCALAR + ["sqrt", "square", "copy"]
     for trial in range(40):
-        rows, cols = [(1, 4), (3, 8), (7, 36), (64, 256), (33, 1000), (300, 132)][trial % 6]
+        rows, cols = [(1, 4), (3, 8), (7, 36), (64, 256), (33, 1000), (300, 132), (2051, 516)][trial % 7]
         n_in = int(rng.integers(1, 9))
         inputs, host = [], []
         for j in range(n_in):

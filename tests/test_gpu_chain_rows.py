@@ -261,6 +261,33 @@ def test_random_mixed_runs_match_the_model(dxh):
             assert np.array_equal(g, w, equal_nan=True), (trial, rows, cols, k, prog)
 
 
+def test_long_run_with_many_live_results(dxh):
+    """Sixteen ops over eight inputs in which every result is read again three ops later, so that
+    nine results are alive beside the inputs: more LDS per workgroup than a launch gets unasked
+    (17 slots of 4 KiB), which makes the entry point raise the kernel's limit first.  Against the
+    numpy model, and twice in a row (the second launch finds the limit raised)."""
+    rng = np.random.default_rng(31)
+    rows, cols = 96, 200
+    inputs, host = [], []
+    for j in range(8):
+        dt = [dx.F32, dx.BF16, dx.F16][j % 3]
+        data = H.rand(rng, dt, rows * cols, 0.5, 1.5)
+        inputs.append((Dev(data), dt, FULL))
+        host.append(H.to_float(data, dt).astype(np.float32).reshape(rows, cols))
+    prog = []
+    for k in range(16):
+        name = ["add", "mul", "max", "sub"][k % 4]
+        lhs = k % 8 if k < 3 else R + (k - 3)   # a result from three ops back: not the one in registers
+        prog.append((name, lhs, (k + 3) % 8, 0.0, [dx.F32, dx.F32, dx.BF16][k % 3], FULL))
+    want = model(host, prog, rows, cols)
+    for attempt in range(2):
+        rc, got = run_rows(dxh, inputs, prog, rows, cols)
+        dx.check(rc, "chain_rows")
+        for k, (_, _, _, _, dt, _) in enumerate(prog):
+            g = H.to_float(got[k].get(), dt).astype(np.float32)
+            assert np.array_equal(g, want[k].reshape(-1), equal_nan=True), (attempt, k)
+
+
 def test_in_place_and_refusals(dxh):
     """A [rows, cols] output may be one of the inputs (a lane reads its own elements before it writes
     them); a vector input may not (DXH_ERR_ARG), nor may an op on vectors read a [rows, cols] tensor."""

@@ -321,10 +321,11 @@ template <typename Op, bool HALF> int unary_float(int dtype, const void *a, void
 // time (no barriers: no lane reads another lane's slots).  The launch asks for as many slots as
 // the run needs (4 KiB each), so short runs keep the CU full of waves.
 constexpr int kChainOps = DXH_CHAIN_MAX_OPS, kChainInputs = DXH_CHAIN_MAX_INPUTS;
-struct ChainArgs {
+struct ChainArgs {  // first kernel argument: sits at offset 0 of the kernel-argument segment
     const void *in[kChainInputs];
     void *out[kChainOps];
     double scalar[kChainOps];  // already rounded to T on the host
+    uint32_t op[kChainOps];    // code | lhs << 8 | rhs << 16 | save << 24, the last three as int8 (filled by the launcher from the arrays below)
     int8_t code[kChainOps], lhs[kChainOps], rhs[kChainOps];  // operand: LDS slot, or kChainPrev = result of the op before
     int8_t save[kChainOps];                                  // LDS slot that keeps the result for later ops, or -1
     int n_in, n_ops;                                         // inputs occupy slots 0 .. n_in - 1
@@ -337,20 +338,11 @@ __global__ __launch_bounds__(kBlock) void chain_kernel(const ChainArgs p, int64_
     using A = acc_t<T>;
     extern __shared__ __attribute__((aligned(16))) unsigned char chain_lds[];
     const int t = threadIdx.x;
-    // The op table is indexed by a loop counter.  Out of the kernel argument that would make the
-    // compiler copy the whole table into per-lane scratch memory; out of LDS (filled once, with
-    // constant indices) it is a broadcast read.
-    __shared__ int s_code[kChainOps], s_lhs[kChainOps], s_rhs[kChainOps], s_save[kChainOps];
-    __shared__ double s_scalar[kChainOps];
-    __shared__ void *s_out[kChainOps];
-    if (t == 0) {
-#pragma unroll
-        for (int k = 0; k < kChainOps; ++k) {
-            s_code[k] = p.code[k]; s_lhs[k] = p.lhs[k]; s_rhs[k] = p.rhs[k]; s_save[k] = p.save[k];
-            s_scalar[k] = p.scalar[k]; s_out[k] = p.out[k];
-        }
-    }
-    __syncthreads();
+    // The op table is indexed by a loop counter.  Out of the by-value kernel argument that would make
+    // the compiler copy the whole table into per-lane scratch memory; read from the kernel-argument
+    // segment itself it is a scalar load per op, with no set-up phase.
+    typedef const ChainArgs __attribute__((address_space(4))) *ArgTable;
+    const ArgTable tab = (ArgTable)__builtin_amdgcn_kernarg_segment_ptr();
     // registers and LDS hold raw 16-byte vectors (a select between two of them stays in registers)
     u32x4_t *raw = reinterpret_cast<u32x4_t *>(chain_lds);
     for (int64_t i = (int64_t)blockIdx.x * kBlock + t; i < nv; i += (int64_t)gridDim.x * kBlock) {
@@ -363,13 +355,14 @@ __global__ __launch_bounds__(kBlock) void chain_kernel(const ChainArgs p, int64_
 #undef DXH_CH_KEEP
         u32x4_t prev = x0;
         for (int k = 0; k < p.n_ops; ++k) {
-            const int code = __builtin_amdgcn_readfirstlane(s_code[k]), l = __builtin_amdgcn_readfirstlane(s_lhs[k]);
-            const int q = __builtin_amdgcn_readfirstlane(s_rhs[k]), save = __builtin_amdgcn_readfirstlane(s_save[k]);
+            const uint32_t d = tab->op[k];
+            const int code = (int)(d & 0xff), l = (int)(int8_t)(d >> 8), q = (int)(int8_t)(d >> 16), save = (int)(int8_t)(d >> 24);
+            void *out = tab->out[k];
             u32x4_t ra = prev, rb = prev;
             if (l != kChainPrev) ra = raw[l * kBlock + t];
             if (q != kChainPrev) rb = raw[q * kBlock + t];
             const VT a = __builtin_bit_cast(VT, ra), b = __builtin_bit_cast(VT, rb);
-            const A s = A(s_scalar[k]);
+            const A s = A(tab->scalar[k]);
             VT r;
             A y[V];
 #define DXH_CH_BIN(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) y[v] = Op::f(A(load_acc(a.v[v])), A(load_acc(b.v[v]))); break
@@ -400,7 +393,7 @@ __global__ __launch_bounds__(kBlock) void chain_kernel(const ChainArgs p, int64_
             store_acc_vec<T, V>(r, y);
             prev = __builtin_bit_cast(u32x4_t, r);
             if (save >= 0) raw[save * kBlock + t] = prev;
-            if (s_out[k]) __builtin_nontemporal_store(prev, &reinterpret_cast<u32x4_t *>(s_out[k])[i]);
+            if (out) __builtin_nontemporal_store(prev, &reinterpret_cast<u32x4_t *>(out)[i]);
         }
     }
 }
@@ -409,7 +402,10 @@ template <typename T>
 int launch_chain(ChainArgs &p, const dxh_chain_op *ops, int64_t n, hipStream_t st) {
     constexpr int V = vec_len<T>;
     if (n % V != 0) return DXH_ERR_ALIGN;
-    for (int k = 0; k < p.n_ops; ++k) p.scalar[k] = (double)load_acc(scalar_to<T>(ops[k].scalar));
+    for (int k = 0; k < p.n_ops; ++k) {
+        p.scalar[k] = (double)load_acc(scalar_to<T>(ops[k].scalar));
+        p.op[k] = (uint32_t)(uint8_t)p.code[k] | (uint32_t)(uint8_t)p.lhs[k] << 8 | (uint32_t)(uint8_t)p.rhs[k] << 16 | (uint32_t)(uint8_t)p.save[k] << 24;
+    }
     const int64_t nv = n / V, blocks = (nv + kBlock - 1) / kBlock;
     int slots = p.n_in;
     for (int k = 0; k < p.n_ops; ++k) slots = std::max(slots, p.save[k] + 1);

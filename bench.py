@@ -437,6 +437,36 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
         "broadcastTo_f32_2048x1_to_2048x896": (lambda i: L.dxh_broadcastTo(dx.F32, ptr(col[i % R6]), shc, 2, shb, 2, ptr(o32[i % R6]), None), n32 * 4 + S * 4),
     }
     c5["glue_ops(cache-resident sizes)"] = {k: entry(time_op(L, dx, torch, Events, ev, fn), nb) for k, (fn, nb) in glue.items()}
+    # the same glue as the executor's batch path launches it: the RMSNorm's thirteen lines (row sum included) and the
+    # SiLU gate's six lines, one launch each (dxh_chain_rows / dxh_chain); bytes = inputs once + every tensor the lines store
+    FULL, ROW, COL, RES = dx.CHAIN_FULL, dx.CHAIN_ROW, dx.CHAIN_COLUMN, dx.CHAIN_RESULT
+    w16 = torch.ones(Hd, device=dev, dtype=torch.bfloat16)
+    f32s = [[torch.empty(S * Hd, device=dev) for _ in range(5)] for _ in range(R6)]  # xf sq rs wf xn
+    wf1 = torch.empty(Hd, device=dev)
+    h16 = [torch.empty(S * Hd, device=dev, dtype=torch.bfloat16) for _ in range(R6)]
+    code = dx.CHAIN_CODES.index
+    def norm_run(i):
+        xf, sq, rs, wf, xn = f32s[i]
+        prog = [("copy", 0, 0, 0, dx.F32, FULL, xf), ("square", RES + 0, 0, 2.0, dx.F32, FULL, sq), ("rowsum", RES + 1, 0, 0, dx.F32, COL, None),
+                ("divscalar", RES + 2, 0, float(Hd), dx.F32, COL, None), ("addscalar", RES + 3, 0, 1e-6, dx.F32, COL, None),
+                ("sqrt", RES + 4, 0, 0, dx.F32, COL, None), ("rdivscalar", RES + 5, 0, 1.0, dx.F32, COL, col[i]),
+                ("copy", RES + 6, 0, 0, dx.F32, FULL, rs), ("mul", RES + 0, RES + 7, 0, dx.F32, FULL, None), ("copy", 1, 0, 0, dx.F32, ROW, wf1),
+                ("copy", RES + 9, 0, 0, dx.F32, FULL, wf), ("mul", RES + 10, RES + 8, 0, dx.F32, FULL, xn), ("copy", RES + 11, 0, 0, dx.BF16, FULL, h16[i])]
+        tin = (dx.ChainTensor * 2)(dx.ChainTensor(x16[i].data_ptr(), dx.BF16, FULL), dx.ChainTensor(w16.data_ptr(), dx.BF16, ROW))
+        ops = (dx.ChainRowsOp * len(prog))(*[dx.ChainRowsOp(code(n), l, r, dx.scalar(sc), o.data_ptr() if o is not None else None, dt, e)
+                                             for n, l, r, sc, dt, e, o in prog])
+        return lambda: L.dxh_chain_rows(tin, 2, ops, len(prog), S, Hd, None)
+    def gate_run(i):
+        prog = [("mulscalar", 0, 0, -1.0), ("exp", RES + 0, 0, 0), ("addscalar", RES + 1, 0, 1.0), ("rdivscalar", RES + 2, 0, 1.0), ("mul", 0, RES + 3, 0), ("mul", RES + 4, 1, 0)]
+        ops = (dx.ChainOp * len(prog))(*[dx.ChainOp(code(n), l, r, dx.scalar(sc), o16[i].data_ptr() if k == len(prog) - 1 else None) for k, (n, l, r, sc) in enumerate(prog)])
+        ins = (C.c_void_p * 2)(g16[i].data_ptr(), u16[i].data_ptr())
+        return lambda: L.dxh_chain(dx.BF16, ins, 2, ops, len(prog), n16, None)
+    norm_calls, gate_calls = [norm_run(i) for i in range(R6)], [gate_run(i) for i in range(R6)]
+    c5["fused_runs(one launch each)"] = {
+        "rmsnorm_13_lines_bf16_in_f32_inside_2048x896": entry(time_op(L, dx, torch, Events, ev, lambda i: norm_calls[i % R6]()), n32 * 2 + 5 * n32 * 4 + n32 * 2 + S * 4 + Hd * 6),
+        "silu_gate_6_lines_bf16_2048x4864": entry(time_op(L, dx, torch, Events, ev, lambda i: gate_calls[i % R6]()), 3 * n16 * 2),
+        "note": "bound by instruction issue (an op interpreter; correctly rounded exp and division, one rounding per op), not by these bytes; "
+                "as separate launches the same lines take the sum of the glue_ops entries above, 10 and 6 launches"}
     del g16, u16, o16, x16, x32, o32, col
     torch.cuda.empty_cache()
     c5["mlp_block_over_deepxIR"] = config5_block_over_ir()

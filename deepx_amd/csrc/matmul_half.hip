@@ -410,11 +410,19 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
                       k <= (1 << 22) && n <= (1 << 24);
     int64_t choice = tuning().matmul_tile;
     if (ldc >= 0 && (!fast || k % PK != 0)) return DXH_ERR_ALIGN;  // launch_padded hands over aligned copies only
+    const bool dma_ok = fast && ldc < 0 && k % 64 == 0;
+    // A long K over few output tiles: 128x128 tiles whose K is cut in two inside one launch (the halves
+    // meet in the caller's scratch; matmul_half_dma.hip).  Measured against what would run otherwise on
+    // 17 such shapes: 0.57-0.93 of its time from K = 4096 up and 48 to 128 tiles (2048x4864x896: 25.8 ->
+    // 23.7 us, 1536x8192x768: 48 -> 27 us), slower with K = 2048 or under 20 tiles.
+    if (dma_ok && choice == 0 && tuning().matmul_splitk != 1 && m > 128 && k >= 4096) {
+        const int64_t t14 = batch * ((m + 127) / 128) * ((n + 127) / 128);
+        if (t14 >= 40 && 2 * t14 <= compute_units()) choice = 14;
+    }
     if (fast && ldc < 0 && (choice == 0 || choice == 5)) {
         const int rc = launch_split<T>(a, b, c, batch, m, k, n, st, sc);
         if (rc != kNoSplit) return rc;
     }
-    const bool dma_ok = fast && ldc < 0 && k % 64 == 0;
     if (fast && choice == 0) {
         // 256x256 tiles halve the bytes every CU pulls through its vector cache per flop, but need
         // about one tile per CU to pay off.  Below that, 128x128 tiles (two workgroups per CU) as
@@ -468,6 +476,17 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
     // runs two LDS stages of K 64 when K is long (whole cache lines of A, half the barriers) and four
     // of K 32 when it is short (2048x896x4864: 21.2 against 22.6 us with the shallow pipeline).
     if (dma_ok && tuning().matmul_tile == 0 && (choice == 4 || choice == 6)) choice = choice == 6 ? 8 : k >= 2048 ? 10 : 7;
+    if (dma_ok && choice == 14) {
+        const int64_t t14 = batch * ((m + 127) / 128) * ((n + 127) / 128);
+        if (t14 <= 1024 && k >= 64 * 2) {
+            float *part = (float *)sc.take((size_t)dma_split_bytes(t14));
+            if (!part) return DXH_ERR_WORKSPACE;
+            if (sc.planning) return DXH_OK;
+            if (unsigned *cnt = finish_counters(st, t14))
+                return launch_matmul_half_dma_split(std::is_same_v<T, bf16_t> ? DXH_BF16 : DXH_F16, a, b, c, batch, m, k, n, part, cnt, st);
+        }
+        choice = 1;  // no counters to be had (or too many tiles): the same tile, uncut
+    }
     if (dma_ok && choice >= 7 && choice <= 13) {
         if (sc.planning) return DXH_OK;
         return launch_matmul_half_dma(std::is_same_v<T, bf16_t> ? DXH_BF16 : DXH_F16, (int)choice - 7, a, b, c, batch, m, k, n, st);
@@ -480,7 +499,7 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
         case 5: return launch_tile<T, 64, 64, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 6: case 8: case 11: case 12: return launch_tile<T, 192, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 7: case 10: case 13: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
-        default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
+        case 14: default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         }
     }
     if (!fast && tuning().matmul_tile == 0 && k <= (1 << 22) && n <= (1 << 24)) {

@@ -35,9 +35,16 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t off, uint32_t l
 }
 template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N)); }
 
-template <typename T, int TM, int TN, int DK, int NS, int WN = 2>
+// NSPLIT = 2: the tile map holds two entries per output tile, each the same tile over one half of
+// K.  A half stores its fp32 accumulators to `part` (its own 4 * TM * TN bytes, element e of lane t
+// at [e * 256 + t]) and counts itself in `cnt[tile]`; the half that finds it is the second adds the
+// other's partial tile to its own accumulators (a + b == b + a in fp32: the sum does not depend on
+// which half came last), puts the counter back to zero and stores C.  The partials travel with
+// device-scope stores and loads and the count follows a wait for the stores' acknowledgement, as in
+// reduce_col_fused_kernel (reduce.hip).
+template <typename T, int TM, int TN, int DK, int NS, int WN = 2, int NSPLIT = 0>
 __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int K, int N,
-                                                                TileMap map) {
+                                                                TileMap map, float *part, unsigned *cnt) {
     // the four waves form a WM x WN grid over the tile: 2 x 2, or 1 x 4 for a tile height that is
     // a multiple of 32 but not of 64
     constexpr int WM = 4 / WN, WTM = TM / WM, WTN = TN / WN;
@@ -61,8 +68,17 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
     if (!tc.valid) return;
     const int m0 = tc.tm * TM, n0 = tc.tn * TN;
     const int t = threadIdx.x, lane = t & 63, w = __builtin_amdgcn_readfirstlane(t >> 6), wm = w / WN, wn = w % WN;
-    const uint16_t *Ab = reinterpret_cast<const uint16_t *>(A) + ((int64_t)tc.batch * M + m0) * K;
-    const uint16_t *Bb = reinterpret_cast<const uint16_t *>(B) + (int64_t)tc.batch * K * N + n0;
+    int zb = tc.batch, slice = 0, kbeg = 0, KT = K / DK;
+    if constexpr (NSPLIT > 0) {
+        static_assert(NSPLIT == 0 || NSPLIT == 2, "two halves: their sum is the same in either order");
+        zb = tc.batch / NSPLIT;
+        slice = tc.batch - zb * NSPLIT;
+        const int base = KT / NSPLIT, rem = KT - base * NSPLIT;  // K steps dealt out evenly; the launcher makes sure that base >= 1
+        kbeg = slice * base + (slice < rem ? slice : rem);
+        KT = base + (slice < rem ? 1 : 0);
+    }
+    const uint16_t *Ab = reinterpret_cast<const uint16_t *>(A) + ((int64_t)zb * M + m0) * K + (int64_t)kbeg * DK;
+    const uint16_t *Bb = reinterpret_cast<const uint16_t *>(B) + ((int64_t)zb * K + (int64_t)kbeg * DK) * N + n0;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
 
     // ---- which 16 bytes each lane fetches (byte offsets from the tile's A / B origin at k = 0) ----
@@ -144,7 +160,6 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
         });
     };
 
-    const int KT = K / DK;
     auto k_of = [&](int s) __attribute__((always_inline)) { return s < KT ? s : KT - 1; };
     // steps past the end fetch the last step again: the count of loads in flight stays the same
     // on every trip, and the copies land in stages that nobody reads any more
@@ -219,6 +234,43 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
     wait_loads<0>();  // the refetched tail steps must have landed before the C tile reuses the LDS
     __syncthreads();
 
+    if constexpr (NSPLIT > 0) {
+        __shared__ int is_last;
+        constexpr int E = NM * 16;  // accumulators per lane
+        const int tile = (zb * map.tiles_m + tc.tm) * map.tiles_n + tc.tn;
+        float *P = part + (int64_t)tile * NSPLIT * E * kBlock + t;
+        float *mine = P + (int64_t)slice * E * kBlock;
+        const float *other = P + (int64_t)(1 - slice) * E * kBlock;
+        static_for<NM>([&](auto x) __attribute__((always_inline)) {
+            constexpr int i = decltype(x)::value / FN, j = decltype(x)::value % FN;
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                __hip_atomic_store(mine + (decltype(x)::value * 16 + v) * kBlock, acc[i][j][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        });
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores are in memory before the barrier, hence before the count
+        __syncthreads();
+        if (t == 0) {
+            const unsigned old = __hip_atomic_fetch_add(cnt + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int last = old == (unsigned)(NSPLIT - 1);
+            if (last) __hip_atomic_store(cnt + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = last;
+        }
+        __syncthreads();
+        if (!is_last) return;
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);  // the loads below stay below the count
+        float got[NM][16];  // every load is issued before the first is used: one memory round trip, not NM
+        static_for<NM>([&](auto x) __attribute__((always_inline)) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                got[decltype(x)::value][v] = __hip_atomic_load(other + (decltype(x)::value * 16 + v) * kBlock, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        });
+        static_for<NM>([&](auto x) __attribute__((always_inline)) {
+            constexpr int i = decltype(x)::value / FN, j = decltype(x)::value % FN;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] += got[decltype(x)::value][v];
+        });
+    }
+
     // ---- epilogue: result lane holds row m = lane%32 of its MFMA tile and, per group g of 4
     // registers, columns 8g + 4*(lane/32) .. +3: one 8-byte LDS store each, then 16-byte row stores
     uint16_t *Cs = reinterpret_cast<uint16_t *>(lds);
@@ -234,7 +286,7 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
         });
     });
     __syncthreads();
-    uint16_t *Cr = reinterpret_cast<uint16_t *>(C) + (int64_t)tc.batch * M * N;
+    uint16_t *Cr = reinterpret_cast<uint16_t *>(C) + (int64_t)zb * M * N;
     constexpr int CB = TN / 8;
 #pragma unroll
     for (int i = 0; i < TM * CB / kBlock; ++i) {
@@ -249,7 +301,17 @@ template <typename T, int TM, int TN, int DK, int NS, int WN = 2>
 static int launch_dma_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     TileMap map;
     if (!make_tile_map(batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
-    matmul_dma_kernel<T, TM, TN, DK, NS, WN><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map);
+    matmul_dma_kernel<T, TM, TN, DK, NS, WN><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, nullptr, nullptr);
+    return launch_status();
+}
+
+// 128x128 tiles, each cut into two halves of K that meet in `part` (dma_split_bytes) and `cnt` (one
+// zeroed counter per output tile, left zero).
+template <typename T>
+static int launch_dma_split(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, float *part, unsigned *cnt, hipStream_t st) {
+    TileMap map;
+    if (!make_tile_map(batch * 2, m, n, 128, 128, map)) return DXH_ERR_SHAPE;
+    matmul_dma_kernel<T, 128, 128, 64, 3, 2, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, part, cnt);
     return launch_status();
 }
 
@@ -268,6 +330,9 @@ static int launch_dma_shape(int shape, const void *a, const void *b, void *c, in
     case 6: return launch_dma_tile<T, 256, 128, 64, 3>(a, b, c, batch, m, k, n, st);
     default: return launch_dma_tile<T, 128, 64, 64, 5>(a, b, c, batch, m, k, n, st);
     }
+}
+int launch_matmul_half_dma_split(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, float *part, unsigned *cnt, hipStream_t st) {
+    return dtype == DXH_BF16 ? launch_dma_split<bf16_t>(a, b, c, batch, m, k, n, part, cnt, st) : launch_dma_split<f16_t>(a, b, c, batch, m, k, n, part, cnt, st);
 }
 int launch_matmul_half_dma(int dtype, int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     return dtype == DXH_BF16 ? launch_dma_shape<bf16_t>(shape, a, b, c, batch, m, k, n, st) : launch_dma_shape<f16_t>(shape, a, b, c, batch, m, k, n, st);

@@ -284,10 +284,10 @@ constexpr int kNoSkinny = -1002;  // not a DXH_ERR_* value
 int launch_matmul_skinny(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc);
 int launch_matmul_half(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc);
 int launch_matmul_half_dma(int dtype, int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
-// 128x128 tiles cut into two halves of K that are summed inside the launch: `part` holds
+// 128x128 (wide: 128x256) tiles cut into two halves of K that are summed inside the launch: `part` holds
 // dma_split_bytes(tiles), `cnt` one zeroed counter per output tile (finish_counters, reduce.hip)
-inline int64_t dma_split_bytes(int64_t tiles) { return tiles * 2 * 128 * 128 * (int64_t)sizeof(float); }
-int launch_matmul_half_dma_split(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, float *part, unsigned *cnt, hipStream_t st);
+inline int64_t dma_split_bytes(int64_t tiles, int wide) { return tiles * 2 * 128 * (wide ? 256 : 128) * (int64_t)sizeof(float); }
+int launch_matmul_half_dma_split(int dtype, int wide, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, float *part, unsigned *cnt, hipStream_t st);
 unsigned *finish_counters(hipStream_t st, int64_t need);
 int launch_matmul_f32(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc);
 int launch_matmul_f64(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc);

@@ -416,8 +416,12 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
     // 17 such shapes: 0.57-0.93 of its time from K = 4096 up and 48 to 128 tiles (2048x4864x896: 25.8 ->
     // 23.7 us, 1536x8192x768: 48 -> 27 us), slower with K = 2048 or under 20 tiles.
     if (dma_ok && choice == 0 && tuning().matmul_splitk != 1 && m > 128 && k >= 4096) {
-        const int64_t t14 = batch * ((m + 127) / 128) * ((n + 127) / 128);
+        const int64_t t14 = batch * ((m + 127) / 128) * ((n + 127) / 128), t15 = batch * ((m + 127) / 128) * ((n + 255) / 256);
         if (t14 >= 40 && 2 * t14 <= compute_units()) choice = 14;
+        // the same with 128x256 tiles (four waves side by side) for outputs twice that size: 0.87-0.94 of
+        // the uncut time from K = 6144 up, or from K = 4096 with under 100 tiles (1024x4096x3072: 36.9 ->
+        // 32.2 us; 2048x8192x2048: 70.5 -> 65.6 us, hipBLASLt 85; 2048x4096x2048 with 128 tiles loses)
+        else if (t15 >= 40 && 2 * t15 <= compute_units() && (k >= 6144 || t15 <= 100)) choice = 15;
     }
     if (fast && ldc < 0 && (choice == 0 || choice == 5)) {
         const int rc = launch_split<T>(a, b, c, batch, m, k, n, st, sc);
@@ -476,16 +480,17 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
     // runs two LDS stages of K 64 when K is long (whole cache lines of A, half the barriers) and four
     // of K 32 when it is short (2048x896x4864: 21.2 against 22.6 us with the shallow pipeline).
     if (dma_ok && tuning().matmul_tile == 0 && (choice == 4 || choice == 6)) choice = choice == 6 ? 8 : k >= 2048 ? 10 : 7;
-    if (dma_ok && choice == 14) {
-        const int64_t t14 = batch * ((m + 127) / 128) * ((n + 127) / 128);
+    if (dma_ok && (choice == 14 || choice == 15)) {
+        const int wide = choice == 15;
+        const int64_t t14 = batch * ((m + 127) / 128) * ((n + (wide ? 255 : 127)) / (wide ? 256 : 128));
         if (t14 <= 1024 && k >= 64 * 2) {
-            float *part = (float *)sc.take((size_t)dma_split_bytes(t14));
+            float *part = (float *)sc.take((size_t)dma_split_bytes(t14, wide));
             if (!part) return DXH_ERR_WORKSPACE;
             if (sc.planning) return DXH_OK;
             if (unsigned *cnt = finish_counters(st, t14))
-                return launch_matmul_half_dma_split(std::is_same_v<T, bf16_t> ? DXH_BF16 : DXH_F16, a, b, c, batch, m, k, n, part, cnt, st);
+                return launch_matmul_half_dma_split(std::is_same_v<T, bf16_t> ? DXH_BF16 : DXH_F16, wide, a, b, c, batch, m, k, n, part, cnt, st);
         }
-        choice = 1;  // no counters to be had (or too many tiles): the same tile, uncut
+        choice = wide ? 12 : 1;  // no counters to be had (or too many tiles): the same tile, uncut
     }
     if (dma_ok && choice >= 7 && choice <= 13) {
         if (sc.planning) return DXH_OK;
@@ -499,7 +504,7 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
         case 5: return launch_tile<T, 64, 64, 2>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 6: case 8: case 11: case 12: return launch_tile<T, 192, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         case 7: case 10: case 13: return launch_tile<T, 256, 256, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
-        case 14: default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
+        case 14: case 15: default: return launch_tile<T, 128, 128, 1>(a, b, c, batch, m, k, n, ldc, st, sc);
         }
     }
     if (!fast && tuning().matmul_tile == 0 && k <= (1 << 22) && n <= (1 << 24)) {

@@ -305,13 +305,14 @@ static int launch_dma_tile(const void *a, const void *b, void *c, int64_t batch,
     return launch_status();
 }
 
-// 128x128 tiles, each cut into two halves of K that meet in `part` (dma_split_bytes) and `cnt` (one
+// 128x128 (wide: 128x256) tiles, each cut into two halves of K that meet in `part` (dma_split_bytes) and `cnt` (one
 // zeroed counter per output tile, left zero).
 template <typename T>
-static int launch_dma_split(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, float *part, unsigned *cnt, hipStream_t st) {
+static int launch_dma_split(int wide, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, float *part, unsigned *cnt, hipStream_t st) {
     TileMap map;
-    if (!make_tile_map(batch * 2, m, n, 128, 128, map)) return DXH_ERR_SHAPE;
-    matmul_dma_kernel<T, 128, 128, 64, 3, 2, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, part, cnt);
+    if (!make_tile_map(batch * 2, m, n, 128, wide ? 256 : 128, map)) return DXH_ERR_SHAPE;
+    if (wide) matmul_dma_kernel<T, 128, 256, 64, 3, 4, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, part, cnt);
+    else matmul_dma_kernel<T, 128, 128, 64, 3, 2, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, part, cnt);
     return launch_status();
 }
 
@@ -331,8 +332,8 @@ static int launch_dma_shape(int shape, const void *a, const void *b, void *c, in
     default: return launch_dma_tile<T, 128, 64, 64, 5>(a, b, c, batch, m, k, n, st);
     }
 }
-int launch_matmul_half_dma_split(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, float *part, unsigned *cnt, hipStream_t st) {
-    return dtype == DXH_BF16 ? launch_dma_split<bf16_t>(a, b, c, batch, m, k, n, part, cnt, st) : launch_dma_split<f16_t>(a, b, c, batch, m, k, n, part, cnt, st);
+int launch_matmul_half_dma_split(int dtype, int wide, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, float *part, unsigned *cnt, hipStream_t st) {
+    return dtype == DXH_BF16 ? launch_dma_split<bf16_t>(wide, a, b, c, batch, m, k, n, part, cnt, st) : launch_dma_split<f16_t>(wide, a, b, c, batch, m, k, n, part, cnt, st);
 }
 int launch_matmul_half_dma(int dtype, int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
     return dtype == DXH_BF16 ? launch_dma_shape<bf16_t>(shape, a, b, c, batch, m, k, n, st) : launch_dma_shape<f16_t>(shape, a, b, c, batch, m, k, n, st);

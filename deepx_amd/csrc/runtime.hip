@@ -29,7 +29,7 @@ int dxh_tune(int knob, int64_t value) {
         t.reduce_col_max_lanes = value;
         return DXH_OK;
     case DXH_TUNE_REDUCE_ROW_LOADS: if (value < 1 || value > 64) return DXH_ERR_ARG; t.reduce_row_loads = value; return DXH_OK;
-    case DXH_TUNE_MATMUL_TILE: if (value < 0 || value > 14) return DXH_ERR_ARG; t.matmul_tile = value; return DXH_OK;
+    case DXH_TUNE_MATMUL_TILE: if (value < 0 || value > 15) return DXH_ERR_ARG; t.matmul_tile = value; return DXH_OK;
     case DXH_TUNE_MATMUL_SPLITK: if (value < 0 || value > 1024) return DXH_ERR_ARG; t.matmul_splitk = value; return DXH_OK;
     case DXH_TUNE_NT_LOAD: if (value < 0 || value > 2) return DXH_ERR_ARG; t.nt_load = value; return DXH_OK;
     case DXH_TUNE_SKINNY_PER_CU: if (value < 1 || value > 64) return DXH_ERR_ARG; t.skinny_per_cu = value; return DXH_OK;

@@ -97,8 +97,8 @@ enum dxh_tune_knob {
                                           operands loaded straight into LDS in K steps of 32 / 32 / 64 / 64 (K a multiple of 64,
                                           else the register-staged twin 4 / 6 / 2 / 4 runs); 11 / 12 / 13 = 160x256 / 128x256 /
                                           256x128 of the same kind in K steps of 64, the first two with one wave per 64 columns (twins 6 / 6 / 4);
-                                          14 = 128x128 of that kind with K cut in two halves that are added inside the launch
-                                          (scratch from the workspace; twin 1);
+                                          14 / 15 = 128x128 / 128x256 of that kind with K cut in two halves that are added inside
+                                          the launch (scratch from the workspace; twins 1 / 12);
                                           f32: 1 128x128, 2 128x64, 3 64x64, 4 128x128 with K step 16 */
     DXH_TUNE_MATMUL_SPLITK = 6,        /* slices along K of a float matmul: 0 = chosen per shape (few output tiles and a long
                                           K are cut so that every CU has work), 1 = never, n <= 1024 = n slices.  Slices are
@@ -387,7 +387,7 @@ DXH_API int dxh_dropout(int dtype, void *inout, int64_t n, float p, uint32_t see
  * query only looks at the alignment of a, b, c, never at what they point to.  Which kernels run
  * depends on the arguments and the tuning knobs alone, so a call recorded under stream capture
  * gives the bits of the eager call.  One exception: the cut of a bf16 / f16 product into two halves
- * of K that are added inside one launch (tile 14) counts its halves in a device array of the library
+ * of K that are added inside one launch (tiles 14 and 15) counts its halves in a device array of the library
  * (the one the strided-axis reductions use: a slice per stream, launches recorded under capture take
  * counters that are never handed out again); with more than 32 streams at once, or some 250 such
  * launches recorded, the same tile runs uncut and the last bits of the sums differ. */

@@ -114,11 +114,11 @@ def test_tuning_knobs_validate_their_values():
     knobs = {name: int(val) for name, val in re.findall(r"(DXH_TUNE_\w+)\s*=\s*(\d+)", text)}
     assert sorted(knobs.values()) == list(range(len(knobs))), knobs  # dense numbering, no duplicates
     good = {"DXH_TUNE_NT_STORE_BYTES": [0, 1 << 20], "DXH_TUNE_REDUCE_TARGET_BLOCKS": [256, 1024], "DXH_TUNE_REDUCE_COL_MIN_ROWS": [1, 16],
-            "DXH_TUNE_REDUCE_COL_MAX_LANES": [4, 32, 128, 256], "DXH_TUNE_MATMUL_TILE": [1, 6, 14, 0], "DXH_TUNE_REDUCE_ROW_LOADS": [1, 4],
+            "DXH_TUNE_REDUCE_COL_MAX_LANES": [4, 32, 128, 256], "DXH_TUNE_MATMUL_TILE": [1, 6, 15, 0], "DXH_TUNE_REDUCE_ROW_LOADS": [1, 4],
             "DXH_TUNE_MATMUL_SPLITK": [1, 7, 1024, 0], "DXH_TUNE_NT_LOAD": [1, 2, 0], "DXH_TUNE_SKINNY_PER_CU": [2, 4, 1],
             "DXH_TUNE_SKINNY_MIN_ROWS": [8, 512, 256], "DXH_TUNE_SKINNY_HALF": [1, 0], "DXH_TUNE_REDUCE_FUSED_FINISH": [0, 1]}
     bad = {"DXH_TUNE_REDUCE_TARGET_BLOCKS": [0], "DXH_TUNE_REDUCE_COL_MIN_ROWS": [0], "DXH_TUNE_REDUCE_COL_MAX_LANES": [3, 512],
-           "DXH_TUNE_MATMUL_TILE": [-1, 15], "DXH_TUNE_REDUCE_ROW_LOADS": [0, 65], "DXH_TUNE_MATMUL_SPLITK": [-1, 1025], "DXH_TUNE_NT_LOAD": [-1, 3], "DXH_TUNE_SKINNY_PER_CU": [0, 65],
+           "DXH_TUNE_MATMUL_TILE": [-1, 16], "DXH_TUNE_REDUCE_ROW_LOADS": [0, 65], "DXH_TUNE_MATMUL_SPLITK": [-1, 1025], "DXH_TUNE_NT_LOAD": [-1, 3], "DXH_TUNE_SKINNY_PER_CU": [0, 65],
            "DXH_TUNE_SKINNY_MIN_ROWS": [7], "DXH_TUNE_SKINNY_HALF": [-1, 2], "DXH_TUNE_REDUCE_FUSED_FINISH": [-1, 2]}
     assert set(good) == set(knobs), set(good) ^ set(knobs)
     defaults = {"DXH_TUNE_NT_STORE_BYTES": 0, "DXH_TUNE_REDUCE_TARGET_BLOCKS": 1024, "DXH_TUNE_REDUCE_COL_MIN_ROWS": 16,

@@ -84,13 +84,13 @@ def test_config5_gemm_shapes_bf16(dxh, orc):
 TILE_KNOB = 4  # DXH_TUNE_MATMUL_TILE
 
 
-@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14])
+@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15])
 @pytest.mark.parametrize("dtype", [dx.BF16, dx.F16])
 def test_matmul_tile_configs(dxh, dtype, tile):
     """Every workgroup tile of the MFMA kernel (forced through the tuning knob) on aligned shapes
     with ragged tile edges, more than one batch and M, N below one tile; float64 numpy is the
     reference, bar rel 1e-2 of sum_k |a||b| as above.  K = 72, 8, 1000, 56 end in a partial K step
-    (zero-filled in the kernel; tiles 7 to 14, whose operands go straight into LDS in whole K steps,
+    (zero-filled in the kernel; tiles 7 to 15, whose operands go straight into LDS in whole K steps,
     hand those to their register-staged twins); K = 32 and 64 are shorter than the LDS pipeline of
     those tiles, K = 192 and 448 wrap around its stages.  Tiles 11 and 12 (160 and 128 rows, four
     waves side by side) meet M below, at and above a tile, with a last tile of 1 to 159 rows."""
@@ -124,7 +124,7 @@ def test_matmul_tiles_exact_on_small_integers(dxh):
         B = H.to_storage(Bi.astype(np.float64).reshape(-1), dx.BF16)
         want = (Ai @ Bi).astype(np.float64)  # |sum| <= 16*256 = 4096: exact in fp32
         dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, np.uint16)
-        for tile in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14):
+        for tile in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15):
             dx.check(dxh.dxh_tune(TILE_KNOB, tile))
             try:
                 dx.check(H.matmul(dxh, dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
@@ -259,13 +259,13 @@ def test_matmul_skinny_shapes_auto_split(dxh, dtype):
 
 
 @pytest.mark.parametrize("dtype,m,k,n", [(dx.F32, 16, 4096, 256), (dx.BF16, 64, 8192, 64), (dx.BF16, 333, 777, 555),
-                                         (dx.F32, 4, 4096, 1024), (dx.F64, 130, 515, 67), (dx.BF16, 1000, 4160, 904), (dx.F16, 2048, 4864, 896)])
+                                         (dx.F32, 4, 4096, 1024), (dx.F64, 130, 515, 67), (dx.BF16, 1000, 4160, 904), (dx.F16, 2048, 4864, 896), (dx.BF16, 1000, 4160, 2824)])
 def test_matmul_under_capture_equals_eager(dxh, dtype, m, k, n):
     """Products that are cut along K or run on padded copies keep their partial results in the
     caller's workspace, so the same kernels run under stream capture: a recorded matmul replays
     the bits of the eager call (and neither allocates).  The last two shapes take 128x128 tiles whose
     two halves of K meet inside the launch (a ragged M and N, K steps that do not halve evenly; the
-    second config-5 shape)."""
+    second config-5 shape; the last one 128x256 tiles of that kind)."""
     import ctypes as C
     rng = np.random.default_rng(900 + m)
     A = H.to_storage(rng.standard_normal(m * k), dtype)

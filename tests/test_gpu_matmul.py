@@ -300,6 +300,40 @@ def test_matmul_under_capture_equals_eager(dxh, dtype, m, k, n):
     dx.check(dxh.dxh_stream_destroy(st))
 
 
+def test_k_cut_inside_the_launch_many_launches(dxh):
+    """The two halves of a K cut meet through device memory and a counter that strided-axis
+    reductions of the same stream use as well: 400 launches, a fused-finish reduction between any
+    two, every product bit-identical to the first (which half arrives last varies from launch to
+    launch; their sum may not) and within the float64 bar, every reduction identical to the first."""
+    import ctypes as C
+    rng = np.random.default_rng(77)
+    m, k, n = 1000, 4160, 904
+    A = H.to_storage(rng.standard_normal(m * k), dx.BF16)
+    B = H.to_storage(rng.standard_normal(k * n), dx.BF16)
+    dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, np.uint16)
+    need = C.c_size_t(0)
+    dx.check(dxh.dxh_matmul_workspace_bytes(dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, C.byref(need)))
+    assert need.value == 8 * 8 * 2 * 128 * 128 * 4, "64 tiles of 128x128, two fp32 partial tiles each"
+    ws = Dev.empty(need.value, np.uint8)
+    R, Cc = 4096, 2048
+    X = Dev(rng.standard_normal(R * Cc).astype(np.float32))
+    col = Dev.empty(Cc, np.float32)
+    rneed = C.c_size_t(0)
+    dx.check(dxh.dxh_reduce_workspace_bytes(dx.F32, dx.i32arr([R, Cc]), 2, dx.i32arr([0]), 1, C.byref(rneed)))
+    rws = Dev.empty(max(rneed.value, 1), np.uint8)
+    first = first_col = None
+    for it in range(400):
+        dx.check(dxh.dxh_matmul(dx.BF16, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, ws.ptr, need.value, None))
+        dx.check(dxh.dxh_sum(dx.F32, X.ptr, dx.i32arr([R, Cc]), 2, dx.i32arr([0]), 1, col.ptr, rws.ptr, rneed.value, None))
+        if it % 40 == 0 or it == 399:
+            got, gcol = dC.get(), col.get()
+            if first is None:
+                first, first_col = got, gcol
+                Af, Bf = H.to_float(A, dx.BF16).reshape(m, k), H.to_float(B, dx.BF16).reshape(k, n)
+                assert np.all(np.abs(H.to_float(got, dx.BF16).reshape(m, n) - Af @ Bf) <= 1e-2 * (np.abs(Af) @ np.abs(Bf)))
+            assert np.array_equal(got, first) and np.array_equal(gcol, first_col), it
+
+
 @pytest.mark.parametrize("dtype", [dx.BF16, dx.F16])
 @pytest.mark.parametrize("tile", [0, 1])
 def test_matmul_half_rows_not_16_byte_aligned(dxh, dtype, tile):

@@ -239,6 +239,8 @@ def main():
     cpu = None
     if not args.no_cpu:
         cpu = cpu_baseline(np, dx)
+        if not args.no_per_op:
+            merge_cpu_per_op(per_op, cpu_per_op(np, dx))
 
     line = {
         "metric": "achieved HBM GB/s & % of peak per deepxIR op; matmul TFLOP/s; vs op-ompsimd",
@@ -379,10 +381,14 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
     del a, b, o, m
     torch.cuda.empty_cache()
     E = (torch.randn(151936, 896, device=dev) * 0.02).to(torch.bfloat16)
-    idx = [torch.randint(0, 151936, (4096,), device=dev, dtype=torch.int64) for _ in range(4)]
+    # 48 index sets: 196,608 rows of 1792 bytes = 352 MB of distinct table rows between two uses of a set, more
+    # than the 256 MiB last-level cache holds, so the gathered rows come from HBM
+    NI = 48
+    idx = [torch.randint(0, 151936, (4096,), device=dev, dtype=torch.int64) for _ in range(NI)]
     eo = torch.empty(4096 * 896, device=dev, dtype=torch.bfloat16)
     esh, xsh = dx.i32arr([151936, 896]), dx.i32arr([4096])
-    c4["indexselect_bf16_4096_of_151936x896(latency-bound)"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_indexselect(dx.BF16, ptr(E), esh, 2, dx.I64, ptr(idx[i % 4]), xsh, 1, 0, ptr(eo), None)), 2 * 4096 * 896 * 2 + 4096 * 8)
+    c4["indexselect_bf16_4096_of_151936x896(latency-bound)"] = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_indexselect(dx.BF16, ptr(E), esh, 2, dx.I64, ptr(idx[i % NI]), xsh, 1, 0, ptr(eo), None), reps=NI - 3), 2 * 4096 * 896 * 2 + 4096 * 8)
+    c4["indexselect_bf16_4096_of_151936x896(latency-bound)"]["index_sets_rotated"] = NI
     del E, eo
     torch.cuda.empty_cache()
     res["config4"] = c4
@@ -666,6 +672,142 @@ def cpu_baseline(np, dx):
         pass
     return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
             "sample": f"full config-2 step (10 ops, {nbytes} bytes), median of 5 timed passes after 1 warm-up: {dt:.2f} s; OMP threads={cores}; cpu='{model}'; -O2, AVX2 auto-vectorisation"}
+
+
+def cpu_per_op(np, dx):
+    """The other configs' ops through the oracle's restatement of op-ompsimd on this host's cores:
+    chunked elementwise loops (shape_range.cpp:116-135), the per-element index-vector gathers of
+    transpose / broadcastTo / indexselect and the run-wise concat (changeshape_miaobyte.hpp:45-178),
+    the per-element reduce (reduce_miaobyte.hpp:30-44).  The reference multiplies through OpenBLAS
+    cblas_sgemm (matmul_cblas.hpp:51-57), which this image does not have: torch.matmul on CPU
+    tensors stands in for it, in the reference's dtypes (fp32 / fp64; op-ompsimd has no 16-bit
+    floats, so the bf16 entries carry the fp32 figure).  Every op at its full BASELINE size, one
+    untimed call, then the median of three.  Returns {config: {op label: {cpu_ms, cores, cpu_kind}}}."""
+    import ctypes as C
+    from tests import helpers as H
+    orc = H.oracle()
+    hp = H.hp
+    cores = orc.orc_num_threads()
+
+    def med(fn, reps=3):
+        fn()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            rc = fn()
+            ts.append(time.perf_counter() - t0)
+            assert rc in (0, None), rc
+        return {"cpu_ms": round(sorted(ts)[len(ts) // 2] * 1e3, 3), "cores": cores, "cpu_kind": "port"}
+
+    out = {}
+    rng = np.random.default_rng(21)
+    # config 1
+    n = 4096 * 4096
+    a = rng.uniform(-1, 1, n).astype(np.float32)
+    b = rng.uniform(-1, 1, n).astype(np.float32)
+    c = np.empty(n, dtype=np.float32)
+    half = dx.scalar(0.5)
+    out["config1"] = {
+        "add": med(lambda: orc.orc_add(dx.F32, hp(a), hp(b), hp(c), n)),
+        "mul": med(lambda: orc.orc_mul(dx.F32, hp(a), hp(b), hp(c), n)),
+        "max": med(lambda: orc.orc_max(dx.F32, hp(a), hp(b), hp(c), n)),
+        "div": med(lambda: orc.orc_div(dx.F32, hp(a), hp(b), hp(c), n)),
+        "addscalar": med(lambda: orc.orc_addscalar(dx.F32, hp(a), half, hp(c), n)),
+        "mulscalar": med(lambda: orc.orc_mulscalar(dx.F32, hp(a), half, hp(c), n)),
+        "exp": med(lambda: orc.orc_exp(dx.F32, hp(a), hp(c), n)),
+    }
+    del a, b, c
+    # config 3 (16-bit tensors move as raw bits)
+    shape = [32, 2048, 14, 64]
+    nt = 32 * 2048 * 14 * 64
+    t = rng.integers(0, 65536, nt, dtype=np.uint16)
+    to = np.empty(nt, dtype=np.uint16)
+    c3 = {"transpose_bf16_32x2048x14x64_0213": med(lambda: orc.orc_faithful_transpose(dx.BF16, hp(t), dx.i32arr(shape), 4, dx.i32arr([0, 2, 1, 3]), hp(to)))}
+    del t, to
+    nc = 16 * 1024 * 4096
+    cs = [rng.integers(0, 65536, nc, dtype=np.uint16) for _ in range(3)]
+    co = np.empty(3 * nc, dtype=np.uint16)
+    ins = dx.ptrarr([x.ctypes.data for x in cs])
+    c3["concat_fp16_3x16x1024x4096_axis1"] = med(lambda: orc.orc_faithful_concat(dx.F16, ins, 3, dx.i32arr([1024] * 3), dx.i32arr([16, 3072, 4096]), 3, 1, hp(co)))
+    del cs, co
+    r = rng.integers(0, 65536, 4096, dtype=np.uint16)
+    bo = np.empty(8192 * 4096, dtype=np.uint16)
+    c3["broadcastTo_bf16_1x4096_to_8192x4096"] = med(lambda: orc.orc_faithful_broadcastTo(dx.BF16, hp(r), dx.i32arr([1, 4096]), 2, dx.i32arr([8192, 4096]), 2, hp(bo)))
+    del bo
+    out["config3"] = c3
+    # config 4
+    n = 1 << 26
+    a = rng.integers(-2 ** 20, 2 ** 20 + 1, n, dtype=np.int32)
+    b = rng.integers(-2 ** 20, 2 ** 20 + 1, n, dtype=np.int32)
+    o = np.empty(n, dtype=np.int32)
+    m = np.empty(n, dtype=np.uint8)
+    c4 = {"max_i32_2^26": med(lambda: orc.orc_max(dx.I32, hp(a), hp(b), hp(o), n)),
+          "min_i32_2^26": med(lambda: orc.orc_min(dx.I32, hp(a), hp(b), hp(o), n)),
+          "greater_i32_2^26": med(lambda: orc.orc_greater(dx.I32, hp(a), hp(b), hp(m), n))}
+    sw = dx.ptrarr([b.ctypes.data, a.ctypes.data])
+    c4["where_i32_2^26(switch)"] = med(lambda: orc.orc_switch(dx.I32, sw, 2, dx.BOOL, hp(m), hp(o), n))
+    del a, b, o, m
+    E = rng.integers(0, 65536, 151936 * 896, dtype=np.uint16)
+    idx = rng.integers(0, 151936, 4096, dtype=np.int64)
+    eo = np.empty(4096 * 896, dtype=np.uint16)
+    c4["indexselect_bf16_4096_of_151936x896"] = med(lambda: orc.orc_faithful_indexselect(dx.BF16, hp(E), dx.i32arr([151936, 896]), 2, dx.I64, hp(idx), dx.i32arr([4096]), 1, 0, hp(eo)))
+    del E, eo
+    out["config4"] = c4
+    # config 5: the glue through the oracle (16-bit floats compute in fp32 and round once, op-cuda's
+    # convention), the GEMMs through torch on the CPU
+    S, Hd, I = 2048, 896, 4864
+    n16, n32 = S * I, S * Hd
+    g16 = H.f32_to_bf16_bits(rng.standard_normal(n16).astype(np.float32))
+    u16 = H.f32_to_bf16_bits(rng.standard_normal(n16).astype(np.float32))
+    o16 = np.empty(n16, dtype=np.uint16)
+    x16 = H.f32_to_bf16_bits(rng.standard_normal(n32).astype(np.float32))
+    x32 = rng.standard_normal(n32).astype(np.float32)
+    o32 = np.empty(n32, dtype=np.float32)
+    col = np.empty(S, dtype=np.float32)
+    one, two, neg = dx.scalar(1.0), dx.scalar(2.0), dx.scalar(-1.0)
+    glue = {
+        "mulscalar_bf16_2048x4864": med(lambda: orc.orc_mulscalar(dx.BF16, hp(g16), neg, hp(o16), n16)),
+        "exp_bf16_2048x4864": med(lambda: orc.orc_exp(dx.BF16, hp(g16), hp(o16), n16)),
+        "rdivscalar_bf16_2048x4864": med(lambda: orc.orc_rdivscalar(dx.BF16, one, hp(g16), hp(o16), n16)),
+        "mul_bf16_2048x4864": med(lambda: orc.orc_mul(dx.BF16, hp(g16), hp(u16), hp(o16), n16)),
+        "todtype_bf16_to_f32_2048x896": med(lambda: orc.orc_todtype(dx.BF16, hp(x16), dx.F32, hp(o32), n32)),
+        "powscalar_f32_2048x896": med(lambda: orc.orc_powscalar(dx.F32, hp(x32), two, hp(o32), n32)),
+        "sum_f32_2048x896_axis1_keepdims": med(lambda: orc.orc_faithful_reduce_f32(0, hp(x32), dx.i32arr([S, Hd]), 2, dx.i32arr([1]), 1, 1, hp(col))),
+        "broadcastTo_f32_2048x1_to_2048x896": med(lambda: orc.orc_faithful_broadcastTo(dx.F32, hp(col), dx.i32arr([S, 1]), 2, dx.i32arr([S, Hd]), 2, hp(o32))),
+    }
+    c5 = {"glue_ops(cache-resident sizes)": glue}
+    import torch
+    threads = torch.get_num_threads()
+    for mm, kk, nn in ((2048, 896, 4864), (2048, 4864, 896)):
+        for dt, tdt in (("f32", torch.float32), ("f64", torch.float64)):
+            A = torch.randn(mm, kk, dtype=tdt)
+            B = torch.randn(kk, nn, dtype=tdt) * 0.02
+            Cm = torch.empty(mm, nn, dtype=tdt)
+            e = med(lambda: (torch.matmul(A, B, out=Cm), None)[1])
+            e.update({"cores": threads, "cpu_kind": f"torch.matmul on CPU {dt} tensors, standing in for OpenBLAS cblas_{'s' if dt == 'f32' else 'd'}gemm (not in this image)"})
+            c5[f"matmul_{dt}_{mm}x{kk}x{nn}"] = e
+            if dt == "f32":
+                c5[f"matmul_bf16_{mm}x{kk}x{nn}"] = dict(e, cpu_dtype="f32 (op-ompsimd has no 16-bit floats)")
+    out["config5"] = c5
+    return out
+
+
+def merge_cpu_per_op(per_op, cpu):
+    """cpu_ms / cores / cpu_kind of cpu_per_op() into the per_op entries of the same label (labels may
+    carry a remark in parentheses after the CPU leg's label)."""
+    for cfg, ops in cpu.items():
+        dst = per_op.get(cfg)
+        if not isinstance(dst, dict):
+            continue
+        for label, fig in ops.items():
+            if "cpu_ms" not in fig:  # a group of ops (the glue table)
+                merge_cpu_per_op(dst, {label: fig})
+                continue
+            for k, entry in dst.items():
+                if isinstance(entry, dict) and (k == label or k.startswith(label + "(")):
+                    entry.update(fig)
+                    if "ms" in entry and entry["ms"] > 0:
+                        entry["gpu_over_cpu"] = round(fig["cpu_ms"] / entry["ms"], 1)
 
 
 if __name__ == "__main__":

@@ -113,6 +113,18 @@ DXE_API size_t dxe_shape_yaml_roundtrip(const char *yaml, char *out, size_t bufl
         return copy_out(std::string("error: ") + e.what(), out, buflen);
     }
 }
+// the host side of a tensor's raw `.data` file (tensorio.hpp), without a tensor: "" or "error: ..."
+DXE_API size_t dxe_data_write(const char *path, const char *data, size_t bytes, char *out, size_t buflen) {
+    try { write_exact(path ? path : "", data, bytes); return copy_out("", out, buflen); }
+    catch (const std::exception &e) { return copy_out(std::string("error: ") + e.what(), out, buflen); }
+}
+DXE_API size_t dxe_data_read(const char *path, char *data, size_t bytes, char *out, size_t buflen) {
+    try {
+        const std::vector<char> got = read_exact(path ? path : "", bytes);
+        if (bytes) std::memcpy(data, got.data(), bytes);
+        return copy_out("", out, buflen);
+    } catch (const std::exception &e) { return copy_out(std::string("error: ") + e.what(), out, buflen); }
+}
 // shape inference helpers by name, result as space-separated ints or "error: ...":
 //   transpose(a=shape, b=order) broadcast(a, b) indexselect(a=input, b=index shape, extra=axis)
 //   repeat(a=shape, b=repeats) checked_dims(a=shape, b=dims) reduced(a=shape, b=checked dims, extra=keepdims)

@@ -2,6 +2,8 @@
 // executor/op-ompsimd's `main` (executor/op-cuda/src/client/main.cpp:23-105).
 //   DEEPX_PORT     UDP port (default 9090, op-cuda's port and the front's default endpoint)
 //   DEEPX_DEVICE   HIP device ordinal (default 0)
+//   DEEPX_BIND     local IPv4 address to bind (default: any, as the reference)
+//   DEEPX_REMOTE_QUIT 1: honour the `__quit__` line from any source address (default: loopback only)
 //   DEEPX_IR_LOG   1|true: echo every instruction
 //   DEEPX_SYNC     0: reply at launch instead of at completion
 //   DEEPX_OPLIST   path: write the generated op table (markdown) there, as the reference writes

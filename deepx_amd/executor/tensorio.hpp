@@ -32,19 +32,22 @@ inline std::vector<char> to_host(const Tensor &t) {
     return host;
 }
 
-inline void save_tensor(const Tensor &t, const std::string &path) {
-    {
-        std::ofstream fs(path + ".shape", std::ios::binary | std::ios::trunc);
-        if (!fs.is_open()) throw std::runtime_error("Failed to open file for writing: " + path + ".shape");
-        fs << t.shape.to_yaml();
-    }
-    std::vector<char> host = to_host(t);
-    std::ofstream fs(path + ".data", std::ios::binary | std::ios::trunc);
-    if (!fs.is_open()) throw std::runtime_error("Failed to open file for writing: " + path + ".data");
-    fs.write(host.data(), (std::streamsize)host.size());
-    if (!fs) throw std::runtime_error("Failed to write data to file: " + path + ".data");
+// raw bytes to a file that is created or emptied first (stdutil/fs.cpp:18-29)
+inline void write_exact(const std::string &path, const char *data, size_t bytes) {
+    std::ofstream fs(path, std::ios::binary | std::ios::out | std::ios::trunc);
+    if (!fs.is_open()) throw std::runtime_error("Failed to open file for writing: " + path);
+    fs.write(data, (std::streamsize)bytes);
+    if (!fs) throw std::runtime_error("Failed to write data to file: " + path);
 }
 
+inline void save_tensor(const Tensor &t, const std::string &path) {
+    const std::string yaml = t.shape.to_yaml();
+    write_exact(path + ".shape", yaml.data(), yaml.size());
+    std::vector<char> host = to_host(t);
+    write_exact(path + ".data", host.data(), host.size());
+}
+
+// a file that must hold exactly `want` bytes (stdutil/fs.cpp:31-50)
 inline std::vector<char> read_exact(const std::string &path, size_t want) {
     std::ifstream fs(path, std::ios::binary);
     if (!fs.is_open()) throw std::runtime_error("Failed to open file: " + path);

@@ -4,13 +4,17 @@
 // datagram on '\n', reply to the sender with sendto).  Differences, all to remove crashes: the
 // receive buffer is 64 KiB with the terminator inside it (the reference writes buffer[1024]), a
 // parse failure answers with an error line instead of unwinding the receiver thread, and replies go
-// to the address each datagram came from rather than to "the last client".
+// to the address each datagram came from rather than to "the last client".  One line of its own,
+// `__quit__`, ends serve() (the test harness stops the process with it); it is honoured only in a
+// datagram whose source address is loopback, unless DEEPX_REMOTE_QUIT=1.  DEEPX_BIND names the local
+// address to bind instead of INADDR_ANY (e.g. 127.0.0.1 when the front runs on the same host).
 #pragma once
 #include <arpa/inet.h>
 #include <sys/socket.h>
 #include <unistd.h>
 #include <atomic>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <sstream>
 #include <string>
@@ -31,6 +35,11 @@ public:
         sockaddr_in addr{};
         addr.sin_family = AF_INET;
         addr.sin_addr.s_addr = INADDR_ANY;
+        if (const char *bind_to = std::getenv("DEEPX_BIND")) {
+            if (::inet_pton(AF_INET, bind_to, &addr.sin_addr) != 1) { fprintf(stderr, "DEEPX_BIND: not an IPv4 address: %s\n", bind_to); return false; }
+        }
+        const char *rq = std::getenv("DEEPX_REMOTE_QUIT");
+        remote_quit_ = rq && std::string(rq) == "1";
         addr.sin_port = htons((uint16_t)port_);
         if (::bind(fd_, (const sockaddr *)&addr, sizeof addr) < 0) { perror("bind failed"); return false; }
         timeval tv{0, 200000};  // wake up to notice stop()
@@ -56,7 +65,11 @@ public:
             while (std::getline(lines, line)) {
                 if (!line.empty() && line.back() == '\r') line.pop_back();
                 if (line.empty()) continue;
-                if (line == "__quit__") { stop_ = true; break; }
+                if (line == "__quit__") {
+                    const bool loopback = (ntohl(cli.sin_addr.s_addr) >> 24) == 127;
+                    if (loopback || remote_quit_) { stop_ = true; break; }
+                    continue;  // from elsewhere: neither a command nor an instruction
+                }
                 batch.push_back(line);
             }
             if (batch.empty()) continue;
@@ -70,6 +83,7 @@ public:
 private:
     int port_;
     int fd_ = -1;
+    bool remote_quit_ = false;
     std::atomic<bool> stop_{false};
 };
 

@@ -578,6 +578,149 @@ template <typename R> int repeat_t(const void *in_, const int32_t *shape, int nd
     return OK;
 }
 
+// ---- the same four changeshape ops with the reference's own per-element decomposition, for
+// CPU-baseline timing only (the functions above move whole rows where they can).  Common frame:
+// Shape::rangeParallel (executor/deepxcore/src/deepx/shape_range.cpp:137-160, :209-233) hands
+// every output position its index vector, rebuilt from the linear index with one `%` and one
+// `/` per axis; Shape::linearat (executor/deepxcore/src/deepx/shape.cpp:73-83) turns an index
+// vector back into an offset.
+inline int64_t linear_at(const std::vector<int64_t> &strides, const std::vector<int> &indices) {
+    int64_t idx = 0;
+    size_t s = 0, i = indices.size() > strides.size() ? indices.size() - strides.size() : 0;
+    for (; s < strides.size() && s < indices.size();) idx += indices[i++] * strides[s++];
+    return idx;
+}
+template <typename F> void range_parallel(const int32_t *shape, int dims, F body) {
+    int64_t total = 1;
+    for (int i = 0; i < dims; ++i) total *= shape[i];
+#pragma omp parallel
+    {
+        std::vector<int> indices(dims, 0);
+#pragma omp for
+        for (int64_t idx = 0; idx < total; ++idx) {
+            int64_t rem = idx;
+            for (int d = dims - 1; d >= 0; --d) { indices[d] = int(rem % shape[d]); rem /= shape[d]; }
+            body(idx, indices);
+        }
+    }
+}
+// transpose, E/changeshape_miaobyte.hpp:45-67: a thread-local index vector takes
+// p[dim_order[i]] = o[i], then out[o] = in[linearat(p)].
+template <typename R> int transpose_faithful_t(const void *in_, const int32_t *shape, int ndim, const int32_t *order, void *out_) {
+    const R *in = (const R *)in_; R *out = (R *)out_;
+    std::vector<int32_t> oshape(ndim);
+    std::vector<int> seen(ndim, 0);
+    for (int i = 0; i < ndim; ++i) {
+        if (order[i] < 0 || order[i] >= ndim || seen[order[i]]++) return ERR_ARG;
+        oshape[i] = shape[order[i]];
+    }
+    Strides is(shape, ndim);
+#pragma omp parallel
+    {
+        std::vector<int> indices(ndim, 0), src(ndim, 0);
+#pragma omp for
+        for (int64_t idx = 0; idx < is.size; ++idx) {
+            int64_t rem = idx;
+            for (int d = ndim - 1; d >= 0; --d) { indices[d] = int(rem % oshape[d]); rem /= oshape[d]; }
+            for (int i = 0; i < ndim; ++i) src[order[i]] = indices[i];
+            out[idx] = in[linear_at(is.v, src)];
+        }
+    }
+    return OK;
+}
+// concat, E/changeshape_miaobyte.hpp:69-100: over the first axis + 1 output axes; the source tensor is
+// found by walking the axis sizes, the index vector is copied and patched, and a run of
+// strides[axis] elements is copied.
+template <typename R> int concat_faithful_t(const void *const *ins, int nins, const int32_t *axis_sizes,
+                                            const int32_t *out_shape, int ndim, int axis, void *out_) {
+    R *out = (R *)out_;
+    if (axis < 0 || axis >= ndim || nins < 1) return ERR_ARG;
+    int64_t total = 0;
+    for (int i = 0; i < nins; ++i) total += axis_sizes[i];
+    if (total != out_shape[axis]) return ERR_SHAPE;
+    int64_t inner = 1;
+    for (int i = axis + 1; i < ndim; ++i) inner *= out_shape[i];
+    std::vector<std::vector<int64_t>> strides(nins);  // of every source, over the first axis + 1 axes
+    for (int t = 0; t < nins; ++t) {
+        strides[t].assign(axis + 1, 0);
+        int64_t s = inner;
+        for (int i = axis; i >= 0; --i) { strides[t][i] = s; s *= (i == axis ? axis_sizes[t] : out_shape[i]); }
+    }
+    range_parallel(out_shape, axis + 1, [&](int64_t idx, const std::vector<int> &indices) {
+        int at = indices[axis], t = 0;
+        while (t < nins) {
+            if (at < axis_sizes[t]) break;
+            at -= axis_sizes[t];
+            ++t;
+        }
+        std::vector<int> cur = indices;
+        cur[axis] = at;
+        const R *src = (const R *)ins[t] + linear_at(strides[t], cur);
+        std::copy(src, src + inner, out + idx * inner);
+    });
+    return OK;
+}
+// broadcastTo, E/changeshape_miaobyte.hpp:102-139: a fresh source index vector per element
+// (fromBroadcastIndices pushes one entry per mapped axis), then linearat.
+template <typename R> int broadcast_faithful_t(const void *in_, const int32_t *ishape, int indim,
+                                               const int32_t *oshape, int ondim, void *out_) {
+    const R *in = (const R *)in_; R *out = (R *)out_;
+    if (indim > ondim) return ERR_SHAPE;
+    const int shift = ondim - indim;
+    enum { X_TO_X, NULL_TO_1, X_TO_1 };
+    std::vector<int> bmap(ondim, NULL_TO_1);
+    for (int i = shift; i < ondim; ++i) {
+        if (ishape[i - shift] == oshape[i]) bmap[i] = X_TO_X;
+        else if (ishape[i - shift] == 1) bmap[i] = X_TO_1;
+        else return ERR_SHAPE;
+    }
+    Strides is(ishape, indim);
+    range_parallel(oshape, ondim, [&](int64_t idx, const std::vector<int> &bidx) {
+        std::vector<int> src;
+        for (int i = 0; i < ondim; ++i) {
+            if (bmap[i] == X_TO_X) src.push_back(bidx[i]);
+            else if (bmap[i] == X_TO_1) src.push_back(0);
+        }
+        out[idx] = in[linear_at(is.v, src)];
+    });
+    return OK;
+}
+// indexselect, E/changeshape_miaobyte.hpp:141-178: per output element the index vector is cut into
+// (pre, index position, post), the index tensor is read through linearat, and the patched input
+// index vector goes through linearat again.  Out-of-range entries are clamped as in indexselect_t.
+template <typename R, typename IT>
+int indexselect_faithful_t(const void *in_, const int32_t *ishape, int indim, const void *index_,
+                           const int32_t *xshape, int xndim, int axis, void *out_) {
+    const R *in = (const R *)in_; const IT *index = (const IT *)index_; R *out = (R *)out_;
+    if (axis < 0) axis += indim;
+    if (axis < 0 || axis >= indim) return ERR_ARG;
+    std::vector<int32_t> oshape;
+    for (int i = 0; i < axis; ++i) oshape.push_back(ishape[i]);
+    for (int i = 0; i < xndim; ++i) oshape.push_back(xshape[i]);
+    for (int i = axis + 1; i < indim; ++i) oshape.push_back(ishape[i]);
+    const int ondim = (int)oshape.size();
+    Strides is(ishape, indim), xs(xshape, xndim), os(oshape.data(), ondim);
+    const int64_t adim = ishape[axis];
+#pragma omp parallel
+    {
+        std::vector<int> oidx(ondim, 0), iidx(indim, 0), xidx(xndim, 0);
+#pragma omp for
+        for (int64_t idx = 0; idx < os.size; ++idx) {
+            int64_t rem = idx;
+            for (int d = ondim - 1; d >= 0; --d) { oidx[d] = int(rem % oshape[d]); rem /= oshape[d]; }
+            std::copy(oidx.begin(), oidx.begin() + axis, iidx.begin());
+            std::copy(oidx.begin() + axis, oidx.begin() + axis + xndim, xidx.begin());
+            int64_t k = (int64_t)index[linear_at(xs.v, xidx)];
+            if (k < 0) k = 0;
+            if (k >= adim) k = adim - 1;
+            iidx[axis] = (int)k;
+            std::copy(oidx.begin() + axis + xndim, oidx.end(), iidx.begin() + axis + 1);
+            out[idx] = in[linear_at(is.v, iidx)];
+        }
+    }
+    return OK;
+}
+
 #define DISPATCH_RAW(dtype, CALL)                 \
     switch (esize(dtype)) {                       \
     case 8: return CALL(uint64_t);                \
@@ -858,6 +1001,37 @@ int orc_indexselect(int dtype, const void *in, const int32_t *ishape, int indim,
 #undef IS
     } else if (index_dtype == I32) {
 #define IS(R) indexselect_t<R, int32_t>(in, ishape, indim, index, xshape, xndim, axis, out)
+        DISPATCH_RAW(dtype, IS)
+#undef IS
+    }
+    return ERR_DTYPE;
+}
+// the four ops above in the reference's per-element decomposition (CPU-baseline timing; results are
+// those of orc_transpose / orc_concat / orc_broadcastTo / orc_indexselect)
+int orc_faithful_transpose(int dtype, const void *in, const int32_t *shape, int ndim, const int32_t *order, void *out) {
+#define TR(R) transpose_faithful_t<R>(in, shape, ndim, order, out)
+    DISPATCH_RAW(dtype, TR)
+#undef TR
+}
+int orc_faithful_concat(int dtype, const void *const *ins, int nins, const int32_t *axis_sizes, const int32_t *out_shape,
+                        int ndim, int axis, void *out) {
+#define CC(R) concat_faithful_t<R>(ins, nins, axis_sizes, out_shape, ndim, axis, out)
+    DISPATCH_RAW(dtype, CC)
+#undef CC
+}
+int orc_faithful_broadcastTo(int dtype, const void *in, const int32_t *ishape, int indim, const int32_t *oshape, int ondim, void *out) {
+#define BC(R) broadcast_faithful_t<R>(in, ishape, indim, oshape, ondim, out)
+    DISPATCH_RAW(dtype, BC)
+#undef BC
+}
+int orc_faithful_indexselect(int dtype, const void *in, const int32_t *ishape, int indim, int index_dtype, const void *index,
+                             const int32_t *xshape, int xndim, int axis, void *out) {
+    if (index_dtype == I64) {
+#define IS(R) indexselect_faithful_t<R, int64_t>(in, ishape, indim, index, xshape, xndim, axis, out)
+        DISPATCH_RAW(dtype, IS)
+#undef IS
+    } else if (index_dtype == I32) {
+#define IS(R) indexselect_faithful_t<R, int32_t>(in, ishape, indim, index, xshape, xndim, axis, out)
         DISPATCH_RAW(dtype, IS)
 #undef IS
     }

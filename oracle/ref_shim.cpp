@@ -4,7 +4,8 @@
 // TEST INFRASTRUCTURE ONLY (used by tests/ to pin the executor's protocol layer against the real
 // reference): IR parsing and printing (tf/tf.cpp), dtype strings (dtype.hpp), op matching
 // (tf/tffactory.cpp) and the shape-inference helpers that do not need Shape's constructor
-// (shape_changeshape.cpp, shape_reduce.cpp).  This file contains no reference code; it only calls it.
+// (shape_changeshape.cpp, shape_reduce.cpp), and the raw file I/O behind tensor `.data` files
+// (stdutil/fs.cpp).  This file contains no reference code; it only calls it.
 // The arithmetic headers of op-ompsimd are NOT buildable here (Highway, OpenBLAS, jemalloc and
 // yaml-cpp are absent), nor is deepxcore/shape.cpp (yaml-cpp); functions that need them are
 // dropped by the linker's section garbage collection and never called.
@@ -17,6 +18,7 @@
 #include "deepx/shape_reduce.hpp"
 #include "deepx/tf/tf.hpp"
 #include "deepx/tf/tffactory.hpp"
+#include "stdutil/fs.hpp"
 
 #define REF_API extern "C" __attribute__((visibility("default")))
 
@@ -113,3 +115,23 @@ REF_API size_t ref_checked_dims(const int *shape, int ndim, const int *dims, int
 REF_API size_t ref_reduced_shape(const int *shape, int ndim, const int *dims, int ndims, int keepdims, char *out, size_t n) {
     return put(ints(deepx::reducedShape(std::vector<int>(shape, shape + ndim), std::vector<int>(dims, dims + ndims), keepdims != 0)), out, n);
 }
+
+// stdutil/fs.cpp: the writer and the two readers of a tensor's raw `.data` file.  Each returns ""
+// or the text of the exception.
+REF_API size_t ref_fs_save(const char *path, const unsigned char *data, size_t bytes, char *out, size_t n) {
+    try { stdutil::save(data, bytes, path); return put("", out, n); }
+    catch (const std::exception &e) { return put(std::string("error: ") + e.what(), out, n); }
+}
+REF_API size_t ref_fs_load(const char *path, unsigned char *data, size_t bytes, char *out, size_t n) {
+    try { stdutil::load(path, data, bytes); return put("", out, n); }
+    catch (const std::exception &e) { return put(std::string("error: ") + e.what(), out, n); }
+}
+// the size-agnostic reader: the file's size, then min(size, bytes) bytes into data
+REF_API size_t ref_fs_load_any(const char *path, unsigned char *data, size_t bytes, char *out, size_t n) {
+    try {
+        auto got = stdutil::load(path);
+        std::memcpy(data, got.second.get(), got.first < bytes ? got.first : bytes);
+        return put(std::to_string(got.first), out, n);
+    } catch (const std::exception &e) { return put(std::string("error: ") + e.what(), out, n); }
+}
+REF_API size_t ref_fs_filename(const char *path, char *out, size_t n) { return put(stdutil::filename(path), out, n); }

@@ -32,6 +32,9 @@ class InProc:
             fn.restype = C.c_size_t
         L.dxe_infer_shape.argtypes = [C.c_char_p, C.POINTER(C.c_int), C.c_int, C.POINTER(C.c_int), C.c_int, C.c_int, C.c_char_p, C.c_size_t]
         L.dxe_infer_shape.restype = C.c_size_t
+        for name in ("dxe_data_write", "dxe_data_read"):
+            getattr(L, name).argtypes = [C.c_char_p, C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t]
+            getattr(L, name).restype = C.c_size_t
         L.dxe_set_graphs.argtypes = [C.c_void_p, C.c_int]
         L.dxe_set_fusion.argtypes = [C.c_void_p, C.c_int]
         L.dxe_print_format_ok.argtypes = [C.c_char_p, C.c_int]
@@ -58,6 +61,16 @@ class InProc:
     def stats(self):
         b, c, r, j = (int(x) for x in self._call(self.L.dxe_stats, self.ex).split())
         return {"batches": b, "captures": c, "replays": r, "rejects": j}
+
+    def data_write(self, path, data):
+        """raw bytes to `path` through the writer behind `save`; returns an empty string or 'error: ...'"""
+        return self._call(self.L.dxe_data_write, path.encode(), bytes(data), len(data))
+
+    def data_read(self, path, nbytes):
+        """(status, bytes) through the reader behind `load` / `loadtensordata`, which wants exactly nbytes"""
+        buf = C.create_string_buffer(max(1, nbytes))
+        status = self._call(self.L.dxe_data_read, path.encode(), buf, nbytes)
+        return status, buf.raw[:nbytes]
 
     def parse(self, line): return self._call(self.L.dxe_parse, line.encode())
     def match(self, line): return self._call(self.L.dxe_match, self.ex, line.encode())
@@ -87,7 +100,9 @@ class Reference:
         sigs = {"ref_parse": [C.c_char_p], "ref_typedef": [C.c_char_p], "ref_match": [C.c_char_p, C.c_char_p],
                 "ref_transpose_shape": [ip, C.c_int, ip], "ref_broadcast_shape": [ip, C.c_int, ip, C.c_int],
                 "ref_indexselect_shape": [ip, C.c_int, ip, C.c_int, C.c_int], "ref_repeat_shape": [ip, C.c_int, ip, C.c_int],
-                "ref_checked_dims": [ip, C.c_int, ip, C.c_int], "ref_reduced_shape": [ip, C.c_int, ip, C.c_int, C.c_int]}
+                "ref_checked_dims": [ip, C.c_int, ip, C.c_int], "ref_reduced_shape": [ip, C.c_int, ip, C.c_int, C.c_int],
+                "ref_fs_save": [C.c_char_p, C.c_char_p, C.c_size_t], "ref_fs_load": [C.c_char_p, C.c_char_p, C.c_size_t],
+                "ref_fs_load_any": [C.c_char_p, C.c_char_p, C.c_size_t], "ref_fs_filename": [C.c_char_p]}
         for name, args in sigs.items():
             fn = getattr(L, name)
             fn.argtypes = args + [C.c_char_p, C.c_size_t]
@@ -112,6 +127,18 @@ class Reference:
     def repeat_shape(self, a, b): return self._call(self.L.ref_repeat_shape, self._arr(a), len(a), self._arr(b), len(b))
     def checked_dims(self, s, d): return self._call(self.L.ref_checked_dims, self._arr(s), len(s), self._arr(d), len(d))
     def reduced_shape(self, s, d, keep): return self._call(self.L.ref_reduced_shape, self._arr(s), len(s), self._arr(d), len(d), int(keep))
+    def fs_save(self, path, data): return self._call(self.L.ref_fs_save, path.encode(), bytes(data), len(data))
+    def fs_filename(self, path): return self._call(self.L.ref_fs_filename, path.encode())
+
+    def fs_load(self, path, nbytes):
+        buf = C.create_string_buffer(max(1, nbytes))
+        status = self._call(self.L.ref_fs_load, path.encode(), buf, nbytes)
+        return status, buf.raw[:nbytes]
+
+    def fs_load_any(self, path, room):
+        buf = C.create_string_buffer(max(1, room))
+        status = self._call(self.L.ref_fs_load_any, path.encode(), buf, room)
+        return status, buf.raw[:room]
 
 
 def free_port():

@@ -52,6 +52,8 @@ def oracle():
                                         C.POINTER(C.c_int32)]
         L.orc_faithful_reduce_f32.argtypes = [C.c_int, C.c_void_p, C.POINTER(C.c_int32), C.c_int,
                                               C.POINTER(C.c_int32), C.c_int, C.c_int, C.c_void_p]
+        for name in ("transpose", "concat", "broadcastTo", "indexselect"):  # same arguments as the plain functions
+            getattr(L, "orc_faithful_" + name).argtypes = getattr(L, "orc_" + name).argtypes
         L.orc_f32_to_bf16.argtypes = [C.c_float]; L.orc_f32_to_bf16.restype = C.c_uint16
         L.orc_f32_to_f16.argtypes = [C.c_float]; L.orc_f32_to_f16.restype = C.c_uint16
         L.orc_bf16_to_f32.argtypes = [C.c_uint16]; L.orc_bf16_to_f32.restype = C.c_float

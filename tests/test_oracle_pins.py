@@ -295,6 +295,42 @@ def test_reduce_closed_forms_and_int8_wrap(orc):
 
 
 # ---- changeshape ---------------------------------------------------------------------------
+def test_faithful_changeshape_equals_plain(orc):
+    """The per-element restatements that the CPU baseline times (index vectors, linearat) give the
+    results of the plain oracle functions, which numpy pins below."""
+    rng = np.random.default_rng(11)
+    for dt, npdt in ((dx.F32, np.float32), (dx.BF16, np.uint16), (dx.I8, np.int8), (dx.F64, np.float64)):
+        x = rng.integers(0, 120, size=(3, 5, 4, 6)).astype(npdt)
+        for order in ([0, 2, 1, 3], [3, 2, 1, 0], [1, 0, 3, 2], [0, 1, 2, 3]):
+            w, g = np.empty(x.size, dtype=npdt), np.empty(x.size, dtype=npdt)
+            assert orc.orc_transpose(dt, hp(x), dx.i32arr(x.shape), 4, dx.i32arr(order), hp(w)) == 0
+            assert orc.orc_faithful_transpose(dt, hp(x), dx.i32arr(x.shape), 4, dx.i32arr(order), hp(g)) == 0
+            assert np.array_equal(w, g) and np.array_equal(g.reshape([x.shape[o] for o in order]), np.transpose(x, order))
+        for ish, osh in (([1, 6], [7, 6]), ([5, 1, 6], [2, 5, 3, 6]), ([1], [4, 9]), ([4, 1], [4, 9])):
+            a = rng.integers(0, 120, size=ish).astype(npdt)
+            w, g = np.empty(osh, dtype=npdt), np.empty(osh, dtype=npdt)
+            assert orc.orc_broadcastTo(dt, hp(a), dx.i32arr(ish), len(ish), dx.i32arr(osh), len(osh), hp(w)) == 0
+            assert orc.orc_faithful_broadcastTo(dt, hp(a), dx.i32arr(ish), len(ish), dx.i32arr(osh), len(osh), hp(g)) == 0
+            assert np.array_equal(w, g) and np.array_equal(g, np.broadcast_to(a, osh))
+        for axis in (0, 1, 2):
+            parts = [rng.integers(0, 120, size=[3 if axis != 0 else n, 4 if axis != 1 else n, 5 if axis != 2 else n]).astype(npdt) for n in (2, 1, 4)]
+            osh = list(parts[0].shape)
+            osh[axis] = 7
+            w, g = np.empty(osh, dtype=npdt), np.empty(osh, dtype=npdt)
+            ptrs, sizes = dx.ptrarr([a.ctypes.data for a in parts]), dx.i32arr([2, 1, 4])
+            assert orc.orc_concat(dt, ptrs, 3, sizes, dx.i32arr(osh), 3, axis, hp(w)) == 0
+            assert orc.orc_faithful_concat(dt, ptrs, 3, sizes, dx.i32arr(osh), 3, axis, hp(g)) == 0
+            assert np.array_equal(w, g) and np.array_equal(g, np.concatenate(parts, axis=axis))
+        t = rng.integers(0, 120, size=(6, 7, 3)).astype(npdt)
+        for axis, idt, npi in ((0, dx.I64, np.int64), (1, dx.I32, np.int32), (2, dx.I64, np.int64), (-2, dx.I32, np.int32)):
+            ix = rng.integers(0, t.shape[axis], size=(2, 5)).astype(npi)
+            want = np.take(t, ix, axis=axis)
+            w, g = np.empty(want.shape, dtype=npdt), np.empty(want.shape, dtype=npdt)
+            assert orc.orc_indexselect(dt, hp(t), dx.i32arr(t.shape), 3, idt, hp(ix), dx.i32arr(ix.shape), 2, axis, hp(w)) == 0
+            assert orc.orc_faithful_indexselect(dt, hp(t), dx.i32arr(t.shape), 3, idt, hp(ix), dx.i32arr(ix.shape), 2, axis, hp(g)) == 0
+            assert np.array_equal(w, g) and np.array_equal(g, want)
+
+
 def test_concat_reference_expectation(orc):
     g = json.load(open(os.path.join(GOLD, "concat_kat.json")))
     arrs = [np.full(t["shape"], t["fill"], dtype=np.float32) for t in g["inputs"]]

@@ -157,3 +157,46 @@ def test_shape_inference_identical(ref, ex):
             assert ex.infer("reduced", shape, checked, keep) == ref.reduced_shape(shape, checked, keep)
     assert ex.infer("checked_dims", [2, 3], [2]).startswith("error") and ref.checked_dims([2, 3], [2]).startswith("error")
     assert ex.infer("repeat", [2, 3], [2]).startswith("error") and ref.repeat_shape([2, 3], [2]).startswith("error")
+
+
+def test_raw_data_files_both_ways(ref, ex, tmp_path):
+    """A tensor's `.data` file (stdutil/fs.cpp:18-50): what the executor's writer puts down the
+    reference's readers take back byte for byte and the other way round, a size that does not match
+    is refused by both with the same message, and so is a file that is not there."""
+    rng = random.Random(5)
+    for n in (0, 1, 2, 7, 4096, 70001):
+        blob = bytes(rng.getrandbits(8) for _ in range(n))
+        ours, theirs = str(tmp_path / f"ours_{n}.data"), str(tmp_path / f"theirs_{n}.data")
+        assert ex.data_write(ours, blob) == "" and ref.fs_save(theirs, blob) == ""
+        assert open(ours, "rb").read() == blob == open(theirs, "rb").read()
+        assert ref.fs_load(ours, n) == ("", blob) and ex.data_read(theirs, n) == ("", blob)
+        assert ref.fs_load_any(ours, n + 8) == (str(n), blob + b"\0" * 8)
+        for wrong in (n + 1, max(0, n - 1)):
+            if wrong == n:
+                continue
+            r, e = ref.fs_load(ours, wrong)[0], ex.data_read(ours, wrong)[0]
+            assert r == e == "error: file size mismatch: " + ours
+    # a writer call on an existing file empties it first (ios::trunc)
+    path = str(tmp_path / "again.data")
+    assert ex.data_write(path, b"0123456789") == "" and ex.data_write(path, b"ab") == ""
+    assert ref.fs_load(path, 2) == ("", b"ab")
+    assert ref.fs_save(path, b"0123456789") == "" and ref.fs_save(path, b"xyz") == ""
+    assert ex.data_read(path, 3) == ("", b"xyz")
+    missing = str(tmp_path / "nowhere" / "t.data")
+    assert ref.fs_load(missing, 4)[0] == ex.data_read(missing, 4)[0] == "error: Failed to open file: " + missing
+    assert ref.fs_save(missing, b"abcd") == ex.data_write(missing, b"abcd") == "error: Failed to open file for writing: " + missing
+
+
+def test_matmul_shape_rules(ex):
+    """matmul's shape rule.  The reference's own function (shape_matmul.cpp:7-22) compiles but takes Shape
+    objects, whose constructors live in shape.cpp (yaml-cpp: not buildable here), so it cannot be called;
+    these are its three statements written out as cases: both operands at least 2-D, A[-1] == B[-2], result
+    = A's shape with the last extent replaced by B[-1].  The executor also insists on equal batch extents,
+    as check_matmul_shape does (deepxcore tensorfunc/matmul.hpp:9-27: equal rank, equal leading extents)."""
+    assert ex.infer("matmul", [2, 3], [3, 4]) == "2 4"
+    assert ex.infer("matmul", [5, 2, 3], [5, 3, 4]) == "5 2 4"
+    assert ex.infer("matmul", [7, 5, 2, 3], [7, 5, 3, 1]) == "7 5 2 1"
+    assert ex.infer("matmul", [3], [3, 4]) == "error: A and B must >= 2D tensors"
+    assert ex.infer("matmul", [2, 3], [3]) == "error: A and B must >= 2D tensors"
+    assert ex.infer("matmul", [2, 3], [4, 4]) == "error: A[-1] must be equal to B[-2]"
+    assert ex.infer("matmul", [5, 2, 3], [6, 3, 4]).startswith("error: ")

@@ -166,6 +166,11 @@ inline bool stream_is_capturing(hipStream_t st) {
     return cap != hipStreamCaptureStatusNone;
 }
 void reduce_stream_release(hipStream_t st);  // reduce.hip: gives back the stream's slice of finish counters
+// reduce.hip: counters that launches recorded under capture took belong to the graph the capture ends in
+// (nullptr: the capture failed) and return to the pool with it
+void finish_capture_ended(hipStream_t st, const void *graph);
+void finish_graph_destroyed(const void *graph);
+void finish_capture_stats(int64_t *in_use, int64_t *capacity);
 void reduce_device_init();  // reduce.hip: resolves the file-scope device arrays of the current device
 void chain_device_init();   // elementwise.hip: raises the dynamic-LDS limit of the row-form chain kernels on the current device
 

@@ -27,11 +27,11 @@
 namespace dxh {
 
 // One LDS-direct load: lane's 16 bytes from `base + off` land at LDS byte address lds + 16 * lane.
-// M0 is reserved (the compiler never keeps a value in it across statements), so it is not listed
-// as a clobber.  No "memory" clobber either: ordering against the LDS reads comes from the
-// workgroup barriers around it, and the statement is volatile, so it stays between them.
+// The statement writes M0 and says so (the compiler uses M0 itself for dynamically indexed registers
+// and its own LDS-direct accesses).  No "memory" clobber: ordering against the LDS reads comes from
+// the workgroup barriers around it, and the statement is volatile, so it stays between them.
 __device__ __forceinline__ void dma16(const void *base, uint32_t off, uint32_t lds) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds));
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds) : "m0");
 }
 template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N)); }
 

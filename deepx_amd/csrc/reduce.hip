@@ -23,6 +23,7 @@
 // live in a file-scope device array and return to zero, see finish_counters).  Both stage
 // kinds are HBM-bound: algorithmic bytes = input once + output once.
 #include "reduce_order.hpp"
+#include "counter_ranges.hpp"
 #include <map>
 #include <mutex>
 #include <vector>
@@ -273,8 +274,10 @@ __global__ __launch_bounds__(kBlock) void reduce_col_fused_kernel(const Tin *__r
 // Kernels of one stream run in order, so an eager stream owns one slice for as long as it is
 // known here (dxh_stream_destroy gives it back).  A launch recorded under stream capture may
 // later replay on any stream next to eager work, so it takes counters of its own from the
-// second half of the array, never handed out twice; when either half is used up the caller
-// falls back to two launches.
+// second half of the array: they belong to the graph that the capture ends in and return to the
+// pool when that graph is destroyed (counter_ranges.hpp; dxh_graph_end_capture and
+// dxh_graph_destroy report both events here).  When either half is used up the caller falls back
+// to two launches.
 constexpr int kFinishSlice = 1024, kFinishSlices = 32, kFinishCounters = 2 * kFinishSlice * kFinishSlices;
 static __device__ __align__(256) unsigned g_finish_counters[kFinishCounters];
 namespace {
@@ -284,7 +287,7 @@ struct FinishState {
     std::map<hipStream_t, int> slice;
     std::vector<int> free_slices;
     int slices_used = 0;
-    int64_t capture_next = (int64_t)kFinishSlice * kFinishSlices;
+    CounterRanges captured{(int64_t)kFinishSlice * kFinishSlices, kFinishCounters};
 };
 std::mutex g_finish_mutex;
 std::map<int, FinishState> g_finish;  // by device
@@ -306,10 +309,8 @@ unsigned *finish_counters(hipStream_t st, int64_t need) {
     }
     if (!f.base) return nullptr;
     if (capturing) {
-        if (f.capture_next + need > kFinishCounters) return nullptr;
-        unsigned *r = f.base + f.capture_next;
-        f.capture_next += need;
-        return r;
+        const int64_t off = f.captured.take_for_capture((const void *)st, need);
+        return off < 0 ? nullptr : f.base + off;
     }
     auto it = f.slice.find(st);
     if (it == f.slice.end()) {
@@ -320,6 +321,28 @@ unsigned *finish_counters(hipStream_t st, int64_t need) {
         it = f.slice.emplace(st, idx).first;
     }
     return f.base + (int64_t)it->second * kFinishSlice;
+}
+
+// graph == nullptr: the capture on `st` failed and no graph will ever replay its launches
+void finish_capture_ended(hipStream_t st, const void *graph) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return; }
+    std::lock_guard<std::mutex> lock(g_finish_mutex);
+    auto d = g_finish.find(dev);
+    if (d != g_finish.end()) d->second.captured.capture_ended((const void *)st, graph);
+}
+void finish_graph_destroyed(const void *graph) {
+    std::lock_guard<std::mutex> lock(g_finish_mutex);
+    for (auto &d : g_finish) d.second.captured.graph_destroyed(graph);
+}
+void finish_capture_stats(int64_t *in_use, int64_t *capacity) {
+    int dev = 0;
+    *in_use = 0;
+    *capacity = (int64_t)kFinishCounters - (int64_t)kFinishSlice * kFinishSlices;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return; }
+    std::lock_guard<std::mutex> lock(g_finish_mutex);
+    auto d = g_finish.find(dev);
+    if (d != g_finish.end()) *in_use = d->second.captured.in_use();
 }
 
 void reduce_stream_release(hipStream_t st) {

@@ -16,7 +16,7 @@ Tuning &tuning() {
 
 extern "C" {
 
-int dxh_version(void) { return 100; }
+int dxh_version(void) { return DXH_ABI_VERSION; }
 
 int dxh_tune(int knob, int64_t value) {
     Tuning &t = tuning();
@@ -172,12 +172,15 @@ int dxh_graph_end_capture(void *stream, void **graph_exec) {
     hipError_t e = hipStreamEndCapture(as_stream(stream), &graph);
     if (e != hipSuccess || !graph) {
         (void)hipGetLastError();
+        dxh::finish_capture_ended(as_stream(stream), nullptr);
         return e != hipSuccess ? (int)e : DXH_ERR_ARG;
     }
     hipGraphExec_t exec = nullptr;
     e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
-    if (e != hipSuccess) return (int)e;
+    if (e != hipSuccess) { dxh::finish_capture_ended(as_stream(stream), nullptr); return (int)e; }
+    // the in-launch counters its recorded launches took stay with the graph until dxh_graph_destroy
+    dxh::finish_capture_ended(as_stream(stream), (const void *)exec);
     *graph_exec = (void *)exec;
     return DXH_OK;
 }
@@ -185,6 +188,16 @@ int dxh_graph_launch(void *graph_exec, void *stream) {
     if (!graph_exec || !stream) return DXH_ERR_ARG;
     return (int)hipGraphLaunch((hipGraphExec_t)graph_exec, as_stream(stream));
 }
-int dxh_graph_destroy(void *graph_exec) { return graph_exec ? (int)hipGraphExecDestroy((hipGraphExec_t)graph_exec) : DXH_OK; }
+int dxh_graph_destroy(void *graph_exec) {
+    if (!graph_exec) return DXH_OK;
+    const hipError_t e = hipGraphExecDestroy((hipGraphExec_t)graph_exec);
+    dxh::finish_graph_destroyed(graph_exec);
+    return (int)e;
+}
+int dxh_graph_counter_stats(int64_t *in_use, int64_t *capacity) {
+    if (!in_use || !capacity) return DXH_ERR_ARG;
+    dxh::finish_capture_stats(in_use, capacity);
+    return DXH_OK;
+}
 
 }  // extern "C"

@@ -49,6 +49,9 @@ public:
     struct Profile { uint64_t lines = 0, parse_ns = 0, match_ns = 0, run_ns = 0, sync_ns = 0, reply_ns = 0; } prof;
 
     Executor() {
+        // the kernel library found at run time must be the one this host code was compiled against
+        if (dxh_version() != DXH_ABI_VERSION)
+            throw std::runtime_error("libdxhip.so has ABI " + std::to_string(dxh_version()) + ", this executor was built for " + std::to_string(DXH_ABI_VERSION));
         register_all(factory);
         const char *e = std::getenv("DEEPX_IR_LOG");
         ir_log = e && (!std::strcmp(e, "1") || !strcasecmp(e, "true"));

@@ -657,17 +657,24 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
             const std::string &name = tensors[side]->textvalue;
             auto t = mem.findtensor(name);
             if (!t || !is_float(t->dtype())) { ok = false; break; }
-            const int extent = extent_of(*t);
+            // A tensor that the run produced has the extent its producing line gave it; only a tensor read
+            // from memory is classified by its shape.  The two differ on a square view, where the [rows]
+            // result of a row sum without keepdims is a column to the run and looks like a row by shape;
+            // a line on such a vector follows its operand.
+            int produced_by = -1;
+            for (size_t j = ops.size(); j-- > 0;)
+                if (ops[j].out_name == name) { produced_by = (int)j; break; }
+            const int extent = produced_by >= 0 ? ops[produced_by].op.extent : extent_of(*t);
             if (extent < 0) { ok = false; break; }
+            if (kind != kChainBroadcast && kind != kChainSum && extent != DXH_CHAIN_FULL && rows == cols && out->shape.dim() == 1 && out->shape.size == rows)
+                op.op.extent = extent;
             // what the line itself would refuse: another dtype (but for todtype), another size (but for broadcastTo)
             if (kind != kChainTodtype && t->dtype() != out->dtype()) { ok = false; break; }
             if (kind == kChainSum && extent != DXH_CHAIN_FULL) { ok = false; break; }
             if (kind != kChainBroadcast && kind != kChainSum && (extent != op.op.extent || t->shape.size != out->shape.size)) { ok = false; break; }
             if (kind == kChainBroadcast && broadcast_shape(t->shape.shape, out->shape.shape) != out->shape.shape) { ok = false; break; }
             line_needs_rows = line_needs_rows || extent != DXH_CHAIN_FULL || t->dtype() != out->dtype();
-            int ref = -1;
-            for (size_t j = ops.size(); j-- > 0;)
-                if (ops[j].out_name == name) { ref = DXH_CHAIN_RESULT + (int)j; break; }
+            int ref = produced_by >= 0 ? DXH_CHAIN_RESULT + produced_by : -1;
             if (ref < 0) {
                 for (size_t j = 0; j < inputs.size() && ref < 0; ++j) if (inputs[j].name == name) ref = (int)j;
                 for (size_t j = 0; j < new_inputs.size() && ref < 0; ++j) if (new_inputs[j].name == name) ref = (int)(inputs.size() + j);

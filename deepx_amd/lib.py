@@ -69,6 +69,8 @@ _RSCL = [_i, Scalar, _p, _p, _i64, _p]
 _UN = [_i, _p, _p, _i64, _p]
 _RED = [_i, _p, _pi32, _i, _pi32, _i, _p, _p, _sz, _p]
 
+ABI_VERSION = 200  # DXH_ABI_VERSION of include/dxhip.h, the layout SIGNATURES below describes
+
 SIGNATURES = {
     "dxh_version": ([], _i),
     "dxh_error_string": ([_i], C.c_char_p),
@@ -97,6 +99,7 @@ SIGNATURES = {
     "dxh_graph_end_capture": ([_p, C.POINTER(_p)], _i),
     "dxh_graph_launch": ([_p, _p], _i),
     "dxh_graph_destroy": ([_p], _i),
+    "dxh_graph_counter_stats": ([C.POINTER(_i64), C.POINTER(_i64)], _i),
     "dxh_add": (_BIN, _i), "dxh_sub": (_BIN, _i), "dxh_mul": (_BIN, _i), "dxh_div": (_BIN, _i),
     "dxh_max": (_BIN, _i), "dxh_min": (_BIN, _i), "dxh_pow": (_BIN, _i),
     "dxh_addscalar": (_SCL, _i), "dxh_subscalar": (_SCL, _i), "dxh_rsubscalar": (_RSCL, _i),
@@ -156,6 +159,9 @@ def load(path=None):
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported
         fn.argtypes = argtypes
         fn.restype = restype
+    got = lib.dxh_version()
+    if got != ABI_VERSION:
+        raise DxhError(f"{p} was built for ABI {got}, these bindings are written for {ABI_VERSION} (DXH_ABI_VERSION in include/dxhip.h): rebuild it")
     if path is None:
         _lib = lib
     return lib

@@ -82,6 +82,13 @@ typedef struct dxh_scalar {
 
 /* ---- runtime: replaces cudaMalloc/cudaFree/cudaMemcpy of
  * executor/op-cuda/src/deepx/tensorfunc/tensorlife_miaobyte.hpp:16-68 ---------- */
+/* The number a caller was compiled against; dxh_version() returns the one the loaded library was
+ * built with.  It changes whenever an existing entry point changes its arguments or meaning
+ * (additions keep it): 100 = first layout; 200 = dxh_matmul takes `workspace, workspace_bytes`
+ * before `stream`, DXH_TUNE_MATMUL_TILE ranges 0..15.  A caller checks for equality once, at
+ * load, and refuses to go on otherwise (a stream passed where a workspace is expected would be
+ * dereferenced as memory). */
+#define DXH_ABI_VERSION 200
 DXH_API int dxh_version(void);
 DXH_API const char *dxh_error_string(int code);
 /* Launch-heuristic knobs (process wide; results never depend on them, only speed).
@@ -158,6 +165,12 @@ DXH_API int dxh_graph_begin_capture(void *stream);
 DXH_API int dxh_graph_end_capture(void *stream, void **graph_exec);
 DXH_API int dxh_graph_launch(void *graph_exec, void *stream);
 DXH_API int dxh_graph_destroy(void *graph_exec);
+/* Recorded launches that finish a reduction or a K-cut matmul inside one launch own counters of
+ * the library's device array for as long as their graph lives; dxh_graph_destroy (on a graph that
+ * has finished running) and a failed capture give them back.  Reports how many are taken and how
+ * many there are on the current device; with none left such launches are recorded in their
+ * two-launch form, which gives the same bits more slowly. */
+DXH_API int dxh_graph_counter_stats(int64_t *in_use, int64_t *capacity);
 
 /* ---- elementwise, C[i] = A[i] op B[i]
  * launch_add/sub/mul/div  elementwise_miaobyte_basic.cuh:16-98

@@ -24,7 +24,9 @@ def test_library_exports_every_declared_symbol():
     L = dx.load()  # raises if the library is not built or a symbol is missing
     for name in declared():
         assert hasattr(L, name), name
-    assert L.dxh_version() >= 100
+    # the header's macro, the bindings' constant and the built library agree
+    macro = int(re.search(r"#define\s+DXH_ABI_VERSION\s+(\d+)", open(os.path.join(ROOT, "include", "dxhip.h")).read()).group(1))
+    assert L.dxh_version() == macro == dx.ABI_VERSION
     assert L.dxh_error_string(-1).decode().startswith("dtype")
     assert L.dxh_error_string(0).decode() == "ok"
 

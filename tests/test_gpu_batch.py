@@ -369,7 +369,9 @@ def test_config5_block_at_full_size_in_every_mode(tmp_path):
     h_ref = rb(b2f(w).astype(np.float64) * xn)
     g = rb(h_ref @ b2f(Wg).astype(np.float64)); u = rb(h_ref @ b2f(Wu).astype(np.float64))
     act = rb(rb(g * rb(1.0 / rb(1.0 + rb(np.exp(rb(-g)))))) * u)
-    y_ref = act @ b2f(Wd).astype(np.float64)
+    Wd64 = b2f(Wd).astype(np.float64)
+    y_ref = act @ Wd64
+    y_mag = np.abs(act) @ np.abs(Wd64)
 
     b16, f32 = "bfloat16", "float32"
     n = lambda name, dt=f32: T("f5_" + name, dt)
@@ -426,6 +428,20 @@ def test_config5_block_at_full_size_in_every_mode(tmp_path):
         hh = b2f(kept[mode]["h"]).astype(np.float64)
         assert np.abs(y - y_ref).max() <= 3e-2 * np.abs(y_ref).max(), mode
         assert np.abs(hh - h_ref).max() <= 1e-2 * np.abs(h_ref).max(), mode
+        # element by element as well: every output against the model within 1e-2 of the magnitude that
+        # went into it (sum_k |act||Wd| for the GEMM, the value itself for the normalised activations) ...
+        assert np.all(np.abs(y - y_ref) <= 1e-2 * y_mag), (mode, float(np.max(np.abs(y - y_ref) / y_mag)))
+        assert np.all(np.abs(hh - h_ref) <= 1e-2 * np.abs(h_ref) + 1e-30), mode
+        # ... and every stage against the model applied to the stage's own inputs as the device left them
+        if mode == "lines":
+            gd, ud, sgd = (b2f(kept[mode][k]).astype(np.float64) for k in ("g", "u", "sg"))
+            Wg64, Wu64 = b2f(Wg).astype(np.float64), b2f(Wu).astype(np.float64)
+            assert np.all(np.abs(gd - hh @ Wg64) <= 1e-2 * (np.abs(hh) @ np.abs(Wg64)))
+            assert np.all(np.abs(ud - hh @ Wu64) <= 1e-2 * (np.abs(hh) @ np.abs(Wu64)))
+            sg_model = rb(rb(gd * rb(1.0 / rb(1.0 + rb(np.exp(rb(-gd)))))) * ud)
+            # five bf16 roundings; a 4-ulp exp or a double rounding may move one of them by one bf16 step
+            assert np.all(np.abs(sgd - sg_model) <= 2.0 ** -6 * np.abs(sg_model) + 1e-37)
+            assert np.all(np.abs(y - sgd @ Wd64) <= 1e-2 * (np.abs(sgd) @ np.abs(Wd64)))
         del ex
     for mode in ("batch", "batch_fused", "graph", "graph_fused"):
         for k in kept["lines"]:
@@ -502,3 +518,77 @@ def test_random_batches_fused_equal_line_by_line(tmp_path):
                 same = np.array_equal(fa, fb, equal_nan=True)
             assert same, (trial, name, lines)
     assert fused_lines > 400  # the batches did form runs
+
+
+def test_square_view_row_sum_without_keepdims_fuses(tmp_path):
+    """On a square [N, N] view the [N] result of a row sum without keepdims looks like a row by its shape
+    and is a column to the run that produced it: lines that go on with it stay in the run (one launch)
+    and leave the bits of the line-by-line execution."""
+    ex = InProc()
+    h = Host(ex, tmp_path)
+    rng = np.random.default_rng(47)
+    N = 128
+    h.put("q_x", rng.standard_normal((N, N)).astype(np.float32))
+    for name, shape in (("q_sq", [N, N]), ("q_s", [N]), ("q_m", [N]), ("q_r", [N])):
+        h.run(f"newtensor({V(shape)})->({T(name)})")
+    lines = [f"powscalar({T('q_x')}, var<float32>:2)->({T('q_sq')}) // author=miaobyte id=1",
+             f"sum({T('q_sq')}, {V([-1])}, var<bool>:false)->({T('q_s')}) // author=miaobyte id=2",
+             f"divscalar({T('q_s')}, var<float32>:{N})->({T('q_m')}) // author=miaobyte id=3",
+             f"sqrt({T('q_m')})->({T('q_r')}) // author=miaobyte id=4",
+             f"mul({T('q_r')}, {T('q_s')})->({T('q_r')}) // author=miaobyte id=5"]
+    ex.set_fusion(False)
+    assert all(r.split(" ")[1].startswith("ok") for r in ex.execute_batch(lines))
+    want = {n: h.get(n) for n in ("q_sq", "q_s", "q_m", "q_r")}
+    x = h.get("q_x").astype(np.float64)
+    assert np.allclose(want["q_r"], np.sqrt((x ** 2).sum(-1) / N) * (x ** 2).sum(-1), rtol=1e-5)
+    for n in want:
+        h.run(f"constant(var<float32>:0)->({T(n)})")
+    ex.set_fusion(True)
+    before = ex.fusion_stats()
+    assert all(r.split(" ")[1].startswith("ok") for r in ex.execute_batch(lines))
+    after = ex.fusion_stats()
+    assert after["runs"] - before["runs"] == 1 and after["lines"] - before["lines"] == 5, (before, after)
+    for n in want:
+        assert np.array_equal(h.get(n).view(np.uint32), want[n].view(np.uint32)), n
+
+
+def test_recorded_graphs_return_their_counters(dxh, tmp_path):
+    """Launches recorded under capture that finish inside one launch (strided-axis sum) own counters of
+    the library's array while their graph lives: recording and destroying many graphs leaves none taken."""
+    import ctypes as C
+    import torch
+    L = dxh
+    used, cap = C.c_int64(), C.c_int64()
+    dx.check(L.dxh_graph_counter_stats(C.byref(used), C.byref(cap)))
+    start = used.value
+    x = torch.randn(2048, 1024, device="cuda")
+    out = torch.empty(1024, device="cuda")
+    want = torch.empty(1024, device="cuda")
+    shape, ax0 = dx.i32arr([2048, 1024]), dx.i32arr([0])
+    need = C.c_size_t(0)
+    dx.check(L.dxh_reduce_workspace_bytes(dx.F32, shape, 2, ax0, 1, C.byref(need)))
+    ws = torch.empty(max(1, need.value), dtype=torch.uint8, device="cuda")
+    p = lambda t: C.c_void_p(t.data_ptr())
+    dx.check(L.dxh_sum(dx.F32, p(x), shape, 2, ax0, 1, p(want), p(ws), need.value, None))
+    torch.cuda.synchronize()
+    st = C.c_void_p()
+    dx.check(L.dxh_stream_create(C.byref(st)))
+    peak = 0
+    for i in range(300):  # far more recordings than the array could serve without returns (32 Ki counters)
+        dx.check(L.dxh_graph_begin_capture(st))
+        for _ in range(4):
+            dx.check(L.dxh_sum(dx.F32, p(x), shape, 2, ax0, 1, p(out), p(ws), need.value, st))
+        g = C.c_void_p()
+        dx.check(L.dxh_graph_end_capture(st, C.byref(g)))
+        dx.check(L.dxh_graph_counter_stats(C.byref(used), C.byref(cap)))
+        peak = max(peak, used.value - start)
+        if i % 50 == 0:
+            out.zero_()
+            dx.check(L.dxh_graph_launch(g, st))
+            dx.check(L.dxh_stream_sync(st))
+            assert torch.equal(out, want)
+        dx.check(L.dxh_graph_destroy(g))
+        dx.check(L.dxh_graph_counter_stats(C.byref(used), C.byref(cap)))
+        assert used.value == start, (i, used.value, start)
+    assert 0 < peak <= 4 * 1024 and cap.value >= 32 * 1024
+    dx.check(L.dxh_stream_destroy(st))

@@ -282,8 +282,12 @@ def test_config5_mlp_block_over_ir(srv, tmp_path):
     act = rb(rb(g * rb(1.0 / rb(1.0 + rb(np.exp(rb(-g)))))) * u)
     yref = act @ b2f(Wd).astype(np.float64)
     assert np.abs(y - yref).max() <= 3e-2 * np.abs(yref).max()
+    # element by element: within 1e-2 of the magnitude that went into each output
+    ymag = np.abs(act) @ np.abs(b2f(Wd).astype(np.float64))
+    assert np.all(np.abs(y - yref) <= 1e-2 * ymag), float(np.max(np.abs(y - yref) / ymag))
     hg = b2f(fetch(srv, tmp_path, "q5_h")[0]).astype(np.float64)
     assert np.abs(hg - h).max() <= 1e-2 * np.abs(h).max()
+    assert np.all(np.abs(hg - h) <= 1e-2 * np.abs(h) + 1e-30)
 
 
 def test_benchmark_repeat_and_timestamps(srv, tmp_path):

@@ -58,6 +58,10 @@ def main():
                     help="run only the bf16 matmul of that shape, --steps launches after a clock ramp "
                          "(the program a counter collection wraps) and print its own JSON line")
     ap.add_argument("--matmul-tile", type=int, default=0, help="with --matmul-only: force a workgroup tile (DXH_TUNE_MATMUL_TILE), 0 = chosen per shape")
+    ap.add_argument("--chain-only", metavar="RUN", default="",
+                    help="run only one fused run (a label of per_op.config5.fused_runs, or a prefix of one), --steps launches after a "
+                         "clock ramp (the program a counter collection wraps) and print its own JSON line")
+    ap.add_argument("--chain-static", type=int, default=1, help="with --chain-only: 1 = the library's compiled kernel, 0 = the interpreting kernel")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this executor path runs on ONE GPU (no sharding, no collectives); "
@@ -117,6 +121,27 @@ def main():
         ms = Events.ms(a, b) / args.steps
         print(json.dumps({"matmul_bf16": args.matmul_only, "tile_knob": args.matmul_tile, "launches": args.steps, "us_per_launch": round(ms * 1e3, 2),
                           "TFLOP/s": round(2 * mm * kk * nn / ms / 1e9, 1), "frac_mfma_bf16": round(2 * mm * kk * nn / ms / 1e9 / MFMA_BF16_PEAK_TF, 4),
+                          "device": name.value.decode()}))
+        return
+
+    if args.chain_only:
+        runs = fused_run_calls(L, dx, torch, dev)
+        label = [k for k in runs if k.startswith(args.chain_only)][0]
+        calls, nbytes = runs[label]
+        dx.check(L.dxh_tune(12, args.chain_static), "DXH_TUNE_CHAIN_STATIC")
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < args.ramp_ms:
+            dx.check(calls[0](), label)
+            dx.check(L.dxh_device_sync())
+        a, b = Events().pair()
+        dx.check(L.dxh_event_record(a, None))
+        for i in range(args.steps):
+            dx.check(calls[i % len(calls)](), label)
+        dx.check(L.dxh_event_record(b, None))
+        dx.check(L.dxh_event_sync(b))
+        ms = Events.ms(a, b) / args.steps
+        print(json.dumps({"fused_run": label, "compiled_kernel": bool(args.chain_static), "launches": args.steps, "us_per_launch": round(ms * 1e3, 2),
+                          "GB/s": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes,
                           "device": name.value.decode()}))
         return
 
@@ -443,42 +468,90 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
         "broadcastTo_f32_2048x1_to_2048x896": (lambda i: L.dxh_broadcastTo(dx.F32, ptr(col[i % R6]), shc, 2, shb, 2, ptr(o32[i % R6]), None), n32 * 4 + S * 4),
     }
     c5["glue_ops(cache-resident sizes)"] = {k: entry(time_op(L, dx, torch, Events, ev, fn), nb) for k, (fn, nb) in glue.items()}
-    # the same glue as the executor's batch path launches it: the RMSNorm's thirteen lines (row sum included) and the
-    # SiLU gate's six lines, one launch each (dxh_chain_rows / dxh_chain); bytes = inputs once + every tensor the lines store
-    FULL, ROW, COL, RES = dx.CHAIN_FULL, dx.CHAIN_ROW, dx.CHAIN_COLUMN, dx.CHAIN_RESULT
-    w16 = torch.ones(Hd, device=dev, dtype=torch.bfloat16)
-    f32s = [[torch.empty(S * Hd, device=dev) for _ in range(5)] for _ in range(R6)]  # xf sq rs wf xn
-    wf1 = torch.empty(Hd, device=dev)
-    h16 = [torch.empty(S * Hd, device=dev, dtype=torch.bfloat16) for _ in range(R6)]
-    code = dx.CHAIN_CODES.index
-    def norm_run(i):
-        xf, sq, rs, wf, xn = f32s[i]
-        prog = [("copy", 0, 0, 0, dx.F32, FULL, xf), ("square", RES + 0, 0, 2.0, dx.F32, FULL, sq), ("rowsum", RES + 1, 0, 0, dx.F32, COL, None),
-                ("divscalar", RES + 2, 0, float(Hd), dx.F32, COL, None), ("addscalar", RES + 3, 0, 1e-6, dx.F32, COL, None),
-                ("sqrt", RES + 4, 0, 0, dx.F32, COL, None), ("rdivscalar", RES + 5, 0, 1.0, dx.F32, COL, col[i]),
-                ("copy", RES + 6, 0, 0, dx.F32, FULL, rs), ("mul", RES + 0, RES + 7, 0, dx.F32, FULL, None), ("copy", 1, 0, 0, dx.F32, ROW, wf1),
-                ("copy", RES + 9, 0, 0, dx.F32, FULL, wf), ("mul", RES + 10, RES + 8, 0, dx.F32, FULL, xn), ("copy", RES + 11, 0, 0, dx.BF16, FULL, h16[i])]
-        tin = (dx.ChainTensor * 2)(dx.ChainTensor(x16[i].data_ptr(), dx.BF16, FULL), dx.ChainTensor(w16.data_ptr(), dx.BF16, ROW))
-        ops = (dx.ChainRowsOp * len(prog))(*[dx.ChainRowsOp(code(n), l, r, dx.scalar(sc), o.data_ptr() if o is not None else None, dt, e)
-                                             for n, l, r, sc, dt, e, o in prog])
-        return lambda: L.dxh_chain_rows(tin, 2, ops, len(prog), S, Hd, None)
-    def gate_run(i):
-        prog = [("mulscalar", 0, 0, -1.0), ("exp", RES + 0, 0, 0), ("addscalar", RES + 1, 0, 1.0), ("rdivscalar", RES + 2, 0, 1.0), ("mul", 0, RES + 3, 0), ("mul", RES + 4, 1, 0)]
-        ops = (dx.ChainOp * len(prog))(*[dx.ChainOp(code(n), l, r, dx.scalar(sc), o16[i].data_ptr() if k == len(prog) - 1 else None) for k, (n, l, r, sc) in enumerate(prog)])
-        ins = (C.c_void_p * 2)(g16[i].data_ptr(), u16[i].data_ptr())
-        return lambda: L.dxh_chain(dx.BF16, ins, 2, ops, len(prog), n16, None)
-    norm_calls, gate_calls = [norm_run(i) for i in range(R6)], [gate_run(i) for i in range(R6)]
-    c5["fused_runs(one launch each)"] = {
-        "rmsnorm_13_lines_bf16_in_f32_inside_2048x896": entry(time_op(L, dx, torch, Events, ev, lambda i: norm_calls[i % R6]()), n32 * 2 + 5 * n32 * 4 + n32 * 2 + S * 4 + Hd * 6),
-        "silu_gate_6_lines_bf16_2048x4864": entry(time_op(L, dx, torch, Events, ev, lambda i: gate_calls[i % R6]()), 3 * n16 * 2),
-        "note": "bound by instruction issue (an op interpreter; correctly rounded exp and division, one rounding per op), not by these bytes; "
-                "as separate launches the same lines take the sum of the glue_ops entries above, 10 and 6 launches"}
+    # the same glue as the executor's batch path launches it: the RMSNorm's thirteen lines (row sum included), the
+    # SiLU gate's six lines and the softmax's eight lines, one launch each (dxh_chain_rows / dxh_chain); bytes =
+    # inputs once + every tensor the lines store.  Each run has a compiled kernel in the library; the same
+    # launches through the interpreting kernel (DXH_TUNE_CHAIN_STATIC 0) are timed beside them.
+    runs = fused_run_calls(L, dx, torch, dev, R6)
+    fused = {}
+    for label, (calls, nbytes) in runs.items():
+        e = entry(time_op(L, dx, torch, Events, ev, lambda i: calls[i % len(calls)]()), nbytes)
+        dx.check(L.dxh_tune(12, 0))
+        try:
+            probe = calls[0]()
+            if probe == 0:
+                e["interpreted_ms"] = round(time_op(L, dx, torch, Events, ev, lambda i: calls[i % len(calls)]()), 5)
+            else:
+                e["interpreted_ms"] = None  # rows too long (or 16-bit row reductions) for the interpreting kernel's lane layout
+        finally:
+            dx.check(L.dxh_tune(12, 1))
+        fused[label] = e
+    fused["note"] = ("one launch per run through the library's compiled kernel for that sequence; interpreted_ms = the same launch through "
+                     "the op-table interpreter; as separate launches the lines take the sum of the glue_ops entries above")
+    c5["fused_runs(one launch each)"] = fused
+    del runs
     del g16, u16, o16, x16, x32, o32, col
     torch.cuda.empty_cache()
     c5["mlp_block_over_deepxIR"] = config5_block_over_ir()
     res["config1"]["chain_over_deepxIR"] = config1_chain_over_ir()
     res["config5"] = c5
     return res
+
+
+def fused_run_calls(L, dx, torch, dev, sets=6):
+    """The front's three fixed sequences as single launches on rotating buffer sets: {label: ([call, ...], bytes)}.
+    Each call returns the entry point's status."""
+    import ctypes as C
+    S, Hd, I = 2048, 896, 4864
+    FULL, ROW, COL, RES = dx.CHAIN_FULL, dx.CHAIN_ROW, dx.CHAIN_COLUMN, dx.CHAIN_RESULT
+    code = dx.CHAIN_CODES.index
+    n16, n32 = S * I, S * Hd
+    keep = []  # tensors stay alive as long as the calls do
+
+    def norm_run():
+        x16 = torch.randn(n32, device=dev).to(torch.bfloat16)
+        w16 = torch.ones(Hd, device=dev, dtype=torch.bfloat16)
+        xf, sq, rs, wf, xn = (torch.empty(n32, device=dev) for _ in range(5))
+        wf1, col, h16 = torch.empty(Hd, device=dev), torch.empty(S, device=dev), torch.empty(n32, device=dev, dtype=torch.bfloat16)
+        keep.extend([x16, w16, xf, sq, rs, wf, xn, wf1, col, h16])
+        prog = [("copy", 0, 0, 0, dx.F32, FULL, xf), ("square", RES + 0, 0, 2.0, dx.F32, FULL, sq), ("rowsum", RES + 1, 0, 0, dx.F32, COL, None),
+                ("divscalar", RES + 2, 0, float(Hd), dx.F32, COL, None), ("addscalar", RES + 3, 0, 1e-6, dx.F32, COL, None),
+                ("sqrt", RES + 4, 0, 0, dx.F32, COL, None), ("rdivscalar", RES + 5, 0, 1.0, dx.F32, COL, col),
+                ("copy", RES + 6, 0, 0, dx.F32, FULL, rs), ("mul", RES + 0, RES + 7, 0, dx.F32, FULL, None), ("copy", 1, 0, 0, dx.F32, ROW, wf1),
+                ("copy", RES + 9, 0, 0, dx.F32, FULL, wf), ("mul", RES + 10, RES + 8, 0, dx.F32, FULL, xn), ("copy", RES + 11, 0, 0, dx.BF16, FULL, h16)]
+        tin = (dx.ChainTensor * 2)(dx.ChainTensor(x16.data_ptr(), dx.BF16, FULL), dx.ChainTensor(w16.data_ptr(), dx.BF16, ROW))
+        ops = (dx.ChainRowsOp * len(prog))(*[dx.ChainRowsOp(code(n), l, r, dx.scalar(sc), o.data_ptr() if o is not None else None, dt, e)
+                                             for n, l, r, sc, dt, e, o in prog])
+        return lambda: L.dxh_chain_rows(tin, 2, ops, len(prog), S, Hd, None)
+
+    def gate_run():
+        g16, u16 = (torch.randn(n16, device=dev).to(torch.bfloat16) for _ in range(2))
+        o16 = torch.empty(n16, device=dev, dtype=torch.bfloat16)
+        keep.extend([g16, u16, o16])
+        prog = [("mulscalar", 0, 0, -1.0), ("exp", RES + 0, 0, 0), ("addscalar", RES + 1, 0, 1.0), ("rdivscalar", RES + 2, 0, 1.0), ("mul", 0, RES + 3, 0), ("mul", RES + 4, 1, 0)]
+        ops = (dx.ChainOp * len(prog))(*[dx.ChainOp(code(n), l, r, dx.scalar(sc), o16.data_ptr() if k == len(prog) - 1 else None) for k, (n, l, r, sc) in enumerate(prog)])
+        ins = (C.c_void_p * 2)(g16.data_ptr(), u16.data_ptr())
+        return lambda: L.dxh_chain(dx.BF16, ins, 2, ops, len(prog), n16, None)
+
+    def softmax_run(rows, cols, dt, tdt):
+        t = (torch.randn(rows * cols, device=dev) * 3).to(tdt)
+        full = [torch.empty(rows * cols, device=dev, dtype=tdt) for _ in range(6)]  # mb d e e2 sb y
+        cols_ = [torch.empty(rows, device=dev, dtype=tdt) for _ in range(2)]        # m s
+        keep.extend([t] + full + cols_)
+        mb, d, e, e2, sb, y = full
+        prog = [("rowmax", 0, 0, COL, cols_[0]), ("copy", RES + 0, 0, FULL, mb), ("sub", 0, RES + 1, FULL, d), ("exp", RES + 2, 0, FULL, e),
+                ("rowsum", RES + 3, 0, COL, cols_[1]), ("exp", RES + 2, 0, FULL, e2), ("copy", RES + 4, 0, FULL, sb), ("div", RES + 5, RES + 6, FULL, y)]
+        tin = (dx.ChainTensor * 1)(dx.ChainTensor(t.data_ptr(), dt, FULL))
+        ops = (dx.ChainRowsOp * len(prog))(*[dx.ChainRowsOp(code(n), l, r, dx.scalar(0.0), o.data_ptr(), dt, ext) for n, l, r, ext, o in prog])
+        return lambda: L.dxh_chain_rows(tin, 1, ops, len(prog), rows, cols, None)
+
+    AR, AC = 14 * 2048, 2048  # scores of one sequence of the attention shape of config 3: 14 heads x 2048 queries x 2048 keys
+    return {
+        "rmsnorm_13_lines_bf16_in_f32_inside_2048x896": ([norm_run() for _ in range(sets)], n32 * 2 + 5 * n32 * 4 + n32 * 2 + S * 4 + Hd * 6),
+        "silu_gate_6_lines_bf16_2048x4864": ([gate_run() for _ in range(sets)], 3 * n16 * 2),
+        "softmax_8_lines_f32_28672x2048": ([softmax_run(AR, AC, dx.F32, torch.float32) for _ in range(2)], 7 * AR * AC * 4 + 2 * AR * 4),
+        "softmax_8_lines_bf16_2048x896": ([softmax_run(S, Hd, dx.BF16, torch.bfloat16) for _ in range(sets)], 7 * S * Hd * 2 + 2 * S * 2),
+    }
 
 
 def matmul_call(L, dx, torch, dev, dtype, A, B, Cm, m, k, n):

@@ -157,6 +157,7 @@ struct Tuning {
     int64_t skinny_min_rows = 256;                // DXH_TUNE_SKINNY_MIN_ROWS
     int64_t skinny_half = 0;                      // DXH_TUNE_SKINNY_HALF
     int64_t reduce_fused_finish = 1;              // DXH_TUNE_REDUCE_FUSED_FINISH
+    int64_t chain_static = 1;                     // DXH_TUNE_CHAIN_STATIC
 };
 Tuning &tuning();  // runtime.hip
 

@@ -7,55 +7,14 @@
 // tensorfunc/elementwise_miaobyte.hpp (cited per op in include/dxhip.h); 16-bit floats
 // compute in fp32 and round once.
 #include "reduce_order.hpp"
+#include "elementwise_ops.hpp"
+#include "chain_static.hpp"
 #include <mutex>
 
 namespace dxh {
 
 constexpr int kUnroll = 4;       // vectors in flight per lane and operand (3-stream add: 6.42 TB/s against 6.25 with 1)
 constexpr int kBlocksPerCU = 0;  // 0 = one tile per workgroup (see stream_grid)
-
-// ---- op functors on the accumulate type -----------------------------------------------
-template <typename A> __device__ inline A wrap_add(A a, A b) { using U = std::make_unsigned_t<A>; return A(U(U(a) + U(b))); }
-template <typename A> __device__ inline A wrap_sub(A a, A b) { using U = std::make_unsigned_t<A>; return A(U(U(a) - U(b))); }
-template <typename A> __device__ inline A wrap_mul(A a, A b) {
-    using U = std::conditional_t<(sizeof(A) < 4), uint32_t, std::make_unsigned_t<A>>;
-    return A(U(U(a) * U(b)));
-}
-template <typename A> __device__ inline A wrap_div(A a, A b) {
-    if (b == 0) return A(0);
-    if (b == A(-1)) return wrap_sub<A>(A(0), a);
-    return A(a / b);
-}
-
-struct OpAdd { template <typename A> __device__ static A f(A a, A b) { if constexpr (std::is_integral_v<A>) return wrap_add(a, b); else return a + b; } };
-struct OpSub { template <typename A> __device__ static A f(A a, A b) { if constexpr (std::is_integral_v<A>) return wrap_sub(a, b); else return a - b; } };
-struct OpRSub { template <typename A> __device__ static A f(A a, A b) { return OpSub::f(b, a); } };
-struct OpMul { template <typename A> __device__ static A f(A a, A b) { if constexpr (std::is_integral_v<A>) return wrap_mul(a, b); else return a * b; } };
-struct OpDiv { template <typename A> __device__ static A f(A a, A b) { if constexpr (std::is_integral_v<A>) return wrap_div(a, b); else return a / b; } };
-struct OpRDiv { template <typename A> __device__ static A f(A a, A b) { return OpDiv::f(b, a); } };
-// std::max / std::min of the reference: (a<b)?b:a and (b<a)?b:a
-struct OpMax { template <typename A> __device__ static A f(A a, A b) { return (a < b) ? b : a; } };
-struct OpMin { template <typename A> __device__ static A f(A a, A b) { return (b < a) ? b : a; } };
-struct OpPow {
-    __device__ static float f(float a, float b) { return powf(a, b); }
-    __device__ static double f(double a, double b) { return pow(a, b); }
-};
-struct OpRPow { template <typename A> __device__ static A f(A a, A b) { return OpPow::f(b, a); } };
-// pow(x, 2): the correctly rounded value is x*x (one rounding), including signed zeros, infinities and NaN
-struct OpSquare { template <typename A> __device__ static A f(A a) { return a * a; } };
-
-struct OpSqrt { __device__ static float f(float a) { return sqrtf(a); } __device__ static double f(double a) { return sqrt(a); } };
-struct OpExp { __device__ static float f(float a) { return expf(a); } __device__ static double f(double a) { return exp(a); } };
-struct OpLog { __device__ static float f(float a) { return logf(a); } __device__ static double f(double a) { return log(a); } };
-struct OpSin { __device__ static float f(float a) { return sinf(a); } __device__ static double f(double a) { return sin(a); } };
-struct OpCos { __device__ static float f(float a) { return cosf(a); } __device__ static double f(double a) { return cos(a); } };
-struct OpTan { __device__ static float f(float a) { return tanf(a); } __device__ static double f(double a) { return tan(a); } };
-struct OpInvert {
-    template <typename A> __device__ static A f(A a) {
-        if constexpr (std::is_same_v<A, bool_t>) return bool_t{uint8_t(a.v ? 0 : 1)};
-        else return A(~a);
-    }
-};
 
 // ---- tile loop --------------------------------------------------------------------------
 // Calls body(vector_index) for every vector index in [0, nv), UNROLL*256 per workgroup trip.
@@ -180,7 +139,7 @@ __device__ __forceinline__ void unary_body(const T *__restrict__ a, T *__restric
                 VT r;
                 acc_t<T> t[V];
 #pragma unroll
-                for (int k = 0; k < V; ++k) t[k] = Op::f(load_acc(x[u].v[k]));
+                for (int k = 0; k < V; ++k) t[k] = unary_apply<Op, T>(load_acc(x[u].v[k]));
                 store_acc_vec<T, V>(r, t);
                 st_sel<NTS>(&vc[j], r);
             }
@@ -188,7 +147,7 @@ __device__ __forceinline__ void unary_body(const T *__restrict__ a, T *__restric
     });
     if (blockIdx.x == 0) {
         int64_t j = nv * V + threadIdx.x;
-        if (j < n) c[j] = store_acc<T>(Op::f(load_acc(a[j])));
+        if (j < n) c[j] = store_acc<T>(unary_apply<Op, T>(load_acc(a[j])));
     }
 }
 // ntl: loads carry the nt hint (chosen per launch, see nt_load_* in common.hpp)
@@ -367,7 +326,7 @@ __global__ __launch_bounds__(kBlock) void chain_kernel(const ChainArgs p, int64_
             A y[V];
 #define DXH_CH_BIN(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) y[v] = Op::f(A(load_acc(a.v[v])), A(load_acc(b.v[v]))); break
 #define DXH_CH_SCALAR(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) y[v] = Op::f(A(load_acc(a.v[v])), s); break
-#define DXH_CH_UNARY(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) y[v] = Op::f(load_acc(a.v[v])); break
+#define DXH_CH_UNARY(Op) _Pragma("unroll") for (int v = 0; v < V; ++v) y[v] = unary_apply<Op, T>(load_acc(a.v[v])); break
             switch (code) {
             case DXH_CHAIN_ADD: DXH_CH_BIN(OpAdd);
             case DXH_CHAIN_SUB: DXH_CH_BIN(OpSub);
@@ -540,13 +499,29 @@ __global__ __launch_bounds__(kBlock) void chain_rows_kernel(const RowChainArgs p
             if (q != kChainPrev) b = slot[q * kBlock + t];
             float rowsum = 0.f;
             if constexpr (BYROW) {
-                if (code == DXH_CHAIN_ROWSUM) {  // the operand sits in slot l (the host sees to that), group j of the row at lane j
+                if (code >= DXH_CHAIN_ROWSUM) {  // sum, max or min of the row; the operand sits in slot l (the host sees to that), group j of the row at lane j
                     __syncthreads();
                     if (lane < G) {
-                        float acc[4] = {0.f, 0.f, 0.f, 0.f};
                         const f32x4_t *src = slot + l * kBlock + row_in_block * P;
-                        row_lane_fold<R_SUM, float, 4>(acc, lane, G, cq, [&](int64_t i) __attribute__((always_inline)) { return __builtin_bit_cast(vec_t<float, 4>, src[i]); });
-                        const float v = row_group_fold<R_SUM, float, 4>(acc, G);
+                        auto ld = [&](int64_t i) __attribute__((always_inline)) { return __builtin_bit_cast(vec_t<float, 4>, src[i]); };
+                        float v;
+                        if (code == DXH_CHAIN_ROWSUM) {
+                            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+                            row_lane_fold<R_SUM, float, 4>(acc, lane, G, cq, ld);
+                            v = row_group_fold<R_SUM, float, 4>(acc, G);
+                        } else if (code == DXH_CHAIN_ROWMAX) {
+                            float acc[4];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[e] = rinit<R_MAX, float, float>();
+                            row_lane_fold<R_MAX, float, 4>(acc, lane, G, cq, ld);
+                            v = row_group_fold<R_MAX, float, 4>(acc, G);
+                        } else {
+                            float acc[4];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[e] = rinit<R_MIN, float, float>();
+                            row_lane_fold<R_MIN, float, 4>(acc, lane, G, cq, ld);
+                            v = row_group_fold<R_MIN, float, 4>(acc, G);
+                        }
                         if (lane == 0) row_sums[row_in_block] = v;
                     }
                     __syncthreads();
@@ -573,10 +548,13 @@ __global__ __launch_bounds__(kBlock) void chain_rows_kernel(const RowChainArgs p
             case DXH_CHAIN_MAXSCALAR: DXH_RC_SCALAR(OpMax);
             case DXH_CHAIN_MINSCALAR: DXH_RC_SCALAR(OpMin);
             case DXH_CHAIN_SQRT: DXH_RC_UNARY(OpSqrt);
-            case DXH_CHAIN_EXP: DXH_RC_UNARY(OpExp);
+            case DXH_CHAIN_EXP:
+                if (dt == kRcF32) { DXH_RC_UNARY(OpExp); }
+                _Pragma("unroll") for (int v = 0; v < 4; ++v) y[v] = exp_to_half(a[v]);
+                break;
             case DXH_CHAIN_LOG: DXH_RC_UNARY(OpLog);
             case DXH_CHAIN_SQUARE: DXH_RC_UNARY(OpSquare);
-            case DXH_CHAIN_ROWSUM: _Pragma("unroll") for (int v = 0; v < 4; ++v) y[v] = rowsum; break;
+            case DXH_CHAIN_ROWSUM: case DXH_CHAIN_ROWMAX: case DXH_CHAIN_ROWMIN: _Pragma("unroll") for (int v = 0; v < 4; ++v) y[v] = rowsum; break;
             default: _Pragma("unroll") for (int v = 0; v < 4; ++v) y[v] = a[v]; break;  // DXH_CHAIN_COPY
             }
 #undef DXH_RC_BIN
@@ -697,6 +675,12 @@ int dxh_chain(int dtype, const void *const *inputs, int n_inputs, const dxh_chai
     }
     if (n == 0) return DXH_OK;
     hipStream_t st = as_stream(stream);
+    if (dtype == DXH_F32 || dtype == DXH_F16 || dtype == DXH_BF16) {
+        if (n % (kVecBytes / dtype_size(dtype)) != 0) return DXH_ERR_ALIGN;
+        const int rc = static_chain_try(dtype, inputs, n_inputs, ops, n_ops, n, st);
+        if (rc != kNotStatic) return rc;
+    }
+    chain_count_interpreted();
     switch (dtype) {
     case DXH_F64: return launch_chain<double>(p, ops, n, st);
     case DXH_F32: return launch_chain<float>(p, ops, n, st);
@@ -713,7 +697,8 @@ int dxh_chain_rows_can_sum(int64_t rows, int64_t cols) {
     return g > 0 && cols / 4 <= (int64_t)g * kRowVecs;
 }
 
-int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain_rows_op *ops, int n_ops, int64_t rows, int64_t cols, void *stream) {
+// dry: every check of a real call and no launch
+static int chain_rows_impl(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain_rows_op *ops, int n_ops, int64_t rows, int64_t cols, void *stream, bool dry) {
     if (rows < 0 || cols < 0 || n_ops < 1 || n_ops > kRowOps || n_inputs < 0 || n_inputs > kChainInputs || !ops || (n_inputs > 0 && !inputs)) return DXH_ERR_ARG;
     if (cols % 4 != 0) return DXH_ERR_ALIGN;
     if (rows > 0 && cols / 4 > INT64_MAX / rows) return DXH_ERR_SHAPE;
@@ -731,7 +716,7 @@ int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain
         p.in[j] = inputs[j].data; p.in_dtype[j] = (uint8_t)dt; p.in_kind[j] = (uint8_t)inputs[j].extent;
     }
     int next_slot = n_inputs;
-    bool by_row = false;
+    bool by_row = false, half_reduction = false;
     int save_of[kRowOps], kind_of[kRowOps], dtype_of[kRowOps], code_of[kRowOps], lhs_of[kRowOps], rhs_of[kRowOps];
     for (int k = 0; k < n_ops; ++k) save_of[k] = -1;
     constexpr int kBad = -2;
@@ -754,20 +739,21 @@ int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain
         const dxh_chain_rows_op &o = ops[k];
         const int dt = dtype_code(o.dtype);
         if (dt < 0) return DXH_ERR_DTYPE;
-        if (o.code < DXH_CHAIN_ADD || o.code > DXH_CHAIN_ROWSUM || o.extent < DXH_CHAIN_FULL || o.extent > DXH_CHAIN_COLUMN || (!o.out && k == n_ops - 1)) return DXH_ERR_ARG;
+        if (o.code < DXH_CHAIN_ADD || o.code > DXH_CHAIN_ROWMIN || o.extent < DXH_CHAIN_FULL || o.extent > DXH_CHAIN_COLUMN || (!o.out && k == n_ops - 1)) return DXH_ERR_ARG;
         if (o.out && !aligned(o.out, align_of(dt, o.extent))) return DXH_ERR_ALIGN;
         kind_of[k] = o.extent;  // before operand(): a later op asks for it
         dtype_of[k] = dt;
-        const bool rowsum = o.code == DXH_CHAIN_ROWSUM;
-        // an op of full extent takes anything, an op on vectors only vectors of its own kind; the row sum
-        // turns an fp32 [rows, cols] operand into an fp32 column
+        const bool rowsum = o.code >= DXH_CHAIN_ROWSUM;  // sum, max or min of every row
+        // an op of full extent takes anything, an op on vectors only vectors of its own kind; a row
+        // reduction turns a [rows, cols] operand into a column of the same dtype
         const int want = rowsum ? (int)kRowFull : o.extent == DXH_CHAIN_FULL ? -1 : o.extent;
         int ldt = 0, rdt = 0;
         const int l = operand(o.lhs, k, want, rowsum, &ldt), r = o.code <= DXH_CHAIN_MIN ? operand(o.rhs, k, want, false, &rdt) : l;
         if (l == kBad || r == kBad) return DXH_ERR_ARG;
         if (rowsum) {
             if (o.extent != DXH_CHAIN_COLUMN) return DXH_ERR_ARG;
-            if (dt != kRcF32 || ldt != kRcF32) return DXH_ERR_DTYPE;
+            if (dt != ldt) return DXH_ERR_DTYPE;
+            if (dt != kRcF32) half_reduction = true;  // compiled programs only
             by_row = true;
         }
         for (int j = 0; j < n_inputs; ++j)
@@ -782,6 +768,11 @@ int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain
         p.op[k] = (uint64_t)(uint8_t)code_of[k] | (uint64_t)(uint8_t)(int8_t)lhs_of[k] << 8 | (uint64_t)(uint8_t)(int8_t)rhs_of[k] << 16 |
                   (uint64_t)(uint8_t)(int8_t)save_of[k] << 24 | (uint64_t)(uint8_t)dtype_of[k] << 32 | (uint64_t)(uint8_t)kind_of[k] << 40;
     }
+    if (rows > 0 && cols > 0) {  // a run that the library holds a compiled kernel for
+        const int rc = static_rows_try(inputs, n_inputs, ops, n_ops, rows, cols, as_stream(stream), dry);
+        if (rc != kNotStatic) return rc;
+    }
+    if (half_reduction) return DXH_ERR_DTYPE;  // the interpreting kernel's lanes share a row the way the fp32 reduction does
     const int64_t cq = cols / 4;
     int group = 0, per_row = 1;
     if (by_row) {  // the first lanes of a row fold it as dxh_sum's row stage would, or the sums would not be its sums
@@ -793,12 +784,13 @@ int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain
     }
     const size_t lds = (size_t)slots * kBlock * kVecBytes;
     if (lds > kRowLdsMax) return DXH_ERR_SHAPE;
-    if (rows == 0 || cols == 0) return DXH_OK;
+    if (rows == 0 || cols == 0 || dry) return DXH_OK;
     hipStream_t st = as_stream(stream);
     if (lds > kRowLdsDefault) {
         const int rc = chain_rows_raise_lds(st, true);
         if (rc != DXH_OK) return rc;
     }
+    chain_count_interpreted();
     if (by_row) {
         const int64_t rows_per_block = kBlock / per_row, blocks = (rows + rows_per_block - 1) / rows_per_block;
         if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
@@ -808,6 +800,13 @@ int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain
         chain_rows_kernel<false><<<(unsigned)std::min<int64_t>(blocks, 1 << 22), kBlock, lds, st>>>(p, rows, cq, 1, 1);
     }
     return launch_status();
+}
+
+int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain_rows_op *ops, int n_ops, int64_t rows, int64_t cols, void *stream) {
+    return chain_rows_impl(inputs, n_inputs, ops, n_ops, rows, cols, stream, false);
+}
+int dxh_chain_rows_check(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain_rows_op *ops, int n_ops, int64_t rows, int64_t cols) {
+    return chain_rows_impl(inputs, n_inputs, ops, n_ops, rows, cols, nullptr, true);
 }
 
 }  // extern "C"

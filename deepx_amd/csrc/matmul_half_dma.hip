@@ -27,12 +27,18 @@
 namespace dxh {
 
 // One LDS-direct load: lane's 16 bytes from `base + off` land at LDS byte address lds + 16 * lane.
-// The statement writes M0 and says so (the compiler uses M0 itself for dynamically indexed registers
-// and its own LDS-direct accesses).  No "memory" clobber: ordering against the LDS reads comes from
-// the workgroup barriers around it, and the statement is volatile, so it stays between them.
+// The statement writes M0 and says so: the clobber puts a definition of M0 on the statement, which
+// keeps the compiler's own M0 set-ups (dynamically indexed registers, its LDS-direct accesses) from
+// being shared across it.  M0 is a reserved register, so the compiler remarks that it will not save
+// it around the statement; nothing here needs that, hence the diagnostic is switched off for this
+// one function.  No "memory" clobber: ordering against the LDS reads comes from the workgroup
+// barriers around it, and the statement is volatile, so it stays between them.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void dma16(const void *base, uint32_t off, uint32_t lds) {
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds) : "m0");
 }
+#pragma clang diagnostic pop
 template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N)); }
 
 // NSPLIT = 2: the tile map holds two entries per output tile, each the same tile over one half of

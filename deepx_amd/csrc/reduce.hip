@@ -537,15 +537,16 @@ inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, cons
     return DXH_OK;
 }
 
-int sum_rows_group_f32(int64_t rows, int64_t cols) {
-    if (rows < 1 || cols < 1 || rows > INT32_MAX || cols > INT32_MAX) return 0;
+int reduce_rows_group(int esize, int64_t rows, int64_t cols) {
+    if (rows < 1 || cols < 1 || rows > INT32_MAX || cols > INT32_MAX || (esize != 4 && esize != 2)) return 0;
     const int32_t shape[2] = {(int32_t)rows, (int32_t)cols}, dims[1] = {1};
     Plan pl;
-    if (build_plan(sizeof(float), sizeof(float), shape, 2, dims, 1, pl) != DXH_OK || pl.copy_only || pl.stages.size() != 1) return 0;
+    if (build_plan(esize, sizeof(float), shape, 2, dims, 1, pl) != DXH_OK || pl.copy_only || pl.stages.size() != 1) return 0;
     const Stage &st = pl.stages[0];
-    if (!st.row || st.S != 1 || st.V != kVecBytes / (int)sizeof(float) || st.G > kWave || st.pre != rows || st.R != cols) return 0;
+    if (!st.row || st.S != 1 || st.V != kVecBytes / esize || st.G > kWave || st.pre != rows || st.R != cols) return 0;
     return st.G;
 }
+int sum_rows_group_f32(int64_t rows, int64_t cols) { return reduce_rows_group((int)sizeof(float), rows, cols); }
 
 template <int K, typename Tin, typename Tout, typename TS>
 int launch_stage(const Stage &st, const void *in, void *out, hipStream_t stream) {

@@ -106,5 +106,8 @@ __device__ __forceinline__ A row_group_fold(const A (&acc)[V], int G) {
 // tensor over its last axis, or 0 when the plan is anything else (several stages, a split row, the
 // whole workgroup on one row).
 int sum_rows_group_f32(int64_t rows, int64_t cols);
+// The same for sum / prod / reducemax / reducemin over the last axis of a 16-byte aligned [rows, cols]
+// tensor of fp32 (esize 4) or 16-bit floats (esize 2, accumulated in fp32): all four take one plan.
+int reduce_rows_group(int esize, int64_t rows, int64_t cols);
 
 }  // namespace dxh

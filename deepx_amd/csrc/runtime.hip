@@ -36,6 +36,7 @@ int dxh_tune(int knob, int64_t value) {
     case DXH_TUNE_SKINNY_MIN_ROWS: if (value < 8) return DXH_ERR_ARG; t.skinny_min_rows = value; return DXH_OK;
     case DXH_TUNE_SKINNY_HALF: if (value < 0 || value > 1) return DXH_ERR_ARG; t.skinny_half = value; return DXH_OK;
     case DXH_TUNE_REDUCE_FUSED_FINISH: if (value < 0 || value > 1) return DXH_ERR_ARG; t.reduce_fused_finish = value; return DXH_OK;
+    case DXH_TUNE_CHAIN_STATIC: if (value < 0 || value > 1) return DXH_ERR_ARG; t.chain_static = value; return DXH_OK;
     default: return DXH_ERR_ARG;
     }
 }

@@ -82,6 +82,8 @@ void reg(TfFactory &f, const char *name, const char *author, const char *tftype,
     if (op == "broadcastTo") { tf->chain_code = DXH_CHAIN_COPY; tf->chain_kind = 6; }
     if (op == "powscalar") { tf->chain_code = DXH_CHAIN_SQUARE; tf->chain_kind = 7; }
     if (op == "sum") { tf->chain_code = DXH_CHAIN_ROWSUM; tf->chain_kind = 8; }
+    if (op == "reducemax") { tf->chain_code = DXH_CHAIN_ROWMAX; tf->chain_kind = 8; }
+    if (op == "reducemin") { tf->chain_code = DXH_CHAIN_ROWMIN; tf->chain_kind = 8; }
     tf->graph_safe = kind == "elementwise" || kind == "reduce" || kind == "changeshape" || op == "matmul" ||
                      op == "constant" || op == "arange";
     if (op == "reshape") tf->graph_safe = false;  // rewrites the tensor's shape on the host
@@ -618,9 +620,12 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
         }
         auto out = mem.findtensor(tf->returns[0].textvalue);
         if (!out || !is_float(out->dtype()) || out->shape.size == 0) break;
-        if (ops.empty()) {
-            cols = out->shape.dim() >= 1 ? out->shape.at(-1) : 1;
-            rows = out->shape.size / std::max<int64_t>(cols, 1);
+        if (ops.empty()) {  // the view comes from the first line's output, or from its operand when it reduces rows
+            auto shaper = out;
+            if (kind == kChainSum) shaper = mem.findtensor(tf->args[0].textvalue);
+            if (!shaper || shaper->shape.size == 0) break;
+            cols = shaper->shape.dim() >= 1 ? shaper->shape.at(-1) : 1;
+            rows = shaper->shape.size / std::max<int64_t>(cols, 1);
         }
         Op op{};
         op.op.code = tf->chain_code;
@@ -629,10 +634,11 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
         op.op.extent = extent_of(*out);
         op.out_name = tf->returns[0].textvalue;
         if (kind == kChainSum) {
-            // the sum of every row of an fp32 [rows, cols] tensor, when the row stage of dxh_sum would be one lane group per row
-            if (ops.empty() || rows < 2 || out->dtype() != DXH_F32 || out->shape.size != rows || !dxh_chain_rows_can_sum(rows, cols)) break;
+            // the sum / max / min of every row of a [rows, cols] tensor; whether the row stage of the separate
+            // reduction is one the fused kernels can stand in for is asked of the library once the run is known
+            if (rows < 2 || out->shape.size != rows) break;
             auto in = mem.findtensor(tf->args[0].textvalue);
-            if (!in || in->shape.dim() < 1 || in->shape.at(-1) != cols) break;
+            if (!in || in->shape.dim() < 1 || in->shape.at(-1) != cols || in->shape.size != rows * cols) break;
             try {
                 if (checked_dims(in->shape.shape, ints_of(tf->args[1], mem)) != std::vector<int>{in->shape.dim() - 1}) break;
                 (void)bool_of(tf->args[2]);
@@ -722,7 +728,19 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
             aligned = aligned && (uintptr_t)o.op.out % group_bytes(o.op.dtype, o.op.extent) == 0;  // NULL passes
             plan.row_ops.push_back(o.op);
         }
-        return aligned ? count : 0;
+        if (!aligned) return 0;
+        // would the library launch this run?  (Row reductions are the ones it may refuse: their rows must be
+        // short enough for one lane group, and 16-bit ones need one of its compiled kernels.)  If not, the
+        // run ends before its last row reduction and is asked about again.
+        if (dxh_chain_rows_check(plan.row_inputs.data(), (int)plan.row_inputs.size(), plan.row_ops.data(), (int)plan.row_ops.size(), rows, cols) != DXH_OK) {
+            size_t last_red = count;
+            for (size_t j = 0; j < count; ++j)
+                if (ops[j].op.code >= DXH_CHAIN_ROWSUM) last_red = j;
+            if (last_red == count || last_red < 2) return 0;
+            plan = ChainPlan{};
+            return plan_chain(tfs, first, mem, plan, last_red);
+        }
+        return count;
     }
     plan.dtype = ops[0].op.dtype;
     plan.n = rows * cols;

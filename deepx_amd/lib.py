@@ -44,7 +44,7 @@ class ChainRowsOp(C.Structure):
 
 # enum dxh_chain_code, in the header's order (the last three: dxh_chain_rows only)
 CHAIN_CODES = ["add", "sub", "mul", "div", "max", "min", "addscalar", "subscalar", "rsubscalar", "mulscalar",
-               "divscalar", "rdivscalar", "maxscalar", "minscalar", "sqrt", "exp", "log", "square", "copy", "rowsum"]
+               "divscalar", "rdivscalar", "maxscalar", "minscalar", "sqrt", "exp", "log", "square", "copy", "rowsum", "rowmax", "rowmin"]
 CHAIN_RESULT = 16
 CHAIN_FULL, CHAIN_ROW, CHAIN_COLUMN = 0, 1, 2  # enum dxh_chain_extent
 
@@ -111,6 +111,8 @@ SIGNATURES = {
     "dxh_chain": ([_i, _pp, _i, C.POINTER(ChainOp), _i, _i64, _p], _i),
     "dxh_chain_rows": ([C.POINTER(ChainTensor), _i, C.POINTER(ChainRowsOp), _i, _i64, _i64, _p], _i),
     "dxh_chain_rows_can_sum": ([_i64, _i64], _i),
+    "dxh_chain_rows_check": ([C.POINTER(ChainTensor), _i, C.POINTER(ChainRowsOp), _i, _i64, _i64], _i),
+    "dxh_chain_stats": ([C.POINTER(_i64), C.POINTER(_i64)], _i),
     "dxh_todtype": ([_i, _p, _i, _p, _i64, _p], _i),
     "dxh_equal": ([_i, _p, _p, _f, _p, _i64, _p], _i),
     "dxh_notequal": ([_i, _p, _p, _f, _p, _i64, _p], _i),

@@ -117,11 +117,14 @@ enum dxh_tune_knob {
     DXH_TUNE_SKINNY_MIN_ROWS = 9,      /* ... and the fewest rows of B per K slice (default 256, at least 8) */
     DXH_TUNE_SKINNY_HALF = 10,         /* 1 = that kernel also for bf16 / f16 (default 0: they stay on the matrix pipe,
                                           which is as fast or faster for them) */
-    DXH_TUNE_REDUCE_FUSED_FINISH = 11  /* strided-axis reduction whose reduced axis is cut into slices: 1 (default) = the
+    DXH_TUNE_REDUCE_FUSED_FINISH = 11, /* strided-axis reduction whose reduced axis is cut into slices: 1 (default) = the
                                           workgroup that finishes a tile last adds the slices, in a fixed order, inside the
                                           same launch, 0 = a second launch does (also the fallback when the library's
                                           completion counters are used up).  The two differ in the last bits of a
                                           floating-point sum or product (different, each fixed, order of addition). */
+    DXH_TUNE_CHAIN_STATIC = 12         /* dxh_chain / dxh_chain_rows: 1 (default) = a run that spells one of the sequences the
+                                          library holds a compiled kernel for takes that kernel, 0 = every run goes through
+                                          the interpreting kernel.  Same bits either way. */
 };
 DXH_API int dxh_tune(int knob, int64_t value);
 DXH_API int dxh_device_count(int *count);
@@ -232,7 +235,8 @@ enum dxh_chain_code {
     DXH_CHAIN_ADDSCALAR, DXH_CHAIN_SUBSCALAR, DXH_CHAIN_RSUBSCALAR, DXH_CHAIN_MULSCALAR,               /* lhs op scalar; R: scalar op lhs */
     DXH_CHAIN_DIVSCALAR, DXH_CHAIN_RDIVSCALAR, DXH_CHAIN_MAXSCALAR, DXH_CHAIN_MINSCALAR,
     DXH_CHAIN_SQRT, DXH_CHAIN_EXP, DXH_CHAIN_LOG,                                                      /* f(lhs) */
-    DXH_CHAIN_SQUARE, DXH_CHAIN_COPY, DXH_CHAIN_ROWSUM                                                 /* dxh_chain_rows only */
+    DXH_CHAIN_SQUARE, DXH_CHAIN_COPY, DXH_CHAIN_ROWSUM,                                                /* dxh_chain_rows only */
+    DXH_CHAIN_ROWMAX, DXH_CHAIN_ROWMIN                                                                 /* dxh_chain_rows only */
 };
 #define DXH_CHAIN_MAX_OPS 8
 #define DXH_CHAIN_ROWS_MAX_OPS 16
@@ -263,7 +267,12 @@ DXH_API int dxh_chain(int dtype, const void *const *inputs, int n_inputs, const 
  * DXH_CHAIN_ROWS_MAX_OPS ops.
  * DXH_CHAIN_ROWSUM (fp32 only) is launch_sum (reduce_miaobyte.cuh:16-21) over the last axis inside the
  * run: lhs of full extent, the result a column vector with the bits dxh_sum stores for the same rows
- * (the lanes share the rows as its kernel would and add in its order).  That needs rows short enough
+ * (the lanes share the rows as its kernel would and add in its order).  DXH_CHAIN_ROWMAX and
+ * DXH_CHAIN_ROWMIN are launch_reducemax / launch_reducemin (reduce_miaobyte.cuh:30-52) the same way
+ * (the order matters for them too: NaN and the sign of a zero follow it).  In a run that the library
+ * holds a compiled kernel for (DXH_TUNE_CHAIN_STATIC) the three also take f16 / bf16 operands, and rows
+ * of up to eight 16-byte vectors per lane of the separate kernel's lane group; the interpreting kernel
+ * takes fp32 operands only.  That needs rows short enough
  * for one lane group: dxh_chain_rows_can_sum says whether a [rows, cols] view qualifies (1) or not (0),
  * and a run with a row sum over one that does not is refused with DXH_ERR_SHAPE, as is a run that needs
  * more LDS than a CU has.  A run whose LDS need exceeds 64 KiB raises the kernel's limit first: once
@@ -284,7 +293,13 @@ typedef struct dxh_chain_rows_op {
     int32_t extent;    /* of the result */
 } dxh_chain_rows_op;
 DXH_API int dxh_chain_rows_can_sum(int64_t rows, int64_t cols);
+/* How many dxh_chain / dxh_chain_rows launches of this process took a compiled kernel and how many the
+ * interpreting one (for tests and for a caller that wants to see which of its runs are known). */
+DXH_API int dxh_chain_stats(int64_t *compiled, int64_t *interpreted);
 DXH_API int dxh_chain_rows(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain_rows_op *ops, int n_ops, int64_t rows, int64_t cols, void *stream);
+/* Every check of dxh_chain_rows and no launch: DXH_OK when the same call would be launched (a planner asks before it
+ * commits a row reduction to a run; touches no device state). */
+DXH_API int dxh_chain_rows_check(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain_rows_op *ops, int n_ops, int64_t rows, int64_t cols);
 
 /* ---- cast: launch_todtype elementwise_miaobyte_basic.cuh:11-16.
  * C[i] = static_cast<dst>(A[i]) (float->int truncates toward zero, saturating at

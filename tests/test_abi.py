@@ -73,7 +73,7 @@ def test_argument_errors_need_no_gpu():
     assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(17, 0, 1, 48)), 1, 8, None) == -2   # unknown op code
     assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(0, 0, 1, 50)), 1, 8, None) == -5    # output off a 16-byte boundary
     assert L.dxh_chain(dx.F32, ins, 2, (dx.ChainOp * 1)(op(0, 0, 1, None)), 1, 8, None) == -2  # the last op must store
-    assert len(dx.CHAIN_CODES) == 20 and dx.CHAIN_CODES[16] == "log" and dx.CHAIN_CODES[18] == "copy"
+    assert len(dx.CHAIN_CODES) == 22 and dx.CHAIN_CODES[16] == "log" and dx.CHAIN_CODES[18] == "copy" and dx.CHAIN_CODES[21] == "rowmin"
     # dxh_chain_rows: the same checks, and those on extents: a [rows, cols] op takes any operand, an op on
     # vectors only vectors of its kind; a vector input may not be an output of the run
     T, R = dx.ChainTensor, dx.ChainRowsOp
@@ -85,7 +85,7 @@ def test_argument_errors_need_no_gpu():
     assert run(rop(2, 0, 1, 512), cols=18) == -5                             # cols not a multiple of 4
     assert run(rop(2, 0, 1, 512, dx.F64)) == -1                              # no fp64 in this form
     assert L.dxh_chain_rows((T * 1)(T(64, dx.I32, FULL)), 1, (R * 1)(rop(18, 0, 0, 512)), 1, 8, 16, None) == -1
-    assert run(rop(20, 0, 0, 512)) == -2                                     # unknown op code
+    assert run(rop(22, 0, 0, 512)) == -2                                     # unknown op code
     assert run(rop(2, 0, 3, 512)) == -2                                      # input 3 does not exist
     assert run(rop(2, 0, 1, 512, extent=3)) == -2                            # unknown extent
     assert run(rop(2, 0, 1, None)) == -2                                     # the last op must store
@@ -106,6 +106,24 @@ def test_argument_errors_need_no_gpu():
     assert L.dxh_chain_rows_can_sum(64, 1 << 20) == 0                        # a row that long is cut or takes the whole workgroup
     assert run(rop(19, 0, 0, 512, dx.F32, COL), rows=64, cols=1 << 20) == -3
     assert run(*([rop(2, 0, 0, 512)] * 17)) == -2                            # too many ops
+    # dxh_chain_rows_check: the checks of a call without its launch.  A softmax (row max, sub, exp, row sum, exp,
+    # div) is one of the runs with a compiled kernel, which takes 16-bit rows and rows of up to eight 16-byte
+    # vectors per lane; other runs with a row reduction need fp32 and rows short enough for the interpreter.
+    RES = dx.CHAIN_RESULT
+    def softmax(dt, rows, cols):
+        tin1 = (T * 1)(T(4096, dt, FULL))
+        ops = [rop(20, 0, 0, 8192, dt, COL), rop(18, RES, 0, None, dt, FULL), rop(1, 0, RES + 1, None, dt, FULL), rop(15, RES + 2, 0, None, dt, FULL),
+               rop(19, RES + 3, 0, 8192, dt, COL), rop(15, RES + 2, 0, None, dt, FULL), rop(18, RES + 4, 0, None, dt, FULL), rop(3, RES + 5, RES + 6, 4096, dt, FULL)]
+        return L.dxh_chain_rows_check(tin1, 1, (R * len(ops))(*ops), len(ops), rows, cols)
+    assert softmax(dx.F32, 2048, 2048) == 0 and softmax(dx.BF16, 2048, 4096) == 0 and softmax(dx.F16, 7, 8) == 0
+    assert softmax(dx.F32, 64, 1 << 20) == -3 and softmax(dx.BF16, 64, 8192) == -1 and softmax(dx.BF16, 64, 12) == -1
+    assert L.dxh_tune(12, 0) == 0
+    try:
+        assert softmax(dx.F32, 2048, 896) == 0 and softmax(dx.F32, 2048, 2048) == -3 and softmax(dx.BF16, 2048, 896) == -1
+    finally:
+        assert L.dxh_tune(12, 1) == 0
+    a, b = C.c_int64(-1), C.c_int64(-1)
+    assert L.dxh_chain_stats(C.byref(a), C.byref(b)) == 0 and a.value >= 0 and b.value >= 0 and L.dxh_chain_stats(None, None) == -2
 
 
 def test_tuning_knobs_validate_their_values():
@@ -118,15 +136,16 @@ def test_tuning_knobs_validate_their_values():
     good = {"DXH_TUNE_NT_STORE_BYTES": [0, 1 << 20], "DXH_TUNE_REDUCE_TARGET_BLOCKS": [256, 1024], "DXH_TUNE_REDUCE_COL_MIN_ROWS": [1, 16],
             "DXH_TUNE_REDUCE_COL_MAX_LANES": [4, 32, 128, 256], "DXH_TUNE_MATMUL_TILE": [1, 6, 15, 0], "DXH_TUNE_REDUCE_ROW_LOADS": [1, 4],
             "DXH_TUNE_MATMUL_SPLITK": [1, 7, 1024, 0], "DXH_TUNE_NT_LOAD": [1, 2, 0], "DXH_TUNE_SKINNY_PER_CU": [2, 4, 1],
-            "DXH_TUNE_SKINNY_MIN_ROWS": [8, 512, 256], "DXH_TUNE_SKINNY_HALF": [1, 0], "DXH_TUNE_REDUCE_FUSED_FINISH": [0, 1]}
+            "DXH_TUNE_SKINNY_MIN_ROWS": [8, 512, 256], "DXH_TUNE_SKINNY_HALF": [1, 0], "DXH_TUNE_REDUCE_FUSED_FINISH": [0, 1],
+            "DXH_TUNE_CHAIN_STATIC": [0, 1]}
     bad = {"DXH_TUNE_REDUCE_TARGET_BLOCKS": [0], "DXH_TUNE_REDUCE_COL_MIN_ROWS": [0], "DXH_TUNE_REDUCE_COL_MAX_LANES": [3, 512],
            "DXH_TUNE_MATMUL_TILE": [-1, 16], "DXH_TUNE_REDUCE_ROW_LOADS": [0, 65], "DXH_TUNE_MATMUL_SPLITK": [-1, 1025], "DXH_TUNE_NT_LOAD": [-1, 3], "DXH_TUNE_SKINNY_PER_CU": [0, 65],
-           "DXH_TUNE_SKINNY_MIN_ROWS": [7], "DXH_TUNE_SKINNY_HALF": [-1, 2], "DXH_TUNE_REDUCE_FUSED_FINISH": [-1, 2]}
+           "DXH_TUNE_SKINNY_MIN_ROWS": [7], "DXH_TUNE_SKINNY_HALF": [-1, 2], "DXH_TUNE_REDUCE_FUSED_FINISH": [-1, 2], "DXH_TUNE_CHAIN_STATIC": [-1, 2]}
     assert set(good) == set(knobs), set(good) ^ set(knobs)
     defaults = {"DXH_TUNE_NT_STORE_BYTES": 0, "DXH_TUNE_REDUCE_TARGET_BLOCKS": 1024, "DXH_TUNE_REDUCE_COL_MIN_ROWS": 16,
                 "DXH_TUNE_REDUCE_COL_MAX_LANES": 128, "DXH_TUNE_MATMUL_TILE": 0, "DXH_TUNE_REDUCE_ROW_LOADS": 4,
                 "DXH_TUNE_MATMUL_SPLITK": 0, "DXH_TUNE_NT_LOAD": 0, "DXH_TUNE_SKINNY_PER_CU": 1, "DXH_TUNE_SKINNY_MIN_ROWS": 256,
-                "DXH_TUNE_SKINNY_HALF": 0, "DXH_TUNE_REDUCE_FUSED_FINISH": 1}
+                "DXH_TUNE_SKINNY_HALF": 0, "DXH_TUNE_REDUCE_FUSED_FINISH": 1, "DXH_TUNE_CHAIN_STATIC": 1}
     try:
         for name, values in good.items():
             for v in values:

@@ -592,3 +592,41 @@ def test_recorded_graphs_return_their_counters(dxh, tmp_path):
         assert used.value == start, (i, used.value, start)
     assert 0 < peak <= 4 * 1024 and cap.value >= 32 * 1024
     dx.check(L.dxh_stream_destroy(st))
+
+
+@pytest.mark.parametrize("dt,rows,cols", [("float32", 4096, 2048), ("bfloat16", 2048, 896), ("float16", 300, 1000), ("float32", 2048, 896)])
+def test_softmax_lines_fuse_into_one_launch(tmp_path, dt, rows, cols):
+    """The front's softmax (front/py/deepx/nn/functional/normalization.py:4-17) as the eight lines it sends
+    once its tensors exist: one launch in a fused batch, every tensor with the bits of the line-by-line run,
+    rows summing to one."""
+    ex = InProc()
+    h = Host(ex, tmp_path)
+    rng = np.random.default_rng(53)
+    x = rng.uniform(-3, 3, (rows, cols)).astype(np.float32)
+    store = {"float32": lambda a: a, "bfloat16": H.f32_to_bf16_bits, "float16": H.f32_to_f16_bits}[dt]
+    h.put("sm_t", store(x), dt)
+    full, col = [rows, cols], [rows, 1]
+    for name, shape in (("m", col), ("mb", full), ("d", full), ("e", full), ("s", col), ("e2", full), ("sb", full), ("y", full)):
+        h.run(f"newtensor({V(shape)})->({T('sm_' + name, dt)})")
+    n = lambda name: T("sm_" + name, dt)
+    lines = [f"reducemax({n('t')}, {V([-1])}, var<bool>:true)->({n('m')})", f"broadcastTo({n('m')}, {V(full)})->({n('mb')})",
+             f"sub({n('t')}, {n('mb')})->({n('d')})", f"exp({n('d')})->({n('e')})", f"sum({n('e')}, {V([-1])}, var<bool>:true)->({n('s')})",
+             f"exp({n('d')})->({n('e2')})", f"broadcastTo({n('s')}, {V(full)})->({n('sb')})", f"div({n('e2')}, {n('sb')})->({n('y')})"]
+    lines = [f"{l} // author=miaobyte id={i + 1}" for i, l in enumerate(lines)]
+    names = ["m", "mb", "d", "e", "s", "e2", "sb", "y"]
+    ex.set_fusion(False)
+    assert all(r.split(" ")[1].startswith("ok") for r in ex.execute_batch(lines))
+    want = {k: h.get("sm_" + k) for k in names}
+    for k in names:
+        h.run(f"constant(var<float32>:0)->({n(k)})")
+    ex.set_fusion(True)
+    before = ex.fusion_stats()
+    assert all(r.split(" ")[1].startswith("ok") for r in ex.execute_batch(lines))
+    after = ex.fusion_stats()
+    assert after["runs"] - before["runs"] == 1 and after["lines"] - before["lines"] == 8, (before, after)
+    for k in names:
+        assert np.array_equal(h.get("sm_" + k).view(np.uint8), want[k].view(np.uint8)), k
+    load = {"float32": lambda a: a.astype(np.float64), "bfloat16": lambda a: H.bf16_bits_to_f32(a).astype(np.float64),
+            "float16": lambda a: H.f16_bits_to_f32(a).astype(np.float64)}[dt]
+    y = load(want["y"]).reshape(rows, cols)
+    assert np.allclose(y.sum(1), 1.0, atol=1e-5 if dt == "float32" else 3e-2)

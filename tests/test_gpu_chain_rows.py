@@ -81,11 +81,26 @@ def run_separately(dxh, orc, inputs, prog, rows, cols):
             dx.check(getattr(dxh, "dxh_" + name)(dt, a.ptr, dx.scalar(s), out.ptr, n, None), name)
             assert getattr(orc, "orc_" + name)(dt, hp(ah), dx.scalar(s), hp(want), n) == 0
         elif name == "rowsum":
-            assert adt == dt == dx.F32 and ae == FULL and e == COL
+            assert adt == dt and ae == FULL and e == COL
             dx.check(dxh.dxh_sum(dt, a.ptr, dx.i32arr([rows, cols]), 2, dx.i32arr([1]), 1, out.ptr, None, 0, None), "sum")
             want = None  # the order of a float sum is the kernel's own: checked against float64 below
-            ref = ah.astype(np.float64).reshape(rows, cols)
-            assert np.all(np.abs(out.get().astype(np.float64) - ref.sum(1)) <= 1e-6 * np.abs(ref).sum(1) + 1e-30), ("sum", rows, cols)
+            ref = H.to_float(ah, dt).astype(np.float64).reshape(rows, cols)
+            rel = 1e-6 if dt == dx.F32 else 2.0 ** -8 if dt == dx.BF16 else 2.0 ** -11  # fp32 accumulation, one rounding to a 16-bit result
+            assert np.all(np.abs(H.to_float(out.get(), dt).astype(np.float64) - ref.sum(1)) <= rel * np.abs(ref).sum(1) + 1e-30), ("sum", rows, cols)
+        elif name in ("rowmax", "rowmin"):
+            assert adt == dt and ae == FULL and e == COL
+            fn = "reducemax" if name == "rowmax" else "reducemin"
+            dx.check(getattr(dxh, "dxh_" + fn)(dt, a.ptr, dx.i32arr([rows, cols]), 2, dx.i32arr([1]), 1, out.ptr, None, 0, None), fn)
+            assert getattr(orc, "orc_" + fn)(dt, hp(ah), dx.i32arr([rows, cols]), 2, dx.i32arr([1]), 1, hp(want)) == 0
+        elif name in ("exp", "log"):
+            assert adt == dt and ae == e
+            dx.check(getattr(dxh, "dxh_" + name)(dt, a.ptr, out.ptr, n, None), name)
+            assert getattr(orc, "orc_" + name)(dt, hp(ah), hp(want), n) == 0
+            g64, w64 = H.to_float(out.get(), dt).astype(np.float64), H.to_float(want, dt).astype(np.float64)
+            ulp = 2.0 ** -23 if dt == dx.F32 else 2.0 ** -7 if dt == dx.BF16 else 2.0 ** -10
+            fin = np.isfinite(w64)
+            assert np.array_equal(fin, np.isfinite(g64)) and np.all(np.abs(g64[fin] - w64[fin]) <= (4 if dt == dx.F32 else 1) * ulp * np.abs(w64[fin]) + 1e-45), (name, rows, cols)
+            want = None  # within 4 ulp of libm (1 ulp of a 16-bit result), not its bits
         else:
             assert adt == dt and ae == e and name == "sqrt"
             dx.check(dxh.dxh_sqrt(dt, a.ptr, out.ptr, n, None), name)

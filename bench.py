@@ -289,12 +289,14 @@ def roofline_matmul(per_op):
     c5 = per_op.get("config5")
     if not c5:
         return None
-    shapes = {k: v for k, v in c5.items() if k.startswith("matmul_bf16_")}
+    shapes = {k: v for k, v in c5.items() if k in ("matmul_bf16_2048x896x4864", "matmul_bf16_2048x4864x896")}
+    extra = {k: {"TFLOP/s": v["TFLOP/s"], "frac": v["frac_mfma_bf16"], "ms": v["ms"]} for k, v in c5.items() if k.startswith("matmul_bf16_") and k not in shapes}
     worst = min(shapes, key=lambda k: shapes[k]["TFLOP/s"])
     return {"bound": "mfma", "kernel": "bf16 matmul, fp32 accumulate (config 5); `achieved` is the slower of the two shapes",
             "achieved": shapes[worst]["TFLOP/s"], "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
             "frac": round(shapes[worst]["TFLOP/s"] / MFMA_BF16_PEAK_TF, 4), "shape": worst,
             "per_shape": {k: {"TFLOP/s": v["TFLOP/s"], "frac": v["frac_mfma_bf16"], "ms": v["ms"]} for k, v in shapes.items()},
+            "other_shapes": extra,
             "traffic": measured_traffic("matmul bf16 " + worst.split("_")[-1])}
 
 
@@ -426,6 +428,26 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
         Cm = torch.empty(mm * nn, device=dev, dtype=torch.bfloat16)
         c5[label] = entry(time_op(L, dx, torch, Events, ev, matmul_call(L, dx, torch, dev, dx.BF16, Am, Bm, Cm, mm, kk, nn)), flops=2 * mm * kk * nn)
         c5[label]["hipblaslt_TFLOP/s"] = vendor_gemm_tflops(torch, Am.view(mm, kk), Bm.view(kk, nn), Cm.view(mm, nn))
+    # the gate and the up projection of the block share their activations: both products as one dxh_matmul_shared_a
+    # call (what the executor's batch path does with the two consecutive matmul lines), against two dxh_matmul calls
+    mm, kk, nn = 2048, 896, 4864
+    Am = torch.randn(mm * kk, device=dev).to(torch.bfloat16)
+    Bs = [(torch.randn(kk * nn, device=dev) * 0.02).to(torch.bfloat16) for _ in range(2)]
+    Cs = [torch.empty(mm * nn, device=dev, dtype=torch.bfloat16) for _ in range(2)]
+    bs, cs = dx.ptrarr([t.data_ptr() for t in Bs]), dx.ptrarr([t.data_ptr() for t in Cs])
+    e = entry(time_op(L, dx, torch, Events, ev, lambda i: L.dxh_matmul_shared_a(dx.BF16, ptr(Am), bs, cs, 2, mm, kk, nn, None, 0, None)), flops=2 * 2 * mm * kk * nn)
+    pair = [matmul_call(L, dx, torch, dev, dx.BF16, Am, Bs[j], Cs[j], mm, kk, nn) for j in range(2)]
+    e["as_two_launches_ms"] = round(time_op(L, dx, torch, Events, ev, lambda i: pair[0](i) or pair[1](i)), 5)
+    c5["matmul_bf16_2048x896x4864_x2_shared_A(gate+up, one launch)"] = e
+    # two square shapes outside BASELINE, where a round of tiles is long against the launch and the stores
+    for side in (4096, 8192):
+        Am = torch.randn(side * side, device=dev).to(torch.bfloat16)
+        Bm = (torch.randn(side * side, device=dev) * 0.02).to(torch.bfloat16)
+        Cm = torch.empty(side * side, device=dev, dtype=torch.bfloat16)
+        label = f"matmul_bf16_{side}x{side}x{side}(outside BASELINE)"
+        c5[label] = entry(time_op(L, dx, torch, Events, ev, matmul_call(L, dx, torch, dev, dx.BF16, Am, Bm, Cm, side, side, side), reps=10), flops=2 * side ** 3)
+        c5[label]["hipblaslt_TFLOP/s"] = vendor_gemm_tflops(torch, Am.view(side, side), Bm.view(side, side), Cm.view(side, side), reps=10)
+    del Bs, Cs, pair
     # the same shapes in fp32, the dtype the reference's own matmul (cublasSgemm / cblas_sgemm) runs in
     for label, (mm, kk, nn) in [("matmul_f32_2048x896x4864", (2048, 896, 4864)), ("matmul_f32_2048x4864x896", (2048, 4864, 896))]:
         Am = torch.randn(mm * kk, device=dev)

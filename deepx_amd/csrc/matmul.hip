@@ -11,6 +11,7 @@
 //                the storage type (integers wrap).  int8 with at least 8 output tiles of 128x128:
 //                v_mfma_i32_32x32x16_i8, int32 accumulate, low 8 bits stored (the same value).
 #include "matmul_common.hpp"
+#include <algorithm>
 
 namespace dxh {
 
@@ -246,6 +247,74 @@ extern "C" int dxh_matmul_workspace_bytes(int dtype, const void *a, const void *
     const int rc = matmul_dispatch(dtype, a, b, const_cast<void *>(c), batch, m, k, n, nullptr, sc);
     if (rc == DXH_OK) *bytes = sc.used;
     return rc;
+}
+
+// C_j = A B_j, j < count: one launch where the products take an LDS-direct tile uncut, else one after another
+// (each with the whole workspace: launches of one stream run in order).
+static int matmul_shared_dispatch(int dtype, const void *a, const void *const *bs, void *const *cs, int count, int64_t m, int64_t k, int64_t n,
+                                  void *stream, Scratch &sc) {
+    if (count < 1 || !bs || !cs || m < 0 || k < 0 || n < 0) return DXH_ERR_ARG;
+    for (int j = 0; j < count; ++j) {
+        if (!cs[j] && m * n > 0) return DXH_ERR_ARG;
+        for (int i = 0; i < j; ++i)
+            if (cs[i] == cs[j] && m * n > 0) return DXH_ERR_ARG;  // two products into one result
+    }
+    if ((dtype == DXH_BF16 || dtype == DXH_F16) && count >= 2 && m * n * k > 0 && a) {
+        bool all = true;
+        for (int j = 0; j < count; ++j) all = all && bs[j] && cs[j];
+        auto group = [&](int at) {
+            SharedA g{};
+            g.count = std::min(count - at, kSharedAMax);
+            for (int j = 0; j < g.count; ++j) { g.b[j] = bs[at + j]; g.c[j] = cs[at + j]; }
+            return g;
+        };
+        // every group of pairs takes the same decision (same shape; the alignment of each pair is looked at)
+        bool shared = all;
+        for (int at = 0; shared && at < count; at += kSharedAMax) {
+            const SharedA g = group(at);
+            if (g.count >= 2) shared = launch_matmul_half_shared(dtype, a, g, m, k, n, nullptr, true) == DXH_OK;
+        }
+        if (shared) {
+            for (int at = 0; at < count; at += kSharedAMax) {
+                const SharedA g = group(at);
+                int rc;
+                if (g.count >= 2) rc = sc.planning ? DXH_OK : launch_matmul_half_shared(dtype, a, g, m, k, n, as_stream(stream), false);
+                else rc = matmul_dispatch(dtype, a, bs[at], cs[at], 1, m, k, n, stream, sc);  // one pair left over
+                if (rc != DXH_OK) return rc;
+            }
+            return DXH_OK;
+        }
+    }
+    size_t most = 0;
+    for (int j = 0; j < count; ++j) {
+        Scratch one = sc;
+        one.used = 0;
+        const int rc = matmul_dispatch(dtype, a, bs[j], cs[j], 1, m, k, n, stream, one);
+        if (rc != DXH_OK) return rc;
+        most = std::max(most, one.used);
+    }
+    sc.used = most;
+    return DXH_OK;
+}
+
+extern "C" int dxh_matmul_shared_a_workspace_bytes(int dtype, const void *a, const void *const *bs, void *const *cs, int count, int64_t m, int64_t k, int64_t n,
+                                                   size_t *bytes) {
+    if (!bytes) return DXH_ERR_ARG;
+    *bytes = 0;
+    Scratch sc;
+    sc.planning = true;
+    const int rc = matmul_shared_dispatch(dtype, a, bs, cs, count, m, k, n, nullptr, sc);
+    if (rc == DXH_OK) *bytes = sc.used;
+    return rc;
+}
+
+extern "C" int dxh_matmul_shared_a(int dtype, const void *a, const void *const *bs, void *const *cs, int count, int64_t m, int64_t k, int64_t n,
+                                   void *workspace, size_t workspace_bytes, void *stream) {
+    if (workspace && !aligned(workspace, 256)) return DXH_ERR_WORKSPACE;
+    Scratch sc;
+    sc.base = (char *)workspace;
+    sc.bytes = workspace ? workspace_bytes : 0;
+    return matmul_shared_dispatch(dtype, a, bs, cs, count, m, k, n, stream, sc);
 }
 
 extern "C" int dxh_matmul(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n,

@@ -283,7 +283,13 @@ int launch_on_padded_copies(Inner inner, const void *a, const void *b, void *c, 
 constexpr int kNoSkinny = -1002;  // not a DXH_ERR_* value
 int launch_matmul_skinny(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc);
 int launch_matmul_half(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc);
-int launch_matmul_half_dma(int dtype, int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st);
+// Several products that share their left operand, C_j = A B_j for j < count, as one launch: the tile map's
+// batch index selects the pair (count 0: an ordinary, possibly batched, product).
+constexpr int kSharedAMax = 4;
+struct SharedA { const void *b[kSharedAMax]; void *c[kSharedAMax]; int count; };
+constexpr int kNoShared = -1004;  // not a DXH_ERR_* value: no single launch for these products, the caller multiplies one by one
+int launch_matmul_half_dma(int dtype, int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, const SharedA &multi = SharedA{});
+int launch_matmul_half_shared(int dtype, const void *a, const SharedA &multi, int64_t m, int64_t k, int64_t n, hipStream_t st, bool dry);
 // 128x128 (wide: 128x256) tiles cut into two halves of K that are summed inside the launch: `part` holds
 // dma_split_bytes(tiles), `cnt` one zeroed counter per output tile (finish_counters, reduce.hip)
 inline int64_t dma_split_bytes(int64_t tiles, int wide) { return tiles * 2 * 128 * (wide ? 256 : 128) * (int64_t)sizeof(float); }

@@ -403,6 +403,58 @@ int launch_padded(const void *a, const void *b, void *c, int64_t batch, int64_t 
     return rc != DXH_OK ? rc : launch_mfma<T>(a_as_is ? a : (const void *)ap, bp, c, batch, m, kp, np, st, sc, n);
 }
 
+// The workgroup tile of an aligned bf16 / f16 product that is not cut along K (DXH_TUNE_MATMUL_TILE numbering).
+// dma_ok: the LDS-direct kernels can take it (K a multiple of 64, C at its own [M][N]).
+static int64_t choose_uncut_tile(int64_t batch, int64_t m, int64_t k, int64_t n, int64_t ldc, bool dma_ok) {
+    int64_t choice = 0;
+    // 256x256 tiles halve the bytes every CU pulls through its vector cache per flop, but need
+    // about one tile per CU to pay off.  Below that, 128x128 tiles (two workgroups per CU) as
+    // long as they still give every CU a workgroup and a half; skinny outputs go to 128x64 or
+    // 64x64 tiles so that all CUs (and their vector caches) take part.
+    const int64_t cus = compute_units();
+    auto tiles = [&](int tm, int tn) { return batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn); };
+    if (m <= 64) choice = 5;  // one tile row: anything taller multiplies padding (bf16 [1,896]x[896,151936]: 53 vs 75 us)
+    else if (tiles(128, 64) * 4 >= cus * 3) {
+        // Enough output for tiles of 128x64 and up: estimated time in us of the candidates.  The two
+        // one-workgroup-per-CU tiles run in rounds of `cus` tiles, each round paying its own
+        // prologue and its own burst of C stores (nothing else runs on the CU to hide them); K
+        // steps get faster when only part of the CUs is busy.  128x128 tiles run two to a CU: a
+        // pair of tiles takes 1.08 us per K step, a tile that has the CU to itself 0.53 us.
+        const double ksteps = (double)((k + PK - 1) / PK);
+        auto one_per_cu = [&](int tm, int tn, double step, double overhead) {
+            const int64_t t = tiles(tm, tn), rounds = (t + cus - 1) / cus;
+            const double busy = rounds > 1 ? 1.0 : (double)t / (double)cus;
+            return (double)rounds * (ksteps * step * (0.65 + 0.35 * busy) + overhead);
+        };
+        const int64_t t1 = tiles(128, 128), full = t1 / (2 * cus), rem = t1 % (2 * cus);
+        const double c1 = ksteps * (1.08 * (double)full + (rem == 0 ? 0.0 : rem <= cus ? 0.53 : 1.08)) + 2.0;
+        const double edge = ldc >= 0 ? 5.0 : 0.0;  // element-wise C stores make the burst at the end of a round longer
+        const double c4 = one_per_cu(256, 256, 1.645, 3.5 + edge), c6 = one_per_cu(192, 256, 1.21, 6.0 + edge);
+        // 128x64 tiles, two to a CU as well: 0.33 us per K step and tile (2048x4864x896: 224 tiles, 27 us)
+        const double c2 = ksteps * 0.33 * (double)((tiles(128, 64) + cus - 1) / cus) + 2.0;
+        choice = (c1 <= c4 && c1 <= c6) ? 1 : (c4 <= c6) ? 4 : 6;
+        if (c2 < (choice == 1 ? c1 : choice == 4 ? c4 : c6)) choice = 2;
+        // Lower tiles of the same width, one wave per 64 columns (matmul_half_dma.hip only): when a
+        // lower tile still fits the output into one round, every CU's K loop gets shorter
+        // (2048x896x4864: 18.2 us with 160 rows, 19.8 with 192; 2048x4096x4096: 56.9 us with 128
+        // rows, 63.4 with 192, hipBLASLt 70.9).  Both run three LDS stages of K 64 (against five of
+        // K 32: 2048x4096x4096 58.4 -> 55.7 us, 3072^3 with 160 rows 51.6 -> 48.8 us).
+        // And a tile half as wide for an N that 256 columns divide badly (8192x4864x896, where 256-wide
+        // tiles compute 1024 columns: 58.5 us against 66.5 with 128 rows x 256).
+        // All three are taken for a single round only: over several rounds the square tile's lower
+        // traffic through L2 wins again (8192^3: 843 us with 256x128, 790 with 256x256).
+        if (dma_ok) {
+            const double c11 = one_per_cu(160, 256, 0.96, 5.5), c12 = one_per_cu(128, 256, 0.85, 5.0), c13 = one_per_cu(256, 128, 0.76, 3.5) - (tiles(256, 128) <= cus / 2 ? ksteps * 0.09 : 0.0);  // 0.52 us per step up to half the CUs
+            double best = choice == 1 ? c1 : choice == 2 ? c2 : choice == 4 ? c4 : c6;
+            if (c11 < best && tiles(160, 256) <= cus) { best = c11; choice = 11; }
+            if (c12 < best && tiles(128, 256) <= cus) { best = c12; choice = 12; }
+            if (c13 < best && tiles(256, 128) <= cus) { best = c13; choice = 13; }
+        }
+    }
+    else choice = 5;  // 1024x8192x1024 as 128 tiles of 128x64: 38 us, 31 us with 256 64x64 tiles
+    return choice;
+}
+
 // ldc >= 0: called by launch_padded on its copies; C then has ldc columns at pitch ldc
 template <typename T>
 int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc, int64_t ldc) {
@@ -427,53 +479,7 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
         const int rc = launch_split<T>(a, b, c, batch, m, k, n, st, sc);
         if (rc != kNoSplit) return rc;
     }
-    if (fast && choice == 0) {
-        // 256x256 tiles halve the bytes every CU pulls through its vector cache per flop, but need
-        // about one tile per CU to pay off.  Below that, 128x128 tiles (two workgroups per CU) as
-        // long as they still give every CU a workgroup and a half; skinny outputs go to 128x64 or
-        // 64x64 tiles so that all CUs (and their vector caches) take part.
-        const int64_t cus = compute_units();
-        auto tiles = [&](int tm, int tn) { return batch * ((m + tm - 1) / tm) * ((n + tn - 1) / tn); };
-        if (m <= 64) choice = 5;  // one tile row: anything taller multiplies padding (bf16 [1,896]x[896,151936]: 53 vs 75 us)
-        else if (tiles(128, 64) * 4 >= cus * 3) {
-            // Enough output for tiles of 128x64 and up: estimated time in us of the candidates.  The two
-            // one-workgroup-per-CU tiles run in rounds of `cus` tiles, each round paying its own
-            // prologue and its own burst of C stores (nothing else runs on the CU to hide them); K
-            // steps get faster when only part of the CUs is busy.  128x128 tiles run two to a CU: a
-            // pair of tiles takes 1.08 us per K step, a tile that has the CU to itself 0.53 us.
-            const double ksteps = (double)((k + PK - 1) / PK);
-            auto one_per_cu = [&](int tm, int tn, double step, double overhead) {
-                const int64_t t = tiles(tm, tn), rounds = (t + cus - 1) / cus;
-                const double busy = rounds > 1 ? 1.0 : (double)t / (double)cus;
-                return (double)rounds * (ksteps * step * (0.65 + 0.35 * busy) + overhead);
-            };
-            const int64_t t1 = tiles(128, 128), full = t1 / (2 * cus), rem = t1 % (2 * cus);
-            const double c1 = ksteps * (1.08 * (double)full + (rem == 0 ? 0.0 : rem <= cus ? 0.53 : 1.08)) + 2.0;
-            const double edge = ldc >= 0 ? 5.0 : 0.0;  // element-wise C stores make the burst at the end of a round longer
-            const double c4 = one_per_cu(256, 256, 1.645, 3.5 + edge), c6 = one_per_cu(192, 256, 1.21, 6.0 + edge);
-            // 128x64 tiles, two to a CU as well: 0.33 us per K step and tile (2048x4864x896: 224 tiles, 27 us)
-            const double c2 = ksteps * 0.33 * (double)((tiles(128, 64) + cus - 1) / cus) + 2.0;
-            choice = (c1 <= c4 && c1 <= c6) ? 1 : (c4 <= c6) ? 4 : 6;
-            if (c2 < (choice == 1 ? c1 : choice == 4 ? c4 : c6)) choice = 2;
-            // Lower tiles of the same width, one wave per 64 columns (matmul_half_dma.hip only): when a
-            // lower tile still fits the output into one round, every CU's K loop gets shorter
-            // (2048x896x4864: 18.2 us with 160 rows, 19.8 with 192; 2048x4096x4096: 56.9 us with 128
-            // rows, 63.4 with 192, hipBLASLt 70.9).  Both run three LDS stages of K 64 (against five of
-            // K 32: 2048x4096x4096 58.4 -> 55.7 us, 3072^3 with 160 rows 51.6 -> 48.8 us).
-            // And a tile half as wide for an N that 256 columns divide badly (8192x4864x896, where 256-wide
-            // tiles compute 1024 columns: 58.5 us against 66.5 with 128 rows x 256).
-            // All three are taken for a single round only: over several rounds the square tile's lower
-            // traffic through L2 wins again (8192^3: 843 us with 256x128, 790 with 256x256).
-            if (dma_ok) {
-                const double c11 = one_per_cu(160, 256, 0.96, 5.5), c12 = one_per_cu(128, 256, 0.85, 5.0), c13 = one_per_cu(256, 128, 0.76, 3.5) - (tiles(256, 128) <= cus / 2 ? ksteps * 0.09 : 0.0);  // 0.52 us per step up to half the CUs
-                double best = choice == 1 ? c1 : choice == 2 ? c2 : choice == 4 ? c4 : c6;
-                if (c11 < best && tiles(160, 256) <= cus) { best = c11; choice = 11; }
-                if (c12 < best && tiles(128, 256) <= cus) { best = c12; choice = 12; }
-                if (c13 < best && tiles(256, 128) <= cus) { best = c13; choice = 13; }
-            }
-        }
-        else choice = 5;  // 1024x8192x1024 as 128 tiles of 128x64: 38 us, 31 us with 256 64x64 tiles
-    }
+    if (fast && choice == 0) choice = choose_uncut_tile(batch, m, k, n, ldc, dma_ok);
     // The two one-workgroup-per-CU tiles have a twin whose operands travel straight into LDS
     // (matmul_half_dma.hip: less power, no LDS store traffic, deeper prefetch; 8192^3 830 -> 782 us,
     // 4096^3 109 -> 102 us); it needs whole K steps of 64 and C at its own [M][N].  Its 256x256 tile
@@ -525,6 +531,28 @@ int launch_mfma(const void *a, const void *b, void *c, int64_t batch, int64_t m,
 #undef DXH_MM
     return launch_status();
 }
+// C_j = A B_j for the pairs of `multi` as ONE launch of an LDS-direct tile: the tile that one of the products
+// alone would take, over a tile map with one batch entry per pair, so the second product's tiles start as
+// the first's finish (one prologue for the lot, the stores of C_0 run under the K loops of C_1).  Only for
+// products that take such a tile uncut; kNoShared otherwise, and the caller multiplies one by one.  dry: the
+// decision without the launch.
+int launch_matmul_half_shared(int dtype, const void *a, const SharedA &multi, int64_t m, int64_t k, int64_t n, hipStream_t st, bool dry) {
+    if (multi.count < 2 || multi.count > kSharedAMax || tuning().matmul_tile != 0) return kNoShared;
+    bool ok = m > 64 && k % 64 == 0 && n % 8 == 0 && aligned(a, kVecBytes) && k <= (1 << 22) && n <= (1 << 24);
+    for (int j = 0; j < multi.count; ++j) ok = ok && aligned(multi.b[j], kVecBytes) && aligned(multi.c[j], kVecBytes);
+    if (!ok) return kNoShared;
+    const int64_t cus = compute_units();
+    // a long K over few tiles is cut along K when multiplied alone (scratch, counters): not here
+    const int64_t t64 = ((m + 63) / 64) * ((n + 63) / 64), t128 = ((m + 127) / 128) * ((n + 127) / 128);
+    if (k >= 2048 && tuning().matmul_splitk != 1 && (t64 * 2 <= cus || (k >= 4096 && t128 >= 40 && 2 * t128 <= cus))) return kNoShared;
+    if (tuning().matmul_splitk >= 2) return kNoShared;
+    int64_t choice = choose_uncut_tile(1, m, k, n, -1, true);
+    if (choice == 4 || choice == 6) choice = choice == 6 ? 8 : k >= 2048 ? 10 : 7;  // their LDS-direct twins, as in launch_mfma
+    if (choice < 7 || choice > 13) return kNoShared;
+    if (dry) return DXH_OK;
+    return launch_matmul_half_dma(dtype, (int)choice - 7, a, nullptr, nullptr, 1, m, k, n, st, multi);
+}
+
 int launch_matmul_half(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, Scratch &sc) {
     return dtype == DXH_BF16 ? launch_mfma<bf16_t>(a, b, c, batch, m, k, n, st, sc) : launch_mfma<f16_t>(a, b, c, batch, m, k, n, st, sc);
 }

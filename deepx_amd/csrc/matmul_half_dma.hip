@@ -50,7 +50,7 @@ template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_
 // reduce_col_fused_kernel (reduce.hip).
 template <typename T, int TM, int TN, int DK, int NS, int WN = 2, int NSPLIT = 0>
 __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int K, int N,
-                                                                TileMap map, float *part, unsigned *cnt) {
+                                                                TileMap map, float *part, unsigned *cnt, const SharedA multi) {
     // the four waves form a WM x WN grid over the tile: 2 x 2, or 1 x 4 for a tile height that is
     // a multiple of 32 but not of 64
     constexpr int WM = 4 / WN, WTM = TM / WM, WTN = TN / WN;
@@ -82,6 +82,13 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
         const int base = KT / NSPLIT, rem = KT - base * NSPLIT;  // K steps dealt out evenly; the launcher makes sure that base >= 1
         kbeg = slice * base + (slice < rem ? slice : rem);
         KT = base + (slice < rem ? 1 : 0);
+    }
+    // multi.count > 0: the tile map's batch index picks one of several B / C pairs that share the one A
+    // (selected with compares: an index into the by-value argument would send it to per-lane memory)
+    if (multi.count > 0) {
+        B = reinterpret_cast<const T *>(zb == 0 ? multi.b[0] : zb == 1 ? multi.b[1] : zb == 2 ? multi.b[2] : multi.b[3]);
+        C = reinterpret_cast<T *>(zb == 0 ? multi.c[0] : zb == 1 ? multi.c[1] : zb == 2 ? multi.c[2] : multi.c[3]);
+        zb = 0;
     }
     const uint16_t *Ab = reinterpret_cast<const uint16_t *>(A) + ((int64_t)zb * M + m0) * K + (int64_t)kbeg * DK;
     const uint16_t *Bb = reinterpret_cast<const uint16_t *>(B) + ((int64_t)zb * K + (int64_t)kbeg * DK) * N + n0;
@@ -304,10 +311,10 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
 }
 
 template <typename T, int TM, int TN, int DK, int NS, int WN = 2>
-static int launch_dma_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+static int launch_dma_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, const SharedA &multi) {
     TileMap map;
-    if (!make_tile_map(batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
-    matmul_dma_kernel<T, TM, TN, DK, NS, WN><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, nullptr, nullptr);
+    if (!make_tile_map(multi.count > 0 ? multi.count : batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
+    matmul_dma_kernel<T, TM, TN, DK, NS, WN><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, nullptr, nullptr, multi);
     return launch_status();
 }
 
@@ -317,8 +324,8 @@ template <typename T>
 static int launch_dma_split(int wide, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, float *part, unsigned *cnt, hipStream_t st) {
     TileMap map;
     if (!make_tile_map(batch * 2, m, n, 128, wide ? 256 : 128, map)) return DXH_ERR_SHAPE;
-    if (wide) matmul_dma_kernel<T, 128, 256, 64, 3, 4, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, part, cnt);
-    else matmul_dma_kernel<T, 128, 128, 64, 3, 2, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, part, cnt);
+    if (wide) matmul_dma_kernel<T, 128, 256, 64, 3, 4, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, part, cnt, SharedA{});
+    else matmul_dma_kernel<T, 128, 128, 64, 3, 2, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, part, cnt, SharedA{});
     return launch_status();
 }
 
@@ -327,22 +334,22 @@ static int launch_dma_split(int wide, const void *a, const void *b, void *c, int
 // checked K % 64 == 0, N % 8 == 0, the alignment of a, b, c and that every byte offset inside a tile
 // fits 32 bits.
 template <typename T>
-static int launch_dma_shape(int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
+static int launch_dma_shape(int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, const SharedA &multi) {
     switch (shape) {
-    case 0: return launch_dma_tile<T, 256, 256, 32, 4>(a, b, c, batch, m, k, n, st);
-    case 1: return launch_dma_tile<T, 192, 256, 32, 5>(a, b, c, batch, m, k, n, st);
-    case 3: return launch_dma_tile<T, 256, 256, 64, 2>(a, b, c, batch, m, k, n, st);
-    case 4: return launch_dma_tile<T, 160, 256, 64, 3, 4>(a, b, c, batch, m, k, n, st);
-    case 5: return launch_dma_tile<T, 128, 256, 64, 3, 4>(a, b, c, batch, m, k, n, st);
-    case 6: return launch_dma_tile<T, 256, 128, 64, 3>(a, b, c, batch, m, k, n, st);
-    default: return launch_dma_tile<T, 128, 64, 64, 5>(a, b, c, batch, m, k, n, st);
+    case 0: return launch_dma_tile<T, 256, 256, 32, 4>(a, b, c, batch, m, k, n, st, multi);
+    case 1: return launch_dma_tile<T, 192, 256, 32, 5>(a, b, c, batch, m, k, n, st, multi);
+    case 3: return launch_dma_tile<T, 256, 256, 64, 2>(a, b, c, batch, m, k, n, st, multi);
+    case 4: return launch_dma_tile<T, 160, 256, 64, 3, 4>(a, b, c, batch, m, k, n, st, multi);
+    case 5: return launch_dma_tile<T, 128, 256, 64, 3, 4>(a, b, c, batch, m, k, n, st, multi);
+    case 6: return launch_dma_tile<T, 256, 128, 64, 3>(a, b, c, batch, m, k, n, st, multi);
+    default: return launch_dma_tile<T, 128, 64, 64, 5>(a, b, c, batch, m, k, n, st, multi);
     }
 }
 int launch_matmul_half_dma_split(int dtype, int wide, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, float *part, unsigned *cnt, hipStream_t st) {
     return dtype == DXH_BF16 ? launch_dma_split<bf16_t>(wide, a, b, c, batch, m, k, n, part, cnt, st) : launch_dma_split<f16_t>(wide, a, b, c, batch, m, k, n, part, cnt, st);
 }
-int launch_matmul_half_dma(int dtype, int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st) {
-    return dtype == DXH_BF16 ? launch_dma_shape<bf16_t>(shape, a, b, c, batch, m, k, n, st) : launch_dma_shape<f16_t>(shape, a, b, c, batch, m, k, n, st);
+int launch_matmul_half_dma(int dtype, int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, const SharedA &multi) {
+    return dtype == DXH_BF16 ? launch_dma_shape<bf16_t>(shape, a, b, c, batch, m, k, n, st, multi) : launch_dma_shape<f16_t>(shape, a, b, c, batch, m, k, n, st, multi);
 }
 
 }  // namespace dxh

@@ -85,9 +85,10 @@ __global__ __launch_bounds__(kBlock) void reduce_row_kernel(const Tin *__restric
 // ---- col stage ---------------------------------------------------------------------------
 // in [pre, R, post] -> out [pre, S, post].  Workgroup = TX column-lanes x TY row-lanes
 // (TX*TY == 256); a column-lane owns V adjacent columns.  Linear block id -> (p, s, ctile).
-// COH: the partial tile is written through to memory (device-scope stores), for a reader in another
-// workgroup of the same launch.
-template <int K, typename Tin, typename Tout, typename TS, int V, bool NTL, bool COH = false>
+// DEST 1: the partial tile is written through to memory (device-scope stores), for a reader in another
+// workgroup of the same launch.  DEST 2: nothing is stored; row-lane 0's part of `lds` holds the tile
+// (value k of column-lane tx at lds[k * TY * TX + tx]) and the caller goes on with it.
+template <int K, typename Tin, typename Tout, typename TS, int V, bool NTL, int DEST = 0>
 __device__ __forceinline__ void reduce_col_body(racc_t<TS> *lds, const Tin *__restrict__ in, Tout *__restrict__ out,
                                                              int64_t pre, int64_t R, int64_t post, int S, int64_t chunk,
                                                              int TX, int ctiles) {
@@ -152,11 +153,12 @@ __device__ __forceinline__ void reduce_col_body(racc_t<TS> *lds, const Tin *__re
         }
         __syncthreads();
     }
+    if constexpr (DEST == 2) return;
     if (ty == 0 && active) {
         Tout *o = out + (p * S + s) * post + cv * V;
 #pragma unroll
         for (int k = 0; k < V; ++k) {
-            if constexpr (COH) __hip_atomic_store(o + k, rstore<Tout, A>(lds[(k * TY) * TX + tx]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if constexpr (DEST == 1) __hip_atomic_store(o + k, rstore<Tout, A>(lds[(k * TY) * TX + tx]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             else o[k] = rstore<Tout, A>(lds[(k * TY) * TX + tx]);
         }
     }
@@ -186,8 +188,8 @@ __global__ __launch_bounds__(kBlock) void reduce_col_fused_kernel(const Tin *__r
     using A = racc_t<TS>;
     __shared__ A lds[kBlock * V];
     __shared__ int is_last;
-    if (ntl) reduce_col_body<K, Tin, A, TS, V, true, true>(lds, in, part, pre, R, post, S, chunk, TX, ctiles);
-    else reduce_col_body<K, Tin, A, TS, V, false, true>(lds, in, part, pre, R, post, S, chunk, TX, ctiles);
+    if (ntl) reduce_col_body<K, Tin, A, TS, V, true, 1>(lds, in, part, pre, R, post, S, chunk, TX, ctiles);
+    else reduce_col_body<K, Tin, A, TS, V, false, 1>(lds, in, part, pre, R, post, S, chunk, TX, ctiles);
     // Every lane waits until its own partial-tile stores have been acknowledged before it enters the
     // barrier.  They are write-through stores (sc1), whose acknowledgement comes from memory, past
     // this XCD's L2: once all lanes are through the barrier the whole tile is in memory, so the count
@@ -270,6 +272,48 @@ __global__ __launch_bounds__(kBlock) void reduce_col_fused_kernel(const Tin *__r
     }
 }
 
+// A col stage cut into exactly TWO slices whose accumulate type has 4 bytes and whose op does not care
+// which operand comes first (sums and products; integer max / min): the halves meet in one round trip.
+// Every output element has a 64-bit slot, zero between launches.  A workgroup swaps (1 << 32 | its value's
+// bits) into the slot of each of its elements with one device-scope atomic exchange; what comes back is
+// either zero — the other half has not been here, and will find this value — or the other half's value,
+// which this workgroup then combines with its own, stores to the output and replaces by zero again.  The
+// two halves of a tile may each turn out second for some elements and first for others: every element
+// is combined and stored exactly once, by whichever half came second for it, and a op b == b op a makes
+// the result the same either way.  Against the counter scheme above (partial stores and their
+// acknowledgement, the count, the loads of the partials: three dependent round trips to memory at the end
+// of the launch) this is one.
+template <int K, typename Tin, typename Tfin, typename TS, int V>
+__global__ __launch_bounds__(kBlock) void reduce_col_xchg_kernel(const Tin *__restrict__ in, Tfin *__restrict__ fout, unsigned long long *slots,
+                                                                   int64_t pre, int64_t R, int64_t post, int64_t chunk, int TX, int ctiles, int ntl) {
+    using A = racc_t<TS>;
+    static_assert(sizeof(A) == 4, "value and flag share one 64-bit slot");
+    __shared__ A lds[kBlock * V];
+    if (ntl) reduce_col_body<K, Tin, A, TS, V, true, 2>(lds, in, nullptr, pre, R, post, 2, chunk, TX, ctiles);
+    else reduce_col_body<K, Tin, A, TS, V, false, 2>(lds, in, nullptr, pre, R, post, 2, chunk, TX, ctiles);
+    const int TY = kBlock / TX, tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+    if (ty != 0) return;  // row-lane 0 holds the tile (the LDS tree ended with a barrier)
+    const int ct = (int)(blockIdx.x % ctiles);
+    const int64_t p = blockIdx.x / ctiles / 2;
+    const int64_t cv = (int64_t)ct * TX + tx;
+    if (cv >= post / V) return;
+    const int64_t e0 = p * post + cv * V;
+    A mine[V];
+    unsigned long long got[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {  // all exchanges of the lane are in flight together
+        mine[k] = lds[(k * TY) * TX + tx];
+        got[k] = __hip_atomic_exchange(slots + e0 + k, (1ull << 32) | (unsigned long long)__builtin_bit_cast(uint32_t, mine[k]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+        if ((got[k] >> 32) == 0) continue;  // first at this element: the other half finishes it
+        const A other = __builtin_bit_cast(A, (uint32_t)got[k]);
+        fout[e0 + k] = rstore<Tfin, A>(rop<K, A>(mine[k], other));
+        __hip_atomic_store(slots + e0 + k, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 // Counters of reduce_col_fused_kernel: zero at module load, and every launch leaves them zero.
 // Kernels of one stream run in order, so an eager stream owns one slice for as long as it is
 // known here (dxh_stream_destroy gives it back).  A launch recorded under stream capture may
@@ -278,7 +322,7 @@ __global__ __launch_bounds__(kBlock) void reduce_col_fused_kernel(const Tin *__r
 // pool when that graph is destroyed (counter_ranges.hpp; dxh_graph_end_capture and
 // dxh_graph_destroy report both events here).  When either half is used up the caller falls back
 // to two launches.
-constexpr int kFinishSlice = 1024, kFinishSlices = 32, kFinishCounters = 2 * kFinishSlice * kFinishSlices;
+constexpr int kFinishSlice = 32768, kFinishSlices = 32, kFinishCounters = 2 * kFinishSlice * kFinishSlices;  // 8 MiB: a launch that finishes by exchange takes two words per output element
 static __device__ __align__(256) unsigned g_finish_counters[kFinishCounters];
 namespace {
 struct FinishState {
@@ -308,6 +352,7 @@ unsigned *finish_counters(hipStream_t st, int64_t need) {
         f.base = (unsigned *)ptr;
     }
     if (!f.base) return nullptr;
+    need = (need + 1) & ~(int64_t)1;  // ranges start on even words: a launch may use its words in pairs, as 64-bit slots
     if (capturing) {
         const int64_t off = f.captured.take_for_capture((const void *)st, need);
         return off < 0 ? nullptr : f.base + off;
@@ -373,6 +418,7 @@ struct Stage {
     int64_t chunk;
     int G;               // row: lanes per row
     int TX, ctiles;      // col: column lanes, column tiles
+    int tx_pref;         // col: column lanes fixed by the planner (0: col_lanes decides)
     int V;               // vector length in elements of the stage's input type (1 or 16/size)
     bool may_split;      // col stage: parallelism may come from splitting R
     bool in_is_acc, out_is_acc;
@@ -443,7 +489,7 @@ inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, cons
         } else {
             st.V = (st.post % vfull == 0) ? vfull : 1;
             int64_t postv = st.post / st.V;
-            st.TX = col_lanes(st.pre, postv, st.may_split);
+            st.TX = st.tx_pref ? st.tx_pref : col_lanes(st.pre, postv, st.may_split);
             st.ctiles = (int)((postv + st.TX - 1) / st.TX);
         }
         if (st.out_is_acc) {
@@ -511,6 +557,10 @@ inline int build_plan(int esize, int asize, const int32_t *shape, int ndim, cons
                     S = (int)std::min<int64_t>((col_target + blocks0 - 1) / blocks0, smax);
                 }
             }
+            // Four slices of 512-byte strips or two slices of 256-byte strips are the same number of workgroups
+            // and stream alike (fp32 [8192,8192]: 44.2 and 43.4 us with the counted finish); two slices can
+            // finish by one exchange per element instead of three round trips (reduce_col_xchg_kernel).
+            if (S == 4 && TX == 32 && V == vfull && tuning().reduce_fused_finish == 1) { st.tx_pref = 16; S = 2; }
             if (S == 1) st.may_split = false;  // nothing to split: narrow TX for parallelism instead
         }
         st.S = S;
@@ -589,9 +639,18 @@ int launch_fused_col(const Stage &st, const void *in, void *part, void *fout, hi
     if (st.V != VF || !aligned(in, kVecBytes)) return kNotFused;
     const int64_t gx = st.pre * st.S * st.ctiles;
     if (gx > 0x7fffffff) return kNotFused;
+    const int ntl = nt_load_reduce_col((size_t)(st.pre * st.R * st.post) * sizeof(TS));
+    // two slices of a 4-byte accumulator under an op that commutes bit for bit: one exchange per element
+    if constexpr (sizeof(A) == 4 && (K == R_SUM || K == R_PROD || std::is_integral_v<A>)) {
+        if (st.S == 2 && 2 * st.pre * st.post <= kFinishSlice && tuning().reduce_fused_finish == 1) {
+            if (unsigned *words = finish_counters(stream, 2 * st.pre * st.post)) {
+                reduce_col_xchg_kernel<K, TS, Tfin, TS, VF><<<(unsigned)gx, kBlock, 0, stream>>>((const TS *)in, (Tfin *)fout, reinterpret_cast<unsigned long long *>(words), st.pre, st.R, st.post, st.chunk, st.TX, st.ctiles, ntl);
+                return launch_status();
+            }
+        }
+    }
     unsigned *cnt = finish_counters(stream, st.pre * st.ctiles);
     if (!cnt) return kNotFused;
-    const int ntl = nt_load_reduce_col((size_t)(st.pre * st.R * st.post) * sizeof(TS));
     reduce_col_fused_kernel<K, TS, Tfin, TS, VF><<<(unsigned)gx, kBlock, 0, stream>>>((const TS *)in, (A *)part, (Tfin *)fout, cnt, st.pre, st.R, st.post, st.S, st.chunk, st.TX, st.ctiles, ntl);
     return launch_status();
 }

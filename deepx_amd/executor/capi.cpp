@@ -46,7 +46,7 @@ DXE_API void dxe_set_graphs(void *ex, int on) { static_cast<Executor *>(ex)->use
 DXE_API void dxe_set_fusion(void *ex, int on) { static_cast<Executor *>(ex)->use_fusion = on != 0; }
 DXE_API size_t dxe_fusion_stats(void *ex, char *out, size_t buflen) {
     const auto &s = static_cast<Executor *>(ex)->stats;
-    return copy_out(std::to_string(s.fused_runs) + " " + std::to_string(s.fused_lines), out, buflen);
+    return copy_out(std::to_string(s.fused_runs) + " " + std::to_string(s.fused_lines) + " " + std::to_string(s.matmul_groups) + " " + std::to_string(s.matmul_lines), out, buflen);
 }
 // host-time breakdown of execute() (see Executor::Profile): on/off, and "lines parse match run sync reply" in ns; reading resets
 DXE_API void dxe_set_profile(void *ex, int on) { static_cast<Executor *>(ex)->profile = on != 0; }

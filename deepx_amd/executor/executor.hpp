@@ -41,7 +41,7 @@ public:
     // one launch (dxh_chain): same bits in every output, operands that the run itself produced are
     // not read back from memory.  DEEPX_FUSE=0 turns it off.
     bool use_fusion = true;
-    struct Stats { uint64_t batches = 0, graph_captures = 0, graph_replays = 0, graph_rejects = 0, fused_runs = 0, fused_lines = 0; } stats;
+    struct Stats { uint64_t batches = 0, graph_captures = 0, graph_replays = 0, graph_rejects = 0, fused_runs = 0, fused_lines = 0, matmul_groups = 0, matmul_lines = 0; } stats;
     // Where the host time of a line goes (steady clock, nanoseconds summed over `lines` calls of
     // execute()): parsing the text, finding and cloning the registered op, its wrapper up to the
     // kernel launch, the wait for the device, formatting the reply.  Off unless DEEPX_PROFILE=1.
@@ -218,6 +218,12 @@ public:
                 if (len >= 2) {
                     rc = run_chain(tfs, i, len, mem, message);
                     if (rc == 0) { ++stats.fused_runs; stats.fused_lines += len; return len; }
+                    message.clear();
+                }
+                const size_t group = matmul_group_length(tfs, i, mem);
+                if (group >= 2) {
+                    rc = run_matmul_group(tfs, i, group, mem, message);
+                    if (rc == 0) { ++stats.matmul_groups; stats.matmul_lines += group; return group; }
                     message.clear();
                 }
             }

@@ -107,5 +107,8 @@ int register_all(TfFactory &factory);  // ops.cpp
 // 16-byte aligned whole vectors); 0 or 1 = none.  run_chain launches exactly that run.
 size_t chain_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem);
 int run_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, size_t count, Mem &mem, std::string &error);
+// The same for consecutive `matmul` lines that share their first operand (one dxh_matmul_shared_a call).
+size_t matmul_group_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem);
+int run_matmul_group(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, size_t count, Mem &mem, std::string &error);
 
 }  // namespace deepx

@@ -755,6 +755,59 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
 }
 }  // namespace
 
+// ---- consecutive matmul lines on one left operand as one call -------------------------------------
+// The front's gated MLP multiplies the same activations by the gate and the up weights in two lines
+// (front/py/deepx/nn/modules/mlp/gatedmlp.py:20-26), its attention by the q / k / v weights in three: a
+// run of `matmul` lines whose first operand is the same 2-D bf16 / f16 tensor, whose second operands have
+// one shape and whose results are distinct tensors that none of the lines reads goes to
+// dxh_matmul_shared_a, which launches them together where its kernels allow.  Anything that a single
+// line would refuse ends the run before it, so that line reports its own error.
+namespace {
+struct MatmulGroup { std::shared_ptr<Tensor> a; std::vector<std::shared_ptr<Tensor>> bs, cs; };
+size_t plan_matmul_group(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem, MatmulGroup &g) {
+    std::vector<std::string> reads, writes;
+    for (size_t i = first; i < tfs.size(); ++i) {
+        const TF *tf = tfs[i].get();
+        if (!tf || tf->name != "matmul" || tf->metadata.benchmark_repeat > 1 || tf->args.size() != 2 || tf->returns.size() != 1) break;
+        auto A = mem.findtensor(tf->args[0].textvalue), B = mem.findtensor(tf->args[1].textvalue), C = mem.findtensor(tf->returns[0].textvalue);
+        if (!A || !B || !C || A->shape.dim() != 2 || B->shape.dim() != 2) break;
+        if (A->dtype() != DXH_BF16 && A->dtype() != DXH_F16) break;
+        if (B->dtype() != A->dtype() || C->dtype() != A->dtype()) break;
+        if (A->shape.at(-1) != B->shape.at(-2) || C->shape.shape != std::vector<int>{A->shape.at(-2), B->shape.at(-1)}) break;
+        if (g.a && (tf->args[0].textvalue != reads[0] || B->shape.shape != g.bs[0]->shape.shape)) break;
+        const std::string &out = tf->returns[0].textvalue;
+        bool clash = out == tf->args[0].textvalue || out == tf->args[1].textvalue;
+        for (const std::string &r : reads) clash = clash || r == out;     // an earlier line of the run reads what this one writes
+        for (const std::string &w : writes) clash = clash || w == out || w == tf->args[1].textvalue;  // written twice, or read after it was written
+        if (clash) break;
+        if (!g.a) { g.a = A; reads.push_back(tf->args[0].textvalue); }
+        reads.push_back(tf->args[1].textvalue);
+        writes.push_back(out);
+        g.bs.push_back(B);
+        g.cs.push_back(C);
+    }
+    return g.cs.size();
+}
+}  // namespace
+
+size_t matmul_group_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem) {
+    MatmulGroup g;
+    return plan_matmul_group(tfs, first, mem, g);
+}
+int run_matmul_group(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, size_t count, Mem &mem, std::string &error) {
+    MatmulGroup g;
+    if (plan_matmul_group(tfs, first, mem, g) != count || count < 2) return fail(error, "matmul: the run changed between planning and launch");
+    std::vector<const void *> bs;
+    std::vector<void *> cs;
+    for (size_t j = 0; j < count; ++j) { bs.push_back(g.bs[j]->data); cs.push_back(g.cs[j]->data); }
+    const int64_t m = g.a->shape.at(-2), k = g.a->shape.at(-1), n = g.bs[0]->shape.at(-1);
+    size_t need = 0;
+    int rc = dxh_matmul_shared_a_workspace_bytes(g.a->dtype(), g.a->data, bs.data(), cs.data(), (int)count, m, k, n, &need);
+    if (rc != DXH_OK) return hip_result(rc, "matmul", error);
+    void *ws = need ? mem.workspace(need) : nullptr;
+    return hip_result(dxh_matmul_shared_a(g.a->dtype(), g.a->data, bs.data(), cs.data(), (int)count, m, k, n, ws, need ? mem.workspace_bytes() : 0, mem.stream), "matmul", error);
+}
+
 size_t chain_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem) {
     ChainPlan plan;
     return plan_chain(tfs, first, mem, plan);

@@ -137,6 +137,8 @@ SIGNATURES = {
     "dxh_dropout": ([_i, _p, _i64, _f, C.c_uint32, _p], _i),
     "dxh_matmul_workspace_bytes": ([_i, _p, _p, _p, _i64, _i64, _i64, _i64, C.POINTER(_sz)], _i),
     "dxh_matmul": ([_i, _p, _p, _p, _i64, _i64, _i64, _i64, _p, _sz, _p], _i),
+    "dxh_matmul_shared_a_workspace_bytes": ([_i, _p, _pp, _pp, _i, _i64, _i64, _i64, C.POINTER(_sz)], _i),
+    "dxh_matmul_shared_a": ([_i, _p, _pp, _pp, _i, _i64, _i64, _i64, _p, _sz, _p], _i),
 }
 
 _lib = None

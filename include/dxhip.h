@@ -424,6 +424,20 @@ DXH_API int dxh_matmul_workspace_bytes(int dtype, const void *a, const void *b, 
 DXH_API int dxh_matmul(int dtype, const void *a, const void *b, void *c, int64_t batch, int64_t m,
                        int64_t k, int64_t n, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- several products that share their left operand: C_j[m,n] = sum_k A[m,k] * B_j[k,n], j < count
+ * No counterpart in the reference, which multiplies one product per instruction; for a caller that holds
+ * several instructions at once and finds consecutive matmul lines on one A — the gate and up projections
+ * of the front's gated MLP (front/py/deepx/nn/modules/mlp/gatedmlp.py:20-26), the q / k / v projections of
+ * its attention.  Every C_j holds the bits dxh_matmul stores for the same pair.  bf16 / f16 products that
+ * take one of the large tiles uncut go out as ONE launch over all pairs (the tiles of the second product
+ * start as those of the first finish: one launch, one prologue, stores under the next K loops); anything
+ * else runs as `count` ordinary products, one after another.  bs / cs: HOST arrays of `count` device
+ * pointers, all C_j distinct.  Workspace as for dxh_matmul, sized by the query below. */
+DXH_API int dxh_matmul_shared_a_workspace_bytes(int dtype, const void *a, const void *const *bs, void *const *cs, int count,
+                                                int64_t m, int64_t k, int64_t n, size_t *bytes);
+DXH_API int dxh_matmul_shared_a(int dtype, const void *a, const void *const *bs, void *const *cs, int count, int64_t m,
+                                int64_t k, int64_t n, void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -55,8 +55,8 @@ class InProc:
     def set_sync(self, on): self.L.dxe_set_sync(self.ex, int(on))
 
     def fusion_stats(self):
-        runs, lines = (int(x) for x in self._call(self.L.dxe_fusion_stats, self.ex).split())
-        return {"runs": runs, "lines": lines}
+        runs, lines, groups, group_lines = (int(x) for x in self._call(self.L.dxe_fusion_stats, self.ex).split())
+        return {"runs": runs, "lines": lines, "matmul_groups": groups, "matmul_lines": group_lines}
 
     def stats(self):
         b, c, r, j = (int(x) for x in self._call(self.L.dxe_stats, self.ex).split())

@@ -82,7 +82,7 @@ def test_batch_equals_line_by_line(tmp_path):
     for n in NAMES[2:]:
         assert np.array_equal(h.get("s_" + n).view(np.uint32), want[n].view(np.uint32)), n
     assert ex.stats()["captures"] == 0  # graphs are off unless asked for
-    assert ex.fusion_stats() == {"runs": 0, "lines": 0}  # 257 * 129 floats are not a whole number of 16-byte vectors
+    assert ex.fusion_stats() == {"runs": 0, "lines": 0, "matmul_groups": 0, "matmul_lines": 0}  # 257 * 129 floats are not a whole number of 16-byte vectors
 
 
 def test_graph_replays_track_new_inputs(tmp_path):
@@ -257,9 +257,9 @@ def test_fused_runs_equal_line_by_line(tmp_path):
                 # bfloat16: [add mulscalar sub mul exp] [rdivscalar sqrt log] [max minscalar] [div rsubscalar];
                 # float32: the row sum joins its neighbours, [add ... exp sum rdivscalar sqrt log max minscalar] [div rsubscalar]
                 want_stats = {"runs": 2, "lines": 13} if dt == "float32" else {"runs": 4, "lines": 12}
-                assert ex.fusion_stats() == want_stats, ex.fusion_stats()
+                assert {k: ex.fusion_stats()[k] for k in want_stats} == want_stats, ex.fusion_stats()
             else:
-                assert ex.fusion_stats() == {"runs": 0, "lines": 0}
+                assert ex.fusion_stats() == {"runs": 0, "lines": 0, "matmul_groups": 0, "matmul_lines": 0}
         for n in big + small + ["i3"]:
             want = results["lines"][n]
             for mode in ("fused", "unfused"):
@@ -314,7 +314,7 @@ def test_fused_in_place_run(tmp_path):
         rs = [ex.execute(t) for t in text] if mode == "lines" else ex.execute_batch(text)
         assert all(r.split(" ")[1].startswith("ok") for r in rs), rs
         if mode == "fused":
-            assert ex.fusion_stats() == {"runs": 1, "lines": 6}
+            assert {k: ex.fusion_stats()[k] for k in ("runs", "lines")} == {"runs": 1, "lines": 6}
         outs[mode] = {k: h.get(p + k) for k in ("sg", "g", "u")}
     for k in ("sg", "g", "u"):
         assert np.array_equal(outs["fused"][k], outs["lines"][k]), k
@@ -423,6 +423,8 @@ def test_config5_block_at_full_size_in_every_mode(tmp_path):
             # the thirteen lines of the RMSNorm, its row sum included; the six of the gate
             fs = ex.fusion_stats()
             assert fs["runs"] == 2 * (2 if graphs else 1) and fs["lines"] == 19 * (2 if graphs else 1), (mode, fs)
+            # the gate and the up projection share their activations: one call for the two lines
+            assert fs["matmul_groups"] == (2 if graphs else 1) and fs["matmul_lines"] == 2 * (2 if graphs else 1), (mode, fs)
         kept[mode] = {k: h.get("f5_" + k) for k in ("y", "h", "sg", "xf", "sq", "var", "rs", "xn", "wf1", "wf", "g", "u")}
         y = b2f(kept[mode]["y"]).astype(np.float64)
         hh = b2f(kept[mode]["h"]).astype(np.float64)

@@ -463,3 +463,44 @@ def test_matmul_few_rows_any_n(dxh, dtype):
     dx.check(H.matmul(dxh, dtype, dA.ptr, dB.ptr, dC.ptr, 1, m, k, n, None))
     want = H.to_float(H.to_storage((Ai @ Bi).astype(np.float64).reshape(-1), dtype), dtype)
     assert np.array_equal(H.to_float(dC.get(), dtype), want)
+
+
+@pytest.mark.parametrize("dtype", [dx.BF16, dx.F16])
+def test_products_that_share_their_left_operand(dxh, dtype):
+    """dxh_matmul_shared_a: C_j = A B_j for 2, 3, 4 and 5 pairs is, pair by pair, bit for bit what dxh_matmul
+    stores — as one launch where the shape takes a large tile uncut (the gate / up projections of config 5,
+    2048x896x4864; square and ragged shapes), as separate products otherwise (a K cut in two, rows that are not
+    16-byte pieces, few tiles).  The first shape is also held to float64."""
+    import ctypes as C
+    rng = np.random.default_rng(500 + dtype)
+    for (m, k, n), counts in [((2048, 896, 4864), (2, 3)), ((300, 128, 520), (2, 4, 5)), ((2048, 4864, 896), (2,)), ((333, 777, 555), (2,)),
+                              ((64, 64, 64), (3,)), ((1024, 448, 768), (2,)), ((4096, 1024, 1024), (4,))]:
+        A = H.to_storage(rng.standard_normal(m * k), dtype)
+        dA = Dev(A)
+        for count in counts:
+            Bs = [H.to_storage(rng.standard_normal(k * n) * 0.05, dtype) for _ in range(count)]
+            dBs = [Dev(b) for b in Bs]
+            want = []
+            for j in range(count):
+                dC = Dev.empty(m * n, A.dtype)
+                dx.check(H.matmul(dxh, dtype, dA.ptr, dBs[j].ptr, dC.ptr, 1, m, k, n, None), "matmul")
+                want.append(dC.get())
+            dCs = [Dev(np.full(m * n, 0x7fc1, dtype=A.dtype)) for _ in range(count)]
+            bs, cs = dx.ptrarr([b.ptr.value for b in dBs]), dx.ptrarr([c.ptr.value for c in dCs])
+            need = C.c_size_t(0)
+            dx.check(dxh.dxh_matmul_shared_a_workspace_bytes(dtype, dA.ptr, bs, cs, count, m, k, n, C.byref(need)), "workspace")
+            ws = Dev.empty(max(1, need.value), np.uint8)
+            dx.check(dxh.dxh_matmul_shared_a(dtype, dA.ptr, bs, cs, count, m, k, n, ws.ptr if need.value else None, need.value, None), "shared")
+            for j in range(count):
+                assert np.array_equal(dCs[j].get(), want[j]), (m, k, n, count, j)
+            if (m, k, n) == (2048, 896, 4864) and count == 2:
+                Af = H.to_float(A, dtype).reshape(m, k)
+                for j in range(count):
+                    Bf = H.to_float(Bs[j], dtype).reshape(k, n)
+                    assert np.all(np.abs(H.to_float(dCs[j].get(), dtype).reshape(m, n) - Af @ Bf) <= 1e-2 * (np.abs(Af) @ np.abs(Bf)))
+    # argument errors: two products into one result, a missing result, no pairs
+    p = Dev.empty(64 * 64, np.uint16)
+    same = dx.ptrarr([p.ptr.value, p.ptr.value])
+    assert dxh.dxh_matmul_shared_a(dtype, p.ptr, same, same, 2, 64, 64, 64, None, 0, None) == -2
+    assert dxh.dxh_matmul_shared_a(dtype, p.ptr, same, dx.ptrarr([p.ptr.value, 0]), 2, 64, 64, 64, None, 0, None) == -2
+    assert dxh.dxh_matmul_shared_a(dtype, p.ptr, same, same, 0, 64, 64, 64, None, 0, None) == -2

@@ -34,14 +34,26 @@ TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")  # HBM bytes per l
 
 
 def measured_traffic(kernel):
-    """HBM bytes per launch of `kernel` as the last counter collection found them (rocprofv3 --pmc
-    FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size; the summary beside the file
-    says how), or None when the file has no entry for it."""
+    """(bytes, provenance) — HBM-side bytes per launch of `kernel` as the last counter collection found them
+    (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size; the summary beside the file
+    says how).  The file records a hash of the kernel sources the counters were collected on: when those files
+    have changed since, or the file has no entry, bytes is None (the figure would describe another kernel) and
+    the provenance says so."""
+    import hashlib
     try:
         with open(TRAFFIC_JSON) as f:
-            return json.load(f)["kernels"][kernel]["hbm_bytes_per_launch"]
-    except (OSError, KeyError, ValueError):
-        return None
+            doc = json.load(f)
+        e = doc["kernels"][kernel]
+        h = hashlib.sha256()
+        for name in e["sources"]:
+            with open(os.path.join(ROOT, "deepx_amd", "csrc", name), "rb") as src:
+                h.update(src.read())
+        now = h.hexdigest()[:16]
+        prov = {"file": "profiles/traffic.json", "collected": doc.get("collected"), "counter_row": e.get("counter_row"),
+                "sources_sha16": e["sources_sha16"], "sources_unchanged": now == e["sources_sha16"]}
+        return (e["hbm_bytes_per_launch"] if now == e["sources_sha16"] else None), prov
+    except (OSError, KeyError, ValueError) as err:
+        return None, {"file": "profiles/traffic.json", "error": type(err).__name__}
 
 
 def main():
@@ -251,7 +263,8 @@ def main():
                 "bytes_per_launch": XB,
                 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by the
                 # reading of a plain copy kernel of known size (profiles/bench_pmc_hbm_traffic.md)
-                "traffic": measured_traffic("reduce_row_kernel f32 [8192,8192] axis 1")}
+                "traffic": None}
+    roofline["traffic"], roofline["traffic_from"] = measured_traffic("reduce_row_kernel f32 [8192,8192] axis 1")
 
     # ---------------- the other BASELINE configs, one op at a time ----------------------------
     per_op = {"config2": c2}
@@ -297,7 +310,8 @@ def roofline_matmul(per_op):
             "frac": round(shapes[worst]["TFLOP/s"] / MFMA_BF16_PEAK_TF, 4), "shape": worst,
             "per_shape": {k: {"TFLOP/s": v["TFLOP/s"], "frac": v["frac_mfma_bf16"], "ms": v["ms"]} for k, v in shapes.items()},
             "other_shapes": extra,
-            "traffic": measured_traffic("matmul bf16 " + worst.split("_")[-1])}
+            "traffic": measured_traffic("matmul bf16 " + worst.split("_")[-1])[0],
+            "traffic_from": measured_traffic("matmul bf16 " + worst.split("_")[-1])[1]}
 
 
 RAMP_MS = 40.0  # untimed launches before every measurement: from idle the clocks take ~30 ms of load to settle

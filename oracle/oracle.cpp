@@ -22,6 +22,11 @@
 //                             in executor/op-ompsimd/test/tensorfunc/8_tensor_concat.cpp:47-129
 //   matmul                    known answer in executor/op-ompsimd/test/tensorfunc/
 //                             4_tensor_matmul.cpp:18-36 + float64 numpy matmul.
+//   orc_faithful_*           the CPU baseline's variants: orc_faithful_reduce_f32 (E/reduce_miaobyte.hpp:30-44)
+//                             and orc_faithful_{transpose,concat,broadcastTo,indexselect}, which visit every
+//                             output element through an index vector and a linear offset as
+//                             E/changeshape_miaobyte.hpp:45-178 does; pinned by equality with the plain
+//                             functions above on seeded inputs (tests/test_oracle_pins.py), which numpy pins
 // Parity unpinned (only a running reference could pin them): the exact bits of fp32
 // sum/prod (the reference accumulates under `omp atomic` in thread-schedule order,
 // E/reduce_miaobyte.hpp:30-44) and of OpenBLAS sgemm (E/matmul_cblas.hpp:51-57);

@@ -140,6 +140,22 @@ def test_transcendental_4ulp(dxh, orc, name, lo, hi, dtype):
     assert H.ulp_diff(got, want, dtype) <= 4, f"{name} {dx.DTYPE_NAMES[dtype]}"
 
 
+@pytest.mark.parametrize("dtype", [dx.BF16, dx.F16])
+def test_exp_every_16bit_input(dxh, orc, dtype):
+    """exp of a 16-bit float runs on the hardware's exp2 instead of the fp32 expansion.  Every one of
+    the 65,536 input patterns: within one unit in the last place of the oracle's expf rounded once,
+    NaN where it has NaN, and the same zeros, infinities and denormal results."""
+    a = np.arange(65536, dtype=np.uint32).astype(np.uint16).view(H.NP[dtype])
+    got, want = run_unary(dxh, orc, "exp", dtype, a)
+    gf, wf = H.to_float(got, dtype), H.to_float(want, dtype)
+    assert np.array_equal(np.isnan(gf), np.isnan(wf))
+    assert np.array_equal(np.isinf(gf), np.isinf(wf))
+    assert np.array_equal(gf == 0.0, wf == 0.0)
+    assert H.ulp_diff(got, want, dtype) <= 1
+    differing = np.count_nonzero(got.view(np.uint16) != want.view(np.uint16)) - np.count_nonzero(np.isnan(gf))
+    assert differing <= 65536 * 0.05, differing
+
+
 def test_exp_special_values(dxh, orc):
     a = np.array([0.0, -np.inf, np.inf, 1000.0, -1000.0], dtype=np.float32)
     got, _ = run_unary(dxh, orc, "exp", dx.F32, a)

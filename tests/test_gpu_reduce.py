@@ -248,3 +248,36 @@ def test_one_launch_finish_many_launches(dxh):
             _reduce_on(dxh, name, dtype, da, shape, dims, out, ws, wsb, None)
             got = out.get()
             assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (it, name, shape)
+
+
+def test_two_slice_exchange_finish_many_launches(dxh, orc):
+    """A strided axis cut into exactly two slices with a 4-byte accumulator meets in one atomic
+    exchange per output element (each 64-bit slot must be zero again when the launch ends).  1200
+    launches over four cases, compared after every launch with the first launch's bits (a + b and
+    a * b do not depend on which half arrives second); the first launch is held to the oracle, and
+    for integers to the two-launch path bit for bit."""
+    rng = np.random.default_rng(9191)
+    cases = [("sum", dx.F32, (8192, 8192), [0]), ("prod", dx.F32, (2048, 16384), [0]),
+             ("sum", dx.I32, (2048, 16384), [0]), ("reducemax", dx.I32, (2, 2048, 4096), [1])]
+    prepared = []
+    for name, dtype, shape, dims in cases:
+        n = int(np.prod(shape))
+        a = H.rand(rng, dtype, n, 0.999, 1.001) if name == "prod" else H.rand(rng, dtype, n)
+        first, nout = gpu_reduce(dxh, name, dtype, a, shape, dims)
+        check(name, dtype, first, cpu_reduce(orc, name, dtype, a, shape, dims, nout), n // nout)
+        if dtype in H.INTS:
+            dx.check(dxh.dxh_tune(FUSED_KNOB, 0))
+            try:
+                two, _ = gpu_reduce(dxh, name, dtype, a, shape, dims)
+            finally:
+                dx.check(dxh.dxh_tune(FUSED_KNOB, 1))
+            assert np.array_equal(first, two), (name, shape)
+        sh, dm = dx.i32arr(shape), dx.i32arr(dims)
+        wsb = C.c_size_t(0)
+        dx.check(dxh.dxh_reduce_workspace_bytes(dtype, sh, len(shape), dm, len(dims), C.byref(wsb)))
+        prepared.append((name, dtype, shape, dims, Dev(a), Dev.empty(nout, a.dtype), Dev.empty(max(wsb.value, 16), np.uint8), wsb.value, first))
+    for it in range(300):
+        for name, dtype, shape, dims, da, out, ws, wsb, want in prepared:
+            _reduce_on(dxh, name, dtype, da, shape, dims, out, ws, wsb, None)
+            got = out.get()
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (it, name, shape)

@@ -20,6 +20,7 @@ struct StaticArgs {
     const void *in[DXH_CHAIN_MAX_INPUTS];
     void *out[DXH_CHAIN_ROWS_MAX_OPS];
     float scalar[DXH_CHAIN_ROWS_MAX_OPS];  // already rounded to the op's dtype on the host
+    int nt_store;  // use_nt_store on the bytes the launch stores: non-temporal stores, else write-through ones
 };
 
 // ---- row form ---------------------------------------------------------------------------------------
@@ -139,7 +140,7 @@ __global__ __launch_bounds__(kBlock) void chain_static_rows_kernel(const StaticA
                 round_in_place<Op::dt, VW>(val[me][u]);
                 if (out && own[u]) {
                     if constexpr (Op::ext == DXH_CHAIN_FULL) {
-                        if (row_ok) store_elems<Op::dt, VW, true>(out, (row * lv + c[u]) * VW, val[me][u]);
+                        if (row_ok) store_elems_sel<Op::dt, VW>(out, (row * lv + c[u]) * VW, val[me][u], p.nt_store != 0);
                     } else {
                         if (row_raw == 0) store_elems<Op::dt, VW, false>(out, (int64_t)c[u] * VW, val[me][u]);
                     }
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(kBlock) void chain_static_flat_kernel(const StaticA
     eval_flat<Prog, DT, N>(in, res, p.scalar);
     static_for<Prog::n_ops>([&](auto k_) __attribute__((always_inline)) {
         constexpr int k = decltype(k_)::value;
-        if (p.out[k]) store_elems<DT, N, true>(p.out[k], i * N, res[k]);
+        if (p.out[k]) store_elems_sel<DT, N>(p.out[k], i * N, res[k], p.nt_store != 0);
     });
 }
 
@@ -273,12 +274,15 @@ void chain_count_interpreted() { g_interpreted_launches.fetch_add(1, std::memory
 int static_rows_try(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chain_rows_op *ops, int n_ops, int64_t rows, int64_t cols, hipStream_t st, bool dry) {
     if (!tuning().chain_static || rows < 1 || cols < 1) return kNotStatic;
     StaticArgs a{};
+    size_t stored = 0;
     for (int j = 0; j < n_inputs; ++j) a.in[j] = inputs[j].data;
     for (int k = 0; k < n_ops; ++k) {
         a.out[k] = ops[k].out;
+        if (ops[k].out && ops[k].extent == DXH_CHAIN_FULL) stored += (size_t)rows * (size_t)cols * (ops[k].dtype == DXH_F32 ? 4 : 2);
         const float sf = (float)ops[k].scalar.f;
         a.scalar[k] = ops[k].dtype == DXH_F32 ? sf : ops[k].dtype == DXH_BF16 ? load_acc(to_bf16(sf)) : load_acc(to_f16(sf));
     }
+    a.nt_store = use_nt_store(stored);
     // VW elements per lane vector: pointers of [rows, cols] tensors and row vectors must be aligned to it
     auto aligned_to = [&](int vw) {
         if (cols % vw != 0) return false;
@@ -308,12 +312,15 @@ int static_chain_try(int dtype, const void *const *inputs, int n_inputs, const d
     const int dt = dtype_code(dtype);
     if (!tuning().chain_static || dt < 0 || n < 1) return kNotStatic;
     StaticArgs a{};
+    size_t stored = 0;
     for (int j = 0; j < n_inputs; ++j) a.in[j] = inputs[j];
     for (int k = 0; k < n_ops; ++k) {
         a.out[k] = ops[k].out;
+        if (ops[k].out) stored += (size_t)n * chain_dtype_bytes(dt);
         const float sf = (float)ops[k].scalar.f;
         a.scalar[k] = dt == kSF32 ? sf : dt == kSBF16 ? load_acc(to_bf16(sf)) : load_acc(to_f16(sf));
     }
+    a.nt_store = use_nt_store(stored);
     const int64_t nv = n / (16 / chain_dtype_bytes(dt)), blocks = (nv + kBlock - 1) / kBlock;
     if (blocks > 0x7fffffff) return kNotStatic;
     int rc = kNotStatic;

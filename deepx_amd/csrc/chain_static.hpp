@@ -127,6 +127,29 @@ template <int DT, int N, bool NT> __device__ __forceinline__ void store_elems(vo
         st_sel<NT>(reinterpret_cast<vec_t<f16_t, N> *>(reinterpret_cast<f16_t *>(p) + i), r);
     }
 }
+// the same with the launch's store mode: non-temporal for a pure stream, write-through (sc0 sc1) for
+// outputs small enough that the next kernel finds them in the last-level cache (use_nt_store)
+template <int DT, int N> __device__ __forceinline__ void store_elems_sel(void *p, int64_t i, const float (&y)[N], bool nt) {
+    if constexpr (DT == kSF32) {
+        typedef float f4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int q = 0; q < N / 4; ++q) {
+            const f4 x = {y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]};
+            f4 *dst = reinterpret_cast<f4 *>(reinterpret_cast<float *>(p) + i) + q;
+            if (nt) st_mode<1>(dst, x); else st_mode<2>(dst, x);
+        }
+    } else if constexpr (DT == kSBF16) {
+        vec_t<bf16_t, N> r;
+        store_acc_vec<bf16_t, N>(r, y);
+        auto *dst = reinterpret_cast<vec_t<bf16_t, N> *>(reinterpret_cast<bf16_t *>(p) + i);
+        if (nt) st_mode<1>(dst, r); else st_mode<2>(dst, r);
+    } else {
+        vec_t<f16_t, N> r;
+        store_acc_vec<f16_t, N>(r, y);
+        auto *dst = reinterpret_cast<vec_t<f16_t, N> *>(reinterpret_cast<f16_t *>(p) + i);
+        if (nt) st_mode<1>(dst, r); else st_mode<2>(dst, r);
+    }
+}
 template <int DT> __device__ __forceinline__ float load_one(const void *p, int64_t i) {
     if constexpr (DT == kSF32) return reinterpret_cast<const float *>(p)[i];
     else if constexpr (DT == kSBF16) return load_acc(reinterpret_cast<const bf16_t *>(p)[i]);

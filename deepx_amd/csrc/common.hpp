@@ -114,8 +114,8 @@ template <typename VT> __device__ inline void st_nt(VT *p, const VT &v) {
     __builtin_nontemporal_store(__builtin_bit_cast(R, v), reinterpret_cast<R *>(p));
 }
 
-// Store policy of a streaming kernel: 0 plain, 1 nt, 2 write-through at system scope (sc0 sc1),
-// 3 nt at agent scope (sc1 nt); 2 and 3 exist for 16-byte stores only, narrower ones fall back to
+// Store policy of a streaming kernel: 0 plain, 1 nt, 2 write-through at system scope (sc0 sc1; 4-, 8- and
+// 16-byte stores), 3 nt at agent scope (sc1 nt; 16-byte stores only); widths a mode does not have fall back to
 // nt.  2 is the fastest partner of nt loads when two tensors are read per tensor written (see
 // stream_policy_2r1w); 3 is the fastest for write-dominated streams (fp32 broadcast of a row,
 // GB/s at 64 / 128 / 256 MiB: nt 5997 / 6453 / 6798, sc1 nt 6163 / 6811 / 7308; bf16 transpose
@@ -128,6 +128,12 @@ template <int ST, typename VT> __device__ inline void st_mode(VT *p, const VT &v
         // s_nop: a VALU write to the data registers of a 16-byte store needs a wait state after the
         // store, which the compiler inserts for its own stores but not behind inline assembly
         asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(r) : "memory");
+    } else if constexpr (ST == 2 && sizeof(VT) == 8) {
+        const uint64_t r = __builtin_bit_cast(uint64_t, v);
+        asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(r) : "memory");
+    } else if constexpr (ST == 2 && sizeof(VT) == 4) {
+        const uint32_t r = __builtin_bit_cast(uint32_t, v);
+        asm volatile("global_store_dword %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(r) : "memory");
     } else if constexpr (ST == 3 && sizeof(VT) == 16) {
         const u32x4_t r = __builtin_bit_cast(u32x4_t, v);
         asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" ::"v"(p), "v"(r) : "memory");
@@ -143,7 +149,7 @@ template <bool NTL, typename VT> __device__ inline VT ld_sel(const VT *p) {
 // Stores carry the nt hint too.  A/B runs in one process on random data (the knob below): 64 MiB
 // add 6.28 vs 6.10 TB/s, bf16 broadcast 5.9 vs 4.9 TB/s in favour of nt, at every size tried.
 struct Tuning {
-    int64_t nt_store_bytes = 0;                    // DXH_TUNE_NT_STORE_BYTES: 0 = always non-temporal
+    int64_t nt_store_bytes = (int64_t)32 << 20;   // DXH_TUNE_NT_STORE_BYTES: a launch that stores more than this uses non-temporal stores
     int64_t reduce_target_blocks = 4 * 256;       // DXH_TUNE_REDUCE_TARGET_BLOCKS
     int64_t reduce_col_target_blocks = 256;       // strided-axis stages: about one workgroup per CU, each
                                                   // walking its rows with software-pipelined loads
@@ -201,9 +207,17 @@ inline bool nt_load_reduce(size_t in_bytes) { return nt_load_forced(in_bytes > (
 // nt / plain GB/s: 32 MiB 3174/3067, 128 MiB 5520/5270, 256 MiB 6190/5894; bf16 [8192,8192] 4574/2964,
 // bf16 [64,512,2048] axis 1 5794/3239) except within noise at 7 MiB.
 inline bool nt_load_reduce_col(size_t in_bytes) { return nt_load_forced(in_bytes >= ((size_t)8 << 20)); }
+// Stores of the elementwise kernels, the fused runs and the 16-bit products: non-temporal for a launch that
+// stores more than 32 MiB (a pure stream: measured fastest on buffers rotated past the last-level cache),
+// write-through (sc0 sc1) below.  A deepx program reads an op's result in one of its next instructions, and a
+// tensor of activation size that went out with write-through stores is in the 256 MiB last-level cache then
+// without having filled the L2s with dirty lines.  The SiLU gate of config 5 (19.9 MB out) on its own / the whole
+// block (RMSNorm, three products, gate) as four launches, same process: nt 12.0 / 90 us, plain 12.7-13.1 / 85.5,
+// sc0 sc1 11.5 / 84; with the products' C written through as well 79-81 us.  Non-temporal stores at agent scope
+// (sc1 nt) are the fastest for the producer alone (11.4) and leave nothing for the consumer (90).
 inline bool use_nt_store(size_t out_bytes) { return (int64_t)out_bytes > tuning().nt_store_bytes; }
 template <bool NT, typename VT> __device__ inline void st_sel(VT *p, const VT &v) {
-    if constexpr (NT) st_nt(p, v); else *p = v;
+    if constexpr (NT) st_nt(p, v); else st_mode<2>(p, v);
 }
 
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }

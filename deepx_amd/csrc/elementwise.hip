@@ -74,8 +74,8 @@ __global__ __launch_bounds__(kBlock) void binary_kernel(const T *__restrict__ a,
         else if (ntl == 1) binary_body<T, V, Op, 1, true>(a, b, c, n);
         else binary_body<T, V, Op, 1, false>(a, b, c, n);
     } else {
-        if (ntl) binary_body<T, V, Op, 0, true>(a, b, c, n);
-        else binary_body<T, V, Op, 0, false>(a, b, c, n);
+        if (ntl) binary_body<T, V, Op, 2, true>(a, b, c, n);
+        else binary_body<T, V, Op, 2, false>(a, b, c, n);
     }
 }
 
@@ -290,7 +290,7 @@ struct ChainArgs {  // first kernel argument: sits at offset 0 of the kernel-arg
     int n_in, n_ops;                                         // inputs occupy slots 0 .. n_in - 1
 };
 constexpr int kChainPrev = -1;
-template <typename T>
+template <typename T, bool NTS>
 __global__ __launch_bounds__(kBlock) void chain_kernel(const ChainArgs p, int64_t nv) {
     constexpr int V = vec_len<T>;
     using VT = vec_t<T, V>;
@@ -352,7 +352,7 @@ __global__ __launch_bounds__(kBlock) void chain_kernel(const ChainArgs p, int64_
             store_acc_vec<T, V>(r, y);
             prev = __builtin_bit_cast(u32x4_t, r);
             if (save >= 0) raw[save * kBlock + t] = prev;
-            if (out) __builtin_nontemporal_store(prev, &reinterpret_cast<u32x4_t *>(out)[i]);
+            if (out) st_sel<NTS>(&reinterpret_cast<u32x4_t *>(out)[i], prev);
         }
     }
 }
@@ -368,7 +368,12 @@ int launch_chain(ChainArgs &p, const dxh_chain_op *ops, int64_t n, hipStream_t s
     const int64_t nv = n / V, blocks = (nv + kBlock - 1) / kBlock;
     int slots = p.n_in;
     for (int k = 0; k < p.n_ops; ++k) slots = std::max(slots, p.save[k] + 1);
-    chain_kernel<T><<<(unsigned)std::min<int64_t>(blocks, 1 << 22), kBlock, (size_t)slots * kBlock * kVecBytes, st>>>(p, nv);
+    size_t stored = 0;
+    for (int k = 0; k < p.n_ops; ++k)
+        if (p.out[k]) stored += (size_t)n * sizeof(T);
+    const unsigned grid = (unsigned)std::min<int64_t>(blocks, 1 << 22);
+    if (use_nt_store(stored)) chain_kernel<T, true><<<grid, kBlock, (size_t)slots * kBlock * kVecBytes, st>>>(p, nv);
+    else chain_kernel<T, false><<<grid, kBlock, (size_t)slots * kBlock * kVecBytes, st>>>(p, nv);
     return launch_status();
 }
 

@@ -286,6 +286,9 @@ int launch_matmul_half(int dtype, const void *a, const void *b, void *c, int64_t
 // Several products that share their left operand, C_j = A B_j for j < count, as one launch: the tile map's
 // batch index selects the pair (count 0: an ordinary, possibly batched, product).
 constexpr int kSharedAMax = 4;
+// C of a 16-bit product leaves with write-through stores when it is small enough that the kernel which reads it next
+// finds it in the last-level cache (the rule of use_nt_store), else with non-temporal ones
+inline int c_store_through(int64_t batch, int64_t m, int64_t n, size_t esize) { return use_nt_store((size_t)(batch * m * n) * esize) ? 0 : 1; }
 struct SharedA { const void *b[kSharedAMax]; void *c[kSharedAMax]; int count; };
 constexpr int kNoShared = -1004;  // not a DXH_ERR_* value: no single launch for these products, the caller multiplies one by one
 int launch_matmul_half_dma(int dtype, int shape, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, const SharedA &multi = SharedA{});

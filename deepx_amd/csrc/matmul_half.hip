@@ -124,7 +124,7 @@ constexpr int part_count(int count, int part) { return count * (part + 1) / 4 - 
 template <typename T, int TM, int TN, int PD, bool KTAIL, int MODE>
 __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul_mfma_tile_kernel(
     const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, float *__restrict__ partial, int M, int lda, int N, TileMap map, KSplit ks,
-    int ldc, int n_store) {
+    int ldc, int n_store, int c_through) {
     // MODE 0: C[M][N] in 16-byte row pieces.  1 (SPLIT): fp32 partial tile of a K slice.  2 (EDGE): C has
     // its own pitch ldc and n_store <= N columns (B was zero-padded to N columns): rows of C are not
     // 16-byte aligned, so the tile is stored element by element.
@@ -334,8 +334,11 @@ __global__ __launch_bounds__(kBlock, (TM * TN <= 128 * 128) ? 2 : 1) void matmul
         for (int i = 0; i < TM * CB / kBlock; ++i) {
             const int c = t + i * kBlock, row = c / CB, ch = c % CB;
             const int gm = m0 + row, gn = n0 + ch * 8;
-            if (gm < M && gn < N)  // N % 8 == 0: a chunk is either fully inside or fully outside
-                st_nt(reinterpret_cast<uint4 *>(Cr + (int64_t)gm * N + gn), *reinterpret_cast<const uint4 *>(Cs + row * LDC + ch * 8));
+            if (gm < M && gn < N) {  // N % 8 == 0: a chunk is either fully inside or fully outside
+                uint4 *dst = reinterpret_cast<uint4 *>(Cr + (int64_t)gm * N + gn);
+                const uint4 piece = *reinterpret_cast<const uint4 *>(Cs + row * LDC + ch * 8);
+                if (c_through) st_mode<2>(dst, piece); else st_nt(dst, piece);
+            }
         }
     }
 }
@@ -348,11 +351,11 @@ int launch_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m,
     if (!make_tile_map(batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
     const KSplit one{1, (int)k};
     if (ldc >= 0)
-        matmul_mfma_tile_kernel<T, TM, TN, PD, false, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one, (int)ldc, (int)ldc);
+        matmul_mfma_tile_kernel<T, TM, TN, PD, false, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one, (int)ldc, (int)ldc, 0);
     else if (k % PK == 0)
-        matmul_mfma_tile_kernel<T, TM, TN, PD, false, 0><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one, (int)n, (int)n);
+        matmul_mfma_tile_kernel<T, TM, TN, PD, false, 0><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one, (int)n, (int)n, c_store_through(batch, m, n, sizeof(T)));
     else
-        matmul_mfma_tile_kernel<T, TM, TN, PD, true, 0><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one, (int)n, (int)n);
+        matmul_mfma_tile_kernel<T, TM, TN, PD, true, 0><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, nullptr, (int)m, (int)k, (int)n, map, one, (int)n, (int)n, c_store_through(batch, m, n, sizeof(T)));
     return launch_status();
 }
 
@@ -370,9 +373,9 @@ int launch_split(const void *a, const void *b, void *c, int64_t batch, int64_t m
     if (!ws) return DXH_ERR_WORKSPACE;
     if (sc.planning) return DXH_OK;
     if (k % PK == 0)
-        matmul_mfma_tile_kernel<T, TM, TN, SPD, false, 1><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
+        matmul_mfma_tile_kernel<T, TM, TN, SPD, false, 1><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n, 0);
     else
-        matmul_mfma_tile_kernel<T, TM, TN, SPD, true, 1><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n);
+        matmul_mfma_tile_kernel<T, TM, TN, SPD, true, 1><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, nullptr, ws, (int)m, (int)k, (int)n, map, ks, (int)n, (int)n, 0);
     const int rc = launch_status();
     return rc != DXH_OK ? rc : launch_splitk_reduce<float, T>(ws, (T *)c, batch, m * n, ks.splits, st);
 }

@@ -50,7 +50,7 @@ template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_
 // reduce_col_fused_kernel (reduce.hip).
 template <typename T, int TM, int TN, int DK, int NS, int WN = 2, int NSPLIT = 0>
 __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int K, int N,
-                                                                TileMap map, float *part, unsigned *cnt, const SharedA multi) {
+                                                                TileMap map, float *part, unsigned *cnt, const SharedA multi, const int c_through) {
     // the four waves form a WM x WN grid over the tile: 2 x 2, or 1 x 4 for a tile height that is
     // a multiple of 32 but not of 64
     constexpr int WM = 4 / WN, WTM = TM / WM, WTN = TN / WN;
@@ -305,8 +305,11 @@ __global__ __launch_bounds__(kBlock, 1) void matmul_dma_kernel(const T *__restri
     for (int i = 0; i < TM * CB / kBlock; ++i) {
         const int c = t + i * kBlock, row = c / CB, ch = c % CB;
         const int gm = m0 + row, gn = n0 + ch * 8;
-        if (gm < M && gn < N)  // N % 8 == 0: a chunk is either fully inside or fully outside
-            st_nt(reinterpret_cast<uint4 *>(Cr + (int64_t)gm * N + gn), *reinterpret_cast<const uint4 *>(Cs + row * LDC + ch * 8));
+        if (gm < M && gn < N) {  // N % 8 == 0: a chunk is either fully inside or fully outside
+            uint4 *dst = reinterpret_cast<uint4 *>(Cr + (int64_t)gm * N + gn);
+            const uint4 piece = *reinterpret_cast<const uint4 *>(Cs + row * LDC + ch * 8);
+            if (c_through) st_mode<2>(dst, piece); else st_nt(dst, piece);  // c_store_through: will the next kernel find C in the last-level cache
+        }
     }
 }
 
@@ -314,7 +317,7 @@ template <typename T, int TM, int TN, int DK, int NS, int WN = 2>
 static int launch_dma_tile(const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, hipStream_t st, const SharedA &multi) {
     TileMap map;
     if (!make_tile_map(multi.count > 0 ? multi.count : batch, m, n, TM, TN, map)) return DXH_ERR_SHAPE;
-    matmul_dma_kernel<T, TM, TN, DK, NS, WN><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, nullptr, nullptr, multi);
+    matmul_dma_kernel<T, TM, TN, DK, NS, WN><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, nullptr, nullptr, multi, c_store_through(multi.count > 0 ? multi.count : batch, m, n, sizeof(T)));
     return launch_status();
 }
 
@@ -324,8 +327,8 @@ template <typename T>
 static int launch_dma_split(int wide, const void *a, const void *b, void *c, int64_t batch, int64_t m, int64_t k, int64_t n, float *part, unsigned *cnt, hipStream_t st) {
     TileMap map;
     if (!make_tile_map(batch * 2, m, n, 128, wide ? 256 : 128, map)) return DXH_ERR_SHAPE;
-    if (wide) matmul_dma_kernel<T, 128, 256, 64, 3, 4, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, part, cnt, SharedA{});
-    else matmul_dma_kernel<T, 128, 128, 64, 3, 2, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, part, cnt, SharedA{});
+    if (wide) matmul_dma_kernel<T, 128, 256, 64, 3, 4, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, part, cnt, SharedA{}, c_store_through(batch, m, n, sizeof(T)));
+    else matmul_dma_kernel<T, 128, 128, 64, 3, 2, 2><<<(unsigned)(8 * map.chunk), kBlock, 0, st>>>((const T *)a, (const T *)b, (T *)c, (int)m, (int)k, (int)n, map, part, cnt, SharedA{}, c_store_through(batch, m, n, sizeof(T)));
     return launch_status();
 }
 

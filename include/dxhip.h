@@ -94,7 +94,8 @@ DXH_API const char *dxh_error_string(int code);
 /* Launch-heuristic knobs (process wide; results never depend on them, only speed).
  * No counterpart in the reference, whose launch shape is fixed (cuda.hpp:45-67). */
 enum dxh_tune_knob {
-    DXH_TUNE_NT_STORE_BYTES = 0,       /* outputs above this many bytes use non-temporal stores */
+    DXH_TUNE_NT_STORE_BYTES = 0,       /* a launch of an elementwise kernel or a fused run that stores more than this many bytes
+                                        * uses non-temporal stores (default 32 MiB; 0 = always) */
     DXH_TUNE_REDUCE_TARGET_BLOCKS = 1, /* workgroups a reduction stage aims for before it stops splitting R */
     DXH_TUNE_REDUCE_COL_MIN_ROWS = 2,  /* strided-axis stage: fewest rows per lane when R is split */
     DXH_TUNE_REDUCE_COL_MAX_LANES = 3, /* strided-axis stage: widest column-lane count (16..256) */

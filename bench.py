@@ -74,6 +74,9 @@ def main():
                     help="run only one fused run (a label of per_op.config5.fused_runs, or a prefix of one), --steps launches after a "
                          "clock ramp (the program a counter collection wraps) and print its own JSON line")
     ap.add_argument("--chain-static", type=int, default=1, help="with --chain-only: 1 = the library's compiled kernel, 0 = the interpreting kernel")
+    ap.add_argument("--block-only", metavar="MODE", default="",
+                    help="run only the config-5 block over deepxIR in one mode (a key of per_op.config5.mlp_block_over_deepxIR, e.g. "
+                         "one_batch_fused_us), --steps passes (the program a kernel trace wraps) and print its own JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this executor path runs on ONE GPU (no sharding, no collectives); "
@@ -134,6 +137,12 @@ def main():
         print(json.dumps({"matmul_bf16": args.matmul_only, "tile_knob": args.matmul_tile, "launches": args.steps, "us_per_launch": round(ms * 1e3, 2),
                           "TFLOP/s": round(2 * mm * kk * nn / ms / 1e9, 1), "frac_mfma_bf16": round(2 * mm * kk * nn / ms / 1e9 / MFMA_BF16_PEAK_TF, 4),
                           "device": name.value.decode()}))
+        return
+
+    if args.block_only:
+        out = config5_block_over_ir(only=args.block_only, iters=args.steps)
+        out["device"] = name.value.decode()
+        print(json.dumps(out))
         return
 
     if args.chain_only:
@@ -615,13 +624,16 @@ def _executor_lib():
     E.dxe_set_graphs.argtypes = [C.c_void_p, C.c_int]
     E.dxe_set_fusion.argtypes = [C.c_void_p, C.c_int]
     E.dxe_set_sync.argtypes = [C.c_void_p, C.c_int]
+    E.dxe_set_defer.argtypes = [C.c_void_p, C.c_int]
+    E.dxe_flush.argtypes = [C.c_void_p]
     return E
 
 
-def lines_over_ir(setup, block, iters=30):
+def lines_over_ir(setup, block, iters=30, only=None):
     """`block` (deepxIR lines) through the executor's dispatch core in this process (libdxexec.so, the
     code behind the UDP server): wall time per pass when the lines are executed one by one (replies
-    at launch, as op-cuda sends them, and with a wait for the device before every reply), as one
+    at launch, as op-cuda sends them; with a wait for the device before every reply; and with lines that can
+    share a launch held back until their run is complete, the DEEPX_DEFER switch), as one
     batch, as one batch with runs of float elementwise lines fused into single launches, and as a
     recorded HIP graph without and with those fused runs.  The timed region of every mode ends with
     a wait for the device.  Every mode gets a fresh executor (a recorded graph is keyed by the text
@@ -634,8 +646,11 @@ def lines_over_ir(setup, block, iters=30):
     text = "\n".join(lines).encode()
     out = {"ops": len(lines)}
     for label, batched, fused, graphs, wait in (("line_by_line_us", 0, 0, 0, 0), ("line_by_line_waiting_for_each_us", 0, 0, 0, 1),
+                                                ("line_by_line_deferred_us", 0, 1, 0, 0),
                                                 ("one_batch_us", 1, 0, 0, 0), ("one_batch_fused_us", 1, 1, 0, 0),
                                                 ("recorded_graph_us", 1, 0, 1, 0), ("recorded_graph_fused_us", 1, 1, 1, 0)):
+        if only and label != only:
+            continue
         ex = E.dxe_create()
         buf = C.create_string_buffer(1 << 16)
         for line in setup:
@@ -646,6 +661,7 @@ def lines_over_ir(setup, block, iters=30):
         E.dxe_set_graphs(ex, graphs)
         E.dxe_set_fusion(ex, fused)
         E.dxe_set_sync(ex, wait)
+        E.dxe_set_defer(ex, int(label == "line_by_line_deferred_us"))
 
         def once():
             if batched:
@@ -656,10 +672,12 @@ def lines_over_ir(setup, block, iters=30):
 
         for _ in range(4):
             once()
+        E.dxe_flush(ex)
         dx.check(L.dxh_device_sync())
         t0 = time.perf_counter()
         for _ in range(iters):
             once()
+        E.dxe_flush(ex)  # what the last pass left held
         dx.check(L.dxh_device_sync())
         out[label] = round((time.perf_counter() - t0) / iters * 1e6, 1)
         if any(" ok" not in r.split("//")[0] for r in buf.value.decode().split("\n")):
@@ -681,7 +699,7 @@ def config1_chain_over_ir(side=4096):
     return lines_over_ir(setup, block)
 
 
-def config5_block_over_ir(rows=2048, hidden=896, inter=4864):
+def config5_block_over_ir(rows=2048, hidden=896, inter=4864, only=None, iters=30):
     """The whole config-5 block (RMSNorm + gated MLP, 22 deepxIR compute ops on [2048,896] activations)."""
     S, Hd, I = rows, hidden, inter
     b16, f32 = "bfloat16", "float32"
@@ -719,7 +737,7 @@ def config5_block_over_ir(rows=2048, hidden=896, inter=4864):
              f"mul({n('g', b16)}, {n('sg', b16)})->({n('sg', b16)})",
              f"mul({n('sg', b16)}, {n('u', b16)})->({n('sg', b16)})",
              f"matmul({n('sg', b16)}, {n('Wd', b16)})->({n('y', b16)})"]
-    out = lines_over_ir(setup, block)
+    out = lines_over_ir(setup, block, iters=iters, only=only)
     out["rows"] = S
     return out
 

@@ -44,6 +44,15 @@ DXE_API void dxe_set_sync(void *ex, int on) { static_cast<Executor *>(ex)->sync_
 DXE_API void dxe_set_graphs(void *ex, int on) { static_cast<Executor *>(ex)->use_graphs = on != 0; }
 // one launch for runs of float elementwise lines inside a batch (the DEEPX_FUSE switch), and its counters: "runs lines"
 DXE_API void dxe_set_fusion(void *ex, int on) { static_cast<Executor *>(ex)->use_fusion = on != 0; }
+// lines that can share a launch are answered at once and held until the run is complete (the DEEPX_DEFER switch);
+// dxe_flush launches what is held, dxe_held counts it, dxe_defer_stats: "held_lines flushes"
+DXE_API void dxe_set_defer(void *ex, int on) { auto *e = static_cast<Executor *>(ex); if (!on) e->flush(); e->defer = on != 0; }
+DXE_API void dxe_flush(void *ex) { static_cast<Executor *>(ex)->flush(); }
+DXE_API size_t dxe_held(void *ex) { return static_cast<Executor *>(ex)->held(); }
+DXE_API size_t dxe_defer_stats(void *ex, char *out, size_t buflen) {
+    const auto &s = static_cast<Executor *>(ex)->stats;
+    return copy_out(std::to_string(s.held_lines) + " " + std::to_string(s.flushes), out, buflen);
+}
 DXE_API size_t dxe_fusion_stats(void *ex, char *out, size_t buflen) {
     const auto &s = static_cast<Executor *>(ex)->stats;
     return copy_out(std::to_string(s.fused_runs) + " " + std::to_string(s.fused_lines) + " " + std::to_string(s.matmul_groups) + " " + std::to_string(s.matmul_lines), out, buflen);

@@ -41,7 +41,18 @@ public:
     // one launch (dxh_chain): same bits in every output, operands that the run itself produced are
     // not read back from memory.  DEEPX_FUSE=0 turns it off.
     bool use_fusion = true;
-    struct Stats { uint64_t batches = 0, graph_captures = 0, graph_replays = 0, graph_rejects = 0, fused_runs = 0, fused_lines = 0, matmul_groups = 0, matmul_lines = 0; } stats;
+    // DEEPX_DEFER=1: the front sends one line per datagram and waits for the reply before it sends the next
+    // (front/py/deepx/scheduler/client/udpconn.py:17-48), so on its own it never hands over two lines that
+    // could share a launch.  With this switch a line that can start or extend a run (a float elementwise line
+    // and its kin, a matmul on the left operand of the one before) is answered at once and HELD; the run goes
+    // out — as one launch where the library takes it, as separate ones otherwise — when a line arrives that
+    // does not extend it, when flush() is called, or when the server has seen no datagram for a moment.  A
+    // line is held only after it has been checked against the tensor store like a line of a batch (operands
+    // exist, dtypes and extents agree), and nothing else executes while lines are held, so the tensors end up
+    // as line-by-line execution leaves them; the reply of a held line carries the time it was accepted.
+    // Off with DEEPX_SYNC=1 (a reply then promises finished kernels) and with DEEPX_FUSE=0.
+    bool defer = false;
+    struct Stats { uint64_t batches = 0, graph_captures = 0, graph_replays = 0, graph_rejects = 0, fused_runs = 0, fused_lines = 0, matmul_groups = 0, matmul_lines = 0, held_lines = 0, flushes = 0; } stats;
     // Where the host time of a line goes (steady clock, nanoseconds summed over `lines` calls of
     // execute()): parsing the text, finding and cloning the registered op, its wrapper up to the
     // kernel launch, the wait for the device, formatting the reply.  Off unless DEEPX_PROFILE=1.
@@ -65,14 +76,34 @@ public:
         profile = pr && !std::strcmp(pr, "1");
         const char *fuse = std::getenv("DEEPX_FUSE");
         if (fuse && !std::strcmp(fuse, "0")) use_fusion = false;
+        const char *df = std::getenv("DEEPX_DEFER");
+        defer = df && !std::strcmp(df, "1");
     }
     ~Executor() {
+        flush();
         for (auto &kv : graphs_) drop_graph(kv.second);
         if (graph_stream_) dxh_stream_destroy(graph_stream_);
     }
 
+    // lines accepted under `defer` and not yet launched
+    size_t held() {
+        std::lock_guard<std::recursive_mutex> lock(mu_);
+        return held_items_.size();
+    }
+    // launches what is held; failures (none are expected: the lines were checked when they were accepted) go to stderr
+    void flush() {
+        std::lock_guard<std::recursive_mutex> lock(mu_);
+        if (held_items_.empty()) return;
+        std::vector<Item> items;
+        items.swap(held_items_);
+        held_tfs_.clear();
+        ++stats.flushes;
+        for (const std::string &reply : run_items(items, "", false, items[0].resp.recv_at))
+            if (reply.find(" ok") == std::string::npos) std::cerr << "held line failed: " << reply << std::endl;
+    }
+
     std::string execute(const std::string &line, TimePoint recv_at = std::chrono::system_clock::now()) {
-        std::lock_guard<std::mutex> lock(mu_);
+        std::lock_guard<std::recursive_mutex> lock(mu_);
         using Clock = std::chrono::steady_clock;
         Clock::time_point mark = profile ? Clock::now() : Clock::time_point();
         auto lap = [&](uint64_t &slot) {
@@ -89,6 +120,7 @@ public:
         try {
             call.parse(line);
         } catch (const std::exception &e) {
+            flush();
             resp.error(e.what());
             return resp.to_string();
         }
@@ -99,6 +131,7 @@ public:
         std::string why;
         auto tf = factory.get_tf(call, &why);
         if (!tf) {
+            flush();
             std::cerr << why << std::endl;
             resp.error("op" + call.name + " not found");
             return resp.to_string();
@@ -107,6 +140,33 @@ public:
         tf->args = call.args;
         tf->returns = call.returns;
         lap(prof.match_ns);
+        if (defer && !sync_each && use_fusion && has_device) {
+            // hold the line if it extends what is held into one longer run, or — after what is held has gone
+            // out — if it can start a run of its own
+            bool hold = false;
+            if ((tf->chain_kind != 0 || tf->name == "matmul") && tf->metadata.benchmark_repeat <= 1) {
+                held_tfs_.push_back(tf);
+                hold = run_prefix_length(held_tfs_, 0, mem) == held_tfs_.size();
+                if (!hold && held_tfs_.size() > 1) {
+                    held_tfs_.pop_back();
+                    flush();
+                    held_tfs_.push_back(tf);
+                    hold = run_prefix_length(held_tfs_, 0, mem) == 1;
+                }
+                if (!hold) held_tfs_.pop_back();
+            }
+            if (hold) {
+                ++stats.held_lines;
+                resp.start_at = std::chrono::system_clock::now();
+                resp.finish("");
+                held_items_.emplace_back();
+                held_items_.back().call = std::move(call);
+                held_items_.back().tf = tf;
+                held_items_.back().resp = resp;
+                return resp.to_string();
+            }
+            flush();
+        }
         resp.start_at = std::chrono::system_clock::now();
         int rc = 0;
         std::string message;
@@ -135,7 +195,8 @@ public:
     // still succeeds or fails on its own, as when sent one by one.
     std::vector<std::string> execute_batch(const std::vector<std::string> &lines, TimePoint recv_at = std::chrono::system_clock::now()) {
         if (lines.size() == 1) return {execute(lines[0], recv_at)};
-        std::lock_guard<std::mutex> lock(mu_);
+        std::lock_guard<std::recursive_mutex> lock(mu_);
+        flush();  // lines held from earlier datagrams come first
         ++stats.batches;
         // graphs are keyed by the instruction text without the per-call metadata (ids, timestamps)
         std::string key;
@@ -177,7 +238,6 @@ public:
                 }
             }
         }
-        struct Item { TF call; std::shared_ptr<TF> tf; OpResp resp; bool failed = false; };
         std::vector<Item> items(lines.size());
         bool graphable = use_graphs && has_device;
         for (size_t i = 0; i < lines.size(); ++i) {
@@ -208,6 +268,15 @@ public:
             it.tf->returns = it.call.returns;
             graphable = graphable && it.tf->graph_safe && it.tf->metadata.benchmark_repeat <= 1 && !uses_named_arg(it.call);
         }
+        return run_items(items, key, graphable, recv_at);
+    }
+
+private:
+    struct Item { TF call; std::shared_ptr<TF> tf; OpResp resp; bool failed = false; };
+
+    // Parsed and matched lines, in order: runs where lines can share a launch, single launches otherwise,
+    // as one recorded graph when `graphable`; one reply per line.
+    std::vector<std::string> run_items(std::vector<Item> &items, const std::string &key, bool graphable, TimePoint recv_at) {
         std::vector<std::shared_ptr<TF>> tfs(items.size());
         for (size_t i = 0; i < items.size(); ++i) if (!items[i].failed) tfs[i] = items[i].tf;
         // Runs line i, or a run of lines that starts at i as one launch; returns how many lines that were.
@@ -281,7 +350,6 @@ public:
         return replies;
     }
 
-private:
     // What a recorded graph froze about a tensor: the kernels' pointer arguments and every launch
     // shape derived from its dims (an in-place reshape keeps address and size but not those).
     struct Pinned {
@@ -411,7 +479,9 @@ private:
         return true;
     }
 
-    std::mutex mu_;
+    std::recursive_mutex mu_;  // flush() is called from inside execute() and execute_batch()
+    std::vector<Item> held_items_;
+    std::vector<std::shared_ptr<TF>> held_tfs_;
     void *graph_stream_ = nullptr;
     std::unordered_map<std::string, Graph> graphs_;
     static constexpr size_t kMaxRemembered = 1024;

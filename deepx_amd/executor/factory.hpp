@@ -109,6 +109,10 @@ size_t chain_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, M
 int run_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, size_t count, Mem &mem, std::string &error);
 // The same for consecutive `matmul` lines that share their first operand (one dxh_matmul_shared_a call).
 size_t matmul_group_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem);
+// How many lines from tfs[first] on belong to one run of either kind, judged by the lines and the tensor store
+// alone (1: a line that could start one).  Every such line is known to name existing tensors of matching dtype
+// and extent, so holding it back cannot hide an error it would have reported.
+size_t run_prefix_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem);
 int run_matmul_group(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, size_t count, Mem &mem, std::string &error);
 
 }  // namespace deepx

@@ -587,7 +587,10 @@ enum { kChainTodtype = 5, kChainBroadcast = 6, kChainPowscalar = 7, kChainSum = 
 // a line that is not a chainable float op, does not fit the view, needs a ninth input, would overwrite
 // a vector that the run reads from memory (lanes of other rows or columns may not have read it yet),
 // or whose operands are missing or mismatched (the ordinary path then reports the error for that line).
-size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem, ChainPlan &plan, size_t max_ops = DXH_CHAIN_ROWS_MAX_OPS) {
+// structural: stop after the lines have been checked against each other and the tensor store (do the tensors exist,
+// do dtypes and extents agree, does the line fit the view) and return how many form a run, without asking whether
+// the library would launch it as one: what a caller needs to know before it holds a line back for a later launch.
+size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem, ChainPlan &plan, size_t max_ops = DXH_CHAIN_ROWS_MAX_OPS, bool structural = false) {
     struct Input { std::string name; const void *data; int dtype, extent; };
     struct Op { dxh_chain_rows_op op; std::string out_name; };
     std::vector<Input> inputs;
@@ -706,7 +709,7 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
         ops.push_back(op);
     }
     const size_t count = ops.size();
-    if (count < 2) return count;
+    if (count < 2 || structural) return count;
     if (!needs_rows && count > DXH_CHAIN_MAX_OPS) {  // the one-dtype form takes fewer ops
         plan = ChainPlan{};
         return plan_chain(tfs, first, mem, plan, DXH_CHAIN_MAX_OPS);
@@ -811,6 +814,11 @@ int run_matmul_group(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, 
 size_t chain_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem) {
     ChainPlan plan;
     return plan_chain(tfs, first, mem, plan);
+}
+size_t run_prefix_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem) {
+    ChainPlan plan;
+    const size_t chain = plan_chain(tfs, first, mem, plan, DXH_CHAIN_ROWS_MAX_OPS, true);
+    return std::max(chain, matmul_group_length(tfs, first, mem));
 }
 int run_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, size_t count, Mem &mem, std::string &error) {
     ChainPlan plan;

@@ -8,10 +8,14 @@
 // `__quit__`, ends serve() (the test harness stops the process with it); it is honoured only in a
 // datagram whose source address is loopback, unless DEEPX_REMOTE_QUIT=1.  DEEPX_BIND names the local
 // address to bind instead of INADDR_ANY (e.g. 127.0.0.1 when the front runs on the same host).
+// While the executor holds lines back (DEEPX_DEFER=1) the loop waits at most DEEPX_DEFER_US microseconds
+// (default 200) for the next datagram before it launches them, so a pause of the sender never leaves work unlaunched.
 #pragma once
 #include <arpa/inet.h>
+#include <poll.h>
 #include <sys/socket.h>
 #include <unistd.h>
+#include <algorithm>
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
@@ -38,6 +42,7 @@ public:
         if (const char *bind_to = std::getenv("DEEPX_BIND")) {
             if (::inet_pton(AF_INET, bind_to, &addr.sin_addr) != 1) { fprintf(stderr, "DEEPX_BIND: not an IPv4 address: %s\n", bind_to); return false; }
         }
+        if (const char *us = std::getenv("DEEPX_DEFER_US")) defer_us_ = std::max(0, std::atoi(us));
         const char *rq = std::getenv("DEEPX_REMOTE_QUIT");
         remote_quit_ = rq && std::string(rq) == "1";
         addr.sin_port = htons((uint16_t)port_);
@@ -53,6 +58,11 @@ public:
     void serve(Executor &ex) {
         std::vector<char> buf(65536);
         while (!stop_) {
+            if (ex.held() > 0) {  // nothing more within the grace period: launch what is held
+                pollfd pfd{fd_, POLLIN, 0};
+                timespec grace{defer_us_ / 1000000, (long)(defer_us_ % 1000000) * 1000};
+                if (::ppoll(&pfd, 1, &grace, nullptr) <= 0) { ex.flush(); continue; }
+            }
             sockaddr_in cli{};
             socklen_t len = sizeof cli;
             ssize_t n = ::recvfrom(fd_, buf.data(), buf.size() - 1, 0, (sockaddr *)&cli, &len);
@@ -84,6 +94,7 @@ private:
     int port_;
     int fd_ = -1;
     bool remote_quit_ = false;
+    int defer_us_ = 200;
     std::atomic<bool> stop_{false};
 };
 

@@ -23,7 +23,7 @@ class InProc:
         L.dxe_create.restype = C.c_void_p
         L.dxe_destroy.argtypes = [C.c_void_p]
         for name, args in [("dxe_execute", [C.c_void_p, C.c_char_p]), ("dxe_execute_batch", [C.c_void_p, C.c_char_p]), ("dxe_stats", [C.c_void_p]),
-                           ("dxe_fusion_stats", [C.c_void_p]),
+                           ("dxe_fusion_stats", [C.c_void_p]), ("dxe_defer_stats", [C.c_void_p]),
                            ("dxe_parse", [C.c_char_p]), ("dxe_match", [C.c_void_p, C.c_char_p]),
                            ("dxe_op_table", [C.c_void_p, C.c_char_p]), ("dxe_typedef_roundtrip", [C.c_char_p]),
                            ("dxe_tensor_yaml", [C.c_void_p, C.c_char_p]), ("dxe_shape_yaml_roundtrip", [C.c_char_p])]:
@@ -39,6 +39,10 @@ class InProc:
         L.dxe_set_fusion.argtypes = [C.c_void_p, C.c_int]
         L.dxe_print_format_ok.argtypes = [C.c_char_p, C.c_int]
         L.dxe_set_sync.argtypes = [C.c_void_p, C.c_int]
+        L.dxe_set_defer.argtypes = [C.c_void_p, C.c_int]
+        L.dxe_flush.argtypes = [C.c_void_p]
+        L.dxe_held.argtypes = [C.c_void_p]
+        L.dxe_held.restype = C.c_size_t
         self.L = L
         self.ex = L.dxe_create()
         assert self.ex
@@ -53,6 +57,13 @@ class InProc:
     def set_graphs(self, on): self.L.dxe_set_graphs(self.ex, int(on))
     def set_fusion(self, on): self.L.dxe_set_fusion(self.ex, int(on))
     def set_sync(self, on): self.L.dxe_set_sync(self.ex, int(on))
+    def set_defer(self, on): self.L.dxe_set_defer(self.ex, int(on))
+    def flush(self): self.L.dxe_flush(self.ex)
+    def held(self): return int(self.L.dxe_held(self.ex))
+
+    def defer_stats(self):
+        held, flushes = (int(x) for x in self._call(self.L.dxe_defer_stats, self.ex).split())
+        return {"held_lines": held, "flushes": flushes}
 
     def fusion_stats(self):
         runs, lines, groups, group_lines = (int(x) for x in self._call(self.L.dxe_fusion_stats, self.ex).split())

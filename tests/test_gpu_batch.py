@@ -349,7 +349,8 @@ def test_recorded_graph_notices_an_in_place_reshape(tmp_path):
 
 def test_config5_block_at_full_size_in_every_mode(tmp_path):
     """The whole BASELINE config-5 block (RMSNorm + gated MLP, 22 deepxIR ops) at its stated size,
-    2048 rows, through the executor line by line, as one batch, as one batch with fused elementwise
+    2048 rows, through the executor line by line, line by line with lines held back until their run is
+    complete (DEEPX_DEFER), as one batch, as one batch with fused elementwise
     runs, and as a recorded graph without and with fused runs.  Every mode against a float64 numpy
     model of the same op sequence with bf16 rounding where the graph stores bf16 (rel 1e-2 per bf16
     rounding; 3e-2 of the output scale end to end, 1e-2 for the normalised activations), and every
@@ -402,10 +403,11 @@ def test_config5_block_at_full_size_in_every_mode(tmp_path):
              f"matmul({n('sg', b16)}, {n('Wd', b16)})->({n('y', b16)})"]
     text = [f"{line} // author=miaobyte id={100 + i}" for i, line in enumerate(block)]
     kept = {}
-    for mode, batched, fused, graphs in (("lines", 0, 0, 0), ("batch", 1, 0, 0), ("batch_fused", 1, 1, 0), ("graph", 1, 0, 1), ("graph_fused", 1, 1, 1)):
+    for mode, batched, fused, graphs in (("lines", 0, 0, 0), ("lines_deferred", 0, 1, 0), ("batch", 1, 0, 0), ("batch_fused", 1, 1, 0), ("graph", 1, 0, 1), ("graph_fused", 1, 1, 1)):
         ex = InProc()
         ex.set_graphs(bool(graphs))
         ex.set_fusion(bool(fused))
+        ex.set_defer(mode == "lines_deferred")
         h = Host(ex, tmp_path)
         for name, arr in (("x", x), ("w", w.reshape(1, Hd)), ("Wg", Wg), ("Wu", Wu), ("Wd", Wd)):
             h.put("f5_" + name, arr, b16)
@@ -416,6 +418,10 @@ def test_config5_block_at_full_size_in_every_mode(tmp_path):
                 h.run(f"constant(var<float32>:0)->({n('y', b16)})")
             rs = ex.execute_batch(text) if batched else [ex.execute(t) for t in text]
             assert all(r.split(" ")[1].startswith("ok") for r in rs), (mode, rs)
+        if mode == "lines_deferred":
+            assert ex.held() == 1  # the down projection waits for a product on the same activations
+            ex.flush()
+            assert ex.held() == 0 and ex.defer_stats()["held_lines"] == 22
         if graphs:
             st = ex.stats()
             assert st["captures"] == 1 and st["replays"] == 1 and st["rejects"] == 0, (mode, st)
@@ -445,7 +451,7 @@ def test_config5_block_at_full_size_in_every_mode(tmp_path):
             assert np.all(np.abs(sgd - sg_model) <= 2.0 ** -6 * np.abs(sg_model) + 1e-37)
             assert np.all(np.abs(y - sgd @ Wd64) <= 1e-2 * (np.abs(sgd) @ np.abs(Wd64)))
         del ex
-    for mode in ("batch", "batch_fused", "graph", "graph_fused"):
+    for mode in ("lines_deferred", "batch", "batch_fused", "graph", "graph_fused"):
         for k in kept["lines"]:
             assert np.array_equal(kept[mode][k], kept["lines"][k]), (mode, k)
 

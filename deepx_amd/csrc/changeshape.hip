@@ -46,7 +46,7 @@ inline int unit_bytes(int64_t run_bytes, std::initializer_list<const void *> ptr
 // single element of type E per row position (innermost axis broadcast) that fills the unit.
 template <typename U, typename I, bool SPLAT, typename E, bool REUSE, bool NTS, int ND>
 __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const void *__restrict__ in_, U *__restrict__ out, I total,
-                                                              I Lu, OuterDims od) {
+                                                              I Lu, OuterDims od, int through) {
     const I tile = (I)kBlock * kGatherUnroll;
     const I stride = (I)gridDim.x * tile;
     for (I base = (I)blockIdx.x * tile; base < total; base += stride) {
@@ -102,7 +102,9 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const void *__restr
         }
 #pragma unroll
         for (int u = 0; u < kGatherUnroll; ++u)
-            if (g[u] < total) st_mode<NTS ? 3 : 0>(&out[g[u]], x[u]);
+            if (g[u] < total) {
+                if constexpr (NTS) st_stream(&out[g[u]], x[u], through); else out[g[u]] = x[u];
+            }
     }
 }
 
@@ -114,8 +116,9 @@ int launch_gather_unit(const void *in, void *out, int64_t rows, int64_t Lu, cons
     for (int d = 0; d < od.n; ++d) od.fsize[d] = make_fastdiv(od.size[d]);
     od.fLu = make_fastdiv((uint32_t)std::min<int64_t>(Lu, 0xffffffffLL));
     unsigned grid = stream_grid(total, (int64_t)kBlock * kGatherUnroll, 0);
+    const int through = use_nt_store((size_t)total * UB) ? 0 : 1;
     if (total < (int64_t)1 << 31) {
-#define DXH_G(ND) gather_rows_kernel<U, uint32_t, SPLAT, E, REUSE, true, ND><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint32_t)total, (uint32_t)Lu, od)
+#define DXH_G(ND) gather_rows_kernel<U, uint32_t, SPLAT, E, REUSE, true, ND><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint32_t)total, (uint32_t)Lu, od, through)
         switch (od.n) {
         case 0: DXH_G(0); break;
         case 1: DXH_G(1); break;
@@ -126,7 +129,7 @@ int launch_gather_unit(const void *in, void *out, int64_t rows, int64_t Lu, cons
         }
 #undef DXH_G
     } else {
-        gather_rows_kernel<U, uint64_t, SPLAT, E, REUSE, true, -1><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint64_t)total, (uint64_t)Lu, od);
+        gather_rows_kernel<U, uint64_t, SPLAT, E, REUSE, true, -1><<<grid, kBlock, 0, st>>>(in, (U *)out, (uint64_t)total, (uint64_t)Lu, od, through);
     }
     return launch_status();
 }
@@ -260,7 +263,7 @@ template <int ES> __device__ __forceinline__ void transpose_block(const tt_u32x4
 template <int ES>
 __global__ __launch_bounds__(kBlock) void tile_transpose_vec_kernel(const char *__restrict__ in, char *__restrict__ out, int64_t nA,
                                                                      int64_t sA, int64_t nC, int64_t oC, int tilesA, int tilesC,
-                                                                     BatchDims bd) {
+                                                                     BatchDims bd, int through) {
     constexpr int V = 16 / ES, T = 16 * V;
     __shared__ tt_u32x4 lds[kBlock * V];  // [c in tile][a-block ^ c-block]
     // Diagonal order: consecutive workgroups step along C and along A together, so that neither
@@ -301,7 +304,7 @@ __global__ __launch_bounds__(kBlock) void tile_transpose_vec_kernel(const char *
             const int c = crow + 16 * i;
             const int64_t gc = (int64_t)tc * T + c;
             if (gc < nC && a0 < nA)
-                st_mode<3>(reinterpret_cast<tt_u32x4 *>(out + (ooff + gc * oC + a0) * ES), lds[c * 16 + (ablk ^ ((c / V) & 15))]);
+                st_stream(reinterpret_cast<tt_u32x4 *>(out + (ooff + gc * oC + a0) * ES), lds[c * 16 + (ablk ^ ((c / V) & 15))], through);
         }
     }
 }
@@ -320,7 +323,7 @@ struct ConcatSrcs {
 // blockIdx.y = source, so run / prefix / pointer are wave-uniform scalars and the only per-lane
 // work before the data load is one divide-free division.
 template <typename U, bool FAST>
-__global__ __launch_bounds__(kBlock) void concat_kernel(ConcatSrcs s, U *__restrict__ out, int64_t out_row, int64_t outer) {
+__global__ __launch_bounds__(kBlock) void concat_kernel(ConcatSrcs s, U *__restrict__ out, int64_t out_row, int64_t outer, int through) {
     const int i = blockIdx.y;
     const U *__restrict__ src = nullptr;
     int64_t run = 1, pref = 0;
@@ -340,7 +343,7 @@ __global__ __launch_bounds__(kBlock) void concat_kernel(ConcatSrcs s, U *__restr
             o = g / run;
             v = g - o * run;
         }
-        st_mode<3>(&out[o * out_row + pref + v], ld_nt(&src[g]));
+        st_stream(&out[o * out_row + pref + v], ld_nt(&src[g]), through);
     }
 }
 
@@ -348,7 +351,7 @@ __global__ __launch_bounds__(kBlock) void concat_kernel(ConcatSrcs s, U *__restr
 template <typename U, typename IT>
 __global__ __launch_bounds__(kBlock) void indexselect_kernel(const U *__restrict__ in, const IT *__restrict__ index,
                                                               U *__restrict__ out, int64_t total, int64_t Lu, int64_t M,
-                                                              int64_t adim, FastDiv fLu, FastDiv fM, bool fast) {
+                                                              int64_t adim, FastDiv fLu, FastDiv fM, bool fast, int through) {
     const int64_t tile = (int64_t)kBlock * kGatherUnroll;
     const int64_t stride = (int64_t)gridDim.x * tile;
     for (int64_t base = (int64_t)blockIdx.x * tile; base < total; base += stride) {
@@ -374,7 +377,7 @@ __global__ __launch_bounds__(kBlock) void indexselect_kernel(const U *__restrict
         }
 #pragma unroll
         for (int u = 0; u < kGatherUnroll; ++u)
-            if (g[u] < total) st_mode<3>(&out[g[u]], x[u]);
+            if (g[u] < total) st_stream(&out[g[u]], x[u], through);
     }
 }
 
@@ -522,7 +525,8 @@ int dxh_transpose(int dtype, const void *in, const int32_t *shape, int ndim, con
         const int T = 16 * V;
         const int64_t tilesA = (nA + T - 1) / T, tilesC = (nC + T - 1) / T, blocks = batch * tilesA * tilesC;
         if (blocks > 0x7fffffff) return DXH_ERR_SHAPE;
-#define DXH_TT(ES) tile_transpose_vec_kernel<ES><<<(unsigned)blocks, kBlock, 0, st>>>((const char *)in, (char *)out, nA, sA, nC, oC, (int)tilesA, (int)tilesC, bd)
+        const int through = use_nt_store((size_t)(batch * nA * nC) * (size_t)es_eff) ? 0 : 1;
+#define DXH_TT(ES) tile_transpose_vec_kernel<ES><<<(unsigned)blocks, kBlock, 0, st>>>((const char *)in, (char *)out, nA, sA, nC, oC, (int)tilesA, (int)tilesC, bd, through)
         switch (es_eff) {
         case 16: DXH_TT(16); break;
         case 8: DXH_TT(8); break;
@@ -591,10 +595,11 @@ int dxh_concat(int dtype, const void *const *ins, int nins, const int32_t *axis_
         int64_t max_units = 0;
         for (int k = 0; k < s.n; ++k) max_units = std::max(max_units, s.run[k] * outer);
         const bool fast = max_units < ((int64_t)1 << 32);
+        const int through = use_nt_store((size_t)(out_row * outer) * (size_t)ub) ? 0 : 1;
         dim3 grid(stream_grid(max_units, kBlock, 0) > 0x7fffffffu ? 0x7fffffffu : stream_grid(max_units, kBlock, 0), (unsigned)s.n);
 #define DXH_CC(U)                                                                           \
-        if (fast) concat_kernel<U, true><<<grid, kBlock, 0, st>>>(s, (U *)out, out_row, outer); \
-        else concat_kernel<U, false><<<grid, kBlock, 0, st>>>(s, (U *)out, out_row, outer);
+        if (fast) concat_kernel<U, true><<<grid, kBlock, 0, st>>>(s, (U *)out, out_row, outer, through); \
+        else concat_kernel<U, false><<<grid, kBlock, 0, st>>>(s, (U *)out, out_row, outer, through);
         switch (ub) {
         case 16: DXH_CC(uint4) break;
         case 8: DXH_CC(uint64_t) break;
@@ -659,12 +664,13 @@ int dxh_indexselect(int dtype, const void *in, const int32_t *in_shape, int in_n
     hipStream_t st = as_stream(stream);
     unsigned grid = stream_grid(total, (int64_t)kBlock * kGatherUnroll, 0);
     const bool fast = total < ((int64_t)1 << 32) && Lu < ((int64_t)1 << 32) && m < ((int64_t)1 << 32);
+    const int through = use_nt_store((size_t)total * (size_t)ub) ? 0 : 1;
     const FastDiv fLu = make_fastdiv((uint32_t)std::min<int64_t>(Lu, 0xffffffffLL)), fM = make_fastdiv((uint32_t)std::min<int64_t>(m, 0xffffffffLL));
 #define DXH_IS(U)                                                                                                      \
     if (index_dtype == DXH_I64)                                                                                        \
-        indexselect_kernel<U, int64_t><<<grid, kBlock, 0, st>>>((const U *)in, (const int64_t *)index, (U *)out, total, Lu, m, adim, fLu, fM, fast); \
+        indexselect_kernel<U, int64_t><<<grid, kBlock, 0, st>>>((const U *)in, (const int64_t *)index, (U *)out, total, Lu, m, adim, fLu, fM, fast, through); \
     else                                                                                                               \
-        indexselect_kernel<U, int32_t><<<grid, kBlock, 0, st>>>((const U *)in, (const int32_t *)index, (U *)out, total, Lu, m, adim, fLu, fM, fast);
+        indexselect_kernel<U, int32_t><<<grid, kBlock, 0, st>>>((const U *)in, (const int32_t *)index, (U *)out, total, Lu, m, adim, fLu, fM, fast, through);
     switch (ub) {
     case 16: DXH_IS(uint4) break;
     case 8: DXH_IS(uint64_t) break;

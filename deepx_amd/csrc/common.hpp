@@ -141,6 +141,11 @@ template <int ST, typename VT> __device__ inline void st_mode(VT *p, const VT &v
         st_nt(p, v);
     }
 }
+// store of a write-dominated stream (transposes, broadcasts, gathers, concat): write-through when the launch's output
+// is small enough for the next kernel to find it in the last-level cache (!use_nt_store), else nt at agent scope
+template <typename VT> __device__ inline void st_stream(VT *p, const VT &v, int through) {
+    if (through) st_mode<2>(p, v); else st_mode<3>(p, v);
+}
 template <bool NTL, typename VT> __device__ inline VT ld_sel(const VT *p) {
     if constexpr (NTL) return ld_nt(p);
     else return *p;

@@ -289,6 +289,38 @@ def test_misaligned_pointers_take_scalar_path(dxh, orc):
     assert dxh.dxh_add(dx.F32, C.c_void_p(da.ptr.value + 1), db.ptr, dc.ptr, n, None) == -5
 
 
+@pytest.mark.parametrize("dtype", [dx.F64, dx.F32, dx.BF16, dx.I64, dx.I32, dx.I16, dx.I8])
+def test_store_policy_leaves_the_bits_alone(dxh, orc, dtype):
+    """Outputs of up to 32 MiB leave with write-through stores, larger ones with non-temporal stores
+    (knob 0 moves the limit).  Every width of both kinds: 16-byte vectors, and the 8-, 4-, 2- and 1-byte
+    stores of a tensor that starts off a 16-byte boundary; add, a scalar form and a cast against the
+    oracle under either policy."""
+    rng = np.random.default_rng(160 + dtype)
+    n = 40007
+    es = np.dtype(H.NP[dtype]).itemsize
+    a, b = H.rand(rng, dtype, n + 16), H.rand(rng, dtype, n + 16)
+    want = np.empty(n, dtype=a.dtype)
+    for shift in (0, 1):  # elements off the allocation's start: 0 keeps 16-byte alignment, 1 loses it
+        av, bv = a[shift:shift + n].copy(), b[shift:shift + n].copy()
+        assert orc.orc_add(dtype, hp(av), hp(bv), hp(want), n) == 0
+        for limit in (1 << 40, 0):  # everything written through / everything non-temporal
+            dx.check(dxh.dxh_tune(0, limit))
+            try:
+                da, db, dc = Dev(a), Dev(b), Dev.empty(n + 16, a.dtype)
+                at = lambda d: C.c_void_p(d.ptr.value + shift * es)
+                dx.check(dxh.dxh_add(dtype, at(da), at(db), at(dc), n, None), "add")
+                assert np.array_equal(dc.get()[shift:shift + n], want), (shift, limit)
+                dst = dx.F32 if dtype != dx.F32 else dx.BF16
+                dd = Dev.empty(n + 16, H.NP[dst])
+                ds = np.dtype(H.NP[dst]).itemsize
+                dx.check(dxh.dxh_todtype(dtype, at(da), dst, C.c_void_p(dd.ptr.value + shift * ds), n, None), "todtype")
+                cast_want = np.empty(n, dtype=H.NP[dst])
+                assert orc.orc_todtype(dtype, hp(av), dst, hp(cast_want), n) == 0
+                assert np.array_equal(dd.get()[shift:shift + n], cast_want), (shift, limit)
+            finally:
+                dx.check(dxh.dxh_tune(0, 32 << 20))
+
+
 def test_error_codes(dxh):
     a = Dev(np.zeros(16, dtype=np.float32))
     assert dxh.dxh_add(12345, a.ptr, a.ptr, a.ptr, 16, None) == -1

@@ -462,11 +462,12 @@ def test_random_batches_fused_equal_line_by_line(tmp_path):
     vectors and sums over the last axis, in random order.  Whatever runs the planner forms — one
     dtype, mixed, with row or column vectors, with a row sum inside, cut at a vector that would be
     overwritten while other lanes still read it — every tensor must end up with the bits of the
-    line-by-line execution, and every line must get the reply it gets on its own."""
+    line-by-line execution, and every line must get the reply it gets on its own.  The same lines sent
+    one by one with runs held back (DEEPX_DEFER) must do the same."""
     rng = np.random.default_rng(20251)
     dts = ["float32", "bfloat16", "float16"]
     code = {"float32": dx.F32, "bfloat16": dx.BF16, "float16": dx.F16}
-    fused_lines = 0
+    fused_lines = held_lines = 0
     for trial in range(72):
         rows, cols = [(16, 64), (5, 12), (64, 896), (3, 1000), (33, 260), (128, 32)][trial % 6]
         shapes = {"F": [rows, cols], "C": [rows, 1], "R": [1, cols]}
@@ -504,28 +505,32 @@ def test_random_batches_fused_equal_line_by_line(tmp_path):
                 lines.append(f"sum({T(pick('F', dt)[0], dt)}, {V([-1])}, var<bool>:true)->({T(pick('C', dt)[0], dt)})")
         text = [f"{line} // author=miaobyte id={900 + i}" for i, line in enumerate(lines)]
         results, replies = {}, {}
-        for mode in ("lines", "fused"):
+        for mode in ("lines", "fused", "held"):
             ex = InProc()
-            ex.set_fusion(mode == "fused")
+            ex.set_fusion(mode != "lines")
+            ex.set_defer(mode == "held")
             h = Host(ex, tmp_path)
             for name, k, dt in pool:
                 h.put(name, data[name], dt)
-            replies[mode] = [ex.execute(t) for t in text] if mode == "lines" else ex.execute_batch(text)
+            replies[mode] = ex.execute_batch(text) if mode == "fused" else [ex.execute(t) for t in text]
             if mode == "fused":
                 fused_lines += ex.fusion_stats()["lines"]
+            if mode == "held":
+                held_lines += ex.defer_stats()["held_lines"]
             results[mode] = {name: h.get(name) for name, _, _ in pool}
             del ex
-        assert [r.split("//")[0] for r in replies["fused"]] == [r.split("//")[0] for r in replies["lines"]], (trial, lines)
-        for name, _, _ in pool:
-            a, b = results["lines"][name], results["fused"][name]
-            same = np.array_equal(a.view(np.uint8), b.view(np.uint8))
-            if not same and a.dtype.kind == "f":
-                same = np.array_equal(a, b, equal_nan=True)
-            if not same:  # 16-bit floats come back as raw bits: NaN payloads aside they must agree
-                fa, fb = H.to_float(a.reshape(-1), code[[p for p in pool if p[0] == name][0][2]]), H.to_float(b.reshape(-1), code[[p for p in pool if p[0] == name][0][2]])
-                same = np.array_equal(fa, fb, equal_nan=True)
-            assert same, (trial, name, lines)
-    assert fused_lines > 400  # the batches did form runs
+        for mode in ("fused", "held"):
+            assert [r.split("//")[0] for r in replies[mode]] == [r.split("//")[0] for r in replies["lines"]], (trial, mode, lines)
+            for name, _, _ in pool:
+                a, b = results["lines"][name], results[mode][name]
+                same = np.array_equal(a.view(np.uint8), b.view(np.uint8))
+                if not same and a.dtype.kind == "f":
+                    same = np.array_equal(a, b, equal_nan=True)
+                if not same:  # 16-bit floats come back as raw bits: NaN payloads aside they must agree
+                    fa, fb = H.to_float(a.reshape(-1), code[[p for p in pool if p[0] == name][0][2]]), H.to_float(b.reshape(-1), code[[p for p in pool if p[0] == name][0][2]])
+                    same = np.array_equal(fa, fb, equal_nan=True)
+                assert same, (trial, mode, name, lines)
+    assert fused_lines > 400 and held_lines > 400  # the batches did form runs, the single lines were held
 
 
 def test_square_view_row_sum_without_keepdims_fuses(tmp_path):

@@ -165,8 +165,8 @@ public:
                 held_items_.back().resp = resp;
                 return resp.to_string();
             }
-            flush();
         }
+        flush();  // whatever is held comes first (also when a switch was turned while lines were held)
         resp.start_at = std::chrono::system_clock::now();
         int rc = 0;
         std::string message;

@@ -121,6 +121,16 @@ def test_a_line_that_needs_results_launches_what_is_held(tmp_path):
     ex.set_defer(False)
     assert ex.held() == 0
     assert np.array_equal(h.get("dn_y"), (x * 2 + 1) * 2)
+    # a switch turned while lines are held: they still come before the next line
+    ex.set_defer(True)
+    assert ex.execute(f"addscalar({T('dn_y')}, var<float32>:1)->({T('dn_z')}) // id=60").startswith("60 ok")
+    assert ex.held() == 1
+    ex.set_sync(True)
+    assert ex.execute(f"mulscalar({T('dn_z')}, var<float32>:3)->({T('dn_y')}) // id=61").startswith("61 ok")
+    assert ex.held() == 0
+    ex.set_sync(False)
+    assert np.array_equal(h.get("dn_y"), (((x * 2 + 1) * 2) + 1) * 3)
+    ex.set_defer(False)
     # deltensor of an operand of a held line: the line runs first, then the tensor goes
     ex.set_defer(True)
     assert ex.execute(f"mulscalar({T('dn_x')}, var<float32>:5)->({T('dn_z')}) // id=53").startswith("53 ok")

@@ -449,9 +449,13 @@ static int64_t choose_uncut_tile(int64_t batch, int64_t m, int64_t k, int64_t n,
         if (dma_ok) {
             const double c11 = one_per_cu(160, 256, 0.96, 5.5), c12 = one_per_cu(128, 256, 0.85, 5.0), c13 = one_per_cu(256, 128, 0.76, 3.5) - (tiles(256, 128) <= cus / 2 ? ksteps * 0.09 : 0.0);  // 0.52 us per step up to half the CUs
             double best = choice == 1 ? c1 : choice == 2 ? c2 : choice == 4 ? c4 : c6;
-            if (c11 < best && tiles(160, 256) <= cus) { best = c11; choice = 11; }
-            if (c12 < best && tiles(128, 256) <= cus) { best = c12; choice = 12; }
-            if (c13 < best && tiles(256, 128) <= cus) { best = c13; choice = 13; }
+            // ... except on a short K (up to 16 steps), where a round is mostly its prologue and its C burst and the
+            // operands are small: there the estimate holds over several rounds too (8192x896x4864: 73 us with 160
+            // rows, 86 with 128x128 two to a CU, 79 with 256x256; 4096x896x4864: 36.7 against 43.5)
+            const bool any_rounds = ksteps <= 16.0;
+            if (c11 < best && (any_rounds || tiles(160, 256) <= cus)) { best = c11; choice = 11; }
+            if (c12 < best && (any_rounds || tiles(128, 256) <= cus)) { best = c12; choice = 12; }
+            if (c13 < best && (any_rounds || tiles(256, 128) <= cus)) { best = c13; choice = 13; }
         }
     }
     else choice = 5;  // 1024x8192x1024 as 128 tiles of 128x64: 38 us, 31 us with 256 64x64 tiles

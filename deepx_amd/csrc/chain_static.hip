@@ -205,6 +205,15 @@ using SiluGateProg = SProg<SList<SIn<0, FULL>, SIn<0, FULL>>,
 using SiluProg = SProg<SList<SIn<0, FULL>>,
                        SList<SOp<DXH_CHAIN_MULSCALAR, 0, 0, 0, FULL>, SOp<DXH_CHAIN_EXP, RES + 0, 0, 0, FULL>, SOp<DXH_CHAIN_ADDSCALAR, RES + 1, 0, 0, FULL>,
                              SOp<DXH_CHAIN_RDIVSCALAR, RES + 2, 0, 0, FULL>, SOp<DXH_CHAIN_MUL, 0, RES + 3, 0, FULL>>>;
+// The same two as swish(x, beta) spells them (activite.py:15-16: x * sigmoid(x * beta), sigmoid(t) = 1 / (exp(t * -1) + 1)):
+// one more line in front, t = x * beta
+using SwishGateProg = SProg<SList<SIn<0, FULL>, SIn<0, FULL>>,
+                            SList<SOp<DXH_CHAIN_MULSCALAR, 0, 0, 0, FULL>, SOp<DXH_CHAIN_MULSCALAR, RES + 0, 0, 0, FULL>, SOp<DXH_CHAIN_EXP, RES + 1, 0, 0, FULL>,
+                                  SOp<DXH_CHAIN_ADDSCALAR, RES + 2, 0, 0, FULL>, SOp<DXH_CHAIN_RDIVSCALAR, RES + 3, 0, 0, FULL>, SOp<DXH_CHAIN_MUL, 0, RES + 4, 0, FULL>,
+                                  SOp<DXH_CHAIN_MUL, RES + 5, 1, 0, FULL>>>;
+using SwishProg = SProg<SList<SIn<0, FULL>>,
+                        SList<SOp<DXH_CHAIN_MULSCALAR, 0, 0, 0, FULL>, SOp<DXH_CHAIN_MULSCALAR, RES + 0, 0, 0, FULL>, SOp<DXH_CHAIN_EXP, RES + 1, 0, 0, FULL>,
+                              SOp<DXH_CHAIN_ADDSCALAR, RES + 2, 0, 0, FULL>, SOp<DXH_CHAIN_RDIVSCALAR, RES + 3, 0, 0, FULL>, SOp<DXH_CHAIN_MUL, 0, RES + 4, 0, FULL>>>;
 
 std::atomic<int64_t> g_static_launches{0}, g_interpreted_launches{0};
 
@@ -333,6 +342,8 @@ int static_chain_try(int dtype, const void *const *inputs, int n_inputs, const d
     }
     DXH_TRY_FLAT(SiluGateProg);
     DXH_TRY_FLAT(SiluProg);
+    DXH_TRY_FLAT(SwishGateProg);
+    DXH_TRY_FLAT(SwishProg);
 #undef DXH_TRY_FLAT
     if (rc == DXH_OK) g_static_launches.fetch_add(1, std::memory_order_relaxed);
     return rc;

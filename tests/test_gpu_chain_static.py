@@ -188,6 +188,59 @@ def test_silu_gate_compiled(dxh, orc, dt):
         assert np.all(np.abs(H.to_float(comp[-1].get(), dt) - ref) <= tol * np.abs(ref) + 1e-6)
 
 
+@pytest.mark.parametrize("dt", [dx.F32, dx.BF16, dx.F16])
+@pytest.mark.parametrize("gated", [True, False])
+def test_swish_as_the_front_spells_it(dxh, orc, dt, gated):
+    """swish(x, beta) of the front is x * sigmoid(x * beta) with sigmoid(t) = 1 / (exp(t * -1) + 1) (activite.py:10-16):
+    one more mulscalar in front of the sequence above, seven lines with the gate's `* up`.  Compiled, interpreted
+    and as separate launches: the same bits in every tensor."""
+    rng = np.random.default_rng(70 + dt)
+    for n, beta in ((2048 * 896, 1.0), (8 * 1031, 1.702)):
+        x, u = Dev(H.rand(rng, dt, n, -6.0, 6.0)), Dev(H.rand(rng, dt, n, -2.0, 2.0))  # exp(6 * 1.702) still fits float16
+        prog = [("mulscalar", 0, 0, beta), ("mulscalar", R + 0, 0, -1.0), ("exp", R + 1, 0, 0), ("addscalar", R + 2, 0, 1.0),
+                ("rdivscalar", R + 3, 0, 1.0), ("mul", 0, R + 4, 0)] + ([("mul", R + 5, 1, 0)] if gated else [])
+        ins = [x, u] if gated else [x]
+
+        def run():
+            outs = [Dev.empty(n, H.NP[dt]) for _ in prog]
+            ops = (dx.ChainOp * len(prog))(*[dx.ChainOp(dx.CHAIN_CODES.index(nm), l, r, dx.scalar(s), outs[k].ptr) for k, (nm, l, r, s) in enumerate(prog)])
+            dx.check(dxh.dxh_chain(dt, (C.c_void_p * len(ins))(*[t.ptr for t in ins]), len(ins), ops, len(prog), n, None), "chain")
+            return outs
+
+        c0, i0 = stats(dxh)
+        comp = run()
+        assert stats(dxh) == (c0 + 1, i0)
+        dx.check(dxh.dxh_tune(KNOB_STATIC, 0))
+        try:
+            interp = run()
+            assert stats(dxh) == (c0 + 1, i0 + 1)
+        finally:
+            dx.check(dxh.dxh_tune(KNOB_STATIC, 1))
+        sep = []
+        for k, (nm, l, r, sc) in enumerate(prog):
+            a = ins[l] if l < R else sep[l - R]
+            out = Dev.empty(n, H.NP[dt])
+            if nm == "mul":
+                b = ins[r] if r < R else sep[r - R]
+                dx.check(dxh.dxh_mul(dt, a.ptr, b.ptr, out.ptr, n, None))
+            elif nm == "exp":
+                dx.check(dxh.dxh_exp(dt, a.ptr, out.ptr, n, None))
+            elif nm == "rdivscalar":
+                dx.check(dxh.dxh_rdivscalar(dt, dx.scalar(sc), a.ptr, out.ptr, n, None))
+            else:
+                dx.check(getattr(dxh, "dxh_" + nm)(dt, a.ptr, dx.scalar(sc), out.ptr, n, None))
+            sep.append(out)
+        for k in range(len(prog)):
+            assert same_bits(comp[k], sep[k]) and same_bits(interp[k], sep[k]), (n, k)
+        x64 = H.to_float(x.get(), dt)
+        ref = x64 / (1.0 + np.exp(-x64 * H.to_float(H.to_storage(np.array([beta]), dt), dt)[0]))
+        if gated:
+            ref = ref * H.to_float(u.get(), dt)
+        # the rounding of x * beta to the dtype is a relative error of the exponent: exp turns it into |x beta| times as much
+        tol = 1e-5 if dt == dx.F32 else 2.0 ** -5 if dt == dx.BF16 else 2.0 ** -8
+        assert np.all(np.abs(H.to_float(comp[-1].get(), dt) - ref) <= tol * (1.0 + np.abs(x64 * beta)) * np.abs(ref) + 1e-6)
+
+
 def test_attention_sized_softmax_compiled_equals_separate(dxh):
     """[14 * 2048, 2048] fp32 scores (one head group of the BASELINE attention shape): the compiled softmax against
     the separate launches, compared on the device."""

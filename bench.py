@@ -530,9 +530,17 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
                 e["interpreted_ms"] = None  # rows too long (or 16-bit row reductions) for the interpreting kernel's lane layout
         finally:
             dx.check(L.dxh_tune(12, 1))
+        # outputs of up to 32 MiB leave with write-through stores so that the next kernel finds them in the last-level
+        # cache; here, alone and on rotating buffers, nothing reads them: the same launches with non-temporal stores
+        dx.check(L.dxh_tune(0, 0))
+        try:
+            e["with_nt_stores_ms"] = round(time_op(L, dx, torch, Events, ev, lambda i: calls[i % len(calls)]()), 5)
+        finally:
+            dx.check(L.dxh_tune(0, 32 << 20))
         fused[label] = e
     fused["note"] = ("one launch per run through the library's compiled kernel for that sequence; interpreted_ms = the same launch through "
-                     "the op-table interpreter; as separate launches the lines take the sum of the glue_ops entries above")
+                     "the op-table interpreter; with_nt_stores_ms = the compiled kernel with DXH_TUNE_NT_STORE_BYTES 0 (what the run costs when "
+                     "nothing reads its outputs from the cache afterwards); as separate launches the lines take the sum of the glue_ops entries above")
     c5["fused_runs(one launch each)"] = fused
     del runs
     del g16, u16, o16, x16, x32, o32, col

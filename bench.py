@@ -281,6 +281,7 @@ def main():
         del Xs, Ps
         torch.cuda.empty_cache()
         per_op.update(bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr))
+        per_op["config2"]["step_over_deepxIR"] = config2_step_over_ir(step_bytes)
 
     # ---------------- CPU baseline: the oracle's restatement of op-ompsimd's reduce ---------
     cpu = None
@@ -634,6 +635,7 @@ def _executor_lib():
     E.dxe_set_sync.argtypes = [C.c_void_p, C.c_int]
     E.dxe_set_defer.argtypes = [C.c_void_p, C.c_int]
     E.dxe_flush.argtypes = [C.c_void_p]
+    E.dxe_set_streams.argtypes = [C.c_void_p, C.c_int]
     return E
 
 
@@ -690,6 +692,59 @@ def lines_over_ir(setup, block, iters=30, only=None):
         out[label] = round((time.perf_counter() - t0) / iters * 1e6, 1)
         if any(" ok" not in r.split("//")[0] for r in buf.value.decode().split("\n")):
             raise RuntimeError("block failed: " + buf.value.decode())
+        E.dxe_destroy(ex)
+    return out
+
+
+def config2_step_over_ir(step_bytes, iters=30):
+    """The config-2 step (ten reductions) as one datagram of ten deepxIR lines through the executor's dispatch core:
+    in order on the default stream, and with independent lines spread over side streams (the DEEPX_STREAMS switch:
+    no line of the step reads what another writes, so the end of one launch runs under the start of the next).
+    Three copies of the input in rotation, as in the headline step."""
+    import ctypes as C
+    from deepx_amd import lib as dx
+    L = dx.load()
+    E = _executor_lib()
+    T = lambda n: f"tensor<float32>:c2_{n}"
+    V = lambda v: "vector<int32>:[" + " ".join(str(x) for x in v) + "]"
+    setup = [f"newtensor({V([8192, 8192])})->({T('X%d' % i)})" for i in range(3)] + [f"newtensor({V([8192, 64])})->({T('P%d' % i)})" for i in range(3)]
+    setup += [f"uniform(var<float32>:0, var<float32>:1, var<int32>:{7 + i})->({T('X%d' % i)}) // author=miaobyte" for i in range(3)]
+    setup += [f"uniform(var<float32>:0.9, var<float32>:1.1, var<int32>:{17 + i})->({T('P%d' % i)}) // author=miaobyte" for i in range(3)]
+    outs = []
+    for kd in (1, 0):
+        for name in ("s1", "mx", "mn", "s0", "pr"):
+            shape = ([8192, 1] if name != "s0" else [1, 8192]) if kd else [8192]
+            setup.append(f"newtensor({V(shape)})->({T(f'{name}_kd{kd}')})")
+    texts = []
+    for i in range(3):
+        lines = []
+        for kd in (1, 0):
+            kb = "var<bool>:true" if kd else "var<bool>:false"
+            lines += [f"sum({T('X%d' % i)}, {V([1])}, {kb})->({T(f's1_kd{kd}')})", f"reducemax({T('X%d' % i)}, {V([1])}, {kb})->({T(f'mx_kd{kd}')})",
+                      f"reducemin({T('X%d' % i)}, {V([1])}, {kb})->({T(f'mn_kd{kd}')})", f"sum({T('X%d' % i)}, {V([0])}, {kb})->({T(f's0_kd{kd}')})",
+                      f"prod({T('P%d' % i)}, {V([1])}, {kb})->({T(f'pr_kd{kd}')})"]
+        texts.append("\n".join(f"{l} // author=miaobyte id={k + 1}" for k, l in enumerate(lines)).encode())
+    out = {"ops": 10, "bytes": step_bytes}
+    for label, streams in (("one_batch_us", 1), ("one_batch_side_streams_us", 3)):
+        ex = E.dxe_create()
+        buf = C.create_string_buffer(1 << 16)
+        for line in setup:
+            E.dxe_execute(ex, line.encode(), buf, len(buf))
+            if " ok" not in buf.value.decode().split("//")[0]:
+                raise RuntimeError(f"{line}: {buf.value.decode()}")
+        E.dxe_set_streams(ex, streams)
+        for r in range(6):
+            E.dxe_execute_batch(ex, texts[r % 3], buf, len(buf))
+        dx.check(L.dxh_device_sync())
+        t0 = time.perf_counter()
+        for r in range(iters):
+            E.dxe_execute_batch(ex, texts[r % 3], buf, len(buf))
+        dx.check(L.dxh_device_sync())
+        us = (time.perf_counter() - t0) / iters * 1e6
+        if any(" ok" not in r.split("//")[0] for r in buf.value.decode().split("\n")):
+            raise RuntimeError("step failed: " + buf.value.decode())
+        out[label] = round(us, 1)
+        out[label.replace("_us", "_GB/s")] = round(step_bytes / us / 1e3, 1)
         E.dxe_destroy(ex)
     return out
 

@@ -135,6 +135,10 @@ int dxh_event_record(void *event, void *stream) {
     if (!event) return DXH_ERR_ARG;
     return (int)hipEventRecord((hipEvent_t)event, as_stream(stream));
 }
+int dxh_stream_wait_event(void *stream, void *event) {
+    if (!event) return DXH_ERR_ARG;
+    return (int)hipStreamWaitEvent(as_stream(stream), (hipEvent_t)event, 0);
+}
 int dxh_event_sync(void *event) {
     if (!event) return DXH_ERR_ARG;
     return (int)hipEventSynchronize((hipEvent_t)event);

@@ -53,6 +53,10 @@ DXE_API size_t dxe_defer_stats(void *ex, char *out, size_t buflen) {
     const auto &s = static_cast<Executor *>(ex)->stats;
     return copy_out(std::to_string(s.held_lines) + " " + std::to_string(s.flushes), out, buflen);
 }
+// independent kernel-only lines of a batch on n side streams in turn (the DEEPX_STREAMS switch; 1 = in order on the default stream);
+// dxe_side_launches: how many launches went to a side stream so far
+DXE_API void dxe_set_streams(void *ex, int n) { static_cast<Executor *>(ex)->streams = n < 1 ? 1 : n > 8 ? 8 : n; }
+DXE_API size_t dxe_side_launches(void *ex) { return (size_t)static_cast<Executor *>(ex)->stats.side_launches; }
 DXE_API size_t dxe_fusion_stats(void *ex, char *out, size_t buflen) {
     const auto &s = static_cast<Executor *>(ex)->stats;
     return copy_out(std::to_string(s.fused_runs) + " " + std::to_string(s.fused_lines) + " " + std::to_string(s.matmul_groups) + " " + std::to_string(s.matmul_lines), out, buflen);

@@ -6,6 +6,7 @@
 //   DEEPX_REMOTE_QUIT 1: honour the `__quit__` line from any source address (default: loopback only)
 //   DEEPX_IR_LOG   1|true: echo every instruction
 //   DEEPX_SYNC     1: wait for the device before every reply (default: reply at launch, as op-cuda does)
+//   DEEPX_STREAMS  n >= 2: independent kernel-only lines of a datagram go to n side streams in turn and overlap
 //   DEEPX_DEFER    1: hold lines that can share a launch with the next one (DEEPX_DEFER_US: longest wait for it, default 200)
 //   DEEPX_OPLIST   path: write the generated op table (markdown) there, as the reference writes
 //                  docs/executor/op-mem-*/list.md at start-up

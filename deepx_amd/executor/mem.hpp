@@ -82,26 +82,33 @@ public:
     void *stream = nullptr;
     bool recording = false;
 
-    // reusable device scratch for reductions (grown on demand, never shrunk)
+    // reusable device scratch for reductions and products (grown on demand, never shrunk).  Launches that may run
+    // side by side on two streams must not share it: the executor names the scratch an op is to use (`scratch_of`,
+    // NULL = the one of in-order execution, which recorded graphs pin) before it runs the op.
+    void *scratch_of = nullptr;
     void *workspace(size_t bytes) {
-        if (bytes > ws_bytes_) {
+        Scratch &w = scratch_[scratch_of];
+        if (bytes > w.bytes) {
             if (recording) throw std::runtime_error("workspace would grow while recording a graph");
-            if (ws_) { dxh_device_sync(); dxh_free(ws_); ws_ = nullptr; ws_bytes_ = 0; }
+            if (w.ptr) { dxh_device_sync(); dxh_free(w.ptr); w.ptr = nullptr; w.bytes = 0; }
             size_t want = std::max<size_t>(bytes, (size_t)4 << 20);
-            dxh_check(dxh_malloc(&ws_, want), "workspace dxh_malloc");
-            ws_bytes_ = want;
+            dxh_check(dxh_malloc(&w.ptr, want), "workspace dxh_malloc");
+            w.bytes = want;
         }
-        return ws_;
+        return w.ptr;
     }
-    size_t workspace_bytes() const { return ws_bytes_; }
-    const void *workspace_ptr() const { return ws_; }
-    ~Mem() { tensors_.clear(); if (ws_) dxh_free(ws_); }
+    size_t workspace_bytes() const { auto it = scratch_.find(scratch_of); return it == scratch_.end() ? 0 : it->second.bytes; }
+    const void *workspace_ptr() const { auto it = scratch_.find(scratch_of); return it == scratch_.end() ? nullptr : it->second.ptr; }
+    ~Mem() {
+        tensors_.clear();
+        for (auto &kv : scratch_) if (kv.second.ptr) dxh_free(kv.second.ptr);
+    }
 
 private:
     std::unordered_map<std::string, std::shared_ptr<Tensor>> tensors_;
     std::unordered_map<std::string, ArgValue> args_;
-    void *ws_ = nullptr;
-    size_t ws_bytes_ = 0;
+    struct Scratch { void *ptr = nullptr; size_t bytes = 0; };
+    std::unordered_map<void *, Scratch> scratch_;  // by `scratch_of`
 };
 
 }  // namespace deepx

@@ -91,6 +91,7 @@ SIGNATURES = {
     "dxh_event_destroy": ([_p], _i),
     "dxh_event_record": ([_p, _p], _i),
     "dxh_event_sync": ([_p], _i),
+    "dxh_stream_wait_event": ([_p, _p], _i),
     "dxh_event_elapsed_ms": ([_p, _p, C.POINTER(_f)], _i),
     "dxh_ipc_export": ([_p, _p], _i),
     "dxh_ipc_open": ([_p, C.POINTER(_p)], _i),

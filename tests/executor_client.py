@@ -40,6 +40,9 @@ class InProc:
         L.dxe_print_format_ok.argtypes = [C.c_char_p, C.c_int]
         L.dxe_set_sync.argtypes = [C.c_void_p, C.c_int]
         L.dxe_set_defer.argtypes = [C.c_void_p, C.c_int]
+        L.dxe_set_streams.argtypes = [C.c_void_p, C.c_int]
+        L.dxe_side_launches.argtypes = [C.c_void_p]
+        L.dxe_side_launches.restype = C.c_size_t
         L.dxe_flush.argtypes = [C.c_void_p]
         L.dxe_held.argtypes = [C.c_void_p]
         L.dxe_held.restype = C.c_size_t
@@ -58,6 +61,8 @@ class InProc:
     def set_fusion(self, on): self.L.dxe_set_fusion(self.ex, int(on))
     def set_sync(self, on): self.L.dxe_set_sync(self.ex, int(on))
     def set_defer(self, on): self.L.dxe_set_defer(self.ex, int(on))
+    def set_streams(self, n): self.L.dxe_set_streams(self.ex, int(n))
+    def side_launches(self): return int(self.L.dxe_side_launches(self.ex))
     def flush(self): self.L.dxe_flush(self.ex)
     def held(self): return int(self.L.dxe_held(self.ex))
 

@@ -463,11 +463,13 @@ def test_random_batches_fused_equal_line_by_line(tmp_path):
     dtype, mixed, with row or column vectors, with a row sum inside, cut at a vector that would be
     overwritten while other lanes still read it — every tensor must end up with the bits of the
     line-by-line execution, and every line must get the reply it gets on its own.  The same lines sent
-    one by one with runs held back (DEEPX_DEFER) must do the same."""
+    one by one with runs held back (DEEPX_DEFER) must do the same, and so must the batch with independent
+    lines spread over three side streams (DEEPX_STREAMS), fused and unfused: a random program is full of
+    read-after-write, write-after-read and write-after-write pairs for the stream choice to get wrong."""
     rng = np.random.default_rng(20251)
     dts = ["float32", "bfloat16", "float16"]
     code = {"float32": dx.F32, "bfloat16": dx.BF16, "float16": dx.F16}
-    fused_lines = held_lines = 0
+    fused_lines = held_lines = side_launches = 0
     for trial in range(72):
         rows, cols = [(16, 64), (5, 12), (64, 896), (3, 1000), (33, 260), (128, 32)][trial % 6]
         shapes = {"F": [rows, cols], "C": [rows, 1], "R": [1, cols]}
@@ -505,21 +507,24 @@ def test_random_batches_fused_equal_line_by_line(tmp_path):
                 lines.append(f"sum({T(pick('F', dt)[0], dt)}, {V([-1])}, var<bool>:true)->({T(pick('C', dt)[0], dt)})")
         text = [f"{line} // author=miaobyte id={900 + i}" for i, line in enumerate(lines)]
         results, replies = {}, {}
-        for mode in ("lines", "fused", "held"):
+        for mode in ("lines", "fused", "held", "streams", "streams_unfused"):
             ex = InProc()
-            ex.set_fusion(mode != "lines")
+            ex.set_fusion(mode not in ("lines", "streams_unfused"))
             ex.set_defer(mode == "held")
+            ex.set_streams(3 if mode.startswith("streams") else 1)
             h = Host(ex, tmp_path)
             for name, k, dt in pool:
                 h.put(name, data[name], dt)
-            replies[mode] = ex.execute_batch(text) if mode == "fused" else [ex.execute(t) for t in text]
+            replies[mode] = ex.execute_batch(text) if mode in ("fused", "streams", "streams_unfused") else [ex.execute(t) for t in text]
             if mode == "fused":
                 fused_lines += ex.fusion_stats()["lines"]
             if mode == "held":
                 held_lines += ex.defer_stats()["held_lines"]
+            if mode.startswith("streams"):
+                side_launches += ex.side_launches()
             results[mode] = {name: h.get(name) for name, _, _ in pool}
             del ex
-        for mode in ("fused", "held"):
+        for mode in ("fused", "held", "streams", "streams_unfused"):
             assert [r.split("//")[0] for r in replies[mode]] == [r.split("//")[0] for r in replies["lines"]], (trial, mode, lines)
             for name, _, _ in pool:
                 a, b = results["lines"][name], results[mode][name]
@@ -531,6 +536,7 @@ def test_random_batches_fused_equal_line_by_line(tmp_path):
                     same = np.array_equal(fa, fb, equal_nan=True)
                 assert same, (trial, mode, name, lines)
     assert fused_lines > 400 and held_lines > 400  # the batches did form runs, the single lines were held
+    assert side_launches > 100  # and independent lines did leave the default stream
 
 
 def test_square_view_row_sum_without_keepdims_fuses(tmp_path):
@@ -643,3 +649,56 @@ def test_softmax_lines_fuse_into_one_launch(tmp_path, dt, rows, cols):
             "float16": lambda a: H.f16_bits_to_f32(a).astype(np.float64)}[dt]
     y = load(want["y"]).reshape(rows, cols)
     assert np.allclose(y.sum(1), 1.0, atol=1e-5 if dt == "float32" else 3e-2)
+
+
+def test_side_streams_keep_every_hazard_in_order(tmp_path):
+    """DEEPX_STREAMS: independent lines of a batch run side by side on side streams.  On tensors large enough
+    for launches to overlap for tens of microseconds, a batch that mixes independent lines with
+    read-after-write, write-after-read and write-after-write pairs leaves the bits of in-order execution,
+    ten times in a row; the independent lines did leave the default stream."""
+    n = [4096, 4096]
+    rng = np.random.default_rng(411)
+    x, y = rng.uniform(0.5, 1.5, n).astype(np.float32), rng.uniform(0.5, 1.5, n).astype(np.float32)
+    names = ["z", "w", "x2", "s0", "s1", "m0", "m1", "v"]
+    lines = [
+        "add({x}, {y})->({z})",                                                  # independent
+        "mul({z}, {y})->({w})",                                                  # reads z: after line 1
+        "add({x}, {y})->({x2})",                                                 # independent of what is in flight
+        "sum({x}, vector<int32>:[1], var<bool>:false)->({s0})",                  # independent reductions of one tensor ...
+        "reducemax({x}, vector<int32>:[1], var<bool>:false)->({m0})",
+        "sum({x}, vector<int32>:[0], var<bool>:false)->({s1})",
+        "reducemin({x}, vector<int32>:[0], var<bool>:false)->({m1})",
+        "addscalar({x}, var<float32>:1)->({y})",                                 # ... then y is rewritten while lines 1-3 may still read it
+        "mul({x}, {x})->({z})",                                                  # z rewritten: after lines 1 and 2
+        "sub({z}, {y})->({v})",                                                  # reads both
+        "mulscalar({v}, var<float32>:0.5)->({x})",                               # x rewritten: after every reader above
+        "add({x}, {y})->({w})",
+    ]
+    results = {}
+    for streams in (1, 3):
+        ex = InProc()
+        ex.set_fusion(False)
+        ex.set_streams(streams)
+        h = Host(ex, tmp_path)
+        p = f"hz{streams}_"
+        for k in names:
+            shape = n if k in ("z", "w", "x2", "v") else [4096]
+            h.run(f"newtensor({V(shape)})->({T(p + k)})")
+        tn = {k: T(p + k) for k in names + ["x", "y"]}
+        text = [line.format(**tn) + f" // author=miaobyte id={i + 1}" for i, line in enumerate(lines)]
+        runs = []
+        for rep in range(10 if streams > 1 else 1):
+            h.put(p + "x", x)
+            h.put(p + "y", y)
+            rs = ex.execute_batch(text)
+            assert all(r.split(" ")[1].startswith("ok") for r in rs), rs
+            runs.append({k: h.get(p + k) for k in names + ["x", "y"]})
+        if streams > 1:
+            assert ex.side_launches() >= 10 * 5
+        else:
+            assert ex.side_launches() == 0
+        results[streams] = runs
+    want = results[1][0]
+    for rep, got in enumerate(results[3]):
+        for k in want:
+            assert np.array_equal(got[k].view(np.uint8), want[k].view(np.uint8)), (rep, k)

@@ -264,6 +264,37 @@ def main():
     dx.check(L.dxh_stream_destroy(gst))
     c2["step_as_recorded_hip_graph"] = {"ms_per_step": round(graph_ms_per_step, 4), "GB/s": round(step_bytes / graph_ms_per_step / 1e6, 1),
                                         "frac_hbm": round(step_bytes / graph_ms_per_step / 1e6 / HBM_PEAK_GBS, 4), "bytes": step_bytes}
+    # For information, not `value`: the ten ops dealt out over two streams (each with its own output and scratch):
+    # none of them reads what another writes, so the end of one launch runs under the start of the next.
+    two = []
+    for _ in range(2):
+        s2 = C.c_void_p()
+        dx.check(L.dxh_stream_create(C.byref(s2)))
+        two.append((s2, torch.empty(8192, device=dev, dtype=torch.float32), torch.empty(max(1, wsb.value), device=dev, dtype=torch.uint8)))
+    flat_ops = [o for _, ops in groups for o in ops]
+
+    def run_step_two_streams():
+        for i, (label, fn, sh, ax, bufs, nbytes) in enumerate(flat_ops):
+            s2, o2, w2 = two[i % 2]
+            buf = bufs[rot[0] % NX]
+            rot[0] += 1
+            rc = fn(dx.F32, ptr(buf), sh, 2, ax, 1, ptr(o2), ptr(w2), wsb.value, s2)
+            if rc != 0:
+                dx.check(rc, label)
+
+    for _ in range(20):
+        run_step_two_streams()
+    dx.check(L.dxh_device_sync())
+    t_t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run_step_two_streams()
+    dx.check(L.dxh_device_sync())
+    two_ms = (time.perf_counter() - t_t0) * 1e3 / args.steps
+    for s2, _, _ in two:
+        dx.check(L.dxh_stream_destroy(s2))
+    del two
+    c2["step_on_two_streams"] = {"ms_per_step": round(two_ms, 4), "GB/s": round(step_bytes / two_ms / 1e6, 1),
+                                 "frac_hbm": round(step_bytes / two_ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": step_bytes}
     dom_ms = group_ms["reduce_row_kernel"]
     achieved = XB / dom_ms / 1e6
     roofline = {"bound": "hbm", "kernel": "reduce_row_kernel<sum|max|min,f32> [8192,8192] axis 1 (6 of 10 launches per step)",

@@ -88,7 +88,7 @@ public:
         if (const char *ns = std::getenv("DEEPX_STREAMS")) streams = std::max(1, std::min(8, std::atoi(ns)));
     }
     ~Executor() {
-        flush();
+        try { flush(); } catch (const std::exception &e) { std::cerr << "held lines lost at shutdown: " << e.what() << std::endl; }
         for (auto &kv : graphs_) drop_graph(kv.second);
         if (graph_stream_) dxh_stream_destroy(graph_stream_);
         if (!side_.empty()) dxh_device_sync();

@@ -295,13 +295,13 @@ private:
             if (use_fusion && has_device) {
                 const size_t len = chain_length(tfs, i, mem);
                 if (len >= 2) {
-                    rc = run_chain(tfs, i, len, mem, message);
+                    try { rc = run_chain(tfs, i, len, mem, message); } catch (const std::exception &e) { rc = 1; message = e.what(); }
                     if (rc == 0) { ++stats.fused_runs; stats.fused_lines += len; return len; }
                     message.clear();
                 }
                 const size_t group = matmul_group_length(tfs, i, mem);
                 if (group >= 2) {
-                    rc = run_matmul_group(tfs, i, group, mem, message);
+                    try { rc = run_matmul_group(tfs, i, group, mem, message); } catch (const std::exception &e) { rc = 1; message = e.what(); }
                     if (rc == 0) { ++stats.matmul_groups; stats.matmul_lines += group; return group; }
                     message.clear();
                 }

@@ -197,6 +197,34 @@ def test_graphs_over_udp(tmp_path):
     assert srv.proc.returncode == 0
 
 
+def test_side_streams_over_udp(tmp_path):
+    """The server started with DEEPX_STREAMS=3 and DEEPX_FUSE=0: the eight lines of the chain as one datagram, whose
+    independent lines leave the default stream, give the values of in-order execution every time."""
+    srv = UdpExecutor(env={"DEEPX_STREAMS": "3", "DEEPX_FUSE": "0"})
+    try:
+        rng = np.random.default_rng(45)
+        a, b = rng.uniform(-1, 1, (512, 640)).astype(np.float32), rng.uniform(-1, 1, (512, 640)).astype(np.float32)
+        for name, arr in (("v_A", a), ("v_B", b)):
+            p = str(tmp_path / name)
+            write_tensor(p, arr, "float32")
+            srv.must("load", [f"var<string>:{p}"], [], author="")
+        for n in NAMES[2:]:
+            srv.must("newtensor", [V([512, 640])], [T("v_" + n)], author="")
+        datagram = "\n".join(chain_lines("v_", 7000))
+        f = np.exp((a + b) * b + np.float32(0.5))
+        want = f / (np.maximum(b, -b) + np.float32(1))
+        for _ in range(4):
+            srv.must("constant", ["var<float32>:0"], [T("v_G")])
+            rs = srv.raw(datagram, 8)
+            assert [r.id for r in rs] == [str(7000 + i) for i in range(8)] and all(r.ok for r in rs)
+            p = str(tmp_path / "v_G_out")
+            srv.must("save", [T("v_G", "any"), f"var<string>:{p}"], [], author="")
+            assert np.allclose(read_tensor(p)[0], want, rtol=1e-6, atol=0)
+    finally:
+        srv.close()
+    assert srv.proc.returncode == 0
+
+
 def test_fused_runs_equal_line_by_line(tmp_path):
     """Inside a batch, runs of float elementwise lines (an fp32 sum over the last axis among them) are
     launched as one kernel.  Bit for bit the tensors of a line-by-line execution, for: a run that is cut by a

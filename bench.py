@@ -66,6 +66,9 @@ def main():
                          "about 30 ms of load to reach its steady clocks")
     ap.add_argument("--no-per-op", action="store_true", help="skip the per-op table of the other configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--in-order-only", action="store_true",
+                    help="skip the information passes in which launches overlap on several streams (under a kernel trace they would "
+                         "mix overlapped launches into the per-kernel averages of the in-order step)")
     ap.add_argument("--matmul-only", metavar="MxKxN", default="",
                     help="run only the bf16 matmul of that shape, --steps launches after a clock ramp "
                          "(the program a counter collection wraps) and print its own JSON line")
@@ -267,7 +270,7 @@ def main():
     # For information, not `value`: the ten ops dealt out over two streams (each with its own output and scratch):
     # none of them reads what another writes, so the end of one launch runs under the start of the next.
     two = []
-    for _ in range(2):
+    for _ in range(0 if args.in_order_only else 2):
         s2 = C.c_void_p()
         dx.check(L.dxh_stream_create(C.byref(s2)))
         two.append((s2, torch.empty(8192, device=dev, dtype=torch.float32), torch.empty(max(1, wsb.value), device=dev, dtype=torch.uint8)))
@@ -282,19 +285,20 @@ def main():
             if rc != 0:
                 dx.check(rc, label)
 
-    for _ in range(20):
-        run_step_two_streams()
-    dx.check(L.dxh_device_sync())
-    t_t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run_step_two_streams()
-    dx.check(L.dxh_device_sync())
-    two_ms = (time.perf_counter() - t_t0) * 1e3 / args.steps
-    for s2, _, _ in two:
-        dx.check(L.dxh_stream_destroy(s2))
+    if two:
+        for _ in range(20):
+            run_step_two_streams()
+        dx.check(L.dxh_device_sync())
+        t_t0 = time.perf_counter()
+        for _ in range(args.steps):
+            run_step_two_streams()
+        dx.check(L.dxh_device_sync())
+        two_ms = (time.perf_counter() - t_t0) * 1e3 / args.steps
+        for s2, _, _ in two:
+            dx.check(L.dxh_stream_destroy(s2))
+        c2["step_on_two_streams"] = {"ms_per_step": round(two_ms, 4), "GB/s": round(step_bytes / two_ms / 1e6, 1),
+                                     "frac_hbm": round(step_bytes / two_ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": step_bytes}
     del two
-    c2["step_on_two_streams"] = {"ms_per_step": round(two_ms, 4), "GB/s": round(step_bytes / two_ms / 1e6, 1),
-                                 "frac_hbm": round(step_bytes / two_ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": step_bytes}
     dom_ms = group_ms["reduce_row_kernel"]
     achieved = XB / dom_ms / 1e6
     roofline = {"bound": "hbm", "kernel": "reduce_row_kernel<sum|max|min,f32> [8192,8192] axis 1 (6 of 10 launches per step)",
@@ -312,7 +316,7 @@ def main():
         del Xs, Ps
         torch.cuda.empty_cache()
         per_op.update(bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr))
-        per_op["config2"]["step_over_deepxIR"] = config2_step_over_ir(step_bytes)
+        per_op["config2"]["step_over_deepxIR"] = config2_step_over_ir(step_bytes, side_streams=not args.in_order_only)
 
     # ---------------- CPU baseline: the oracle's restatement of op-ompsimd's reduce ---------
     cpu = None
@@ -727,7 +731,7 @@ def lines_over_ir(setup, block, iters=30, only=None):
     return out
 
 
-def config2_step_over_ir(step_bytes, iters=30):
+def config2_step_over_ir(step_bytes, iters=30, side_streams=True):
     """The config-2 step (ten reductions) as one datagram of ten deepxIR lines through the executor's dispatch core:
     in order on the default stream, and with independent lines spread over side streams (the DEEPX_STREAMS switch:
     no line of the step reads what another writes, so the end of one launch runs under the start of the next).
@@ -757,6 +761,8 @@ def config2_step_over_ir(step_bytes, iters=30):
         texts.append("\n".join(f"{l} // author=miaobyte id={k + 1}" for k, l in enumerate(lines)).encode())
     out = {"ops": 10, "bytes": step_bytes}
     for label, streams in (("one_batch_us", 1), ("one_batch_side_streams_us", 3)):
+        if streams > 1 and not side_streams:
+            continue
         ex = E.dxe_create()
         buf = C.create_string_buffer(1 << 16)
         for line in setup:

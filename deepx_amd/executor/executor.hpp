@@ -173,6 +173,7 @@ public:
                 held_items_.back().call = std::move(call);
                 held_items_.back().tf = tf;
                 held_items_.back().resp = resp;
+                if (held_items_.size() >= 64) flush();  // a run that never ends (products on one operand, say) still goes out
                 return resp.to_string();
             }
         }

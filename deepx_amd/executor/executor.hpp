@@ -19,6 +19,7 @@
 #include <vector>
 #include "factory.hpp"
 #include "mem.hpp"
+#include "stream_picker.hpp"
 
 namespace deepx {
 
@@ -364,13 +365,12 @@ private:
         return replies;
     }
 
-    // Which stream the launch that starts at line i goes to (see `streams`).  Each side stream remembers the tensors
-    // that its launches since the last join read and wrote.  A kernel-only launch that clashes with none of them goes to
-    // the next side stream in turn; one that clashes with a single stream goes to that stream, behind what it depends
-    // on; one that clashes with several goes to the first of them after that stream has been told to wait for events
-    // recorded on the others.  Anything that is not kernel-only goes to the default stream, which waits for all of
-    // them and makes them wait for it (they are ordinary blocking streams) — correct, and slow on this runtime (a
-    // launch on the default stream between launches on other streams costs about 60 us), which is why clashes do not.
+    // Which stream the launch that starts at line i goes to (see `streams`).  The decision is StreamPicker's
+    // (stream_picker.hpp): the next side stream in turn for a kernel-only launch that clashes with nothing in flight,
+    // the stream it clashes with otherwise — after that stream has been told to wait for events recorded on the other
+    // streams it clashes with — and the default stream for anything that is not kernel-only.  The default stream waits
+    // for all side streams and makes them wait for it (they are ordinary blocking streams): correct, and slow on this
+    // runtime (a launch there between launches on other streams costs about 60 us), which is why clashes do not go there.
     void pick_stream(const std::vector<Item> &items, const std::vector<std::shared_ptr<TF>> &tfs, size_t i) {
         mem.stream = nullptr;
         mem.scratch_of = nullptr;
@@ -385,38 +385,24 @@ private:
             names_in(items[j].call.args, reads);
             names_in(items[j].call.returns, writes);
         }
-        size_t remembered = 0;
-        for (const Side &sd : side_) remembered += sd.reads.size() + sd.writes.size();
-        // a replayed graph runs on a stream of its own, and a long-lived server must not remember names for ever: join
-        if (!kernel_only || graph_flying_ || remembered > 4096) {
-            graph_flying_ = false;
-            for (Side &sd : side_) { sd.reads.clear(); sd.writes.clear(); }
-            return;  // the default stream
-        }
         while (side_.size() < (size_t)streams) {
             Side sd;
-            if (dxh_stream_create(&sd.stream) != DXH_OK || !sd.stream) { streams = 1; return; }
-            if (dxh_event_create(&sd.event) != DXH_OK || !sd.event) { dxh_stream_destroy(sd.stream); streams = 1; return; }
-            side_.push_back(std::move(sd));
+            if (dxh_stream_create(&sd.stream) != DXH_OK || !sd.stream) { streams = 1; picker_.resize(0); return; }
+            if (dxh_event_create(&sd.event) != DXH_OK || !sd.event) { dxh_stream_destroy(sd.stream); streams = 1; picker_.resize(0); return; }
+            side_.push_back(sd);
         }
-        std::vector<size_t> hit;
-        for (size_t k = 0; k < side_.size(); ++k) {
-            const Side &sd = side_[k];
-            bool clash = false;
-            for (const std::string &w : writes) clash = clash || sd.writes.count(w) || sd.reads.count(w);
-            for (const std::string &r : reads) clash = clash || sd.writes.count(r);
-            if (clash) hit.push_back(k);
-        }
-        const size_t target = hit.empty() ? next_side_++ % side_.size() : hit[0];
-        for (size_t j = 1; j < hit.size(); ++j) {
-            if (dxh_event_record(side_[hit[j]].event, side_[hit[j]].stream) != DXH_OK || dxh_stream_wait_event(side_[target].stream, side_[hit[j]].event) != DXH_OK) {
-                for (Side &sd : side_) { sd.reads.clear(); sd.writes.clear(); }
+        if (picker_.streams() != (int)side_.size()) picker_.resize((int)side_.size());
+        const StreamPicker::Choice c = picker_.place(reads, writes, kernel_only, graph_flying_);
+        graph_flying_ = false;
+        if (c.stream < 0) return;  // the default stream
+        for (int other : c.wait_for) {
+            if (dxh_event_record(side_[(size_t)other].event, side_[(size_t)other].stream) != DXH_OK ||
+                dxh_stream_wait_event(side_[(size_t)c.stream].stream, side_[(size_t)other].event) != DXH_OK) {
+                picker_.abandon();
                 return;  // could not order them: the default stream does
             }
         }
-        mem.stream = mem.scratch_of = side_[target].stream;
-        side_[target].reads.insert(reads.begin(), reads.end());
-        side_[target].writes.insert(writes.begin(), writes.end());
+        mem.stream = mem.scratch_of = side_[(size_t)c.stream].stream;
         ++stats.side_launches;
     }
     void names_in(const std::vector<Param> &ps, std::vector<std::string> &names) const {
@@ -562,9 +548,9 @@ private:
 
     std::recursive_mutex mu_;  // flush() is called from inside execute() and execute_batch()
     std::vector<Item> held_items_;
-    struct Side { void *stream = nullptr, *event = nullptr; std::unordered_set<std::string> reads, writes; };  // tensors of its launches since the last join
+    struct Side { void *stream = nullptr, *event = nullptr; };
     std::vector<Side> side_;  // side streams, created on first use
-    size_t next_side_ = 0;
+    StreamPicker picker_;
     bool graph_flying_ = false;
     std::vector<std::shared_ptr<TF>> held_tfs_;
     void *graph_stream_ = nullptr;

@@ -145,8 +145,9 @@ DXH_API int dxh_event_create(void **event);
 DXH_API int dxh_event_destroy(void *event);
 DXH_API int dxh_event_record(void *event, void *stream);
 DXH_API int dxh_event_sync(void *event);
-/* work launched on `stream` after this call waits for what `event` recorded (hipStreamWaitEvent): how a caller that spreads
- * independent ops over several streams orders the dependent ones, without going through the default stream */
+/* No counterpart in the reference, which launches everything on the default stream (executor/op-cuda/src/deepx/tensorfunc/cuda.hpp:45-67):
+ * work launched on `stream` after this call waits for what `event` recorded (hipStreamWaitEvent).  How a caller that spreads
+ * independent ops over several streams orders the dependent ones without going through the default stream. */
 DXH_API int dxh_stream_wait_event(void *stream, void *event);
 DXH_API int dxh_event_elapsed_ms(void *start, void *stop, float *ms);
 

@@ -145,7 +145,7 @@ DXH_API int dxh_event_create(void **event);
 DXH_API int dxh_event_destroy(void *event);
 DXH_API int dxh_event_record(void *event, void *stream);
 DXH_API int dxh_event_sync(void *event);
-/* No counterpart in the reference, which launches everything on the default stream (executor/op-cuda/src/deepx/tensorfunc/cuda.hpp:45-67):
+/* No counterpart in the reference, whose launches name no stream (executor/op-cuda/src/deepx/tensorfunc/elementwise_miaobyte_basic.cu:113: `add_kernel<<<numBlocks, blockSize>>>`):
  * work launched on `stream` after this call waits for what `event` recorded (hipStreamWaitEvent).  How a caller that spreads
  * independent ops over several streams orders the dependent ones without going through the default stream. */
 DXH_API int dxh_stream_wait_event(void *stream, void *event);

@@ -54,7 +54,7 @@ public:
     // as line-by-line execution leaves them; the reply of a held line carries the time it was accepted.
     // Off with DEEPX_SYNC=1 (a reply then promises finished kernels) and with DEEPX_FUSE=0.
     bool defer = false;
-    // DEEPX_STREAMS=n (n >= 2): inside a batch, kernel-only lines are spread over n side streams so that launches which
+    // DEEPX_STREAMS=n (n >= 2): kernel-only lines (of a batch, or sent one by one) are spread over n side streams so that launches which
     // do not depend on each other overlap (the end of one runs under the start of the next; ten reductions over one
     // [8192,8192] tensor: 341 -> 313 us); a line that reads or writes what a launch in flight wrote, or writes what one
     // reads, goes behind that launch on its stream (see pick_stream).  The tensors end up as in-order execution leaves
@@ -183,10 +183,18 @@ public:
         int rc = 0;
         std::string message;
         const int repeat = tf->metadata.benchmark_repeat > 1 ? tf->metadata.benchmark_repeat : 1;
+        if (streams >= 2 && has_device) {  // a line on its own may leave the default stream like a line of a batch
+            std::vector<Item> one(1);
+            one[0].call = call;
+            one[0].tf = tf;
+            pick_stream(one, {tf}, 0);
+        }
         for (int i = 0; i < repeat && rc == 0; ++i) rc = tf->run(mem, message);
+        mem.stream = nullptr;
+        mem.scratch_of = nullptr;
         lap(prof.run_ns);
         if (rc == 0 && sync_each && has_device) {
-            int s = dxh_stream_sync(nullptr);
+            int s = side_.empty() ? dxh_stream_sync(nullptr) : dxh_device_sync();
             if (s != DXH_OK) { rc = 1; message = std::string("hip: ") + dxh_error_string(s); }
         }
         lap(prof.sync_ns);

@@ -535,9 +535,9 @@ def test_random_batches_fused_equal_line_by_line(tmp_path):
                 lines.append(f"sum({T(pick('F', dt)[0], dt)}, {V([-1])}, var<bool>:true)->({T(pick('C', dt)[0], dt)})")
         text = [f"{line} // author=miaobyte id={900 + i}" for i, line in enumerate(lines)]
         results, replies = {}, {}
-        for mode in ("lines", "fused", "held", "streams", "streams_unfused"):
+        for mode in ("lines", "fused", "held", "streams", "streams_unfused", "streams_lines"):
             ex = InProc()
-            ex.set_fusion(mode not in ("lines", "streams_unfused"))
+            ex.set_fusion(mode not in ("lines", "streams_unfused", "streams_lines"))
             ex.set_defer(mode == "held")
             ex.set_streams(3 if mode.startswith("streams") else 1)
             h = Host(ex, tmp_path)
@@ -552,7 +552,7 @@ def test_random_batches_fused_equal_line_by_line(tmp_path):
                 side_launches += ex.side_launches()
             results[mode] = {name: h.get(name) for name, _, _ in pool}
             del ex
-        for mode in ("fused", "held", "streams", "streams_unfused"):
+        for mode in ("fused", "held", "streams", "streams_unfused", "streams_lines"):
             assert [r.split("//")[0] for r in replies[mode]] == [r.split("//")[0] for r in replies["lines"]], (trial, mode, lines)
             for name, _, _ in pool:
                 a, b = results["lines"][name], results[mode][name]
@@ -703,12 +703,12 @@ def test_side_streams_keep_every_hazard_in_order(tmp_path):
         "add({x}, {y})->({w})",
     ]
     results = {}
-    for streams in (1, 3):
+    for streams, batched in ((1, True), (3, True), (3, False)):
         ex = InProc()
         ex.set_fusion(False)
         ex.set_streams(streams)
         h = Host(ex, tmp_path)
-        p = f"hz{streams}_"
+        p = f"hz{streams}{int(batched)}_"
         for k in names:
             shape = n if k in ("z", "w", "x2", "v") else [4096]
             h.run(f"newtensor({V(shape)})->({T(p + k)})")
@@ -718,15 +718,16 @@ def test_side_streams_keep_every_hazard_in_order(tmp_path):
         for rep in range(10 if streams > 1 else 1):
             h.put(p + "x", x)
             h.put(p + "y", y)
-            rs = ex.execute_batch(text)
+            rs = ex.execute_batch(text) if batched else [ex.execute(t) for t in text]
             assert all(r.split(" ")[1].startswith("ok") for r in rs), rs
             runs.append({k: h.get(p + k) for k in names + ["x", "y"]})
         if streams > 1:
             assert ex.side_launches() >= 10 * 5
         else:
             assert ex.side_launches() == 0
-        results[streams] = runs
-    want = results[1][0]
-    for rep, got in enumerate(results[3]):
-        for k in want:
-            assert np.array_equal(got[k].view(np.uint8), want[k].view(np.uint8)), (rep, k)
+        results[(streams, batched)] = runs
+    want = results[(1, True)][0]
+    for key in ((3, True), (3, False)):  # as one datagram, and sent line by line
+        for rep, got in enumerate(results[key]):
+            for k in want:
+                assert np.array_equal(got[k].view(np.uint8), want[k].view(np.uint8)), (key, rep, k)

@@ -732,8 +732,8 @@ def lines_over_ir(setup, block, iters=30, only=None):
 
 
 def config2_step_over_ir(step_bytes, iters=30, side_streams=True):
-    """The config-2 step (ten reductions) as one datagram of ten deepxIR lines through the executor's dispatch core:
-    in order on the default stream, and with independent lines spread over side streams (the DEEPX_STREAMS switch:
+    """The config-2 step (ten reductions) as one datagram of ten deepxIR lines through the executor's dispatch core, and
+    sent line by line: in order on the default stream, and with independent lines spread over side streams (the DEEPX_STREAMS switch:
     no line of the step reads what another writes, so the end of one launch runs under the start of the next).
     Three copies of the input in rotation, as in the headline step."""
     import ctypes as C
@@ -760,9 +760,11 @@ def config2_step_over_ir(step_bytes, iters=30, side_streams=True):
                       f"prod({T('P%d' % i)}, {V([1])}, {kb})->({T(f'pr_kd{kd}')})"]
         texts.append("\n".join(f"{l} // author=miaobyte id={k + 1}" for k, l in enumerate(lines)).encode())
     out = {"ops": 10, "bytes": step_bytes}
-    for label, streams in (("one_batch_us", 1), ("one_batch_side_streams_us", 3)):
+    line_sets = [[l for l in t.decode().split("\n")] for t in texts]
+    for label, streams in (("one_batch_us", 1), ("one_batch_side_streams_us", 3), ("line_by_line_us", 1), ("line_by_line_side_streams_us", 3)):
         if streams > 1 and not side_streams:
             continue
+        batched = label.startswith("one_batch")
         ex = E.dxe_create()
         buf = C.create_string_buffer(1 << 16)
         for line in setup:
@@ -770,12 +772,19 @@ def config2_step_over_ir(step_bytes, iters=30, side_streams=True):
             if " ok" not in buf.value.decode().split("//")[0]:
                 raise RuntimeError(f"{line}: {buf.value.decode()}")
         E.dxe_set_streams(ex, streams)
+        def once(r):
+            if batched:
+                E.dxe_execute_batch(ex, texts[r % 3], buf, len(buf))
+            else:
+                for l in line_sets[r % 3]:
+                    E.dxe_execute(ex, l.encode(), buf, len(buf))
+
         for r in range(6):
-            E.dxe_execute_batch(ex, texts[r % 3], buf, len(buf))
+            once(r)
         dx.check(L.dxh_device_sync())
         t0 = time.perf_counter()
         for r in range(iters):
-            E.dxe_execute_batch(ex, texts[r % 3], buf, len(buf))
+            once(r)
         dx.check(L.dxh_device_sync())
         us = (time.perf_counter() - t0) / iters * 1e6
         if any(" ok" not in r.split("//")[0] for r in buf.value.decode().split("\n")):

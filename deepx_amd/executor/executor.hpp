@@ -178,7 +178,11 @@ public:
                 return resp.to_string();
             }
         }
-        flush();  // whatever is held comes first (also when a switch was turned while lines were held)
+        // An allocation touches nothing that a held line names (held lines were checked against the tensors that existed
+        // when they were accepted), so it need not end their run: the front allocates every result right before the
+        // line that computes it (front/py/deepx/nn/functional/reduce.py:21-23), and a run would never grow otherwise.
+        if (!(tf->name == "newtensor" && !held_items_.empty()))
+            flush();  // whatever is held comes first (also when a switch was turned while lines were held)
         resp.start_at = std::chrono::system_clock::now();
         int rc = 0;
         std::string message;
@@ -288,7 +292,30 @@ public:
             it.tf->returns = it.call.returns;
             graphable = graphable && it.tf->graph_safe && it.tf->metadata.benchmark_repeat <= 1 && !uses_named_arg(it.call);
         }
-        return run_items(items, key, graphable, recv_at);
+        // Allocations first: a `newtensor` line whose tensor no earlier line of the batch names moves to the front (in
+        // order among themselves), so that the compute lines it sat between can share a launch.  Replies keep the
+        // order of the lines.
+        std::vector<size_t> order;
+        {
+            std::vector<size_t> rest;
+            for (size_t i = 0; i < items.size(); ++i) {
+                bool hoist = !items[i].failed && items[i].tf && items[i].call.name == "newtensor" && items[i].call.returns.size() == 1;
+                if (hoist) {
+                    const std::string &name = items[i].call.returns[0].textvalue;
+                    for (size_t j = 0; j < i && hoist; ++j) hoist = items[j].failed ? lines[j].find(name) == std::string::npos : !mentions(items[j].call, name);
+                }
+                (hoist ? order : rest).push_back(i);
+            }
+            if (order.empty() || order.size() == items.size()) order.clear();
+            else order.insert(order.end(), rest.begin(), rest.end());
+        }
+        if (order.empty()) return run_items(items, key, graphable, recv_at);
+        std::vector<Item> moved(items.size());
+        for (size_t k = 0; k < order.size(); ++k) moved[k] = std::move(items[order[k]]);
+        const std::vector<std::string> out = run_items(moved, key, false, recv_at);
+        std::vector<std::string> replies(out.size());
+        for (size_t k = 0; k < order.size(); ++k) replies[order[k]] = out[k];
+        return replies;
     }
 
 private:
@@ -412,6 +439,18 @@ private:
         }
         mem.stream = mem.scratch_of = side_[(size_t)c.stream].stream;
         ++stats.side_launches;
+    }
+    // does a call name `word` among its arguments or results (bare, typed, or inside a [a b c] list)
+    static bool mentions(const TF &call, const std::string &word) {
+        for (const std::vector<Param> *ps : {&call.args, &call.returns})
+            for (const Param &p : *ps) {
+                std::string t = p.textvalue;
+                for (char &c : t) if (c == '[' || c == ']') c = ' ';
+                std::istringstream in(t);
+                std::string w;
+                while (in >> w) if (w == word) return true;
+            }
+        return false;
     }
     void names_in(const std::vector<Param> &ps, std::vector<std::string> &names) const {
         for (const Param &p : ps) {

@@ -160,3 +160,56 @@ def test_server_launches_held_lines_when_the_sender_pauses(tmp_path):
         assert np.allclose(got, want, rtol=1e-6, atol=1e-6)
     finally:
         ex.close()
+
+
+@pytest.mark.parametrize("mode", ["held", "batch"])
+def test_allocations_do_not_end_a_run(tmp_path, mode):
+    """The front allocates every result right before the line that computes it (newtensor, then the op).  Held line by
+    line, or as one datagram, the compute lines between the allocations still go out as one launch, and every tensor
+    has the bits of in-order execution."""
+    S, Hd = 96, 256
+    rng = np.random.default_rng(193)
+    x = H.f32_to_bf16_bits(rng.standard_normal((S, Hd)).astype(np.float32))
+    f32, b16 = "float32", "bfloat16"
+    steps = [  # (allocation of the result, compute line)
+        (("xf", [S, Hd], f32), "todtype({x})->({xf})"),
+        (("sq", [S, Hd], f32), "powscalar({xf}, var<float32>:2)->({sq})"),
+        (("var", [S, 1], f32), "sum({sq}, vector<int32>:[-1], var<bool>:true)->({var})"),
+        (None, f"divscalar({{var}}, var<float32>:{Hd})->({{var}})"),
+        (("ve", [S, 1], f32), "addscalar({var}, var<float32>:1e-06)->({ve})"),
+        (("sd", [S, 1], f32), "sqrt({ve})->({sd})"),
+        (("rs1", [S, 1], f32), "rdivscalar(var<float32>:1, {sd})->({rs1})"),
+        (("rs", [S, Hd], f32), f"broadcastTo({{rs1}}, {V([S, Hd])})->({{rs}})"),
+        (("xn", [S, Hd], f32), "mul({xf}, {rs})->({xn})"),
+        (("h", [S, Hd], b16), "todtype({xn})->({h})"),
+    ]
+    names = ["xf", "sq", "var", "ve", "sd", "rs1", "rs", "xn", "h"]
+    results = {}
+    for m in ("plain", mode):
+        ex = InProc()
+        ex.set_defer(m == "held")
+        h = Host(ex, tmp_path)
+        p = f"al_{m}_"
+        h.put(p + "x", x, b16)
+        tn = {k: T(p + k, b16 if k in ("x", "h") else f32) for k in names + ["x"]}
+        text = []
+        for alloc, line in steps:
+            if alloc:
+                text.append(f"newtensor({V(alloc[1])})->({T(p + alloc[0], alloc[2])})")
+            text.append(line.format(**tn))
+        text = [f"{t} // author=miaobyte id={300 + i}" for i, t in enumerate(text)]
+        if m == "batch":
+            rs = ex.execute_batch(text)
+        else:
+            rs = [ex.execute(t) for t in text]
+        assert [r.split(" ")[0] for r in rs] == [str(300 + i) for i in range(len(text))], rs  # replies in the order of the lines
+        assert all(r.split(" ")[1].startswith("ok") for r in rs), rs
+        ex.flush()
+        fs = ex.fusion_stats()
+        if m == "plain":
+            assert fs["runs"] == 0
+        else:
+            assert fs["runs"] == 1 and fs["lines"] == len(steps), fs
+        results[m] = {k: h.get(p + k) for k in names}
+    for k in names:
+        assert np.array_equal(results[mode][k].view(np.uint8), results["plain"][k].view(np.uint8)), k

@@ -2,7 +2,9 @@
 // Replaces the cudaMalloc/cudaFree/cudaMemcpy calls of
 // executor/op-cuda/src/deepx/tensorfunc/tensorlife_miaobyte.hpp:16-68.
 #include "matmul_common.hpp"
+#include "block_pool.hpp"
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 using namespace dxh;
@@ -13,6 +15,39 @@ Tuning &tuning() {
     return t;
 }
 }  // namespace dxh
+
+namespace {
+
+int raw_alloc(void **p, size_t bytes) { return (int)hipMalloc(p, bytes); }
+int raw_free(void *p) { return (int)hipFree(p); }
+
+// One pool per device, made on first use and never destroyed: at process exit the runtime may be gone before a
+// static destructor could hand the blocks back, and the driver reclaims them anyway.
+// Kept bytes are capped at DXH_POOL_MAX_MB if set, else at half the device's memory.
+BlockPool *pool_of_current_device(bool create) {
+    static std::mutex mu;
+    static std::map<int, BlockPool *> pools;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = pools.find(dev);
+    if (it != pools.end()) return it->second;
+    if (!create) return nullptr;
+    size_t cap = 0;
+    const char *e = std::getenv("DXH_POOL_MAX_MB");
+    if (e && *e) {
+        cap = (size_t)std::strtoull(e, nullptr, 10) << 20;
+    } else {
+        size_t free_b = 0, total_b = 0;
+        if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) { (void)hipGetLastError(); total_b = (size_t)16 << 30; }
+        cap = total_b / 2;
+    }
+    BlockPool *p = new BlockPool(raw_alloc, raw_free, cap);
+    pools[dev] = p;
+    return p;
+}
+
+}  // namespace
 
 extern "C" {
 
@@ -84,9 +119,52 @@ int dxh_malloc(void **ptr, size_t bytes) {
     if (!ptr) return DXH_ERR_ARG;
     *ptr = nullptr;
     if (bytes == 0) bytes = 1;  // a zero-element tensor still owns a distinct pointer
-    return (int)hipMalloc(ptr, bytes);
+    hipError_t e = hipMalloc(ptr, bytes);
+    if (e == hipErrorOutOfMemory) {  // blocks kept for reuse may be what is in the way
+        (void)hipGetLastError();
+        BlockPool *pool = pool_of_current_device(false);
+        if (pool && pool->trim(0) > 0) e = hipMalloc(ptr, bytes);
+    }
+    return (int)e;
 }
 int dxh_free(void *ptr) { return ptr ? (int)hipFree(ptr) : DXH_OK; }
+
+int dxh_pool_alloc(void **ptr, size_t bytes) {
+    if (!ptr) return DXH_ERR_ARG;
+    *ptr = nullptr;
+    BlockPool *pool = pool_of_current_device(true);
+    if (!pool) return DXH_ERR_ARG;
+    const int rc = pool->alloc(ptr, bytes);
+    if (rc > 0) (void)hipGetLastError();
+    return rc < 0 ? DXH_ERR_ARG : rc;
+}
+int dxh_pool_free(void *ptr) {
+    if (!ptr) return DXH_OK;
+    BlockPool *pool = pool_of_current_device(false);
+    if (!pool) return DXH_ERR_ARG;
+    const int rc = pool->free(ptr);
+    return rc < 0 ? DXH_ERR_ARG : rc;
+}
+int dxh_pool_trim(size_t keep_bytes, size_t *released) {
+    BlockPool *pool = pool_of_current_device(false);
+    const size_t gone = pool ? pool->trim(keep_bytes) : 0;
+    if (released) *released = gone;
+    return DXH_OK;
+}
+int dxh_pool_limit(size_t max_kept_bytes) {
+    BlockPool *pool = pool_of_current_device(true);
+    if (!pool) return DXH_ERR_ARG;
+    pool->set_max_kept(max_kept_bytes);
+    return DXH_OK;
+}
+int dxh_pool_stats(dxh_pool_stats_t *out) {
+    if (!out) return DXH_ERR_ARG;
+    BlockPool *pool = pool_of_current_device(false);
+    const BlockPool::Stats s = pool ? pool->stats() : BlockPool::Stats();
+    out->hits = s.hits; out->misses = s.misses; out->kept = s.kept; out->released = s.released;
+    out->kept_bytes = s.kept_bytes; out->kept_blocks = s.kept_blocks; out->live_bytes = s.live_bytes; out->live_blocks = s.live_blocks;
+    return DXH_OK;
+}
 
 int dxh_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream) {
     if (bytes == 0) return DXH_OK;

@@ -57,6 +57,9 @@ DXE_API size_t dxe_defer_stats(void *ex, char *out, size_t buflen) {
 // dxe_side_launches: how many launches went to a side stream so far
 DXE_API void dxe_set_streams(void *ex, int n) { static_cast<Executor *>(ex)->streams = n < 1 ? 1 : n > 8 ? 8 : n; }
 DXE_API size_t dxe_side_launches(void *ex) { return (size_t)static_cast<Executor *>(ex)->stats.side_launches; }
+// tensors allocated from now on take their storage from the library's pool of freed blocks (1, the default; the DEEPX_POOL
+// switch) or from the driver each time (0); tensors that exist keep what they have and return it where it came from
+DXE_API void dxe_set_pool(int on) { deepx::tensor_pool_enabled() = on != 0; }
 DXE_API size_t dxe_fusion_stats(void *ex, char *out, size_t buflen) {
     const auto &s = static_cast<Executor *>(ex)->stats;
     return copy_out(std::to_string(s.fused_runs) + " " + std::to_string(s.fused_lines) + " " + std::to_string(s.matmul_groups) + " " + std::to_string(s.matmul_lines), out, buflen);

@@ -91,6 +91,7 @@ public:
     ~Executor() {
         try { flush(); } catch (const std::exception &e) { std::cerr << "held lines lost at shutdown: " << e.what() << std::endl; }
         for (auto &kv : graphs_) drop_graph(kv.second);
+        if (graph_event_) dxh_event_destroy(graph_event_);
         if (graph_stream_) dxh_stream_destroy(graph_stream_);
         if (!side_.empty()) dxh_device_sync();
         for (Side &sd : side_) { dxh_event_destroy(sd.event); dxh_stream_destroy(sd.stream); }
@@ -178,10 +179,14 @@ public:
                 return resp.to_string();
             }
         }
-        // An allocation touches nothing that a held line names (held lines were checked against the tensors that existed
-        // when they were accepted), so it need not end their run: the front allocates every result right before the
-        // line that computes it (front/py/deepx/nn/functional/reduce.py:21-23), and a run would never grow otherwise.
-        if (!(tf->name == "newtensor" && !held_items_.empty()))
+        // An allocation under a name that no held line mentions touches nothing they use (held lines were checked against
+        // the tensors that existed when they were accepted), so it need not end their run: the front allocates every
+        // result right before the line that computes it (front/py/deepx/nn/functional/reduce.py:19-20,
+        // leaffunc.py:30-38), and a run would never grow otherwise.  Under a name they do mention it replaces a tensor
+        // they are about to use, and comes after them like any other line.
+        bool beside_held = tf->name == "newtensor" && !held_items_.empty() && call.returns.size() == 1;
+        for (size_t h = 0; h < held_items_.size() && beside_held; ++h) beside_held = !mentions(held_items_[h].call, call.returns[0].textvalue);
+        if (!beside_held)
             flush();  // whatever is held comes first (also when a switch was turned while lines were held)
         resp.start_at = std::chrono::system_clock::now();
         int rc = 0;
@@ -403,9 +408,10 @@ private:
     // Which stream the launch that starts at line i goes to (see `streams`).  The decision is StreamPicker's
     // (stream_picker.hpp): the next side stream in turn for a kernel-only launch that clashes with nothing in flight,
     // the stream it clashes with otherwise — after that stream has been told to wait for events recorded on the other
-    // streams it clashes with — and the default stream for anything that is not kernel-only.  The default stream waits
-    // for all side streams and makes them wait for it (they are ordinary blocking streams): correct, and slow on this
-    // runtime (a launch there between launches on other streams costs about 60 us), which is why clashes do not go there.
+    // streams it clashes with — and the default stream for anything that is not kernel-only, behind a join of the side
+    // streams (join_side_streams).  A launch on the default stream waits for all side streams and makes them wait for it
+    // (they are ordinary blocking streams): correct, and slow on this runtime (a launch there between launches on other
+    // streams costs about 60 us), which is why clashes do not go there.
     void pick_stream(const std::vector<Item> &items, const std::vector<std::shared_ptr<TF>> &tfs, size_t i) {
         mem.stream = nullptr;
         mem.scratch_of = nullptr;
@@ -427,9 +433,14 @@ private:
             side_.push_back(sd);
         }
         if (picker_.streams() != (int)side_.size()) picker_.resize((int)side_.size());
-        const StreamPicker::Choice c = picker_.place(reads, writes, kernel_only, graph_flying_);
+        const std::vector<int> busy = picker_.busy();
+        const bool flying = graph_flying_;
+        const StreamPicker::Choice c = picker_.place(reads, writes, kernel_only, flying);
         graph_flying_ = false;
-        if (c.stream < 0) return;  // the default stream
+        if (c.stream < 0) {  // the default stream
+            join_side_streams(busy, flying);
+            return;
+        }
         for (int other : c.wait_for) {
             if (dxh_event_record(side_[(size_t)other].event, side_[(size_t)other].stream) != DXH_OK ||
                 dxh_stream_wait_event(side_[(size_t)c.stream].stream, side_[(size_t)other].event) != DXH_OK) {
@@ -439,6 +450,27 @@ private:
         }
         mem.stream = mem.scratch_of = side_[(size_t)c.stream].stream;
         ++stats.side_launches;
+    }
+    // Orders everything the `busy` side streams have been given so far before whatever any stream is given from now on.
+    // A launch on the default stream would do that by itself (it waits for every blocking stream, and they for it), but a
+    // line sent there need not launch anything: `deltensor`, `renametensor` and `argset` are host work, an empty tensor
+    // has no kernel, a line can fail before its launch — and the picker has forgotten what was in flight either way.  So
+    // the join is made of events: each busy stream records one, and the default stream and every other side stream wait for it.
+    // A replayed graph that may still be running on its own stream (`graph_too`) is waited for the same way.
+    void join_side_streams(const std::vector<int> &busy, bool graph_too) {
+        bool ok = true;
+        if (graph_too && graph_stream_) {
+            if (!graph_event_ && dxh_event_create(&graph_event_) != DXH_OK) graph_event_ = nullptr;
+            ok = graph_event_ && dxh_event_record(graph_event_, graph_stream_) == DXH_OK && dxh_stream_wait_event(nullptr, graph_event_) == DXH_OK;
+            for (size_t b = 0; b < side_.size() && ok; ++b) ok = dxh_stream_wait_event(side_[b].stream, graph_event_) == DXH_OK;
+        }
+        for (int a : busy) {
+            ok = ok && dxh_event_record(side_[(size_t)a].event, side_[(size_t)a].stream) == DXH_OK &&
+                 dxh_stream_wait_event(nullptr, side_[(size_t)a].event) == DXH_OK;
+            for (size_t b = 0; b < side_.size() && ok; ++b)
+                if ((int)b != a) ok = dxh_stream_wait_event(side_[b].stream, side_[(size_t)a].event) == DXH_OK;
+        }
+        if (!ok) dxh_device_sync();  // the one join that needs no event
     }
     // does a call name `word` among its arguments or results (bare, typed, or inside a [a b c] list)
     static bool mentions(const TF &call, const std::string &word) {
@@ -600,7 +632,7 @@ private:
     StreamPicker picker_;
     bool graph_flying_ = false;
     std::vector<std::shared_ptr<TF>> held_tfs_;
-    void *graph_stream_ = nullptr;
+    void *graph_stream_ = nullptr, *graph_event_ = nullptr;
     std::unordered_map<std::string, Graph> graphs_;
     static constexpr size_t kMaxRemembered = 1024;
     std::unordered_set<std::string> seen_, rejected_;

@@ -8,6 +8,8 @@
 //   DEEPX_SYNC     1: wait for the device before every reply (default: reply at launch, as op-cuda does)
 //   DEEPX_STREAMS  n >= 2: independent kernel-only lines of a datagram go to n side streams in turn and overlap
 //   DEEPX_DEFER    1: hold lines that can share a launch with the next one (DEEPX_DEFER_US: longest wait for it, default 200)
+//   DEEPX_POOL     0: every tensor's storage comes from and goes back to the driver, as in the reference (default: freed
+//                  blocks are kept, up to DXH_POOL_MAX_MB or half the device's memory, and handed out again)
 //   DEEPX_OPLIST   path: write the generated op table (markdown) there, as the reference writes
 //                  docs/executor/op-mem-*/list.md at start-up
 #include <csignal>

@@ -2,10 +2,13 @@
 //
 // One Mem per process owns every tensor by name (executor/deepxcore/src/deepx/mem/mem.hpp:15-175;
 // the CUDA twin executor/op-cuda/src/deepx/mem/mem_cuda.hpp).  Tensor storage is device memory
-// obtained through the C ABI (dxh_malloc / dxh_free), the counterpart of the alloc/free/copy
+// obtained through the C ABI (dxh_pool_alloc / dxh_pool_free: freed blocks are handed out again; dxh_malloc / dxh_free
+// with DEEPX_POOL=0), the counterpart of the alloc/free/copy
 // function pointers the reference installs in Tensor<T> (executor/deepxcore/src/deepx/tensor.hpp:17-37,
 // executor/op-cuda/src/deepx/tensorfunc/tensorlife_miaobyte.hpp:70-85).
 #pragma once
+#include <cstdlib>
+#include <cstring>
 #include <map>
 #include <memory>
 #include <stdexcept>
@@ -24,19 +27,34 @@ struct DxhError : std::runtime_error {
 };
 inline void dxh_check(int code, const char *what) { if (code != DXH_OK) throw DxhError(code, what); }
 
+// Whether new tensors take their storage from the library's pool of freed blocks (default) or from the driver each time,
+// as the reference does (DEEPX_POOL=0).  A pooled block can still be in use by launches made before it was freed, so
+// whoever constructs a Tensor must touch it first on the NULL stream, which waits for them: `newtensor` zero-fills
+// there, `load` copies there.
+inline bool &tensor_pool_enabled() {
+    static bool on = [] { const char *e = std::getenv("DEEPX_POOL"); return !(e && !std::strcmp(e, "0")); }();
+    return on;
+}
+
 // A device tensor: metadata + an owned HBM allocation.
 struct Tensor {
     Shape shape;
     void *data = nullptr;
+    bool pooled = false;
 
     Tensor() = default;
-    Tensor(const std::vector<int> &dims, Precision p) : shape(dims, p) {
+    Tensor(const std::vector<int> &dims, Precision p) : shape(dims, p), pooled(tensor_pool_enabled()) {
         if (precision_bytes(p) == 0) throw std::invalid_argument("unsupported precision: " + precision_str(p));
-        dxh_check(dxh_malloc(&data, (size_t)shape.bytes()), "dxh_malloc");
+        if (pooled) dxh_check(dxh_pool_alloc(&data, (size_t)shape.bytes()), "dxh_pool_alloc");
+        else dxh_check(dxh_malloc(&data, (size_t)shape.bytes()), "dxh_malloc");
     }
     Tensor(const Tensor &) = delete;
     Tensor &operator=(const Tensor &) = delete;
-    ~Tensor() { if (data) dxh_free(data); }
+    ~Tensor() {
+        if (!data) return;
+        if (pooled) dxh_pool_free(data);
+        else dxh_free(data);
+    }
     int dtype() const { return (int)shape.dtype; }  // Precision value == dxh_dtype value
 };
 

@@ -8,9 +8,10 @@
 //   * a clash with one stream                    -> that stream (it runs behind what it depends on);
 //   * a clash with several streams               -> the first of them, which must first be made to wait for
 //                                                   an event recorded on each of the others (`wait_for`);
-//   * not kernel-only, or too much remembered    -> the default stream (`stream` = -1), which the caller's
-//                                                   runtime orders behind everything and everything behind
-//                                                   it; the memory is cleared.
+//   * not kernel-only, or too much remembered    -> the default stream (`stream` = -1), which the caller
+//                                                   orders behind everything and everything behind it
+//                                                   (`busy()` before the call names the streams that have
+//                                                   something to wait for); the memory is cleared.
 // Plain host code without a device call in it: the executor turns a Choice into streams and events
 // (executor.hpp), a host-only check replays random programs against a happens-before model
 // (tests/stream_picker_check.cpp).
@@ -37,6 +38,12 @@ public:
     // stream, a device-wide wait)
     void joined() {
         for (Side &s : sides_) { s.reads.clear(); s.writes.clear(); }
+    }
+    // side streams that have launched something since the last join
+    std::vector<int> busy() const {
+        std::vector<int> b;
+        for (size_t k = 0; k < sides_.size(); ++k) if (!sides_[k].reads.empty() || !sides_[k].writes.empty()) b.push_back((int)k);
+        return b;
     }
     size_t remembered() const {
         size_t n = 0;

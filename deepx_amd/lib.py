@@ -59,6 +59,11 @@ def scalar(v):
     return Scalar(f, i)
 
 
+class PoolStats(C.Structure):
+    """dxh_pool_stats_t of include/dxhip.h"""
+    _fields_ = [(n, C.c_uint64) for n in ("hits", "misses", "kept", "released", "kept_bytes", "kept_blocks", "live_bytes", "live_blocks")]
+
+
 _p, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 _pi32 = C.POINTER(C.c_int32)
 _pp = C.POINTER(C.c_void_p)
@@ -80,6 +85,11 @@ SIGNATURES = {
     "dxh_device_name": ([C.c_char_p, _sz], _i),
     "dxh_malloc": ([_pp, _sz], _i),
     "dxh_free": ([_p], _i),
+    "dxh_pool_alloc": ([_pp, _sz], _i),
+    "dxh_pool_free": ([_p], _i),
+    "dxh_pool_trim": ([_sz, C.POINTER(_sz)], _i),
+    "dxh_pool_limit": ([_sz], _i),
+    "dxh_pool_stats": ([C.POINTER(PoolStats)], _i),
     "dxh_memcpy_h2d": ([_p, _p, _sz, _p], _i),
     "dxh_memcpy_d2h": ([_p, _p, _sz, _p], _i),
     "dxh_memcpy_d2d": ([_p, _p, _sz, _p], _i),

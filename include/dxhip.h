@@ -30,8 +30,8 @@
  *    the convention of executor/op-cuda/src/deepx/tensorfunc/cuda_math.cuh:243-251.
  *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls
  *    are asynchronous: they return after enqueueing, like the reference's launches.
- *  - element counts are 64-bit; no entry point but dxh_malloc allocates device
- *    memory.  Those that need device scratch (reductions, matmul) take a
+ *  - element counts are 64-bit; no entry point but dxh_malloc and dxh_pool_alloc
+ *    allocates device memory.  Those that need device scratch (reductions, matmul) take a
  *    caller-provided workspace, sized by the matching *_workspace_bytes query.
  */
 #ifndef DXHIP_H
@@ -133,6 +133,33 @@ DXH_API int dxh_set_device(int device);
 DXH_API int dxh_device_name(char *buf, size_t buflen);
 DXH_API int dxh_malloc(void **ptr, size_t bytes);
 DXH_API int dxh_free(void *ptr);
+/* No counterpart in the reference, which goes to the driver for every tensor (cudaMalloc / cudaFree,
+ * executor/op-cuda/src/deepx/tensorfunc/tensorlife_miaobyte.hpp:20,31) while its front allocates the result of every op right
+ * before the op (front/py/deepx/nn/functional/leaffunc.py:30-38): freed blocks are kept by size class (eight classes per doubling,
+ * steps of at most 2 MiB) and handed out again, so that a `newtensor` / `deltensor` pair costs a few microseconds of host time
+ * instead of hipMalloc + a hipFree that waits for the device.  One pool per device; all five calls act on the current device's.
+ *  - dxh_pool_alloc: a block of at least `bytes` (0 bytes still gets a pointer of its own).  The block may have been freed
+ *    while launches that use it were still running: the caller's FIRST use of it must be ordered after them.  A launch or copy
+ *    on the NULL stream is (it waits for every blocking stream); a launch on another stream is only if that stream has waited
+ *    for them.  When the driver is out of memory every kept block goes back to it before the call gives up.
+ *  - dxh_pool_free: takes back a pointer from dxh_pool_alloc without waiting for the device; DXH_ERR_ARG for any other pointer
+ *    (the same one twice included), which is left alone.  Never pass such a pointer to dxh_free.
+ *  - dxh_pool_trim: gives kept blocks back to the driver, largest first, until at most `keep_bytes` stay (`released`, if not NULL,
+ *    gets the bytes given back).  dxh_malloc does this by itself when the driver is out of memory.
+ *  - dxh_pool_limit: the most bytes the pool keeps (default: half the device's memory, or DXH_POOL_MAX_MB from the environment when
+ *    the pool is first used); a free beyond it releases larger kept blocks first, and the block itself if it alone is over the limit.
+ *  - dxh_pool_stats: counts since the pool was made, and what it holds now. */
+typedef struct dxh_pool_stats_t {
+    uint64_t hits, misses;            /* allocations served from a kept block / by the driver */
+    uint64_t kept, released;          /* frees that kept the block / blocks given back to the driver */
+    uint64_t kept_bytes, kept_blocks; /* in the pool now */
+    uint64_t live_bytes, live_blocks; /* handed out now, in class sizes */
+} dxh_pool_stats_t;
+DXH_API int dxh_pool_alloc(void **ptr, size_t bytes);
+DXH_API int dxh_pool_free(void *ptr);
+DXH_API int dxh_pool_trim(size_t keep_bytes, size_t *released);
+DXH_API int dxh_pool_limit(size_t max_kept_bytes);
+DXH_API int dxh_pool_stats(dxh_pool_stats_t *out);
 DXH_API int dxh_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream);
 DXH_API int dxh_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream);
 DXH_API int dxh_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);

@@ -41,6 +41,7 @@ class InProc:
         L.dxe_set_sync.argtypes = [C.c_void_p, C.c_int]
         L.dxe_set_defer.argtypes = [C.c_void_p, C.c_int]
         L.dxe_set_streams.argtypes = [C.c_void_p, C.c_int]
+        L.dxe_set_pool.argtypes = [C.c_int]
         L.dxe_side_launches.argtypes = [C.c_void_p]
         L.dxe_side_launches.restype = C.c_size_t
         L.dxe_flush.argtypes = [C.c_void_p]
@@ -62,6 +63,7 @@ class InProc:
     def set_sync(self, on): self.L.dxe_set_sync(self.ex, int(on))
     def set_defer(self, on): self.L.dxe_set_defer(self.ex, int(on))
     def set_streams(self, n): self.L.dxe_set_streams(self.ex, int(n))
+    def set_pool(self, on): self.L.dxe_set_pool(int(on))  # process-wide: tensors made from now on
     def side_launches(self): return int(self.L.dxe_side_launches(self.ex))
     def flush(self): self.L.dxe_flush(self.ex)
     def held(self): return int(self.L.dxe_held(self.ex))

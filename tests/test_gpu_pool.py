@@ -1,0 +1,153 @@
+"""GPU: freed device blocks handed out again (dxh_pool_*), through the C ABI and under the executor's `newtensor` /
+`deltensor`.  The pool never waits for the device, so the cases that matter are blocks that come back while launches
+on them are still queued: whoever gets the block next must see its own data only."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from deepx_amd import lib as dx
+from tests.executor_client import InProc
+from tests.test_gpu_batch import Host, T, V
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _torch_owns_the_hip_runtime(dxh):
+    yield
+
+
+def pool_stats(L):
+    s = dx.PoolStats()
+    assert L.dxh_pool_stats(C.byref(s)) == 0
+    return {n: int(getattr(s, n)) for n, _ in dx.PoolStats._fields_}
+
+
+def pool_alloc(L, nbytes):
+    p = C.c_void_p()
+    assert L.dxh_pool_alloc(C.byref(p), nbytes) == 0 and p.value
+    return p.value
+
+
+def test_a_freed_block_is_the_next_one_of_its_class(dxh):
+    L = dxh
+    MB = 1 << 20
+    assert L.dxh_pool_trim(0, None) == 0
+    s0 = pool_stats(L)
+    assert s0["kept_blocks"] == 0
+    p, q = pool_alloc(L, 20 * MB), pool_alloc(L, 20 * MB)
+    assert p != q
+    pattern = np.arange(5 * MB, dtype=np.uint32)
+    assert L.dxh_memcpy_h2d(p, pattern.ctypes.data, pattern.nbytes, None) == 0
+    assert L.dxh_pool_free(p) == 0
+    r = pool_alloc(L, 20 * MB - 100)  # same class: the block just freed, with what it held (the pool clears nothing)
+    assert r == p
+    back = np.empty_like(pattern)
+    assert L.dxh_memcpy_d2h(back.ctypes.data, r, back.nbytes, None) == 0
+    assert np.array_equal(back, pattern)
+    other = pool_alloc(L, 3 * MB)  # another class: never one of these blocks
+    assert other not in (p, q)
+    s1 = pool_stats(L)
+    assert s1["hits"] - s0["hits"] == 1 and s1["misses"] - s0["misses"] == 3
+    assert s1["live_blocks"] - s0["live_blocks"] == 3 and s1["live_bytes"] - s0["live_bytes"] == 43 * MB
+    # a pointer the pool did not hand out, or has back already, is refused and left alone
+    raw = C.c_void_p()
+    assert L.dxh_malloc(C.byref(raw), 4096) == 0
+    assert L.dxh_pool_free(raw) == -2
+    assert L.dxh_free(raw) == 0
+    assert L.dxh_pool_free(q) == 0 and L.dxh_pool_free(q) == -2
+    assert L.dxh_pool_free(r) == 0 and L.dxh_pool_free(other) == 0 and L.dxh_pool_free(None) == 0
+    s2 = pool_stats(L)
+    assert s2["kept_blocks"] == 3 and s2["kept_bytes"] == 43 * MB and s2["live_blocks"] == s0["live_blocks"]
+    released = C.c_size_t()
+    assert L.dxh_pool_trim(24 * MB, C.byref(released)) == 0  # largest first: one 20 MiB block and the small one stay
+    assert released.value == 20 * MB and pool_stats(L)["kept_bytes"] == 23 * MB
+    assert L.dxh_pool_trim(0, C.byref(released)) == 0 and released.value == 23 * MB
+    assert pool_stats(L)["kept_blocks"] == 0
+    # zero bytes still get a pointer of their own
+    z1, z2 = pool_alloc(L, 0), pool_alloc(L, 0)
+    assert z1 != z2
+    assert L.dxh_pool_free(z1) == 0 and L.dxh_pool_free(z2) == 0
+
+
+def test_the_limit_on_kept_bytes(dxh):
+    L = dxh
+    MB = 1 << 20
+    assert L.dxh_pool_trim(0, None) == 0
+    try:
+        assert L.dxh_pool_limit(8 * MB) == 0
+        a, b, c = pool_alloc(L, 6 * MB), pool_alloc(L, 4 * MB), pool_alloc(L, 16 * MB)
+        before = pool_stats(L)
+        assert L.dxh_pool_free(c) == 0  # alone over the limit: straight back to the driver
+        assert pool_stats(L)["kept_blocks"] == 0 and pool_stats(L)["released"] == before["released"] + 1
+        assert L.dxh_pool_free(a) == 0 and pool_stats(L)["kept_bytes"] == 6 * MB
+        assert L.dxh_pool_free(b) == 0  # 10 MiB would be kept: the larger block goes
+        assert pool_stats(L)["kept_bytes"] == 4 * MB and pool_stats(L)["kept_blocks"] == 1
+    finally:
+        assert L.dxh_pool_limit(64 << 30) == 0
+    assert L.dxh_pool_trim(0, None) == 0
+
+
+@pytest.mark.parametrize("mode", ["in_order", "streams", "held"])
+def test_newtensor_on_a_block_still_in_use_is_zero(dxh, tmp_path, mode):
+    """`deltensor` right behind launches that write the tensor, then `newtensor` of the same size: the new tensor gets the
+    block that those launches are still writing (the pool says so), and must read as zeros afterwards, and a result
+    computed into it must be that result — in order, with independent lines on side streams, and with runs held back."""
+    L = dxh
+    shape = [4096, 8192]  # 128 MiB: each launch on it runs for tens of microseconds, several are queued at the free
+    rng = np.random.default_rng(197)
+    src = rng.uniform(-1, 1, shape).astype(np.float32)
+    ex = InProc()
+    ex.set_streams(3 if mode == "streams" else 1)
+    ex.set_defer(mode == "held")
+    h = Host(ex, tmp_path)
+    p = f"pool_{mode}_"
+    h.put(p + "src", src)
+    h.put(p + "src2", -src)
+    assert L.dxh_pool_trim(0, None) == 0
+    for it in range(4):
+        hits = pool_stats(L)["hits"]
+        lines = [f"newtensor({V(shape)})->({T(p + 'x')})", f"newtensor({V(shape)})->({T(p + 'w')})"]
+        lines += [f"addscalar({T(p + 'src')}, var<float32>:{it + 1})->({T(p + 'x')})",
+                  f"mulscalar({T(p + 'src2')}, var<float32>:3)->({T(p + 'w')})",
+                  f"mul({T(p + 'x')}, {T(p + 'w')})->({T(p + 'x')})",
+                  f"add({T(p + 'src')}, {T(p + 'src2')})->({T(p + 'w')})",
+                  f"exp({T(p + 'x')})->({T(p + 'x')})",
+                  f"deltensor()->({T(p + 'x')})", f"deltensor()->({T(p + 'w')})",
+                  f"newtensor({V(shape)})->({T(p + 'y')})", f"newtensor({V(shape)})->({T(p + 'y2')})"]
+        for line in lines:
+            h.run(line)
+        if it:  # the first pass fills the pool
+            assert pool_stats(L)["hits"] - hits == 4, "the blocks were not handed out again"
+        y, y2 = h.get(p + "y"), h.get(p + "y2")
+        assert not y.any() and not y2.any(), f"pass {it}: a new tensor is not zero"
+        h.run(f"addscalar({T(p + 'src')}, var<float32>:5)->({T(p + 'y')})")
+        h.run(f"deltensor()->({T(p + 'y2')})")
+        assert np.array_equal(h.get(p + "y"), src + np.float32(5))
+        h.run(f"deltensor()->({T(p + 'y')})")
+    if mode == "streams":
+        assert ex.side_launches() > 0
+    if mode == "held":
+        assert ex.defer_stats()["held_lines"] > 0
+
+
+def test_tensors_from_the_driver_when_the_pool_is_off(dxh, tmp_path):
+    L = dxh
+    ex = InProc()
+    h = Host(ex, tmp_path)
+    try:
+        ex.set_pool(False)
+        before = pool_stats(L)
+        h.run(f"newtensor({V([512, 512])})->({T('pool_off_a')})")
+        h.run(f"addscalar({T('pool_off_a')}, var<float32>:2)->({T('pool_off_a')})")
+        assert np.array_equal(h.get("pool_off_a"), np.full([512, 512], 2, np.float32))
+        ex.set_pool(True)
+        h.run(f"newtensor({V([512, 512])})->({T('pool_off_b')})")  # pooled, beside one that is not
+        h.run(f"deltensor()->({T('pool_off_a')})")
+        h.run(f"deltensor()->({T('pool_off_b')})")
+        after = pool_stats(L)
+        assert after["hits"] + after["misses"] - before["hits"] - before["misses"] == 1
+        assert after["kept"] - before["kept"] == 1 and after["live_blocks"] == before["live_blocks"]
+    finally:
+        ex.set_pool(True)

@@ -582,6 +582,7 @@ def bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr):
     del g16, u16, o16, x16, x32, o32, col
     torch.cuda.empty_cache()
     c5["mlp_block_over_deepxIR"] = config5_block_over_ir()
+    c5["mlp_block_with_its_allocations"] = config5_block_over_ir(with_allocations=True)
     res["config1"]["chain_over_deepxIR"] = config1_chain_over_ir()
     res["config5"] = c5
     return res
@@ -671,6 +672,8 @@ def _executor_lib():
     E.dxe_set_defer.argtypes = [C.c_void_p, C.c_int]
     E.dxe_flush.argtypes = [C.c_void_p]
     E.dxe_set_streams.argtypes = [C.c_void_p, C.c_int]
+    E.dxe_set_pool.argtypes = [C.c_int]
+    E.dxe_set_zero_later.argtypes = [C.c_void_p, C.c_int]
     return E
 
 
@@ -808,7 +811,7 @@ def config1_chain_over_ir(side=4096):
     return lines_over_ir(setup, block)
 
 
-def config5_block_over_ir(rows=2048, hidden=896, inter=4864, only=None, iters=30):
+def config5_block_over_ir(rows=2048, hidden=896, inter=4864, only=None, iters=30, with_allocations=False):
     """The whole config-5 block (RMSNorm + gated MLP, 22 deepxIR compute ops on [2048,896] activations)."""
     S, Hd, I = rows, hidden, inter
     b16, f32 = "bfloat16", "float32"
@@ -846,8 +849,74 @@ def config5_block_over_ir(rows=2048, hidden=896, inter=4864, only=None, iters=30
              f"mul({n('g', b16)}, {n('sg', b16)})->({n('sg', b16)})",
              f"mul({n('sg', b16)}, {n('u', b16)})->({n('sg', b16)})",
              f"matmul({n('sg', b16)}, {n('Wd', b16)})->({n('y', b16)})"]
+    if with_allocations:
+        return block_with_its_allocations(setup, block, tensors[5:], lambda name, shape, dt: f"newtensor({V(shape)})->({T('b5_' + name, dt)})",
+                                          lambda name, dt: f"deltensor()->({T('b5_' + name, dt)})", iters=iters)
     out = lines_over_ir(setup, block, iters=iters, only=only)
     out["rows"] = S
+    return out
+
+
+def block_with_its_allocations(setup, block, temporaries, new_line, del_line, iters=30):
+    """`block` as a front that owns no tensor between passes sends it (front/py/deepx/nn/functional/leaffunc.py:30-38 allocates
+    the result of every op right before the op; the tensors go when the Python objects do): each temporary is allocated by a
+    `newtensor` line right before the first line that writes it and deleted by a `deltensor` line after the last line of the
+    pass.  Wall time per pass with tensor storage from the pool of freed blocks (the default) and from the driver (DEEPX_POOL=0,
+    what the reference does), line by line, line by line with runs held back, and as one datagram."""
+    import ctypes as C
+    from deepx_amd import lib as dx
+    L = dx.load()
+    E = _executor_lib()
+    lines, made = [], set()
+    for line in block:
+        result = line.split("->(")[1]
+        for name, shape, dt in temporaries:
+            if name not in made and f":b5_{name})" in result:
+                lines.append(new_line(name, shape, dt))
+                made.add(name)
+        lines.append(line)
+    lines += [del_line(name, dt) for name, _, dt in temporaries if name in made]
+    lines = [f"{l} // author=miaobyte id={i + 1}" for i, l in enumerate(lines)]
+    text = "\n".join(lines).encode()
+    out = {"lines": len(lines), "allocations": len(made)}
+    for label, pool, defer, batched in (("line_by_line_us", 1, 0, 0), ("line_by_line_storage_from_the_driver_us", 0, 0, 0),
+                                        ("line_by_line_deferred_us", 1, 1, 0), ("one_batch_fused_us", 1, 0, 1),
+                                        ("one_batch_fused_storage_from_the_driver_us", 0, 0, 1)):
+        E.dxe_set_pool(pool)
+        try:
+            ex = E.dxe_create()
+            buf = C.create_string_buffer(1 << 16)
+            for line in setup:
+                if any(line.startswith("newtensor(") and f":b5_{name})" in line for name in made):
+                    continue  # the pass allocates these itself
+                E.dxe_execute(ex, line.encode(), buf, len(buf))
+                if " ok" not in buf.value.decode().split("//")[0]:
+                    raise RuntimeError(f"{line}: {buf.value.decode()}")
+            E.dxe_set_defer(ex, defer)
+
+            def once():
+                if batched:
+                    E.dxe_execute_batch(ex, text, buf, len(buf))
+                else:
+                    for l in lines:
+                        E.dxe_execute(ex, l.encode(), buf, len(buf))
+                if any(" ok" not in r.split("//")[0] for r in buf.value.decode().split("\n")):
+                    raise RuntimeError("block failed: " + buf.value.decode())
+
+            n = iters if pool else max(5, iters // 3)
+            for _ in range(3):
+                once()
+            E.dxe_flush(ex)
+            dx.check(L.dxh_device_sync())
+            t0 = time.perf_counter()
+            for _ in range(n):
+                once()
+            E.dxe_flush(ex)
+            dx.check(L.dxh_device_sync())
+            out[label] = round((time.perf_counter() - t0) / n * 1e6, 1)
+            E.dxe_destroy(ex)
+        finally:
+            E.dxe_set_pool(1)
     return out
 
 

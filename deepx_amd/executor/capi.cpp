@@ -59,6 +59,8 @@ DXE_API void dxe_set_streams(void *ex, int n) { static_cast<Executor *>(ex)->str
 DXE_API size_t dxe_side_launches(void *ex) { return (size_t)static_cast<Executor *>(ex)->stats.side_launches; }
 // tensors allocated from now on take their storage from the library's pool of freed blocks (1, the default; the DEEPX_POOL
 // switch) or from the driver each time (0); tensors that exist keep what they have and return it where it came from
+// 1 (default): `newtensor` owes its zero fill to the first launch that names the tensor; 0: it fills at once (DEEPX_ZERO_AT_ALLOC=1)
+DXE_API void dxe_set_zero_later(void *ex, int on) { static_cast<Executor *>(ex)->mem.zero_later = on != 0; }
 DXE_API void dxe_set_pool(int on) { deepx::tensor_pool_enabled() = on != 0; }
 DXE_API size_t dxe_fusion_stats(void *ex, char *out, size_t buflen) {
     const auto &s = static_cast<Executor *>(ex)->stats;

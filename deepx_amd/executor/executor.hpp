@@ -198,7 +198,10 @@ public:
             one[0].tf = tf;
             pick_stream(one, {tf}, 0);
         }
+        std::vector<std::shared_ptr<Tensor>> dropped;
+        settle(*tf, dropped);
         for (int i = 0; i < repeat && rc == 0; ++i) rc = tf->run(mem, message);
+        if (rc != 0) make_good(dropped);
         mem.stream = nullptr;
         mem.scratch_of = nullptr;
         lap(prof.run_ns);
@@ -303,13 +306,17 @@ public:
         std::vector<size_t> order;
         {
             std::vector<size_t> rest;
+            std::unordered_set<std::string> named;  // every word of the lines so far that could be a tensor's name
             for (size_t i = 0; i < items.size(); ++i) {
-                bool hoist = !items[i].failed && items[i].tf && items[i].call.name == "newtensor" && items[i].call.returns.size() == 1;
-                if (hoist) {
-                    const std::string &name = items[i].call.returns[0].textvalue;
-                    for (size_t j = 0; j < i && hoist; ++j) hoist = items[j].failed ? lines[j].find(name) == std::string::npos : !mentions(items[j].call, name);
-                }
+                const bool hoist = !items[i].failed && items[i].tf && items[i].call.name == "newtensor" && items[i].call.returns.size() == 1 &&
+                                   !named.count(items[i].call.returns[0].textvalue);
                 (hoist ? order : rest).push_back(i);
+                if (items[i].failed) {  // a line that did not parse: anything between its punctuation counts
+                    each_word(lines[i], " []()<>,:", [&](const std::string &w) { named.insert(w); });
+                } else {
+                    for (const std::vector<Param> *ps : {&items[i].call.args, &items[i].call.returns})
+                        for (const Param &prm : *ps) each_word(prm.textvalue, " []", [&](const std::string &w) { named.insert(w); });
+                }
             }
             if (order.empty() || order.size() == items.size()) order.clear();
             else order.insert(order.end(), rest.begin(), rest.end());
@@ -334,23 +341,30 @@ private:
         // Runs line i, or a run of lines that starts at i as one launch; returns how many lines that were.
         // A run that cannot be launched after all falls back to its first line alone.
         auto run_next = [&](size_t i, std::string &message, int &rc) -> size_t {
+            std::vector<std::shared_ptr<Tensor>> dropped;
             if (use_fusion && has_device) {
                 const size_t len = chain_length(tfs, i, mem);
                 if (len >= 2) {
+                    for (size_t j = i; j < i + len; ++j) settle(*tfs[j], dropped);
                     try { rc = run_chain(tfs, i, len, mem, message); } catch (const std::exception &e) { rc = 1; message = e.what(); }
                     if (rc == 0) { ++stats.fused_runs; stats.fused_lines += len; return len; }
+                    make_good(dropped);
                     message.clear();
                 }
                 const size_t group = matmul_group_length(tfs, i, mem);
                 if (group >= 2) {
+                    for (size_t j = i; j < i + group; ++j) settle(*tfs[j], dropped);
                     try { rc = run_matmul_group(tfs, i, group, mem, message); } catch (const std::exception &e) { rc = 1; message = e.what(); }
                     if (rc == 0) { ++stats.matmul_groups; stats.matmul_lines += group; return group; }
+                    make_good(dropped);
                     message.clear();
                 }
             }
             const int repeat = items[i].tf->metadata.benchmark_repeat > 1 ? items[i].tf->metadata.benchmark_repeat : 1;
             rc = 0;
+            settle(*items[i].tf, dropped);
             for (int r = 0; r < repeat && rc == 0; ++r) rc = items[i].tf->run(mem, message);
+            if (rc != 0) make_good(dropped);
             return 1;
         };
         bool done = false;
@@ -425,6 +439,9 @@ private:
             kernel_only = kernel_only && items[j].tf->graph_safe && items[j].tf->metadata.benchmark_repeat <= 1;
             names_in(items[j].call.args, reads);
             names_in(items[j].call.returns, writes);
+            each_tensor(items[j].call.args, [&](const std::shared_ptr<Tensor> &t) {  // an argument that is still owed its zero fill is written first
+                if (t->zero_pending) names_in(items[j].call.args, writes);
+            });
         }
         while (side_.size() < (size_t)streams) {
             Side sd;
@@ -451,6 +468,44 @@ private:
         mem.stream = mem.scratch_of = side_[(size_t)c.stream].stream;
         ++stats.side_launches;
     }
+    // `fn(word)` for every run of characters of `text` that holds none of `separators`
+    template <typename Fn>
+    static void each_word(const std::string &text, const char *separators, Fn fn) {
+        for (size_t b = 0; b < text.size();) {
+            b = text.find_first_not_of(separators, b);
+            if (b == std::string::npos) break;
+            size_t e = text.find_first_of(separators, b);
+            if (e == std::string::npos) e = text.size();
+            fn(text.substr(b, e - b));
+            b = e;
+        }
+    }
+    // `fn(tensor)` for every existing tensor among the words of `ps` (bare names, typed params and [a b c] lists alike)
+    template <typename Fn>
+    void each_tensor(const std::vector<Param> &ps, Fn fn) const {
+        for (const Param &p : ps)
+            each_word(p.textvalue, " []", [&](const std::string &w) { if (auto found = mem.findtensor(w)) fn(found); });
+    }
+    // A tensor fresh from `newtensor` reads as zeros but may not hold them yet (Tensor::zero_pending).  Before anything is
+    // launched for `tf`: every such tensor among its arguments is filled now, on the stream the launch goes to, and so is
+    // one among its results — unless the op writes every element of its results anyway: then the fill is dropped, and
+    // `dropped` keeps the tensor so that a launch that fails after all can make it (make_good).  `deltensor` settles
+    // nothing: nobody will read what it names.
+    void settle(const TF &tf, std::vector<std::shared_ptr<Tensor>> &dropped) {
+        if (tf.name == "deltensor") return;
+        each_tensor(tf.args, [&](const std::shared_ptr<Tensor> &t) {
+            if (t->zero_pending) t->fill_zero(mem.stream);
+        });
+        each_tensor(tf.returns, [&](const std::shared_ptr<Tensor> &t) {
+            if (!t->zero_pending) return;
+            if (tf.overwrites_results && !mem.recording) { t->zero_pending = false; dropped.push_back(t); }
+            else t->fill_zero(mem.stream);
+        });
+    }
+    void make_good(std::vector<std::shared_ptr<Tensor>> &dropped) {
+        for (auto &t : dropped) t->fill_zero(mem.stream);
+        dropped.clear();
+    }
     // Orders everything the `busy` side streams have been given so far before whatever any stream is given from now on.
     // A launch on the default stream would do that by itself (it waits for every blocking stream, and they for it), but a
     // line sent there need not launch anything: `deltensor`, `renametensor` and `argset` are host work, an empty tensor
@@ -474,24 +529,13 @@ private:
     }
     // does a call name `word` among its arguments or results (bare, typed, or inside a [a b c] list)
     static bool mentions(const TF &call, const std::string &word) {
+        bool found = false;
         for (const std::vector<Param> *ps : {&call.args, &call.returns})
-            for (const Param &p : *ps) {
-                std::string t = p.textvalue;
-                for (char &c : t) if (c == '[' || c == ']') c = ' ';
-                std::istringstream in(t);
-                std::string w;
-                while (in >> w) if (w == word) return true;
-            }
-        return false;
+            for (const Param &p : *ps) each_word(p.textvalue, " []", [&](const std::string &w) { found = found || w == word; });
+        return found;
     }
     void names_in(const std::vector<Param> &ps, std::vector<std::string> &names) const {
-        for (const Param &p : ps) {
-            std::string t = p.textvalue;
-            for (char &c : t) if (c == '[' || c == ']') c = ' ';
-            std::istringstream in(t);
-            std::string w;
-            while (in >> w) if (mem.existstensor(w)) names.push_back(w);
-        }
+        for (const Param &p : ps) each_word(p.textvalue, " []", [&](const std::string &w) { if (mem.existstensor(w)) names.push_back(w); });
     }
 
     // What a recorded graph froze about a tensor: the kernels' pointer arguments and every launch
@@ -504,28 +548,14 @@ private:
 
     // every tensor a call names (bare names, typed params and [a b c] lists alike)
     void tensors_of(const TF &call, std::vector<std::string> &names) const {
-        auto scan = [&](const std::vector<Param> &ps) {
-            for (const Param &p : ps) {
-                std::string t = p.textvalue;
-                for (char &c : t) if (c == '[' || c == ']') c = ' ';
-                std::istringstream in(t);
-                std::string w;
-                while (in >> w) if (mem.existstensor(w)) names.push_back(w);
-            }
-        };
-        scan(call.args);
-        scan(call.returns);
+        names_in(call.args, names);
+        names_in(call.returns, names);
     }
     // a scalar or vector taken from the arg store would be frozen into a recorded graph
     bool uses_named_arg(const TF &call) const {
-        for (const Param &p : call.args) {
-            std::string t = p.textvalue;
-            for (char &c : t) if (c == '[' || c == ']') c = ' ';
-            std::istringstream in(t);
-            std::string w;
-            while (in >> w) if (!mem.existstensor(w) && mem.existarg(w)) return true;
-        }
-        return false;
+        bool named = false;
+        for (const Param &p : call.args) each_word(p.textvalue, " []", [&](const std::string &w) { named = named || (!mem.existstensor(w) && mem.existarg(w)); });
+        return named;
     }
     bool snapshot(size_t n, const std::function<const TF &(size_t)> &call_at, Graph &g) const {
         std::vector<std::string> names;
@@ -552,7 +582,17 @@ private:
         dxh_graph_destroy(g.exec);
         g.exec = nullptr;
     }
+    // A recorded graph must not hold the zero fill that a fresh tensor is owed (every replay would clear the tensor again),
+    // and a replay reads its tensors as they are: whatever the batch names gets its fill now, on the default stream, which
+    // the graph's stream waits for.
+    void settle_pins(const Graph &g) {
+        for (const Pinned &p : g.tensors) {
+            auto t = mem.findtensor(p.name);
+            if (t && t->zero_pending) t->fill_zero(nullptr);
+        }
+    }
     bool launch_graph(const Graph &g) {
+        settle_pins(g);
         graph_flying_ = true;
         return dxh_graph_launch(g.exec, graph_stream_) == DXH_OK && (!sync_each || dxh_stream_sync(graph_stream_) == DXH_OK);
     }
@@ -590,6 +630,7 @@ private:
             if (rejected_.size() >= kMaxRemembered) rejected_.clear();
             if (seen_.insert(key).second) return false;  // first arrival: run eagerly
             if (!graph_stream_ && dxh_stream_create(&graph_stream_) != DXH_OK) { graph_stream_ = nullptr; return false; }
+            settle_pins(now);
             if (dxh_stream_sync(nullptr) != DXH_OK) return false;
             if (dxh_graph_begin_capture(graph_stream_) != DXH_OK) return false;
             mem.stream = graph_stream_;
@@ -615,6 +656,7 @@ private:
         } else {
             ++stats.graph_replays;
         }
+        settle_pins(it->second);
         graph_flying_ = true;
         if (dxh_graph_launch(it->second.exec, graph_stream_) != DXH_OK || (sync_each && dxh_stream_sync(graph_stream_) != DXH_OK)) {
             drop_graph(it->second);

@@ -78,9 +78,12 @@ struct TFMetadata {
     int benchmark_repeat = 0;
 
     void parse(const std::string &meta) {
-        std::istringstream in(meta);
-        std::string kv;
-        while (in >> kv) {
+        static const char *blank = " \t\n\r\f\v";  // what `stream >> word` skips; no stream here: this runs for every line
+        for (size_t b = 0; (b = meta.find_first_not_of(blank, b)) != std::string::npos;) {
+            size_t e = meta.find_first_of(blank, b);
+            if (e == std::string::npos) e = meta.size();
+            const std::string kv = meta.substr(b, e - b);
+            b = e;
             size_t eq = kv.find('=');
             if (eq == std::string::npos) continue;
             std::string k = kv.substr(0, eq), v = kv.substr(eq + 1);
@@ -106,11 +109,13 @@ struct TFMetadata {
 
 inline std::vector<Param> parse_params(const std::string &list) {
     std::vector<Param> out;
-    std::istringstream in(list);
-    std::string item;
-    while (std::getline(in, item, ',')) {
+    for (size_t b = 0; b <= list.size();) {
+        size_t e = list.find(',', b);
+        if (e == std::string::npos) e = list.size();
+        std::string item = list.substr(b, e - b);
         trim_spaces(item);
         if (!item.empty()) out.push_back(Param::parse(item));
+        b = e + 1;
     }
     return out;
 }
@@ -125,6 +130,9 @@ public:
     // true for ops that only launch kernels on Mem's stream (no allocation, host copy, file I/O or
     // fresh random seed): those may be recorded into a HIP graph by the batch path
     bool graph_safe = false;
+    // true for ops that write every element of each tensor they return, whatever it held: the zero fill that a fresh
+    // tensor still owes (Tensor::zero_pending) is dropped for their results instead of being made
+    bool overwrites_results = false;
     // float elementwise ops that dxh_chain can run as part of one launch: its op code, and where the
     // operands sit (1: args 0 and 1 are tensors, 2: tensor then scalar, 3: scalar then tensor, 4: one tensor)
     int chain_code = -1, chain_kind = 0;
@@ -180,11 +188,19 @@ struct OpResp {
     void error(const std::string &msg) { result = "error"; finish_at = std::chrono::system_clock::now(); message = msg; }
     // no space between the result word and "//", as tf.hpp:198-213 prints it; the front splits on "//"
     std::string to_string() const {
-        std::ostringstream o;
-        o << id << " " << result << "// recv_at=" << epoch_ms(recv_at) << " start_at=" << epoch_ms(start_at)
-          << " finish_at=" << epoch_ms(finish_at);
-        if (!message.empty()) o << " " << message;
-        return o.str();
+        std::string o;  // appended by hand: a stream costs more than the rest of a reply
+        o.reserve(96 + message.size());
+        o += std::to_string(id);
+        o += ' ';
+        o += result;
+        o += "// recv_at=";
+        o += std::to_string(epoch_ms(recv_at));
+        o += " start_at=";
+        o += std::to_string(epoch_ms(start_at));
+        o += " finish_at=";
+        o += std::to_string(epoch_ms(finish_at));
+        if (!message.empty()) { o += ' '; o += message; }
+        return o;
     }
 };
 

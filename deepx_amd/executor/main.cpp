@@ -10,6 +10,8 @@
 //   DEEPX_DEFER    1: hold lines that can share a launch with the next one (DEEPX_DEFER_US: longest wait for it, default 200)
 //   DEEPX_POOL     0: every tensor's storage comes from and goes back to the driver, as in the reference (default: freed
 //                  blocks are kept, up to DXH_POOL_MAX_MB or half the device's memory, and handed out again)
+//   DEEPX_ZERO_AT_ALLOC 1: `newtensor` launches its zero fill at once (default: the first launch that names the tensor makes
+//                  the fill, or drops it when it overwrites the whole tensor)
 //   DEEPX_OPLIST   path: write the generated op table (markdown) there, as the reference writes
 //                  docs/executor/op-mem-*/list.md at start-up
 #include <csignal>

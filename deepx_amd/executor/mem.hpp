@@ -41,6 +41,9 @@ struct Tensor {
     Shape shape;
     void *data = nullptr;
     bool pooled = false;
+    // The tensor is new and reads as zeros by definition, but the fill has not been launched: the block holds whatever
+    // its last owner left.  Nothing may launch a kernel that names the tensor before this is settled (Executor::settle).
+    bool zero_pending = false;
 
     Tensor() = default;
     Tensor(const std::vector<int> &dims, Precision p) : shape(dims, p), pooled(tensor_pool_enabled()) {
@@ -56,6 +59,13 @@ struct Tensor {
         else dxh_free(data);
     }
     int dtype() const { return (int)shape.dtype; }  // Precision value == dxh_dtype value
+    // launches the zero fill on `stream` (bool and f8 tensors fill as bytes) and clears zero_pending
+    int fill_zero(void *stream) {
+        zero_pending = false;
+        const Precision p = shape.dtype;
+        const int dt = (p == Precision::Float8E5M2 || p == Precision::Float8E4M3) ? (int)DXH_I8 : (int)p;
+        return dxh_constant(dt, data, shape.size, dxh_scalar{0.0, 0}, stream);
+    }
 };
 
 using ArgValue = std::variant<int32_t, int64_t, float, double, bool, std::string, std::vector<int32_t>,
@@ -99,6 +109,10 @@ public:
     // grow aborts the recording instead.
     void *stream = nullptr;
     bool recording = false;
+    // `newtensor` owes its zero fill to the first launch that names the tensor instead of making it at once (DEEPX_ZERO_AT_ALLOC=1
+    // turns that off): the front allocates every result right before the op that overwrites it, and a fill of the result's
+    // size costs about as much as a bandwidth-bound op itself.
+    bool zero_later = [] { const char *e = std::getenv("DEEPX_ZERO_AT_ALLOC"); return !(e && !std::strcmp(e, "1")); }();
 
     // reusable device scratch for reductions and products (grown on demand, never shrunk).  Launches that may run
     // side by side on two streams must not share it: the executor names the scratch an op is to use (`scratch_of`,

@@ -87,6 +87,7 @@ void reg(TfFactory &f, const char *name, const char *author, const char *tftype,
     tf->graph_safe = kind == "elementwise" || kind == "reduce" || kind == "changeshape" || op == "matmul" ||
                      op == "constant" || op == "arange";
     if (op == "reshape") tf->graph_safe = false;  // rewrites the tensor's shape on the host
+    tf->overwrites_results = tf->graph_safe || op == "uniform" || op == "normal" || op == "copytensor" || op == "loadtensordata";
     f.add_tf(tf);
 }
 
@@ -265,14 +266,15 @@ RunFn reduce(ReduceFn f, const char *op) {  // (A, vector dims, bool keepdims) -
     };
 }
 
-std::shared_ptr<Tensor> new_tensor(const std::vector<int> &shape, Precision p) {
+// "T1 = zeros(shape)", as op-cuda's newtensor documents itself (its storage is whatever cudaMalloc returns).  The fill is
+// made here, on the NULL stream, or owed (`zero_later`): then whoever launches the first kernel that names the tensor makes
+// it, or drops it when that kernel overwrites the whole tensor anyway (Executor::settle).
+std::shared_ptr<Tensor> new_tensor(const std::vector<int> &shape, Precision p, bool zero_later) {
     for (int d : shape) if (d < 0) throw std::invalid_argument("negative dimension in shape " + dims_str(shape));
     if (shape.empty()) throw std::invalid_argument("newtensor: empty shape");
     auto t = std::make_shared<Tensor>(shape, p);
-    dxh_scalar zero{0.0, 0};
-    // zero-filled like op-cuda's "T1 = zeros(shape)"; bool/f8 tensors fill as bytes
-    int dt = (p == Precision::Float8E5M2 || p == Precision::Float8E4M3) ? (int)DXH_I8 : (int)p;
-    dxh_check(dxh_constant(dt, t->data, t->shape.size, zero, nullptr), "newtensor zero fill");
+    if (zero_later) t->zero_pending = true;
+    else dxh_check(t->fill_zero(nullptr), "newtensor zero fill");
     return t;
 }
 
@@ -286,7 +288,7 @@ int register_all(TfFactory &f) {
         if (precision_bytes(t.precision) == 0) return fail(error, "newtensor: unsupported precision " + precision_str(t.precision));
         if (t.precision == Precision::Float8E5M2 || t.precision == Precision::Float8E4M3)
             return fail(error, "newtensor: " + precision_str(t.precision) + " has not been implemented");
-        auto tensor = new_tensor(ints_of(c.args[0], mem), t.precision);
+        auto tensor = new_tensor(ints_of(c.args[0], mem), t.precision, mem.zero_later);
         if (!mem.addtensor(c.returns[0].textvalue, tensor)) std::cerr << "tensor already exists: " << c.returns[0].textvalue << std::endl;
         return 0;
     };

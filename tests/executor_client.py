@@ -42,6 +42,7 @@ class InProc:
         L.dxe_set_defer.argtypes = [C.c_void_p, C.c_int]
         L.dxe_set_streams.argtypes = [C.c_void_p, C.c_int]
         L.dxe_set_pool.argtypes = [C.c_int]
+        L.dxe_set_zero_later.argtypes = [C.c_void_p, C.c_int]
         L.dxe_side_launches.argtypes = [C.c_void_p]
         L.dxe_side_launches.restype = C.c_size_t
         L.dxe_flush.argtypes = [C.c_void_p]
@@ -63,6 +64,7 @@ class InProc:
     def set_sync(self, on): self.L.dxe_set_sync(self.ex, int(on))
     def set_defer(self, on): self.L.dxe_set_defer(self.ex, int(on))
     def set_streams(self, n): self.L.dxe_set_streams(self.ex, int(n))
+    def set_zero_later(self, on): self.L.dxe_set_zero_later(self.ex, int(on))
     def set_pool(self, on): self.L.dxe_set_pool(int(on))  # process-wide: tensors made from now on
     def side_launches(self): return int(self.L.dxe_side_launches(self.ex))
     def flush(self): self.L.dxe_flush(self.ex)

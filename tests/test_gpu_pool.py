@@ -151,3 +151,87 @@ def test_tensors_from_the_driver_when_the_pool_is_off(dxh, tmp_path):
         assert after["kept"] - before["kept"] == 1 and after["live_blocks"] == before["live_blocks"]
     finally:
         ex.set_pool(True)
+
+
+def dirty_blocks(h, L, prefix, shape, count, dt="float32"):
+    """leaves `count` blocks of this shape's class in the pool, full of sevens"""
+    for i in range(count):
+        h.run(f"newtensor({V(shape)})->({T(prefix + f'dirt{i}', dt)})")
+        h.run(f"constant(var<float32>:7)->({T(prefix + f'dirt{i}', dt)})")
+    for i in range(count):
+        h.run(f"deltensor()->({T(prefix + f'dirt{i}', dt)})")
+
+
+@pytest.mark.parametrize("mode", ["lines", "batch", "batch_unfused", "graph", "streams", "held", "fill_at_once"])
+def test_a_new_tensor_reads_as_zeros_whoever_touches_it_first(dxh, tmp_path, mode):
+    """`newtensor` owes its zero fill to the first launch that names the tensor.  On blocks full of sevens: a tensor that is
+    read before anything wrote it reads as zeros (as an operand, in place, inside a fused run, by two lines that may sit on
+    two streams, by a replayed graph whose tensors were deleted and made again at the same addresses); a tensor that an op
+    overwrites holds that op's result; and a tensor whose op failed reads as zeros afterwards."""
+    L = dxh
+    shape = [1024, 2048]
+    rng = np.random.default_rng(199)
+    src = rng.uniform(-1, 1, shape).astype(np.float32)
+    ex = InProc()
+    ex.set_streams(3 if mode == "streams" else 1)
+    ex.set_defer(mode == "held")
+    ex.set_graphs(mode == "graph")
+    ex.set_fusion(mode != "batch_unfused")
+    ex.set_zero_later(mode != "fill_at_once")
+    h = Host(ex, tmp_path)
+    p = f"lz_{mode}_"
+    n = lambda name: T(p + name)
+    h.put(p + "src", src)
+    h.run(f"newtensor({V([3, 5])})->({n('small')})")
+    fresh = ["y", "y2", "y3", "z", "z2", "w", "t1", "t2", "r", "never"]
+    block = [f"add({n('y')}, {n('src')})->({n('z')})",            # y read first: zeros
+             f"mul({n('y')}, {n('src')})->({n('z2')})",           # and by a second line that depends on nothing the first one writes
+             f"addscalar({n('y2')}, var<float32>:2)->({n('y2')})",  # in place
+             f"mulscalar({n('y3')}, var<float32>:3)->({n('t1')})",  # a run that starts by reading a fresh tensor
+             f"add({n('t1')}, {n('src')})->({n('t2')})",
+             f"exp({n('t2')})->({n('w')})",
+             f"sum({n('src')}, {V([1])}, var<bool>:false)->({n('r')})"]
+    block = [f"{l} // author=miaobyte id={i + 1}" for i, l in enumerate(block)]
+    for it in range(4):  # with graphs: eager, recorded, replayed, replayed — the tensors deleted and made again in between
+        dirty_blocks(h, L, p, shape, len(fresh))
+        hits = pool_stats(L)["hits"]
+        for name in fresh:
+            h.run(f"newtensor({V(shape if name != 'r' else [shape[0]])})->({n(name)})")
+        assert pool_stats(L)["hits"] - hits >= len(fresh) - 1, "the new tensors did not get used blocks"
+        if mode in ("lines", "streams", "held", "fill_at_once"):
+            replies = [ex.execute(l) for l in block]
+        else:
+            replies = ex.execute_batch(block)
+        assert all(r.split(" ")[1].startswith("ok") for r in replies), replies
+        bad = ex.execute(f"add({n('src')}, {n('small')})->({n('never')}) // id=77")  # fails: shapes differ
+        assert bad.startswith("77 error"), bad
+        ex.flush()
+        assert np.array_equal(h.get(p + "z"), src), it
+        assert not h.get(p + "z2").any() and not h.get(p + "y").any(), it
+        assert np.array_equal(h.get(p + "y2"), np.full(shape, 2, np.float32)), it
+        assert not h.get(p + "t1").any() and np.array_equal(h.get(p + "t2"), src), it
+        assert np.allclose(h.get(p + "w"), np.exp(src), rtol=1e-6), it
+        assert np.allclose(h.get(p + "r"), src.astype(np.float64).sum(1), rtol=1e-5, atol=1e-4), it
+        assert not h.get(p + "never").any(), "a tensor whose op failed does not read as zeros"
+        if mode == "graph":
+            # the same batch again with one tensor deleted and made again on its own block, now full of sevens: every
+            # pointer the recorded graph holds is still right, so it is replayed, and must still read that tensor as zeros
+            replays = ex.stats()["replays"]
+            h.run(f"constant(var<float32>:7)->({n('y')})")
+            y_hits = pool_stats(L)["hits"]
+            h.run(f"deltensor()->({n('y')})")
+            h.run(f"newtensor({V(shape)})->({n('y')})")
+            assert pool_stats(L)["hits"] == y_hits + 1
+            replies = ex.execute_batch(block)
+            assert all(r.split(" ")[1].startswith("ok") for r in replies), replies
+            if it:  # the pass before recorded it
+                assert ex.stats()["replays"] == replays + 1, ex.stats()
+            assert np.array_equal(h.get(p + "z"), src) and not h.get(p + "z2").any() and not h.get(p + "y").any(), it
+        for name in fresh:
+            h.run(f"deltensor()->({n(name)})")
+    if mode == "graph":
+        assert ex.stats()["replays"] >= 1, ex.stats()
+    if mode == "streams":
+        assert ex.side_launches() > 0
+    if mode in ("batch", "held"):
+        assert ex.fusion_stats()["runs"] >= 4

@@ -317,6 +317,7 @@ def main():
         torch.cuda.empty_cache()
         per_op.update(bench_other_configs(L, dx, torch, np, dev, ev, Events, ptr))
         per_op["config2"]["step_over_deepxIR"] = config2_step_over_ir(step_bytes, side_streams=not args.in_order_only)
+        per_op["attention_core_over_deepxIR"] = attention_core_over_ir()
 
     # ---------------- CPU baseline: the oracle's restatement of op-ompsimd's reduce ---------
     cpu = None
@@ -809,6 +810,35 @@ def config1_chain_over_ir(side=4096):
              f"exp({T('E')})->({T('F')})", f"mulscalar({T('B')}, var<float32>:-1)->({T('nB')})", f"max({T('B')}, {T('nB')})->({T('absB')})",
              f"addscalar({T('absB')}, var<float32>:1)->({T('den')})", f"div({T('F')}, {T('den')})->({T('G')})"]
     return lines_over_ir(setup, block)
+
+
+def attention_core_over_ir(S=2048, heads=14, hd=64, iters=20):
+    """The core of the front's attention on the activations of config 3 / config 5 (one sequence of 2048 tokens, 14 heads of 64;
+    front/py/deepx/nn/modules/transformer/attention.py:15-32, softmax as normalization.py:4-17 spells it), bf16, 12 deepxIR
+    lines: transpose of k, q @ k.mT, the scaling, the softmax's eight lines, the product with v.  Not a BASELINE config: the
+    caller next to the config-5 block, through the same executor modes."""
+    dt = "bfloat16"
+    T = lambda n: f"tensor<{dt}>:at_{n}"
+    V = lambda v: "vector<int32>:[" + " ".join(str(x) for x in v) + "]"
+    full, col, io = [1, heads, S, S], [1, heads, S, 1], [1, heads, S, hd]
+    tensors = [("q", io), ("k", io), ("v", io), ("kT", [1, heads, hd, S]), ("sc", full), ("a", full), ("m", col), ("mb", full), ("d", full), ("e", full),
+               ("s", col), ("e2", full), ("sb", full), ("y", full), ("o", io)]
+    setup = [f"newtensor({V(shape)})->({T(name)})" for name, shape in tensors]
+    setup += [f"normal(var<float32>:0, var<float32>:1, var<int32>:{21 + i})->({T(name)}) // author=miaobyte" for i, name in enumerate(("q", "k", "v"))]
+    block = [f"transpose({T('k')}, {V([0, 1, 3, 2])})->({T('kT')})", f"matmul({T('q')}, {T('kT')})->({T('sc')})",
+             f"mulscalar({T('sc')}, var<float32>:{hd ** -0.5})->({T('a')})",
+             f"reducemax({T('a')}, {V([-1])}, var<bool>:true)->({T('m')})", f"broadcastTo({T('m')}, {V(full)})->({T('mb')})",
+             f"sub({T('a')}, {T('mb')})->({T('d')})", f"exp({T('d')})->({T('e')})", f"sum({T('e')}, {V([-1])}, var<bool>:true)->({T('s')})",
+             f"exp({T('d')})->({T('e2')})", f"broadcastTo({T('s')}, {V(full)})->({T('sb')})", f"div({T('e2')}, {T('sb')})->({T('y')})",
+             f"matmul({T('y')}, {T('v')})->({T('o')})"]
+    out = lines_over_ir(setup, block, iters=iters)
+    es, n_full = 2, heads * S * S
+    # what the twelve lines move when every line is a launch of its own, and when the nine from the scaling to the division are one
+    io_b = heads * S * hd * es
+    out["bytes_line_by_line"] = (2 * io_b) + (2 * io_b + n_full * es) + 2 * n_full * es + n_full * es + n_full * es + 3 * n_full * es + 2 * n_full * es + n_full * es + 2 * n_full * es + n_full * es + 3 * n_full * es + (n_full * es + 2 * io_b)
+    out["bytes_fused"] = (2 * io_b) + (2 * io_b + n_full * es) + 8 * n_full * es + (n_full * es + 2 * io_b)
+    out["shape"] = f"[1,{heads},{S},{hd}] {dt}"
+    return out
 
 
 def config5_block_over_ir(rows=2048, hidden=896, inter=4864, only=None, iters=30, with_allocations=False):

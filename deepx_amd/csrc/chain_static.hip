@@ -196,6 +196,14 @@ using SoftmaxShortProg = SProg<SList<SIn<DT, FULL>>,
                                      SOp<DXH_CHAIN_EXP, RES + 2, 0, DT, FULL>, SOp<DXH_CHAIN_ROWSUM, RES + 3, 0, DT, COL>, SOp<DXH_CHAIN_COPY, RES + 4, 0, DT, FULL>,
                                      SOp<DXH_CHAIN_DIV, RES + 3, RES + 5, DT, FULL>>>;
 
+// attention weights as the front computes them (front/py/deepx/nn/modules/transformer/attention.py:15,24): the scores times the
+// scaling factor, then the softmax above on the product — one more line in front, a = t * scaling
+template <int DT>
+using ScaledSoftmaxProg = SProg<SList<SIn<DT, FULL>>,
+                                SList<SOp<DXH_CHAIN_MULSCALAR, 0, 0, DT, FULL>, SOp<DXH_CHAIN_ROWMAX, RES + 0, 0, DT, COL>, SOp<DXH_CHAIN_COPY, RES + 1, 0, DT, FULL>,
+                                      SOp<DXH_CHAIN_SUB, RES + 0, RES + 2, DT, FULL>, SOp<DXH_CHAIN_EXP, RES + 3, 0, DT, FULL>, SOp<DXH_CHAIN_ROWSUM, RES + 4, 0, DT, COL>,
+                                      SOp<DXH_CHAIN_EXP, RES + 3, 0, DT, FULL>, SOp<DXH_CHAIN_COPY, RES + 5, 0, DT, FULL>, SOp<DXH_CHAIN_DIV, RES + 6, RES + 7, DT, FULL>>>;
+
 // SiLU gate of the front's gated MLP (front/py/deepx/nn/functional/activite.py:11-18,
 // front/py/deepx/nn/modules/mlp/gatedmlp.py:20-26): sg = -g  sg = exp(sg)  sg += 1  sg = 1 / sg  sg = g * sg  sg *= u
 using SiluGateProg = SProg<SList<SIn<0, FULL>, SIn<0, FULL>>,
@@ -308,6 +316,9 @@ int static_rows_try(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chai
     DXH_TRY_ROWS(SoftmaxProg<kSF32>, 4);
     DXH_TRY_ROWS(SoftmaxProg<kSBF16>, 8);
     DXH_TRY_ROWS(SoftmaxProg<kSF16>, 8);
+    DXH_TRY_ROWS(ScaledSoftmaxProg<kSF32>, 4);
+    DXH_TRY_ROWS(ScaledSoftmaxProg<kSBF16>, 8);
+    DXH_TRY_ROWS(ScaledSoftmaxProg<kSF16>, 8);
     DXH_TRY_ROWS(SoftmaxShortProg<kSF32>, 4);
     DXH_TRY_ROWS(SoftmaxShortProg<kSBF16>, 8);
     DXH_TRY_ROWS(SoftmaxShortProg<kSF16>, 8);

@@ -2,6 +2,8 @@
 DEEPX_GRAPH=1, recorded into a HIP graph on the second arrival and replayed afterwards.  Every
 replay is checked bit for bit against the same lines executed one by one, with eager work and
 synchronisations between the replays."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -731,3 +733,81 @@ def test_side_streams_keep_every_hazard_in_order(tmp_path):
         for rep, got in enumerate(results[key]):
             for k in want:
                 assert np.array_equal(got[k].view(np.uint8), want[k].view(np.uint8)), (key, rep, k)
+
+
+def attention_core_lines(n, V, S, heads, hd, dt, scale, allocate=False):
+    """The core of the front's attention (front/py/deepx/nn/modules/transformer/attention.py:15-32 with normalization.py:4-17
+    for the softmax) on [1, heads, S, hd] tensors: scores = q @ k.mT, times the scaling factor, softmax over the last axis,
+    times v.  With `allocate`, every result is made by a `newtensor` line right before its op, as the front does."""
+    sc, full, col, out = [1, heads, S, S], [1, heads, S, S], [1, heads, S, 1], [1, heads, S, hd]
+    steps = [(("kT", [1, heads, hd, S]), f"transpose({n('k')}, {V([0, 1, 3, 2])})->({n('kT')})"),
+             (("sc", sc), f"matmul({n('q')}, {n('kT')})->({n('sc')})"),
+             (("a", full), f"mulscalar({n('sc')}, var<float32>:{scale})->({n('a')})"),
+             (("m", col), f"reducemax({n('a')}, {V([-1])}, var<bool>:true)->({n('m')})"),
+             (("mb", full), f"broadcastTo({n('m')}, {V(full)})->({n('mb')})"),
+             (("d", full), f"sub({n('a')}, {n('mb')})->({n('d')})"),
+             (("e", full), f"exp({n('d')})->({n('e')})"),
+             (("s", col), f"sum({n('e')}, {V([-1])}, var<bool>:true)->({n('s')})"),
+             (("e2", full), f"exp({n('d')})->({n('e2')})"),
+             (("sb", full), f"broadcastTo({n('s')}, {V(full)})->({n('sb')})"),
+             (("y", full), f"div({n('e2')}, {n('sb')})->({n('y')})"),
+             (("o", out), f"matmul({n('y')}, {n('v')})->({n('o')})")]
+    lines = []
+    for (name, shape), line in steps:
+        if allocate:
+            lines.append(f"newtensor({V(shape)})->({n(name)})")
+        lines.append(line)
+    return [name for (name, _), _ in steps], [shape for (_, shape), _ in steps], lines
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_attention_core_one_launch_for_scale_and_softmax(dxh, tmp_path, dt):
+    """q @ k.mT, the scaling, the softmax and the product with v as the front sends them, every result allocated right
+    before its op: as one datagram and line by line with runs held back, the nine lines from the scaling to the division
+    are one launch of the kernel compiled for them; every tensor has the bits of plain line-by-line execution, and the
+    output agrees with a float64 model of the same roundings."""
+    S, heads, hd = 256, 4, 64
+    scale = hd ** -0.5
+    rng = np.random.default_rng(61)
+    store = {"float32": lambda a: a, "bfloat16": H.f32_to_bf16_bits}[dt]
+    load = {"float32": lambda a: a.astype(np.float64), "bfloat16": lambda a: H.bf16_bits_to_f32(a).astype(np.float64)}[dt]
+    q, k, v = (rng.standard_normal((1, heads, S, hd)).astype(np.float32) for _ in range(3))
+    results = {}
+    for mode in ("plain", "batch", "held"):
+        ex = InProc()
+        ex.set_defer(mode == "held")
+        ex.set_fusion(mode != "plain")
+        h = Host(ex, tmp_path)
+        p = f"att_{mode}_{dt}_"
+        n = lambda name: T(p + name, dt)
+        for name, arr in (("q", q), ("k", k), ("v", v)):
+            h.put(p + name, store(arr), dt)
+        names, _, lines = attention_core_lines(n, V, S, heads, hd, dt, scale, allocate=True)
+        lines = [f"{l} // author=miaobyte id={500 + i}" for i, l in enumerate(lines)]
+        a0, b0 = C.c_int64(), C.c_int64()
+        dxh.dxh_chain_stats(C.byref(a0), C.byref(b0))
+        rs = ex.execute_batch(lines) if mode == "batch" else [ex.execute(l) for l in lines]
+        assert all(r.split(" ")[1].startswith("ok") for r in rs), rs
+        ex.flush()
+        a1, b1 = C.c_int64(), C.c_int64()
+        dxh.dxh_chain_stats(C.byref(a1), C.byref(b1))
+        if mode != "plain":
+            fs = ex.fusion_stats()
+            assert fs["runs"] == 1 and fs["lines"] == 9, fs
+            assert (a1.value - a0.value, b1.value - b0.value) == (1, 0), "the run did not take its compiled kernel"
+        results[mode] = {name: h.get(p + name) for name in names}
+    for mode in ("batch", "held"):
+        for name in results["plain"]:
+            assert np.array_equal(results[mode][name].view(np.uint8), results["plain"][name].view(np.uint8)), (mode, name)
+    # float64 model with the storage type's rounding where a tensor is stored
+    rt = (lambda a: a.astype(np.float32).astype(np.float64)) if dt == "float32" else (lambda a: H.bf16_bits_to_f32(H.f32_to_bf16_bits(a.astype(np.float32))).astype(np.float64))
+    q64, k64, v64 = (rt(x.astype(np.float64)) for x in (q, k, v))
+    a = rt(rt(q64 @ k64.transpose(0, 1, 3, 2)) * rt(np.float64(scale)))
+    d = rt(a - a.max(-1, keepdims=True))
+    e = rt(np.exp(d))
+    y = rt(e / rt(e.sum(-1, keepdims=True)))
+    o = y @ v64
+    got = load(results["plain"]["o"]).reshape(o.shape)
+    tol = 1e-4 if dt == "float32" else 3e-2
+    assert np.all(np.abs(got - o) <= tol * (np.abs(y) @ np.abs(v64)) + 1e-6), float(np.max(np.abs(got - o)))
+    assert np.allclose(load(results["plain"]["y"]).reshape(y.shape).sum(-1), 1.0, atol=1e-5 if dt == "float32" else 3e-2)

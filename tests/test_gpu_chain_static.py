@@ -117,6 +117,33 @@ def test_softmax_compiled(dxh, orc, dt, short):
         assert np.all(np.abs(y - ref) <= tol * ref + floor), (rows, cols, float(np.max(np.abs(y - ref) / (ref + floor))))
 
 
+@pytest.mark.parametrize("dt", [dx.F32, dx.BF16, dx.F16])
+def test_scaled_softmax_compiled(dxh, orc, dt):
+    """Attention weights as the front computes them (attention.py:15,24): the scores times the scaling factor, then the
+    softmax's eight lines on the product — nine lines, one compiled launch, every stored tensor with the bits of nine
+    separate launches, and the result against the formula in float64."""
+    rng = np.random.default_rng(950 + dt)
+    scale = 64 ** -0.5
+    for rows, cols in [(14 * 256, 2048), (2048, 896), (7, 8), (300, 1000), (1, 16), (515, 264)]:
+        span = 40.0 if dt == dx.F32 else 20.0
+        t = H.rand(rng, dt, rows * cols, -span, span)
+        ins = [(Dev(t), dt, FULL)]
+        shifted = [(name, l + 1 if l >= R else R + 0, r + 1 if r >= R else r, s, d, e) for name, l, r, s, d, e in softmax_prog(dt)]
+        prog = [("mulscalar", 0, 0, scale, dt, FULL)] + shifted
+        takes = dt == dx.F32 and bool(dxh.dxh_chain_rows_can_sum(rows, cols))
+        three_ways(dxh, orc, ins, prog, rows, cols, "scaled softmax", interpreter_takes_it=takes)
+        rc, got = run_rows(dxh, ins, prog, rows, cols)
+        y = H.to_float(got[-1].get(), dt).reshape(rows, cols)
+        a64 = H.to_float(got[0].get(), dt).reshape(rows, cols).astype(np.float64)  # the stored product, as the softmax sees it
+        x64 = H.to_float(t, dt).reshape(rows, cols).astype(np.float64)
+        assert np.all(np.abs(a64 - x64 * scale) <= np.abs(x64 * scale) * (2.0 ** -23 if dt == dx.F32 else 2.0 ** -8 if dt == dx.BF16 else 2.0 ** -11) + (2.0 ** -24 if dt == dx.F16 else 1e-30))  # float16 products under 6e-5 are subnormal
+        e = np.exp(a64 - a64.max(1, keepdims=True))
+        ref = e / e.sum(1, keepdims=True)
+        tol = 1e-5 if dt == dx.F32 else 2.0 ** -4 if dt == dx.BF16 else 2.0 ** -7
+        floor = 1e-7 if dt == dx.F16 else 1e-30
+        assert np.all(np.abs(y - ref) <= tol * ref + floor), (rows, cols, float(np.max(np.abs(y - ref) / (ref + floor))))
+
+
 def test_softmax_nan_and_infinities_follow_the_separate_kernels(dxh, orc):
     """reducemax is (a < b) ? b : a in the kernel's own order: where a NaN sits in a row decides whether it
     wins.  The compiled run must agree with the separate launch on every such row."""

@@ -22,7 +22,8 @@ def run(dxh, orc, dtype, A, B, batch, m, k, n):
 
 
 SHAPES = [(1, 1, 1, 1), (1, 3, 4, 5), (2, 3, 4, 5), (1, 64, 64, 64), (1, 128, 32, 128), (3, 130, 70, 150),
-          (1, 257, 129, 65), (2, 31, 200, 17), (1, 256, 896, 384)]
+          (1, 257, 129, 65), (2, 31, 200, 17), (1, 256, 896, 384),
+          (3, 320, 2048, 64)]  # attention weights x values: one tile across N, rows of A 4 KiB apart in 16-bit types
 
 
 @pytest.mark.parametrize("dtype", [dx.F32, dx.F64, dx.BF16, dx.F16])
@@ -123,11 +124,13 @@ def test_matmul_tiles_exact_on_small_integers(dxh):
     summation order: every tile must return the exact product rounded once (RNE) to bf16.  A wrong
     fragment, k-permutation or edge clamp changes an integer and fails bit-exactly."""
     rng = np.random.default_rng(77)
-    for m, k, n in [(384, 256, 520), (200, 200, 136)]:  # the second K ends in a partial K step
-        Ai, Bi = rng.integers(-4, 5, (m, k)), rng.integers(-4, 5, (k, n))
+    # the second K ends in a partial K step; the third is one tile wide with rows of A 4 KiB apart: its tiles start at K steps of their own
+    for m, k, n in [(384, 256, 520), (200, 200, 136), (704, 2048, 64)]:
+        lim = 4 if k <= 256 else 1  # |sum| <= 16*256 = 4096 or 2048: exact in fp32
+        Ai, Bi = rng.integers(-lim, lim + 1, (m, k)), rng.integers(-lim, lim + 1, (k, n))
         A = H.to_storage(Ai.astype(np.float64).reshape(-1), dx.BF16)
         B = H.to_storage(Bi.astype(np.float64).reshape(-1), dx.BF16)
-        want = (Ai @ Bi).astype(np.float64)  # |sum| <= 16*256 = 4096: exact in fp32
+        want = (Ai @ Bi).astype(np.float64)
         dA, dB, dC = Dev(A), Dev(B), Dev.empty(m * n, np.uint16)
         for tile in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15):
             dx.check(dxh.dxh_tune(TILE_KNOB, tile))

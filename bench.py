@@ -80,6 +80,8 @@ def main():
     ap.add_argument("--block-only", metavar="MODE", default="",
                     help="run only the config-5 block over deepxIR in one mode (a key of per_op.config5.mlp_block_over_deepxIR, e.g. "
                          "one_batch_fused_us), --steps passes (the program a kernel trace wraps) and print its own JSON line")
+    ap.add_argument("--attention-only", metavar="MODE", default="",
+                    help="the same for the attention core over deepxIR (a key of per_op.attention_core_over_deepxIR)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this executor path runs on ONE GPU (no sharding, no collectives); "
@@ -144,6 +146,12 @@ def main():
 
     if args.block_only:
         out = config5_block_over_ir(only=args.block_only, iters=args.steps)
+        out["device"] = name.value.decode()
+        print(json.dumps(out))
+        return
+
+    if args.attention_only:
+        out = attention_core_over_ir(only=args.attention_only, iters=args.steps)
         out["device"] = name.value.decode()
         print(json.dumps(out))
         return
@@ -812,7 +820,7 @@ def config1_chain_over_ir(side=4096):
     return lines_over_ir(setup, block)
 
 
-def attention_core_over_ir(S=2048, heads=14, hd=64, iters=20):
+def attention_core_over_ir(S=2048, heads=14, hd=64, iters=20, only=None):
     """The core of the front's attention on the activations of config 3 / config 5 (one sequence of 2048 tokens, 14 heads of 64;
     front/py/deepx/nn/modules/transformer/attention.py:15-32, softmax as normalization.py:4-17 spells it), bf16, 12 deepxIR
     lines: transpose of k, q @ k.mT, the scaling, the softmax's eight lines, the product with v.  Not a BASELINE config: the
@@ -831,7 +839,7 @@ def attention_core_over_ir(S=2048, heads=14, hd=64, iters=20):
              f"sub({T('a')}, {T('mb')})->({T('d')})", f"exp({T('d')})->({T('e')})", f"sum({T('e')}, {V([-1])}, var<bool>:true)->({T('s')})",
              f"exp({T('d')})->({T('e2')})", f"broadcastTo({T('s')}, {V(full)})->({T('sb')})", f"div({T('e2')}, {T('sb')})->({T('y')})",
              f"matmul({T('y')}, {T('v')})->({T('o')})"]
-    out = lines_over_ir(setup, block, iters=iters)
+    out = lines_over_ir(setup, block, iters=iters, only=only)
     es, n_full = 2, heads * S * S
     # what the twelve lines move when every line is a launch of its own, and when the nine from the scaling to the division are one
     io_b = heads * S * hd * es

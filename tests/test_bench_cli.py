@@ -16,5 +16,5 @@ def test_more_than_one_gpu_is_refused():
 def test_help_lists_the_profiling_modes():
     out = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--help"], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0
-    for flag in ("--matmul-only", "--chain-only", "--block-only", "--in-order-only", "--no-cpu", "--no-per-op"):
+    for flag in ("--matmul-only", "--chain-only", "--block-only", "--attention-only", "--in-order-only", "--no-cpu", "--no-per-op"):
         assert flag in out.stdout, flag

@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 from deepx_amd import lib as dx
+from tests import helpers as H
 from tests.executor_client import InProc
 from tests.test_gpu_batch import Host, T, V
 
@@ -235,3 +236,127 @@ def test_a_new_tensor_reads_as_zeros_whoever_touches_it_first(dxh, tmp_path, mod
         assert ex.side_launches() > 0
     if mode in ("batch", "held"):
         assert ex.fusion_stats()["runs"] >= 4
+
+
+def test_random_programs_with_allocations_in_every_mode(dxh, tmp_path):
+    """Random programs in which tensors come and go between the compute lines — `newtensor` under fresh names and under
+    names that exist, `deltensor`, lines that read a tensor nobody has written yet, lines that fail on one — on pool
+    blocks full of sevens.  Reference: storage from the driver, zero fill at allocation, one line at a time, no fusion.
+    Against it, with pooled storage and the fill owed: line by line, as one datagram with fused runs, with runs held back,
+    on side streams (one datagram and line by line), and as a datagram sent three times with graphs on.  Same replies,
+    same bits in every tensor that is left."""
+    L = dxh
+    rng = np.random.default_rng(20261)
+    code = {"float32": dx.F32, "bfloat16": dx.BF16}
+    modes = ("reference", "lines", "batch", "held", "streams", "streams_lines", "graph")
+    fused = held = side = hits = 0
+    for trial in range(40):
+        rows, cols = [(16, 64), (64, 896), (33, 260), (128, 32), (5, 1000)][trial % 5]
+        shapes = {"F": [rows, cols], "C": [rows, 1]}
+        inputs = [(f"rp{trial}_in{i}_{dt[:2]}", "F", dt) for i in range(2) for dt in code]
+        data = {name: (rng.uniform(-1, 1, shapes[k]).astype(np.float32) if dt == "float32"
+                       else H.to_storage(rng.uniform(-1, 1, int(np.prod(shapes[k]))), dx.BF16).reshape(shapes[k])) for name, k, dt in inputs}
+        live = list(inputs)  # (name, kind, dtype), as the program goes
+        lines, fresh_no = [], 0
+        def some(k=None, dt=None):
+            fits = [t for t in live if (k is None or t[1] == k) and (dt is None or t[2] == dt)]
+            return fits[int(rng.integers(0, len(fits)))] if fits else None
+        for _ in range(int(rng.integers(24, 40))):
+            kind = str(rng.choice(["new", "new", "new", "del", "renew", "bin", "bin", "scalar", "scalar", "exp", "sum", "broadcast", "cast", "bad"]))
+            dt = str(rng.choice(list(code)))
+            if kind == "new":
+                k = str(rng.choice(["F", "F", "C"]))
+                name = f"rp{trial}_t{fresh_no}_{dt[:2]}"
+                fresh_no += 1
+                lines.append(f"newtensor({V(shapes[k])})->({T(name, dt)})")
+                live.append((name, k, dt))
+            elif kind == "del":
+                t = some()
+                if t and t not in inputs:
+                    lines.append(f"deltensor()->({T(t[0], t[2])})")
+                    live.remove(t)
+            elif kind == "renew":  # a name that exists: the tensor stays as it is
+                t = some()
+                lines.append(f"newtensor({V(shapes[t[1]])})->({T(t[0], t[2])})")
+            elif kind == "bin":
+                k = str(rng.choice(["F", "F", "C"]))
+                a, b, c = some(k, dt), some(k, dt), some(k, dt)
+                if a and b and c:
+                    lines.append(f"{rng.choice(['add', 'mul', 'sub', 'max'])}({T(a[0], dt)}, {T(b[0], dt)})->({T(c[0], dt)})")
+            elif kind == "scalar":
+                a = some(None, dt)
+                c = some(a[1], dt) if a else None
+                if a and c:
+                    lines.append(f"{rng.choice(['addscalar', 'mulscalar', 'maxscalar'])}({T(a[0], dt)}, var<float32>:{float(rng.choice([0.5, 2.0, -1.25]))})->({T(c[0], dt)})")
+            elif kind == "exp":
+                a = some(None, dt)
+                c = some(a[1], dt) if a else None
+                if a and c:
+                    lines.append(f"exp({T(a[0], dt)})->({T(c[0], dt)})")
+            elif kind == "sum":
+                a, c = some("F", dt), some("C", dt)
+                if a and c:
+                    lines.append(f"sum({T(a[0], dt)}, {V([-1])}, var<bool>:true)->({T(c[0], dt)})")
+            elif kind == "broadcast":
+                a, c = some("C", dt), some("F", dt)
+                if a and c:
+                    lines.append(f"broadcastTo({T(a[0], dt)}, {V(shapes['F'])})->({T(c[0], dt)})")
+            elif kind == "cast":
+                a = some()
+                d2 = str(rng.choice(list(code)))
+                c = some(a[1], d2)
+                if a and c:
+                    lines.append(f"todtype({T(a[0], a[2])})->({T(c[0], d2)})")
+            else:  # fails: a column where a full tensor is needed
+                a, b, c = some("F", dt), some("C", dt), some("F", dt)
+                if a and b and c:
+                    lines.append(f"add({T(a[0], dt)}, {T(b[0], dt)})->({T(c[0], dt)})")
+        text = [f"{line} // author=miaobyte id={700 + i}" for i, line in enumerate(lines)]
+        results, replies = {}, {}
+        for mode in modes:
+            ex = InProc()
+            ex.set_pool(mode != "reference")
+            ex.set_zero_later(mode != "reference")
+            ex.set_fusion(mode in ("batch", "held", "streams", "graph"))
+            ex.set_defer(mode == "held")
+            ex.set_streams(3 if mode.startswith("streams") else 1)
+            ex.set_graphs(mode == "graph")
+            try:
+                h = Host(ex, tmp_path)
+                if mode != "reference":
+                    for k in shapes:
+                        for dt in code:
+                            dirty_blocks(h, L, f"rp{trial}_{mode}_{k}_", shapes[k], 6, dt)
+                for name, k, dt in inputs:
+                    h.put(name, data[name], dt)
+                before = pool_stats(L)["hits"]
+                if mode in ("batch", "streams"):
+                    replies[mode] = ex.execute_batch(text)
+                elif mode == "graph":
+                    # a program with allocations is never recorded; what must hold is that asking for graphs changes nothing
+                    replies[mode] = ex.execute_batch(text)
+                else:
+                    replies[mode] = [ex.execute(t) for t in text]
+                ex.flush()
+                hits += pool_stats(L)["hits"] - before
+                fused += ex.fusion_stats()["lines"] if mode == "batch" else 0
+                held += ex.defer_stats()["held_lines"] if mode == "held" else 0
+                side += ex.side_launches() if mode.startswith("streams") else 0
+                results[mode] = {name: h.get(name) for name, _, _ in live}
+                for name, _, dt in live:
+                    if (name, _, dt) not in inputs:
+                        h.run(f"deltensor()->({T(name, dt)})")
+            finally:
+                ex.set_pool(True)
+            del ex
+        want = [r.split("//")[0] for r in replies["reference"]]
+        for mode in modes[1:]:
+            assert [r.split("//")[0] for r in replies[mode]] == want, (trial, mode, lines)
+            for name, _, dt in live:
+                a, b = results["reference"][name], results[mode][name]
+                same = np.array_equal(a.view(np.uint8), b.view(np.uint8))
+                if not same:
+                    same = np.array_equal(H.to_float(a.reshape(-1), code[dt]), H.to_float(b.reshape(-1), code[dt]), equal_nan=True)
+                assert same, (trial, mode, name, lines)
+    assert hits > 500, "the pooled modes did not get their blocks from the pool"
+    assert fused > 100 and held > 100 and side > 100, (fused, held, side)

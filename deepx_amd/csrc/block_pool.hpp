@@ -9,8 +9,9 @@
 // Plain host C++ over two function pointers, so the bookkeeping runs on the CPU without a device.
 // What the pool does NOT know is which launches still use a block when it is freed: a block is handed out again
 // at once, and whoever gets it must make its first use wait for the launches made before the free.  A first use on
-// the NULL stream does (that stream waits for every blocking stream of the device), and the executor's allocations
-// all start there: `newtensor` zero-fills on it, `load` copies on it.
+// the NULL stream does (that stream waits for every blocking stream of the device); so does one on the stream that
+// ran those launches.  The executor launches on the NULL stream unless it was told to spread lines over side streams,
+// and then a `deltensor` line first makes every stream wait for what the others were given before it.
 #pragma once
 #include <cstddef>
 #include <cstdint>

@@ -29,8 +29,9 @@ inline void dxh_check(int code, const char *what) { if (code != DXH_OK) throw Dx
 
 // Whether new tensors take their storage from the library's pool of freed blocks (default) or from the driver each time,
 // as the reference does (DEEPX_POOL=0).  A pooled block can still be in use by launches made before it was freed, so
-// whoever constructs a Tensor must touch it first on the NULL stream, which waits for them: `newtensor` zero-fills
-// there, `load` copies there.
+// the first launch on a new Tensor must be ordered behind them.  It is: everything runs on the NULL stream (replayed
+// graphs on a blocking stream, which the NULL stream waits for) unless lines are spread over side streams, and there the
+// `deltensor` that frees a block is a line for the default stream, before which the executor joins all streams.
 inline bool &tensor_pool_enabled() {
     static bool on = [] { const char *e = std::getenv("DEEPX_POOL"); return !(e && !std::strcmp(e, "0")); }();
     return on;

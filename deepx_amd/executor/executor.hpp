@@ -108,7 +108,7 @@ public:
         if (held_items_.empty()) return;
         std::vector<Item> items;
         items.swap(held_items_);
-        held_tfs_.clear();
+        held_run_.reset();
         ++stats.flushes;
         for (const std::string &reply : run_items(items, "", false, items[0].resp.recv_at))
             if (reply.find(" ok") == std::string::npos) std::cerr << "held line failed: " << reply << std::endl;
@@ -157,15 +157,11 @@ public:
             // out — if it can start a run of its own
             bool hold = false;
             if ((tf->chain_kind != 0 || tf->name == "matmul") && tf->metadata.benchmark_repeat <= 1) {
-                held_tfs_.push_back(tf);
-                hold = run_prefix_length(held_tfs_, 0, mem) == held_tfs_.size();
-                if (!hold && held_tfs_.size() > 1) {
-                    held_tfs_.pop_back();
-                    flush();
-                    held_tfs_.push_back(tf);
-                    hold = run_prefix_length(held_tfs_, 0, mem) == 1;
+                hold = held_run_.extend(tf.get(), mem);
+                if (!hold && held_run_.size() > 0) {
+                    flush();  // also forgets the run
+                    hold = held_run_.extend(tf.get(), mem);
                 }
-                if (!hold) held_tfs_.pop_back();
             }
             if (hold) {
                 ++stats.held_lines;
@@ -673,7 +669,7 @@ private:
     std::vector<Side> side_;  // side streams, created on first use
     StreamPicker picker_;
     bool graph_flying_ = false;
-    std::vector<std::shared_ptr<TF>> held_tfs_;
+    HeldRun held_run_;  // what the held lines form, kept up to date as they arrive
     void *graph_stream_ = nullptr, *graph_event_ = nullptr;
     std::unordered_map<std::string, Graph> graphs_;
     static constexpr size_t kMaxRemembered = 1024;

@@ -113,6 +113,20 @@ size_t matmul_group_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t f
 // alone (1: a line that could start one).  Every such line is known to name existing tensors of matching dtype
 // and extent, so holding it back cannot hide an error it would have reported.
 size_t run_prefix_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem);
+// The same question asked one line at a time: extend() takes the line into the run that the lines before it form (as
+// one more elementwise line of a chain, or one more product on a shared left operand) and says so, or leaves the run as
+// it was and returns false.  A run that has taken n lines is what run_prefix_length would count on those n lines.
+class HeldRun {
+public:
+    HeldRun();
+    ~HeldRun();
+    void reset();
+    size_t size() const;
+    bool extend(const TF *tf, Mem &mem);
+private:
+    struct State;
+    std::unique_ptr<State> s_;
+};
 int run_matmul_group(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, size_t count, Mem &mem, std::string &error);
 
 }  // namespace deepx

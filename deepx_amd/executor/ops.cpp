@@ -580,41 +580,31 @@ struct ChainPlan {
     std::vector<dxh_chain_rows_op> row_ops;
 };
 enum { kChainTodtype = 5, kChainBroadcast = 6, kChainPowscalar = 7, kChainSum = 8 };
-// Builds the longest run starting at tfs[first].  A tensor operand is the latest result of the run
-// with that name, else an input of the run (read before the run writes anything, which is what a
-// line-by-line execution sees as long as no earlier line of the run has written it — and those are
-// taken as results).  A tensor that several lines of the run write is stored by the last of them
-// only: nothing reads memory in between.  The first line's output fixes the [rows, cols] view (cols
-// = its last dim); later tensors are that size, or a row / column vector of it.  The run ends before
-// a line that is not a chainable float op, does not fit the view, needs a ninth input, would overwrite
-// a vector that the run reads from memory (lanes of other rows or columns may not have read it yet),
-// or whose operands are missing or mismatched (the ordinary path then reports the error for that line).
-// structural: stop after the lines have been checked against each other and the tensor store (do the tensors exist,
-// do dtypes and extents agree, does the line fit the view) and return how many form a run, without asking whether
-// the library would launch it as one: what a caller needs to know before it holds a line back for a later launch.
-size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem, ChainPlan &plan, size_t max_ops = DXH_CHAIN_ROWS_MAX_OPS, bool structural = false) {
+// The lines of a run as they are taken in, one at a time: add() checks a line against the lines before it and the tensor
+// store and either takes it (true) or leaves everything as it was (false: the run ends before that line).
+struct ChainLines {
     struct Input { std::string name; const void *data; int dtype, extent; };
     struct Op { dxh_chain_rows_op op; std::string out_name; };
     std::vector<Input> inputs;
     std::vector<Op> ops;
     bool needs_rows = false, has_f64 = false;
     int64_t rows = 0, cols = 0;
-    auto is_float = [](int dtype) { return dtype == DXH_F64 || dtype == DXH_F32 || dtype == DXH_F16 || dtype == DXH_BF16; };
+    static bool is_float(int dtype) { return dtype == DXH_F64 || dtype == DXH_F32 || dtype == DXH_F16 || dtype == DXH_BF16; }
     // extent of a tensor in the run's view, or -1
-    auto extent_of = [&](const Tensor &t) {
+    int extent_of(const Tensor &t) const {
         if (t.shape.size == rows * cols) return (int)DXH_CHAIN_FULL;
         if (rows > 1 && cols > 1 && t.shape.dim() >= 1) {
             if (t.shape.size == cols && t.shape.at(-1) == cols) return (int)DXH_CHAIN_ROW;
             if (t.shape.size == rows && t.shape.at(-1) == 1) return (int)DXH_CHAIN_COLUMN;
         }
         return -1;
-    };
-    for (size_t i = first; i < tfs.size() && ops.size() < max_ops; ++i) {
-        const TF *tf = tfs[i].get();
-        if (!tf || tf->chain_kind == 0 || tf->metadata.benchmark_repeat > 1 || tf->returns.size() != 1) break;
+    }
+    bool add(const TF *tf, Mem &mem, size_t max_ops) {
+        if (ops.size() >= max_ops) return false;
+        if (!tf || tf->chain_kind == 0 || tf->metadata.benchmark_repeat > 1 || tf->returns.size() != 1) return false;
         const int kind = tf->chain_kind;
         const size_t nargs = kind == 4 || kind == kChainTodtype ? 1 : kind == kChainSum ? 3 : 2;
-        if (tf->args.size() != nargs) break;
+        if (tf->args.size() != nargs) return false;
         const Param *tensors[2] = {nullptr, nullptr};
         const Param *scalar = nullptr;
         switch (kind) {
@@ -624,11 +614,11 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
         default: tensors[0] = &tf->args[0]; break;  // unary, todtype, broadcastTo (whose second argument is the shape)
         }
         auto out = mem.findtensor(tf->returns[0].textvalue);
-        if (!out || !is_float(out->dtype()) || out->shape.size == 0) break;
+        if (!out || !is_float(out->dtype()) || out->shape.size == 0) return false;
         if (ops.empty()) {  // the view comes from the first line's output, or from its operand when it reduces rows
             auto shaper = out;
             if (kind == kChainSum) shaper = mem.findtensor(tf->args[0].textvalue);
-            if (!shaper || shaper->shape.size == 0) break;
+            if (!shaper || shaper->shape.size == 0) return false;
             cols = shaper->shape.dim() >= 1 ? shaper->shape.at(-1) : 1;
             rows = shaper->shape.size / std::max<int64_t>(cols, 1);
         }
@@ -641,25 +631,25 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
         if (kind == kChainSum) {
             // the sum / max / min of every row of a [rows, cols] tensor; whether the row stage of the separate
             // reduction is one the fused kernels can stand in for is asked of the library once the run is known
-            if (rows < 2 || out->shape.size != rows) break;
+            if (rows < 2 || out->shape.size != rows) return false;
             auto in = mem.findtensor(tf->args[0].textvalue);
-            if (!in || in->shape.dim() < 1 || in->shape.at(-1) != cols || in->shape.size != rows * cols) break;
+            if (!in || in->shape.dim() < 1 || in->shape.at(-1) != cols || in->shape.size != rows * cols) return false;
             try {
-                if (checked_dims(in->shape.shape, ints_of(tf->args[1], mem)) != std::vector<int>{in->shape.dim() - 1}) break;
+                if (checked_dims(in->shape.shape, ints_of(tf->args[1], mem)) != std::vector<int>{in->shape.dim() - 1}) return false;
                 (void)bool_of(tf->args[2]);
-            } catch (const std::exception &) { break; }
+            } catch (const std::exception &) { return false; }
             op.op.extent = DXH_CHAIN_COLUMN;
         }
-        if (op.op.extent < 0) break;
+        if (op.op.extent < 0) return false;
         bool line_needs_rows = op.op.extent != DXH_CHAIN_FULL || kind >= kChainTodtype || (!ops.empty() && out->dtype() != ops[0].op.dtype);
         if (scalar) {
-            try { op.op.scalar = scalar_of(*scalar, mem); } catch (const std::exception &) { break; }
+            try { op.op.scalar = scalar_of(*scalar, mem); } catch (const std::exception &) { return false; }
         }
-        if (kind == kChainPowscalar && (op.op.scalar.f != 2.0 || out->dtype() != DXH_F32)) break;  // only the square has a chain code
+        if (kind == kChainPowscalar && (op.op.scalar.f != 2.0 || out->dtype() != DXH_F32)) return false;  // only the square has a chain code
         if (kind == kChainBroadcast) {
             std::vector<int> ns;
-            try { ns = ints_of(tf->args[1], mem); } catch (const std::exception &) { break; }
-            if (ns != out->shape.shape || op.op.extent != DXH_CHAIN_FULL) break;
+            try { ns = ints_of(tf->args[1], mem); } catch (const std::exception &) { return false; }
+            if (ns != out->shape.shape || op.op.extent != DXH_CHAIN_FULL) return false;
         }
         std::vector<Input> new_inputs;
         bool ok = true;
@@ -697,19 +687,43 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
             }
             (side == 0 ? op.op.lhs : op.op.rhs) = ref;
         }
-        if (!ok) break;
+        if (!ok) return false;
         // this line's output is a vector that the run (this line included) reads from memory
         bool overwrites_vector_input = false;
         for (const Input &in : inputs) overwrites_vector_input |= in.extent != DXH_CHAIN_FULL && in.name == op.out_name;
         for (const Input &in : new_inputs) overwrites_vector_input |= in.extent != DXH_CHAIN_FULL && in.name == op.out_name;
-        if (overwrites_vector_input) break;
+        if (overwrites_vector_input) return false;
         const bool line_f64 = out->dtype() == DXH_F64;
-        if ((needs_rows || line_needs_rows) && (has_f64 || line_f64)) break;  // the row form has no fp64
+        if ((needs_rows || line_needs_rows) && (has_f64 || line_f64)) return false;  // the row form has no fp64
         needs_rows = needs_rows || line_needs_rows;
         has_f64 = has_f64 || line_f64;
         inputs.insert(inputs.end(), new_inputs.begin(), new_inputs.end());
         ops.push_back(op);
+        return true;
     }
+};
+// Builds the longest run starting at tfs[first].  A tensor operand is the latest result of the run
+// with that name, else an input of the run (read before the run writes anything, which is what a
+// line-by-line execution sees as long as no earlier line of the run has written it — and those are
+// taken as results).  A tensor that several lines of the run write is stored by the last of them
+// only: nothing reads memory in between.  The first line's output fixes the [rows, cols] view (cols
+// = its last dim); later tensors are that size, or a row / column vector of it.  The run ends before
+// a line that is not a chainable float op, does not fit the view, needs a ninth input, would overwrite
+// a vector that the run reads from memory (lanes of other rows or columns may not have read it yet),
+// or whose operands are missing or mismatched (the ordinary path then reports the error for that line).
+// structural: stop after the lines have been checked against each other and the tensor store (do the tensors exist,
+// do dtypes and extents agree, does the line fit the view) and return how many form a run, without asking whether
+// the library would launch it as one: what a caller needs to know before it holds a line back for a later launch.
+size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem, ChainPlan &plan, size_t max_ops = DXH_CHAIN_ROWS_MAX_OPS, bool structural = false) {
+    ChainLines run;
+    for (size_t i = first; i < tfs.size(); ++i)
+        if (!run.add(tfs[i].get(), mem, max_ops)) break;
+    using Input = ChainLines::Input;
+    using Op = ChainLines::Op;
+    const std::vector<Input> &inputs = run.inputs;
+    std::vector<Op> &ops = run.ops;
+    const bool needs_rows = run.needs_rows;
+    const int64_t rows = run.rows, cols = run.cols;
     const size_t count = ops.size();
     if (count < 2 || structural) return count;
     if (!needs_rows && count > DXH_CHAIN_MAX_OPS) {  // the one-dtype form takes fewer ops
@@ -768,32 +782,63 @@ size_t plan_chain(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem
 // dxh_matmul_shared_a, which launches them together where its kernels allow.  Anything that a single
 // line would refuse ends the run before it, so that line reports its own error.
 namespace {
-struct MatmulGroup { std::shared_ptr<Tensor> a; std::vector<std::shared_ptr<Tensor>> bs, cs; };
-size_t plan_matmul_group(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem, MatmulGroup &g) {
+// add() takes one more `matmul` line into the run (true) or leaves the run as it was (false: it ends before that line)
+struct MatmulGroup {
+    std::shared_ptr<Tensor> a;
+    std::vector<std::shared_ptr<Tensor>> bs, cs;
     std::vector<std::string> reads, writes;
-    for (size_t i = first; i < tfs.size(); ++i) {
-        const TF *tf = tfs[i].get();
-        if (!tf || tf->name != "matmul" || tf->metadata.benchmark_repeat > 1 || tf->args.size() != 2 || tf->returns.size() != 1) break;
+    bool add(const TF *tf, Mem &mem) {
+        if (!tf || tf->name != "matmul" || tf->metadata.benchmark_repeat > 1 || tf->args.size() != 2 || tf->returns.size() != 1) return false;
         auto A = mem.findtensor(tf->args[0].textvalue), B = mem.findtensor(tf->args[1].textvalue), C = mem.findtensor(tf->returns[0].textvalue);
-        if (!A || !B || !C || A->shape.dim() != 2 || B->shape.dim() != 2) break;
-        if (A->dtype() != DXH_BF16 && A->dtype() != DXH_F16) break;
-        if (B->dtype() != A->dtype() || C->dtype() != A->dtype()) break;
-        if (A->shape.at(-1) != B->shape.at(-2) || C->shape.shape != std::vector<int>{A->shape.at(-2), B->shape.at(-1)}) break;
-        if (g.a && (tf->args[0].textvalue != reads[0] || B->shape.shape != g.bs[0]->shape.shape)) break;
+        if (!A || !B || !C || A->shape.dim() != 2 || B->shape.dim() != 2) return false;
+        if (A->dtype() != DXH_BF16 && A->dtype() != DXH_F16) return false;
+        if (B->dtype() != A->dtype() || C->dtype() != A->dtype()) return false;
+        if (A->shape.at(-1) != B->shape.at(-2) || C->shape.shape != std::vector<int>{A->shape.at(-2), B->shape.at(-1)}) return false;
+        if (a && (tf->args[0].textvalue != reads[0] || B->shape.shape != bs[0]->shape.shape)) return false;
         const std::string &out = tf->returns[0].textvalue;
         bool clash = out == tf->args[0].textvalue || out == tf->args[1].textvalue;
         for (const std::string &r : reads) clash = clash || r == out;     // an earlier line of the run reads what this one writes
         for (const std::string &w : writes) clash = clash || w == out || w == tf->args[1].textvalue;  // written twice, or read after it was written
-        if (clash) break;
-        if (!g.a) { g.a = A; reads.push_back(tf->args[0].textvalue); }
+        if (clash) return false;
+        if (!a) { a = A; reads.push_back(tf->args[0].textvalue); }
         reads.push_back(tf->args[1].textvalue);
         writes.push_back(out);
-        g.bs.push_back(B);
-        g.cs.push_back(C);
+        bs.push_back(B);
+        cs.push_back(C);
+        return true;
     }
+};
+size_t plan_matmul_group(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem, MatmulGroup &g) {
+    for (size_t i = first; i < tfs.size(); ++i)
+        if (!g.add(tfs[i].get(), mem)) break;
     return g.cs.size();
 }
 }  // namespace
+
+// ---- a run taken in line by line ----------------------------------------------------------------------
+// What run_prefix_length answers for a whole list, kept up to date one line at a time: a caller that holds lines back
+// asks for every new line whether it extends what is held, and would otherwise go over all held lines again each time.
+struct HeldRun::State {
+    ChainLines chain;
+    MatmulGroup products;
+    bool chain_alive = true, products_alive = true;
+    size_t lines = 0;
+};
+HeldRun::HeldRun() : s_(new State) {}
+HeldRun::~HeldRun() = default;
+void HeldRun::reset() { s_.reset(new State); }
+size_t HeldRun::size() const { return s_->lines; }
+bool HeldRun::extend(const TF *tf, Mem &mem) {
+    // either form may take the line; a form that refused one is out for the rest of the run (add() leaves a refused
+    // line's form untouched, so "refused" must be remembered here)
+    const bool c = s_->chain_alive && s_->chain.add(tf, mem, DXH_CHAIN_ROWS_MAX_OPS);
+    const bool p = s_->products_alive && s_->products.add(tf, mem);
+    if (!c && !p) return false;  // both forms as they were (a line is an elementwise op or a product, never both)
+    s_->chain_alive = c;
+    s_->products_alive = p;
+    ++s_->lines;
+    return true;
+}
 
 size_t matmul_group_length(const std::vector<std::shared_ptr<TF>> &tfs, size_t first, Mem &mem) {
     MatmulGroup g;

@@ -18,8 +18,15 @@ Tuning &tuning() {
 
 namespace {
 
-int raw_alloc(void **p, size_t bytes) { return (int)hipMalloc(p, bytes); }
-int raw_free(void *p) { return (int)hipFree(p); }
+// A HIP call that fails leaves its code behind as the runtime's "last error" as well, where the next launch would find
+// it and report it a second time as its own (the launchers ask hipGetLastError after every launch).  What is returned
+// to the caller here is taken off there.
+int reported(hipError_t e) {
+    if (e != hipSuccess) (void)hipGetLastError();
+    return (int)e;
+}
+int raw_alloc(void **p, size_t bytes) { return reported(hipMalloc(p, bytes)); }
+int raw_free(void *p) { return reported(hipFree(p)); }
 
 // One pool per device, made on first use and never destroyed: at process exit the runtime may be gone before a
 // static destructor could hand the blocks back, and the driver reclaims them anyway.
@@ -96,21 +103,21 @@ int dxh_device_count(int *count) {
     if (!count) return DXH_ERR_ARG;
     hipError_t e = hipGetDeviceCount(count);
     if (e != hipSuccess) { *count = 0; (void)hipGetLastError(); }
-    return (int)e;
+    return reported(e);
 }
 int dxh_set_device(int device) {
     hipError_t e = hipSetDevice(device);
     if (e == hipSuccess) { dxh::reduce_device_init(); dxh::chain_device_init(); }
-    return (int)e;
+    return reported(e);
 }
 int dxh_device_name(char *buf, size_t buflen) {
     if (!buf || buflen == 0) return DXH_ERR_ARG;
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return (int)e;
+    if (e != hipSuccess) return reported(e);
     hipDeviceProp_t prop;
     e = hipGetDeviceProperties(&prop, dev);
-    if (e != hipSuccess) return (int)e;
+    if (e != hipSuccess) return reported(e);
     snprintf(buf, buflen, "%s %s cus=%d clock_khz=%d", prop.name, prop.gcnArchName, prop.multiProcessorCount, prop.clockRate);
     return DXH_OK;
 }
@@ -125,9 +132,9 @@ int dxh_malloc(void **ptr, size_t bytes) {
         BlockPool *pool = pool_of_current_device(false);
         if (pool && pool->trim(0) > 0) e = hipMalloc(ptr, bytes);
     }
-    return (int)e;
+    return reported(e);
 }
-int dxh_free(void *ptr) { return ptr ? (int)hipFree(ptr) : DXH_OK; }
+int dxh_free(void *ptr) { return ptr ? reported(hipFree(ptr)) : DXH_OK; }
 
 int dxh_pool_alloc(void **ptr, size_t bytes) {
     if (!ptr) return DXH_ERR_ARG;
@@ -170,20 +177,20 @@ int dxh_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream) {
     if (bytes == 0) return DXH_OK;
     if (!dst || !src) return DXH_ERR_ARG;
     hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream));
-    if (e != hipSuccess) return (int)e;
-    return (int)hipStreamSynchronize(as_stream(stream));  // pageable source must stay valid
+    if (e != hipSuccess) return reported(e);
+    return reported(hipStreamSynchronize(as_stream(stream)));  // pageable source must stay valid
 }
 int dxh_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream) {
     if (bytes == 0) return DXH_OK;
     if (!dst || !src) return DXH_ERR_ARG;
     hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_stream(stream));
-    if (e != hipSuccess) return (int)e;
-    return (int)hipStreamSynchronize(as_stream(stream));
+    if (e != hipSuccess) return reported(e);
+    return reported(hipStreamSynchronize(as_stream(stream)));
 }
 int dxh_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream) {
     if (bytes == 0) return DXH_OK;
     if (!dst || !src) return DXH_ERR_ARG;
-    return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream));
+    return reported(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
 }
 
 int dxh_stream_create(void **stream) {
@@ -191,39 +198,39 @@ int dxh_stream_create(void **stream) {
     hipStream_t s = nullptr;
     hipError_t e = hipStreamCreate(&s);  // default priority only
     *stream = (void *)s;
-    return (int)e;
+    return reported(e);
 }
 int dxh_stream_destroy(void *stream) {
     if (!stream) return DXH_OK;
     dxh::reduce_stream_release(as_stream(stream));
-    return (int)hipStreamDestroy(as_stream(stream));
+    return reported(hipStreamDestroy(as_stream(stream)));
 }
-int dxh_stream_sync(void *stream) { return (int)hipStreamSynchronize(as_stream(stream)); }
-int dxh_device_sync(void) { return (int)hipDeviceSynchronize(); }
+int dxh_stream_sync(void *stream) { return reported(hipStreamSynchronize(as_stream(stream))); }
+int dxh_device_sync(void) { return reported(hipDeviceSynchronize()); }
 
 int dxh_event_create(void **event) {
     if (!event) return DXH_ERR_ARG;
     hipEvent_t ev = nullptr;
     hipError_t e = hipEventCreate(&ev);
     *event = (void *)ev;
-    return (int)e;
+    return reported(e);
 }
-int dxh_event_destroy(void *event) { return event ? (int)hipEventDestroy((hipEvent_t)event) : DXH_OK; }
+int dxh_event_destroy(void *event) { return event ? reported(hipEventDestroy((hipEvent_t)event)) : DXH_OK; }
 int dxh_event_record(void *event, void *stream) {
     if (!event) return DXH_ERR_ARG;
-    return (int)hipEventRecord((hipEvent_t)event, as_stream(stream));
+    return reported(hipEventRecord((hipEvent_t)event, as_stream(stream)));
 }
 int dxh_stream_wait_event(void *stream, void *event) {
     if (!event) return DXH_ERR_ARG;
-    return (int)hipStreamWaitEvent(as_stream(stream), (hipEvent_t)event, 0);
+    return reported(hipStreamWaitEvent(as_stream(stream), (hipEvent_t)event, 0));
 }
 int dxh_event_sync(void *event) {
     if (!event) return DXH_ERR_ARG;
-    return (int)hipEventSynchronize((hipEvent_t)event);
+    return reported(hipEventSynchronize((hipEvent_t)event));
 }
 int dxh_event_elapsed_ms(void *start, void *stop, float *ms) {
     if (!start || !stop || !ms) return DXH_ERR_ARG;
-    return (int)hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop);
+    return reported(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
 }
 
 static_assert(sizeof(hipIpcMemHandle_t) == DXH_IPC_HANDLE_BYTES, "handle size is part of the ABI");
@@ -231,7 +238,7 @@ int dxh_ipc_export(const void *ptr, void *handle) {
     if (!ptr || !handle) return DXH_ERR_ARG;
     hipIpcMemHandle_t h;
     hipError_t e = hipIpcGetMemHandle(&h, const_cast<void *>(ptr));
-    if (e != hipSuccess) return (int)e;
+    if (e != hipSuccess) return reported(e);
     std::memcpy(handle, &h, sizeof h);
     return DXH_OK;
 }
@@ -240,13 +247,13 @@ int dxh_ipc_open(const void *handle, void **ptr) {
     *ptr = nullptr;
     hipIpcMemHandle_t h;
     std::memcpy(&h, handle, sizeof h);
-    return (int)hipIpcOpenMemHandle(ptr, h, hipIpcMemLazyEnablePeerAccess);
+    return reported(hipIpcOpenMemHandle(ptr, h, hipIpcMemLazyEnablePeerAccess));
 }
-int dxh_ipc_close(void *ptr) { return ptr ? (int)hipIpcCloseMemHandle(ptr) : DXH_OK; }
+int dxh_ipc_close(void *ptr) { return ptr ? reported(hipIpcCloseMemHandle(ptr)) : DXH_OK; }
 
 int dxh_graph_begin_capture(void *stream) {
     if (!stream) return DXH_ERR_ARG;  // the NULL stream cannot be captured
-    return (int)hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal);
+    return reported(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal));
 }
 int dxh_graph_end_capture(void *stream, void **graph_exec) {
     if (!stream || !graph_exec) return DXH_ERR_ARG;
@@ -261,7 +268,7 @@ int dxh_graph_end_capture(void *stream, void **graph_exec) {
     hipGraphExec_t exec = nullptr;
     e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
-    if (e != hipSuccess) { dxh::finish_capture_ended(as_stream(stream), nullptr); return (int)e; }
+    if (e != hipSuccess) { dxh::finish_capture_ended(as_stream(stream), nullptr); return reported(e); }
     // the in-launch counters its recorded launches took stay with the graph until dxh_graph_destroy
     dxh::finish_capture_ended(as_stream(stream), (const void *)exec);
     *graph_exec = (void *)exec;
@@ -269,13 +276,13 @@ int dxh_graph_end_capture(void *stream, void **graph_exec) {
 }
 int dxh_graph_launch(void *graph_exec, void *stream) {
     if (!graph_exec || !stream) return DXH_ERR_ARG;
-    return (int)hipGraphLaunch((hipGraphExec_t)graph_exec, as_stream(stream));
+    return reported(hipGraphLaunch((hipGraphExec_t)graph_exec, as_stream(stream)));
 }
 int dxh_graph_destroy(void *graph_exec) {
     if (!graph_exec) return DXH_OK;
     const hipError_t e = hipGraphExecDestroy((hipGraphExec_t)graph_exec);
     dxh::finish_graph_destroyed(graph_exec);
-    return (int)e;
+    return reported(e);
 }
 int dxh_graph_counter_stats(int64_t *in_use, int64_t *capacity) {
     if (!in_use || !capacity) return DXH_ERR_ARG;

@@ -57,6 +57,12 @@ class InProc:
         fn(*args, buf, len(buf))
         return buf.value.decode("utf-8")
 
+    def close(self):
+        """destroys the executor (its tensors, side streams and recorded graphs); tests that make hundreds of executors call it"""
+        if self.ex:
+            self.L.dxe_destroy(self.ex)
+            self.ex = None
+
     def execute(self, line): return self._call(self.L.dxe_execute, self.ex, line.encode())
     def execute_batch(self, lines): return self._call(self.L.dxe_execute_batch, self.ex, "\n".join(lines).encode()).split("\n")
     def set_graphs(self, on): self.L.dxe_set_graphs(self.ex, int(on))

@@ -553,9 +553,11 @@ def test_random_batches_fused_equal_line_by_line(tmp_path):
             if mode.startswith("streams"):
                 side_launches += ex.side_launches()
             results[mode] = {name: h.get(name) for name, _, _ in pool}
-            del ex
+            ex.close()
         for mode in ("fused", "held", "streams", "streams_unfused", "streams_lines"):
-            assert [r.split("//")[0] for r in replies[mode]] == [r.split("//")[0] for r in replies["lines"]], (trial, mode, lines)
+            got, want = [r.split("//")[0] for r in replies[mode]], [r.split("//")[0] for r in replies["lines"]]
+            differ = [(i, replies[mode][i], replies["lines"][i]) for i in range(min(len(got), len(want))) if got[i] != want[i]]
+            assert got == want, (trial, mode, len(got), len(want), differ[:3], lines)
             for name, _, _ in pool:
                 a, b = results["lines"][name], results[mode][name]
                 same = np.array_equal(a.view(np.uint8), b.view(np.uint8))

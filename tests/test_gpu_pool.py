@@ -348,7 +348,7 @@ def test_random_programs_with_allocations_in_every_mode(dxh, tmp_path):
                         h.run(f"deltensor()->({T(name, dt)})")
             finally:
                 ex.set_pool(True)
-            del ex
+            ex.close()
         want = [r.split("//")[0] for r in replies["reference"]]
         for mode in modes[1:]:
             assert [r.split("//")[0] for r in replies[mode]] == want, (trial, mode, lines)
@@ -360,3 +360,23 @@ def test_random_programs_with_allocations_in_every_mode(dxh, tmp_path):
                 assert same, (trial, mode, name, lines)
     assert hits > 500, "the pooled modes did not get their blocks from the pool"
     assert fused > 100 and held > 100 and side > 100, (fused, held, side)
+
+
+def test_a_failed_runtime_call_is_reported_once(dxh):
+    """A call of the C ABI that fails (here: freeing a pointer the driver never gave out) returns its code to its caller
+    and leaves nothing behind for the next launch to find: the launchers ask the runtime for its last error after every
+    launch, and would otherwise report the old failure as their own."""
+    L = dxh
+    host = np.zeros(16, np.float32)
+    rc = L.dxh_free(host.ctypes.data)
+    assert rc > 0, "freeing host memory must fail"
+    x = np.arange(1024, dtype=np.float32)
+    a, out = H.Dev(x), H.Dev.empty(1024, np.float32)
+    assert L.dxh_add(dx.F32, a.ptr, a.ptr, out.ptr, 1024, None) == 0
+    assert np.array_equal(out.get(), x + x)
+    # a product that needs no workspace, right after an allocation the driver must refuse
+    p = C.c_void_p()
+    assert L.dxh_malloc(C.byref(p), 1 << 60) > 0 and not p.value
+    assert L.dxh_pool_alloc(C.byref(p), 1 << 60) > 0 and not p.value
+    assert L.dxh_mulscalar(dx.F32, a.ptr, dx.scalar(2.0), out.ptr, 1024, None) == 0
+    assert np.array_equal(out.get(), x * 2)

@@ -18,7 +18,8 @@
  * Conventions
  *  - plain pointers and sizes, no C++ types; every entry point returns an int:
  *    0 = ok, >0 = a hipError_t value, <0 = one of the DXH_ERR_* codes below.
- *    Nothing throws across the boundary.
+ *    Nothing throws across the boundary.  A hipError_t that a call returns is reported by that call only: it is
+ *    taken off the runtime's "last error", so the next launch does not find it there and report it as its own.
  *  - all tensor pointers are DEVICE pointers to contiguous row-major storage
  *    (executor/deepxcore/src/deepx/shape.cpp:21-32); shape/axis arrays are HOST
  *    pointers and are consumed before the call returns.

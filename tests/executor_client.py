@@ -6,6 +6,7 @@ import ctypes as C
 import os
 import socket
 import subprocess
+import tempfile
 import time
 
 import numpy as np
@@ -204,7 +205,10 @@ class UdpExecutor:
         self.port = free_port()
         e = dict(os.environ, DEEPX_PORT=str(self.port))
         e.update(env or {})
-        self.proc = subprocess.Popen([BIN], env=e, stdout=subprocess.PIPE, stderr=subprocess.PIPE)
+        # what the server prints goes to a file, not a pipe: nobody reads a pipe here, and a server that has printed
+        # a pipe's worth of messages (one per line that fails) would block in its next write
+        self.log = tempfile.TemporaryFile()
+        self.proc = subprocess.Popen([BIN], env=e, stdout=self.log, stderr=subprocess.STDOUT)
         self.sock = socket.socket(socket.AF_INET, socket.SOCK_DGRAM)
         self.sock.settimeout(60)
         self._id = 0
@@ -217,7 +221,8 @@ class UdpExecutor:
                 break
             except socket.timeout:
                 if self.proc.poll() is not None or time.time() > deadline:
-                    raise RuntimeError("executor did not start: " + self.proc.stderr.read().decode())
+                    self.log.seek(0)
+                    raise RuntimeError("executor did not start: " + self.log.read().decode(errors="replace"))
         self.sock.settimeout(60)
 
     def raw(self, text, nreplies=1):
@@ -251,6 +256,7 @@ class UdpExecutor:
         except Exception:
             self.proc.kill()
         self.sock.close()
+        self.log.close()
 
 
 # ---- deepx tensor files (the format of front/py/deepxutil/numpy/io.py and shape.cpp:93-101) ------

@@ -86,6 +86,17 @@ def same_bits(a, b):
     return np.array_equal(a.get().view(np.uint8), b.get().view(np.uint8))
 
 
+def same_bits_nans_aside(a, b, dtype):
+    """the same bits wherever the result is a number, and NaN in the same places: which NaN an op returns (sign, payload) is
+    the compiler's choice per kernel — sqrt of a negative float16 comes back as 0x7e00 from one kernel and 0xfe00 from another"""
+    x, y = a.get(), b.get()
+    if np.array_equal(x.view(np.uint8), y.view(np.uint8)):
+        return True
+    fx, fy = H.to_float(x, dtype), H.to_float(y, dtype)
+    nan = np.isnan(fx)
+    return bool(nan.any()) and np.array_equal(nan, np.isnan(fy)) and np.array_equal(x[~nan], y[~nan])
+
+
 @pytest.mark.parametrize("dtype", [dx.F32, dx.BF16, dx.F16, dx.F64])
 def test_config1_chain_in_one_launch(dxh, orc, dtype):
     """The 8-op elementwise chain of BASELINE config 1 (abs composed from mulscalar and max) and
@@ -128,7 +139,7 @@ def test_random_runs_match_separate_calls(dxh, orc, dtype):
         dx.check(rc, "chain")
         check_against_oracle(orc, dtype, inputs, prog, got, n, ("random run", trial, n))
         for k, (g, w) in enumerate(zip(got, want)):
-            assert same_bits(g, w), (dtype, trial, n, prog, k)
+            assert same_bits_nans_aside(g, w, dtype), (dtype, trial, n, prog, k)
 
 
 def test_in_place_and_argument_checks(dxh):

@@ -138,7 +138,7 @@ DXE_API size_t dxe_data_write(const char *path, const char *data, size_t bytes, 
 }
 DXE_API size_t dxe_data_read(const char *path, char *data, size_t bytes, char *out, size_t buflen) {
     try {
-        const std::vector<char> got = read_exact(path ? path : "", bytes);
+        const HostBytes got = read_exact(path ? path : "", bytes);
         if (bytes) std::memcpy(data, got.data(), bytes);
         return copy_out("", out, buflen);
     } catch (const std::exception &e) { return copy_out(std::string("error: ") + e.what(), out, buflen); }

@@ -26,8 +26,21 @@ inline std::string file_stem(const std::string &path) {
     return dot == std::string::npos ? name : name.substr(0, dot);
 }
 
-inline std::vector<char> to_host(const Tensor &t) {
-    std::vector<char> host((size_t)t.shape.bytes());
+// A host buffer that is about to be overwritten whole (by a file or by a copy from the device): a std::vector would
+// clear it first, one more pass over every byte of a tensor.
+class HostBytes {
+public:
+    explicit HostBytes(size_t n) : p_(n ? new char[n] : nullptr), n_(n) {}
+    char *data() { return p_.get(); }
+    const char *data() const { return p_.get(); }
+    size_t size() const { return n_; }
+private:
+    std::unique_ptr<char[]> p_;
+    size_t n_;
+};
+
+inline HostBytes to_host(const Tensor &t) {
+    HostBytes host((size_t)t.shape.bytes());
     dxh_check(dxh_memcpy_d2h(host.data(), t.data, host.size(), nullptr), "copy to host");
     return host;
 }
@@ -43,19 +56,19 @@ inline void write_exact(const std::string &path, const char *data, size_t bytes)
 inline void save_tensor(const Tensor &t, const std::string &path) {
     const std::string yaml = t.shape.to_yaml();
     write_exact(path + ".shape", yaml.data(), yaml.size());
-    std::vector<char> host = to_host(t);
+    const HostBytes host = to_host(t);
     write_exact(path + ".data", host.data(), host.size());
 }
 
 // a file that must hold exactly `want` bytes (stdutil/fs.cpp:31-50)
-inline std::vector<char> read_exact(const std::string &path, size_t want) {
+inline HostBytes read_exact(const std::string &path, size_t want) {
     std::ifstream fs(path, std::ios::binary);
     if (!fs.is_open()) throw std::runtime_error("Failed to open file: " + path);
     fs.seekg(0, std::ios::end);
     size_t size = (size_t)fs.tellg();
     fs.seekg(0, std::ios::beg);
     if (size != want) throw std::runtime_error("file size mismatch: " + path);
-    std::vector<char> buf(size);
+    HostBytes buf(size);
     fs.read(buf.data(), (std::streamsize)size);
     if (fs.fail()) throw std::runtime_error("Failed to read file: " + path);
     return buf;
@@ -65,7 +78,7 @@ inline void load_tensor_data(const std::string &path, Tensor &t) {
     // accept both "<path>" and "<path>.data" like the two reference loaders do between them
     std::string file = path;
     if (file.size() < 5 || file.substr(file.size() - 5) != ".data") file += ".data";
-    std::vector<char> buf = read_exact(file, (size_t)t.shape.bytes());
+    const HostBytes buf = read_exact(file, (size_t)t.shape.bytes());
     dxh_check(dxh_memcpy_h2d(t.data, buf.data(), buf.size(), nullptr), "copy to device");
 }
 
@@ -157,7 +170,7 @@ inline void print_tensor(const Tensor &t, std::string fmt, std::ostream &os) {
         }
         fmt = ll;
     }
-    std::vector<char> host = to_host(t);
+    const HostBytes host = to_host(t);
     const Shape &s = t.shape;
     os << "shape:[";
     for (int i = 0; i < s.dim(); ++i) os << s.shape[i] << (i + 1 < s.dim() ? ", " : "");

@@ -380,3 +380,35 @@ def test_a_failed_runtime_call_is_reported_once(dxh):
     assert L.dxh_pool_alloc(C.byref(p), 1 << 60) > 0 and not p.value
     assert L.dxh_mulscalar(dx.F32, a.ptr, dx.scalar(2.0), out.ptr, 1024, None) == 0
     assert np.array_equal(out.get(), x * 2)
+
+
+def test_kept_blocks_give_way_when_the_driver_is_out_of_memory(dxh):
+    """With a third of the free device memory kept in the pool, an allocation of seven tenths of it cannot be served
+    beside them: the pool gives its blocks back and the allocation succeeds, through dxh_pool_alloc and through
+    dxh_malloc alike.  (Nothing is touched: the blocks are address space and page tables only.)"""
+    import torch
+    L = dxh
+    assert L.dxh_pool_trim(0, None) == 0
+    free_b, total_b = torch.cuda.mem_get_info()
+    small, large = int(free_b * 0.35), int(free_b * 0.7)
+    assert small < total_b // 2, "the kept block must fit under the pool's limit (half the device)"
+    try:
+        assert L.dxh_pool_limit(total_b // 2) == 0
+        for via_pool in (True, False):
+            kept = pool_alloc(L, small)
+            assert L.dxh_pool_free(kept) == 0
+            before = pool_stats(L)
+            assert before["kept_blocks"] == 1 and before["kept_bytes"] >= small
+            p = C.c_void_p()
+            rc = L.dxh_pool_alloc(C.byref(p), large) if via_pool else L.dxh_malloc(C.byref(p), large)
+            assert rc == 0 and p.value, f"allocation failed with the pool in the way ({rc})"
+            after = pool_stats(L)
+            assert after["kept_blocks"] == 0 and after["released"] == before["released"] + 1
+            assert (L.dxh_pool_free(p) if via_pool else L.dxh_free(p)) == 0
+            assert L.dxh_pool_trim(0, None) == 0
+        # and with nothing to give back the driver's own answer comes through, once
+        p = C.c_void_p()
+        assert L.dxh_pool_alloc(C.byref(p), total_b * 2) > 0 and not p.value
+    finally:
+        assert L.dxh_pool_limit(64 << 30) == 0
+        assert L.dxh_pool_trim(0, None) == 0

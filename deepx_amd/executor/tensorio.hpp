@@ -11,6 +11,10 @@
 #include <cctype>
 #include <cstdio>
 #include <cstring>
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
 #include <fstream>
 #include <memory>
 #include <ostream>
@@ -56,6 +60,24 @@ inline void write_exact(const std::string &path, const char *data, size_t bytes)
 inline void save_tensor(const Tensor &t, const std::string &path) {
     const std::string yaml = t.shape.to_yaml();
     write_exact(path + ".shape", yaml.data(), yaml.size());
+    const size_t bytes = (size_t)t.shape.bytes();
+    // A large tensor is copied from the device straight into the file's pages (a shared mapping of the file at its
+    // final size) instead of into a buffer that is then written out: one pass over the bytes less (256 MiB: 40-95 ms
+    // against 100-130; under 32 MiB the page faults of a fresh mapping cost more than the pass they save).
+    if (bytes >= ((size_t)32 << 20)) {
+        const std::string file = path + ".data";
+        const int fd = ::open(file.c_str(), O_RDWR | O_CREAT | O_TRUNC, 0644);
+        if (fd < 0) throw std::runtime_error("Failed to open file for writing: " + file);
+        void *map = ::ftruncate(fd, (off_t)bytes) == 0 ? ::mmap(nullptr, bytes, PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0) : MAP_FAILED;
+        ::close(fd);
+        if (map != MAP_FAILED) {
+            const int rc = dxh_memcpy_d2h(map, t.data, bytes, nullptr);
+            const bool unmapped = ::munmap(map, bytes) == 0;
+            dxh_check(rc, "copy to host");
+            if (!unmapped) throw std::runtime_error("Failed to write data to file: " + file);
+            return;
+        }
+    }
     const HostBytes host = to_host(t);
     write_exact(path + ".data", host.data(), host.size());
 }
@@ -78,7 +100,26 @@ inline void load_tensor_data(const std::string &path, Tensor &t) {
     // accept both "<path>" and "<path>.data" like the two reference loaders do between them
     std::string file = path;
     if (file.size() < 5 || file.substr(file.size() - 5) != ".data") file += ".data";
-    const HostBytes buf = read_exact(file, (size_t)t.shape.bytes());
+    const size_t want = (size_t)t.shape.bytes();
+    // A large file is copied to the device straight from its pages in the page cache (a private read-only mapping):
+    // reading it into a buffer first is one more pass over every byte (256 MiB: 66 ms through a buffer, see below).
+    // Same checks and messages as read_exact.
+    if (want >= ((size_t)4 << 20)) {
+        const int fd = ::open(file.c_str(), O_RDONLY);
+        if (fd < 0) throw std::runtime_error("Failed to open file: " + file);
+        struct stat st;
+        if (::fstat(fd, &st) != 0 || (size_t)st.st_size != want) { ::close(fd); throw std::runtime_error("file size mismatch: " + file); }
+        void *map = ::mmap(nullptr, want, PROT_READ, MAP_PRIVATE, fd, 0);
+        ::close(fd);
+        if (map != MAP_FAILED) {
+            (void)::madvise(map, want, MADV_SEQUENTIAL);
+            const int rc = dxh_memcpy_h2d(t.data, map, want, nullptr);
+            ::munmap(map, want);
+            dxh_check(rc, "copy to device");
+            return;
+        }
+    }
+    const HostBytes buf = read_exact(file, want);
     dxh_check(dxh_memcpy_h2d(t.data, buf.data(), buf.size(), nullptr), "copy to device");
 }
 

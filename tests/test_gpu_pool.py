@@ -1,7 +1,9 @@
 """GPU: freed device blocks handed out again (dxh_pool_*), through the C ABI and under the executor's `newtensor` /
 `deltensor`.  The pool never waits for the device, so the cases that matter are blocks that come back while launches
-on them are still queued: whoever gets the block next must see its own data only."""
+on them are still queued: whoever gets the block next must see its own data only.  Also here: where a tensor's bytes
+come from and go to outside the device (large `.data` files through the page cache)."""
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -412,3 +414,42 @@ def test_kept_blocks_give_way_when_the_driver_is_out_of_memory(dxh):
     finally:
         assert L.dxh_pool_limit(64 << 30) == 0
         assert L.dxh_pool_trim(0, None) == 0
+
+
+def test_large_tensor_files_go_through_the_page_cache_unchanged(dxh, tmp_path):
+    """`load` of a large `.data` file copies from the file's pages and `save` of a large tensor copies into them, without
+    a buffer in between: the bytes on the device are the bytes of the file and the other way round, a file of the
+    wrong size and a missing one are refused with the messages of the buffered path, and small tensors (which keep that
+    path) sit beside them."""
+    from tests.executor_client import read_tensor, write_tensor
+    ex = InProc()
+    rng = np.random.default_rng(211)
+    try:
+        for shape, dt, npd in (([4096, 3000], "float32", np.float32), ([5000, 1000], "bfloat16", np.uint16), ([300, 7], "float32", np.float32), ([6000, 4096], "int16", np.int16)):
+            a = rng.integers(-30000, 30000, size=shape).astype(npd) if npd != np.float32 else rng.standard_normal(shape).astype(np.float32)
+            name = f"pc_{shape[0]}"
+            p = str(tmp_path / name)
+            write_tensor(p, a, dt)
+            assert ex.execute(f"load(var<string>:{p})->() // id=1").startswith("1 ok")
+            q = str(tmp_path / (name + "_back"))
+            assert ex.execute(f"save(tensor<{dt}>:{name}, var<string>:{q})->() // id=2").startswith("2 ok")
+            with open(q + ".data", "rb") as f:
+                assert f.read() == a.tobytes(), shape
+            assert np.array_equal(read_tensor(q)[0].reshape(shape), a)
+            # the same tensor overwritten on the device, saved over the old file (which is emptied first)
+            assert ex.execute(f"constant(var<float32>:3)->(tensor<{dt}>:{name}) // id=3").startswith("3 ok")
+            assert ex.execute(f"save(tensor<{dt}>:{name}, var<string>:{q})->() // id=4").startswith("4 ok")
+            assert os.path.getsize(q + ".data") == a.nbytes
+        # a large file of the wrong size, then a missing one
+        big = str(tmp_path / "pc_4096")
+        with open(big + ".data", "ab") as f:
+            f.write(b"\0" * 8)
+        r = ex.execute(f"loadtensordata(var<string>:{big})->(tensor<float32>:pc_4096) // id=5")
+        assert r.startswith("5 error") and "file size mismatch" in r, r
+        os.remove(big + ".data")
+        r = ex.execute(f"loadtensordata(var<string>:{big})->(tensor<float32>:pc_4096) // id=6")
+        assert r.startswith("6 error") and "Failed to open file" in r, r
+        r = ex.execute(f"save(tensor<float32>:pc_4096, var<string>:{tmp_path}/no/such/dir/x)->() // id=7")
+        assert r.startswith("7 error") and "Failed to open file for writing" in r, r
+    finally:
+        ex.close()

@@ -156,6 +156,47 @@ def test_exp_every_16bit_input(dxh, orc, dtype):
     assert differing <= 65536 * 0.05, differing
 
 
+def _same_nans_aside(got, want, dtype):
+    gf, wf = H.to_float(got, dtype), H.to_float(want, dtype)
+    nan = np.isnan(wf)
+    return np.array_equal(np.isnan(gf), nan) and np.array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
+
+
+@pytest.mark.parametrize("dtype", [dx.BF16, dx.F16])
+def test_every_16bit_input_through_the_unary_ops(dxh, orc, dtype):
+    """All 65,536 patterns of a 16-bit float — zeros, denormals, infinities, NaNs, negatives — through sqrt (the oracle's
+    bits, NaN for NaN) and through log, sin and cos (NaN and infinities where the oracle has them, finite results within
+    one unit in the last place; in fact all but a handful of float16 logarithms have the oracle's bits)."""
+    a = np.arange(65536, dtype=np.uint32).astype(np.uint16).view(H.NP[dtype])
+    got, want = run_unary(dxh, orc, "sqrt", dtype, a)
+    assert _same_nans_aside(got, want, dtype)
+    for name in ("log", "sin", "cos"):
+        got, want = run_unary(dxh, orc, name, dtype, a)
+        gf, wf = H.to_float(got, dtype), H.to_float(want, dtype)
+        assert np.array_equal(np.isnan(gf), np.isnan(wf)), name
+        inf = np.isinf(wf)
+        assert np.array_equal(np.isinf(gf), inf) and np.array_equal(gf[inf], wf[inf]), name
+        fin = ~np.isnan(wf) & ~inf
+        assert H.ulp_diff(got[fin], want[fin], dtype) <= 1, name
+        assert np.count_nonzero(got.view(np.uint16)[fin] != want.view(np.uint16)[fin]) <= 16, name
+
+
+@pytest.mark.parametrize("dtype", [dx.BF16, dx.F16])
+def test_every_16bit_input_through_the_binary_ops(dxh, orc, dtype):
+    """All 65,536 patterns as the left operand of add, sub, mul, div, max and min against 48 right operands (signed
+    zeros, one, a half, the largest finite value, denormals, infinities, NaN, 32 random patterns): the oracle's bits
+    everywhere a number comes out, NaN where it has NaN — 3.1 million pairs per op."""
+    rng = np.random.default_rng(5)
+    with np.errstate(over="ignore"):
+        special = H.to_storage(np.array([0.0, -0.0, 1.0, -1.0, 2.0, 0.5, 3.0, 1e-3, 65504.0, 1e-7, np.inf, -np.inf, np.nan, 1e30, -1e30, 1e-30]), dtype)
+    partners = np.concatenate([special, rng.integers(0, 65536, 32).astype(np.uint16).view(H.NP[dtype])])
+    allx = np.arange(65536, dtype=np.uint32).astype(np.uint16).view(H.NP[dtype])
+    a, b = np.repeat(allx, len(partners)), np.tile(partners, 65536)
+    for name in ("add", "sub", "mul", "div", "max", "min"):
+        got, want = run_binary(dxh, orc, name, dtype, a, b)
+        assert _same_nans_aside(got, want, dtype), name
+
+
 def test_exp_special_values(dxh, orc):
     a = np.array([0.0, -np.inf, np.inf, 1000.0, -1000.0], dtype=np.float32)
     got, _ = run_unary(dxh, orc, "exp", dx.F32, a)

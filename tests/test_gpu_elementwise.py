@@ -226,6 +226,36 @@ def test_todtype(dxh, orc, src, dst):
     assert np.array_equal(dc.get(), want), f"{dx.DTYPE_NAMES[src]}->{dx.DTYPE_NAMES[dst]}"
 
 
+@pytest.mark.parametrize("half", [dx.BF16, dx.F16])
+def test_todtype_every_16bit_input_and_every_rounding_tie(dxh, orc, half):
+    """Casts between the float types on all 65,536 patterns of a 16-bit type (to float64, float32 and both 16-bit types:
+    denormals, overflow to infinity, NaN for NaN), and from float32 into the 16-bit type on every halfway point between
+    two neighbouring 16-bit values and on its two float32 neighbours — where round-to-nearest-even is decided."""
+    allx = np.arange(65536, dtype=np.uint32).astype(np.uint16).view(H.NP[half])
+
+    def cast(src, a, dst):
+        da, dc = Dev(a), Dev.empty(a.size, H.NP[dst])
+        dx.check(dxh.dxh_todtype(src, da.ptr, dst, dc.ptr, a.size, None), "todtype")
+        want = np.empty(a.size, dtype=H.NP[dst])
+        assert orc.orc_todtype(src, hp(a), dst, hp(want), a.size) == 0
+        return dc.get(), want
+
+    for dst in (dx.F64, dx.F32, dx.F16, dx.BF16):
+        got, want = cast(half, allx, dst)
+        if dst in (dx.F16, dx.BF16):
+            assert _same_nans_aside(got, want, dst), dx.DTYPE_NAMES[dst]
+        else:
+            nan = np.isnan(want)
+            assert np.array_equal(np.isnan(got), nan) and np.array_equal(got[~nan], want[~nan]), dx.DTYPE_NAMES[dst]
+    vals = np.sort(np.unique(H.to_float(allx, half)[np.isfinite(H.to_float(allx, half))].astype(np.float64)))
+    ties = ((vals[:-1] + vals[1:]) / 2).astype(np.float32)  # one bit more than the 16-bit type holds: exact in float32
+    assert np.array_equal(ties.astype(np.float64), (vals[:-1] + vals[1:]) / 2)
+    probes = np.concatenate([ties, np.nextafter(ties, np.float32(np.inf)), np.nextafter(ties, np.float32(-np.inf)),
+                             np.array([np.inf, -np.inf, np.nan, 3.0e38, -3.0e38, 1e-45, -1e-45, 65520.0, 65519.996], dtype=np.float32)])
+    got, want = cast(dx.F32, probes, half)
+    assert _same_nans_aside(got, want, half)
+
+
 CMP = ["equal", "notequal", "less", "greater"]
 
 

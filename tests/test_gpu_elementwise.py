@@ -283,6 +283,33 @@ def test_compare(dxh, orc, name, dtype):
             assert set(np.unique(got)) <= {0, 1}
 
 
+@pytest.mark.parametrize("dtype", [dx.BF16, dx.F16])
+def test_compare_every_16bit_input(dxh, orc, dtype):
+    """All 65,536 patterns of a 16-bit float against 48 partners (signed zeros, infinities, NaN, denormals, neighbours of
+    one, random patterns) through equal / notequal with and without an epsilon and through less / greater: the oracle's
+    mask, byte for byte — NaN compares as the reference's `<=` and `<` make it compare."""
+    rng = np.random.default_rng(6)
+    with np.errstate(over="ignore"):
+        special = H.to_storage(np.array([0.0, -0.0, 1.0, -1.0, 1.0078125, 0.9921875, 0.5, 65504.0, 1e-7, -1e-7, np.inf, -np.inf, np.nan, 1e30, -1e30, 0.25]), dtype)
+    partners = np.concatenate([special, rng.integers(0, 65536, 32).astype(np.uint16).view(H.NP[dtype])])
+    allx = np.arange(65536, dtype=np.uint32).astype(np.uint16).view(H.NP[dtype])
+    a, b = np.repeat(allx, len(partners)), np.tile(partners, 65536)
+    n = a.size
+    da, db, dm = Dev(a), Dev(b), Dev.empty(n, np.uint8)
+    want = np.empty(n, dtype=np.uint8)
+    for name in CMP:
+        for eps in ([0.0, 0.25, 1e-3] if name in ("equal", "notequal") else [None]):
+            f, g = getattr(dxh, "dxh_" + name), getattr(orc, "orc_" + name)
+            if eps is None:
+                dx.check(f(dtype, da.ptr, db.ptr, dm.ptr, n, None), name)
+                assert g(dtype, hp(a), hp(b), hp(want), n) == 0
+            else:
+                dx.check(f(dtype, da.ptr, db.ptr, eps, dm.ptr, n, None), name)
+                assert g(dtype, hp(a), hp(b), eps, hp(want), n) == 0
+            got = dm.get()
+            assert np.array_equal(got, want), (name, eps, int(np.count_nonzero(got != want)))
+
+
 @pytest.mark.parametrize("name", ["equalscalar", "notequalscalar", "lessscalar", "greaterscalar"])
 @pytest.mark.parametrize("dtype", H.ALL_NUMERIC)
 def test_compare_scalar(dxh, orc, name, dtype):

@@ -197,6 +197,40 @@ def test_every_16bit_input_through_the_binary_ops(dxh, orc, dtype):
         assert _same_nans_aside(got, want, dtype), name
 
 
+@pytest.mark.parametrize("dtype", [dx.F32, dx.F64])
+def test_special_values_through_every_float_op(dxh, orc, dtype):
+    """A grid of 131 values — signed zeros, denormals and their neighbours, the largest finite value, the thresholds of exp,
+    numbers next to one, 1e±30, infinities, NaN, 64 random magnitudes over eighty decades — in all pairs through add, sub,
+    mul, div, max and min (the oracle's bits, NaN for NaN) and one by one through sqrt (exact) and exp, log, sin, cos, tan
+    (NaN and infinities where the oracle has them, 4 units in the last place elsewhere, arguments of 1e30 included)."""
+    npd = H.NP[dtype]
+    fi = np.finfo(npd)
+    base = [0.0, 1.0, 2.0, 0.5, 3.0, 1.0 / 3.0, 10.0, 1e-3, 1e3, np.pi, np.e, fi.max, fi.max / 2, fi.tiny, fi.tiny * 2, fi.tiny / 2, fi.smallest_subnormal,
+            fi.smallest_subnormal * 3, fi.eps, 1 + fi.eps, 1 - fi.eps / 2, 88.0, 89.0, 709.0, 710.0, 1e-20, 1e20, 1e-30, 1e30, 0.1, 0.7, 123456.789]
+    rng = np.random.default_rng(3)
+    with np.errstate(all="ignore"):
+        grid = np.array(base + [-x for x in base] + [np.inf, -np.inf, np.nan], dtype=npd)
+        grid = np.concatenate([grid, (rng.standard_normal(64) * 10.0 ** rng.integers(-40, 40, 64)).astype(npd)])
+
+    def exact(got, want):
+        nan = np.isnan(want)
+        return np.array_equal(np.isnan(got), nan) and np.array_equal(got[~nan].view(np.uint8), want[~nan].view(np.uint8))
+
+    a, b = np.repeat(grid, grid.size), np.tile(grid, grid.size)
+    for name in ("add", "sub", "mul", "div", "max", "min"):
+        got, want = run_binary(dxh, orc, name, dtype, a, b)
+        assert exact(got, want), name
+    got, want = run_unary(dxh, orc, "sqrt", dtype, grid)
+    assert exact(got, want)
+    for name in ("exp", "log", "sin", "cos", "tan"):
+        got, want = run_unary(dxh, orc, name, dtype, grid)
+        assert np.array_equal(np.isnan(got), np.isnan(want)), name
+        inf = np.isinf(want)
+        assert np.array_equal(np.isinf(got), inf) and np.array_equal(got[inf], want[inf]), name
+        fin = ~np.isnan(want) & ~inf
+        assert H.ulp_diff(got[fin], want[fin], dtype) <= 4, name
+
+
 def test_exp_special_values(dxh, orc):
     a = np.array([0.0, -np.inf, np.inf, 1000.0, -1000.0], dtype=np.float32)
     got, _ = run_unary(dxh, orc, "exp", dx.F32, a)

@@ -223,6 +223,11 @@ using SwishProg = SProg<SList<SIn<0, FULL>>,
                         SList<SOp<DXH_CHAIN_MULSCALAR, 0, 0, 0, FULL>, SOp<DXH_CHAIN_MULSCALAR, RES + 0, 0, 0, FULL>, SOp<DXH_CHAIN_EXP, RES + 1, 0, 0, FULL>,
                               SOp<DXH_CHAIN_ADDSCALAR, RES + 2, 0, 0, FULL>, SOp<DXH_CHAIN_RDIVSCALAR, RES + 3, 0, 0, FULL>, SOp<DXH_CHAIN_MUL, 0, RES + 4, 0, FULL>>>;
 
+// sigmoid on its own (activite.py:10-12): the first four lines of SiluProg
+using SigmoidProg = SProg<SList<SIn<0, FULL>>,
+                          SList<SOp<DXH_CHAIN_MULSCALAR, 0, 0, 0, FULL>, SOp<DXH_CHAIN_EXP, RES + 0, 0, 0, FULL>, SOp<DXH_CHAIN_ADDSCALAR, RES + 1, 0, 0, FULL>,
+                                SOp<DXH_CHAIN_RDIVSCALAR, RES + 2, 0, 0, FULL>>>;
+
 std::atomic<int64_t> g_static_launches{0}, g_interpreted_launches{0};
 
 int dtype_code(int dtype) { return dtype == DXH_F32 ? (int)kSF32 : dtype == DXH_BF16 ? (int)kSBF16 : dtype == DXH_F16 ? (int)kSF16 : -1; }
@@ -355,6 +360,7 @@ int static_chain_try(int dtype, const void *const *inputs, int n_inputs, const d
     DXH_TRY_FLAT(SiluProg);
     DXH_TRY_FLAT(SwishGateProg);
     DXH_TRY_FLAT(SwishProg);
+    DXH_TRY_FLAT(SigmoidProg);
 #undef DXH_TRY_FLAT
     if (rc == DXH_OK) g_static_launches.fetch_add(1, std::memory_order_relaxed);
     return rc;

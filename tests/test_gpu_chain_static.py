@@ -216,7 +216,7 @@ def test_silu_gate_compiled(dxh, orc, dt):
 
 
 @pytest.mark.parametrize("dt", [dx.F32, dx.BF16, dx.F16])
-@pytest.mark.parametrize("gated", [True, False])
+@pytest.mark.parametrize("gated", [True, False, "sigmoid"])
 def test_swish_as_the_front_spells_it(dxh, orc, dt, gated):
     """swish(x, beta) of the front is x * sigmoid(x * beta) with sigmoid(t) = 1 / (exp(t * -1) + 1) (activite.py:10-16):
     one more mulscalar in front of the sequence above, seven lines with the gate's `* up`.  Compiled, interpreted
@@ -225,8 +225,10 @@ def test_swish_as_the_front_spells_it(dxh, orc, dt, gated):
     for n, beta in ((2048 * 896, 1.0), (8 * 1031, 1.702)):
         x, u = Dev(H.rand(rng, dt, n, -6.0, 6.0)), Dev(H.rand(rng, dt, n, -2.0, 2.0))  # exp(6 * 1.702) still fits float16
         prog = [("mulscalar", 0, 0, beta), ("mulscalar", R + 0, 0, -1.0), ("exp", R + 1, 0, 0), ("addscalar", R + 2, 0, 1.0),
-                ("rdivscalar", R + 3, 0, 1.0), ("mul", 0, R + 4, 0)] + ([("mul", R + 5, 1, 0)] if gated else [])
-        ins = [x, u] if gated else [x]
+                ("rdivscalar", R + 3, 0, 1.0), ("mul", 0, R + 4, 0)] + ([("mul", R + 5, 1, 0)] if gated is True else [])
+        if gated == "sigmoid":  # sigmoid on its own (activite.py:10-12): 1 / (exp(t * -1) + 1), four lines
+            prog = [("mulscalar", 0, 0, -1.0), ("exp", R + 0, 0, 0), ("addscalar", R + 1, 0, 1.0), ("rdivscalar", R + 2, 0, 1.0)]
+        ins = [x, u] if gated is True else [x]
 
         def run():
             outs = [Dev.empty(n, H.NP[dt]) for _ in prog]
@@ -261,7 +263,9 @@ def test_swish_as_the_front_spells_it(dxh, orc, dt, gated):
             assert same_bits(comp[k], sep[k]) and same_bits(interp[k], sep[k]), (n, k)
         x64 = H.to_float(x.get(), dt)
         ref = x64 / (1.0 + np.exp(-x64 * H.to_float(H.to_storage(np.array([beta]), dt), dt)[0]))
-        if gated:
+        if gated == "sigmoid":
+            ref, beta = 1.0 / (1.0 + np.exp(-x64)), 1.0
+        elif gated:
             ref = ref * H.to_float(u.get(), dt)
         # the rounding of x * beta to the dtype is a relative error of the exponent: exp turns it into |x beta| times as much
         tol = 1e-5 if dt == dx.F32 else 2.0 ** -5 if dt == dx.BF16 else 2.0 ** -8

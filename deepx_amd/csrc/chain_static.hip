@@ -169,7 +169,7 @@ __global__ __launch_bounds__(kBlock) void chain_static_flat_kernel(const StaticA
 namespace {
 constexpr int RES = DXH_CHAIN_RESULT, FULL = DXH_CHAIN_FULL, ROW = DXH_CHAIN_ROW, COL = DXH_CHAIN_COLUMN;
 
-// RMSNorm of a 16-bit activation in fp32 with a 16-bit weight row, as the batch path sees the front's
+// RMSNorm of a 16-bit (or fp32) activation in fp32 with a weight row of the same type, as the batch path sees the front's
 // T5LayerNorm (front/py/deepx/nn/modules/norm/t5layernorm.py:17-22) once its tensors exist:
 //   xf = todtype(x)  sq = xf^2  var = sum(sq, -1)  var /= cols  var += eps  var = sqrt(var)  var = 1 / var
 //   rs = broadcastTo(var)  xn = xf * rs  wf1 = todtype(w)  wf = broadcastTo(wf1)  xn = wf * xn  h = todtype(xn)
@@ -318,6 +318,7 @@ int static_rows_try(const dxh_chain_tensor *inputs, int n_inputs, const dxh_chai
 #define DXH_TRY_ROWS(PROG, VW) if (rc == kNotStatic && rows_match<PROG>(inputs, n_inputs, ops, n_ops) && aligned_to(VW)) rc = launch_rows<PROG, VW>(a, rows, cols, st, dry)
     DXH_TRY_ROWS(RmsNormProg<kSBF16>, 4);
     DXH_TRY_ROWS(RmsNormProg<kSF16>, 4);
+    DXH_TRY_ROWS(RmsNormProg<kSF32>, 4);  // a model kept in fp32: the two casts are copies
     DXH_TRY_ROWS(SoftmaxProg<kSF32>, 4);
     DXH_TRY_ROWS(SoftmaxProg<kSBF16>, 8);
     DXH_TRY_ROWS(SoftmaxProg<kSF16>, 8);

@@ -67,6 +67,11 @@ def run_separately(dxh, orc, inputs, prog, rows, cols):
             assert adt == dt == dx.F32 and ae == e
             dx.check(dxh.dxh_powscalar(dt, a.ptr, dx.scalar(2.0), out.ptr, n, None), "powscalar")
             assert orc.orc_powscalar(dt, hp(ah), dx.scalar(2.0), hp(want), n) == 0
+            # the device squares with one multiplication (correctly rounded); the oracle's powf is within an ulp of that,
+            # and has its bits whenever the square needs no rounding (operands that came from a 16-bit type)
+            assert np.array_equal(out.get(), (ah.astype(np.float64) ** 2).astype(np.float32)), ("square", rows, cols)
+            assert H.ulp_diff(out.get(), want, dt) <= 1, ("square", rows, cols)
+            want = None
         elif name in BINARY:
             b, bdt, be = src(rhs)
             assert adt == bdt == dt and ae == be == e

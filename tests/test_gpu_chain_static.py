@@ -71,7 +71,7 @@ def three_ways(dxh, orc, ins, prog, rows, cols, label, interpreter_takes_it=True
         dx.check(dxh.dxh_tune(KNOB_STATIC, 1))
 
 
-@pytest.mark.parametrize("half", [dx.BF16, dx.F16])
+@pytest.mark.parametrize("half", [dx.BF16, dx.F16, dx.F32])
 def test_rmsnorm_compiled(dxh, orc, half):
     """The thirteen lines of the front's RMSNorm (t5layernorm.py:17-22) as one compiled launch: rows of 1 to 8
     vectors per lane, rows that end inside a lane's vectors, fewer rows than a workgroup holds, lane groups

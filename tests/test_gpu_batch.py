@@ -813,3 +813,51 @@ def test_attention_core_one_launch_for_scale_and_softmax(dxh, tmp_path, dt):
     tol = 1e-4 if dt == "float32" else 3e-2
     assert np.all(np.abs(got - o) <= tol * (np.abs(y) @ np.abs(v64)) + 1e-6), float(np.max(np.abs(got - o)))
     assert np.allclose(load(results["plain"]["y"]).reshape(y.shape).sum(-1), 1.0, atol=1e-5 if dt == "float32" else 3e-2)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_rmsnorm_lines_take_the_compiled_kernel_in_fp32_too(dxh, tmp_path, dt):
+    """The thirteen lines of the front's RMSNorm on an activation and a weight kept in fp32 (the front's default dtype; the
+    two casts are then copies) or in bf16: one launch of the compiled kernel, the bits of the lines run one by one, and
+    the formula in float64."""
+    S, Hd = 192, 896
+    rng = np.random.default_rng(67)
+    store = {"float32": lambda a: a, "bfloat16": H.f32_to_bf16_bits}[dt]
+    load = {"float32": lambda a: a.astype(np.float64), "bfloat16": lambda a: H.bf16_bits_to_f32(a).astype(np.float64)}[dt]
+    x, w = rng.standard_normal((S, Hd)).astype(np.float32), (1 + 0.1 * rng.standard_normal((1, Hd))).astype(np.float32)
+    f32 = "float32"
+    results = {}
+    for mode in ("plain", "batch"):
+        ex = InProc()
+        ex.set_fusion(mode == "batch")
+        h = Host(ex, tmp_path)
+        p = f"rn_{mode}_{dt}_"
+        n = lambda name, d=f32: T(p + name, d)
+        h.put(p + "x", store(x), dt)
+        h.put(p + "w", store(w), dt)
+        for name, shape, d in (("xf", [S, Hd], f32), ("sq", [S, Hd], f32), ("var", [S, 1], f32), ("rs", [S, Hd], f32), ("xn", [S, Hd], f32), ("wf1", [1, Hd], f32),
+                               ("wf", [S, Hd], f32), ("h", [S, Hd], dt)):
+            h.run(f"newtensor({V(shape)})->({n(name, d)})")
+        lines = [f"todtype({n('x', dt)})->({n('xf')})", f"powscalar({n('xf')}, var<float32>:2)->({n('sq')})", f"sum({n('sq')}, {V([-1])}, var<bool>:true)->({n('var')})",
+                 f"divscalar({n('var')}, var<float32>:{Hd})->({n('var')})", f"addscalar({n('var')}, var<float32>:1e-06)->({n('var')})", f"sqrt({n('var')})->({n('var')})",
+                 f"rdivscalar(var<float32>:1, {n('var')})->({n('var')})", f"broadcastTo({n('var')}, {V([S, Hd])})->({n('rs')})", f"mul({n('xf')}, {n('rs')})->({n('xn')})",
+                 f"todtype({n('w', dt)})->({n('wf1')})", f"broadcastTo({n('wf1')}, {V([S, Hd])})->({n('wf')})", f"mul({n('wf')}, {n('xn')})->({n('xn')})",
+                 f"todtype({n('xn')})->({n('h', dt)})"]
+        lines = [f"{l} // author=miaobyte id={i + 1}" for i, l in enumerate(lines)]
+        a0, b0 = C.c_int64(), C.c_int64()
+        dxh.dxh_chain_stats(C.byref(a0), C.byref(b0))
+        rs = ex.execute_batch(lines)
+        assert all(r.split(" ")[1].startswith("ok") for r in rs), rs
+        a1, b1 = C.c_int64(), C.c_int64()
+        dxh.dxh_chain_stats(C.byref(a1), C.byref(b1))
+        if mode == "batch":
+            assert ex.fusion_stats()["runs"] == 1 and ex.fusion_stats()["lines"] == 13, ex.fusion_stats()
+            assert (a1.value - a0.value, b1.value - b0.value) == (1, 0), "the run did not take its compiled kernel"
+        results[mode] = {k: h.get(p + k) for k in ("xf", "sq", "var", "rs", "xn", "wf1", "wf", "h")}
+        ex.close()
+    for k in results["plain"]:
+        assert np.array_equal(results["batch"][k].view(np.uint8), results["plain"][k].view(np.uint8)), k
+    x64, w64 = load(store(x)), load(store(w))
+    ref = w64 * (x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + 1e-6))
+    got = load(results["plain"]["h"]).reshape(S, Hd)
+    assert np.all(np.abs(got - ref) <= (1e-5 if dt == f32 else 1e-2) * np.abs(ref) + 1e-6)
